@@ -1,0 +1,44 @@
+"""CPU oracle for the per-token log-prob / entropy / policy-loss / advantage path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in ``relax_amd`` (the product) may import
+this package: only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` use it, and only as the checker / timed
+CPU baseline.  Every function is a from-scratch PyTorch-CPU restatement of the
+arithmetic the reference performs, written against the reference source read
+as text, and cites the reference ``file:line`` it follows (paths relative to
+the reference checkout).
+
+Pinning status (what independently fixes each function's output; the tests
+live in ``tests/test_oracle_*.py``):
+
+* ``logprob``            literal vectors of the reference's own tests
+                         (tests/utils/training/test_ppo_logprob_entropy.py:174-337),
+                         ``torch.log_softmax`` / ``Categorical.entropy`` library
+                         routines, fp64 ``gradcheck``, shift invariance, row-sum
+                         of gradient == 0.
+* ``losses.policy_clip`` literals tests/backends/megatron/test_reinforce_plus_plus_loss.py:24-59,
+                         tests/utils/training/test_rloo_advantages.py:263-290.
+* ``losses.approx_kl``   literals tests/utils/training/test_ppo_utils_grpo.py:26-83.
+* ``reducers``           literals test_reinforce_plus_plus_loss.py:62-69,
+                         test_rloo_policy_loss_dispatch.py:98-187,
+                         test_cp_loss_mask_alignment.py:95-139,
+                         test_opd_loss_aggregation.py:36-49, brute force.
+* ``advantages``         literals test_rloo_advantages.py:70-225,
+                         tests/utils/replay/helpers.py:40-55,
+                         test_reinforce_reward_processing.py:43-49, brute-force LOO,
+                         numpy ``std(ddof=1)``.
+* ``policy`` composition hand-derived end-to-end fixture tests/utils/replay/helpers.py:40-55
+                         (loss = -0.02; lp=0.5 case 0.877443).
+* ``lmhead``             ``F.linear`` + ``log_softmax`` (library routine),
+                         test_entropy_grad_wiring.py:68-114 shape/temperature.
+* ``losses.gspo_seq_kl``, ``losses.cispo``, ``opd.full_vocab_reverse_kl``
+  (tail-bin modes), ``advantages.masked_whiten``: no reference test or fixture
+  exists; pinned only by closed forms and brute force written independently of
+  the oracle code (explicit python loops / fp64 autograd / ``scipy``-style
+  textbook formulas).  The exact edge conventions the closed forms do not fix
+  (CISPO ``A == 0`` branch, whiten Bessel switch at n < 2) are taken from
+  reading the reference source; see DESIGN notes in each docstring.
+* ``reducers.seq_mean_token_sum``: the reference has no implementation of this
+  aggregation (only the reducer plug-in point, loss.py:1062-1072)
+  -- **parity unpinned**; defined here as sum_i sum_t x*m / B.
+"""

@@ -1,0 +1,212 @@
+"""Pins oracle.losses / oracle.reducers against the reference's literals, closed forms and brute force (CPU)."""
+
+import math
+
+import pytest
+import torch
+
+from oracle import losses as L
+from oracle import reducers as R
+
+
+def _t(x, dt=torch.float64):
+    return torch.tensor(x, dtype=dt)
+
+
+def test_ppo_clip_and_k2_response_mean_literal(literals):
+    fx = literals["ppo_clip_k2_response_mean"]
+    cur, old, ref, adv = _t(fx["current"]), _t(fx["old"]), _t(fx["reference"]), _t(fx["advantages"])
+    masks = [torch.tensor(m) for m in fx["masks"]]
+    lens = fx["response_lengths"]
+    pg, _ = L.policy_clip(old - cur, adv, *fx["eps"])
+    k2 = L.approx_kl(cur, ref, "k2")
+    red = R.make_reducer(lens, masks)
+    # independent: python loops over tokens
+    exp_pg, exp_k2 = [], []
+    for c, o, r, a in zip(fx["current"], fx["old"], fx["reference"], fx["advantages"]):
+        ratio = math.exp(c - o)
+        exp_pg.append(max(-ratio * a, -min(max(ratio, 0.8), 1.2) * a))
+        exp_k2.append(0.5 * (c - r) ** 2)
+    torch.testing.assert_close(pg, _t(exp_pg), atol=fx["tol"], rtol=fx["tol"])
+    torch.testing.assert_close(k2.double(), _t(exp_k2), atol=fx["tol"], rtol=fx["tol"])
+
+    def resp_mean(vals):
+        out, off = 0.0, 0
+        for n, m in zip(lens, fx["masks"]):
+            out += sum(v * w for v, w in zip(vals[off : off + n], m)) / sum(m)
+            off += n
+        return out / len(lens)
+
+    assert abs(float(red(pg)) / len(lens) - resp_mean(exp_pg)) < fx["tol"]
+    assert abs(float(red(k2)) / len(lens) - resp_mean(exp_k2)) < fx["tol"]
+
+
+def test_masked_tokens_do_not_change_reduction_but_nan_propagates(literals):
+    fx = literals["masked_invariance"]
+    masks = [torch.tensor(m) for m in fx["masks"]]
+    red = R.make_reducer(fx["lengths"], masks)
+    assert torch.equal(red(torch.tensor(fx["base"])), red(torch.tensor(fx["changed"])))
+    bad = torch.tensor([1.0, float("nan"), 3.0, 4.0, float("inf")])
+    assert torch.isnan(red(bad))
+    assert torch.isnan(R.make_reducer(fx["lengths"], masks, per_token=True)(bad))
+
+
+def test_clip_case_literal(literals):
+    fx = literals["clip_case"]
+    pg, cf = L.policy_clip(_t([fx["ppo_kl"]]), _t([fx["advantage"]]), *fx["eps"])
+    assert cf.item() == fx["expected_clipfrac"]
+    assert abs(pg.item() - (-1.2)) < 1e-12
+    loss, cf = L.rloo_loss(_t([fx["rloo_log_prob"]]), _t([1.0]))
+    assert abs(loss.item() - fx["rloo_expected_loss"]) < 1e-12 and cf.item() == fx["rloo_expected_clipfrac"]
+
+
+def test_kl_estimators_literal(literals):
+    fx = literals["kl_estimators"]
+    for kind in ("k1", "k2", "k3", "low_var_kl"):
+        lp, base = fx[kind]["lp"], fx[kind]["base"]
+        got = L.approx_kl(torch.tensor(lp), torch.tensor(base), kind)
+        for g, a, b in zip(got.tolist(), lp, base):
+            d = a - b
+            want = {"k1": d, "k2": d * d / 2, "k3": math.exp(-d) - 1 + d, "low_var_kl": min(10.0, math.exp(-d) - 1 + d)}[kind]
+            assert abs(g - want) < fx["atol"] * max(1.0, abs(want))
+        if kind in ("k2", "k3", "low_var_kl"):
+            assert (got >= 0).all()
+    assert L.approx_kl(torch.tensor(fx["low_var_kl"]["lp"]), torch.zeros(3), "low_var_kl")[0].item() == 10.0
+    with pytest.raises(ValueError, match="Unknown kl_loss_type: unsupported"):
+        L.approx_kl(torch.zeros(2), torch.zeros(2), "unsupported")
+
+
+def test_unbiased_kl_multiplies_ratio():
+    lp, base, ratio = torch.tensor([-0.5, -1.0]), torch.tensor([-0.7, -0.4]), torch.tensor([1.3, 0.6])
+    torch.testing.assert_close(L.approx_kl(lp, base, "k3", ratio), ratio * L.approx_kl(lp, base, "k3"))
+
+
+def test_ppo_clip_gradient_convention_bruteforce():
+    # dloss/dlp = -A*r where unclipped branch is active (incl. inside the clamp range), else 0
+    torch.manual_seed(0)
+    lp = (torch.randn(200, dtype=torch.float64) * 0.3).requires_grad_()
+    old = torch.randn(200, dtype=torch.float64) * 0.3
+    adv = torch.randn(200, dtype=torch.float64)
+    adv[:5] = 0.0
+    loss, _ = L.policy_clip(old - lp, adv, 0.2, 0.28)
+    loss.sum().backward()
+    for i in range(200):
+        r = math.exp(lp[i].item() - old[i].item())
+        a = adv[i].item()
+        inside = 0.8 <= r <= 1.28
+        active = inside or (-r * a > -min(max(r, 0.8), 1.28) * a)
+        want = -a * r if active else 0.0
+        assert abs(lp.grad[i].item() - want) < 1e-12
+
+
+def test_dual_clip_bruteforce():
+    torch.manual_seed(1)
+    kl = torch.randn(100, dtype=torch.float64)
+    adv = torch.randn(100, dtype=torch.float64)
+    loss, _ = L.policy_clip(kl, adv, 0.2, 0.2, 3.0)
+    for i in range(100):
+        r, a = math.exp(-kl[i].item()), adv[i].item()
+        base = max(-r * a, -min(max(r, 0.8), 1.2) * a)
+        want = min(-3.0 * a, base) if a < 0 else base
+        assert abs(loss[i].item() - want) < 1e-12
+
+
+def test_gspo_seq_kl_bruteforce_and_gradient():
+    torch.manual_seed(2)
+    lens = [3, 5, 1]
+    lps = [torch.randn(n, dtype=torch.float64, requires_grad=True) for n in lens]
+    olds = [torch.randn(n, dtype=torch.float64) for n in lens]
+    masks = [torch.tensor([1.0, 0.0, 1.0]).double(), torch.ones(5).double(), torch.zeros(1).double()]
+    out = L.gspo_seq_kl(lps, olds, masks)
+    off = 0
+    for lp, old, m in zip(lps, olds, masks):
+        num = sum((o - l) * w for o, l, w in zip(old.tolist(), lp.tolist(), m.tolist()))
+        k = num / max(sum(m.tolist()), 1.0)
+        for j in range(len(lp)):
+            assert abs(out[off + j].item() - k) < 1e-12
+        off += len(lp)
+    out.sum().backward()
+    # d(sum_t k_i)/dlp_t = -R_i * m_t / clamp(sum m, 1)
+    for lp, m, n in zip(lps, masks, lens):
+        want = -n * m / max(m.sum().item(), 1.0)
+        torch.testing.assert_close(lp.grad, want)
+
+
+def test_cispo_bruteforce_and_gradient():
+    torch.manual_seed(3)
+    lp = torch.randn(300, dtype=torch.float64).requires_grad_()
+    old = lp.detach() + torch.randn(300, dtype=torch.float64) * 0.5
+    adv = torch.randn(300, dtype=torch.float64)
+    adv[:4] = 0.0
+    loss, cf = L.cispo(lp, old - lp, adv, 0.2, 0.28)
+    loss.sum().backward()
+    for i in range(300):
+        r, a = math.exp(lp[i].item() - old[i].item()), adv[i].item()
+        coef = min(r, 1.28) if a >= 0 else max(r, 0.8)  # A == 0 takes the upper-cap branch
+        assert abs(loss[i].item() - (-coef * a * lp[i].item())) < 1e-12
+        assert abs(lp.grad[i].item() - (-coef * a)) < 1e-12
+        assert cf[i].item() == float((a >= 0 and r > 1.28) or (a < 0 and r < 0.8))
+
+
+def test_per_token_path_literal(literals):
+    fx = literals["per_token_loss_path"]
+    masks = [_t(m) for m in fx["masks"]]
+    lp = _t(fx["log_probs"]).requires_grad_()
+    adv = _t(fx["advantages"])
+    red = R.make_reducer(fx["response_lengths"], masks, per_token=True)
+    loss, _ = L.rloo_loss(lp, adv)
+    tok_sum = red(loss)
+    n = R.num_tokens(masks)
+    flat = torch.cat(masks)
+    torch.testing.assert_close(tok_sum, -(adv * lp * flat).sum())
+    assert n.item() == fx["expected_normalizer"]
+    (tok_sum / n).backward()
+    torch.testing.assert_close(lp.grad, -(adv * flat) / fx["expected_normalizer"])
+    mean_red = R.make_reducer(fx["response_lengths"], masks)
+    assert not torch.allclose(tok_sum / n, mean_red(loss.detach()) / 2)
+
+
+def test_target_coordinate_masks_and_counts(literals):
+    fx = literals["target_coordinate_masks"]
+    m = torch.tensor(fx["mask"])
+    red = R.make_reducer([4], [m], per_token=True)
+    assert red(torch.tensor(fx["values"])).item() == fx["token_sum"]
+    assert R.num_tokens([m]).item() == fx["count"] and R.num_tokens([m]).dtype == torch.int64
+    shifted = torch.nn.functional.pad(torch.tensor(fx["sft_mask_in"]), (0, 1))[1:]
+    assert shifted.tolist() == fx["sft_mask_out"] and int(shifted.sum()) == fx["sft_count"]
+
+
+def test_fully_masked_sample_counts_as_one_token():
+    masks = [torch.tensor([0, 0, 0]), torch.tensor([1, 1])]
+    assert R.num_tokens(masks).item() == 3
+    red = R.make_reducer([3, 2], masks)
+    assert red(torch.tensor([5.0, 5.0, 5.0, 2.0, 4.0])).item() == 3.0  # 0/clamp(0,1) + 6/2
+
+
+def test_supplied_sample_denominators():
+    masks = [torch.tensor([1.0, 1.0]), torch.tensor([1.0, 0.0])]
+    red = R.make_reducer([2, 2], masks, sample_denoms=[3, 3])
+    assert abs(red(torch.tensor([3.0, 3.0, 6.0, 9.0])).item() - (6 / 3 + 6 / 3)) < 1e-6
+
+
+def test_opd_token_mean_literal(literals):
+    fx = literals["opd_token_mean"]
+    masks = [torch.tensor(m) for m in fx["masks"]]
+    assert R.token_mean(fx["lengths"], masks)(torch.tensor(fx["values"])).item() == fx["expected"]
+
+
+def test_tis_bruteforce():
+    torch.manual_seed(4)
+    tr, ro = torch.randn(50), torch.randn(50)
+    pg = torch.randn(50)
+    out, met = L.vanilla_tis(pg, tr, ro, 0.0, 2.0)
+    for i in range(50):
+        t = math.exp(tr[i].item() - ro[i].item())
+        w = min(max(t, 0.0), 2.0)
+        assert abs(out[i].item() - pg[i].item() * w) < 1e-5 * max(1, abs(pg[i].item() * w))
+        assert met["tis_clipfrac"][i].item() == float(t > 2.0)
+
+
+def test_sapo_gate_value_at_ratio_one():
+    loss, cf = L.sapo(torch.zeros(2), torch.tensor([1.0, -1.0]), 1.0, 1.05)
+    assert abs(loss[0].item() + 2.0) < 1e-6 and abs(loss[1].item() - 2.0 / 1.05) < 1e-6 and cf.sum() == 0
