@@ -1,0 +1,201 @@
+"""Benchmark of the fused log-prob + entropy + PPO-loss forward+backward at V = 151936, bf16, on one MI355X.
+
+One "step" = one pass of the hot path over one synthetic micro-batch that is already resident in HBM:
+``relax_amd.policy_loss_function(args, batch, logits)`` (log-prob + entropy forward, PPO-clip 0.2/0.28 + k3 KL
+coef 1e-3, token-mean aggregation) followed by ``loss.backward()`` to bf16 dlogits.  Workload = the Qwen3-8B-shaped
+actor step: 16 sequences x 4096 tokens = 65536 rows x 151936 vocabulary, logits ~ N(0, 3) with 5 % spiked rows,
+first 20 % of every sequence masked out.
+
+Prints ONE JSON line (metric, value, roofline of the dominant kernel, CPU baseline of the same arithmetic).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from types import SimpleNamespace
+
+import torch
+
+VOCAB = 151936
+SEQS, SEQ_LEN = 16, 4096
+HBM_PEAK_GBS = 8000.0
+
+
+def make_args():
+    return SimpleNamespace(
+        advantage_estimator="grpo", eps_clip=0.2, eps_clip_high=0.28, entropy_coef=0.0, use_kl_loss=True,
+        kl_loss_coef=1e-3, kl_loss_type="k3", use_unbiased_kl=False, use_rollout_logprobs=False,
+        true_on_policy_mode=False, use_opsm=False, use_tis=False, get_mismatch_metrics=False,
+        rollout_temperature=1.0, calculate_per_token_loss=False, qkv_format="thd", log_probs_chunk_size=-1,
+        opsm_delta=1e-4, tis_clip=2.0, tis_clip_low=0.0, sapo_tau_pos=1.0, sapo_tau_neg=1.05, global_batch_size=SEQS,
+    )
+
+
+def make_workload(device, seqs: int, seq_len: int, vocab: int, seed: int = 0):
+    """Synthetic inputs of the named configuration, generated on the device in row blocks."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    n = seqs * seq_len
+    logits = torch.empty((1, n, vocab), dtype=torch.bfloat16, device=device)
+    flat = logits[0]
+    block = 2048
+    for s in range(0, n, block):
+        e = min(n, s + block)
+        x = torch.randn((e - s, vocab), device=device, generator=g) * 3.0
+        spike = torch.rand(e - s, device=device, generator=g) < 0.05
+        cols = torch.randint(0, vocab, (e - s,), device=device, generator=g)
+        x[spike, cols[spike]] += 15.0
+        flat[s:e] = x.to(torch.bfloat16)
+        del x
+    tokens = [torch.randint(0, vocab, (seq_len,), device=device, generator=g) for _ in range(seqs)]
+    mask = torch.ones(seq_len, device=device)
+    mask[: seq_len // 5] = 0.0
+    # token-mean aggregation over the micro-batch = every sample divided by the total unmasked count
+    total_unmasked = float(mask.sum().item()) * seqs
+    batch = dict(
+        unconcat_tokens=tokens,
+        total_lengths=[seq_len] * seqs,
+        response_lengths=[seq_len] * seqs,  # every row is scored (response == total)
+        loss_masks=[mask.clone() for _ in range(seqs)],
+        advantages=[torch.randn((), device=device, generator=g).expand(seq_len).contiguous() for _ in range(seqs)],
+        relax_amd_sample_denominators=torch.full((seqs,), total_unmasked, device=device),
+    )
+    return logits, batch, g
+
+
+def attach_old_and_ref(batch, logits, args, g):
+    """old = lp + N(0, 0.05), ref = lp + N(0, 0.1) around the model's own log-probs."""
+    import relax_amd
+
+    with torch.no_grad():
+        _, out = relax_amd.get_log_probs_and_entropy(
+            logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=batch["total_lengths"],
+            response_lengths=batch["response_lengths"], with_entropy=False)
+    lps = out["log_probs"]
+    batch["log_probs"] = [lp + 0.05 * torch.randn(lp.shape, device=lp.device, generator=g) for lp in lps]
+    batch["ref_log_probs"] = [lp + 0.1 * torch.randn(lp.shape, device=lp.device, generator=g) for lp in lps]
+
+
+def cpu_baseline(args, rows: int, vocab: int):
+    """The oracle (CPU restatement of the reference's PyTorch ops) on a bounded slice of the same workload."""
+    from oracle import policy as P
+    from oracle import reducers as R
+
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(1, rows, vocab, generator=g) * 3.0).bfloat16().float()  # the reference path receives fp32 logits
+    spike = torch.rand(rows, generator=g) < 0.05
+    x[0, spike, torch.randint(0, vocab, (rows,), generator=g)[spike]] += 15.0
+    x.requires_grad_()
+    toks = [torch.randint(0, vocab, (rows,), generator=g)]
+    mask = torch.ones(rows)
+    mask[: rows // 5] = 0
+    base = torch.full((rows,), -12.0)
+    batch = dict(unconcat_tokens=toks, total_lengths=[rows], response_lengths=[rows], loss_masks=[mask],
+                 advantages=[torch.randn(rows, generator=g)], log_probs=[base], ref_log_probs=[base + 0.1])
+    oargs = P.make_args(eps_clip=0.2, eps_clip_high=0.28, use_kl_loss=True, kl_loss_coef=1e-3, kl_loss_type="k3")
+    red = R.make_reducer([rows], [mask])
+    t0 = time.perf_counter()
+    loss, _ = P.policy_loss_function(oargs, batch, x, red)
+    loss.backward()
+    dt = time.perf_counter() - t0
+    return {
+        "value": rows / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"{rows} rows x {vocab} vocab fp32 logits, fwd+bwd, {dt:.2f} s on {threads} host threads "
+                  f"(of os.cpu_count()={os.cpu_count()}); rows are independent so tokens/s does not depend on N",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--seqs", type=int, default=SEQS)
+    ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
+    ap.add_argument("--vocab", type=int, default=VOCAB)
+    ap.add_argument("--cpu-rows", type=int, default=512, help="rows of the CPU baseline sample (0 = skip)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (rows shard trivially; see DESIGN.md). "
+              "Run with --gpus 1.", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm GPU", file=sys.stderr)
+        return 2
+    import relax_amd
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    args = make_args()
+    logits, batch, g = make_workload(dev, a.seqs, a.seq_len, a.vocab)
+    attach_old_and_ref(batch, logits, args, g)
+    logits.requires_grad_()
+    n_tokens = a.seqs * a.seq_len
+
+    def step(record=None):
+        logits.grad = None
+        if record:
+            record[0].record()
+        loss, _ = relax_amd.policy_loss_function(args, batch, logits, None)
+        if record:
+            record[1].record()
+        loss.backward()
+        if record:
+            record[2].record()
+        return loss
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(a.steps)]
+    t0 = time.perf_counter()
+    for k in range(a.steps):
+        loss = step(events[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / a.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / a.steps
+    ms_per_step = wall * 1e3 / a.steps
+    elem = logits.element_size()
+    # dominant kernel = the dlogits backward: one read + one write of every row
+    bwd_bytes = 2.0 * a.vocab * elem * n_tokens
+    achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+    step_bytes = 3.0 * a.vocab * elem * n_tokens
+    out = {
+        "metric": "tokens/s fused logprob+entropy+loss fwd+bwd @V=151936 bf16; % HBM/MFMA peak",
+        "value": n_tokens / (wall / a.steps),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"Qwen3-8B-shaped actor step: {a.seqs} seqs x {a.seq_len} tokens = {n_tokens} rows x "
+                        f"V={a.vocab} bf16 logits, PPO-clip 0.2/0.28 + k3 KL 1e-3, fwd + bwd to dlogits",
+            "rows": n_tokens, "vocab": a.vocab, "loss": float(loss.item()),
+        },
+        "roofline": {
+            "bound": "hbm", "kernel": "logprob_entropy_bwd_kernel<bf16>", "achieved": achieved,
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_ms": bwd_ms,
+            "forward_ms": fwd_ms, "forward_GBs": a.vocab * elem * n_tokens / (fwd_ms * 1e-3) / 1e9,
+            "step_algorithmic_GBs": step_bytes / (ms_per_step * 1e-3) / 1e9,
+        },
+        "cpu_baseline": cpu_baseline(args, a.cpu_rows, a.vocab) if a.cpu_rows > 0 else None,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

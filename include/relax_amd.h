@@ -1,0 +1,217 @@
+/*
+ * relax_amd -- C ABI of the MI355X (gfx950) kernels for Relax's per-token
+ * log-prob / entropy / policy-loss / advantage path.
+ *
+ * The reference (redai-infra/Relax) has no FFI for this path: it is pure
+ * PyTorch.  Each entry point below therefore cites the reference Python
+ * function whose arithmetic it replaces (paths relative to the reference
+ * checkout).  Conventions:
+ *   - all pointers are DEVICE pointers unless stated otherwise; the caller
+ *     owns every buffer; outputs are caller-allocated; inputs are never
+ *     written;
+ *   - no entry point allocates, frees or synchronises; work is enqueued on
+ *     `stream` (a hipStream_t passed as void*; NULL = the default stream);
+ *   - return value 0 = success, negative = error; the message is available
+ *     from relax_amd_last_error() on the calling thread;
+ *   - `dtype` is one of the RELAX_AMD_* element codes; fp32 is used for all
+ *     per-token side vectors;
+ *   - kernels are deterministic (no floating-point atomics): the same inputs
+ *     give bit-identical outputs run to run.
+ */
+#ifndef RELAX_AMD_H
+#define RELAX_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RELAX_AMD_ABI_VERSION 1
+
+enum { RELAX_AMD_F32 = 0, RELAX_AMD_BF16 = 1, RELAX_AMD_F16 = 2, RELAX_AMD_F64 = 3 };
+
+enum { RELAX_AMD_OK = 0, RELAX_AMD_EINVAL = -1, RELAX_AMD_ELAUNCH = -2, RELAX_AMD_EUNSUPPORTED = -3 };
+
+/* policy-loss flavours (relax/backends/megatron/loss.py:976-1000) */
+enum { RELAX_AMD_LOSS_PPO = 0, RELAX_AMD_LOSS_GSPO = 1, RELAX_AMD_LOSS_CISPO = 2, RELAX_AMD_LOSS_RLOO = 3, RELAX_AMD_LOSS_SAPO = 4 };
+/* KL estimators (relax/utils/training/ppo_utils.py:100-139) */
+enum { RELAX_AMD_KL_NONE = 0, RELAX_AMD_KL_K1 = 1, RELAX_AMD_KL_K2 = 2, RELAX_AMD_KL_K3 = 3, RELAX_AMD_KL_LOW_VAR = 4 };
+/* group reward normalisation (relax/utils/utils.py:199-238) */
+enum { RELAX_AMD_GROUP_CENTER = 0, RELAX_AMD_GROUP_CENTER_STD = 1, RELAX_AMD_GROUP_RLOO = 2 };
+
+/* slots of the metrics vector written by relax_amd_policy_loss */
+enum {
+  RELAX_AMD_M_LOSS = 0,
+  RELAX_AMD_M_PG_LOSS = 1,
+  RELAX_AMD_M_ENTROPY = 2,
+  RELAX_AMD_M_CLIPFRAC = 3,
+  RELAX_AMD_M_PPO_KL = 4,
+  RELAX_AMD_M_KL_LOSS = 5,
+  RELAX_AMD_M_LOGPROB_ABS_DIFF = 6,
+  RELAX_AMD_M_PROB_ABS_DIFF = 7,
+  RELAX_AMD_M_OIS = 8,
+  RELAX_AMD_M_TIS = 9,
+  RELAX_AMD_M_TIS_CLIPFRAC = 10,
+  RELAX_AMD_M_TIS_ABS = 11,
+  RELAX_AMD_M_MISMATCH_KL = 12,
+  RELAX_AMD_M_MISMATCH_K3 = 13,
+  RELAX_AMD_M_OPSM_CLIPFRAC = 14,
+  RELAX_AMD_M_MASK_SUM = 15,
+  RELAX_AMD_NUM_METRICS = 16
+};
+
+int relax_amd_version(void);
+/* Message of the last failing call on this thread ("" if none). Host pointer, valid until the next call. */
+const char* relax_amd_last_error(void);
+
+/*
+ * Target-token log-prob and full-vocab entropy of each row, one streaming
+ * read of the row.  Replaces _VocabParallelLogProbEntropy.forward
+ * (relax/utils/training/ppo_utils.py:481-589, single vocab shard) together
+ * with the per-sample temperature division of get_responses
+ * (relax/backends/megatron/loss.py:184-189).
+ *   logits      [*, vocab] elements of `dtype`, row r at logits + row*row_stride
+ *   row_ids     [n_tokens] int32 logits-row of each token, or NULL (token i = row i)
+ *   targets     [n_tokens] int64 target id of each token (ids outside [0,vocab) give NaN)
+ *   log_prob    [n_tokens] out: (x[target] - logsumexp(x)) with x = logits * inv_temperature
+ *   entropy     [n_tokens] out or NULL: logsumexp(x) - sum_v softmax(x)*x
+ *   lse, spx    [n_tokens] out or NULL: logsumexp(x) and sum_v softmax(x)*x, consumed by the backward
+ */
+int relax_amd_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_tokens, int64_t vocab, int64_t row_stride,
+                                  const int32_t* row_ids, const int64_t* targets, float inv_temperature,
+                                  float* log_prob, float* entropy, float* lse, float* spx, void* stream);
+
+/*
+ * dlogits of the forward above, one read of the row and one write.  Replaces
+ * _VocabParallelLogProbEntropy.backward (ppo_utils.py:591-629):
+ *   dlogits[row] = inv_T * ( g_lp*(onehot(target) - p) + g_ent * p * (spx - x) ),  p = exp(x - lse)
+ * Every one of the n_rows logits rows is written exactly once: rows whose
+ * token_of_row is negative (prompt / padding positions) and rows whose
+ * incoming gradients are both zero are filled with zeros without reading.
+ *   token_of_row [n_rows] int32 token index of each logits row, -1 = no token; NULL = identity
+ *   g_lp, g_ent  [n_tokens] incoming gradients of log_prob / entropy (g_ent may be NULL)
+ *   grad_scale   host scalar multiplied into both incoming gradients
+ *   grad_scale_dev optional device scalar (fp32) multiplied in as well, so an upstream autograd scalar needs no
+ *                host read-back; NULL = 1
+ *   dlogits      [n_rows, vocab] out, elements of `dtype`, row stride d_row_stride
+ */
+int relax_amd_logprob_entropy_bwd(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                                  const int32_t* token_of_row, const int64_t* targets, const float* lse,
+                                  const float* spx, const float* g_lp, const float* g_ent, float grad_scale,
+                                  const float* grad_scale_dev, float inv_temperature, void* dlogits,
+                                  int64_t d_row_stride, void* stream);
+
+/*
+ * Row maps of the packed ("thd") response layout.  Replaces the per-sample
+ * index arithmetic of get_responses (loss.py:103-125, cp_size == 1) and
+ * compute_sft_response_chunk (relax/utils/sft_utils.py:23-40).
+ *   row_begin  [n_samples] int64 first logits row that scores sample i's response
+ *   cu_resp    [n_samples+1] int64 exclusive prefix sum of response lengths
+ *   row_ids    [n_tokens] out int32
+ *   sample_ids [n_tokens] out int32 (may be NULL)
+ *   token_of_row [n_rows] out int32 or NULL: inverse map, -1 where no response token
+ */
+int relax_amd_build_row_maps(const int64_t* row_begin, const int64_t* cu_resp, int64_t n_samples, int64_t n_tokens,
+                             int64_t n_rows, int32_t* row_ids, int32_t* sample_ids, int32_t* token_of_row,
+                             void* stream);
+
+/*
+ * Per-token policy loss, KL penalty, masked per-sample aggregation and the
+ * gradient coefficients d loss / d log_prob, d loss / d entropy.  Replaces the
+ * arithmetic of policy_loss_function (loss.py:961-1134) with
+ * compute_policy_loss / compute_gspo_kl / compute_cispo_loss / compute_rloo_loss
+ * / compute_sapo_loss / compute_approx_kl / compute_opsm_mask
+ * (ppo_utils.py:100-396), vanilla_tis_function (loss.py:741-769) and the
+ * reducers of get_sum_of_sample_mean (relax/backends/megatron/cp_utils.py:144-162).
+ */
+typedef struct relax_amd_policy_loss_args {
+  /* packed per-token inputs, fp32 [n_tokens]; NULL where marked optional */
+  const float* log_prob;
+  const float* old_log_prob;     /* NULL: old = current (true on-policy, ratio == 1) */
+  const float* ref_log_prob;     /* optional: needed when kl_type != NONE */
+  const float* train_log_prob;   /* optional: train-engine log-probs for TIS / mismatch metrics (NULL = current) */
+  const float* rollout_log_prob; /* optional */
+  const float* advantages;
+  const float* loss_mask;        /* mask values as fp32 (multiplied, not tested) */
+  const float* pg_loss_mask;     /* optional: numerator mask of the pg-loss reducer (NULL = loss_mask) */
+  const float* entropy;          /* optional */
+  const int64_t* cu_resp;        /* [n_samples+1] */
+  const float* sample_denom;     /* [n_samples] divisor of each sample's masked sum (already clamped), NULL = 1 */
+  const float* pg_sample_denom;  /* [n_samples] divisor for pg_loss only, NULL = sample_denom */
+  int64_t n_samples;
+  int64_t n_tokens;
+  int32_t loss_kind;             /* RELAX_AMD_LOSS_* */
+  int32_t kl_kind;               /* RELAX_AMD_KL_* */
+  int32_t unbiased_kl;           /* multiply KL by exp(lp - old), gradient flows through the ratio */
+  int32_t use_opsm;
+  int32_t use_tis;               /* apply clamp(exp(train - rollout), tis_lo, tis_hi) to pg_loss */
+  int32_t mismatch_metrics;      /* emit OIS/TIS metrics */
+  int32_t abs_diff_from_old;     /* 1: |old - rollout| metrics use old_log_prob, 0: train_log_prob, 2: current */
+  float eps_clip, eps_clip_high, eps_clip_c; /* eps_clip_c <= 0: no dual clip */
+  float entropy_coef, kl_coef;
+  float tis_lo, tis_hi, opsm_delta, tau_pos, tau_neg;
+  /* outputs */
+  float* coef_log_prob;          /* [n_tokens] d loss / d log_prob */
+  float* coef_entropy;           /* [n_tokens] d loss / d entropy, may be NULL */
+  float* pg_loss_tok;            /* optional per-token outputs [n_tokens] */
+  float* clipfrac_tok;
+  float* ppo_kl_tok;
+  float* kl_tok;
+  float* sample_partials;        /* workspace [n_samples * RELAX_AMD_NUM_METRICS] */
+  float* metrics;                /* [RELAX_AMD_NUM_METRICS] */
+} relax_amd_policy_loss_args;
+
+int relax_amd_policy_loss(const relax_amd_policy_loss_args* args, void* stream);
+
+/*
+ * Per-sample masked sums: out[i] = sum_t values[t] * mask[t] over sample i's tokens (values NULL = 1).
+ * Accumulated in fp64 so integer-valued masks give exact counts.  Replaces loss_mask.sum() per sample
+ * (cp_utils.py:140,222) and, with values, one term of sum_of_token (cp_utils.py:156-162).
+ */
+int relax_amd_segment_sum(const float* values, const float* mask, const int64_t* cu_resp, int64_t n_samples,
+                          double* out, void* stream);
+
+/*
+ * Group-normalised rewards in input order.  Replaces the group loop of
+ * post_process_rewards (relax/utils/utils.py:204-238) and
+ * compute_rloo_leave_one_out_rewards (ppo_utils.py:664-705).
+ *   rewards, out [n] elements of `dtype` (RELAX_AMD_F32 or RELAX_AMD_F64; arithmetic is done in that type)
+ *   group_count [n] out int32: size of the group each sample belongs to (host checks == n_samples_per_prompt)
+ */
+int relax_amd_group_rewards(const void* rewards, int dtype, const int32_t* group_index, int64_t n, int32_t mode,
+                            void* out, int32_t* group_count, void* stream);
+
+/* out[t] = per_sample[i] for every token t of sample i.  Replaces get_grpo_returns (ppo_utils.py:654-661). */
+int relax_amd_broadcast_per_sample(const float* per_sample, const int64_t* cu_resp, int64_t n_samples,
+                                   float* out, void* stream);
+
+/*
+ * Masked whitening with Bessel correction.  Replaces distributed_masked_whiten
+ * (relax/utils/distributed_utils.py:98-158) on one rank.
+ *   partials [3 * relax_amd_whiten_partials(n)] fp64 workspace
+ *   stats    [4] out fp32: sum, sum of squares, mask sum, and 1/sqrt(var+eps)
+ */
+int64_t relax_amd_whiten_partials(int64_t n);
+int relax_amd_masked_whiten(const float* values, const float* mask, int64_t n, int32_t shift_mean, float epsilon,
+                            double* partials, float* stats, float* out, void* stream);
+
+/*
+ * Full-vocab reverse KL(student || teacher) per token and its gradient w.r.t.
+ * the student logits.  The K = vocab case of compute_opd_kl's jsd_alpha == 0
+ * branch (relax/utils/opd/opd_utils.py:1165-1169) on complete log-softmax rows.
+ *   kl, lse_s, lse_t [n_tokens] out
+ *   bwd: dstudent = g[t] * grad_scale * (*grad_scale_dev) * p_s * ((log p_s - log p_t) - kl); rows with a zero
+ *        incoming gradient are zero-filled without reading
+ */
+int relax_amd_reverse_kl_fwd(const void* student, const void* teacher, int dtype, int64_t n_tokens, int64_t vocab,
+                             int64_t row_stride, float* kl, float* lse_s, float* lse_t, void* stream);
+int relax_amd_reverse_kl_bwd(const void* student, const void* teacher, int dtype, int64_t n_tokens, int64_t vocab,
+                             int64_t row_stride, const float* kl, const float* lse_s, const float* lse_t,
+                             const float* g, float grad_scale, const float* grad_scale_dev, void* dstudent,
+                             void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RELAX_AMD_H */

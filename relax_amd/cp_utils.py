@@ -1,0 +1,90 @@
+"""Drop-in counterparts of the masked reducers of ``relax/backends/megatron/cp_utils.py`` at context-parallel
+size 1 (reference lines :125-162 reducers, :209-285 token counts), on the gfx950 segment-sum kernel."""
+
+from __future__ import annotations
+
+import torch
+
+from . import ops
+
+
+def _cu(response_lengths, device) -> torch.Tensor:
+    cu = [0]
+    for r in response_lengths:
+        cu.append(cu[-1] + int(r))
+    return torch.tensor(cu, dtype=torch.int64).to(device)
+
+
+def _mask_sums(loss_masks, cu_resp=None) -> torch.Tensor:
+    """Exact per-sample mask sums (fp64 accumulation in the kernel), returned in the masks' own dtype."""
+    dev = loss_masks[0].device
+    if cu_resp is None:
+        cu_resp = _cu([m.numel() for m in loss_masks], dev)
+    sums = ops.segment_sum(torch.cat([m.reshape(-1) for m in loss_masks]), cu_resp)
+    dt = loss_masks[0].dtype
+    return sums.round().to(dt) if not dt.is_floating_point else sums.to(dt)
+
+
+def sample_denominators(loss_masks, layout=None, sample_denoms=None) -> torch.Tensor:
+    """fp32 [B] divisors ``clamp_min(denom_i, 1)`` of the sample-mean reducer (cp_utils.py:138-149)."""
+    dev = loss_masks[0].device
+    if sample_denoms is None:
+        den = _mask_sums(loss_masks, None if layout is None else layout.cu_resp)
+    else:
+        den = torch.as_tensor(sample_denoms, device=dev)
+    return torch.clamp_min(den, 1).to(torch.float32)
+
+
+class _MaskedSampleReduce(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, mask, cu_resp, inv_den):
+        sums = ops.segment_sum(mask, cu_resp, values=x)
+        ctx.save_for_backward(mask, cu_resp, inv_den)
+        ctx.n, ctx.dtype = x.numel(), x.dtype
+        return (sums.to(torch.float32) * inv_den).sum().to(x.dtype if x.dtype.is_floating_point else torch.float32)
+
+    @staticmethod
+    def backward(ctx, g):
+        mask, cu_resp, inv_den = ctx.saved_tensors
+        per_tok = ops.broadcast_per_sample(inv_den, cu_resp, ctx.n)
+        return (per_tok * mask * g.to(torch.float32)).to(ctx.dtype), None, None, None
+
+
+def get_sum_of_sample_mean(
+    total_lengths,
+    response_lengths,
+    loss_masks,
+    calculate_per_token_loss: bool = False,
+    qkv_format: str = "thd",
+    max_seq_lens=None,
+    padded_total_lengths=None,
+    dynamic_cp_size=None,
+    dynamic_cp_rank=None,
+    sample_denoms=None,
+):
+    """Returns the reducer ``x [N] -> scalar``: sum over samples of the masked mean (or the masked token sum)."""
+    if dynamic_cp_size not in (None, 1):
+        raise NotImplementedError("context parallelism is outside the one-GPU path")
+    dev = loss_masks[0].device
+    cu = _cu(response_lengths, dev)
+    mask = torch.cat([m.reshape(-1) for m in loss_masks]).to(torch.float32)
+    if calculate_per_token_loss:
+        inv = torch.ones(len(response_lengths), dtype=torch.float32, device=dev)
+    else:
+        inv = 1.0 / sample_denominators(loss_masks, None, sample_denoms)
+
+    def reducer(x: torch.Tensor) -> torch.Tensor:
+        return _MaskedSampleReduce.apply(x, mask, cu, inv)
+
+    return reducer
+
+
+def get_cp_local_mask_sums(total_lengths, response_lengths, loss_masks, qkv_format="thd", max_seq_lens=None,
+                           padded_total_lengths=None, dynamic_cp_size=None, dynamic_cp_rank=None) -> torch.Tensor:
+    return _mask_sums(loss_masks)
+
+
+def get_cp_local_num_tokens(total_lengths, response_lengths, loss_masks, qkv_format="thd", max_seq_lens=None,
+                            padded_total_lengths=None, dynamic_cp_size=None, dynamic_cp_rank=None) -> torch.Tensor:
+    """``sum_i clamp_min(sum(mask_i), 1)`` -- a fully masked sample counts as one token (cp_utils.py:283-285)."""
+    return torch.clamp_min(_mask_sums(loss_masks), 1).sum()

@@ -1,0 +1,351 @@
+// Streaming log-prob + entropy forward and dlogits backward over [rows, vocab] logits.
+//
+// One workgroup owns one row.  The row is read once with 16-byte non-temporal loads (8 bf16 / 4 fp32 per lane
+// per load, UNROLL loads in flight per lane); every lane keeps a private online-softmax state (running max, sum of
+// exp, sum of exp * x) in the log2 domain so the inner loop is cvt + fma + v_exp_f32 + add + fma per element and the
+// max rescale is paid once per UNROLL*8 elements.  Lane states are merged by a wave64 xor-butterfly, then across
+// waves through LDS in wave order, so results are bit-identical run to run.
+//
+// Arithmetic follows relax/utils/training/ppo_utils.py:481-629 (reference paths are relative to its checkout):
+//   lp = x[tok] - lse,  H = lse - sum_v p*x,  dx = g_lp*(onehot - p) + g_H*p*(sum_v p*x - x),  x = logits / T.
+#include "device_utils.h"
+#include "relax_amd.h"
+
+namespace relax_amd {
+
+constexpr int kRowThreads = 256;
+constexpr int kRowUnroll = 4;
+
+struct SoftmaxState {
+  float m, s, t;  // max of x*c, sum exp2(x*c - m), sum exp2(x*c - m) * x
+};
+
+template <bool ENTROPY, int K>
+__device__ __forceinline__ void absorb(const float (&v)[K], float c, SoftmaxState& st) {
+  float vmax = v[0];
+#pragma unroll
+  for (int i = 1; i < K; ++i) vmax = fmaxf(vmax, v[i]);
+  const float mc = vmax * c;
+  if (mc > st.m) {
+    const float sc = fast_exp2(st.m - mc);
+    st.s *= sc;
+    st.t *= sc;
+    st.m = mc;
+  }
+#pragma unroll
+  for (int i = 0; i < K; ++i) {
+    const float e = fast_exp2(fmaf(v[i], c, -st.m));
+    st.s += e;
+    if (ENTROPY) st.t = fmaf(e, v[i], st.t);
+  }
+}
+
+__device__ __forceinline__ void merge(SoftmaxState& a, float m2, float s2, float t2) {
+  const float mn = fmaxf(a.m, m2);
+  const float fa = fast_exp2(a.m - mn), fb = fast_exp2(m2 - mn);
+  a.s = a.s * fa + s2 * fb;
+  a.t = a.t * fa + t2 * fb;
+  a.m = mn;
+}
+
+// Reduce the per-lane states of a workgroup; the merged state is valid in thread 0.
+template <int THREADS>
+__device__ __forceinline__ void block_merge(SoftmaxState& st, float (*lds)[3]) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    const float m2 = __shfl_xor(st.m, o, kWave), s2 = __shfl_xor(st.s, o, kWave), t2 = __shfl_xor(st.t, o, kWave);
+    merge(st, m2, s2, t2);
+  }
+  const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+  if (lane == 0) {
+    lds[w][0] = st.m;
+    lds[w][1] = st.s;
+    lds[w][2] = st.t;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 1; i < THREADS / kWave; ++i) merge(st, lds[i][0], lds[i][1], lds[i][2]);
+  }
+}
+
+// Absorb one row into `st`.  VEC selects 16-byte loads (row base and stride 16-byte aligned) or scalar loads.
+template <typename T, bool ENTROPY, bool VEC, int THREADS, int UNROLL>
+__device__ __forceinline__ void scan_row(const T* __restrict__ x, int64_t vocab, float c, SoftmaxState& st) {
+  if (VEC) {
+    constexpr int VN = Row<T>::kPerVec;
+    const u32x4* xv = reinterpret_cast<const u32x4*>(x);
+    const int64_t nvec = vocab / VN;
+    int64_t i = threadIdx.x;
+    for (; i + int64_t(UNROLL - 1) * THREADS < nvec; i += int64_t(UNROLL) * THREADS) {
+      u32x4 raw[UNROLL];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) raw[u] = load_stream(xv + i + int64_t(u) * THREADS);
+      float v[UNROLL * VN];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        float part[VN];
+        Row<T>::unpack(raw[u], part);
+#pragma unroll
+        for (int k = 0; k < VN; ++k) v[u * VN + k] = part[k];
+      }
+      absorb<ENTROPY>(v, c, st);
+    }
+    for (; i < nvec; i += THREADS) {
+      float v[VN];
+      Row<T>::unpack(load_stream(xv + i), v);
+      absorb<ENTROPY>(v, c, st);
+    }
+    for (int64_t e = nvec * VN + threadIdx.x; e < vocab; e += THREADS) {
+      float v[1] = {Row<T>::load1(x + e)};
+      absorb<ENTROPY>(v, c, st);
+    }
+  } else {
+    for (int64_t e = threadIdx.x; e < vocab; e += THREADS) {
+      float v[1] = {Row<T>::load1(x + e)};
+      absorb<ENTROPY>(v, c, st);
+    }
+  }
+}
+
+template <typename T, bool ENTROPY, bool VEC>
+__global__ __launch_bounds__(kRowThreads) void logprob_entropy_fwd_kernel(
+    const T* __restrict__ logits, int64_t row_stride, int64_t vocab, const int32_t* __restrict__ row_ids,
+    const int64_t* __restrict__ targets, float c, float inv_t, float* __restrict__ log_prob,
+    float* __restrict__ entropy, float* __restrict__ lse_out, float* __restrict__ spx_out) {
+  __shared__ float lds[kRowThreads / kWave][3];
+  const int64_t tok = blockIdx.x;
+  const int64_t row = row_ids ? int64_t(row_ids[tok]) : tok;
+  const T* x = logits + row * row_stride;
+  SoftmaxState st{kNegHuge, 0.f, 0.f};
+  scan_row<T, ENTROPY, VEC, kRowThreads, kRowUnroll>(x, vocab, c, st);
+  block_merge<kRowThreads>(st, lds);
+  if (threadIdx.x == 0) {
+    const float lse = st.m * kLn2 + logf(st.s);
+    const int64_t tg = targets[tok];
+    float lp = __builtin_nanf("");
+    if (tg >= 0 && tg < vocab) lp = Row<T>::load1(x + tg) * inv_t - lse;
+    log_prob[tok] = lp;
+    const float spx = (st.t / st.s) * inv_t;
+    if (ENTROPY) {
+      if (entropy) entropy[tok] = lse - spx;
+      if (spx_out) spx_out[tok] = spx;
+    }
+    if (lse_out) lse_out[tok] = lse;
+  }
+}
+
+template <typename T, bool VEC>
+__device__ __forceinline__ void zero_row(T* __restrict__ d, int64_t vocab) {
+  if (VEC) {
+    constexpr int VN = Row<T>::kPerVec;
+    u32x4* dv = reinterpret_cast<u32x4*>(d);
+    const int64_t nvec = vocab / VN;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int64_t i = threadIdx.x; i < nvec; i += kRowThreads) store_stream(dv + i, z);
+    for (int64_t e = nvec * VN + threadIdx.x; e < vocab; e += kRowThreads) Row<T>::store1(d + e, 0.f);
+  } else {
+    for (int64_t e = threadIdx.x; e < vocab; e += kRowThreads) Row<T>::store1(d + e, 0.f);
+  }
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kRowThreads) void logprob_entropy_bwd_kernel(
+    const T* __restrict__ logits, int64_t row_stride, int64_t vocab, const int32_t* __restrict__ token_of_row,
+    const int64_t* __restrict__ targets, const float* __restrict__ lse, const float* __restrict__ spx,
+    const float* __restrict__ g_lp, const float* __restrict__ g_ent, float grad_scale,
+    const float* __restrict__ grad_scale_dev, float c, float inv_t,
+    T* __restrict__ dlogits, int64_t d_stride) {
+  const int64_t row = blockIdx.x;
+  T* d = dlogits + row * d_stride;
+  const int64_t tok = token_of_row ? int64_t(token_of_row[row]) : row;
+  float glp = 0.f, gh = 0.f;
+  if (tok >= 0) {
+    if (grad_scale_dev) grad_scale *= *grad_scale_dev;
+    glp = g_lp[tok] * grad_scale;
+    gh = g_ent ? g_ent[tok] * grad_scale : 0.f;
+  }
+  if (tok < 0 || (glp == 0.f && gh == 0.f)) {
+    zero_row<T, VEC>(d, vocab);
+    return;
+  }
+  const T* x = logits + row * row_stride;
+  const float k0 = -lse[tok] * kLog2e;  // p = exp2(x*c + k0)
+  // d = inv_t * p * (-glp + gh * (spx - x*inv_t))  (+ inv_t*glp at the target)
+  const float b = gh * inv_t;
+  const float a0 = -glp * inv_t + (gh != 0.f ? b * spx[tok] : 0.f);
+  const float a1 = -b * inv_t;
+  const float hot = glp * inv_t;
+  const int64_t tg = targets[tok];
+  if (VEC) {
+    constexpr int VN = Row<T>::kPerVec;
+    const u32x4* xv = reinterpret_cast<const u32x4*>(x);
+    u32x4* dv = reinterpret_cast<u32x4*>(d);
+    const int64_t nvec = vocab / VN;
+    const int64_t tvec = (tg >= 0 && tg < nvec * VN) ? tg / VN : -1;
+    const int tsub = int(tg % VN);
+    int64_t i = threadIdx.x;
+    for (; i + int64_t(kRowUnroll - 1) * kRowThreads < nvec; i += int64_t(kRowUnroll) * kRowThreads) {
+      u32x4 raw[kRowUnroll];
+#pragma unroll
+      for (int u = 0; u < kRowUnroll; ++u) raw[u] = load_stream(xv + i + int64_t(u) * kRowThreads);
+#pragma unroll
+      for (int u = 0; u < kRowUnroll; ++u) {
+        float v[VN];
+        Row<T>::unpack(raw[u], v);
+#pragma unroll
+        for (int k = 0; k < VN; ++k) v[k] = fast_exp2(fmaf(v[k], c, k0)) * fmaf(v[k], a1, a0);
+        if (i + int64_t(u) * kRowThreads == tvec) {
+#pragma unroll
+          for (int k = 0; k < VN; ++k)
+            if (k == tsub) v[k] += hot;
+        }
+        store_stream(dv + i + int64_t(u) * kRowThreads, Row<T>::pack(v));
+      }
+    }
+    for (; i < nvec; i += kRowThreads) {
+      float v[VN];
+      Row<T>::unpack(load_stream(xv + i), v);
+#pragma unroll
+      for (int k = 0; k < VN; ++k) v[k] = fast_exp2(fmaf(v[k], c, k0)) * fmaf(v[k], a1, a0);
+      if (i == tvec) {
+#pragma unroll
+        for (int k = 0; k < VN; ++k)
+          if (k == tsub) v[k] += hot;
+      }
+      store_stream(dv + i, Row<T>::pack(v));
+    }
+    for (int64_t e = nvec * VN + threadIdx.x; e < vocab; e += kRowThreads) {
+      const float xe = Row<T>::load1(x + e);
+      float g = fast_exp2(fmaf(xe, c, k0)) * fmaf(xe, a1, a0);
+      if (e == tg) g += hot;
+      Row<T>::store1(d + e, g);
+    }
+  } else {
+    for (int64_t e = threadIdx.x; e < vocab; e += kRowThreads) {
+      const float xe = Row<T>::load1(x + e);
+      float g = fast_exp2(fmaf(xe, c, k0)) * fmaf(xe, a1, a0);
+      if (e == tg) g += hot;
+      Row<T>::store1(d + e, g);
+    }
+  }
+}
+
+template <typename T>
+static int launch_fwd(const void* logits, int64_t n, int64_t vocab, int64_t stride, const int32_t* row_ids,
+                      const int64_t* targets, float inv_t, float* lp, float* ent, float* lse, float* spx,
+                      hipStream_t s) {
+  const bool vec = aligned16(logits) && (stride * int64_t(sizeof(T))) % 16 == 0;
+  const bool with_ent = ent != nullptr || spx != nullptr;
+  const float c = inv_t * kLog2e;
+  const T* x = static_cast<const T*>(logits);
+  dim3 grid(static_cast<unsigned>(n)), block(kRowThreads);
+#define RELAX_AMD_FWD(E, V) \
+  hipLaunchKernelGGL((logprob_entropy_fwd_kernel<T, E, V>), grid, block, 0, s, x, stride, vocab, row_ids, targets, c, \
+                     inv_t, lp, ent, lse, spx)
+  if (with_ent) {
+    if (vec) RELAX_AMD_FWD(true, true); else RELAX_AMD_FWD(true, false);
+  } else {
+    if (vec) RELAX_AMD_FWD(false, true); else RELAX_AMD_FWD(false, false);
+  }
+#undef RELAX_AMD_FWD
+  return check_launch("logprob_entropy_fwd");
+}
+
+template <typename T>
+static int launch_bwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t stride, const int32_t* token_of_row,
+                      const int64_t* targets, const float* lse, const float* spx, const float* g_lp,
+                      const float* g_ent, float grad_scale, const float* grad_scale_dev, float inv_t, void* dlogits,
+                      int64_t d_stride, hipStream_t s) {
+  const bool vec = aligned16(logits) && aligned16(dlogits) && (stride * int64_t(sizeof(T))) % 16 == 0 &&
+                   (d_stride * int64_t(sizeof(T))) % 16 == 0;
+  const float c = inv_t * kLog2e;
+  dim3 grid(static_cast<unsigned>(n_rows)), block(kRowThreads);
+  const T* x = static_cast<const T*>(logits);
+  T* d = static_cast<T*>(dlogits);
+  if (vec)
+    hipLaunchKernelGGL((logprob_entropy_bwd_kernel<T, true>), grid, block, 0, s, x, stride, vocab, token_of_row,
+                       targets, lse, spx, g_lp, g_ent, grad_scale, grad_scale_dev, c, inv_t, d, d_stride);
+  else
+    hipLaunchKernelGGL((logprob_entropy_bwd_kernel<T, false>), grid, block, 0, s, x, stride, vocab, token_of_row,
+                       targets, lse, spx, g_lp, g_ent, grad_scale, grad_scale_dev, c, inv_t, d, d_stride);
+  return check_launch("logprob_entropy_bwd");
+}
+
+}  // namespace relax_amd
+
+using namespace relax_amd;
+
+static const int64_t kMaxGrid = 2147483647LL;
+
+extern "C" int relax_amd_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_tokens, int64_t vocab,
+                                             int64_t row_stride, const int32_t* row_ids, const int64_t* targets,
+                                             float inv_temperature, float* log_prob, float* entropy, float* lse,
+                                             float* spx, void* stream) {
+  if (n_tokens < 0 || n_tokens > kMaxGrid || vocab <= 0 || row_stride < vocab) {
+    set_error("logprob_entropy_fwd: bad shape n_tokens=%lld vocab=%lld row_stride=%lld", (long long)n_tokens,
+              (long long)vocab, (long long)row_stride);
+    return RELAX_AMD_EINVAL;
+  }
+  if (n_tokens == 0) return RELAX_AMD_OK;
+  if (!logits || !targets || !log_prob) {
+    set_error("logprob_entropy_fwd: logits, targets and log_prob must not be NULL");
+    return RELAX_AMD_EINVAL;
+  }
+  if (!(inv_temperature > 0.f)) {
+    set_error("logprob_entropy_fwd: inv_temperature must be > 0");
+    return RELAX_AMD_EINVAL;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case RELAX_AMD_F32:
+      return launch_fwd<float>(logits, n_tokens, vocab, row_stride, row_ids, targets, inv_temperature, log_prob,
+                               entropy, lse, spx, s);
+    case RELAX_AMD_BF16:
+      return launch_fwd<bf16_t>(logits, n_tokens, vocab, row_stride, row_ids, targets, inv_temperature, log_prob,
+                                entropy, lse, spx, s);
+    case RELAX_AMD_F16:
+      return launch_fwd<f16_t>(logits, n_tokens, vocab, row_stride, row_ids, targets, inv_temperature, log_prob,
+                               entropy, lse, spx, s);
+    default:
+      set_error("logprob_entropy_fwd: unknown dtype code %d", dtype);
+      return RELAX_AMD_EINVAL;
+  }
+}
+
+extern "C" int relax_amd_logprob_entropy_bwd(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
+                                             int64_t row_stride, const int32_t* token_of_row, const int64_t* targets,
+                                             const float* lse, const float* spx, const float* g_lp,
+                                             const float* g_ent, float grad_scale, const float* grad_scale_dev,
+                                             float inv_temperature, void* dlogits, int64_t d_row_stride,
+                                             void* stream) {
+  if (n_rows < 0 || n_rows > kMaxGrid || vocab <= 0 || row_stride < vocab || d_row_stride < vocab) {
+    set_error("logprob_entropy_bwd: bad shape n_rows=%lld vocab=%lld row_stride=%lld d_row_stride=%lld",
+              (long long)n_rows, (long long)vocab, (long long)row_stride, (long long)d_row_stride);
+    return RELAX_AMD_EINVAL;
+  }
+  if (n_rows == 0) return RELAX_AMD_OK;
+  if (!logits || !targets || !lse || !g_lp || !dlogits || (g_ent && !spx)) {
+    set_error("logprob_entropy_bwd: NULL argument (spx is required when g_ent is given)");
+    return RELAX_AMD_EINVAL;
+  }
+  if (!(inv_temperature > 0.f)) {
+    set_error("logprob_entropy_bwd: inv_temperature must be > 0");
+    return RELAX_AMD_EINVAL;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case RELAX_AMD_F32:
+      return launch_bwd<float>(logits, n_rows, vocab, row_stride, token_of_row, targets, lse, spx, g_lp, g_ent,
+                               grad_scale, grad_scale_dev, inv_temperature, dlogits, d_row_stride, s);
+    case RELAX_AMD_BF16:
+      return launch_bwd<bf16_t>(logits, n_rows, vocab, row_stride, token_of_row, targets, lse, spx, g_lp, g_ent,
+                                grad_scale, grad_scale_dev, inv_temperature, dlogits, d_row_stride, s);
+    case RELAX_AMD_F16:
+      return launch_bwd<f16_t>(logits, n_rows, vocab, row_stride, token_of_row, targets, lse, spx, g_lp, g_ent,
+                               grad_scale, grad_scale_dev, inv_temperature, dlogits, d_row_stride, s);
+    default:
+      set_error("logprob_entropy_bwd: unknown dtype code %d", dtype);
+      return RELAX_AMD_EINVAL;
+  }
+}

@@ -1,0 +1,364 @@
+// Per-token policy loss + KL penalty + masked per-sample aggregation + gradient coefficients, in two launches.
+//
+// Launch 1: one workgroup per sample (a response in the packed "thd" layout, delimited by cu_resp).  The workgroup
+// walks its tokens up to three times over KB-sized fp32 side vectors (never over logits):
+//   pass A (GSPO / OPSM only)  sequence KL  k_i = sum((old-lp)*m) / max(sum m, 1)        ppo_utils.py:183-209, 142-180
+//   pass B                     per-token loss terms, masked sums of every metric, and the token-local part of
+//                              d loss / d lp;  for GSPO also G_i = sum_t w_t * A_t * r_i * [unclipped]
+//   pass C (GSPO only)         adds the sequence-coupled gradient  -G_i * m_t / max(sum m, 1)
+// Per-sample sums are divided by the caller's per-sample denominators, exactly the structure of
+// get_sum_of_sample_mean / sum_of_token (relax/backends/megatron/cp_utils.py:144-162).
+// Launch 2: one workgroup adds the per-sample partials in sample order and assembles
+//   loss = pg_loss - entropy_coef * entropy_loss + kl_coef * kl_loss                        loss.py:1084-1100
+// All reductions use a fixed combination order, so results are bit-identical run to run.
+//
+// Gradient conventions reproduced from autograd over the reference's torch ops:
+//   PPO-clip   d/dlp = -A*r when r is inside [1-eps_lo, 1+eps_hi] or the unclipped branch is strictly larger, else 0
+//   dual clip  A<0 and -c*A < clipped loss: 0; tie: half
+//   CISPO      -coef*A (coef, A detached);  RLOO  -A;  SAPO  -A*4*s*(1-s)*r  (s = sigmoid(tau*(r-1)))
+//   k1: 1   k2: d   k3 / low_var: 1-exp(-d)  (low_var: 0 outside the [-10,10] clamp)
+//   unbiased KL multiplies by ratio = exp(lp-old) and adds ratio*kl (the ratio is not detached, loss.py:1091)
+#include "device_utils.h"
+#include "relax_amd.h"
+
+namespace relax_amd {
+
+constexpr int kLossThreads = 512;
+
+struct TokenTerms {
+  float pg, clipfrac, ppo_kl, dpg_dlp, dpg_dkl;
+};
+
+// One token of compute_policy_loss / compute_cispo_loss / compute_rloo_loss / compute_sapo_loss.
+// `kl` is old - lp (token-level) or the sequence KL (GSPO).  dpg_dlp is the derivative through a token-level kl
+// (d kl / d lp = -1) plus any direct lp dependence; dpg_dkl is the derivative w.r.t. kl itself (used by GSPO).
+__device__ __forceinline__ TokenTerms token_loss(int kind, float lp, float kl, float adv, float eps_lo, float eps_hi,
+                                                 float eps_c, float tau_pos, float tau_neg) {
+  TokenTerms t;
+  t.ppo_kl = kl;
+  const float r = expf(-kl);
+  if (kind == RELAX_AMD_LOSS_CISPO) {
+    const float hi = 1.0f + eps_hi, lo = 1.0f - eps_lo;
+    const float coef = adv >= 0.f ? fminf(r, hi) : fmaxf(r, lo);
+    t.pg = -(coef * adv * lp);
+    t.clipfrac = ((adv >= 0.f && r > hi) ? 1.f : 0.f) + ((adv < 0.f && r < lo) ? 1.f : 0.f);
+    t.dpg_dlp = -(coef * adv);
+    t.dpg_dkl = 0.f;
+    return t;
+  }
+  if (kind == RELAX_AMD_LOSS_RLOO) {
+    t.pg = -(adv * lp);
+    t.clipfrac = 0.f;
+    t.dpg_dlp = -adv;
+    t.dpg_dkl = 0.f;
+    return t;
+  }
+  if (kind == RELAX_AMD_LOSS_SAPO) {
+    const float tau = adv > 0.f ? tau_pos : tau_neg;
+    const float s = 1.0f / (1.0f + expf(-tau * (r - 1.0f)));
+    t.pg = -((4.0f / tau) * s * adv);
+    t.clipfrac = (4.0f * s * (1.0f - s)) < 0.9f ? 1.f : 0.f;
+    // d pg / d r = -(4/tau)*adv*tau*s*(1-s);  d r / d kl = -r
+    t.dpg_dkl = 4.0f * adv * s * (1.0f - s) * r;
+    t.dpg_dlp = -t.dpg_dkl;
+    return t;
+  }
+  // PPO clip (also the per-token function GSPO applies to the sequence KL)
+  const float lo = 1.0f - eps_lo, hi = 1.0f + eps_hi;
+  const float l1 = -r * adv;
+  const float rc = fminf(fmaxf(r, lo), hi);
+  const float l2 = -rc * adv;
+  float loss = fmaxf(l1, l2);
+  t.clipfrac = l2 > l1 ? 1.f : 0.f;
+  const bool inside = (r >= lo) && (r <= hi);
+  float dl_dr = (inside || l1 > l2) ? -adv : 0.f;  // ties outside the range only occur at adv == 0
+  if (eps_c > 0.f && adv < 0.f) {
+    const float l3 = -eps_c * adv;
+    if (l3 < loss) {
+      loss = l3;
+      dl_dr = 0.f;
+    } else if (l3 == loss) {
+      dl_dr *= 0.5f;
+    }
+  }
+  t.pg = loss;
+  t.dpg_dkl = -dl_dr * r;  // d r / d kl = -r
+  t.dpg_dlp = dl_dr * r;
+  return t;
+}
+
+__device__ __forceinline__ void kl_term(int kind, float lp, float ref, float& kl, float& dkl_dlp) {
+  const float d = lp - ref;
+  if (kind == RELAX_AMD_KL_K1) {
+    kl = d;
+    dkl_dlp = 1.f;
+  } else if (kind == RELAX_AMD_KL_K2) {
+    kl = d * d / 2.0f;
+    dkl_dlp = d;
+  } else {
+    const float e = expf(-d);
+    kl = e - 1.0f - (-d);
+    dkl_dlp = 1.0f - e;
+  }
+}
+
+__global__ __launch_bounds__(kLossThreads) void policy_loss_sample_kernel(relax_amd_policy_loss_args a) {
+  __shared__ float red[kLossThreads / kWave];
+  const int64_t i = blockIdx.x;
+  const int64_t beg = a.cu_resp[i], end = a.cu_resp[i + 1];
+  const bool gspo = a.loss_kind == RELAX_AMD_LOSS_GSPO;
+  const int kind = gspo ? RELAX_AMD_LOSS_PPO : a.loss_kind;
+  const float den = a.sample_denom ? a.sample_denom[i] : 1.0f;
+  const float pg_den = a.pg_sample_denom ? a.pg_sample_denom[i] : den;
+  const float* pg_mask = a.pg_loss_mask ? a.pg_loss_mask : a.loss_mask;
+
+  float seq_kl = 0.f, seq_cnt = 1.f;
+  if (gspo || a.use_opsm) {
+    float sd = 0.f, sm = 0.f;
+    for (int64_t t = beg + threadIdx.x; t < end; t += kLossThreads) {
+      const float lp = a.log_prob[t];
+      const float old = a.old_log_prob ? a.old_log_prob[t] : lp;
+      const float m = a.loss_mask[t];
+      sd += (old - lp) * m;
+      sm += m;
+    }
+    sd = block_sum<kLossThreads>(sd, red);
+    sm = block_sum<kLossThreads>(sm, red);
+    seq_cnt = fmaxf(sm, 1.0f);
+    seq_kl = sd / seq_cnt;
+  }
+
+  float acc[RELAX_AMD_NUM_METRICS];
+#pragma unroll
+  for (int k = 0; k < RELAX_AMD_NUM_METRICS; ++k) acc[k] = 0.f;
+  float g_seq = 0.f;  // GSPO: sum_t w_t * d pg_t / d kl_i
+
+  for (int64_t t = beg + threadIdx.x; t < end; t += kLossThreads) {
+    const float lp = a.log_prob[t];
+    const float old = a.old_log_prob ? a.old_log_prob[t] : lp;
+    const float adv = a.advantages[t];
+    const float m = a.loss_mask[t];
+    const float mp = pg_mask[t];
+    const float kl_in = gspo ? seq_kl : (old - lp);
+    TokenTerms tt = token_loss(kind, lp, kl_in, adv, a.eps_clip, a.eps_clip_high, a.eps_clip_c, a.tau_pos, a.tau_neg);
+    float w = 1.0f;  // multiplicative, gradient-free weights on pg_loss
+    float drop = 0.f;
+    if (a.use_opsm) {
+      drop = (adv < 0.f && seq_kl > a.opsm_delta) ? 1.f : 0.f;
+      w *= 1.0f - drop;
+    }
+    float tis = 0.f, log_ratio = 0.f, tis_w = 1.f;
+    const bool have_tis = (a.use_tis || a.mismatch_metrics) && a.rollout_log_prob;
+    if (have_tis) {
+      log_ratio = (a.train_log_prob ? a.train_log_prob[t] : lp) - a.rollout_log_prob[t];
+      tis = expf(log_ratio);
+      tis_w = fminf(fmaxf(tis, a.tis_lo), a.tis_hi);
+      w *= tis_w;
+    }
+    const float pg = tt.pg * w;
+    float c_lp = (mp / pg_den) * w * (gspo ? 0.f : tt.dpg_dlp);
+    if (gspo) g_seq += (mp / pg_den) * w * tt.dpg_dkl;
+
+    acc[RELAX_AMD_M_PG_LOSS] += pg * mp;
+    acc[RELAX_AMD_M_CLIPFRAC] += tt.clipfrac * m;
+    acc[RELAX_AMD_M_PPO_KL] += tt.ppo_kl * m;
+    acc[RELAX_AMD_M_MASK_SUM] += m;
+    if (a.entropy) acc[RELAX_AMD_M_ENTROPY] += a.entropy[t] * m;
+    if (a.pg_loss_tok) a.pg_loss_tok[t] = pg;
+    if (a.clipfrac_tok) a.clipfrac_tok[t] = tt.clipfrac;
+    if (a.ppo_kl_tok) a.ppo_kl_tok[t] = tt.ppo_kl;
+
+    if (a.kl_kind != RELAX_AMD_KL_NONE) {
+      float kl, dkl;
+      kl_term(a.kl_kind, lp, a.ref_log_prob[t], kl, dkl);
+      if (a.unbiased_kl) {
+        const float ratio = expf(lp - old);
+        dkl = ratio * dkl + ratio * kl;  // ratio carries gradient (d ratio / d lp = ratio)
+        kl = ratio * kl;
+      }
+      if (a.kl_kind == RELAX_AMD_KL_LOW_VAR) {
+        if (kl < -10.f || kl > 10.f) dkl = 0.f;
+        kl = fminf(fmaxf(kl, -10.f), 10.f);
+      }
+      acc[RELAX_AMD_M_KL_LOSS] += kl * m;
+      c_lp += a.kl_coef * (m / den) * dkl;
+      if (a.kl_tok) a.kl_tok[t] = kl;
+    }
+    if (a.rollout_log_prob) {
+      const float roll = a.rollout_log_prob[t];
+      float side = lp;
+      if (a.abs_diff_from_old == 1) side = old;
+      else if (a.abs_diff_from_old == 0 && a.train_log_prob) side = a.train_log_prob[t];
+      acc[RELAX_AMD_M_LOGPROB_ABS_DIFF] += fabsf(side - roll) * m;
+      acc[RELAX_AMD_M_PROB_ABS_DIFF] += fabsf(expf(side) - expf(roll)) * m;
+    }
+    if (have_tis) {
+      acc[RELAX_AMD_M_OIS] += expf(-tt.ppo_kl) * m;
+      acc[RELAX_AMD_M_TIS] += tis * m;
+      acc[RELAX_AMD_M_TIS_CLIPFRAC] += (tis_w != tis ? 1.f : 0.f) * m;
+      acc[RELAX_AMD_M_TIS_ABS] += fabsf(tis - 1.0f) * m;
+      acc[RELAX_AMD_M_MISMATCH_KL] += (-log_ratio) * m;
+      acc[RELAX_AMD_M_MISMATCH_K3] += (tis - log_ratio - 1.0f) * m;
+    }
+    acc[RELAX_AMD_M_OPSM_CLIPFRAC] += drop;
+    a.coef_log_prob[t] = c_lp;
+    if (a.coef_entropy) a.coef_entropy[t] = -a.entropy_coef * (m / den);
+  }
+
+#pragma unroll
+  for (int k = 0; k < RELAX_AMD_NUM_METRICS; ++k) acc[k] = block_sum<kLossThreads>(acc[k], red);
+  if (gspo) {
+    g_seq = block_sum<kLossThreads>(g_seq, red);
+    // d kl_i / d lp_t = -m_t / max(sum m, 1)
+    for (int64_t t = beg + threadIdx.x; t < end; t += kLossThreads)
+      a.coef_log_prob[t] += g_seq * (-a.loss_mask[t] / seq_cnt);
+  }
+  if (threadIdx.x == 0) {
+    float* out = a.sample_partials + i * RELAX_AMD_NUM_METRICS;
+    out[RELAX_AMD_M_LOSS] = 0.f;
+    out[RELAX_AMD_M_PG_LOSS] = acc[RELAX_AMD_M_PG_LOSS] / pg_den;
+    out[RELAX_AMD_M_MASK_SUM] = acc[RELAX_AMD_M_MASK_SUM];
+    // opsm_clipfrac: dropped-token count over max(sum m, 1) of the sample (ppo_utils.py:175)
+    out[RELAX_AMD_M_OPSM_CLIPFRAC] = acc[RELAX_AMD_M_OPSM_CLIPFRAC] / fmaxf(acc[RELAX_AMD_M_MASK_SUM], 1.0f);
+#pragma unroll
+    for (int k = RELAX_AMD_M_ENTROPY; k <= RELAX_AMD_M_MISMATCH_K3; ++k) out[k] = acc[k] / den;
+  }
+}
+
+__global__ __launch_bounds__(kWave) void policy_loss_finish_kernel(const float* __restrict__ partials,
+                                                                   int64_t n_samples, float entropy_coef,
+                                                                   float kl_coef, int has_kl,
+                                                                   float* __restrict__ metrics) {
+  const int k = threadIdx.x;
+  float total = 0.f;
+  if (k < RELAX_AMD_NUM_METRICS)
+    for (int64_t i = 0; i < n_samples; ++i) total += partials[i * RELAX_AMD_NUM_METRICS + k];
+  const float pg = __shfl(total, RELAX_AMD_M_PG_LOSS, kWave);
+  const float ent = __shfl(total, RELAX_AMD_M_ENTROPY, kWave);
+  const float kl = __shfl(total, RELAX_AMD_M_KL_LOSS, kWave);
+  if (k == RELAX_AMD_M_LOSS) {
+    total = pg - entropy_coef * ent;
+    if (has_kl) total = total + kl_coef * kl;
+  }
+  if (k < RELAX_AMD_NUM_METRICS) metrics[k] = total;
+}
+
+__global__ __launch_bounds__(256) void segment_sum_kernel(const float* __restrict__ values,
+                                                          const float* __restrict__ mask,
+                                                          const int64_t* __restrict__ cu, double* __restrict__ out) {
+  __shared__ double red[256 / kWave];
+  const int64_t i = blockIdx.x;
+  double s = 0.0;
+  for (int64_t t = cu[i] + threadIdx.x; t < cu[i + 1]; t += 256)
+    s += values ? double(values[t] * mask[t]) : double(mask[t]);
+  s = block_sum<256>(s, red);
+  if (threadIdx.x == 0) out[i] = s;
+}
+
+__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* __restrict__ p, int64_t n, int32_t v) {
+  for (int64_t i = blockIdx.x * 256LL + threadIdx.x; i < n; i += int64_t(gridDim.x) * 256) p[i] = v;
+}
+
+__global__ __launch_bounds__(256) void row_maps_kernel(const int64_t* __restrict__ row_begin,
+                                                       const int64_t* __restrict__ cu, int64_t n_rows,
+                                                       int32_t* __restrict__ row_ids, int32_t* __restrict__ sample_ids,
+                                                       int32_t* __restrict__ token_of_row) {
+  const int64_t i = blockIdx.x;
+  const int64_t beg = cu[i], len = cu[i + 1] - cu[i], r0 = row_begin[i];
+  for (int64_t j = threadIdx.x; j < len; j += 256) {
+    const int64_t row = r0 + j;
+    row_ids[beg + j] = int32_t(row);
+    if (sample_ids) sample_ids[beg + j] = int32_t(i);
+    if (token_of_row && row >= 0 && row < n_rows) token_of_row[row] = int32_t(beg + j);
+  }
+}
+
+}  // namespace relax_amd
+
+using namespace relax_amd;
+
+extern "C" int relax_amd_policy_loss(const relax_amd_policy_loss_args* a, void* stream) {
+  if (!a) {
+    set_error("policy_loss: args is NULL");
+    return RELAX_AMD_EINVAL;
+  }
+  if (a->n_samples < 0 || a->n_tokens < 0 || a->n_samples > 2147483647LL) {
+    set_error("policy_loss: bad sizes n_samples=%lld n_tokens=%lld", (long long)a->n_samples, (long long)a->n_tokens);
+    return RELAX_AMD_EINVAL;
+  }
+  if (!a->metrics || !a->sample_partials || !a->cu_resp) {
+    set_error("policy_loss: metrics, sample_partials and cu_resp must not be NULL");
+    return RELAX_AMD_EINVAL;
+  }
+  if (a->n_tokens > 0 && (!a->log_prob || !a->advantages || !a->loss_mask || !a->coef_log_prob)) {
+    set_error("policy_loss: log_prob, advantages, loss_mask and coef_log_prob must not be NULL");
+    return RELAX_AMD_EINVAL;
+  }
+  if (a->loss_kind < RELAX_AMD_LOSS_PPO || a->loss_kind > RELAX_AMD_LOSS_SAPO) {
+    set_error("policy_loss: unknown loss_kind %d", a->loss_kind);
+    return RELAX_AMD_EINVAL;
+  }
+  if (a->kl_kind < RELAX_AMD_KL_NONE || a->kl_kind > RELAX_AMD_KL_LOW_VAR) {
+    set_error("policy_loss: unknown kl_kind %d", a->kl_kind);
+    return RELAX_AMD_EINVAL;
+  }
+  if (a->kl_kind != RELAX_AMD_KL_NONE && a->n_tokens > 0 && !a->ref_log_prob) {
+    set_error("policy_loss: ref_log_prob is required when kl_kind != NONE");
+    return RELAX_AMD_EINVAL;
+  }
+  if (a->eps_clip_c > 0.f && !(a->eps_clip_c > 1.0f)) {
+    set_error("policy_loss: eps_clip_c must be > 1.0 (got %f)", a->eps_clip_c);
+    return RELAX_AMD_EINVAL;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (a->n_samples > 0) {
+    hipLaunchKernelGGL(policy_loss_sample_kernel, dim3(static_cast<unsigned>(a->n_samples)), dim3(kLossThreads), 0, s,
+                       *a);
+    int rc = check_launch("policy_loss_sample");
+    if (rc) return rc;
+  }
+  hipLaunchKernelGGL(policy_loss_finish_kernel, dim3(1), dim3(kWave), 0, s, a->sample_partials, a->n_samples,
+                     a->entropy_coef, a->kl_coef, int(a->kl_kind != RELAX_AMD_KL_NONE), a->metrics);
+  return check_launch("policy_loss_finish");
+}
+
+extern "C" int relax_amd_segment_sum(const float* values, const float* mask, const int64_t* cu_resp, int64_t n_samples,
+                                     double* out, void* stream) {
+  if (n_samples < 0 || n_samples > 2147483647LL) {
+    set_error("segment_sum: bad n_samples %lld", (long long)n_samples);
+    return RELAX_AMD_EINVAL;
+  }
+  if (n_samples == 0) return RELAX_AMD_OK;
+  if (!mask || !cu_resp || !out) {
+    set_error("segment_sum: mask, cu_resp and out must not be NULL");
+    return RELAX_AMD_EINVAL;
+  }
+  hipLaunchKernelGGL(segment_sum_kernel, dim3(static_cast<unsigned>(n_samples)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), values, mask, cu_resp, out);
+  return check_launch("segment_sum");
+}
+
+extern "C" int relax_amd_build_row_maps(const int64_t* row_begin, const int64_t* cu_resp, int64_t n_samples,
+                                        int64_t n_tokens, int64_t n_rows, int32_t* row_ids, int32_t* sample_ids,
+                                        int32_t* token_of_row, void* stream) {
+  if (n_samples < 0 || n_tokens < 0 || n_rows < 0 || n_rows > 2147483647LL || n_tokens > 2147483647LL ||
+      n_samples > 2147483647LL) {
+    set_error("build_row_maps: bad sizes");
+    return RELAX_AMD_EINVAL;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (token_of_row && n_rows > 0) {
+    const unsigned blocks = static_cast<unsigned>((n_rows + 255) / 256 > 4096 ? 4096 : (n_rows + 255) / 256);
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(blocks), dim3(256), 0, s, token_of_row, n_rows, int32_t(-1));
+    int rc = check_launch("fill_i32");
+    if (rc) return rc;
+  }
+  if (n_samples == 0 || n_tokens == 0) return RELAX_AMD_OK;
+  if (!row_begin || !cu_resp || !row_ids) {
+    set_error("build_row_maps: row_begin, cu_resp and row_ids must not be NULL");
+    return RELAX_AMD_EINVAL;
+  }
+  hipLaunchKernelGGL(row_maps_kernel, dim3(static_cast<unsigned>(n_samples)), dim3(256), 0, s, row_begin, cu_resp,
+                     n_rows, row_ids, sample_ids, token_of_row);
+  return check_launch("row_maps");
+}

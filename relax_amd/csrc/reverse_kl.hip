@@ -1,0 +1,294 @@
+// Full-vocab reverse KL(student || teacher) per token and its gradient w.r.t. the student logits.
+//
+// Forward: one workgroup per token streams the student row and the teacher row together (16-byte non-temporal
+// loads) and keeps two online-softmax states per lane:  (m_s, sum e_s, sum e_s*(x_s - x_t))  and  (m_t, sum e_t).
+//   KL = sum_v p_s*(log p_s - log p_t) = sum_v p_s*(x_s - x_t) - lse_s + lse_t
+// which is what the jsd_alpha == 0 branch of compute_opd_kl (relax/utils/opd/opd_utils.py:1165-1169) evaluates when
+// its [R, K] inputs are complete log-softmax rows (K = vocab; the tail bin then carries zero mass).
+// Backward: d KL / d x_s[v] = p_s[v] * ((log p_s[v] - log p_t[v]) - KL); reads both rows once, writes one.
+#include "device_utils.h"
+#include "relax_amd.h"
+
+namespace relax_amd {
+
+constexpr int kKlThreads = 256;
+constexpr int kKlUnroll = 2;
+
+struct KlState {
+  float ms, ss, us, mt, st;
+};
+
+template <int K>
+__device__ __forceinline__ void absorb_pair(const float (&xs)[K], const float (&xt)[K], KlState& q) {
+  float smax = xs[0], tmax = xt[0];
+#pragma unroll
+  for (int i = 1; i < K; ++i) {
+    smax = fmaxf(smax, xs[i]);
+    tmax = fmaxf(tmax, xt[i]);
+  }
+  const float sm = smax * kLog2e, tm = tmax * kLog2e;
+  if (sm > q.ms) {
+    const float sc = fast_exp2(q.ms - sm);
+    q.ss *= sc;
+    q.us *= sc;
+    q.ms = sm;
+  }
+  if (tm > q.mt) {
+    q.st *= fast_exp2(q.mt - tm);
+    q.mt = tm;
+  }
+#pragma unroll
+  for (int i = 0; i < K; ++i) {
+    const float es = fast_exp2(fmaf(xs[i], kLog2e, -q.ms));
+    const float et = fast_exp2(fmaf(xt[i], kLog2e, -q.mt));
+    q.ss += es;
+    q.us = fmaf(es, xs[i] - xt[i], q.us);
+    q.st += et;
+  }
+}
+
+__device__ __forceinline__ void merge_kl(KlState& a, const KlState& b) {
+  const float ms = fmaxf(a.ms, b.ms), mt = fmaxf(a.mt, b.mt);
+  const float fa = fast_exp2(a.ms - ms), fb = fast_exp2(b.ms - ms);
+  a.ss = a.ss * fa + b.ss * fb;
+  a.us = a.us * fa + b.us * fb;
+  a.st = a.st * fast_exp2(a.mt - mt) + b.st * fast_exp2(b.mt - mt);
+  a.ms = ms;
+  a.mt = mt;
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kKlThreads) void reverse_kl_fwd_kernel(const T* __restrict__ student,
+                                                                    const T* __restrict__ teacher, int64_t stride,
+                                                                    int64_t vocab, float* __restrict__ kl,
+                                                                    float* __restrict__ lse_s,
+                                                                    float* __restrict__ lse_t) {
+  __shared__ float lds[kKlThreads / kWave][5];
+  const int64_t tok = blockIdx.x;
+  const T* xs = student + tok * stride;
+  const T* xt = teacher + tok * stride;
+  KlState q{kNegHuge, 0.f, 0.f, kNegHuge, 0.f};
+  if (VEC) {
+    constexpr int VN = Row<T>::kPerVec;
+    const u32x4* sv = reinterpret_cast<const u32x4*>(xs);
+    const u32x4* tv = reinterpret_cast<const u32x4*>(xt);
+    const int64_t nvec = vocab / VN;
+    int64_t i = threadIdx.x;
+    for (; i + int64_t(kKlUnroll - 1) * kKlThreads < nvec; i += int64_t(kKlUnroll) * kKlThreads) {
+      u32x4 rs[kKlUnroll], rt[kKlUnroll];
+#pragma unroll
+      for (int u = 0; u < kKlUnroll; ++u) {
+        rs[u] = load_stream(sv + i + int64_t(u) * kKlThreads);
+        rt[u] = load_stream(tv + i + int64_t(u) * kKlThreads);
+      }
+      float a[kKlUnroll * VN], b[kKlUnroll * VN];
+#pragma unroll
+      for (int u = 0; u < kKlUnroll; ++u) {
+        float pa[VN], pb[VN];
+        Row<T>::unpack(rs[u], pa);
+        Row<T>::unpack(rt[u], pb);
+#pragma unroll
+        for (int k = 0; k < VN; ++k) {
+          a[u * VN + k] = pa[k];
+          b[u * VN + k] = pb[k];
+        }
+      }
+      absorb_pair(a, b, q);
+    }
+    for (; i < nvec; i += kKlThreads) {
+      float a[VN], b[VN];
+      Row<T>::unpack(load_stream(sv + i), a);
+      Row<T>::unpack(load_stream(tv + i), b);
+      absorb_pair(a, b, q);
+    }
+    for (int64_t e = nvec * VN + threadIdx.x; e < vocab; e += kKlThreads) {
+      float a[1] = {Row<T>::load1(xs + e)}, b[1] = {Row<T>::load1(xt + e)};
+      absorb_pair(a, b, q);
+    }
+  } else {
+    for (int64_t e = threadIdx.x; e < vocab; e += kKlThreads) {
+      float a[1] = {Row<T>::load1(xs + e)}, b[1] = {Row<T>::load1(xt + e)};
+      absorb_pair(a, b, q);
+    }
+  }
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    KlState other{__shfl_xor(q.ms, o, kWave), __shfl_xor(q.ss, o, kWave), __shfl_xor(q.us, o, kWave),
+                  __shfl_xor(q.mt, o, kWave), __shfl_xor(q.st, o, kWave)};
+    merge_kl(q, other);
+  }
+  const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+  if (lane == 0) {
+    lds[w][0] = q.ms;
+    lds[w][1] = q.ss;
+    lds[w][2] = q.us;
+    lds[w][3] = q.mt;
+    lds[w][4] = q.st;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int k = 1; k < kKlThreads / kWave; ++k) {
+      KlState other{lds[k][0], lds[k][1], lds[k][2], lds[k][3], lds[k][4]};
+      merge_kl(q, other);
+    }
+    const float ls = q.ms * kLn2 + logf(q.ss);
+    const float lt = q.mt * kLn2 + logf(q.st);
+    kl[tok] = q.us / q.ss - ls + lt;
+    lse_s[tok] = ls;
+    lse_t[tok] = lt;
+  }
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kKlThreads) void reverse_kl_bwd_kernel(
+    const T* __restrict__ student, const T* __restrict__ teacher, int64_t stride, int64_t vocab,
+    const float* __restrict__ kl, const float* __restrict__ lse_s, const float* __restrict__ lse_t,
+    const float* __restrict__ g, float grad_scale, const float* __restrict__ grad_scale_dev,
+    T* __restrict__ dstudent) {
+  const int64_t tok = blockIdx.x;
+  T* d = dstudent + tok * stride;
+  if (grad_scale_dev) grad_scale *= *grad_scale_dev;
+  const float gt = g[tok] * grad_scale;
+  if (gt == 0.f) {
+    if (VEC) {
+      constexpr int VN = Row<T>::kPerVec;
+      const int64_t nvec = vocab / VN;
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      for (int64_t i = threadIdx.x; i < nvec; i += kKlThreads) store_stream(reinterpret_cast<u32x4*>(d) + i, z);
+      for (int64_t e = nvec * VN + threadIdx.x; e < vocab; e += kKlThreads) Row<T>::store1(d + e, 0.f);
+    } else {
+      for (int64_t e = threadIdx.x; e < vocab; e += kKlThreads) Row<T>::store1(d + e, 0.f);
+    }
+    return;
+  }
+  const T* xs = student + tok * stride;
+  const T* xt = teacher + tok * stride;
+  const float k0 = -lse_s[tok] * kLog2e;
+  const float k1 = gt * (lse_t[tok] - lse_s[tok] - kl[tok]);
+  // d = p_s * g * ((x_s - x_t) + lse_t - lse_s - KL)
+  if (VEC) {
+    constexpr int VN = Row<T>::kPerVec;
+    const u32x4* sv = reinterpret_cast<const u32x4*>(xs);
+    const u32x4* tv = reinterpret_cast<const u32x4*>(xt);
+    u32x4* dv = reinterpret_cast<u32x4*>(d);
+    const int64_t nvec = vocab / VN;
+    int64_t i = threadIdx.x;
+    for (; i + int64_t(kKlUnroll - 1) * kKlThreads < nvec; i += int64_t(kKlUnroll) * kKlThreads) {
+      u32x4 rs[kKlUnroll], rt[kKlUnroll];
+#pragma unroll
+      for (int u = 0; u < kKlUnroll; ++u) {
+        rs[u] = load_stream(sv + i + int64_t(u) * kKlThreads);
+        rt[u] = load_stream(tv + i + int64_t(u) * kKlThreads);
+      }
+#pragma unroll
+      for (int u = 0; u < kKlUnroll; ++u) {
+        float a[VN], b[VN];
+        Row<T>::unpack(rs[u], a);
+        Row<T>::unpack(rt[u], b);
+#pragma unroll
+        for (int k = 0; k < VN; ++k) a[k] = fast_exp2(fmaf(a[k], kLog2e, k0)) * fmaf(a[k] - b[k], gt, k1);
+        store_stream(dv + i + int64_t(u) * kKlThreads, Row<T>::pack(a));
+      }
+    }
+    for (; i < nvec; i += kKlThreads) {
+      float a[VN], b[VN];
+      Row<T>::unpack(load_stream(sv + i), a);
+      Row<T>::unpack(load_stream(tv + i), b);
+#pragma unroll
+      for (int k = 0; k < VN; ++k) a[k] = fast_exp2(fmaf(a[k], kLog2e, k0)) * fmaf(a[k] - b[k], gt, k1);
+      store_stream(dv + i, Row<T>::pack(a));
+    }
+    for (int64_t e = nvec * VN + threadIdx.x; e < vocab; e += kKlThreads) {
+      const float a = Row<T>::load1(xs + e), b = Row<T>::load1(xt + e);
+      Row<T>::store1(d + e, fast_exp2(fmaf(a, kLog2e, k0)) * fmaf(a - b, gt, k1));
+    }
+  } else {
+    for (int64_t e = threadIdx.x; e < vocab; e += kKlThreads) {
+      const float a = Row<T>::load1(xs + e), b = Row<T>::load1(xt + e);
+      Row<T>::store1(d + e, fast_exp2(fmaf(a, kLog2e, k0)) * fmaf(a - b, gt, k1));
+    }
+  }
+}
+
+template <typename T>
+static int launch_kl_fwd(const void* s, const void* t, int64_t n, int64_t vocab, int64_t stride, float* kl,
+                         float* ls, float* lt, hipStream_t st) {
+  const bool vec = aligned16(s) && aligned16(t) && (stride * int64_t(sizeof(T))) % 16 == 0;
+  dim3 grid(static_cast<unsigned>(n)), block(kKlThreads);
+  if (vec)
+    hipLaunchKernelGGL((reverse_kl_fwd_kernel<T, true>), grid, block, 0, st, static_cast<const T*>(s),
+                       static_cast<const T*>(t), stride, vocab, kl, ls, lt);
+  else
+    hipLaunchKernelGGL((reverse_kl_fwd_kernel<T, false>), grid, block, 0, st, static_cast<const T*>(s),
+                       static_cast<const T*>(t), stride, vocab, kl, ls, lt);
+  return check_launch("reverse_kl_fwd");
+}
+
+template <typename T>
+static int launch_kl_bwd(const void* s, const void* t, int64_t n, int64_t vocab, int64_t stride, const float* kl,
+                         const float* ls, const float* lt, const float* g, float scale, const float* scale_dev,
+                         void* d, hipStream_t st) {
+  const bool vec = aligned16(s) && aligned16(t) && aligned16(d) && (stride * int64_t(sizeof(T))) % 16 == 0;
+  dim3 grid(static_cast<unsigned>(n)), block(kKlThreads);
+  if (vec)
+    hipLaunchKernelGGL((reverse_kl_bwd_kernel<T, true>), grid, block, 0, st, static_cast<const T*>(s),
+                       static_cast<const T*>(t), stride, vocab, kl, ls, lt, g, scale, scale_dev, static_cast<T*>(d));
+  else
+    hipLaunchKernelGGL((reverse_kl_bwd_kernel<T, false>), grid, block, 0, st, static_cast<const T*>(s),
+                       static_cast<const T*>(t), stride, vocab, kl, ls, lt, g, scale, scale_dev, static_cast<T*>(d));
+  return check_launch("reverse_kl_bwd");
+}
+
+}  // namespace relax_amd
+
+using namespace relax_amd;
+
+static int kl_check(const char* what, int64_t n, int64_t vocab, int64_t stride) {
+  if (n < 0 || n > 2147483647LL || vocab <= 0 || stride < vocab) {
+    set_error("%s: bad shape n_tokens=%lld vocab=%lld row_stride=%lld", what, (long long)n, (long long)vocab,
+              (long long)stride);
+    return RELAX_AMD_EINVAL;
+  }
+  return RELAX_AMD_OK;
+}
+
+extern "C" int relax_amd_reverse_kl_fwd(const void* student, const void* teacher, int dtype, int64_t n_tokens,
+                                        int64_t vocab, int64_t row_stride, float* kl, float* lse_s, float* lse_t,
+                                        void* stream) {
+  if (int rc = kl_check("reverse_kl_fwd", n_tokens, vocab, row_stride)) return rc;
+  if (n_tokens == 0) return RELAX_AMD_OK;
+  if (!student || !teacher || !kl || !lse_s || !lse_t) {
+    set_error("reverse_kl_fwd: NULL argument");
+    return RELAX_AMD_EINVAL;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case RELAX_AMD_F32: return launch_kl_fwd<float>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, s);
+    case RELAX_AMD_BF16: return launch_kl_fwd<bf16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, s);
+    case RELAX_AMD_F16: return launch_kl_fwd<f16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, s);
+    default: set_error("reverse_kl_fwd: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
+  }
+}
+
+extern "C" int relax_amd_reverse_kl_bwd(const void* student, const void* teacher, int dtype, int64_t n_tokens,
+                                        int64_t vocab, int64_t row_stride, const float* kl, const float* lse_s,
+                                        const float* lse_t, const float* g, float grad_scale,
+                                        const float* grad_scale_dev, void* dstudent, void* stream) {
+  if (int rc = kl_check("reverse_kl_bwd", n_tokens, vocab, row_stride)) return rc;
+  if (n_tokens == 0) return RELAX_AMD_OK;
+  if (!student || !teacher || !kl || !lse_s || !lse_t || !g || !dstudent) {
+    set_error("reverse_kl_bwd: NULL argument");
+    return RELAX_AMD_EINVAL;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case RELAX_AMD_F32:
+      return launch_kl_bwd<float>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, g, grad_scale, grad_scale_dev, dstudent, s);
+    case RELAX_AMD_BF16:
+      return launch_kl_bwd<bf16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, g, grad_scale, grad_scale_dev, dstudent, s);
+    case RELAX_AMD_F16:
+      return launch_kl_bwd<f16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, g, grad_scale, grad_scale_dev, dstudent, s);
+    default: set_error("reverse_kl_bwd: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
+  }
+}

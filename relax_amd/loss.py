@@ -1,0 +1,355 @@
+"""Drop-in counterparts of the hot-path functions of ``relax/backends/megatron/loss.py`` at context-parallel
+size 1 in the packed ("thd") layout, running on the gfx950 kernels.
+
+Reference lines (paths relative to the reference checkout):
+  get_responses                   relax/backends/megatron/loss.py:49-191
+  get_log_probs_and_entropy       :290-463
+  compute_advantages_and_returns  :532-738
+  policy_loss_function            :824-1185
+  loss_function                   :1443-1620
+
+Where the reference loops over samples in Python and runs ~10 full [R, V] fp32 passes per sample, these functions
+build the packed row maps once and issue one forward launch and one backward launch for the whole micro-batch.
+``policy_loss_function`` is usable as ``--loss-type custom_loss --custom-loss-function-path
+relax_amd.loss.policy_loss_function``; ``get_log_probs_and_entropy`` as the ``f`` of ``forward_only``.
+"""
+
+from __future__ import annotations
+
+from argparse import Namespace
+from collections.abc import Iterator
+from typing import Any
+
+import torch
+
+from . import ops
+from ._lib import METRIC_SLOTS
+from .cp_utils import get_cp_local_num_tokens, get_sum_of_sample_mean, sample_denominators
+from .ppo_utils import get_grpo_returns
+
+_SLOT = {k: i for i, k in enumerate(METRIC_SLOTS)}
+GRPO_FAMILY = ("grpo", "gspo", "sapo", "cispo", "m2po", "rloo")
+
+
+def _check_logits(logits: torch.Tensor, args) -> torch.Tensor:
+    """[1, T, V] -> [T, V].  fp32 is what stock Megatron hands over; bf16 / fp16 logits are accepted as well."""
+    assert logits.dtype in (torch.float32, torch.bfloat16, torch.float16), f"{logits.dtype}"
+    assert len(logits.shape) == 3, f"{logits.shape}"
+    if getattr(args, "qkv_format", "thd") != "thd":
+        raise NotImplementedError("relax_amd handles the packed 'thd' layout only")
+    assert logits.size(0) == 1, f"{logits.shape}"
+    return logits.squeeze(0)
+
+
+def response_row_begins(total_lengths, response_lengths) -> tuple[list[int], list[bool]]:
+    """First logits row of each sample's response (loss.py:103-125): RL samples are scored by the previous
+    position's logits (start - 1); the SFT convention (response == total) uses start (sft_utils.py:23-40)."""
+    begins, sft = [], []
+    end = 0
+    for total, resp in zip(total_lengths, response_lengths, strict=False):
+        end += total
+        start = end - resp
+        is_sft = resp == total
+        begins.append(start if is_sft else start - 1)
+        sft.append(is_sft)
+    return begins, sft
+
+
+def get_responses(
+    logits: torch.Tensor,
+    *,
+    args: Namespace,
+    unconcat_tokens: list[torch.Tensor],
+    total_lengths: list[int],
+    response_lengths: list[int],
+    max_seq_lens=None,
+    padded_total_lengths=None,
+    apply_temperature: bool = True,
+    dynamic_cp_size=None,
+    dynamic_cp_rank=None,
+) -> Iterator[tuple[torch.Tensor, torch.Tensor]]:
+    """Yields per-sample ``(logits rows [R, V], target ids [R])`` views.  Kept for callers that want the slices;
+    the fused functions below do not iterate samples.  Temperature is applied per chunk like the reference."""
+    flat = _check_logits(logits, args)
+    begins, sft = response_row_begins(total_lengths, response_lengths)
+    for b, is_sft, toks, resp in zip(begins, sft, unconcat_tokens, response_lengths, strict=False):
+        chunk = flat[b : b + resp]
+        targets = torch.nn.functional.pad(toks[1:], (0, 1), value=0) if is_sft else toks[-resp:]
+        if apply_temperature and args.rollout_temperature != 1.0:
+            chunk = chunk / args.rollout_temperature
+        yield chunk, targets
+
+
+class PackedLayout:
+    """Device-side description of one packed micro-batch: response offsets, row maps and packed target ids."""
+
+    def __init__(self, device, n_rows: int, unconcat_tokens, total_lengths, response_lengths, need_inverse: bool):
+        self.response_lengths = [int(r) for r in response_lengths]
+        self.n_samples = len(self.response_lengths)
+        self.n_tokens = sum(self.response_lengths)
+        begins, sft = response_row_begins(total_lengths, response_lengths)
+        for b, r in zip(begins, self.response_lengths):
+            if r > 0 and (b < 0 or b + r > n_rows):
+                raise IndexError(f"response rows [{b}, {b + r}) fall outside the {n_rows} logits rows")
+        cu = [0]
+        for r in self.response_lengths:
+            cu.append(cu[-1] + r)
+        host = torch.tensor([begins + [0], cu], dtype=torch.int64)
+        dev = host.to(device, non_blocking=False)
+        self.row_begin, self.cu_resp = dev[0, : self.n_samples].contiguous(), dev[1].contiguous()
+        self.row_ids, self.sample_ids, self.token_of_row = ops.build_row_maps(
+            self.row_begin, self.cu_resp, self.n_tokens, n_rows, want_inverse=need_inverse
+        )
+        parts = []
+        for toks, is_sft, resp in zip(unconcat_tokens, sft, self.response_lengths, strict=False):
+            parts.append(torch.nn.functional.pad(toks[1:], (0, 1), value=0) if is_sft else toks[-resp:] if resp else toks[:0])
+        self.targets = (
+            torch.cat(parts).to(device=device, dtype=torch.int64) if parts else torch.zeros(0, dtype=torch.int64, device=device)
+        )
+
+    def split(self, flat: torch.Tensor) -> list[torch.Tensor]:
+        return list(torch.split(flat, self.response_lengths))
+
+
+def get_log_probs_and_entropy(
+    logits: torch.Tensor,
+    *,
+    args: Namespace,
+    unconcat_tokens: list[torch.Tensor],
+    total_lengths: list[int],
+    response_lengths: list[int],
+    with_entropy: bool = False,
+    with_topk: bool = False,
+    topk_k=None,
+    gather_topk_token_ids=None,
+    non_loss_data: bool = True,
+    max_seq_lens=None,
+    padded_total_lengths=None,
+    dynamic_cp_size=None,
+    dynamic_cp_rank=None,
+    lm_head_forward=None,
+    **_: Any,
+) -> tuple[torch.Tensor, dict[str, list[torch.Tensor]]]:
+    """One packed launch over every response token; returns ``(empty, {"log_probs": [...], "entropy": [...]})``
+    with per-sample ``[R_i]`` fp32 views, differentiable w.r.t. ``logits``."""
+    assert non_loss_data
+    if with_topk or gather_topk_token_ids is not None:
+        raise NotImplementedError("top-K outputs are not part of the fused path")
+    if lm_head_forward is not None:
+        raise NotImplementedError("pass hidden states and the weight to relax_amd.lm_head instead of a callable")
+    flat = _check_logits(logits, args)
+    want_grad = with_entropy and getattr(args, "entropy_coef", 0.0) != 0
+    needs_bwd = torch.is_grad_enabled() and logits.requires_grad
+    lay = PackedLayout(flat.device, flat.size(0), unconcat_tokens, total_lengths, response_lengths, needs_bwd)
+    inv_t = 1.0 / float(getattr(args, "rollout_temperature", 1.0))
+    if lay.n_tokens == 0:
+        lp = flat.new_zeros((0,), dtype=torch.float32)
+        ent = lp
+    else:
+        lp, ent = ops.LogProbEntropy.apply(
+            flat, lay.targets, lay.row_ids, lay.token_of_row, inv_t, bool(with_entropy), bool(want_grad)
+        )
+    res = {"log_probs": lay.split(lp)}
+    if with_entropy:
+        res["entropy"] = lay.split(ent)
+    return torch.empty((0,), device=logits.device), res
+
+
+# ------------------------------------------------------------------------------------------ fused policy loss
+
+
+class _FusedPolicyLoss(torch.autograd.Function):
+    """logits [T, V] -> scalar loss.  Forward: one log-prob/entropy launch + the policy-loss launches; backward:
+    one dlogits launch fed with the stored d loss / d lp and d loss / d entropy coefficients."""
+
+    @staticmethod
+    def forward(ctx, flat, lay, inv_t, kw):
+        lp, ent, lse, spx = ops.logprob_entropy_fwd(flat, lay.targets, lay.row_ids, inv_t, True)
+        out = ops.policy_loss(log_prob=lp, entropy=ent, cu_resp=lay.cu_resp, **kw)
+        metrics = out["metrics"]
+        entropy_grad = kw.get("entropy_coef", 0.0) != 0
+        ctx.save_for_backward(flat, lay.targets, lse, spx if entropy_grad else None, out["coef_log_prob"],
+                              out["coef_entropy"] if entropy_grad else None, lay.token_of_row)
+        ctx.inv_t = inv_t
+        ctx.mark_non_differentiable(metrics, lp, ent)
+        return metrics[_SLOT["loss"]].clone(), metrics, lp, ent
+
+    @staticmethod
+    def backward(ctx, g_loss, _gm, _glp, _gent):
+        flat, targets, lse, spx, c_lp, c_ent, token_of_row = ctx.saved_tensors
+        scale = g_loss.reshape(1).to(torch.float32).contiguous()
+        d = ops.logprob_entropy_bwd(flat, targets, lse, spx, c_lp, c_ent, token_of_row=token_of_row,
+                                    grad_scale_dev=scale, inv_temperature=ctx.inv_t)
+        return d, None, None, None
+
+
+def _cat_f32(parts, device):
+    if parts is None:
+        return None
+    if isinstance(parts, torch.Tensor):
+        return parts.to(device=device, dtype=torch.float32).reshape(-1)
+    return torch.cat([p.to(device=device).reshape(-1) for p in parts]).to(torch.float32)
+
+
+def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum_of_sample_mean=None):
+    """Fused counterpart of loss.py:824-1185.  Returns ``(loss, metrics)`` with the reference's metric keys.
+
+    ``sum_of_sample_mean`` is accepted for signature compatibility; the same reduction (per-sample masked mean with
+    ``sample_index_mask_sums`` denominators, or the masked token sum when ``args.calculate_per_token_loss``) is
+    evaluated inside the kernel from ``batch``.  A caller-specific reducer can be passed as
+    ``batch["relax_amd_sample_denominators"]`` (per-sample divisors) or, for pg_loss only,
+    ``batch["relax_amd_pg_sample_denominators"]``.
+    """
+    flat = _check_logits(logits, args)
+    dev = flat.device
+    est = args.advantage_estimator
+    if est in ("m2po", "reinforce_plus_plus", "reinforce_plus_plus_baseline"):
+        raise NotImplementedError(f"advantage_estimator {est} is not part of the fused path")
+    if getattr(args, "custom_tis_function_path", None) is not None or getattr(args, "custom_pg_loss_reducer_function_path", None) is not None:
+        raise NotImplementedError("custom TIS / reducer callables cannot run inside the fused kernel")
+    if float(getattr(args, "opd_loss_coef", 0.0) or 0.0) != 0.0:
+        raise NotImplementedError("the OPD loss term is provided by relax_amd.opd_utils, not the fused policy loss")
+    response_lengths, total_lengths = batch["response_lengths"], batch["total_lengths"]
+    needs_bwd = torch.is_grad_enabled() and logits.requires_grad
+    lay = PackedLayout(dev, flat.size(0), batch["unconcat_tokens"], total_lengths, response_lengths, needs_bwd)
+
+    true_on_policy = getattr(args, "true_on_policy_mode", False)
+    use_rollout = getattr(args, "use_rollout_logprobs", False)
+    old = None if true_on_policy else _cat_f32(batch["rollout_log_probs"] if use_rollout else batch["log_probs"], dev)
+    mismatch = bool(getattr(args, "get_mismatch_metrics", False) or getattr(args, "use_tis", False))
+    if mismatch:
+        assert "rollout_log_probs" in batch, "rollout_log_probs must be provided for TIS"
+    rollout = _cat_f32(batch.get("rollout_log_probs"), dev)
+    # train-engine log-probs: batch["log_probs"], or this step's own forward (kernel default) in true on-policy mode
+    train = None if (true_on_policy or not batch.get("log_probs")) else _cat_f32(batch["log_probs"], dev)
+    # which log-probs the |train - rollout| metrics compare (loss.py:1125-1130): 1 = old, 0 = train, 2 = current
+    if not use_rollout:
+        abs_from = 2 if true_on_policy else 1
+    else:
+        abs_from = 0 if train is not None else 2
+    masks = _cat_f32(batch["loss_masks"], dev)
+    per_token = bool(getattr(args, "calculate_per_token_loss", False))
+    denom = batch.get("relax_amd_sample_denominators")
+    if denom is None and not per_token:
+        denom = sample_denominators(batch["loss_masks"], lay, batch.get("sample_index_mask_sums"))
+    pg_denom = batch.get("relax_amd_pg_sample_denominators")
+    use_kl = bool(getattr(args, "use_kl_loss", False))
+    kw = dict(
+        old_log_prob=old,
+        ref_log_prob=_cat_f32(batch["ref_log_probs"], dev) if use_kl else None,
+        train_log_prob=train,
+        rollout_log_prob=rollout,
+        advantages=_cat_f32(batch["advantages"], dev),
+        loss_mask=masks,
+        sample_denom=None if denom is None else denom.to(device=dev, dtype=torch.float32),
+        pg_sample_denom=None if pg_denom is None else pg_denom.to(device=dev, dtype=torch.float32),
+        loss_kind={"grpo": "ppo", "ppo": "ppo"}.get(est, est),
+        kl_kind=args.kl_loss_type if use_kl else None,
+        unbiased_kl=bool(getattr(args, "use_unbiased_kl", False)) and use_kl,
+        use_opsm=bool(getattr(args, "use_opsm", False)),
+        use_tis=bool(getattr(args, "use_tis", False)) or bool(getattr(args, "get_mismatch_metrics", False)),
+        mismatch_metrics=mismatch,
+        abs_diff_from_old=abs_from,
+        eps_clip=args.eps_clip,
+        eps_clip_high=args.eps_clip_high,
+        entropy_coef=float(getattr(args, "entropy_coef", 0.0)),
+        kl_coef=float(getattr(args, "kl_loss_coef", 0.0)) if use_kl else 0.0,
+        tis_lo=float(getattr(args, "tis_clip_low", 0.0)),
+        tis_hi=float(getattr(args, "tis_clip", 2.0)),
+        opsm_delta=float(getattr(args, "opsm_delta", 1e-4)),
+        tau_pos=float(getattr(args, "sapo_tau_pos", 1.0)),
+        tau_neg=float(getattr(args, "sapo_tau_neg", 1.05)),
+    )
+    if kw["loss_kind"] not in ("ppo", "gspo", "cispo", "rloo", "sapo"):
+        raise NotImplementedError(f"advantage_estimator {est} is not supported. ")
+    inv_t = 1.0 / float(getattr(args, "rollout_temperature", 1.0))
+    if lay.n_tokens == 0:
+        loss = 0 * logits.sum()
+        zero = loss.detach().to(torch.float32)
+        metrics = {k: zero.clone() for k in ("loss", "pg_loss", "entropy_loss", "pg_clipfrac", "ppo_kl")}
+        if use_kl:
+            metrics["kl_loss"] = zero.clone()
+        return loss, metrics
+    loss, mvec, lp, ent = _FusedPolicyLoss.apply(flat, lay, inv_t, kw)
+
+    def m(name):
+        return mvec[_SLOT[name]]
+
+    reported = {
+        "loss": m("loss"),
+        "pg_loss": m("pg_loss"),
+        "entropy_loss": m("entropy_loss"),
+        "pg_clipfrac": m("pg_clipfrac"),
+        "ppo_kl": m("ppo_kl"),
+    }
+    if rollout is not None:
+        reported["train_rollout_logprob_abs_diff"] = m("train_rollout_logprob_abs_diff")
+        reported["train_rollout_prob_abs_diff"] = m("train_rollout_prob_abs_diff")
+    if use_kl:
+        reported["kl_loss"] = m("kl_loss")
+    if mismatch:
+        for k in ("ois", "tis", "tis_clipfrac", "tis_abs", "mismatch_kl", "mismatch_k3_kl"):
+            reported[k] = m(k)
+    if kw["use_opsm"]:
+        reported["opsm_clipfrac"] = m("opsm_clipfrac")
+    return loss, reported
+
+
+def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: torch.Tensor, *, lm_head_forward=None,
+                  dp_world_size: int = 1):
+    """Counterpart of loss.py:1443-1620 for ``loss_type == "policy_loss"`` on one GPU: token count, fused loss,
+    Megatron gradient-accumulation scaling, and the ``{"keys", "values"}`` logging dict."""
+    if getattr(args, "loss_type", "policy_loss") != "policy_loss":
+        raise ValueError(f"Unknown loss type: {args.loss_type}") if args.loss_type not in ("value_loss", "sft", "custom_loss") \
+            else NotImplementedError(f"loss type {args.loss_type} is outside the fused policy path")
+    num_tokens = get_cp_local_num_tokens(batch["total_lengths"], batch["response_lengths"], batch["loss_masks"])
+    loss, log = policy_loss_function(args, batch, logits, None)
+    per_token = bool(getattr(args, "calculate_per_token_loss", False))
+    is_dummy = batch.get("__is_dummy__", False)
+    explicit = batch.get("__loss_scale__", None)
+    gbs = batch.get("dynamic_global_batch_size", getattr(args, "global_batch_size", 1))
+    if is_dummy:
+        loss = 0.0 * loss
+    elif not per_token:
+        loss = loss * explicit if explicit is not None else loss * num_microbatches / gbs * dp_world_size
+    effective = torch.zeros_like(num_tokens) if is_dummy else num_tokens
+    denominator = effective if per_token else torch.zeros_like(num_tokens)
+    values = torch.stack([denominator.to(torch.float32)] + [v.to(torch.float32) for v in log.values()])
+    if is_dummy:
+        values = torch.zeros_like(values)
+    normalizer = effective if per_token else torch.tensor(1, device=logits.device)
+    return loss, normalizer, {"keys": list(log.keys()), "values": values}
+
+
+# ------------------------------------------------------------------------------------------------- advantages
+
+
+def compute_advantages_and_returns(args: Namespace, rollout_data: dict) -> None:
+    """GRPO-family branch of loss.py:532-738: broadcast the (already group-normalised) per-sample rewards over each
+    response, optionally whiten across the micro-batch.  Writes ``advantages`` / ``returns`` lists in place."""
+    from .distributed_utils import distributed_masked_whiten
+
+    log_probs = rollout_data.get("rollout_log_probs" if getattr(args, "use_rollout_logprobs", False) else "log_probs")
+    values = rollout_data.get("values")
+    rewards = rollout_data.get("rewards")
+    loss_masks = rollout_data.get("loss_masks")
+    if args.advantage_estimator not in GRPO_FAMILY:
+        raise NotImplementedError(f"advantage_estimator {args.advantage_estimator} is not supported. ")
+    xs = log_probs if log_probs is not None else values
+    if xs is None:
+        return
+    dev = xs[0].device
+    # kl only supplies shape / dtype / device for this estimator family (loss.py:574-591)
+    like = [torch.empty(x.shape, dtype=torch.float32, device=dev) for x in xs]
+    rw = torch.tensor(rewards, dtype=torch.float32, device=dev)
+    returns = get_grpo_returns(rw, like)
+    advantages = list(returns)
+    if getattr(args, "normalize_advantages", False):
+        flat = torch.cat(advantages)
+        masks = torch.cat(loss_masks).to(dev)
+        assert flat.size() == masks.size(), f"Shape mismatch before whitening: advantages {flat.size()}, masks {masks.size()}"
+        if masks.numel() > 0:
+            white = distributed_masked_whiten(flat, masks, process_group=None, shift_mean=True)
+            advantages = list(torch.split(white, [a.size(0) for a in advantages]))
+    rollout_data["advantages"] = advantages
+    rollout_data["returns"] = returns

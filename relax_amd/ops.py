@@ -1,0 +1,314 @@
+"""Tensor-level wrappers over the C ABI: argument checks, output allocation, stream hand-off, autograd glue.
+
+PyTorch is used here only for device memory, streams and autograd bookkeeping; every arithmetic step on the token
+path runs in the HIP kernels of ``librelax_amd.so``.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import BF16, F16, F32, NUM_METRICS, PolicyLossArgs, check, lib
+
+_DTYPE_CODES = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+
+
+def _need_gpu(*tensors) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(
+                "relax_amd kernels run on a ROCm device only (got a CPU tensor); there is no CPU fallback"
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} vs {t.device}")
+    if dev is None:
+        raise RuntimeError("relax_amd op called without any device tensor")
+    return dev
+
+
+def _p(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODES[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported logits dtype {t.dtype}; expected float32, bfloat16 or float16") from None
+
+
+def _rows(t: torch.Tensor) -> torch.Tensor:
+    """2-D view with unit inner stride (copy only if the caller handed something exotic)."""
+    if t.dim() != 2:
+        raise ValueError(f"expected a 2-D [rows, vocab] tensor, got shape {tuple(t.shape)}")
+    if t.size(0) > 1 and t.size(1) > 0 and (t.stride(1) != 1 or t.stride(0) < t.size(1)):
+        t = t.contiguous()
+    elif t.size(1) > 0 and t.stride(1) != 1:
+        t = t.contiguous()
+    return t
+
+
+def _f32(t, dev=None):
+    if t is None:
+        return None
+    if t.dtype != torch.float32 or not t.is_contiguous():
+        t = t.to(torch.float32).contiguous()
+    return t
+
+
+# ------------------------------------------------------------------------------------------------ log-prob / entropy
+
+
+def logprob_entropy_fwd(logits, targets, row_ids=None, inv_temperature: float = 1.0, with_entropy: bool = True,
+                        n_tokens: int | None = None):
+    """Returns (log_prob, entropy | None, lse, spx | None), all fp32 [n_tokens]."""
+    _need_gpu(logits, targets, row_ids)
+    logits = _rows(logits)
+    n = int(targets.numel()) if n_tokens is None else n_tokens
+    if row_ids is None and n != logits.size(0):
+        raise ValueError(f"{n} targets for {logits.size(0)} logits rows")
+    if targets.dtype != torch.int64 or not targets.is_contiguous():
+        targets = targets.to(torch.int64).contiguous()
+    kw = dict(dtype=torch.float32, device=logits.device)
+    lp = torch.empty(n, **kw)
+    lse = torch.empty(n, **kw)
+    ent = torch.empty(n, **kw) if with_entropy else None
+    spx = torch.empty(n, **kw) if with_entropy else None
+    check(lib.relax_amd_logprob_entropy_fwd(
+        _p(logits), _code(logits), n, logits.size(1), logits.stride(0) if logits.size(0) > 1 else logits.size(1),
+        _p(row_ids), _p(targets), float(inv_temperature), _p(lp), _p(ent), _p(lse), _p(spx), _stream()))
+    return lp, ent, lse, spx
+
+
+def logprob_entropy_bwd(logits, targets, lse, spx, g_lp, g_ent=None, token_of_row=None, grad_scale: float = 1.0,
+                        grad_scale_dev=None, inv_temperature: float = 1.0, out=None):
+    """dlogits [rows, vocab] in the logits dtype; every row is written."""
+    _need_gpu(logits, targets, lse, g_lp)
+    logits = _rows(logits)
+    if out is None:
+        out = torch.empty((logits.size(0), logits.size(1)), dtype=logits.dtype, device=logits.device)
+    stride = logits.stride(0) if logits.size(0) > 1 else logits.size(1)
+    check(lib.relax_amd_logprob_entropy_bwd(
+        _p(logits), _code(logits), logits.size(0), logits.size(1), stride, _p(token_of_row), _p(targets), _p(lse),
+        _p(spx), _p(_f32(g_lp)), _p(_f32(g_ent)), float(grad_scale), _p(grad_scale_dev), float(inv_temperature),
+        _p(out), out.stride(0) if out.size(0) > 1 else out.size(1), _stream()))
+    return out
+
+
+class LogProbEntropy(torch.autograd.Function):
+    """(logits [R,V], targets [R]) -> (log_prob [R], entropy [R]); saves the logits reference + O(R) floats."""
+
+    @staticmethod
+    def forward(ctx, logits, targets, row_ids, token_of_row, inv_temperature, with_entropy, with_entropy_grad):
+        with_entropy_grad = bool(with_entropy and with_entropy_grad)
+        x = _rows(logits)
+        if targets.dtype != torch.int64 or not targets.is_contiguous():
+            targets = targets.to(torch.int64).contiguous()
+        lp, ent, lse, spx = logprob_entropy_fwd(x, targets, row_ids, inv_temperature, with_entropy)
+        ctx.save_for_backward(x, targets, lse, spx if with_entropy_grad else None, row_ids, token_of_row)
+        ctx.inv_temperature = inv_temperature
+        ctx.with_entropy_grad = with_entropy_grad
+        if ent is None:
+            ent = lp.new_zeros((0,))
+        if not with_entropy_grad:
+            ctx.mark_non_differentiable(ent)
+        return lp, ent
+
+    @staticmethod
+    def backward(ctx, g_lp, g_ent):
+        x, targets, lse, spx, row_ids, token_of_row = ctx.saved_tensors
+        if g_lp is None:
+            raise RuntimeError("LogProbEntropy expected a materialized grad_log_prob")
+        if not ctx.with_entropy_grad or g_ent is None or g_ent.numel() == 0:
+            g_ent = None
+        if row_ids is not None and token_of_row is None:
+            raise RuntimeError("row_ids without token_of_row cannot be differentiated")
+        d = logprob_entropy_bwd(x, targets, lse, spx, g_lp.reshape(-1), None if g_ent is None else g_ent.reshape(-1),
+                                token_of_row=token_of_row, inv_temperature=ctx.inv_temperature)
+        return d, None, None, None, None, None, None
+
+
+# ------------------------------------------------------------------------------------------------------- row maps
+
+
+def build_row_maps(row_begin, cu_resp, n_tokens: int, n_rows: int, want_inverse: bool = True):
+    """row_begin [B] int64, cu_resp [B+1] int64 (device) -> (row_ids, sample_ids, token_of_row | None), int32."""
+    dev = _need_gpu(row_begin, cu_resp)
+    row_ids = torch.empty(n_tokens, dtype=torch.int32, device=dev)
+    sample_ids = torch.empty(n_tokens, dtype=torch.int32, device=dev)
+    inv = torch.empty(n_rows, dtype=torch.int32, device=dev) if want_inverse else None
+    check(lib.relax_amd_build_row_maps(_p(row_begin), _p(cu_resp), row_begin.numel(), n_tokens, n_rows, _p(row_ids),
+                                       _p(sample_ids), _p(inv), _stream()))
+    return row_ids, sample_ids, inv
+
+
+def segment_sum(mask, cu_resp, values=None):
+    """fp64 [B]: per-sample sum of mask (or values*mask)."""
+    dev = _need_gpu(mask, cu_resp)
+    b = cu_resp.numel() - 1
+    out = torch.empty(b, dtype=torch.float64, device=dev)
+    check(lib.relax_amd_segment_sum(_p(_f32(values)), _p(_f32(mask)), _p(cu_resp), b, _p(out), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------- policy loss
+
+
+def policy_loss(*, log_prob, advantages, loss_mask, cu_resp, old_log_prob=None, ref_log_prob=None,
+                train_log_prob=None, rollout_log_prob=None, entropy=None, pg_loss_mask=None, sample_denom=None,
+                pg_sample_denom=None, loss_kind="ppo", kl_kind=None, unbiased_kl=False, use_opsm=False, use_tis=False,
+                mismatch_metrics=False, abs_diff_from_old=1, eps_clip=0.2, eps_clip_high=0.2, eps_clip_c=None,
+                entropy_coef=0.0, kl_coef=0.0, tis_lo=0.0, tis_hi=2.0, opsm_delta=1e-4, tau_pos=1.0, tau_neg=1.05,
+                per_token_outputs=False):
+    """Runs the two policy-loss launches.  Returns dict(metrics [16], coef_log_prob, coef_entropy, per-token...)."""
+    dev = _need_gpu(log_prob, advantages, loss_mask, cu_resp)
+    n = int(log_prob.numel())
+    b = int(cu_resp.numel()) - 1
+    if loss_kind not in _lib.LOSS_KINDS:
+        raise ValueError(f"unknown loss kind {loss_kind}")
+    if kl_kind not in _lib.KL_KINDS:
+        raise ValueError(f"Unknown kl_loss_type: {kl_kind}")
+    keep = [_f32(t) for t in (log_prob, old_log_prob, ref_log_prob, train_log_prob, rollout_log_prob, advantages,
+                               loss_mask, pg_loss_mask, entropy, sample_denom, pg_sample_denom)]
+    for t in keep[:9]:
+        if t is not None and t.numel() != n:
+            raise ValueError(f"per-token tensor has {t.numel()} elements, expected {n}")
+    for t in keep[9:]:
+        if t is not None and t.numel() != b:
+            raise ValueError(f"per-sample denominator has {t.numel()} elements, expected {b}")
+    kw = dict(dtype=torch.float32, device=dev)
+    out = {
+        "coef_log_prob": torch.empty(n, **kw),
+        "coef_entropy": torch.empty(n, **kw) if entropy is not None else None,
+        "metrics": torch.empty(NUM_METRICS, **kw),
+    }
+    if per_token_outputs:
+        for k in ("pg_loss_tok", "clipfrac_tok", "ppo_kl_tok"):
+            out[k] = torch.empty(n, **kw)
+        out["kl_tok"] = torch.empty(n, **kw) if kl_kind is not None else None
+    partials = torch.empty(max(b, 1) * NUM_METRICS, **kw)
+    a = PolicyLossArgs()
+    (a.log_prob, a.old_log_prob, a.ref_log_prob, a.train_log_prob, a.rollout_log_prob, a.advantages, a.loss_mask,
+     a.pg_loss_mask, a.entropy, a.sample_denom, a.pg_sample_denom) = [None if t is None else t.data_ptr() for t in keep]
+    a.cu_resp = cu_resp.data_ptr()
+    a.n_samples, a.n_tokens = b, n
+    a.loss_kind, a.kl_kind = _lib.LOSS_KINDS[loss_kind], _lib.KL_KINDS[kl_kind]
+    a.unbiased_kl, a.use_opsm, a.use_tis = int(unbiased_kl), int(use_opsm), int(use_tis)
+    a.mismatch_metrics, a.abs_diff_from_old = int(mismatch_metrics), int(abs_diff_from_old)
+    a.eps_clip, a.eps_clip_high = float(eps_clip), float(eps_clip_high)
+    a.eps_clip_c = -1.0 if eps_clip_c is None else float(eps_clip_c)
+    a.entropy_coef, a.kl_coef = float(entropy_coef), float(kl_coef)
+    a.tis_lo, a.tis_hi, a.opsm_delta = float(tis_lo), float(tis_hi), float(opsm_delta)
+    a.tau_pos, a.tau_neg = float(tau_pos), float(tau_neg)
+    a.coef_log_prob = out["coef_log_prob"].data_ptr()
+    a.coef_entropy = None if out["coef_entropy"] is None else out["coef_entropy"].data_ptr()
+    for k in ("pg_loss_tok", "clipfrac_tok", "ppo_kl_tok", "kl_tok"):
+        t = out.get(k)
+        setattr(a, k, None if t is None else t.data_ptr())
+    a.sample_partials = partials.data_ptr()
+    a.metrics = out["metrics"].data_ptr()
+    if cu_resp.dtype != torch.int64:
+        raise TypeError("cu_resp must be int64")
+    check(lib.relax_amd_policy_loss(C.byref(a), _stream()))
+    out["_keepalive"] = (keep, partials)
+    return out
+
+
+# ----------------------------------------------------------------------------------------------------- advantages
+
+
+def group_rewards(rewards, group_index, mode: str):
+    """rewards fp32|fp64 [B], group_index int32 [B] (device) -> (normalised [B] same dtype, group sizes int32 [B])."""
+    dev = _need_gpu(rewards, group_index)
+    n = int(rewards.numel())
+    if rewards.dtype not in (torch.float32, torch.float64):
+        rewards = rewards.float()
+    rewards = rewards.contiguous()
+    out = torch.empty(n, dtype=rewards.dtype, device=dev)
+    cnt = torch.empty(n, dtype=torch.int32, device=dev)
+    code = _lib.F32 if rewards.dtype == torch.float32 else _lib.F64
+    check(lib.relax_amd_group_rewards(_p(rewards), code, _p(group_index.to(torch.int32).contiguous()), n,
+                                      _lib.GROUP_MODES[mode], _p(out), _p(cnt), _stream()))
+    return out, cnt
+
+
+def broadcast_per_sample(per_sample, cu_resp, n_tokens: int):
+    dev = _need_gpu(per_sample, cu_resp)
+    out = torch.empty(n_tokens, dtype=torch.float32, device=dev)
+    check(lib.relax_amd_broadcast_per_sample(_p(_f32(per_sample)), _p(cu_resp), cu_resp.numel() - 1, _p(out),
+                                             _stream()))
+    return out
+
+
+def masked_whiten(values, mask, shift_mean: bool = True, epsilon: float = 1e-8):
+    """Returns (whitened fp32 [N], stats fp32 [4] = sum, sum of squares, mask sum, rstd)."""
+    dev = _need_gpu(values, mask)
+    n = int(values.numel())
+    if n == 0:
+        raise ValueError("masked_whiten needs at least one value")
+    v, m = _f32(values.reshape(-1)), _f32(mask.reshape(-1))
+    partials = torch.empty(3 * lib.relax_amd_whiten_partials(n), dtype=torch.float64, device=dev)
+    stats = torch.empty(4, dtype=torch.float32, device=dev)
+    out = torch.empty(n, dtype=torch.float32, device=dev)
+    check(lib.relax_amd_masked_whiten(_p(v), _p(m), n, int(shift_mean), float(epsilon), _p(partials), _p(stats),
+                                      _p(out), _stream()))
+    return out, stats
+
+
+# ------------------------------------------------------------------------------------------------------ reverse KL
+
+
+def reverse_kl_fwd(student, teacher):
+    _need_gpu(student, teacher)
+    s, t = _rows(student), _rows(teacher)
+    if s.shape != t.shape or s.dtype != t.dtype:
+        raise ValueError(f"student {tuple(s.shape)}/{s.dtype} and teacher {tuple(t.shape)}/{t.dtype} must match")
+    if s.size(0) > 1 and s.stride(0) != t.stride(0):
+        s, t = s.contiguous(), t.contiguous()
+    n = s.size(0)
+    kw = dict(dtype=torch.float32, device=s.device)
+    kl, ls, lt = torch.empty(n, **kw), torch.empty(n, **kw), torch.empty(n, **kw)
+    stride = s.stride(0) if n > 1 else s.size(1)
+    check(lib.relax_amd_reverse_kl_fwd(_p(s), _p(t), _code(s), n, s.size(1), stride, _p(kl), _p(ls), _p(lt),
+                                       _stream()))
+    return kl, ls, lt, s, t
+
+
+def reverse_kl_bwd(s, t, kl, ls, lt, g, grad_scale: float = 1.0, grad_scale_dev=None):
+    n = s.size(0)
+    stride = s.stride(0) if n > 1 else s.size(1)
+    if stride != s.size(1):
+        raise ValueError("reverse_kl_bwd writes a dense gradient: student rows must be contiguous")
+    d = torch.empty_like(s)
+    check(lib.relax_amd_reverse_kl_bwd(_p(s), _p(t), _code(s), n, s.size(1), stride, _p(kl), _p(ls), _p(lt),
+                                       _p(_f32(g)), float(grad_scale), _p(grad_scale_dev), _p(d), _stream()))
+    return d
+
+
+class ReverseKL(torch.autograd.Function):
+    """(student logits [R,V], teacher logits [R,V]) -> per-token KL(student || teacher) [R]; teacher gets no grad."""
+
+    @staticmethod
+    def forward(ctx, student, teacher):
+        kl, ls, lt, s, t = reverse_kl_fwd(student, teacher)
+        if s.size(0) > 1 and s.stride(0) != s.size(1):
+            s, t = s.contiguous(), t.contiguous()
+        ctx.save_for_backward(s, t, kl, ls, lt)
+        return kl
+
+    @staticmethod
+    def backward(ctx, g):
+        s, t, kl, ls, lt = ctx.saved_tensors
+        return reverse_kl_bwd(s, t, kl, ls, lt, g.reshape(-1)), None

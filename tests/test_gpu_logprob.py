@@ -1,0 +1,182 @@
+"""GPU parity of the log-prob / entropy kernels against the oracle, through the C ABI (ctypes).
+
+Tolerances: fp32 inputs 2e-5 abs (fp32 accumulation, different summation order); bf16 / fp16 inputs 2e-3 abs on
+log-probs, entropy and gradients (the bound the benchmark states); indices and masks exact.
+"""
+
+import math
+
+import pytest
+import torch
+
+from oracle import logprob as O
+from tests.gpu_util import announce, require_gpu, spiked_logits
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle(x_cpu, tok_cpu, wl, we, inv_t=1.0):
+    x = x_cpu.clone().requires_grad_()
+    xs = x.float() * inv_t if inv_t != 1.0 else x
+    lp, ent = O.calculate_log_probs_and_entropy(xs, tok_cpu, None, with_entropy=True)
+    ((lp.squeeze(-1) * wl).sum() + (ent * we).sum()).backward()
+    return lp.squeeze(-1).detach(), ent.detach(), x.grad
+
+
+@pytest.mark.parametrize("key", ["logprob_single_rank", "logprob_two_shards"])
+def test_reference_literals(literals, key):
+    import relax_amd
+
+    dev = require_gpu()
+    fx = literals[key]
+    announce("literals", key)
+    x = torch.tensor(fx["logits"], device=dev, requires_grad=True)
+    tok = torch.tensor(fx["tokens"], device=dev)
+    wl, we = torch.tensor(fx["logprob_weights"]), torch.tensor(fx["entropy_weights"])
+    for chunk in (-1, 1, 2, 8):
+        x.grad = None
+        lp, ent = relax_amd.calculate_log_probs_and_entropy(x, tok, None, with_entropy=True, chunk_size=chunk)
+        assert lp.shape == (len(fx["tokens"]), 1) and lp.dtype == torch.float32
+        ((lp.squeeze(-1) * wl.to(dev)).sum() + (ent * we.to(dev)).sum()).backward()
+        rlp, rent, rg = _oracle(torch.tensor(fx["logits"]), torch.tensor(fx["tokens"]), wl, we)
+        torch.testing.assert_close(lp.squeeze(-1).cpu(), rlp, atol=2e-6, rtol=0)
+        torch.testing.assert_close(ent.cpu(), rent, atol=2e-6, rtol=0)
+        torch.testing.assert_close(x.grad.cpu(), rg, atol=2e-6, rtol=0)
+
+
+@pytest.mark.parametrize(
+    "n,v,dtype,scale,tol",
+    [
+        (64, 1003, torch.float32, 2.0, 2e-5),      # unaligned stride -> scalar path
+        (48, 4096, torch.float32, 2.0, 2e-5),      # vector path, exact multiple of the unroll
+        (33, 32000, torch.float32, 2.0, 2e-5),     # first benchmark configuration's vocabulary
+        (40, 4100, torch.bfloat16, 3.0, 2e-3),     # vector path + remainder vectors + scalar tail (4100 % 8 = 4)
+        (24, 151936, torch.bfloat16, 3.0, 2e-3),   # headline vocabulary, spiked rows
+        (24, 151936, torch.float16, 3.0, 2e-3),
+        (3, 7, torch.bfloat16, 1.0, 2e-3),
+    ],
+)
+@pytest.mark.parametrize("inv_t", [1.0, 1 / 0.7])
+def test_forward_backward_vs_oracle(n, v, dtype, scale, tol, inv_t):
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("fwd/bwd", n, v, dtype, inv_t)
+    x = spiked_logits(n, v, scale, dtype, seed=n + v, device=dev)
+    g = torch.Generator().manual_seed(7)
+    tok = torch.randint(0, v, (n,), generator=g)
+    wl, we = torch.randn(n, generator=g), torch.randn(n, generator=g) * 0.3
+    wl[0] = 0.0
+    we[0] = 0.0  # a zero-gradient row must come back exactly zero
+    lp, ent, lse, spx = ops.logprob_entropy_fwd(x, tok.to(dev), None, inv_t, True)
+    d = ops.logprob_entropy_bwd(x, tok.to(dev), lse, spx, wl.to(dev), we.to(dev), inv_temperature=inv_t)
+    rlp, rent, rg = _oracle(x.cpu(), tok, wl, we, inv_t)
+    assert lp.dtype == torch.float32 and d.dtype == dtype and d.shape == x.shape
+    torch.testing.assert_close(lp.cpu(), rlp, atol=tol, rtol=0)
+    torch.testing.assert_close(ent.cpu(), rent, atol=tol, rtol=0)
+    torch.testing.assert_close(d.float().cpu(), rg.float(), atol=tol, rtol=0)
+    assert d[0].abs().max().item() == 0.0
+    # run-to-run determinism (forward-only pass and training pass must agree bit for bit)
+    lp2, ent2, _, _ = ops.logprob_entropy_fwd(x, tok.to(dev), None, inv_t, True)
+    assert torch.equal(lp, lp2) and torch.equal(ent, ent2)
+    # a forward without entropy returns the same log-probs
+    lp3, ent3, _, spx3 = ops.logprob_entropy_fwd(x, tok.to(dev), None, inv_t, False)
+    assert ent3 is None and spx3 is None
+    torch.testing.assert_close(lp3, lp, atol=1e-6, rtol=0)
+
+
+def test_autograd_function_semantics(literals):
+    import relax_amd
+
+    dev = require_gpu()
+    announce("autograd semantics")
+    fx = literals["logprob_single_rank"]
+    x = torch.tensor(fx["logits"], device=dev, requires_grad=True)
+    tok = torch.tensor(fx["tokens"], device=dev)
+    lp, ent = relax_amd.calculate_log_probs_and_entropy(x, tok, None, with_entropy=True, with_entropy_grad=False)
+    assert lp.requires_grad and not ent.requires_grad
+    lp, ent = relax_amd.calculate_log_probs_and_entropy(x, tok, None, with_entropy=False)
+    assert ent is None
+    empty = torch.zeros(0, 4, device=dev)
+    lp, ent = relax_amd.calculate_log_probs_and_entropy(empty, torch.zeros(0, dtype=torch.long, device=dev), None, True)
+    assert lp.shape == (0,) and ent.shape == (0,)
+    # bf16 logits: fp32 outputs, gradient in the logits dtype
+    xb = torch.randn(5, 64, device=dev).bfloat16().requires_grad_()
+    lp, _ = relax_amd.calculate_log_probs_and_entropy(xb, torch.randint(0, 64, (5,), device=dev), None)
+    assert lp.dtype == torch.float32
+    lp.sum().backward()
+    assert xb.grad.dtype == torch.bfloat16
+    # inputs are never written
+    before = xb.detach().clone()
+    relax_amd.calculate_log_probs_and_entropy(xb, torch.randint(0, 64, (5,), device=dev), None, True)
+    assert torch.equal(before, xb.detach())
+
+
+def test_strided_rows_row_ids_and_inverse_map():
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("row maps")
+    t_rows, v = 23, 520
+    big = torch.randn(t_rows, v + 8, device=dev)
+    x = big[:, :v]  # row stride v+8: still 16-byte aligned rows
+    begins = torch.tensor([2, 9, 15], device=dev)
+    lens = [3, 4, 5]
+    cu = torch.tensor([0, 3, 7, 12], device=dev)
+    row_ids, sample_ids, inv = ops.build_row_maps(begins, cu, 12, t_rows)
+    want_rows = [2, 3, 4, 9, 10, 11, 12, 15, 16, 17, 18, 19]
+    assert row_ids.tolist() == want_rows
+    assert sample_ids.tolist() == [0] * 3 + [1] * 4 + [2] * 5
+    want_inv = [-1] * t_rows
+    for k, r in enumerate(want_rows):
+        want_inv[r] = k
+    assert inv.tolist() == want_inv
+    tok = torch.randint(0, v, (12,), device=dev)
+    lp, ent, lse, spx = ops.logprob_entropy_fwd(x, tok, row_ids, 1.0, True)
+    ref = torch.log_softmax(x[want_rows].double(), -1)
+    torch.testing.assert_close(lp.double(), ref[torch.arange(12), tok], atol=2e-5, rtol=0)
+    g = torch.randn(12, device=dev)
+    d = ops.logprob_entropy_bwd(x, tok, lse, spx, g, None, token_of_row=inv)
+    assert d.shape == (t_rows, v)
+    untouched = [r for r in range(t_rows) if r not in want_rows]
+    assert d[untouched].abs().max().item() == 0.0
+    p = ref.exp()
+    want = -p * g.double()[:, None]
+    want[torch.arange(12), tok] += g.double()
+    torch.testing.assert_close(d[want_rows].double(), want, atol=2e-5, rtol=0)
+
+
+def test_invalid_target_gives_nan_not_a_fault():
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("invalid target")
+    x = torch.randn(4, 64, device=dev)
+    tok = torch.tensor([0, 64, -1, 63], device=dev)
+    lp, _, _, _ = ops.logprob_entropy_fwd(x, tok, None, 1.0, True)
+    assert torch.isnan(lp[1]) and torch.isnan(lp[2]) and torch.isfinite(lp[0]) and torch.isfinite(lp[3])
+
+
+def test_full_size_properties_headline_shape():
+    """Size-independent properties at the benchmark's vocabulary on a 4096-row slab, plus an oracle spot check."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    n, v = 4096, 151936
+    announce("full-size properties", n, v)
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = (torch.randn(n, v, device=dev, generator=g) * 3.0).bfloat16()
+    tok = torch.randint(0, v, (n,), device=dev, generator=g)
+    lp, ent, lse, spx = ops.logprob_entropy_fwd(x, tok, None, 1.0, True)
+    assert (lp <= 0).all() and (ent >= 0).all() and (ent <= math.log(v) + 1e-3).all()
+    # shift invariance: adding a constant representable in bf16 steps changes nothing beyond rounding of x itself
+    glp = torch.randn(n, device=dev, generator=g)
+    gen = torch.randn(n, device=dev, generator=g) * 0.1
+    d = ops.logprob_entropy_bwd(x, tok, lse, spx, glp, gen)
+    rowsum = d.float().sum(-1)
+    assert rowsum.abs().max().item() < 5e-2  # sum_v dlogits = 0 up to bf16 rounding of 151936 terms
+    idx = torch.arange(0, n, 128, device=dev)
+    xs = x[idx].cpu()
+    rlp, rent = O.calculate_log_probs_and_entropy(xs, tok[idx].cpu(), None, with_entropy=True)
+    torch.testing.assert_close(lp[idx].cpu(), rlp.squeeze(-1), atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent[idx].cpu(), rent, atol=2e-3, rtol=0)

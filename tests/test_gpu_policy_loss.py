@@ -1,0 +1,271 @@
+"""GPU parity of the fused policy loss (custom_loss plug-in signature) against the oracle composition.
+
+fp32 logits: loss / metrics / dlogits within 2e-5; bf16 logits within 2e-3 (the stated bound).  Token counts and
+row maps are compared exactly.
+"""
+
+import pytest
+import torch
+
+from oracle import policy as P
+from oracle import reducers as R
+from tests.gpu_util import announce, require_gpu
+
+pytestmark = pytest.mark.gpu
+
+
+def _make_batch(seed, tot, resp, v, dtype=torch.float32, int_masks=False, sft_sample=None):
+    g = torch.Generator().manual_seed(seed)
+    t = sum(tot)
+    logits = (torch.randn(1, t, v, generator=g) * 2).to(dtype)
+    toks = [torch.randint(0, v, (n,), generator=g) for n in tot]
+    n = sum(resp)
+    masks = []
+    for r in resp:
+        m = (torch.rand(r, generator=g) > 0.3)
+        masks.append(m.long() if int_masks else m.float())
+    masks[0] = torch.zeros_like(masks[0])  # a fully masked sample exercises clamp_min(denominator, 1)
+    base = -2.0 + 0.3 * torch.randn(n, generator=g)
+    batch = dict(
+        advantages=list(torch.split(torch.randn(n, generator=g), resp)),
+        log_probs=list(torch.split(base, resp)),
+        ref_log_probs=list(torch.split(base + 0.1 * torch.randn(n, generator=g), resp)),
+        rollout_log_probs=list(torch.split(base + 0.05 * torch.randn(n, generator=g), resp)),
+        unconcat_tokens=toks, response_lengths=resp, total_lengths=tot, loss_masks=masks,
+    )
+    return logits, batch
+
+
+def _to_dev(batch, dev):
+    out = {}
+    for k, val in batch.items():
+        if isinstance(val, list) and val and isinstance(val[0], torch.Tensor):
+            out[k] = [x.to(dev) for x in val]
+        else:
+            out[k] = val
+    return out
+
+
+CASES = {
+    "ppo": dict(),
+    "ppo_k3_entropy": dict(eps_clip_high=0.28, use_kl_loss=True, kl_loss_coef=1e-3, kl_loss_type="k3", entropy_coef=0.01),
+    "ppo_unbiased_low_var": dict(use_kl_loss=True, kl_loss_coef=0.05, kl_loss_type="low_var_kl", use_unbiased_kl=True),
+    "ppo_k1": dict(use_kl_loss=True, kl_loss_coef=0.1, kl_loss_type="k1"),
+    "ppo_k2_per_token": dict(use_kl_loss=True, kl_loss_coef=0.1, kl_loss_type="k2", calculate_per_token_loss=True),
+    "gspo": dict(advantage_estimator="gspo", eps_clip=3e-4, eps_clip_high=4e-4),
+    "gspo_wide": dict(advantage_estimator="gspo", eps_clip=0.2, eps_clip_high=0.2, entropy_coef=0.02),
+    "cispo": dict(advantage_estimator="cispo", eps_clip=0.2, eps_clip_high=0.28),
+    "rloo": dict(advantage_estimator="rloo"),
+    "sapo": dict(advantage_estimator="sapo"),
+    "opsm": dict(use_opsm=True, opsm_delta=-1.0),
+    "tis": dict(use_tis=True, tis_clip=1.02, tis_clip_low=0.97),
+    "true_on_policy": dict(true_on_policy_mode=True),
+    "use_rollout_logprobs": dict(use_rollout_logprobs=True),
+    "temperature": dict(rollout_temperature=0.7, entropy_coef=0.01),
+}
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-5), (torch.bfloat16, 2e-3)])
+def test_policy_loss_function_vs_oracle(name, dtype, tol):
+    import relax_amd
+
+    dev = require_gpu()
+    announce("policy_loss", name, dtype)
+    tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 264
+    logits, batch = _make_batch(11, tot, resp, v, dtype)
+    args = P.make_args(**CASES[name])
+    # oracle on CPU (fp32 upcast of the same logits values)
+    lo = logits.float().clone().requires_grad_()
+    red = R.make_reducer(resp, batch["loss_masks"], args.calculate_per_token_loss)
+    ob = dict(batch)
+    want_loss, want_m = P.policy_loss_function(args, ob, lo, red)
+    want_loss.backward()
+    lg = logits.to(dev).requires_grad_()
+    loss, met = relax_amd.policy_loss_function(args, _to_dev(batch, dev), lg, None)
+    loss.backward()
+    assert lg.grad.dtype == dtype and lg.grad.shape == logits.shape
+    assert abs(loss.item() - want_loss.item()) < tol * max(1.0, abs(want_loss.item()))
+    for k, w in want_m.items():
+        assert k in met, f"missing metric {k}"
+        assert abs(met[k].item() - float(w)) < tol * max(1.0, abs(float(w))), (k, met[k].item(), float(w))
+    assert set(met) == set(want_m)
+    torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, atol=tol, rtol=0)
+
+
+def test_sample_index_mask_sums_int_masks_and_sft_row():
+    import relax_amd
+
+    dev = require_gpu()
+    announce("policy_loss denominators / int masks / sft-shaped sample")
+    tot, resp, v = [6, 5, 8], [3, 5, 4], 96  # second sample: response == total (SFT convention)
+    logits, batch = _make_batch(5, tot, resp, v, torch.float32, int_masks=True)
+    batch["sample_index_mask_sums"] = [7, 7, 3]
+    args = P.make_args(entropy_coef=0.01)
+    lo = logits.clone().requires_grad_()
+    red = R.make_reducer(resp, batch["loss_masks"], False, batch["sample_index_mask_sums"])
+    want_loss, want_m = P.policy_loss_function(args, dict(batch), lo, red)
+    want_loss.backward()
+    lg = logits.to(dev).requires_grad_()
+    loss, met = relax_amd.policy_loss_function(args, _to_dev(batch, dev), lg, None)
+    loss.backward()
+    assert abs(loss.item() - want_loss.item()) < 3e-5
+    torch.testing.assert_close(lg.grad.cpu(), lo.grad, atol=3e-5, rtol=0)
+
+
+def test_loss_function_scaling_and_exact_token_count():
+    import relax_amd
+
+    dev = require_gpu()
+    announce("loss_function tail")
+    tot, resp, v = [9, 6, 12], [4, 3, 7], 64
+    logits, batch = _make_batch(3, tot, resp, v, torch.float32, int_masks=True)
+    for per_token in (False, True):
+        args = P.make_args(global_batch_size=8, calculate_per_token_loss=per_token)
+        want_loss, want_norm, want_log = P.loss_function(args, dict(batch), 4, logits, dp_world=2)
+        loss, norm, log = relax_amd.loss_function(args, _to_dev(batch, dev), 4, logits.to(dev), dp_world_size=2)
+        assert log["keys"] == want_log["keys"]
+        assert int(norm.item()) == int(want_norm.item())  # exact
+        torch.testing.assert_close(log["values"].cpu(), want_log["values"].float(), atol=3e-5, rtol=1e-5)
+        assert abs(loss.item() - want_loss.item()) < 3e-5 * max(1, abs(want_loss.item()))
+    n = relax_amd.cp_utils.get_cp_local_num_tokens(tot, resp, [m.to(dev) for m in batch["loss_masks"]])
+    assert n.dtype == torch.int64 and n.item() == R.num_tokens(batch["loss_masks"]).item()
+
+
+def test_get_log_probs_and_entropy_forward_only_matches_training_forward_bitwise():
+    """The forward-only pass and the training forward must give identical log-probs for identical inputs."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("forward_only vs train forward")
+    tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 1000
+    logits, batch = _make_batch(2, tot, resp, v, torch.bfloat16)
+    args = P.make_args(entropy_coef=0.0)
+    db = _to_dev(batch, dev)
+    with torch.no_grad():
+        _, out = relax_amd.get_log_probs_and_entropy(
+            logits.to(dev), args=args, unconcat_tokens=db["unconcat_tokens"], total_lengths=tot,
+            response_lengths=resp, with_entropy=True)
+    assert [x.shape[0] for x in out["log_probs"]] == resp
+    lg = logits.to(dev).requires_grad_()
+    _, out2 = relax_amd.get_log_probs_and_entropy(
+        lg, args=args, unconcat_tokens=db["unconcat_tokens"], total_lengths=tot, response_lengths=resp,
+        with_entropy=True)
+    for a, b in zip(out["log_probs"], out2["log_probs"]):
+        assert torch.equal(a, b)
+    assert not out2["entropy"][0].requires_grad and out2["log_probs"][0].requires_grad
+    _, ref = P.get_log_probs_and_entropy(logits.float(), args=args, unconcat_tokens=batch["unconcat_tokens"],
+                                         total_lengths=tot, response_lengths=resp, with_entropy=True)
+    for a, b in zip(out["log_probs"], ref["log_probs"]):
+        torch.testing.assert_close(a.cpu(), b, atol=2e-3, rtol=0)
+    for a, b in zip(out["entropy"], ref["entropy"]):
+        torch.testing.assert_close(a.cpu(), b, atol=2e-3, rtol=0)
+
+
+def test_grpo_micro_fixture_through_the_kernels(literals):
+    """Reference hand-derived fixture: loss = -0.02 at lp = old; fabricated logits give entropy != 0.5, so the
+    per-token kernel is driven directly with the fixture's per-token values."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("grpo micro fixture")
+    fx = literals["grpo_micro_fixture"]
+    adv = torch.tensor(fx["advantages"], device=dev)
+    cu = torch.tensor([0, 2, 4, 6, 8], device=dev)
+    for lp_val, want in ((0.0, None), (0.5, fx["lp_half_case"])):
+        out = ops.policy_loss(
+            log_prob=torch.full((8,), lp_val, device=dev), old_log_prob=torch.zeros(8, device=dev), advantages=adv,
+            loss_mask=torch.ones(8, device=dev), entropy=torch.full((8,), fx["entropy"], device=dev), cu_resp=cu,
+            sample_denom=torch.full((4,), 2.0, device=dev), entropy_coef=fx["entropy_coef"], eps_clip=0.2, eps_clip_high=0.2)
+        m = dict(zip(["loss", "pg_loss", "entropy_loss", "pg_clipfrac", "ppo_kl"], out["metrics"][:5].tolist()))
+        if want is None:
+            assert abs(m["loss"] - fx["default_loss"]) < 1e-6 and abs(m["pg_loss"]) < 1e-6
+        else:
+            for k in ("loss", "pg_loss", "pg_clipfrac", "ppo_kl", "entropy_loss"):
+                assert abs(m[k] - want[k]) < 2e-5, (k, m[k])
+
+
+def test_standalone_token_losses_vs_oracle():
+    from oracle import losses as L
+    from relax_amd import ppo_utils as K
+
+    dev = require_gpu()
+    announce("standalone token losses")
+    g = torch.Generator().manual_seed(9)
+    n = 777
+    lp = (torch.randn(n, generator=g) * 0.4 - 1).requires_grad_()
+    old = lp.detach() + torch.randn(n, generator=g) * 0.3
+    adv = torch.randn(n, generator=g)
+    adv[:6] = 0
+    w = torch.randn(n, generator=g)
+    lpd = lp.detach().to(dev).requires_grad_()
+
+    def cmp(ref_pair, got_pair, ref_leaf, got_leaf):
+        (ref_pair[0] * w).sum().backward()
+        (got_pair[0] * w.to(dev)).sum().backward()
+        torch.testing.assert_close(got_pair[0].detach().cpu(), ref_pair[0].detach(), atol=2e-5, rtol=1e-5)
+        torch.testing.assert_close(got_pair[1].cpu(), ref_pair[1], atol=0, rtol=0)
+        torch.testing.assert_close(got_leaf.grad.cpu(), ref_leaf.grad, atol=2e-5, rtol=1e-5)
+        ref_leaf.grad = None
+        got_leaf.grad = None
+
+    kl = (old - lp.detach()).requires_grad_()
+    kld = kl.detach().to(dev).requires_grad_()
+    cmp(L.policy_clip(kl, adv, 0.2, 0.28), K.compute_policy_loss(kld, adv.to(dev), 0.2, 0.28), kl, kld)
+    cmp(L.policy_clip(kl, adv, 0.2, 0.28, 3.0), K.compute_policy_loss(kld, adv.to(dev), 0.2, 0.28, 3.0), kl, kld)
+    cmp(L.sapo(kl, adv, 1.0, 1.05), K.compute_sapo_loss(kld, adv.to(dev), 1.0, 1.05), kl, kld)
+    cmp(L.cispo(lp, old - lp, adv, 0.2, 0.28), K.compute_cispo_loss(lpd, old.to(dev) - lpd, adv.to(dev), 0.2, 0.28), lp, lpd)
+    cmp(L.rloo_loss(lp, adv), K.compute_rloo_loss(lpd, adv.to(dev)), lp, lpd)
+    for kind in ("k1", "k2", "k3", "low_var_kl"):
+        ref = L.approx_kl(lp, old, kind)
+        got = K.compute_approx_kl(lpd, old.to(dev), kind)
+        (ref * w).sum().backward()
+        (got * w.to(dev)).sum().backward()
+        torch.testing.assert_close(got.detach().cpu(), ref.detach(), atol=2e-5, rtol=1e-5)
+        torch.testing.assert_close(lpd.grad.cpu(), lp.grad, atol=2e-5, rtol=1e-5)
+        lp.grad = None
+        lpd.grad = None
+    with pytest.raises(AssertionError):
+        K.compute_policy_loss(kld, adv.to(dev), 0.2, 0.2, 0.5)
+    # sequence KL (GSPO) as a standalone, with gradient
+    lens = [300, 77, 400]
+    masks = [(torch.rand(k, generator=g) > 0.4).float() for k in lens]
+    lps = list(torch.split(lp, lens))
+    ref = L.gspo_seq_kl(lps, list(torch.split(old, lens)), masks)
+    got = K.compute_gspo_kl(list(torch.split(lpd, lens)), [o.to(dev) for o in torch.split(old, lens)],
+                            list(torch.split(lpd, lens)), [m.to(dev) for m in masks])
+    (ref * w).sum().backward()
+    (got * w.to(dev)).sum().backward()
+    torch.testing.assert_close(got.detach().cpu(), ref.detach(), atol=2e-5, rtol=1e-5)
+    torch.testing.assert_close(lpd.grad.cpu(), lp.grad, atol=2e-5, rtol=1e-5)
+
+
+def test_reducers_vs_oracle_literals(literals):
+    from relax_amd import cp_utils
+
+    dev = require_gpu()
+    announce("reducers")
+    fx = literals["ppo_clip_k2_response_mean"]
+    masks = [torch.tensor(m, device=dev) for m in fx["masks"]]
+    red = cp_utils.get_sum_of_sample_mean(fx["response_lengths"], fx["response_lengths"], masks)
+    inv = literals["masked_invariance"]
+    a = red(torch.tensor(inv["base"], device=dev))
+    b = red(torch.tensor(inv["changed"], device=dev))
+    assert torch.equal(a, b) and abs(a.item() - (1.0 + 3.5)) < 1e-6
+    fx = literals["per_token_loss_path"]
+    masks = [torch.tensor(m, device=dev, dtype=torch.float64) for m in fx["masks"]]
+    lp = torch.tensor(fx["log_probs"], device=dev, requires_grad=True)
+    adv = torch.tensor(fx["advantages"], device=dev)
+    red = cp_utils.get_sum_of_sample_mean([3, 5], fx["response_lengths"], masks, calculate_per_token_loss=True)
+    n = cp_utils.get_cp_local_num_tokens([3, 5], fx["response_lengths"], masks)
+    assert n.item() == fx["expected_normalizer"]
+    total = red(-(adv * lp))
+    (total / n).backward()
+    flat = torch.cat(masks).float()
+    torch.testing.assert_close(total, -(adv * lp.detach() * flat).sum(), atol=1e-6, rtol=0)
+    torch.testing.assert_close(lp.grad, -(adv * flat) / 5, atol=1e-7, rtol=0)
+    fx = literals["target_coordinate_masks"]
+    m = [torch.tensor(fx["mask"], device=dev)]
+    red = cp_utils.get_sum_of_sample_mean([4], [4], m, calculate_per_token_loss=True)
+    assert red(torch.tensor(fx["values"], device=dev)).item() == fx["token_sum"]
+    assert cp_utils.get_cp_local_num_tokens([4], [4], m).item() == fx["count"]
