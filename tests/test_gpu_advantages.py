@@ -173,7 +173,7 @@ def test_full_vocab_reverse_kl_vs_oracle(n, v, dtype, tol):
     torch.testing.assert_close(got.detach().cpu(), want.detach(), atol=tol, rtol=0)
     assert abs(loss.item() - want_loss.item()) < tol
     assert sd.grad.dtype == dtype
-    torch.testing.assert_close(sd.grad.float().cpu(), sc.grad.float(), atol=tol, rtol=0)
+    torch.testing.assert_close(sd.grad.float().cpu(), sc.grad.float(), atol=tol, rtol=2.0 ** -7 if dtype == torch.bfloat16 else 0)
     assert (got >= -tol).all()
     same = compute_opd_kl_full_vocab(s.to(dev), s.to(dev))
     assert same.abs().max().item() < 1e-5
