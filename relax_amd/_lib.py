@@ -10,6 +10,11 @@ import ctypes as C
 import os
 import re
 
+# PyTorch ships its own copy of the HIP runtime (same soname as the system one).  It must be loaded BEFORE
+# librelax_amd.so so that both bind to one runtime instance: streams and device pointers are only meaningful inside
+# the runtime that created them, and a second instance reports "no ROCm-capable device".
+import torch  # noqa: F401
+
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "librelax_amd.so")
 HEADER_PATH = os.path.join(os.path.dirname(HERE), "include", "relax_amd.h")
