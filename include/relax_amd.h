@@ -211,6 +211,34 @@ int relax_amd_reverse_kl_bwd(const void* student, const void* teacher, int dtype
                              const float* g, float grad_scale, const float* grad_scale_dev, void* dstudent,
                              void* stream);
 
+/*
+ * Fused LM-head projection + log-prob / entropy: logits = hidden @ weight^T are formed tile by tile on the bf16
+ * matrix cores and reduced in registers; the [n_tokens, vocab] logits are never written.  Replaces the
+ * deferred-LM-head branch of get_log_probs_and_entropy (relax/backends/megatron/loss.py:391-419: per sub-chunk
+ * lm_head_forward -> .float() -> /T -> calculate_log_probs_and_entropy) and additionally returns the entropy.
+ *   hidden [n_tokens, hidden_size] bf16 (row stride h_stride), weight [vocab, hidden_size] bf16 (row stride w_stride)
+ *   hidden_size must be a multiple of 32; rows 16-byte aligned
+ *   workspace  relax_amd_lmhead_workspace_bytes(n_tokens) bytes of device memory
+ */
+int64_t relax_amd_lmhead_workspace_bytes(int64_t n_tokens);
+int relax_amd_lmhead_logprob_fwd(const void* hidden, const void* weight, int dtype, int64_t n_tokens,
+                                 int64_t hidden_size, int64_t vocab, int64_t h_stride, int64_t w_stride,
+                                 const int64_t* targets, float inv_temperature, void* workspace, float* log_prob,
+                                 float* entropy, float* lse, float* spx, void* stream);
+/*
+ * Backward helper of the fused LM head: recomputes the logits of n_tokens rows on the matrix cores and writes the
+ * gradient w.r.t. the logits, transposed and in bf16:
+ *   d_t[v, n] = inv_T * ( g_lp[n]*(onehot(target[n]) - p) + g_ent[n] * p * (spx[n] - x) ),  p = exp(x - lse[n])
+ * (autograd through F.linear + _VocabParallelLogProbEntropy.backward, ppo_utils.py:591-629).  The caller contracts
+ * d_t with weight (dhidden) and hidden (dweight) by plain GEMMs, slab by slab, so only one [vocab, n_tokens] slab
+ * exists at a time.  d_t has row stride d_stride >= n_tokens.
+ */
+int relax_amd_lmhead_dlogits_t(const void* hidden, const void* weight, int dtype, int64_t n_tokens,
+                               int64_t hidden_size, int64_t vocab, int64_t h_stride, int64_t w_stride,
+                               const int64_t* targets, const float* lse, const float* spx, const float* g_lp,
+                               const float* g_ent, const float* grad_scale_dev, float inv_temperature, void* d_t,
+                               int64_t d_stride, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

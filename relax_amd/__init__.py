@@ -1,6 +1,6 @@
 """relax_amd: MI355X (gfx950) kernels behind Relax's log-prob / entropy / policy-loss / advantage functions.
 
-Importing the package loads ``librelax_amd.so`` (built in-tree by ``python -m relax_amd.build``); it raises if the
+Importing the package loads ``librelax_amd.so`` (built in-tree by ``python relax_amd/build.py``); it raises if the
 library is missing -- there is no CPU or PyTorch fallback.
 """
 

@@ -64,6 +64,11 @@ SIGNATURES = {
     "relax_amd_whiten_partials": (_i64, [_i64]),
     "relax_amd_masked_whiten": (C.c_int, [_vp, _vp, _i64, _i32, _f32, _vp, _vp, _vp, _vp]),
     "relax_amd_reverse_kl_fwd": (C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "relax_amd_lmhead_workspace_bytes": (_i64, [_i64]),
+    "relax_amd_lmhead_logprob_fwd": (
+        C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _i64, _i64, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "relax_amd_lmhead_dlogits_t": (
+        C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _vp]),
     "relax_amd_reverse_kl_bwd": (C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp]),
 }
 
@@ -78,7 +83,7 @@ def declared_symbols(header_path: str = HEADER_PATH) -> list[str]:
 def _load() -> C.CDLL:
     if not os.path.exists(LIB_PATH):
         raise ImportError(
-            f"{LIB_PATH} is missing: build the HIP extension first (python -m relax_amd.build). "
+            f"{LIB_PATH} is missing: build the HIP extension first (python relax_amd/build.py). "
             "relax_amd has no CPU or PyTorch fallback."
         )
     lib = C.CDLL(LIB_PATH)

@@ -1,6 +1,6 @@
 """Builds ``librelax_amd.so`` (hand-written gfx950 HIP kernels + C ABI) in-tree with hipcc.
 
-Run as ``python -m relax_amd.build``.  The library is written next to this file so it travels with the source tree.
+Run as ``python relax_amd/build.py``.  The library is written next to this file so it travels with the source tree.
 """
 
 from __future__ import annotations

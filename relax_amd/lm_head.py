@@ -1,0 +1,129 @@
+"""Fused LM-head projection + log-prob / entropy on the gfx950 matrix cores.
+
+Counterpart of the deferred-LM-head branch of ``get_log_probs_and_entropy`` (relax/backends/megatron/loss.py:391-419)
+and ``_bypass_output_layer`` (relax/backends/megatron/model.py:93-181): instead of a callable that materialises
+``[sub_chunk, V]`` logits per sub-chunk, the caller passes the hidden states and the LM-head weight and the
+``[N, V]`` logits never reach HBM.  Unlike the reference's chunked path, entropy is available too.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import check, lib
+from .ops import _need_gpu, _p, _stream
+
+# rows of the transposed-gradient slab the backward materialises at a time: [V, SLAB] bf16
+BACKWARD_SLAB = 8192
+
+
+def _bf16_rows(t: torch.Tensor, what: str) -> torch.Tensor:
+    if t.dim() != 2:
+        raise ValueError(f"{what} must be 2-D, got {tuple(t.shape)}")
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"{what} must be bfloat16 (got {t.dtype}); cast before calling, as the reference's "
+                        f"_chunked_call casts the hidden states to the weight dtype")
+    if t.stride(1) != 1 or t.stride(0) % 8 != 0 or t.data_ptr() % 16 != 0:
+        t = t.contiguous()
+    return t
+
+
+def lmhead_logprob_fwd(hidden, weight, targets, inv_temperature: float = 1.0, with_entropy: bool = True):
+    """Returns (log_prob, entropy | None, lse, spx | None), fp32 [N]."""
+    dev = _need_gpu(hidden, weight, targets)
+    n, h = hidden.shape
+    v = weight.size(0)
+    if weight.size(1) != h:
+        raise ValueError(f"hidden size mismatch: hidden {tuple(hidden.shape)} vs weight {tuple(weight.shape)}")
+    kw = dict(dtype=torch.float32, device=dev)
+    lp, lse = torch.empty(n, **kw), torch.empty(n, **kw)
+    ent = torch.empty(n, **kw) if with_entropy else None
+    spx = torch.empty(n, **kw) if with_entropy else None
+    if n == 0:
+        return lp, ent, lse, spx
+    ws = torch.empty(lib.relax_amd_lmhead_workspace_bytes(n), dtype=torch.uint8, device=dev)
+    check(lib.relax_amd_lmhead_logprob_fwd(_p(hidden), _p(weight), _lib.BF16, n, h, v, hidden.stride(0),
+                                           weight.stride(0), _p(targets), float(inv_temperature), _p(ws), _p(lp),
+                                           _p(ent), _p(lse), _p(spx), _stream()))
+    return lp, ent, lse, spx
+
+
+def lmhead_dlogits_t(hidden, weight, targets, lse, spx, g_lp, g_ent, inv_temperature: float, out=None):
+    """bf16 [V, n] slab of d loss / d logits for the ``n`` rows of ``hidden`` (transposed: token-contiguous)."""
+    n, h = hidden.shape
+    v = weight.size(0)
+    if out is None:
+        out = torch.empty((v, n), dtype=torch.bfloat16, device=hidden.device)
+    check(lib.relax_amd_lmhead_dlogits_t(_p(hidden), _p(weight), _lib.BF16, n, h, v, hidden.stride(0),
+                                         weight.stride(0), _p(targets), _p(lse), _p(spx), _p(g_lp), _p(g_ent), None,
+                                         float(inv_temperature), _p(out), out.stride(0), _stream()))
+    return out
+
+
+class FusedLMHeadLogProb(torch.autograd.Function):
+    """(hidden [N,H] bf16, weight [V,H] bf16, targets [N]) -> (log_prob [N], entropy [N]).
+
+    Backward recomputes the logits slab by slab on the matrix cores, emits d loss / d logits for the slab in bf16
+    (never the full [N, V] tensor) and contracts it with the weight (dhidden) and the hidden states (dweight) with
+    plain library GEMMs; dweight is accumulated in fp32 across slabs.
+    """
+
+    @staticmethod
+    def forward(ctx, hidden, weight, targets, inv_temperature, with_entropy, with_entropy_grad):
+        with_entropy_grad = bool(with_entropy and with_entropy_grad)
+        hidden, weight = _bf16_rows(hidden, "hidden"), _bf16_rows(weight, "weight")
+        if targets.dtype != torch.int64 or not targets.is_contiguous():
+            targets = targets.to(torch.int64).contiguous()
+        lp, ent, lse, spx = lmhead_logprob_fwd(hidden, weight, targets, inv_temperature, with_entropy)
+        ctx.save_for_backward(hidden, weight, targets, lse, spx if with_entropy_grad else None)
+        ctx.inv_temperature = inv_temperature
+        ctx.with_entropy_grad = with_entropy_grad
+        if ent is None:
+            ent = lp.new_zeros((0,))
+        if not with_entropy_grad:
+            ctx.mark_non_differentiable(ent)
+        return lp, ent
+
+    @staticmethod
+    def backward(ctx, g_lp, g_ent):
+        hidden, weight, targets, lse, spx = ctx.saved_tensors
+        if g_lp is None:
+            raise RuntimeError("FusedLMHeadLogProb expected a materialized grad_log_prob")
+        g_lp = g_lp.reshape(-1).to(torch.float32).contiguous()
+        if not ctx.with_entropy_grad or g_ent is None or g_ent.numel() == 0:
+            g_ent = None
+        else:
+            g_ent = g_ent.reshape(-1).to(torch.float32).contiguous()
+        n, h = hidden.shape
+        v = weight.size(0)
+        need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        d_hidden = torch.empty_like(hidden) if need_h else None
+        d_weight32 = None
+        slab = torch.empty((v, min(n, BACKWARD_SLAB)), dtype=torch.bfloat16, device=hidden.device)
+        for s in range(0, n, BACKWARD_SLAB):
+            e = min(n, s + BACKWARD_SLAB)
+            d_t = slab[:, : e - s]
+            lmhead_dlogits_t(hidden[s:e], weight, targets[s:e], lse[s:e], None if spx is None else spx[s:e],
+                             g_lp[s:e], None if g_ent is None else g_ent[s:e], ctx.inv_temperature, out=d_t)
+            if need_h:
+                torch.mm(d_t.t(), weight, out=d_hidden[s:e])
+            if need_w:
+                part = torch.mm(d_t, hidden[s:e])
+                if s == 0 and e == n:
+                    return d_hidden, part, None, None, None, None
+                if d_weight32 is None:
+                    d_weight32 = part.to(torch.float32)
+                else:
+                    d_weight32.add_(part)
+        return d_hidden, (d_weight32.to(weight.dtype) if need_w else None), None, None, None, None
+
+
+def lm_head_log_probs_and_entropy(hidden, weight, tokens, temperature: float = 1.0, with_entropy: bool = False,
+                                  with_entropy_grad: bool = True):
+    """``(log_prob [N] fp32, entropy [N] fp32 | None)`` of ``log_softmax(hidden @ weight.T / temperature)``."""
+    lp, ent = FusedLMHeadLogProb.apply(hidden, weight, tokens, 1.0 / float(temperature), bool(with_entropy),
+                                       bool(with_entropy_grad))
+    return lp, (ent if with_entropy else None)

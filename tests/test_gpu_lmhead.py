@@ -1,0 +1,113 @@
+"""GPU parity of the fused LM-head + log-prob / entropy kernels against the oracle (F.linear + log-softmax).
+
+Tolerances follow the reference's own chunked-LM-head test for bf16 operands
+(tests/backends/megatron/test_sft_chunked_ce.py:119-134): loss / log-probs 2e-3 abs, gradients 5e-3 abs
+(+ one bf16 ulp of output rounding for the bf16 gradients).
+"""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import policy as P
+from tests.gpu_util import announce, require_gpu
+
+pytestmark = pytest.mark.gpu
+
+BF16_ULP = 2.0 ** -7
+
+
+def _inputs(n, h, v, seed, w_scale=0.02):
+    g = torch.Generator().manual_seed(seed)
+    hid = torch.randn(n, h, generator=g).bfloat16()
+    w = (torch.randn(v, h, generator=g) * w_scale).bfloat16()
+    tok = torch.randint(0, v, (n,), generator=g)
+    return hid, w, tok, g
+
+
+def _oracle(hid, w, tok, wl, we, temperature):
+    h32 = hid.float().requires_grad_()
+    w32 = w.float().requires_grad_()
+    logits = F.linear(h32, w32) / temperature
+    ls = torch.log_softmax(logits, -1)
+    lp = ls[torch.arange(hid.size(0)), tok]
+    ent = -(ls.exp() * ls).sum(-1)
+    ((lp * wl).sum() + (ent * we).sum()).backward()
+    return lp.detach(), ent.detach(), h32.grad, w32.grad
+
+
+@pytest.mark.parametrize("n,h,v,temperature", [
+    (256, 64, 256, 1.0),        # exactly one tile
+    (300, 128, 1000, 0.7),      # ragged tokens and ragged vocabulary
+    (1024, 256, 5000, 1.0),     # several vocab tiles and splits
+    (70, 4096, 1030, 1.0),      # production hidden size
+])
+def test_forward_backward_vs_oracle(n, h, v, temperature):
+    from relax_amd.lm_head import lm_head_log_probs_and_entropy
+
+    dev = require_gpu()
+    announce("lmhead", n, h, v, temperature)
+    hid, w, tok, g = _inputs(n, h, v, seed=n + v, w_scale=0.3 if h < 1024 else 0.05)
+    # incoming gradients of the size a mean-reduced loss produces: the backward rounds d loss / d logits to bf16
+    # (as autograd does in the reference when the LM head runs in bf16), so O(1) coefficients would put single
+    # elements beyond an absolute 5e-3
+    wl, we = torch.randn(n, generator=g) / 16, torch.randn(n, generator=g) / 32
+    rlp, rent, rgh, rgw = _oracle(hid, w, tok, wl, we, temperature)
+    hd, wd = hid.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    lp, ent = lm_head_log_probs_and_entropy(hd, wd, tok.to(dev), temperature, with_entropy=True)
+    assert lp.dtype == torch.float32 and lp.shape == (n,) and ent.shape == (n,)
+    torch.testing.assert_close(lp.cpu(), rlp, atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent.cpu(), rent, atol=2e-3, rtol=0)
+    ((lp * wl.to(dev)).sum() + (ent * we.to(dev)).sum()).backward()
+    assert hd.grad.dtype == torch.bfloat16 and wd.grad.dtype == torch.bfloat16
+    torch.testing.assert_close(hd.grad.float().cpu(), rgh, atol=5e-3, rtol=2 * BF16_ULP)
+    torch.testing.assert_close(wd.grad.float().cpu(), rgw, atol=5e-3, rtol=2 * BF16_ULP)
+    # deterministic
+    lp2, _ = lm_head_log_probs_and_entropy(hid.to(dev), w.to(dev), tok.to(dev), temperature, with_entropy=True)
+    assert torch.equal(lp2, lp.detach())
+
+
+def test_reference_shaped_case_temperature_and_labels():
+    """Shape of the reference's own deferred-LM-head test (T=256, H=32, V=64, weight*0.02, temperature 0.7)."""
+    from relax_amd.lm_head import lm_head_log_probs_and_entropy
+
+    dev = require_gpu()
+    announce("lmhead reference-shaped")
+    torch.manual_seed(0)
+    hid = torch.randn(256, 32).bfloat16()
+    w = (torch.randn(64, 32) * 0.02).bfloat16()
+    tok = torch.randint(0, 64, (256,))
+    labels = F.pad(tok[1:], (0, 1), value=0)  # SFT alignment: labels are tokens[1:] + [0]
+    want = P.lm_head_log_probs(hid, w, labels, temperature=0.7, sub_chunk=64)
+    got, ent = lm_head_log_probs_and_entropy(hid.to(dev), w.to(dev), labels.to(dev), 0.7)
+    assert ent is None
+    torch.testing.assert_close(got.cpu(), want, atol=2e-3, rtol=0)
+
+
+def test_slabbed_backward_accumulates_dweight(monkeypatch):
+    import relax_amd.lm_head as LH
+
+    dev = require_gpu()
+    announce("lmhead slabbed backward")
+    monkeypatch.setattr(LH, "BACKWARD_SLAB", 256)
+    n, h, v = 700, 64, 900
+    hid, w, tok, g = _inputs(n, h, v, seed=3, w_scale=0.3)
+    wl = torch.randn(n, generator=g) / 16
+    rlp, _, rgh, rgw = _oracle(hid, w, tok, wl, torch.zeros(n), 1.0)
+    hd, wd = hid.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    lp, _ = LH.lm_head_log_probs_and_entropy(hd, wd, tok.to(dev))
+    (lp * wl.to(dev)).sum().backward()
+    torch.testing.assert_close(hd.grad.float().cpu(), rgh, atol=5e-3, rtol=2 * BF16_ULP)
+    torch.testing.assert_close(wd.grad.float().cpu(), rgw, atol=5e-3, rtol=2 * BF16_ULP)
+
+
+def test_argument_errors():
+    from relax_amd.lm_head import lm_head_log_probs_and_entropy
+
+    dev = require_gpu()
+    hid = torch.randn(8, 48, device=dev).bfloat16()  # hidden size not a multiple of 32
+    w = torch.randn(16, 48, device=dev).bfloat16()
+    with pytest.raises(Exception, match="multiple of 32"):
+        lm_head_log_probs_and_entropy(hid, w, torch.zeros(8, dtype=torch.long, device=dev))
+    with pytest.raises(TypeError, match="bfloat16"):
+        lm_head_log_probs_and_entropy(hid.float(), w, torch.zeros(8, dtype=torch.long, device=dev))
