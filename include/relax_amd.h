@@ -212,6 +212,32 @@ int relax_amd_reverse_kl_bwd(const void* student, const void* teacher, int dtype
                              void* stream);
 
 /*
+ * Fused actor step: log-prob + entropy forward, the per-token terms of relax_amd_policy_loss and the dlogits backward
+ * in one launch.  Each workgroup scans its row, derives the token's gradient constants and immediately walks the row
+ * again to emit dlogits; the second walk is served by the L2 / memory-side cache, so HBM sees one read and one write
+ * per row.  Replaces, for one micro-batch, _VocabParallelLogProbEntropy.forward + .backward (ppo_utils.py:481-629)
+ * fused with the per-token part of policy_loss_function (loss.py:961-1100).  Available when d loss / d log_prob of a
+ * token depends on that token only: every loss kind except GSPO, no OPSM (those return RELAX_AMD_EUNSUPPORTED).
+ * Its log-probs / entropy are bit-identical to relax_amd_logprob_entropy_fwd's on the same rows.
+ *   loss        the same argument block relax_amd_policy_loss takes; its log_prob / entropy inputs are ignored
+ *               (they are produced here), coef_log_prob / coef_entropy are written; metrics are NOT produced: call
+ *               relax_amd_policy_loss afterwards with log_prob / entropy set to this call's outputs
+ *   sample_ids  [n_tokens] int32 sample of each token (needed with per-sample denominators)
+ *   grad_scale  host scalar folded into dlogits (the upstream gradient the caller expects, normally 1)
+ *   log_prob, entropy, lse, spx  [n_tokens] out; tokens whose masks are both zero get zeros (their row is not read)
+ *   dlogits     [n_rows, vocab] out, every row written (zero rows where token_of_row < 0 or the coefficients vanish)
+ */
+int relax_amd_actor_step_fused(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                               const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,
+                               float inv_temperature, const relax_amd_policy_loss_args* loss, float grad_scale,
+                               float* log_prob, float* entropy, float* lse, float* spx, void* dlogits,
+                               int64_t d_row_stride, void* stream);
+/* data[row, :] *= *factor_dev in place; returns immediately on the device when the factor is exactly 1.  Lets an
+ * autograd backward apply an upstream scalar that differs from the grad_scale assumed above without a host read. */
+int relax_amd_scale_rows_inplace(void* data, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                                 const float* factor_dev, void* stream);
+
+/*
  * Fused LM-head projection + log-prob / entropy: logits = hidden @ weight^T are formed tile by tile on the bf16
  * matrix cores and reduced in registers; the [n_tokens, vocab] logits are never written.  Replaces the
  * deferred-LM-head branch of get_log_probs_and_entropy (relax/backends/megatron/loss.py:391-419: per sub-chunk

@@ -64,6 +64,10 @@ SIGNATURES = {
     "relax_amd_whiten_partials": (_i64, [_i64]),
     "relax_amd_masked_whiten": (C.c_int, [_vp, _vp, _i64, _i32, _f32, _vp, _vp, _vp, _vp]),
     "relax_amd_reverse_kl_fwd": (C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "relax_amd_actor_step_fused": (
+        C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _vp, _f32, C.POINTER(PolicyLossArgs), _f32, _vp, _vp, _vp,
+                  _vp, _vp, _i64, _vp]),
+    "relax_amd_scale_rows_inplace": (C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp]),
     "relax_amd_lmhead_workspace_bytes": (_i64, [_i64]),
     "relax_amd_lmhead_logprob_fwd": (
         C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _i64, _i64, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -1,136 +1,46 @@
 // Streaming log-prob + entropy forward and dlogits backward over [rows, vocab] logits.
 //
 // One workgroup owns one row.  The row is read once with 16-byte non-temporal loads (8 bf16 / 4 fp32 per lane
-// per load, UNROLL loads in flight per lane); every lane keeps a private online-softmax state (running max, sum of
+// per load, 4 loads in flight per lane); every lane keeps a private online-softmax state (running max, sum of
 // exp, sum of exp * x) in the log2 domain so the inner loop is cvt + fma + v_exp_f32 + add + fma per element and the
-// max rescale is paid once per UNROLL*8 elements.  Lane states are merged by a wave64 xor-butterfly, then across
-// waves through LDS in wave order, so results are bit-identical run to run.
+// max rescale is paid once per 32 elements (row_scan.h).  Lane states are merged by a wave64 xor-butterfly, then
+// across waves through LDS in wave order, so results are bit-identical run to run and identical to the forward
+// half of the fused actor-step kernel.
 //
 // Arithmetic follows relax/utils/training/ppo_utils.py:481-629 (reference paths are relative to its checkout):
 //   lp = x[tok] - lse,  H = lse - sum_v p*x,  dx = g_lp*(onehot - p) + g_H*p*(sum_v p*x - x),  x = logits / T.
 #include "device_utils.h"
 #include "relax_amd.h"
+#include "row_scan.h"
 
 namespace relax_amd {
 
-constexpr int kRowThreads = 256;
+constexpr int kRowThreads = 256;  // backward kernel width
 constexpr int kRowUnroll = 4;
 
-struct SoftmaxState {
-  float m, s, t;  // max of x*c, sum exp2(x*c - m), sum exp2(x*c - m) * x
-};
-
-template <bool ENTROPY, int K>
-__device__ __forceinline__ void absorb(const float (&v)[K], float c, SoftmaxState& st) {
-  float vmax = v[0];
-#pragma unroll
-  for (int i = 1; i < K; ++i) vmax = fmaxf(vmax, v[i]);
-  const float mc = vmax * c;
-  if (mc > st.m) {
-    const float sc = fast_exp2(st.m - mc);
-    st.s *= sc;
-    st.t *= sc;
-    st.m = mc;
-  }
-#pragma unroll
-  for (int i = 0; i < K; ++i) {
-    const float e = fast_exp2(fmaf(v[i], c, -st.m));
-    st.s += e;
-    if (ENTROPY) st.t = fmaf(e, v[i], st.t);
-  }
-}
-
-__device__ __forceinline__ void merge(SoftmaxState& a, float m2, float s2, float t2) {
-  const float mn = fmaxf(a.m, m2);
-  const float fa = fast_exp2(a.m - mn), fb = fast_exp2(m2 - mn);
-  a.s = a.s * fa + s2 * fb;
-  a.t = a.t * fa + t2 * fb;
-  a.m = mn;
-}
-
-// Reduce the per-lane states of a workgroup; the merged state is valid in thread 0.
-template <int THREADS>
-__device__ __forceinline__ void block_merge(SoftmaxState& st, float (*lds)[3]) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) {
-    const float m2 = __shfl_xor(st.m, o, kWave), s2 = __shfl_xor(st.s, o, kWave), t2 = __shfl_xor(st.t, o, kWave);
-    merge(st, m2, s2, t2);
-  }
-  const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
-  if (lane == 0) {
-    lds[w][0] = st.m;
-    lds[w][1] = st.s;
-    lds[w][2] = st.t;
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-#pragma unroll
-    for (int i = 1; i < THREADS / kWave; ++i) merge(st, lds[i][0], lds[i][1], lds[i][2]);
-  }
-}
-
-// Absorb one row into `st`.  VEC selects 16-byte loads (row base and stride 16-byte aligned) or scalar loads.
-template <typename T, bool ENTROPY, bool VEC, int THREADS, int UNROLL>
-__device__ __forceinline__ void scan_row(const T* __restrict__ x, int64_t vocab, float c, SoftmaxState& st) {
-  if (VEC) {
-    constexpr int VN = Row<T>::kPerVec;
-    const u32x4* xv = reinterpret_cast<const u32x4*>(x);
-    const int64_t nvec = vocab / VN;
-    int64_t i = threadIdx.x;
-    for (; i + int64_t(UNROLL - 1) * THREADS < nvec; i += int64_t(UNROLL) * THREADS) {
-      u32x4 raw[UNROLL];
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) raw[u] = load_stream(xv + i + int64_t(u) * THREADS);
-      float v[UNROLL * VN];
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        float part[VN];
-        Row<T>::unpack(raw[u], part);
-#pragma unroll
-        for (int k = 0; k < VN; ++k) v[u * VN + k] = part[k];
-      }
-      absorb<ENTROPY>(v, c, st);
-    }
-    for (; i < nvec; i += THREADS) {
-      float v[VN];
-      Row<T>::unpack(load_stream(xv + i), v);
-      absorb<ENTROPY>(v, c, st);
-    }
-    for (int64_t e = nvec * VN + threadIdx.x; e < vocab; e += THREADS) {
-      float v[1] = {Row<T>::load1(x + e)};
-      absorb<ENTROPY>(v, c, st);
-    }
-  } else {
-    for (int64_t e = threadIdx.x; e < vocab; e += THREADS) {
-      float v[1] = {Row<T>::load1(x + e)};
-      absorb<ENTROPY>(v, c, st);
-    }
-  }
-}
-
-template <typename T, bool ENTROPY, bool VEC>
-__global__ __launch_bounds__(kRowThreads) void logprob_entropy_fwd_kernel(
+template <typename T, bool VEC, int THREADS>
+__global__ __launch_bounds__(THREADS) void logprob_entropy_fwd_kernel(
     const T* __restrict__ logits, int64_t row_stride, int64_t vocab, const int32_t* __restrict__ row_ids,
     const int64_t* __restrict__ targets, float c, float inv_t, float* __restrict__ log_prob,
     float* __restrict__ entropy, float* __restrict__ lse_out, float* __restrict__ spx_out) {
-  __shared__ float lds[kRowThreads / kWave][3];
+  __shared__ float wave_state[THREADS / kWave][3];
   const int64_t tok = blockIdx.x;
   const int64_t row = row_ids ? int64_t(row_ids[tok]) : tok;
   const T* x = logits + row * row_stride;
-  SoftmaxState st{kNegHuge, 0.f, 0.f};
-  scan_row<T, ENTROPY, VEC, kRowThreads, kRowUnroll>(x, vocab, c, st);
-  block_merge<kRowThreads>(st, lds);
+  float x_target = 0.f;
+  int64_t tg = -1;
   if (threadIdx.x == 0) {
-    const float lse = st.m * kLn2 + logf(st.s);
-    const int64_t tg = targets[tok];
-    float lp = __builtin_nanf("");
-    if (tg >= 0 && tg < vocab) lp = Row<T>::load1(x + tg) * inv_t - lse;
+    tg = targets[tok];
+    if (tg >= 0 && tg < vocab) x_target = Row<T>::load1(x + tg);
+  }
+  SoftmaxAcc st = scan_row<T, VEC, true, THREADS>(x, vocab, c);
+  scan_block_merge<THREADS>(st, wave_state);
+  if (threadIdx.x == 0) {
+    float lse, spx, ent, lp;
+    scan_finish(st, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
     log_prob[tok] = lp;
-    const float spx = (st.t / st.s) * inv_t;
-    if (ENTROPY) {
-      if (entropy) entropy[tok] = lse - spx;
-      if (spx_out) spx_out[tok] = spx;
-    }
+    if (entropy) entropy[tok] = ent;
+    if (spx_out) spx_out[tok] = spx;
     if (lse_out) lse_out[tok] = lse;
   }
 }
@@ -236,17 +146,20 @@ static int launch_fwd(const void* logits, int64_t n, int64_t vocab, int64_t stri
                       const int64_t* targets, float inv_t, float* lp, float* ent, float* lse, float* spx,
                       hipStream_t s) {
   const bool vec = aligned16(logits) && (stride * int64_t(sizeof(T))) % 16 == 0;
-  const bool with_ent = ent != nullptr || spx != nullptr;
   const float c = inv_t * kLog2e;
   const T* x = static_cast<const T*>(logits);
-  dim3 grid(static_cast<unsigned>(n)), block(kRowThreads);
-#define RELAX_AMD_FWD(E, V) \
-  hipLaunchKernelGGL((logprob_entropy_fwd_kernel<T, E, V>), grid, block, 0, s, x, stride, vocab, row_ids, targets, c, \
-                     inv_t, lp, ent, lse, spx)
-  if (with_ent) {
-    if (vec) RELAX_AMD_FWD(true, true); else RELAX_AMD_FWD(true, false);
+  dim3 grid(static_cast<unsigned>(n));
+#define RELAX_AMD_FWD(V, TH)                                                                                        \
+  hipLaunchKernelGGL((logprob_entropy_fwd_kernel<T, V, TH>), grid, dim3(TH), 0, s, x, stride, vocab, row_ids, targets, \
+                     c, inv_t, lp, ent, lse, spx)
+  if (!vec) {
+    RELAX_AMD_FWD(false, 256);
   } else {
-    if (vec) RELAX_AMD_FWD(false, true); else RELAX_AMD_FWD(false, false);
+    switch (scan_threads(vocab, Row<T>::kPerVec)) {
+      case 1024: RELAX_AMD_FWD(true, 1024); break;
+      case 512: RELAX_AMD_FWD(true, 512); break;
+      default: RELAX_AMD_FWD(true, 256); break;
+    }
   }
 #undef RELAX_AMD_FWD
   return check_launch("logprob_entropy_fwd");

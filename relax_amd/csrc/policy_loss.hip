@@ -19,98 +19,20 @@
 //   k1: 1   k2: d   k3 / low_var: 1-exp(-d)  (low_var: 0 outside the [-10,10] clamp)
 //   unbiased KL multiplies by ratio = exp(lp-old) and adds ratio*kl (the ratio is not detached, loss.py:1091)
 #include "device_utils.h"
+#include "loss_math.h"
 #include "relax_amd.h"
 
 namespace relax_amd {
 
 constexpr int kLossThreads = 512;
 
-struct TokenTerms {
-  float pg, clipfrac, ppo_kl, dpg_dlp, dpg_dkl;
-};
-
-// One token of compute_policy_loss / compute_cispo_loss / compute_rloo_loss / compute_sapo_loss.
-// `kl` is old - lp (token-level) or the sequence KL (GSPO).  dpg_dlp is the derivative through a token-level kl
-// (d kl / d lp = -1) plus any direct lp dependence; dpg_dkl is the derivative w.r.t. kl itself (used by GSPO).
-__device__ __forceinline__ TokenTerms token_loss(int kind, float lp, float kl, float adv, float eps_lo, float eps_hi,
-                                                 float eps_c, float tau_pos, float tau_neg) {
-  TokenTerms t;
-  t.ppo_kl = kl;
-  const float r = expf(-kl);
-  if (kind == RELAX_AMD_LOSS_CISPO) {
-    const float hi = 1.0f + eps_hi, lo = 1.0f - eps_lo;
-    const float coef = adv >= 0.f ? fminf(r, hi) : fmaxf(r, lo);
-    t.pg = -(coef * adv * lp);
-    t.clipfrac = ((adv >= 0.f && r > hi) ? 1.f : 0.f) + ((adv < 0.f && r < lo) ? 1.f : 0.f);
-    t.dpg_dlp = -(coef * adv);
-    t.dpg_dkl = 0.f;
-    return t;
-  }
-  if (kind == RELAX_AMD_LOSS_RLOO) {
-    t.pg = -(adv * lp);
-    t.clipfrac = 0.f;
-    t.dpg_dlp = -adv;
-    t.dpg_dkl = 0.f;
-    return t;
-  }
-  if (kind == RELAX_AMD_LOSS_SAPO) {
-    const float tau = adv > 0.f ? tau_pos : tau_neg;
-    const float s = 1.0f / (1.0f + expf(-tau * (r - 1.0f)));
-    t.pg = -((4.0f / tau) * s * adv);
-    t.clipfrac = (4.0f * s * (1.0f - s)) < 0.9f ? 1.f : 0.f;
-    // d pg / d r = -(4/tau)*adv*tau*s*(1-s);  d r / d kl = -r
-    t.dpg_dkl = 4.0f * adv * s * (1.0f - s) * r;
-    t.dpg_dlp = -t.dpg_dkl;
-    return t;
-  }
-  // PPO clip (also the per-token function GSPO applies to the sequence KL)
-  const float lo = 1.0f - eps_lo, hi = 1.0f + eps_hi;
-  const float l1 = -r * adv;
-  const float rc = fminf(fmaxf(r, lo), hi);
-  const float l2 = -rc * adv;
-  float loss = fmaxf(l1, l2);
-  t.clipfrac = l2 > l1 ? 1.f : 0.f;
-  const bool inside = (r >= lo) && (r <= hi);
-  float dl_dr = (inside || l1 > l2) ? -adv : 0.f;  // ties outside the range only occur at adv == 0
-  if (eps_c > 0.f && adv < 0.f) {
-    const float l3 = -eps_c * adv;
-    if (l3 < loss) {
-      loss = l3;
-      dl_dr = 0.f;
-    } else if (l3 == loss) {
-      dl_dr *= 0.5f;
-    }
-  }
-  t.pg = loss;
-  t.dpg_dkl = -dl_dr * r;  // d r / d kl = -r
-  t.dpg_dlp = dl_dr * r;
-  return t;
-}
-
-__device__ __forceinline__ void kl_term(int kind, float lp, float ref, float& kl, float& dkl_dlp) {
-  const float d = lp - ref;
-  if (kind == RELAX_AMD_KL_K1) {
-    kl = d;
-    dkl_dlp = 1.f;
-  } else if (kind == RELAX_AMD_KL_K2) {
-    kl = d * d / 2.0f;
-    dkl_dlp = d;
-  } else {
-    const float e = expf(-d);
-    kl = e - 1.0f - (-d);
-    dkl_dlp = 1.0f - e;
-  }
-}
-
 __global__ __launch_bounds__(kLossThreads) void policy_loss_sample_kernel(relax_amd_policy_loss_args a) {
   __shared__ float red[kLossThreads / kWave];
   const int64_t i = blockIdx.x;
   const int64_t beg = a.cu_resp[i], end = a.cu_resp[i + 1];
   const bool gspo = a.loss_kind == RELAX_AMD_LOSS_GSPO;
-  const int kind = gspo ? RELAX_AMD_LOSS_PPO : a.loss_kind;
   const float den = a.sample_denom ? a.sample_denom[i] : 1.0f;
   const float pg_den = a.pg_sample_denom ? a.pg_sample_denom[i] : den;
-  const float* pg_mask = a.pg_loss_mask ? a.pg_loss_mask : a.loss_mask;
 
   float seq_kl = 0.f, seq_cnt = 1.f;
   if (gspo || a.use_opsm) {
@@ -134,75 +56,17 @@ __global__ __launch_bounds__(kLossThreads) void policy_loss_sample_kernel(relax_
   float g_seq = 0.f;  // GSPO: sum_t w_t * d pg_t / d kl_i
 
   for (int64_t t = beg + threadIdx.x; t < end; t += kLossThreads) {
-    const float lp = a.log_prob[t];
-    const float old = a.old_log_prob ? a.old_log_prob[t] : lp;
-    const float adv = a.advantages[t];
-    const float m = a.loss_mask[t];
-    const float mp = pg_mask[t];
-    const float kl_in = gspo ? seq_kl : (old - lp);
-    TokenTerms tt = token_loss(kind, lp, kl_in, adv, a.eps_clip, a.eps_clip_high, a.eps_clip_c, a.tau_pos, a.tau_neg);
-    float w = 1.0f;  // multiplicative, gradient-free weights on pg_loss
-    float drop = 0.f;
-    if (a.use_opsm) {
-      drop = (adv < 0.f && seq_kl > a.opsm_delta) ? 1.f : 0.f;
-      w *= 1.0f - drop;
-    }
-    float tis = 0.f, log_ratio = 0.f, tis_w = 1.f;
-    const bool have_tis = (a.use_tis || a.mismatch_metrics) && a.rollout_log_prob;
-    if (have_tis) {
-      log_ratio = (a.train_log_prob ? a.train_log_prob[t] : lp) - a.rollout_log_prob[t];
-      tis = expf(log_ratio);
-      tis_w = fminf(fmaxf(tis, a.tis_lo), a.tis_hi);
-      w *= tis_w;
-    }
-    const float pg = tt.pg * w;
-    float c_lp = (mp / pg_den) * w * (gspo ? 0.f : tt.dpg_dlp);
-    if (gspo) g_seq += (mp / pg_den) * w * tt.dpg_dkl;
-
-    acc[RELAX_AMD_M_PG_LOSS] += pg * mp;
-    acc[RELAX_AMD_M_CLIPFRAC] += tt.clipfrac * m;
-    acc[RELAX_AMD_M_PPO_KL] += tt.ppo_kl * m;
-    acc[RELAX_AMD_M_MASK_SUM] += m;
-    if (a.entropy) acc[RELAX_AMD_M_ENTROPY] += a.entropy[t] * m;
-    if (a.pg_loss_tok) a.pg_loss_tok[t] = pg;
-    if (a.clipfrac_tok) a.clipfrac_tok[t] = tt.clipfrac;
-    if (a.ppo_kl_tok) a.ppo_kl_tok[t] = tt.ppo_kl;
-
-    if (a.kl_kind != RELAX_AMD_KL_NONE) {
-      float kl, dkl;
-      kl_term(a.kl_kind, lp, a.ref_log_prob[t], kl, dkl);
-      if (a.unbiased_kl) {
-        const float ratio = expf(lp - old);
-        dkl = ratio * dkl + ratio * kl;  // ratio carries gradient (d ratio / d lp = ratio)
-        kl = ratio * kl;
-      }
-      if (a.kl_kind == RELAX_AMD_KL_LOW_VAR) {
-        if (kl < -10.f || kl > 10.f) dkl = 0.f;
-        kl = fminf(fmaxf(kl, -10.f), 10.f);
-      }
-      acc[RELAX_AMD_M_KL_LOSS] += kl * m;
-      c_lp += a.kl_coef * (m / den) * dkl;
-      if (a.kl_tok) a.kl_tok[t] = kl;
-    }
-    if (a.rollout_log_prob) {
-      const float roll = a.rollout_log_prob[t];
-      float side = lp;
-      if (a.abs_diff_from_old == 1) side = old;
-      else if (a.abs_diff_from_old == 0 && a.train_log_prob) side = a.train_log_prob[t];
-      acc[RELAX_AMD_M_LOGPROB_ABS_DIFF] += fabsf(side - roll) * m;
-      acc[RELAX_AMD_M_PROB_ABS_DIFF] += fabsf(expf(side) - expf(roll)) * m;
-    }
-    if (have_tis) {
-      acc[RELAX_AMD_M_OIS] += expf(-tt.ppo_kl) * m;
-      acc[RELAX_AMD_M_TIS] += tis * m;
-      acc[RELAX_AMD_M_TIS_CLIPFRAC] += (tis_w != tis ? 1.f : 0.f) * m;
-      acc[RELAX_AMD_M_TIS_ABS] += fabsf(tis - 1.0f) * m;
-      acc[RELAX_AMD_M_MISMATCH_KL] += (-log_ratio) * m;
-      acc[RELAX_AMD_M_MISMATCH_K3] += (tis - log_ratio - 1.0f) * m;
-    }
-    acc[RELAX_AMD_M_OPSM_CLIPFRAC] += drop;
-    a.coef_log_prob[t] = c_lp;
-    if (a.coef_entropy) a.coef_entropy[t] = -a.entropy_coef * (m / den);
+    const TokenInputs in = load_token_inputs(a, t);
+    TokenResult tr = token_terms(a, in, a.log_prob[t], a.entropy ? a.entropy[t] : 0.f, gspo, seq_kl, den, pg_den);
+#pragma unroll
+    for (int k = 0; k < RELAX_AMD_NUM_METRICS; ++k) acc[k] += tr.metric[k];
+    g_seq += tr.g_seq;
+    if (a.pg_loss_tok) a.pg_loss_tok[t] = tr.pg;
+    if (a.clipfrac_tok) a.clipfrac_tok[t] = tr.clipfrac;
+    if (a.ppo_kl_tok) a.ppo_kl_tok[t] = tr.ppo_kl;
+    if (a.kl_tok && a.kl_kind != RELAX_AMD_KL_NONE) a.kl_tok[t] = tr.kl;
+    a.coef_log_prob[t] = tr.coef_lp;
+    if (a.coef_entropy) a.coef_entropy[t] = tr.coef_ent;
   }
 
 #pragma unroll

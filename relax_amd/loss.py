@@ -159,8 +159,8 @@ def get_log_probs_and_entropy(
 
 
 class _FusedPolicyLoss(torch.autograd.Function):
-    """logits [T, V] -> scalar loss.  Forward: one log-prob/entropy launch + the policy-loss launches; backward:
-    one dlogits launch fed with the stored d loss / d lp and d loss / d entropy coefficients."""
+    """logits [T, V] -> scalar loss, two-launch form.  Forward: one log-prob/entropy launch + the policy-loss
+    launches; backward: one dlogits launch fed with the stored d loss / d lp and d loss / d entropy coefficients."""
 
     @staticmethod
     def forward(ctx, flat, lay, inv_t, kw):
@@ -181,6 +181,39 @@ class _FusedPolicyLoss(torch.autograd.Function):
         d = ops.logprob_entropy_bwd(flat, targets, lse, spx, c_lp, c_ent, token_of_row=token_of_row,
                                     grad_scale_dev=scale, inv_temperature=ctx.inv_t)
         return d, None, None, None
+
+
+class _SinglePassPolicyLoss(torch.autograd.Function):
+    """logits [T, V] -> scalar loss, single-launch form: each workgroup scans its row and at once walks it again
+    (out of cache) to write dlogits for an upstream gradient of 1, so HBM sees one read and one write per row.  The
+    backward multiplies by the actual upstream gradient on the device (a no-op kernel when it is exactly 1)."""
+
+    @staticmethod
+    def forward(ctx, flat, lay, inv_t, kw):
+        out, lp, ent, _lse, _spx, dlogits = ops.actor_step_fused(
+            flat, lay.targets, lay.token_of_row, lay.sample_ids, lay.n_tokens, inv_t, 1.0, cu_resp=lay.cu_resp, **kw)
+        metrics = out["metrics"]
+        ctx.dlogits = dlogits
+        ctx.mark_non_differentiable(metrics, lp, ent)
+        return metrics[_SLOT["loss"]].clone(), metrics, lp, ent
+
+    @staticmethod
+    def backward(ctx, g_loss, _gm, _glp, _gent):
+        d = ctx.dlogits
+        if d is None:
+            raise RuntimeError("the single-pass policy loss holds its gradient once: backward cannot run twice")
+        ctx.dlogits = None
+        ops.scale_rows_inplace(d, g_loss.reshape(1).to(torch.float32).contiguous())
+        return d, None, None, None
+
+
+def _single_pass_ok(args, flat, kw, needs_bwd) -> bool:
+    mode = getattr(args, "relax_amd_single_pass", "auto")
+    if mode in (False, "off") or not needs_bwd:
+        return False
+    if kw["loss_kind"] == "gspo" or kw["use_opsm"]:
+        return False  # sequence-coupled gradients need the per-sequence reduction between forward and backward
+    return True
 
 
 def _cat_f32(parts, device):
@@ -270,7 +303,8 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         if use_kl:
             metrics["kl_loss"] = zero.clone()
         return loss, metrics
-    loss, mvec, lp, ent = _FusedPolicyLoss.apply(flat, lay, inv_t, kw)
+    fn = _SinglePassPolicyLoss if _single_pass_ok(args, flat, kw, needs_bwd) else _FusedPolicyLoss
+    loss, mvec, lp, ent = fn.apply(flat, lay, inv_t, kw)
 
     def m(name):
         return mvec[_SLOT[name]]

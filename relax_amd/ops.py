@@ -166,20 +166,21 @@ def segment_sum(mask, cu_resp, values=None):
 # ---------------------------------------------------------------------------------------------------- policy loss
 
 
-def policy_loss(*, log_prob, advantages, loss_mask, cu_resp, old_log_prob=None, ref_log_prob=None,
-                train_log_prob=None, rollout_log_prob=None, entropy=None, pg_loss_mask=None, sample_denom=None,
-                pg_sample_denom=None, loss_kind="ppo", kl_kind=None, unbiased_kl=False, use_opsm=False, use_tis=False,
-                mismatch_metrics=False, abs_diff_from_old=1, eps_clip=0.2, eps_clip_high=0.2, eps_clip_c=None,
-                entropy_coef=0.0, kl_coef=0.0, tis_lo=0.0, tis_hi=2.0, opsm_delta=1e-4, tau_pos=1.0, tau_neg=1.05,
-                per_token_outputs=False):
-    """Runs the two policy-loss launches.  Returns dict(metrics [16], coef_log_prob, coef_entropy, per-token...)."""
-    dev = _need_gpu(log_prob, advantages, loss_mask, cu_resp)
-    n = int(log_prob.numel())
+def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_prob=None, ref_log_prob=None,
+                 train_log_prob=None, rollout_log_prob=None, entropy=None, pg_loss_mask=None, sample_denom=None,
+                 pg_sample_denom=None, loss_kind="ppo", kl_kind=None, unbiased_kl=False, use_opsm=False,
+                 use_tis=False, mismatch_metrics=False, abs_diff_from_old=1, eps_clip=0.2, eps_clip_high=0.2,
+                 eps_clip_c=None, entropy_coef=0.0, kl_coef=0.0, tis_lo=0.0, tis_hi=2.0, opsm_delta=1e-4,
+                 tau_pos=1.0, tau_neg=1.05, per_token_outputs=False, want_coef_entropy=False):
+    """Fills a ``relax_amd_policy_loss_args`` block; returns (struct, outputs dict holding every live tensor)."""
+    dev = _need_gpu(advantages, loss_mask, cu_resp)
     b = int(cu_resp.numel()) - 1
     if loss_kind not in _lib.LOSS_KINDS:
         raise ValueError(f"unknown loss kind {loss_kind}")
     if kl_kind not in _lib.KL_KINDS:
         raise ValueError(f"Unknown kl_loss_type: {kl_kind}")
+    if cu_resp.dtype != torch.int64:
+        raise TypeError("cu_resp must be int64")
     keep = [_f32(t) for t in (log_prob, old_log_prob, ref_log_prob, train_log_prob, rollout_log_prob, advantages,
                                loss_mask, pg_loss_mask, entropy, sample_denom, pg_sample_denom)]
     for t in keep[:9]:
@@ -191,7 +192,7 @@ def policy_loss(*, log_prob, advantages, loss_mask, cu_resp, old_log_prob=None, 
     kw = dict(dtype=torch.float32, device=dev)
     out = {
         "coef_log_prob": torch.empty(n, **kw),
-        "coef_entropy": torch.empty(n, **kw) if entropy is not None else None,
+        "coef_entropy": torch.empty(n, **kw) if (entropy is not None or want_coef_entropy) else None,
         "metrics": torch.empty(NUM_METRICS, **kw),
     }
     if per_token_outputs:
@@ -219,11 +220,46 @@ def policy_loss(*, log_prob, advantages, loss_mask, cu_resp, old_log_prob=None, 
         setattr(a, k, None if t is None else t.data_ptr())
     a.sample_partials = partials.data_ptr()
     a.metrics = out["metrics"].data_ptr()
-    if cu_resp.dtype != torch.int64:
-        raise TypeError("cu_resp must be int64")
+    out["_keepalive"] = (keep, partials, cu_resp)
+    return a, out
+
+
+def policy_loss(*, log_prob, **kw):
+    """Runs the two policy-loss launches.  Returns dict(metrics [16], coef_log_prob, coef_entropy, per-token...)."""
+    _need_gpu(log_prob)
+    a, out = _policy_args(n=int(log_prob.numel()), log_prob=log_prob, **kw)
     check(lib.relax_amd_policy_loss(C.byref(a), _stream()))
-    out["_keepalive"] = (keep, partials)
     return out
+
+
+def actor_step_fused(logits, targets, token_of_row, sample_ids, n_tokens: int, inv_temperature: float,
+                     grad_scale: float = 1.0, **kw):
+    """One launch: log-prob + entropy forward, per-token loss coefficients and dlogits; then the policy-loss launches
+    for the metrics.  Returns (out dict as policy_loss, log_prob, entropy, lse, spx, dlogits)."""
+    dev = _need_gpu(logits, targets)
+    logits = _rows(logits)
+    if targets.dtype != torch.int64 or not targets.is_contiguous():
+        targets = targets.to(torch.int64).contiguous()
+    f = dict(dtype=torch.float32, device=dev)
+    lp, ent, lse, spx = (torch.empty(n_tokens, **f) for _ in range(4))
+    dlogits = torch.empty((logits.size(0), logits.size(1)), dtype=logits.dtype, device=dev)
+    a, out = _policy_args(n=n_tokens, want_coef_entropy=True, **kw)
+    stride = logits.stride(0) if logits.size(0) > 1 else logits.size(1)
+    check(lib.relax_amd_actor_step_fused(
+        _p(logits), _code(logits), logits.size(0), logits.size(1), stride, _p(token_of_row), _p(sample_ids),
+        _p(targets), float(inv_temperature), C.byref(a), float(grad_scale), _p(lp), _p(ent), _p(lse), _p(spx),
+        _p(dlogits), logits.size(1), _stream()))
+    a.log_prob, a.entropy = lp.data_ptr(), ent.data_ptr()
+    check(lib.relax_amd_policy_loss(C.byref(a), _stream()))
+    return out, lp, ent, lse, spx, dlogits
+
+
+def scale_rows_inplace(data, factor_dev):
+    data2 = data.reshape(-1, data.size(-1))
+    stride = data2.stride(0) if data2.size(0) > 1 else data2.size(1)
+    check(lib.relax_amd_scale_rows_inplace(_p(data2), _code(data2), data2.size(0), data2.size(1), stride,
+                                           _p(factor_dev), _stream()))
+    return data
 
 
 # ----------------------------------------------------------------------------------------------------- advantages

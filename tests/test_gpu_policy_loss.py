@@ -70,14 +70,17 @@ CASES = {
 
 @pytest.mark.parametrize("name", sorted(CASES))
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-5), (torch.bfloat16, 2e-3)])
-def test_policy_loss_function_vs_oracle(name, dtype, tol):
+@pytest.mark.parametrize("single_pass", ["auto", "off"])
+def test_policy_loss_function_vs_oracle(name, dtype, tol, single_pass):
+    """Both kernel paths: the fused single-launch step ("auto" picks it whenever the loss is token-local) and the
+    separate forward / backward launches ("off")."""
     import relax_amd
 
     dev = require_gpu()
-    announce("policy_loss", name, dtype)
+    announce("policy_loss", name, dtype, single_pass)
     tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 264
     logits, batch = _make_batch(11, tot, resp, v, dtype)
-    args = P.make_args(**CASES[name])
+    args = P.make_args(relax_amd_single_pass=single_pass, **CASES[name])
     # oracle on CPU (fp32 upcast of the same logits values)
     lo = logits.float().clone().requires_grad_()
     red = R.make_reducer(resp, batch["loss_masks"], args.calculate_per_token_loss)
@@ -94,6 +97,45 @@ def test_policy_loss_function_vs_oracle(name, dtype, tol):
         assert abs(met[k].item() - float(w)) < tol * max(1.0, abs(float(w))), (k, met[k].item(), float(w))
     assert set(met) == set(want_m)
     torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, atol=tol, rtol=BF16_ULP if dtype == torch.bfloat16 else 0)
+
+
+@pytest.mark.parametrize("v,dtype", [(151936, torch.bfloat16), (32000, torch.float32), (4096, torch.float16),
+                                     (40960, torch.bfloat16), (100000, torch.bfloat16), (4100, torch.bfloat16),
+                                     (1003, torch.float32), (20000, torch.float32)])
+def test_single_pass_matches_two_launch_path_at_real_vocabularies(v, dtype):
+    """Every workgroup width of the fused kernel (256 / 512 / 1024 threads), the scalar-tail and the unaligned
+    scalar path, an upstream gradient != 1 and the one-shot backward."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("single pass vs two launch", v, dtype)
+    tot, resp = [9, 6, 12, 7], [4, 3, 7, 5]
+    logits, batch = _make_batch(17, tot, resp, v, dtype)
+    db = _to_dev(batch, dev)
+    outs = {}
+    for mode in ("auto", "off"):
+        args = P.make_args(relax_amd_single_pass=mode, eps_clip_high=0.28, use_kl_loss=True, kl_loss_coef=1e-3,
+                           kl_loss_type="k3", entropy_coef=0.01)
+        lg = logits.to(dev).requires_grad_()
+        loss, met = relax_amd.policy_loss_function(args, db, lg, None)
+        (loss * 3.0).backward(retain_graph=True)
+        outs[mode] = (loss.detach(), {k: x.clone() for k, x in met.items()}, lg.grad.clone())
+        if mode == "auto":
+            with pytest.raises(RuntimeError, match="cannot run twice"):
+                loss.backward()
+    assert torch.equal(outs["auto"][0], outs["off"][0])  # same forward arithmetic, same reduction order
+    for k in outs["auto"][1]:
+        torch.testing.assert_close(outs["auto"][1][k], outs["off"][1][k], atol=1e-6, rtol=1e-6)
+    ulp = {torch.float32: 1e-6, torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}[dtype]
+    torch.testing.assert_close(outs["auto"][2].float(), outs["off"][2].float(), atol=1e-6, rtol=ulp)
+    # and against the oracle
+    lo = logits.float().clone().requires_grad_()
+    oargs = P.make_args(eps_clip_high=0.28, use_kl_loss=True, kl_loss_coef=1e-3, kl_loss_type="k3", entropy_coef=0.01)
+    want, _ = P.policy_loss_function(oargs, dict(batch), lo, R.make_reducer(resp, batch["loss_masks"]))
+    (want * 3.0).backward()
+    tol = 3e-5 if dtype == torch.float32 else 2e-3
+    assert abs(outs["auto"][0].item() - want.item()) < tol * max(1.0, abs(want.item()))
+    torch.testing.assert_close(outs["auto"][2].float().cpu(), lo.grad, atol=tol, rtol=max(ulp, 1e-5))
 
 
 def test_sample_index_mask_sums_int_masks_and_sft_row():
