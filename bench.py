@@ -2,7 +2,8 @@
 
 One "step" = one pass of the hot path over one synthetic micro-batch that is already resident in HBM:
 ``relax_amd.policy_loss_function(args, batch, logits)`` (log-prob + entropy forward, PPO-clip 0.2/0.28 + k3 KL
-coef 1e-3, token-mean aggregation) followed by ``loss.backward()`` to bf16 dlogits.  Workload = the Qwen3-8B-shaped
+coef 1e-3, token-mean aggregation) followed by ``loss.backward()`` to bf16 dlogits (for this token-local loss the
+library runs both in one fused launch).  Workload = the Qwen3-8B-shaped
 actor step: 16 sequences x 4096 tokens = 65536 rows x 151936 vocabulary, logits ~ N(0, 3) with 5 % spiked rows,
 first 20 % of every sequence masked out.
 
@@ -23,6 +24,10 @@ import torch
 VOCAB = 151936
 SEQS, SEQ_LEN = 16, 4096
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one actor_step_fused launch moves at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# at the L2 <-> fabric boundary (profiles/actor_step_fused_bf16_v151936_n65536.md): 26 780 743 KiB fetched
+# (counter x 2.000) + 19 464 492 KiB written.
+MEASURED_TRAFFIC_FUSED = (26780743 + 19464492) * 1024.0
 
 
 def make_args():
@@ -125,6 +130,8 @@ def main() -> int:
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
     ap.add_argument("--vocab", type=int, default=VOCAB)
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the CPU baseline slab (0 = skip)")
+    ap.add_argument("--two-launch", action="store_true",
+                    help="use the separate forward / backward launches (the path GSPO takes) instead of the fused step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB device copy, the known-size reference for FETCH_SIZE/WRITE_SIZE")
     a = ap.parse_args()
@@ -145,16 +152,15 @@ def main() -> int:
     logits.requires_grad_()
     n_tokens = a.seqs * a.seq_len
 
-    def step(record=None):
+    from relax_amd import ops
+
+    if a.two_launch:
+        args.relax_amd_single_pass = "off"
+
+    def step():
         logits.grad = None
-        if record:
-            record[0].record()
         loss, _ = relax_amd.policy_loss_function(args, batch, logits, None)
-        if record:
-            record[1].record()
         loss.backward()
-        if record:
-            record[2].record()
         return loss
 
     if a.calibrate_copy:
@@ -167,20 +173,29 @@ def main() -> int:
     for _ in range(a.warmup):
         step()
     torch.cuda.synchronize()
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(a.steps)]
+    ops.kernel_events = []  # HIP events around the big launches, on the stream they are launched on
     t0 = time.perf_counter()
-    for k in range(a.steps):
-        loss = step(events[k])
+    for _ in range(a.steps):
+        loss = step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / a.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / a.steps
+    events, ops.kernel_events = ops.kernel_events, None
+    per_kernel = {}
+    for name, e0, e1 in events:
+        per_kernel.setdefault(name, []).append(e0.elapsed_time(e1))
+    kernel_ms = {k: sum(v) / len(v) for k, v in per_kernel.items()}
     ms_per_step = wall * 1e3 / a.steps
     elem = logits.element_size()
-    # dominant kernel = the dlogits backward: one read + one write of every row
-    bwd_bytes = 2.0 * a.vocab * elem * n_tokens
-    achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
-    step_bytes = 3.0 * a.vocab * elem * n_tokens
+    row_bytes = float(a.vocab * elem) * n_tokens
+    if "actor_step_fused" in kernel_ms:
+        # one launch does the forward scan and the dlogits backward: 3*V*s algorithmic bytes per token (forward read,
+        # backward read, dlogits write); its second read is served by cache, see "traffic"
+        dom, dom_name, dom_bytes = kernel_ms["actor_step_fused"], "actor_step_fused_kernel<bf16_t, true, 1024>", 3.0 * row_bytes
+        traffic = MEASURED_TRAFFIC_FUSED if (a.vocab, n_tokens) == (VOCAB, SEQS * SEQ_LEN) else None
+    else:
+        dom, dom_name, dom_bytes = kernel_ms["logprob_entropy_bwd"], "logprob_entropy_bwd_kernel<bf16_t, true>", 2.0 * row_bytes
+        traffic = None
+    achieved = dom_bytes / (dom * 1e-3) / 1e9
     out = {
         "metric": "tokens/s fused logprob+entropy+loss fwd+bwd @V=151936 bf16; % HBM/MFMA peak",
         "value": n_tokens / (wall / a.steps),
@@ -200,11 +215,10 @@ def main() -> int:
             "rows": n_tokens, "vocab": a.vocab, "loss": float(loss.item()),
         },
         "roofline": {
-            "bound": "hbm", "kernel": "logprob_entropy_bwd_kernel<bf16>", "achieved": achieved,
-            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-            "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_ms": bwd_ms,
-            "forward_ms": fwd_ms, "forward_GBs": a.vocab * elem * n_tokens / (fwd_ms * 1e-3) / 1e9,
-            "step_algorithmic_GBs": step_bytes / (ms_per_step * 1e-3) / 1e9,
+            "bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "algorithmic_bytes_per_launch": dom_bytes,
+            "avg_launch_ms": dom, "kernel_ms": kernel_ms,
+            "step_algorithmic_GBs": 3.0 * row_bytes / (ms_per_step * 1e-3) / 1e9,
         },
         "cpu_baseline": cpu_baseline(args, a.cpu_rows, a.vocab) if a.cpu_rows > 0 else None,
     }

@@ -6,13 +6,14 @@ from __future__ import annotations
 import torch
 
 from . import ops
+from ._staging import upload_int64
 
 
 def _cu(response_lengths, device) -> torch.Tensor:
     cu = [0]
     for r in response_lengths:
         cu.append(cu[-1] + int(r))
-    return torch.tensor(cu, dtype=torch.int64).to(device)
+    return upload_int64(cu, device)
 
 
 def _mask_sums(loss_masks, cu_resp=None) -> torch.Tensor:

@@ -24,6 +24,7 @@ import torch
 
 from . import ops
 from ._lib import METRIC_SLOTS
+from ._staging import upload_int64
 from .cp_utils import get_cp_local_num_tokens, get_sum_of_sample_mean, sample_denominators
 from .ppo_utils import get_grpo_returns
 
@@ -94,9 +95,8 @@ class PackedLayout:
         cu = [0]
         for r in self.response_lengths:
             cu.append(cu[-1] + r)
-        host = torch.tensor([begins + [0], cu], dtype=torch.int64)
-        dev = host.to(device, non_blocking=False)
-        self.row_begin, self.cu_resp = dev[0, : self.n_samples].contiguous(), dev[1].contiguous()
+        dev = upload_int64(begins + cu, device)
+        self.row_begin, self.cu_resp = dev[: self.n_samples], dev[self.n_samples :]
         self.row_ids, self.sample_ids, self.token_of_row = ops.build_row_maps(
             self.row_begin, self.cu_resp, self.n_tokens, n_rows, want_inverse=need_inverse
         )

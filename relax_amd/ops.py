@@ -42,6 +42,29 @@ def _stream():
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+# When set to a list, the big launches append (name, start_event, end_event) recorded on the launch stream, so a
+# benchmark can read each kernel's duration without an external profiler.
+kernel_events = None
+
+
+class _timed:
+    def __init__(self, name):
+        self.name = name
+
+    def __enter__(self):
+        if kernel_events is not None:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.end = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+        return self
+
+    def __exit__(self, *exc):
+        if kernel_events is not None:
+            self.end.record()
+            kernel_events.append((self.name, self.start, self.end))
+        return False
+
+
 def _code(t: torch.Tensor) -> int:
     try:
         return _DTYPE_CODES[t.dtype]
@@ -86,9 +109,10 @@ def logprob_entropy_fwd(logits, targets, row_ids=None, inv_temperature: float = 
     lse = torch.empty(n, **kw)
     ent = torch.empty(n, **kw) if with_entropy else None
     spx = torch.empty(n, **kw) if with_entropy else None
-    check(lib.relax_amd_logprob_entropy_fwd(
-        _p(logits), _code(logits), n, logits.size(1), logits.stride(0) if logits.size(0) > 1 else logits.size(1),
-        _p(row_ids), _p(targets), float(inv_temperature), _p(lp), _p(ent), _p(lse), _p(spx), _stream()))
+    with _timed("logprob_entropy_fwd"):
+        check(lib.relax_amd_logprob_entropy_fwd(
+            _p(logits), _code(logits), n, logits.size(1), logits.stride(0) if logits.size(0) > 1 else logits.size(1),
+            _p(row_ids), _p(targets), float(inv_temperature), _p(lp), _p(ent), _p(lse), _p(spx), _stream()))
     return lp, ent, lse, spx
 
 
@@ -100,10 +124,12 @@ def logprob_entropy_bwd(logits, targets, lse, spx, g_lp, g_ent=None, token_of_ro
     if out is None:
         out = torch.empty((logits.size(0), logits.size(1)), dtype=logits.dtype, device=logits.device)
     stride = logits.stride(0) if logits.size(0) > 1 else logits.size(1)
-    check(lib.relax_amd_logprob_entropy_bwd(
-        _p(logits), _code(logits), logits.size(0), logits.size(1), stride, _p(token_of_row), _p(targets), _p(lse),
-        _p(spx), _p(_f32(g_lp)), _p(_f32(g_ent)), float(grad_scale), _p(grad_scale_dev), float(inv_temperature),
-        _p(out), out.stride(0) if out.size(0) > 1 else out.size(1), _stream()))
+    g_lp, g_ent = _f32(g_lp), _f32(g_ent)
+    with _timed("logprob_entropy_bwd"):
+        check(lib.relax_amd_logprob_entropy_bwd(
+            _p(logits), _code(logits), logits.size(0), logits.size(1), stride, _p(token_of_row), _p(targets), _p(lse),
+            _p(spx), _p(g_lp), _p(g_ent), float(grad_scale), _p(grad_scale_dev), float(inv_temperature),
+            _p(out), out.stride(0) if out.size(0) > 1 else out.size(1), _stream()))
     return out
 
 
@@ -245,10 +271,11 @@ def actor_step_fused(logits, targets, token_of_row, sample_ids, n_tokens: int, i
     dlogits = torch.empty((logits.size(0), logits.size(1)), dtype=logits.dtype, device=dev)
     a, out = _policy_args(n=n_tokens, want_coef_entropy=True, **kw)
     stride = logits.stride(0) if logits.size(0) > 1 else logits.size(1)
-    check(lib.relax_amd_actor_step_fused(
-        _p(logits), _code(logits), logits.size(0), logits.size(1), stride, _p(token_of_row), _p(sample_ids),
-        _p(targets), float(inv_temperature), C.byref(a), float(grad_scale), _p(lp), _p(ent), _p(lse), _p(spx),
-        _p(dlogits), logits.size(1), _stream()))
+    with _timed("actor_step_fused"):
+        check(lib.relax_amd_actor_step_fused(
+            _p(logits), _code(logits), logits.size(0), logits.size(1), stride, _p(token_of_row), _p(sample_ids),
+            _p(targets), float(inv_temperature), C.byref(a), float(grad_scale), _p(lp), _p(ent), _p(lse), _p(spx),
+            _p(dlogits), logits.size(1), _stream()))
     a.log_prob, a.entropy = lp.data_ptr(), ent.data_ptr()
     check(lib.relax_amd_policy_loss(C.byref(a), _stream()))
     return out, lp, ent, lse, spx, dlogits
