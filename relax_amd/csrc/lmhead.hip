@@ -5,14 +5,21 @@
 // F.linear -> .float() -> /T -> calculate_log_probs_and_entropy), and adds the entropy the reference leaves out.
 //
 // Tiling.  A workgroup (256 threads = 4 wave64) owns 256 tokens and walks a range of 256-wide vocabulary tiles; the
-// K loop over the hidden size runs in 32-wide slices, double-buffered through LDS (2 x (256+256) rows x 80 B,
-// rows padded by 16 B so the 16-byte fragment reads of 8 consecutive rows hit distinct banks).  The MFMA "A"
-// operand is the WEIGHT tile and "B" the HIDDEN tile, so in the 32x32 accumulator layout a lane's column is a TOKEN
-// and its 16 registers are 16 vocabulary entries: the online softmax over the vocabulary is then a per-lane
-// reduction over 64 accumulator values per token (4 tokens per lane, 12 state registers), with one cross-lane and
-// one cross-wave merge at the very end.  Each wave computes 128 vocab x 128 tokens = 4x4 MFMA tiles (256 fp32
-// accumulators per lane).  Vocabulary ranges are split over workgroups (flash-decoding style) and merged by a small
-// combine kernel; the target logit comes from a gather-dot kernel (one wave per token).
+// K loop over the hidden size runs in 64-wide slices through a two-stage LDS ring (2 x (256 + 256) rows x 128 B).
+// Slices are copied global -> LDS directly (global_load_lds_dwordx4, no staging registers): every lane fetches one
+// 16-byte vector and the wave's 64 vectors land contiguously, i.e. 8 rows x 128 B per instruction.  The LDS has 64
+// four-byte banks and serves 16 lanes of a 16-byte read per clock, so the fragment reads of 16 consecutive rows (same
+// k offset) must hit 16 distinct bank quads: with 128-byte rows the bank quad is (row parity, slot), hence lane
+// (row r, slot v) fetches global vector v ^ ((r >> 1) & 7) and fragment reads apply the same XOR (no padding).  The copy of slice k+1 (or of the next vocabulary tile's
+// first slice) is issued before the MFMAs of slice k and awaited after them, so global latency hides behind 64 MFMAs
+// per wave; fragments for the next 16-wide k-step are fetched from LDS while the current 16 MFMAs issue.
+//
+// The MFMA "A" operand is the WEIGHT tile and "B" the HIDDEN tile, so in the 32x32 accumulator layout a lane's column
+// is a TOKEN and its 16 registers are 16 vocabulary entries: the online softmax over the vocabulary is then a
+// per-lane reduction over 64 accumulator values per token (4 tokens per lane, 12 state registers), with one cross-lane
+// and one cross-wave merge at the very end.  Each wave computes 128 vocab x 128 tokens = 4x4 MFMA tiles (256 fp32
+// accumulators per lane, held in AGPRs).  Vocabulary ranges are split over workgroups (flash-decoding style) and
+// merged by a small combine kernel; the target logit comes from a gather-dot kernel (one wave per token).
 //
 // Workgroup -> (XCD, row block, vocab split) mapping: hardware places consecutive workgroup ids round-robin on the
 // 8 XCDs; the 32 workgroups resident on one XCD are arranged as (32/S) row blocks x S vocab splits so that hidden
@@ -26,14 +33,12 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kLmTile = 256;                 // tokens per workgroup == vocab entries per tile
-constexpr int kLmBK = 32;                    // hidden-size slice per pipeline stage
-constexpr int kLmRow = kLmBK + 8;            // LDS row pitch in bf16: +16 B so 8 consecutive rows hit distinct banks
+constexpr int kLmBK = 64;                    // hidden-size slice per pipeline stage (128 B per row)
 constexpr int kLmThreads = 256;
-constexpr int kLmVecPerRow = kLmBK / 8;                      // 16-byte vectors per slice row
-constexpr int kLmRowsPerPass = kLmThreads / kLmVecPerRow;    // rows one pass of the workgroup covers
-constexpr int kLmPasses = kLmTile / kLmRowsPerPass;          // 16-byte loads per thread per operand slice
-constexpr int kLmStage = 2 * kLmTile * kLmRow;       // bf16 elements per stage (weight rows then hidden rows)
-constexpr int kLmLdsBytes = 2 * kLmStage * 2;        // two stages
+constexpr int kLmPasses = 8;                 // 16-byte copies per thread per operand slice (32 rows per pass)
+constexpr int kLmOperandBytes = kLmTile * kLmBK * 2;   // 32 KB
+constexpr int kLmStageBytes = 2 * kLmOperandBytes;     // weight rows then hidden rows
+constexpr int kLmLdsBytes = 2 * kLmStageBytes;         // two stages: 128 KB
 constexpr int kLmXcds = 8, kLmPerXcd = 32;
 
 struct LmGeom {
@@ -50,85 +55,131 @@ __device__ __forceinline__ bool lm_block_coords(const LmGeom& g, int& rb, int& s
   return rb < g.row_blocks;
 }
 
-// Global -> register -> LDS staging of one 256-row x kLmBK-col bf16 slice of an operand.  The tile base is
-// wave-uniform; each thread keeps kLmPasses 32-bit element offsets (rows past the ragged edge re-read the last valid
-// row; their results are discarded).
-struct LmStager {
-  const uint16_t* base;
-  uint32_t off[kLmPasses];
-  u32x4 reg[kLmPasses];
-  int lds_off;  // bf16 index of this thread's first row/vec inside an operand tile
+// Asynchronous global -> LDS copy of one 256-row x 64-col bf16 slice of an operand.  Thread t covers row t/8 of each
+// 32-row pass and LDS slot t%8; it fetches global vector (t%8) ^ ((row >> 1) & 7) of that row (the same value for
+// every pass).  Rows past the ragged edge re-read the last valid row; their results are discarded by the caller.
+struct LmCopier {
+  const uint16_t* base;     // first row of the tile (wave-uniform)
+  uint32_t off[kLmPasses];  // element offset of this thread's vector in each pass, k-slice 0
 
   __device__ __forceinline__ void init(const uint16_t* matrix, int64_t stride, int64_t row0, int64_t row_limit) {
-    const int r = threadIdx.x / kLmVecPerRow, v = threadIdx.x % kLmVecPerRow;
+    const int r = threadIdx.x >> 3, v = threadIdx.x & 7;
     base = matrix + row0 * stride;
     const int last = int(row_limit - row0);
+    const uint32_t col = uint32_t((v ^ ((r >> 1) & 7)) * 8);
 #pragma unroll
-    for (int i = 0; i < kLmPasses; ++i) {
-      const int row = min(r + kLmRowsPerPass * i, last);
-      off[i] = uint32_t(row) * uint32_t(stride) + uint32_t(v * 8);
+    for (int p = 0; p < kLmPasses; ++p) off[p] = uint32_t(min(r + 32 * p, last)) * uint32_t(stride) + col;
+  }
+  // `tile` = LDS address of this operand's tile in the target stage
+  __device__ __forceinline__ void issue(unsigned char* tile, int kslice) const {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+    for (int p = 0; p < kLmPasses; ++p) {
+      const uint16_t* src = base + off[p] + kslice * kLmBK;
+      unsigned char* dst = tile + (p * 32 + wave * 8) * (kLmBK * 2);  // wave-uniform; lane l lands at dst + 16*l
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src),
+                                       (__attribute__((address_space(3))) void*)(dst), 16, 0, 0);
     }
-    lds_off = r * kLmRow + v * 8;
-  }
-  __device__ __forceinline__ void load(int kslice) {
-#pragma unroll
-    for (int i = 0; i < kLmPasses; ++i)
-      reg[i] = *reinterpret_cast<const u32x4*>(base + off[i] + kslice * kLmBK);
-  }
-  __device__ __forceinline__ void store(uint16_t* tile) const {
-#pragma unroll
-    for (int i = 0; i < kLmPasses; ++i)
-      *reinterpret_cast<u32x4*>(tile + lds_off + i * kLmRowsPerPass * kLmRow) = reg[i];
   }
 };
 
-__device__ __forceinline__ void lm_mma_stage(const uint16_t* ws, const uint16_t* hs, int wv, int wt, int lane,
-                                             floatx16 (&acc)[4][4]) {
-  const int frag = (lane & 31) * kLmRow + (lane >> 5) * 8;
-#pragma unroll
-  for (int ks = 0; ks < kLmBK / 16; ++ks) {
-    bf16x8 a[4], b[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      a[i] = *reinterpret_cast<const bf16x8*>(ws + (wv * 128 + i * 32) * kLmRow + frag + ks * 16);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      b[j] = *reinterpret_cast<const bf16x8*>(hs + (wt * 128 + j * 32) * kLmRow + frag + ks * 16);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
-  }
+// LDS byte offset (inside an operand tile) of the fragment this lane feeds to the MFMA for 16-wide k-step `ks`:
+// row (lane & 31) of a 32-row sub-tile, global vector 2*ks + (lane >> 5), stored at slot vector ^ ((row >> 1) & 7).
+__device__ __forceinline__ int lm_frag_offset(int lane, int ks) {
+  const int row = lane & 31;
+  return row * (kLmBK * 2) + (((2 * ks + (lane >> 5)) ^ ((row >> 1) & 7)) * 16);
 }
 
-// One 256x256 logits tile into `acc` (fp32, un-scaled logits).
-__device__ __forceinline__ void lm_tile_gemm(uint16_t* lds, LmStager& wst, LmStager& hst, int nk, int wv, int wt,
-                                             int lane, floatx16 (&acc)[4][4]) {
+struct LmFrags {
+  bf16x8 a[4], b[4];
+};
+
+__device__ __forceinline__ void lm_load_frags(const unsigned char* ws, const unsigned char* hs, int wv, int wt, int lane,
+                                              int ks, LmFrags& f) {
+  const int fo = lm_frag_offset(lane, ks);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    f.a[i] = *reinterpret_cast<const bf16x8*>(ws + (wv * 128 + i * 32) * (kLmBK * 2) + fo);
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    f.b[j] = *reinterpret_cast<const bf16x8*>(hs + (wt * 128 + j * 32) * (kLmBK * 2) + fo);
+}
+
+__device__ __forceinline__ void lm_mma_frags(const LmFrags& f, floatx16 (&acc)[4][4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
+}
+
+// 64 MFMAs per wave on one stage; the fragments of k-step ks+1 are read from LDS while the MFMAs of ks issue.
+__device__ __forceinline__ void lm_mma_stage(const unsigned char* stage, int wv, int wt, int lane,
+                                             floatx16 (&acc)[4][4]) {
+  const unsigned char* ws = stage;
+  const unsigned char* hs = stage + kLmOperandBytes;
+  LmFrags f0, f1;
+  lm_load_frags(ws, hs, wv, wt, lane, 0, f0);
+  lm_load_frags(ws, hs, wv, wt, lane, 1, f1);
+  lm_mma_frags(f0, acc);
+  lm_load_frags(ws, hs, wv, wt, lane, 2, f0);
+  lm_mma_frags(f1, acc);
+  lm_load_frags(ws, hs, wv, wt, lane, 3, f1);
+  lm_mma_frags(f0, acc);
+  lm_mma_frags(f1, acc);
+}
+
+__device__ __forceinline__ void lm_zero_acc(floatx16 (&acc)[4][4]) {
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-  wst.load(0);
-  hst.load(0);
-  wst.store(lds);
-  hst.store(lds + kLmTile * kLmRow);
+}
+
+// Walks the vocabulary tiles [vt_begin, vt_end) of one 256-token row block as a single software pipeline over
+// (tile, k-slice) and hands every finished 256x256 logits tile (fp32, un-scaled) to `epilogue(acc, v0)`, which runs
+// while the first slice of the next tile is already in flight.
+template <typename Epilogue>
+__device__ __forceinline__ void lm_pipeline(unsigned char* lds, const uint16_t* hidden, const uint16_t* weight,
+                                            const LmGeom& g, int64_t tok0, int vt_begin, int vt_end,
+                                            Epilogue&& epilogue) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wv = wave >> 1, wt = wave & 1;
+  const int nk = int(g.hidden / kLmBK);
+  LmCopier hc, wc;
+  hc.init(hidden, g.h_stride, tok0, g.n_tokens - 1);
+  floatx16 acc[4][4];
+  lm_zero_acc(acc);
+  if (vt_begin >= vt_end) return;
+  wc.init(weight, g.w_stride, int64_t(vt_begin) * kLmTile, g.vocab - 1);
+  int stage = 0;
+  wc.issue(lds, 0);
+  hc.issue(lds + kLmOperandBytes, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  for (int kk = 0; kk < nk; ++kk) {
-    uint16_t* cur = lds + (kk & 1) * kLmStage;
-    uint16_t* nxt = lds + ((kk + 1) & 1) * kLmStage;
-    const bool more = kk + 1 < nk;
-    if (more) {
-      wst.load(kk + 1);
-      hst.load(kk + 1);
+  for (int vt = vt_begin; vt < vt_end; ++vt) {
+    for (int kk = 0; kk + 1 < nk; ++kk) {  // steady state: copy slice kk+1 while multiplying slice kk
+      unsigned char* nxt = lds + (stage ^ 1) * kLmStageBytes;
+      wc.issue(nxt, kk + 1);
+      hc.issue(nxt + kLmOperandBytes, kk + 1);
+      lm_mma_stage(lds + stage * kLmStageBytes, wv, wt, lane, acc);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      stage ^= 1;
     }
-    lm_mma_stage(cur, cur + kLmTile * kLmRow, wv, wt, lane, acc);
-    if (more) {
-      wst.store(nxt);
-      hst.store(nxt + kLmTile * kLmRow);
+    // last slice of the tile: start the next tile's first slice, finish the tile, run its epilogue under the copy
+    if (vt + 1 < vt_end) {
+      unsigned char* nxt = lds + (stage ^ 1) * kLmStageBytes;
+      wc.init(weight, g.w_stride, int64_t(vt + 1) * kLmTile, g.vocab - 1);
+      wc.issue(nxt, 0);
+      hc.issue(nxt + kLmOperandBytes, 0);
     }
+    lm_mma_stage(lds + stage * kLmStageBytes, wv, wt, lane, acc);
+    epilogue(acc, int64_t(vt) * kLmTile);
+    lm_zero_acc(acc);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    stage ^= 1;
   }
 }
 
@@ -170,14 +221,10 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_fwd_kernel(const uint16_
                                                                    const uint16_t* __restrict__ weight, LmGeom g,
                                                                    float c, float* __restrict__ partial) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
   int rb, split;
   if (!lm_block_coords(g, rb, split)) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wv = wave >> 1, wt = wave & 1;
   const int64_t tok0 = int64_t(rb) * kLmTile;
-  const int nk = int(g.hidden / kLmBK);
-  LmStager hst, wst;
-  hst.init(hidden, g.h_stride, tok0, g.n_tokens - 1);
   float m[4], s[4], t[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -187,11 +234,7 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_fwd_kernel(const uint16_
   }
   const int vt_begin = split * g.tiles_per_split;
   const int vt_end = min(g.n_tiles, vt_begin + g.tiles_per_split);
-  for (int vt = vt_begin; vt < vt_end; ++vt) {
-    const int64_t v0 = int64_t(vt) * kLmTile;
-    wst.init(weight, g.w_stride, v0, g.vocab - 1);
-    floatx16 acc[4][4];
-    lm_tile_gemm(lds, wst, hst, nk, wv, wt, lane, acc);
+  lm_pipeline(smem, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
     const int limit = int(min<int64_t>(g.vocab - v0, kLmTile));
     if (limit < kLmTile) {  // ragged last tile: entries past the vocabulary are masked out
 #pragma unroll
@@ -205,7 +248,7 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_fwd_kernel(const uint16_
 #pragma unroll
         for (int j = 0; j < 4; ++j) lm_absorb_block<false>(acc[i][j], 0, 0, c, m[j], s[j], t[j]);
     }
-  }
+  });
   // merge the two lane halves (same tokens, different vocab rows), then the two waves sharing the tokens
   float* red = reinterpret_cast<float*>(smem);  // [2 (wv)][256 tokens][3]
   __syncthreads();
@@ -298,14 +341,10 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_dlogits_kernel(
     const float* __restrict__ g_lp, const float* __restrict__ g_ent, const float* __restrict__ grad_scale_dev,
     uint16_t* __restrict__ d_t, int64_t d_stride) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
   int rb, split;
   if (!lm_block_coords(g, rb, split)) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wv = wave >> 1, wt = wave & 1;
   const int64_t tok0 = int64_t(rb) * kLmTile;
-  const int nk = int(g.hidden / kLmBK);
-  LmStager hst, wst;
-  hst.init(hidden, g.h_stride, tok0, g.n_tokens - 1);
   const float gs = grad_scale_dev ? *grad_scale_dev : 1.0f;
   float k0[4], a0[4], a1[4], hot[4];
   int64_t tg[4], tokj[4];
@@ -323,11 +362,7 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_dlogits_kernel(
   }
   const int vt_begin = split * g.tiles_per_split;
   const int vt_end = min(g.n_tiles, vt_begin + g.tiles_per_split);
-  for (int vt = vt_begin; vt < vt_end; ++vt) {
-    const int64_t v0 = int64_t(vt) * kLmTile;
-    wst.init(weight, g.w_stride, v0, g.vocab - 1);
-    floatx16 acc[4][4];
-    lm_tile_gemm(lds, wst, hst, nk, wv, wt, lane, acc);
+  lm_pipeline(smem, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -346,7 +381,7 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_dlogits_kernel(
           }
         }
       }
-  }
+  });
 }
 
 }  // namespace relax_amd

@@ -123,7 +123,14 @@ class FusedLMHeadLogProb(torch.autograd.Function):
 
 def lm_head_log_probs_and_entropy(hidden, weight, tokens, temperature: float = 1.0, with_entropy: bool = False,
                                   with_entropy_grad: bool = True):
-    """``(log_prob [N] fp32, entropy [N] fp32 | None)`` of ``log_softmax(hidden @ weight.T / temperature)``."""
+    """``(log_prob [N] fp32, entropy [N] fp32 | None)`` of ``log_softmax(hidden @ weight.T / temperature)``.
+
+    The kernels consume the hidden size in 64-wide slices; other sizes are zero-padded here (zeros add nothing to
+    the logits, and autograd through the padding returns gradients of the original shapes)."""
+    pad = (-hidden.size(-1)) % 64
+    if pad:
+        hidden = torch.nn.functional.pad(hidden, (0, pad))
+        weight = torch.nn.functional.pad(weight, (0, pad))
     lp, ent = FusedLMHeadLogProb.apply(hidden, weight, tokens, 1.0 / float(temperature), bool(with_entropy),
                                        bool(with_entropy_grad))
     return lp, (ent if with_entropy else None)

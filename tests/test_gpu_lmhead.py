@@ -102,12 +102,16 @@ def test_slabbed_backward_accumulates_dweight(monkeypatch):
 
 
 def test_argument_errors():
-    from relax_amd.lm_head import lm_head_log_probs_and_entropy
+    from relax_amd.lm_head import lm_head_log_probs_and_entropy, lmhead_logprob_fwd
 
     dev = require_gpu()
-    hid = torch.randn(8, 48, device=dev).bfloat16()  # hidden size not a multiple of 32
+    hid = torch.randn(8, 48, device=dev).bfloat16()  # hidden size not a multiple of 64: the raw op refuses ...
     w = torch.randn(16, 48, device=dev).bfloat16()
-    with pytest.raises(Exception, match="multiple of 32"):
-        lm_head_log_probs_and_entropy(hid, w, torch.zeros(8, dtype=torch.long, device=dev))
+    tok = torch.zeros(8, dtype=torch.long, device=dev)
+    with pytest.raises(Exception, match="multiple of 64"):
+        lmhead_logprob_fwd(hid, w, tok)
+    lp, _ = lm_head_log_probs_and_entropy(hid, w, tok)  # ... and the wrapper pads
+    want = torch.log_softmax(hid.float() @ w.float().t(), -1)[:, 0]
+    torch.testing.assert_close(lp, want, atol=2e-3, rtol=0)
     with pytest.raises(TypeError, match="bfloat16"):
-        lm_head_log_probs_and_entropy(hid.float(), w, torch.zeros(8, dtype=torch.long, device=dev))
+        lm_head_log_probs_and_entropy(hid.float(), w, tok)
