@@ -243,7 +243,7 @@ int relax_amd_scale_rows_inplace(void* data, int dtype, int64_t n_rows, int64_t 
  * deferred-LM-head branch of get_log_probs_and_entropy (relax/backends/megatron/loss.py:391-419: per sub-chunk
  * lm_head_forward -> .float() -> /T -> calculate_log_probs_and_entropy) and additionally returns the entropy.
  *   hidden [n_tokens, hidden_size] bf16 (row stride h_stride), weight [vocab, hidden_size] bf16 (row stride w_stride)
- *   hidden_size must be a multiple of 64; rows 16-byte aligned
+ *   hidden_size must be a multiple of 128; rows 16-byte aligned
  *   workspace  relax_amd_lmhead_workspace_bytes(n_tokens) bytes of device memory
  */
 int64_t relax_amd_lmhead_workspace_bytes(int64_t n_tokens);

@@ -37,8 +37,6 @@ constexpr int kLmBK = 64;                    // hidden-size slice per pipeline s
 constexpr int kLmThreads = 256;
 constexpr int kLmPasses = 8;                 // 16-byte copies per thread per operand slice (32 rows per pass)
 constexpr int kLmOperandBytes = kLmTile * kLmBK * 2;   // 32 KB
-constexpr int kLmStageBytes = 2 * kLmOperandBytes;     // weight rows then hidden rows
-constexpr int kLmLdsBytes = 2 * kLmStageBytes;         // two stages: 128 KB
 constexpr int kLmXcds = 8, kLmPerXcd = 32;
 
 struct LmGeom {
@@ -58,24 +56,35 @@ __device__ __forceinline__ bool lm_block_coords(const LmGeom& g, int& rb, int& s
 // Asynchronous global -> LDS copy of one 256-row x 64-col bf16 slice of an operand.  Thread t covers row t/8 of each
 // 32-row pass and LDS slot t%8; it fetches global vector (t%8) ^ ((row >> 1) & 7) of that row (the same value for
 // every pass).  Rows past the ragged edge re-read the last valid row; their results are discarded by the caller.
+// s_waitcnt immediate for "all vector-memory operations done" (vmcnt = 0, expcnt and lgkmcnt left at their maxima).
+// Issued through the builtin so that the compiler's own wait-count bookkeeping sees it.
+constexpr int kLmWaitCopies = 0x0F70;
+constexpr int kLmWaitEverything = 0x0070;  // vmcnt = 0 and lgkmcnt = 0
+constexpr int kLmWaitAllButLastFrags = 0xC87F;  // lgkmcnt = 8: all LDS reads but the newest fragment set have landed
+
 struct LmCopier {
-  const uint16_t* base;     // first row of the tile (wave-uniform)
-  uint32_t off[kLmPasses];  // element offset of this thread's vector in each pass, k-slice 0
+  const unsigned char* base;  // first row of the tile (wave-uniform, lives in scalar registers)
+  uint32_t off[kLmPasses];    // byte offset of this thread's vector in each pass, k-slice 0
 
   __device__ __forceinline__ void init(const uint16_t* matrix, int64_t stride, int64_t row0, int64_t row_limit) {
     const int r = threadIdx.x >> 3, v = threadIdx.x & 7;
-    base = matrix + row0 * stride;
+    base = reinterpret_cast<const unsigned char*>(matrix + row0 * stride);
     const int last = int(row_limit - row0);
-    const uint32_t col = uint32_t((v ^ ((r >> 1) & 7)) * 8);
+    const uint32_t col = uint32_t((v ^ ((r >> 1) & 7)) * 16);
 #pragma unroll
-    for (int p = 0; p < kLmPasses; ++p) off[p] = uint32_t(min(r + 32 * p, last)) * uint32_t(stride) + col;
+    for (int p = 0; p < kLmPasses; ++p) off[p] = uint32_t(min(r + 32 * p, last)) * uint32_t(stride * 2) + col;
   }
-  // `tile` = LDS address of this operand's tile in the target stage
+  // `tile` = LDS address of this operand's tile in the target stage.  The source address is a scalar base plus a
+  // 32-bit per-lane offset, so each copy needs one address register instead of a 64-bit pair.
   __device__ __forceinline__ void issue(unsigned char* tile, int kslice) const {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    uint64_t slice = reinterpret_cast<uint64_t>(base) + uint64_t(kslice) * (kLmBK * 2);
+    asm volatile("" : "+s"(slice));  // keep scalar + 32-bit lane offset apart (no hoisted 64-bit lane addresses)
 #pragma unroll
     for (int p = 0; p < kLmPasses; ++p) {
-      const uint16_t* src = base + off[p] + kslice * kLmBK;
+      uint32_t lane_off = off[p];
+      asm volatile("" : "+v"(lane_off));  // widen next to the copy so it folds into the scalar-base address form
+      const unsigned char* src = reinterpret_cast<const unsigned char*>(slice + uint64_t(lane_off));
       unsigned char* dst = tile + (p * 32 + wave * 8) * (kLmBK * 2);  // wave-uniform; lane l lands at dst + 16*l
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src),
                                        (__attribute__((address_space(3))) void*)(dst), 16, 0, 0);
@@ -112,20 +121,33 @@ __device__ __forceinline__ void lm_mma_frags(const LmFrags& f, floatx16 (&acc)[4
     for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
 }
 
-// 64 MFMAs per wave on one stage; the fragments of k-step ks+1 are read from LDS while the MFMAs of ks issue.
-__device__ __forceinline__ void lm_mma_stage(const unsigned char* stage, int wv, int wt, int lane,
-                                             floatx16 (&acc)[4][4]) {
-  const unsigned char* ws = stage;
-  const unsigned char* hs = stage + kLmOperandBytes;
+// 64 MFMAs per wave on one stage.  Fragments are double-buffered: the LDS reads of k-step ks+2 are issued before
+// the 16 MFMAs of k-step ks+1 start, and `issue_copies` (the next slice's global -> LDS copies) is slotted in after
+// the first two fragment sets are on their way, so neither LDS nor global latency sits between MFMAs.  The scheduling
+// barriers pin this order (the compiler would otherwise sink each fragment read next to its first use).
+template <typename IssueCopies>
+__device__ __forceinline__ void lm_mma_stage(const unsigned char* ws, const unsigned char* hs, int wv, int wt, int lane,
+                                             floatx16 (&acc)[4][4], IssueCopies&& issue_copies) {
   LmFrags f0, f1;
   lm_load_frags(ws, hs, wv, wt, lane, 0, f0);
   lm_load_frags(ws, hs, wv, wt, lane, 1, f1);
+  __builtin_amdgcn_sched_barrier(0);
+  issue_copies();
+  __builtin_amdgcn_sched_barrier(0);
   lm_mma_frags(f0, acc);
+  __builtin_amdgcn_sched_barrier(0);
   lm_load_frags(ws, hs, wv, wt, lane, 2, f0);
+  __builtin_amdgcn_sched_barrier(0);
   lm_mma_frags(f1, acc);
+  __builtin_amdgcn_sched_barrier(0);
   lm_load_frags(ws, hs, wv, wt, lane, 3, f1);
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(kLmWaitAllButLastFrags);
+  __builtin_amdgcn_sched_barrier(0);
   lm_mma_frags(f0, acc);
+  __builtin_amdgcn_sched_barrier(0);
   lm_mma_frags(f1, acc);
+  __builtin_amdgcn_sched_barrier(0);
 }
 
 __device__ __forceinline__ void lm_zero_acc(floatx16 (&acc)[4][4]) {
@@ -140,46 +162,68 @@ __device__ __forceinline__ void lm_zero_acc(floatx16 (&acc)[4][4]) {
 // Walks the vocabulary tiles [vt_begin, vt_end) of one 256-token row block as a single software pipeline over
 // (tile, k-slice) and hands every finished 256x256 logits tile (fp32, un-scaled) to `epilogue(acc, v0)`, which runs
 // while the first slice of the next tile is already in flight.
+// The two pipeline stages are two distinct LDS objects (not halves of one buffer) so that the compiler can prove that
+// the fragment reads of one stage never alias the in-flight global -> LDS copies into the other; otherwise it waits
+// for the copies before every LDS read and the overlap is lost.
+struct LmLds {
+  unsigned char *w0, *h0, *w1, *h1;  // weight / hidden tile of stage 0 and of stage 1, four separate objects
+};
+
 template <typename Epilogue>
-__device__ __forceinline__ void lm_pipeline(unsigned char* lds, const uint16_t* hidden, const uint16_t* weight,
+__device__ __forceinline__ void lm_pipeline(const LmLds lds, const uint16_t* hidden, const uint16_t* weight,
                                             const LmGeom& g, int64_t tok0, int vt_begin, int vt_end,
                                             Epilogue&& epilogue) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wv = wave >> 1, wt = wave & 1;
-  const int nk = int(g.hidden / kLmBK);
+  const int nk = int(g.hidden / kLmBK);  // even: the hidden size is a multiple of 2 * kLmBK
   LmCopier hc, wc;
   hc.init(hidden, g.h_stride, tok0, g.n_tokens - 1);
   floatx16 acc[4][4];
   lm_zero_acc(acc);
   if (vt_begin >= vt_end) return;
   wc.init(weight, g.w_stride, int64_t(vt_begin) * kLmTile, g.vocab - 1);
-  int stage = 0;
-  wc.issue(lds, 0);
-  hc.issue(lds + kLmOperandBytes, 0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  wc.issue(lds.w0, 0);
+  hc.issue(lds.h0, 0);
+  __builtin_amdgcn_s_waitcnt(kLmWaitCopies);
   __syncthreads();
   for (int vt = vt_begin; vt < vt_end; ++vt) {
-    for (int kk = 0; kk + 1 < nk; ++kk) {  // steady state: copy slice kk+1 while multiplying slice kk
-      unsigned char* nxt = lds + (stage ^ 1) * kLmStageBytes;
-      wc.issue(nxt, kk + 1);
-      hc.issue(nxt + kLmOperandBytes, kk + 1);
-      lm_mma_stage(lds + stage * kLmStageBytes, wv, wt, lane, acc);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // Settle register reloads left over from the epilogue here, once per tile; otherwise the compiler waits for them
+    // at their first use inside the steady-state loop, which also drains the copies issued just before.
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(kLmWaitEverything);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int kk = 0; kk + 2 < nk; kk += 2) {  // steady state: copy slice k+1 while multiplying slice k
+      lm_mma_stage(lds.w0, lds.h0, wv, wt, lane, acc, [&] {
+        wc.issue(lds.w1, kk + 1);
+        hc.issue(lds.h1, kk + 1);
+      });
+      __builtin_amdgcn_s_waitcnt(kLmWaitCopies);
       __syncthreads();
-      stage ^= 1;
+      lm_mma_stage(lds.w1, lds.h1, wv, wt, lane, acc, [&] {
+        wc.issue(lds.w0, kk + 2);
+        hc.issue(lds.h0, kk + 2);
+      });
+      __builtin_amdgcn_s_waitcnt(kLmWaitCopies);
+      __syncthreads();
     }
-    // last slice of the tile: start the next tile's first slice, finish the tile, run its epilogue under the copy
-    if (vt + 1 < vt_end) {
-      unsigned char* nxt = lds + (stage ^ 1) * kLmStageBytes;
-      wc.init(weight, g.w_stride, int64_t(vt + 1) * kLmTile, g.vocab - 1);
-      wc.issue(nxt, 0);
-      hc.issue(nxt + kLmOperandBytes, 0);
-    }
-    lm_mma_stage(lds + stage * kLmStageBytes, wv, wt, lane, acc);
+    // last two slices of the tile; the next tile's first slice is copied under the last one and under the epilogue
+    lm_mma_stage(lds.w0, lds.h0, wv, wt, lane, acc, [&] {
+      wc.issue(lds.w1, nk - 1);
+      hc.issue(lds.h1, nk - 1);
+    });
+    __builtin_amdgcn_s_waitcnt(kLmWaitCopies);
+    __syncthreads();
+    const bool more = vt + 1 < vt_end;
+    if (more) wc.init(weight, g.w_stride, int64_t(vt + 1) * kLmTile, g.vocab - 1);
+    lm_mma_stage(lds.w1, lds.h1, wv, wt, lane, acc, [&] {
+      if (more) {
+        wc.issue(lds.w0, 0);
+        hc.issue(lds.h0, 0);
+      }
+    });
     epilogue(acc, int64_t(vt) * kLmTile);
     lm_zero_acc(acc);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(kLmWaitCopies);
     __syncthreads();
-    stage ^= 1;
   }
 }
 
@@ -220,7 +264,11 @@ __device__ __forceinline__ void lm_absorb_block(const floatx16& blk, int vbase, 
 __global__ __launch_bounds__(kLmThreads, 1) void lmhead_fwd_kernel(const uint16_t* __restrict__ hidden,
                                                                    const uint16_t* __restrict__ weight, LmGeom g,
                                                                    float c, float* __restrict__ partial) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  __shared__ __attribute__((aligned(1024))) unsigned char w0[kLmOperandBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char h0[kLmOperandBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char w1[kLmOperandBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char h1[kLmOperandBytes];
+  unsigned char* smem = w0;
   int rb, split;
   if (!lm_block_coords(g, rb, split)) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wv = wave >> 1, wt = wave & 1;
@@ -234,19 +282,26 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_fwd_kernel(const uint16_
   }
   const int vt_begin = split * g.tiles_per_split;
   const int vt_end = min(g.n_tiles, vt_begin + g.tiles_per_split);
-  lm_pipeline(smem, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
+  lm_pipeline(LmLds{w0, h0, w1, h1}, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
     const int limit = int(min<int64_t>(g.vocab - v0, kLmTile));
     if (limit < kLmTile) {  // ragged last tile: entries past the vocabulary are masked out
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
+        {
           lm_absorb_block<true>(acc[i][j], wv * 128 + i * 32 + 4 * (lane >> 5), limit, c, m[j], s[j], t[j]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) lm_absorb_block<false>(acc[i][j], 0, 0, c, m[j], s[j], t[j]);
+        for (int j = 0; j < 4; ++j) {
+          // one 16-value block at a time: without the barrier all 256 accumulators are copied out of the AGPRs first
+          lm_absorb_block<false>(acc[i][j], 0, 0, c, m[j], s[j], t[j]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
     }
   });
   // merge the two lane halves (same tokens, different vocab rows), then the two waves sharing the tokens
@@ -340,7 +395,10 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_dlogits_kernel(
     const int64_t* __restrict__ targets, const float* __restrict__ lse, const float* __restrict__ spx,
     const float* __restrict__ g_lp, const float* __restrict__ g_ent, const float* __restrict__ grad_scale_dev,
     uint16_t* __restrict__ d_t, int64_t d_stride) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  __shared__ __attribute__((aligned(1024))) unsigned char w0[kLmOperandBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char h0[kLmOperandBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char w1[kLmOperandBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char h1[kLmOperandBytes];
   int rb, split;
   if (!lm_block_coords(g, rb, split)) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wv = wave >> 1, wt = wave & 1;
@@ -362,7 +420,7 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_dlogits_kernel(
   }
   const int vt_begin = split * g.tiles_per_split;
   const int vt_end = min(g.n_tiles, vt_begin + g.tiles_per_split);
-  lm_pipeline(smem, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
+  lm_pipeline(LmLds{w0, h0, w1, h1}, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -380,6 +438,7 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_dlogits_kernel(
             d_t[v * d_stride + tokj[j]] = uint16_t(f32_to_bf16_bits(d));
           }
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
   });
 }
@@ -399,9 +458,9 @@ static int lm_geometry(const char* what, int dtype, int64_t n, int64_t hidden, i
               (long long)vocab);
     return RELAX_AMD_EINVAL;
   }
-  if (hidden % kLmBK != 0 || h_stride % 8 != 0 || w_stride % 8 != 0 || !aligned16(h) || !aligned16(w) ||
+  if (hidden % (2 * kLmBK) != 0 || h_stride % 8 != 0 || w_stride % 8 != 0 || !aligned16(h) || !aligned16(w) ||
       int64_t(kLmTile) * h_stride >= (1LL << 31) || int64_t(kLmTile) * w_stride >= (1LL << 31)) {
-    set_error("%s: hidden size must be a multiple of %d and rows 16-byte aligned (hidden=%lld)", what, kLmBK,
+    set_error("%s: hidden size must be a multiple of %d and rows 16-byte aligned (hidden=%lld)", what, 2 * kLmBK,
               (long long)hidden);
     return RELAX_AMD_EUNSUPPORTED;
   }
@@ -423,17 +482,6 @@ static unsigned lm_grid(const LmGeom& g) {
   const int rb_per_round = kLmXcds * (kLmPerXcd / g.splits);
   const int rounds = (g.row_blocks + rb_per_round - 1) / rb_per_round;
   return unsigned(rounds) * kLmXcds * kLmPerXcd;
-}
-
-template <typename K>
-static int lm_enable_lds(K kernel, const char* what) {
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLmLdsBytes);
-  if (e != hipSuccess) {
-    set_error("%s: cannot reserve %d bytes of LDS: %s", what, kLmLdsBytes, hipGetErrorString(e));
-    return RELAX_AMD_ELAUNCH;
-  }
-  return RELAX_AMD_OK;
 }
 
 extern "C" int64_t relax_amd_lmhead_workspace_bytes(int64_t n_tokens) {
@@ -459,11 +507,10 @@ extern "C" int relax_amd_lmhead_logprob_fwd(const void* hidden, const void* weig
   float* x_target = partial + 8 * 3 * n_tokens;
   const uint16_t* h = static_cast<const uint16_t*>(hidden);
   const uint16_t* w = static_cast<const uint16_t*>(weight);
-  if (int rc = lm_enable_lds(lmhead_fwd_kernel, "lmhead_logprob_fwd")) return rc;
   hipLaunchKernelGGL(lmhead_target_logit_kernel, dim3(unsigned((n_tokens + 3) / 4)), dim3(256), 0, s, h, w, g, targets,
                      x_target);
   if (int rc = check_launch("lmhead_target_logit")) return rc;
-  hipLaunchKernelGGL(lmhead_fwd_kernel, dim3(lm_grid(g)), dim3(kLmThreads), kLmLdsBytes, s, h, w, g,
+  hipLaunchKernelGGL(lmhead_fwd_kernel, dim3(lm_grid(g)), dim3(kLmThreads), 0, s, h, w, g,
                      inv_temperature * kLog2e, partial);
   if (int rc = check_launch("lmhead_fwd")) return rc;
   hipLaunchKernelGGL(lmhead_combine_kernel, dim3(unsigned((n_tokens + 255) / 256)), dim3(256), 0, s, partial, x_target,
@@ -486,8 +533,7 @@ extern "C" int relax_amd_lmhead_dlogits_t(const void* hidden, const void* weight
     return RELAX_AMD_EINVAL;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (int rc = lm_enable_lds(lmhead_dlogits_kernel, "lmhead_dlogits_t")) return rc;
-  hipLaunchKernelGGL(lmhead_dlogits_kernel, dim3(lm_grid(g)), dim3(kLmThreads), kLmLdsBytes, s,
+  hipLaunchKernelGGL(lmhead_dlogits_kernel, dim3(lm_grid(g)), dim3(kLmThreads), 0, s,
                      static_cast<const uint16_t*>(hidden), static_cast<const uint16_t*>(weight), g,
                      inv_temperature * kLog2e, inv_temperature, targets, lse, spx, g_lp, g_ent, grad_scale_dev,
                      static_cast<uint16_t*>(d_t), d_stride);

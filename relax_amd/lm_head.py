@@ -125,9 +125,9 @@ def lm_head_log_probs_and_entropy(hidden, weight, tokens, temperature: float = 1
                                   with_entropy_grad: bool = True):
     """``(log_prob [N] fp32, entropy [N] fp32 | None)`` of ``log_softmax(hidden @ weight.T / temperature)``.
 
-    The kernels consume the hidden size in 64-wide slices; other sizes are zero-padded here (zeros add nothing to
+    The kernels consume the hidden size in pairs of 64-wide slices; other sizes are zero-padded here (zeros add nothing to
     the logits, and autograd through the padding returns gradients of the original shapes)."""
-    pad = (-hidden.size(-1)) % 64
+    pad = (-hidden.size(-1)) % 128
     if pad:
         hidden = torch.nn.functional.pad(hidden, (0, pad))
         weight = torch.nn.functional.pad(weight, (0, pad))

@@ -105,10 +105,10 @@ def test_argument_errors():
     from relax_amd.lm_head import lm_head_log_probs_and_entropy, lmhead_logprob_fwd
 
     dev = require_gpu()
-    hid = torch.randn(8, 48, device=dev).bfloat16()  # hidden size not a multiple of 64: the raw op refuses ...
+    hid = torch.randn(8, 48, device=dev).bfloat16()  # hidden size not a multiple of 128: the raw op refuses ...
     w = torch.randn(16, 48, device=dev).bfloat16()
     tok = torch.zeros(8, dtype=torch.long, device=dev)
-    with pytest.raises(Exception, match="multiple of 64"):
+    with pytest.raises(Exception, match="multiple of 128"):
         lmhead_logprob_fwd(hid, w, tok)
     lp, _ = lm_head_log_probs_and_entropy(hid, w, tok)  # ... and the wrapper pads
     want = torch.log_softmax(hid.float() @ w.float().t(), -1)[:, 0]
