@@ -60,7 +60,6 @@ __device__ __forceinline__ bool lm_block_coords(const LmGeom& g, int& rb, int& s
 // Issued through the builtin so that the compiler's own wait-count bookkeeping sees it.
 constexpr int kLmWaitCopies = 0x0F70;
 constexpr int kLmWaitEverything = 0x0070;  // vmcnt = 0 and lgkmcnt = 0
-constexpr int kLmWaitAllButLastFrags = 0xC87F;  // lgkmcnt = 8: all LDS reads but the newest fragment set have landed
 
 struct LmCopier {
   const unsigned char* base;  // first row of the tile (wave-uniform, lives in scalar registers)
@@ -76,19 +75,20 @@ struct LmCopier {
   }
   // `tile` = LDS address of this operand's tile in the target stage.  The source address is a scalar base plus a
   // 32-bit per-lane offset, so each copy needs one address register instead of a 64-bit pair.
-  __device__ __forceinline__ void issue(unsigned char* tile, int kslice) const {
+  __device__ __forceinline__ void issue_pass(unsigned char* tile, int kslice, int p) const {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     uint64_t slice = reinterpret_cast<uint64_t>(base) + uint64_t(kslice) * (kLmBK * 2);
-    asm volatile("" : "+s"(slice));  // keep scalar + 32-bit lane offset apart (no hoisted 64-bit lane addresses)
+    asm volatile("" : "+s"(slice));  // keep scalar base + 32-bit lane offset apart (no hoisted 64-bit lane addresses)
+    uint32_t lane_off = off[p];
+    asm volatile("" : "+v"(lane_off));  // widen next to the copy so it folds into the scalar-base address form
+    const unsigned char* src = reinterpret_cast<const unsigned char*>(slice + uint64_t(lane_off));
+    unsigned char* dst = tile + (p * 32 + wave * 8) * (kLmBK * 2);  // wave-uniform; lane l lands at dst + 16*l
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src),
+                                     (__attribute__((address_space(3))) void*)(dst), 16, 0, 0);
+  }
+  __device__ __forceinline__ void issue(unsigned char* tile, int kslice) const {
 #pragma unroll
-    for (int p = 0; p < kLmPasses; ++p) {
-      uint32_t lane_off = off[p];
-      asm volatile("" : "+v"(lane_off));  // widen next to the copy so it folds into the scalar-base address form
-      const unsigned char* src = reinterpret_cast<const unsigned char*>(slice + uint64_t(lane_off));
-      unsigned char* dst = tile + (p * 32 + wave * 8) * (kLmBK * 2);  // wave-uniform; lane l lands at dst + 16*l
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src),
-                                       (__attribute__((address_space(3))) void*)(dst), 16, 0, 0);
-    }
+    for (int p = 0; p < kLmPasses; ++p) issue_pass(tile, kslice, p);
   }
 };
 
@@ -99,55 +99,67 @@ __device__ __forceinline__ int lm_frag_offset(int lane, int ks) {
   return row * (kLmBK * 2) + (((2 * ks + (lane >> 5)) ^ ((row >> 1) & 7)) * 16);
 }
 
+// Operands of the 16 MFMAs of one 16-wide k-step: four 32-row weight fragments and four 32-row hidden fragments.
 struct LmFrags {
   bf16x8 a[4], b[4];
 };
 
-__device__ __forceinline__ void lm_load_frags(const unsigned char* ws, const unsigned char* hs, int wv, int wt, int lane,
-                                              int ks, LmFrags& f) {
+// One pipeline stage in LDS (a 64-wide k-slice of both operands) as seen by one wave: its 128 weight rows and its
+// 128 hidden rows.
+struct LmStage {
+  const unsigned char* w;
+  const unsigned char* h;
+};
+
+// LDS read number n (0..7) of the fragment set of k-step `ks`: weight fragments first, then hidden fragments.
+__device__ __forceinline__ void lm_load_frag(const LmStage& st, int lane, int ks, int n, LmFrags& f) {
   const int fo = lm_frag_offset(lane, ks);
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-    f.a[i] = *reinterpret_cast<const bf16x8*>(ws + (wv * 128 + i * 32) * (kLmBK * 2) + fo);
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-    f.b[j] = *reinterpret_cast<const bf16x8*>(hs + (wt * 128 + j * 32) * (kLmBK * 2) + fo);
+  if (n < 4)
+    f.a[n] = *reinterpret_cast<const bf16x8*>(st.w + n * 32 * (kLmBK * 2) + fo);
+  else
+    f.b[n - 4] = *reinterpret_cast<const bf16x8*>(st.h + (n - 4) * 32 * (kLmBK * 2) + fo);
 }
 
-__device__ __forceinline__ void lm_mma_frags(const LmFrags& f, floatx16 (&acc)[4][4]) {
+// The 16 MFMAs of one k-step with other work slotted in between: `between(n)` is emitted right after MFMA n, so LDS
+// reads and global -> LDS copies issue in the shadow of the 8-pass matrix instructions instead of in front of them.
+// The scheduling barriers pin that order (the compiler would otherwise sink every fragment read next to its use).
+template <typename Between>
+__device__ __forceinline__ void lm_mma_group(const LmFrags& f, floatx16 (&acc)[4][4], Between&& between) {
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
+    for (int j = 0; j < 4; ++j) {
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
+      between(i * 4 + j);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 }
 
-// 64 MFMAs per wave on one stage.  Fragments are double-buffered: the LDS reads of k-step ks+2 are issued before
-// the 16 MFMAs of k-step ks+1 start, and `issue_copies` (the next slice's global -> LDS copies) is slotted in after
-// the first two fragment sets are on their way, so neither LDS nor global latency sits between MFMAs.  The scheduling
-// barriers pin this order (the compiler would otherwise sink each fragment read next to its first use).
-template <typename IssueCopies>
-__device__ __forceinline__ void lm_mma_stage(const unsigned char* ws, const unsigned char* hs, int wv, int wt, int lane,
-                                             floatx16 (&acc)[4][4], IssueCopies&& issue_copies) {
-  LmFrags f0, f1;
-  lm_load_frags(ws, hs, wv, wt, lane, 0, f0);
-  lm_load_frags(ws, hs, wv, wt, lane, 1, f1);
-  __builtin_amdgcn_sched_barrier(0);
-  issue_copies();
-  __builtin_amdgcn_sched_barrier(0);
-  lm_mma_frags(f0, acc);
-  __builtin_amdgcn_sched_barrier(0);
-  lm_load_frags(ws, hs, wv, wt, lane, 2, f0);
-  __builtin_amdgcn_sched_barrier(0);
-  lm_mma_frags(f1, acc);
-  __builtin_amdgcn_sched_barrier(0);
-  lm_load_frags(ws, hs, wv, wt, lane, 3, f1);
-  __builtin_amdgcn_sched_barrier(0);
-  __builtin_amdgcn_s_waitcnt(kLmWaitAllButLastFrags);
-  __builtin_amdgcn_sched_barrier(0);
-  lm_mma_frags(f0, acc);
-  __builtin_amdgcn_sched_barrier(0);
-  lm_mma_frags(f1, acc);
-  __builtin_amdgcn_sched_barrier(0);
+// k-steps 0..2 of the slice in `st`; on entry f0 holds (or is receiving) the fragments of k-step 0, on exit f1 those
+// of k-step 3, whose MFMAs are left to the caller: they run after the next barrier and cover the LDS latency of the
+// next slice's first fragments.
+__device__ __forceinline__ void lm_slice_body(const LmStage& st, int lane, LmFrags& f0, LmFrags& f1,
+                                              floatx16 (&acc)[4][4]) {
+  lm_mma_group(f0, acc, [&](int n) {
+    if (n < 8) lm_load_frag(st, lane, 1, n, f1);
+  });
+  lm_mma_group(f1, acc, [&](int n) {
+    if (n < 8) lm_load_frag(st, lane, 2, n, f0);
+  });
+  lm_mma_group(f0, acc, [&](int n) {
+    if (n < 8) lm_load_frag(st, lane, 3, n, f1);
+  });
+}
+
+// The previous slice's last k-step (fragments in f1) while the fragments of k-step 0 of the slice in `st` load into
+// f0 and `copy(n)`, n = 0..15, issues the 16 global -> LDS copies of the slice after it.
+template <typename Copy>
+__device__ __forceinline__ void lm_slice_head(const LmStage& st, int lane, LmFrags& f0, const LmFrags& f1,
+                                              floatx16 (&acc)[4][4], Copy&& copy) {
+  lm_mma_group(f1, acc, [&](int n) {
+    if (n < 8) lm_load_frag(st, lane, 0, n, f0);
+    copy(n);
+  });
 }
 
 __device__ __forceinline__ void lm_zero_acc(floatx16 (&acc)[4][4]) {
@@ -159,14 +171,24 @@ __device__ __forceinline__ void lm_zero_acc(floatx16 (&acc)[4][4]) {
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 }
 
+// "my copies have landed" + workgroup barrier: after it the slice copied last is visible to every wave and every wave
+// has finished reading the stage that is overwritten next.
+__device__ __forceinline__ void lm_slice_sync() {
+  __builtin_amdgcn_s_waitcnt(kLmWaitCopies);
+  __syncthreads();
+}
+
 // Walks the vocabulary tiles [vt_begin, vt_end) of one 256-token row block as a single software pipeline over
 // (tile, k-slice) and hands every finished 256x256 logits tile (fp32, un-scaled) to `epilogue(acc, v0)`, which runs
 // while the first slice of the next tile is already in flight.
-// The two pipeline stages are two distinct LDS objects (not halves of one buffer) so that the compiler can prove that
-// the fragment reads of one stage never alias the in-flight global -> LDS copies into the other; otherwise it waits
-// for the copies before every LDS read and the overlap is lost.
+// Per slice and wave: barrier, then 64 MFMAs with the 32 fragment reads and the 16 copies of the following slice
+// slotted between them.  The slice's last k-step is multiplied after the next barrier, so that barrier's wake-up
+// and the first fragment reads of the new slice are covered by 16 MFMAs already in registers.
+// The four operand tiles of the two-stage ring are distinct LDS objects (not regions of one buffer) so that the
+// compiler can prove that fragment reads from one stage never alias the in-flight copies into the other; otherwise
+// it waits for the copies before every LDS read and the overlap is lost.
 struct LmLds {
-  unsigned char *w0, *h0, *w1, *h1;  // weight / hidden tile of stage 0 and of stage 1, four separate objects
+  unsigned char *w0, *h0, *w1, *h1;  // weight / hidden tile of stage 0 and of stage 1
 };
 
 template <typename Epilogue>
@@ -175,6 +197,8 @@ __device__ __forceinline__ void lm_pipeline(const LmLds lds, const uint16_t* hid
                                             Epilogue&& epilogue) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wv = wave >> 1, wt = wave & 1;
   const int nk = int(g.hidden / kLmBK);  // even: the hidden size is a multiple of 2 * kLmBK
+  const LmStage st0 = {lds.w0 + wv * 128 * (kLmBK * 2), lds.h0 + wt * 128 * (kLmBK * 2)};
+  const LmStage st1 = {lds.w1 + wv * 128 * (kLmBK * 2), lds.h1 + wt * 128 * (kLmBK * 2)};
   LmCopier hc, wc;
   hc.init(hidden, g.h_stride, tok0, g.n_tokens - 1);
   floatx16 acc[4][4];
@@ -183,47 +207,54 @@ __device__ __forceinline__ void lm_pipeline(const LmLds lds, const uint16_t* hid
   wc.init(weight, g.w_stride, int64_t(vt_begin) * kLmTile, g.vocab - 1);
   wc.issue(lds.w0, 0);
   hc.issue(lds.h0, 0);
-  __builtin_amdgcn_s_waitcnt(kLmWaitCopies);
-  __syncthreads();
+  lm_slice_sync();
+  LmFrags f0, f1;
   for (int vt = vt_begin; vt < vt_end; ++vt) {
     // Settle register reloads left over from the epilogue here, once per tile; otherwise the compiler waits for them
     // at their first use inside the steady-state loop, which also drains the copies issued just before.
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(kLmWaitEverything);
     __builtin_amdgcn_sched_barrier(0);
-    for (int kk = 0; kk + 2 < nk; kk += 2) {  // steady state: copy slice k+1 while multiplying slice k
-      lm_mma_stage(lds.w0, lds.h0, wv, wt, lane, acc, [&] {
-        wc.issue(lds.w1, kk + 1);
-        hc.issue(lds.h1, kk + 1);
+    // slice 0 (stage 0): nothing to multiply yet, so its first fragments are waited for in the open
+#pragma unroll
+    for (int n = 0; n < 8; ++n) lm_load_frag(st0, lane, 0, n, f0);
+    wc.issue(lds.w1, 1);
+    hc.issue(lds.h1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    lm_slice_body(st0, lane, f0, f1, acc);
+    lm_slice_sync();
+    for (int s = 1; s + 1 < nk; s += 2) {  // odd slices live in stage 1, even slices in stage 0
+      lm_slice_head(st1, lane, f0, f1, acc, [&](int n) {
+        if (n < 8)
+          wc.issue_pass(lds.w0, s + 1, n);
+        else
+          hc.issue_pass(lds.h0, s + 1, n - 8);
       });
-      __builtin_amdgcn_s_waitcnt(kLmWaitCopies);
-      __syncthreads();
-      lm_mma_stage(lds.w1, lds.h1, wv, wt, lane, acc, [&] {
-        wc.issue(lds.w0, kk + 2);
-        hc.issue(lds.h0, kk + 2);
+      lm_slice_body(st1, lane, f0, f1, acc);
+      lm_slice_sync();
+      lm_slice_head(st0, lane, f0, f1, acc, [&](int n) {
+        if (n < 8)
+          wc.issue_pass(lds.w1, s + 2, n);
+        else
+          hc.issue_pass(lds.h1, s + 2, n - 8);
       });
-      __builtin_amdgcn_s_waitcnt(kLmWaitCopies);
-      __syncthreads();
+      lm_slice_body(st0, lane, f0, f1, acc);
+      lm_slice_sync();
     }
-    // last two slices of the tile; the next tile's first slice is copied under the last one and under the epilogue
-    lm_mma_stage(lds.w0, lds.h0, wv, wt, lane, acc, [&] {
-      wc.issue(lds.w1, nk - 1);
-      hc.issue(lds.h1, nk - 1);
+    // Last slice of the tile (stage 1).  The copies issued under it fetch the next tile's first slice; after the last
+    // tile they re-fetch this tile's first slice, which nobody reads (cheaper than a branch between the MFMAs).
+    if (vt + 1 < vt_end) wc.init(weight, g.w_stride, int64_t(vt + 1) * kLmTile, g.vocab - 1);
+    lm_slice_head(st1, lane, f0, f1, acc, [&](int n) {
+      if (n < 8)
+        wc.issue_pass(lds.w0, 0, n);
+      else
+        hc.issue_pass(lds.h0, 0, n - 8);
     });
-    __builtin_amdgcn_s_waitcnt(kLmWaitCopies);
-    __syncthreads();
-    const bool more = vt + 1 < vt_end;
-    if (more) wc.init(weight, g.w_stride, int64_t(vt + 1) * kLmTile, g.vocab - 1);
-    lm_mma_stage(lds.w1, lds.h1, wv, wt, lane, acc, [&] {
-      if (more) {
-        wc.issue(lds.w0, 0);
-        hc.issue(lds.h0, 0);
-      }
-    });
+    lm_slice_body(st1, lane, f0, f1, acc);
+    lm_mma_group(f1, acc, [](int) {});
     epilogue(acc, int64_t(vt) * kLmTile);
     lm_zero_acc(acc);
-    __builtin_amdgcn_s_waitcnt(kLmWaitCopies);
-    __syncthreads();
+    lm_slice_sync();
   }
 }
 
