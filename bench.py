@@ -8,6 +8,11 @@ actor step: 16 sequences x 4096 tokens = 65536 rows x 151936 vocabulary, logits 
 first 20 % of every sequence masked out.
 
 Prints ONE JSON line (metric, value, roofline of the dominant kernel, CPU baseline of the same arithmetic).
+
+``--workload`` selects the other configurations of the same path, each printed in the same format:
+``lmhead`` (fused LM-head + log-prob/entropy forward and dhidden/dweight backward, hidden [32768, 4096], MFMA-bound),
+``reverse_kl`` (on-policy distillation, student/teacher [16384, 151936], forward + student dlogits),
+``varlen_gspo`` / ``varlen_cispo`` (8 packed sequences of 2k-32k tokens, RLOO advantages, sequence-level losses).
 """
 
 from __future__ import annotations
@@ -24,6 +29,8 @@ import torch
 VOCAB = 151936
 SEQS, SEQ_LEN = 16, 4096
 HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+METRIC = "tokens/s fused logprob+entropy+loss fwd+bwd @V=151936 bf16; % HBM/MFMA peak"
 # HBM bytes one actor_step_fused launch moves at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # at the L2 <-> fabric boundary (profiles/actor_step_fused_bf16_v151936_n65536.md): 26 780 743 KiB fetched
 # (counter x 2.000) + 19 464 492 KiB written.
@@ -121,39 +128,47 @@ def cpu_baseline(args, rows: int, vocab: int, budget_s: float = 12.0, max_reps: 
     }
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--seqs", type=int, default=SEQS)
-    ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
-    ap.add_argument("--vocab", type=int, default=VOCAB)
-    ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the CPU baseline slab (0 = skip)")
-    ap.add_argument("--two-launch", action="store_true",
-                    help="use the separate forward / backward launches (the path GSPO takes) instead of the fused step")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also launch one plain 1 GiB device copy, the known-size reference for FETCH_SIZE/WRITE_SIZE")
-    a = ap.parse_args()
-    if a.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (rows shard trivially; see DESIGN.md). "
-              "Run with --gpus 1.", file=sys.stderr)
-        return 2
-    if not torch.cuda.is_available():
-        print("bench.py needs a ROCm GPU", file=sys.stderr)
-        return 2
+def timed_steps(step, warmup: int, steps: int):
+    """``warmup`` untimed steps, then exactly ``steps`` timed ones bracketed by device synchronisation; returns
+    (wall seconds, {kernel name: mean HIP-event ms per launch, launches per step}, last step's result)."""
+    from relax_amd import ops
+
+    out = None
+    for _ in range(warmup):
+        out = step()
+    torch.cuda.synchronize()
+    ops.kernel_events = []  # HIP events around the big launches, on the stream they are launched on
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    events, ops.kernel_events = ops.kernel_events, None
+    per_kernel = {}
+    for name, e0, e1 in events:
+        per_kernel.setdefault(name, []).append(e0.elapsed_time(e1))
+    kernel_ms = {k: sum(v) / len(v) for k, v in per_kernel.items()}
+    launches = {k: len(v) / steps for k, v in per_kernel.items()}
+    return wall, kernel_ms, launches, out
+
+
+def emit(a, n_tokens, wall, workload, config, roofline, cpu):
+    print(json.dumps({
+        "metric": METRIC, "value": n_tokens / (wall / a.steps), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": wall * 1e3 / a.steps, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": {"workload": workload, **config},
+        "roofline": roofline, "cpu_baseline": cpu,
+    }))
+
+
+def run_actor_step(a, dev) -> None:
     import relax_amd
 
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
     args = make_args()
     logits, batch, g = make_workload(dev, a.seqs, a.seq_len, a.vocab)
     attach_old_and_ref(batch, logits, args, g)
     logits.requires_grad_()
     n_tokens = a.seqs * a.seq_len
-
-    from relax_amd import ops
-
     if a.two_launch:
         args.relax_amd_single_pass = "off"
 
@@ -170,23 +185,9 @@ def main() -> int:
         dst.copy_(src)  # reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
-    for _ in range(a.warmup):
-        step()
-    torch.cuda.synchronize()
-    ops.kernel_events = []  # HIP events around the big launches, on the stream they are launched on
-    t0 = time.perf_counter()
-    for _ in range(a.steps):
-        loss = step()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    events, ops.kernel_events = ops.kernel_events, None
-    per_kernel = {}
-    for name, e0, e1 in events:
-        per_kernel.setdefault(name, []).append(e0.elapsed_time(e1))
-    kernel_ms = {k: sum(v) / len(v) for k, v in per_kernel.items()}
+    wall, kernel_ms, _, loss = timed_steps(step, a.warmup, a.steps)
     ms_per_step = wall * 1e3 / a.steps
-    elem = logits.element_size()
-    row_bytes = float(a.vocab * elem) * n_tokens
+    row_bytes = float(a.vocab * logits.element_size()) * n_tokens
     if "actor_step_fused" in kernel_ms:
         # one launch does the forward scan and the dlogits backward: 3*V*s algorithmic bytes per token (forward read,
         # backward read, dlogits write); its second read is served by cache, see "traffic"
@@ -196,33 +197,201 @@ def main() -> int:
         dom, dom_name, dom_bytes = kernel_ms["logprob_entropy_bwd"], "logprob_entropy_bwd_kernel<bf16_t, true>", 2.0 * row_bytes
         traffic = None
     achieved = dom_bytes / (dom * 1e-3) / 1e9
-    out = {
-        "metric": "tokens/s fused logprob+entropy+loss fwd+bwd @V=151936 bf16; % HBM/MFMA peak",
-        "value": n_tokens / (wall / a.steps),
-        "unit": "tokens/s",
-        "n_gpus": 1,
-        "steps": a.steps,
-        "warmup": a.warmup,
-        "ms_per_step": ms_per_step,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
-        "config": {
-            "workload": f"Qwen3-8B-shaped actor step: {a.seqs} seqs x {a.seq_len} tokens = {n_tokens} rows x "
-                        f"V={a.vocab} bf16 logits, PPO-clip 0.2/0.28 + k3 KL 1e-3, fwd + bwd to dlogits",
-            "rows": n_tokens, "vocab": a.vocab, "loss": float(loss.item()),
-        },
-        "roofline": {
-            "bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "algorithmic_bytes_per_launch": dom_bytes,
-            "avg_launch_ms": dom, "kernel_ms": kernel_ms,
-            "step_algorithmic_GBs": 3.0 * row_bytes / (ms_per_step * 1e-3) / 1e9,
-        },
-        "cpu_baseline": cpu_baseline(args, a.cpu_rows, a.vocab) if a.cpu_rows > 0 else None,
-    }
-    print(json.dumps(out))
+    emit(a, n_tokens, wall,
+         f"Qwen3-8B-shaped actor step: {a.seqs} seqs x {a.seq_len} tokens = {n_tokens} rows x V={a.vocab} bf16 "
+         f"logits, PPO-clip 0.2/0.28 + k3 KL 1e-3, fwd + bwd to dlogits",
+         {"rows": n_tokens, "vocab": a.vocab, "loss": float(loss.item())},
+         {"bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+          "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "algorithmic_bytes_per_launch": dom_bytes,
+          "avg_launch_ms": dom, "kernel_ms": kernel_ms,
+          "step_algorithmic_GBs": 3.0 * row_bytes / (ms_per_step * 1e-3) / 1e9},
+         cpu_baseline(args, a.cpu_rows, a.vocab) if a.cpu_rows > 0 else None)
+
+
+def run_lmhead(a, dev) -> None:
+    """hidden [N, 4096] ~ N(0, 1), weight [V, 4096] ~ N(0, 0.02), scalar PPO-style loss with advantages ~ N(0, 1):
+    forward log-prob + entropy without materialised logits, backward to dhidden and dweight."""
+    from relax_amd.lm_head import lm_head_log_probs_and_entropy
+
+    n, h, v = a.rows or 32768, a.hidden, a.vocab
+    g = torch.Generator(device=dev).manual_seed(0)
+    hidden = torch.randn(n, h, device=dev, generator=g).bfloat16().requires_grad_()
+    weight = (torch.randn(v, h, device=dev, generator=g) * 0.02).bfloat16().requires_grad_()
+    tokens = torch.randint(0, v, (n,), device=dev, generator=g)
+    adv = torch.randn(n, device=dev, generator=g) / n
+
+    def step():
+        hidden.grad = None
+        weight.grad = None
+        lp, ent = lm_head_log_probs_and_entropy(hidden, weight, tokens, 1.0, True, False)
+        loss = -(adv * lp).sum()
+        loss.backward()
+        return loss
+
+    wall, kernel_ms, launches, loss = timed_steps(step, a.warmup, a.steps)
+    # the timed forward region holds the target-logit gather, the MFMA kernel and the split combine; the MFMA kernel
+    # is > 99 % of it (see the rocprofv3 summary), so its event time stands for lmhead_fwd_kernel
+    dom = kernel_ms["lmhead_logprob_fwd"]
+    flops = 2.0 * n * h * v
+    achieved = flops / (dom * 1e-3) / 1e12
+    emit(a, n, wall,
+         f"fused LM-head + log-prob/entropy: hidden bf16 [{n}, {h}], weight bf16 [{v}, {h}], fwd (no logits in HBM) + "
+         f"bwd to dhidden/dweight from a scalar loss",
+         {"rows": n, "hidden": h, "vocab": v, "loss": float(loss.item())},
+         {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
+          "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+          "algorithmic_flops_per_launch": flops, "avg_launch_ms": dom, "kernel_ms": kernel_ms,
+          "launches_per_step": launches,
+          "step_TFLOPs_credited_6NHV": 6.0 * n * h * v / (wall / a.steps) / 1e12},
+         None)
+
+
+def run_reverse_kl(a, dev) -> None:
+    """student / teacher bf16 logits [N, V], teacher = student + N(0, 1); per-token full-vocabulary reverse KL with a
+    15 % zero loss mask, token-mean reduction, backward to the student's dlogits."""
+    from relax_amd import opd_utils
+
+    n, v = a.rows or 16384, a.vocab
+    g = torch.Generator(device=dev).manual_seed(0)
+    student = torch.empty((n, v), dtype=torch.bfloat16, device=dev)
+    teacher = torch.empty_like(student)
+    for s in range(0, n, 2048):
+        e = min(n, s + 2048)
+        x = torch.randn((e - s, v), device=dev, generator=g) * 3.0
+        student[s:e] = x.to(torch.bfloat16)
+        teacher[s:e] = (x + torch.randn((e - s, v), device=dev, generator=g)).to(torch.bfloat16)
+        del x
+    student.requires_grad_()
+    mask = (torch.rand(n, device=dev, generator=g) >= 0.15).float()
+    batch = {"loss_masks": [mask], "response_lengths": [n]}
+
+    def step():
+        student.grad = None
+        kl = opd_utils.compute_opd_kl_full_vocab(student, teacher)
+        loss = opd_utils.reduce_opd_loss(batch, kl)
+        loss.backward()
+        return loss
+
+    wall, kernel_ms, _, loss = timed_steps(step, a.warmup, a.steps)
+    row_bytes = float(v * 2) * n
+    dom = kernel_ms["reverse_kl_bwd"]
+    dom_bytes = 3.0 * row_bytes  # read student + teacher rows, write the student gradient row
+    achieved = dom_bytes / (dom * 1e-3) / 1e9
+    emit(a, n, wall,
+         f"on-policy distillation: student/teacher bf16 logits [{n}, {v}], full-vocab reverse KL, token-mean, fwd + "
+         f"student dlogits bwd",
+         {"rows": n, "vocab": v, "loss": float(loss.item())},
+         {"bound": "hbm", "kernel": "reverse_kl_bwd_kernel<bf16_t>", "achieved": achieved, "peak": HBM_PEAK_GBS,
+          "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": dom_bytes,
+          "avg_launch_ms": dom, "kernel_ms": kernel_ms,
+          "step_algorithmic_GBs": 5.0 * row_bytes / (wall / a.steps) / 1e9},
+         None)
+
+
+def run_varlen(a, dev, loss_kind: str) -> None:
+    """8 packed sequences with lengths ~ U[2k, 32k], 3-6 masked tool-output spans (~30 % of tokens) per sequence,
+    RLOO advantages from rewards ~ U[0, 1] over the group of 8, GSPO (clip 3e-4/4e-4) or CISPO loss,
+    sequence-mean-token-sum aggregation."""
+    import relax_amd
+    from relax_amd import ppo_utils
+
+    cpu = torch.Generator().manual_seed(0)
+    seqs, v = 8, a.vocab
+    lengths = [int(x) for x in torch.randint(2048, 32769, (seqs,), generator=cpu)]
+    while sum(lengths) > 131072:
+        lengths[lengths.index(max(lengths))] //= 2
+    n = sum(lengths)
+    g = torch.Generator(device=dev).manual_seed(0)
+    logits = torch.empty((1, n, v), dtype=torch.bfloat16, device=dev)
+    for s in range(0, n, 2048):
+        e = min(n, s + 2048)
+        logits[0, s:e] = (torch.randn((e - s, v), device=dev, generator=g) * 3.0).to(torch.bfloat16)
+    masks = []
+    for ln in lengths:
+        m = torch.ones(ln)
+        spans = int(torch.randint(3, 7, (1,), generator=cpu))
+        for _ in range(spans):
+            w = int(0.3 * ln / spans)
+            st = int(torch.randint(0, ln - w, (1,), generator=cpu))
+            m[st:st + w] = 0.0
+        masks.append(m.to(dev))
+    args = make_args()
+    args.advantage_estimator = loss_kind
+    args.use_kl_loss = False
+    if loss_kind == "gspo":
+        args.eps_clip, args.eps_clip_high = 3e-4, 4e-4
+    rewards = torch.rand(seqs, generator=cpu).to(dev)
+    shaped = ppo_utils.compute_rloo_leave_one_out_rewards(rewards)
+    batch = dict(
+        unconcat_tokens=[torch.randint(0, v, (ln,), device=dev, generator=g) for ln in lengths],
+        total_lengths=lengths, response_lengths=lengths, loss_masks=masks,
+        advantages=[shaped[i].expand(ln).contiguous() for i, ln in enumerate(lengths)],
+        # sequence-mean-token-sum: every sample's masked token sum is divided by the number of sequences
+        relax_amd_sample_denominators=torch.full((seqs,), float(seqs), device=dev),
+    )
+    attach_old_and_ref(batch, logits, args, g)
+    logits.requires_grad_()
+
+    def step():
+        logits.grad = None
+        loss, _ = relax_amd.policy_loss_function(args, batch, logits, None)
+        loss.backward()
+        return loss
+
+    wall, kernel_ms, _, loss = timed_steps(step, a.warmup, a.steps)
+    row_bytes = float(v * 2) * n
+    name = "actor_step_fused" if "actor_step_fused" in kernel_ms else "logprob_entropy_bwd"
+    dom = kernel_ms[name]
+    dom_bytes = (3.0 if name == "actor_step_fused" else 2.0) * row_bytes
+    achieved = dom_bytes / (dom * 1e-3) / 1e9
+    emit(a, n, wall,
+         f"packed varlen: {seqs} sequences {lengths} = {n} rows x V={v} bf16 logits, ~30 % masked spans, RLOO "
+         f"advantages, {loss_kind.upper()} loss, sequence-mean-token-sum, fwd + bwd to dlogits",
+         {"rows": n, "vocab": v, "loss": float(loss.item()), "lengths": lengths},
+         {"bound": "hbm", "kernel": name + "_kernel<bf16_t>", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+          "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": dom_bytes,
+          "avg_launch_ms": dom, "kernel_ms": kernel_ms,
+          "step_algorithmic_GBs": 3.0 * row_bytes / (wall / a.steps) / 1e9},
+         None)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="actor_step",
+                    choices=["actor_step", "lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo"])
+    ap.add_argument("--seqs", type=int, default=SEQS)
+    ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
+    ap.add_argument("--vocab", type=int, default=VOCAB)
+    ap.add_argument("--rows", type=int, default=0, help="token rows of the lmhead / reverse_kl workloads (0 = default)")
+    ap.add_argument("--hidden", type=int, default=4096, help="hidden size of the lmhead workload")
+    ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the CPU baseline slab (0 = skip)")
+    ap.add_argument("--two-launch", action="store_true",
+                    help="use the separate forward / backward launches (the path GSPO takes) instead of the fused step")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain 1 GiB device copy, the known-size reference for FETCH_SIZE/WRITE_SIZE")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (token rows shard without any exchange). "
+              "Run with --gpus 1.", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm GPU", file=sys.stderr)
+        return 2
+    import relax_amd  # noqa: F401  (fails loudly when the HIP library is missing)
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if a.workload == "actor_step":
+        run_actor_step(a, dev)
+    elif a.workload == "lmhead":
+        run_lmhead(a, dev)
+    elif a.workload == "reverse_kl":
+        run_reverse_kl(a, dev)
+    else:
+        run_varlen(a, dev, a.workload.split("_")[1])
     return 0
 
 

@@ -16,7 +16,8 @@ import re
 import torch  # noqa: F401
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "librelax_amd.so")
+# RELAX_AMD_LIBRARY points at a build of the library kept somewhere else (same ABI); default: next to this file.
+LIB_PATH = os.environ.get("RELAX_AMD_LIBRARY") or os.path.join(HERE, "librelax_amd.so")
 HEADER_PATH = os.path.join(os.path.dirname(HERE), "include", "relax_amd.h")
 
 F32, BF16, F16, F64 = 0, 1, 2, 3

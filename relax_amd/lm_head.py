@@ -14,6 +14,7 @@ import torch
 
 from . import _lib
 from ._lib import check, lib
+from . import ops
 from .ops import _need_gpu, _p, _stream
 
 # rows of the transposed-gradient slab the backward materialises at a time: [V, SLAB] bf16
@@ -45,9 +46,10 @@ def lmhead_logprob_fwd(hidden, weight, targets, inv_temperature: float = 1.0, wi
     if n == 0:
         return lp, ent, lse, spx
     ws = torch.empty(lib.relax_amd_lmhead_workspace_bytes(n), dtype=torch.uint8, device=dev)
-    check(lib.relax_amd_lmhead_logprob_fwd(_p(hidden), _p(weight), _lib.BF16, n, h, v, hidden.stride(0),
-                                           weight.stride(0), _p(targets), float(inv_temperature), _p(ws), _p(lp),
-                                           _p(ent), _p(lse), _p(spx), _stream()))
+    with ops._timed("lmhead_logprob_fwd"):
+        check(lib.relax_amd_lmhead_logprob_fwd(_p(hidden), _p(weight), _lib.BF16, n, h, v, hidden.stride(0),
+                                               weight.stride(0), _p(targets), float(inv_temperature), _p(ws), _p(lp),
+                                               _p(ent), _p(lse), _p(spx), _stream()))
     return lp, ent, lse, spx
 
 
@@ -57,9 +59,10 @@ def lmhead_dlogits_t(hidden, weight, targets, lse, spx, g_lp, g_ent, inv_tempera
     v = weight.size(0)
     if out is None:
         out = torch.empty((v, n), dtype=torch.bfloat16, device=hidden.device)
-    check(lib.relax_amd_lmhead_dlogits_t(_p(hidden), _p(weight), _lib.BF16, n, h, v, hidden.stride(0),
-                                         weight.stride(0), _p(targets), _p(lse), _p(spx), _p(g_lp), _p(g_ent), None,
-                                         float(inv_temperature), _p(out), out.stride(0), _stream()))
+    with ops._timed("lmhead_dlogits_t"):
+        check(lib.relax_amd_lmhead_dlogits_t(_p(hidden), _p(weight), _lib.BF16, n, h, v, hidden.stride(0),
+                                             weight.stride(0), _p(targets), _p(lse), _p(spx), _p(g_lp), _p(g_ent),
+                                             None, float(inv_temperature), _p(out), out.stride(0), _stream()))
     return out
 
 
@@ -109,9 +112,11 @@ class FusedLMHeadLogProb(torch.autograd.Function):
             lmhead_dlogits_t(hidden[s:e], weight, targets[s:e], lse[s:e], None if spx is None else spx[s:e],
                              g_lp[s:e], None if g_ent is None else g_ent[s:e], ctx.inv_temperature, out=d_t)
             if need_h:
-                torch.mm(d_t.t(), weight, out=d_hidden[s:e])
+                with ops._timed("lmhead_dhidden_gemm"):
+                    torch.mm(d_t.t(), weight, out=d_hidden[s:e])
             if need_w:
-                part = torch.mm(d_t, hidden[s:e])
+                with ops._timed("lmhead_dweight_gemm"):
+                    part = torch.mm(d_t, hidden[s:e])
                 if s == 0 and e == n:
                     return d_hidden, part, None, None, None, None
                 if d_weight32 is None:

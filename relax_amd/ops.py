@@ -344,8 +344,9 @@ def reverse_kl_fwd(student, teacher):
     kw = dict(dtype=torch.float32, device=s.device)
     kl, ls, lt = torch.empty(n, **kw), torch.empty(n, **kw), torch.empty(n, **kw)
     stride = s.stride(0) if n > 1 else s.size(1)
-    check(lib.relax_amd_reverse_kl_fwd(_p(s), _p(t), _code(s), n, s.size(1), stride, _p(kl), _p(ls), _p(lt),
-                                       _stream()))
+    with _timed("reverse_kl_fwd"):
+        check(lib.relax_amd_reverse_kl_fwd(_p(s), _p(t), _code(s), n, s.size(1), stride, _p(kl), _p(ls), _p(lt),
+                                           _stream()))
     return kl, ls, lt, s, t
 
 
@@ -355,8 +356,10 @@ def reverse_kl_bwd(s, t, kl, ls, lt, g, grad_scale: float = 1.0, grad_scale_dev=
     if stride != s.size(1):
         raise ValueError("reverse_kl_bwd writes a dense gradient: student rows must be contiguous")
     d = torch.empty_like(s)
-    check(lib.relax_amd_reverse_kl_bwd(_p(s), _p(t), _code(s), n, s.size(1), stride, _p(kl), _p(ls), _p(lt),
-                                       _p(_f32(g)), float(grad_scale), _p(grad_scale_dev), _p(d), _stream()))
+    g = _f32(g)
+    with _timed("reverse_kl_bwd"):
+        check(lib.relax_amd_reverse_kl_bwd(_p(s), _p(t), _code(s), n, s.size(1), stride, _p(kl), _p(ls), _p(lt),
+                                           _p(g), float(grad_scale), _p(grad_scale_dev), _p(d), _stream()))
     return d
 
 
