@@ -17,8 +17,9 @@ from ._lib import check, lib
 from . import ops
 from .ops import _need_gpu, _p, _stream
 
-# rows of the transposed-gradient slab the backward materialises at a time: [V, SLAB] bf16
-BACKWARD_SLAB = 8192
+# rows of the transposed-gradient slab the backward materialises at a time: [V, SLAB] bf16 (10 GB at V = 151936:
+# sized for 288 GB of HBM, so the usual micro-batch is one slab and dweight needs no cross-slab accumulation)
+BACKWARD_SLAB = 32768
 
 
 def _bf16_rows(t: torch.Tensor, what: str) -> torch.Tensor:
