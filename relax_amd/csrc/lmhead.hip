@@ -135,30 +135,42 @@ __device__ __forceinline__ void lm_mma_group(const LmFrags& f, floatx16 (&acc)[4
     }
 }
 
+// The 16 copies of the following slice are spread over the slice's MFMAs, one copy per kLmCopyEvery MFMAs: four
+// waves issuing one 1 KB copy per MFMA ask for twice what the vector-memory path accepts and stall at issue.
+constexpr int kLmCopyEvery = 2;
+template <typename Copy>
+__device__ __forceinline__ void lm_copy_slot(int m, Copy&& copy) {  // m = index of the MFMA just issued, 0..63
+  if (m % kLmCopyEvery == kLmCopyEvery - 1 && m / kLmCopyEvery < 16) copy(m / kLmCopyEvery);
+}
+
 // k-steps 0..2 of the slice in `st`; on entry f0 holds (or is receiving) the fragments of k-step 0, on exit f1 those
 // of k-step 3, whose MFMAs are left to the caller: they run after the next barrier and cover the LDS latency of the
 // next slice's first fragments.
+template <typename Copy>
 __device__ __forceinline__ void lm_slice_body(const LmStage& st, int lane, LmFrags& f0, LmFrags& f1,
-                                              floatx16 (&acc)[4][4]) {
+                                              floatx16 (&acc)[4][4], Copy&& copy) {
   lm_mma_group(f0, acc, [&](int n) {
     if (n < 8) lm_load_frag(st, lane, 1, n, f1);
+    lm_copy_slot(16 + n, copy);
   });
   lm_mma_group(f1, acc, [&](int n) {
     if (n < 8) lm_load_frag(st, lane, 2, n, f0);
+    lm_copy_slot(32 + n, copy);
   });
   lm_mma_group(f0, acc, [&](int n) {
     if (n < 8) lm_load_frag(st, lane, 3, n, f1);
+    lm_copy_slot(48 + n, copy);
   });
 }
 
 // The previous slice's last k-step (fragments in f1) while the fragments of k-step 0 of the slice in `st` load into
-// f0 and `copy(n)`, n = 0..15, issues the 16 global -> LDS copies of the slice after it.
+// f0; `copy(n)`, n = 0..15, issues the n-th global -> LDS copy of the slice after it.
 template <typename Copy>
 __device__ __forceinline__ void lm_slice_head(const LmStage& st, int lane, LmFrags& f0, const LmFrags& f1,
                                               floatx16 (&acc)[4][4], Copy&& copy) {
   lm_mma_group(f1, acc, [&](int n) {
     if (n < 8) lm_load_frag(st, lane, 0, n, f0);
-    copy(n);
+    lm_copy_slot(n, copy);
   });
 }
 
@@ -221,36 +233,42 @@ __device__ __forceinline__ void lm_pipeline(const LmLds lds, const uint16_t* hid
     wc.issue(lds.w1, 1);
     hc.issue(lds.h1, 1);
     __builtin_amdgcn_sched_barrier(0);
-    lm_slice_body(st0, lane, f0, f1, acc);
+    lm_slice_body(st0, lane, f0, f1, acc, [](int) {});
     lm_slice_sync();
     for (int s = 1; s + 1 < nk; s += 2) {  // odd slices live in stage 1, even slices in stage 0
-      lm_slice_head(st1, lane, f0, f1, acc, [&](int n) {
-        if (n < 8)
+      auto copy_to_0 = [&](int n) {
+        if (n < 8) {
           wc.issue_pass(lds.w0, s + 1, n);
-        else
+        } else {
           hc.issue_pass(lds.h0, s + 1, n - 8);
-      });
-      lm_slice_body(st1, lane, f0, f1, acc);
-      lm_slice_sync();
-      lm_slice_head(st0, lane, f0, f1, acc, [&](int n) {
-        if (n < 8)
+        }
+      };
+      auto copy_to_1 = [&](int n) {
+        if (n < 8) {
           wc.issue_pass(lds.w1, s + 2, n);
-        else
+        } else {
           hc.issue_pass(lds.h1, s + 2, n - 8);
-      });
-      lm_slice_body(st0, lane, f0, f1, acc);
+        }
+      };
+      lm_slice_head(st1, lane, f0, f1, acc, copy_to_0);
+      lm_slice_body(st1, lane, f0, f1, acc, copy_to_0);
+      lm_slice_sync();
+      lm_slice_head(st0, lane, f0, f1, acc, copy_to_1);
+      lm_slice_body(st0, lane, f0, f1, acc, copy_to_1);
       lm_slice_sync();
     }
     // Last slice of the tile (stage 1).  The copies issued under it fetch the next tile's first slice; after the last
     // tile they re-fetch this tile's first slice, which nobody reads (cheaper than a branch between the MFMAs).
     if (vt + 1 < vt_end) wc.init(weight, g.w_stride, int64_t(vt + 1) * kLmTile, g.vocab - 1);
-    lm_slice_head(st1, lane, f0, f1, acc, [&](int n) {
-      if (n < 8)
+    auto copy_next_tile = [&](int n) {
+      if (n < 8) {
         wc.issue_pass(lds.w0, 0, n);
-      else
+      } else {
         hc.issue_pass(lds.h0, 0, n - 8);
-    });
-    lm_slice_body(st1, lane, f0, f1, acc);
+      }
+    };
+    lm_slice_head(st1, lane, f0, f1, acc, copy_next_tile);
+    lm_slice_body(st1, lane, f0, f1, acc, copy_next_tile);
     lm_mma_group(f1, acc, [](int) {});
     epilogue(acc, int64_t(vt) * kLmTile);
     lm_zero_acc(acc);
