@@ -267,21 +267,27 @@ def run_reverse_kl(a, dev) -> None:
 
     def step():
         student.grad = None
-        kl = opd_utils.compute_opd_kl_full_vocab(student, teacher)
-        loss = opd_utils.reduce_opd_loss(batch, kl)
+        if a.two_launch:
+            kl = opd_utils.compute_opd_kl_full_vocab(student, teacher)
+            loss = opd_utils.reduce_opd_loss(batch, kl)
+        else:
+            loss, _ = opd_utils.opd_loss_full_vocab(batch, student, teacher)
         loss.backward()
         return loss
 
     wall, kernel_ms, _, loss = timed_steps(step, a.warmup, a.steps)
     row_bytes = float(v * 2) * n
-    dom = kernel_ms["reverse_kl_bwd"]
-    dom_bytes = 3.0 * row_bytes  # read student + teacher rows, write the student gradient row
+    if "reverse_kl_step_fused" in kernel_ms:
+        # forward scan of both rows, re-read of both (served by cache), write of the student gradient
+        dom, dom_name, dom_bytes = kernel_ms["reverse_kl_step_fused"], "reverse_kl_step_kernel<bf16_t, true, 1024>", 5.0 * row_bytes
+    else:
+        dom, dom_name, dom_bytes = kernel_ms["reverse_kl_bwd"], "reverse_kl_bwd_kernel<bf16_t, true>", 3.0 * row_bytes
     achieved = dom_bytes / (dom * 1e-3) / 1e9
     emit(a, n, wall,
          f"on-policy distillation: student/teacher bf16 logits [{n}, {v}], full-vocab reverse KL, token-mean, fwd + "
          f"student dlogits bwd",
          {"rows": n, "vocab": v, "loss": float(loss.item())},
-         {"bound": "hbm", "kernel": "reverse_kl_bwd_kernel<bf16_t>", "achieved": achieved, "peak": HBM_PEAK_GBS,
+         {"bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS,
           "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": dom_bytes,
           "avg_launch_ms": dom, "kernel_ms": kernel_ms,
           "step_algorithmic_GBs": 5.0 * row_bytes / (wall / a.steps) / 1e9},

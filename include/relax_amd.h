@@ -212,6 +212,17 @@ int relax_amd_reverse_kl_bwd(const void* student, const void* teacher, int dtype
                              void* stream);
 
 /*
+ * Forward and backward of the reverse KL in one launch, for a reduction whose gradient w.r.t. each token's KL is
+ * known before the forward runs: the masked token mean of reduce_opd_loss (relax/utils/opd/opd_utils.py:1355-1365),
+ * g[t] = mask[t] / clamp_min(sum mask, 1).  Same outputs as relax_amd_reverse_kl_fwd followed by
+ * relax_amd_reverse_kl_bwd (dstudent row stride = row_stride); each workgroup re-reads its two rows out of cache, so
+ * HBM moves 3*V*s bytes per token instead of 5*V*s.
+ */
+int relax_amd_reverse_kl_step_fused(const void* student, const void* teacher, int dtype, int64_t n_tokens,
+                                    int64_t vocab, int64_t row_stride, const float* g, float grad_scale, float* kl,
+                                    float* lse_s, float* lse_t, void* dstudent, void* stream);
+
+/*
  * Fused actor step: log-prob + entropy forward, the per-token terms of relax_amd_policy_loss and the dlogits backward
  * in one launch.  Each workgroup scans its row, derives the token's gradient constants and immediately walks the row
  * again to emit dlogits; the second walk is served by the L2 / memory-side cache, so HBM sees one read and one write

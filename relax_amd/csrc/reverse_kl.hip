@@ -211,6 +211,156 @@ __global__ __launch_bounds__(kKlThreads) void reverse_kl_bwd_kernel(
   }
 }
 
+// Forward + backward in ONE launch for a loss whose gradient w.r.t. each token's KL is known up front (masked token
+// mean: g = mask / max(sum mask, 1)).  The workgroup scans the student and teacher rows with ordinary (cached) loads,
+// thread 0 finishes KL / lse_s / lse_t, and the workgroup walks both rows again at once -- served by L2 / the
+// memory-side cache -- to stream the student gradient out.  HBM sees 3*V*s bytes per token instead of 5*V*s.
+// Tokens with g == 0 still report their KL but get a zero gradient row without a second walk.
+template <typename T, bool VEC, int THREADS>
+__global__ __launch_bounds__(THREADS) void reverse_kl_step_kernel(
+    const T* __restrict__ student, const T* __restrict__ teacher, int64_t stride, int64_t vocab,
+    const float* __restrict__ g, float grad_scale, float* __restrict__ kl, float* __restrict__ lse_s,
+    float* __restrict__ lse_t, T* __restrict__ dstudent) {
+  __shared__ float lds[THREADS / kWave][5];
+  __shared__ float bc[2];
+  const int tid = threadIdx.x;
+  const int64_t tok = blockIdx.x;
+  const T* xs = student + tok * stride;
+  const T* xt = teacher + tok * stride;
+  T* d = dstudent + tok * stride;
+  const float gt = g[tok] * grad_scale;
+  KlState q{kNegHuge, 0.f, 0.f, kNegHuge, 0.f};
+  constexpr int VN = Row<T>::kPerVec;
+  const int64_t nvec = VEC ? vocab / VN : 0;
+  if (VEC) {
+    const u32x4* sv = reinterpret_cast<const u32x4*>(xs);
+    const u32x4* tv = reinterpret_cast<const u32x4*>(xt);
+    int64_t i = tid;
+    for (; i + int64_t(kKlUnroll - 1) * THREADS < nvec; i += int64_t(kKlUnroll) * THREADS) {
+      u32x4 rs[kKlUnroll], rt[kKlUnroll];
+#pragma unroll
+      for (int u = 0; u < kKlUnroll; ++u) {
+        rs[u] = sv[i + int64_t(u) * THREADS];
+        rt[u] = tv[i + int64_t(u) * THREADS];
+      }
+      float a[kKlUnroll * VN], b[kKlUnroll * VN];
+#pragma unroll
+      for (int u = 0; u < kKlUnroll; ++u) {
+        float pa[VN], pb[VN];
+        Row<T>::unpack(rs[u], pa);
+        Row<T>::unpack(rt[u], pb);
+#pragma unroll
+        for (int k = 0; k < VN; ++k) {
+          a[u * VN + k] = pa[k];
+          b[u * VN + k] = pb[k];
+        }
+      }
+      absorb_pair(a, b, q);
+    }
+    for (; i < nvec; i += THREADS) {
+      float a[VN], b[VN];
+      Row<T>::unpack(sv[i], a);
+      Row<T>::unpack(tv[i], b);
+      absorb_pair(a, b, q);
+    }
+  }
+  for (int64_t e = nvec * VN + tid; e < vocab; e += THREADS) {
+    float a[1] = {Row<T>::load1(xs + e)}, b[1] = {Row<T>::load1(xt + e)};
+    absorb_pair(a, b, q);
+  }
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    KlState other{__shfl_xor(q.ms, o, kWave), __shfl_xor(q.ss, o, kWave), __shfl_xor(q.us, o, kWave),
+                  __shfl_xor(q.mt, o, kWave), __shfl_xor(q.st, o, kWave)};
+    merge_kl(q, other);
+  }
+  const int lane = tid & (kWave - 1), w = tid / kWave;
+  if (lane == 0) {
+    lds[w][0] = q.ms;
+    lds[w][1] = q.ss;
+    lds[w][2] = q.us;
+    lds[w][3] = q.mt;
+    lds[w][4] = q.st;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int k = 1; k < THREADS / kWave; ++k) {
+      KlState other{lds[k][0], lds[k][1], lds[k][2], lds[k][3], lds[k][4]};
+      merge_kl(q, other);
+    }
+    const float ls = q.ms * kLn2 + logf(q.ss);
+    const float lt = q.mt * kLn2 + logf(q.st);
+    const float v = q.us / q.ss - ls + lt;
+    kl[tok] = v;
+    lse_s[tok] = ls;
+    lse_t[tok] = lt;
+    bc[0] = -ls * kLog2e;
+    bc[1] = gt * (lt - ls - v);
+  }
+  __syncthreads();
+  const float k0 = bc[0], k1 = bc[1];
+  // d = p_s * g * ((x_s - x_t) + lse_t - lse_s - KL); last use of both rows: non-temporal loads
+  if (VEC) {
+    const u32x4* sv = reinterpret_cast<const u32x4*>(xs);
+    const u32x4* tv = reinterpret_cast<const u32x4*>(xt);
+    u32x4* dv = reinterpret_cast<u32x4*>(d);
+    if (gt == 0.f) {
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      for (int64_t i = tid; i < nvec; i += THREADS) store_stream(dv + i, z);
+    } else {
+      int64_t i = tid;
+      for (; i + int64_t(kKlUnroll - 1) * THREADS < nvec; i += int64_t(kKlUnroll) * THREADS) {
+        u32x4 rs[kKlUnroll], rt[kKlUnroll];
+#pragma unroll
+        for (int u = 0; u < kKlUnroll; ++u) {
+          rs[u] = load_stream(sv + i + int64_t(u) * THREADS);
+          rt[u] = load_stream(tv + i + int64_t(u) * THREADS);
+        }
+#pragma unroll
+        for (int u = 0; u < kKlUnroll; ++u) {
+          float a[VN], b[VN];
+          Row<T>::unpack(rs[u], a);
+          Row<T>::unpack(rt[u], b);
+#pragma unroll
+          for (int k = 0; k < VN; ++k) a[k] = fast_exp2(fmaf(a[k], kLog2e, k0)) * fmaf(a[k] - b[k], gt, k1);
+          store_stream(dv + i + int64_t(u) * THREADS, Row<T>::pack(a));
+        }
+      }
+      for (; i < nvec; i += THREADS) {
+        float a[VN], b[VN];
+        Row<T>::unpack(load_stream(sv + i), a);
+        Row<T>::unpack(load_stream(tv + i), b);
+#pragma unroll
+        for (int k = 0; k < VN; ++k) a[k] = fast_exp2(fmaf(a[k], kLog2e, k0)) * fmaf(a[k] - b[k], gt, k1);
+        store_stream(dv + i, Row<T>::pack(a));
+      }
+    }
+  }
+  for (int64_t e = nvec * VN + tid; e < vocab; e += THREADS) {
+    const float a = Row<T>::load1(xs + e), b = Row<T>::load1(xt + e);
+    Row<T>::store1(d + e, gt == 0.f ? 0.f : fast_exp2(fmaf(a, kLog2e, k0)) * fmaf(a - b, gt, k1));
+  }
+}
+
+template <typename T>
+static int launch_kl_step(const void* s, const void* t, int64_t n, int64_t vocab, int64_t stride, const float* g,
+                          float scale, float* kl, float* ls, float* lt, void* d, hipStream_t st) {
+  const bool vec = aligned16(s) && aligned16(t) && aligned16(d) && (stride * int64_t(sizeof(T))) % 16 == 0;
+  dim3 grid(static_cast<unsigned>(n));
+#define RELAX_AMD_KL_STEP(V, TH)                                                                                   \
+  hipLaunchKernelGGL((reverse_kl_step_kernel<T, V, TH>), grid, dim3(TH), 0, st, static_cast<const T*>(s),            \
+                     static_cast<const T*>(t), stride, vocab, g, scale, kl, ls, lt, static_cast<T*>(d))
+  if (!vec) {
+    RELAX_AMD_KL_STEP(false, 256);
+  } else if (vocab / Row<T>::kPerVec >= 2048) {  // enough 16-byte vectors to keep 1024 threads busy
+    RELAX_AMD_KL_STEP(true, 1024);
+  } else {
+    RELAX_AMD_KL_STEP(true, 256);
+  }
+#undef RELAX_AMD_KL_STEP
+  return check_launch("reverse_kl_step_fused");
+}
+
 template <typename T>
 static int launch_kl_fwd(const void* s, const void* t, int64_t n, int64_t vocab, int64_t stride, float* kl,
                          float* ls, float* lt, hipStream_t st) {
@@ -290,5 +440,26 @@ extern "C" int relax_amd_reverse_kl_bwd(const void* student, const void* teacher
     case RELAX_AMD_F16:
       return launch_kl_bwd<f16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, g, grad_scale, grad_scale_dev, dstudent, s);
     default: set_error("reverse_kl_bwd: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
+  }
+}
+
+extern "C" int relax_amd_reverse_kl_step_fused(const void* student, const void* teacher, int dtype, int64_t n_tokens,
+                                               int64_t vocab, int64_t row_stride, const float* g, float grad_scale,
+                                               float* kl, float* lse_s, float* lse_t, void* dstudent, void* stream) {
+  if (int rc = kl_check("reverse_kl_step_fused", n_tokens, vocab, row_stride)) return rc;
+  if (n_tokens == 0) return RELAX_AMD_OK;
+  if (!student || !teacher || !g || !kl || !lse_s || !lse_t || !dstudent) {
+    set_error("reverse_kl_step_fused: NULL argument");
+    return RELAX_AMD_EINVAL;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case RELAX_AMD_F32:
+      return launch_kl_step<float>(student, teacher, n_tokens, vocab, row_stride, g, grad_scale, kl, lse_s, lse_t, dstudent, s);
+    case RELAX_AMD_BF16:
+      return launch_kl_step<bf16_t>(student, teacher, n_tokens, vocab, row_stride, g, grad_scale, kl, lse_s, lse_t, dstudent, s);
+    case RELAX_AMD_F16:
+      return launch_kl_step<f16_t>(student, teacher, n_tokens, vocab, row_stride, g, grad_scale, kl, lse_s, lse_t, dstudent, s);
+    default: set_error("reverse_kl_step_fused: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
   }
 }

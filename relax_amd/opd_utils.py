@@ -51,3 +51,43 @@ def reduce_opd_loss(batch: dict, values: torch.Tensor) -> torch.Tensor:
     dev = values.device
     mask = torch.cat([m.reshape(-1) for m in batch["loss_masks"]]).to(device=dev, dtype=torch.float32)
     return _TokenMean.apply(values.to(torch.float32), mask, _cu(batch["response_lengths"], dev))
+
+
+class _FusedOpdLoss(torch.autograd.Function):
+    """student logits [N, V] -> (masked token-mean reverse KL, per-token KL), one launch: the gradient of the token
+    mean w.r.t. each token's KL (mask / clamp_min(sum mask, 1)) is known before the forward, so the kernel writes the
+    student gradient for an upstream gradient of 1 while the rows are still in cache; the backward multiplies by the
+    actual upstream gradient on the device (a no-op kernel when it is exactly 1)."""
+
+    @staticmethod
+    def forward(ctx, student, teacher, mask):
+        den = torch.clamp_min(mask.sum(), 1)
+        g = mask / den
+        kl, _ls, _lt, d = ops.reverse_kl_step_fused(student, teacher, g)
+        ctx.d = d
+        ctx.shape = student.shape
+        ctx.mark_non_differentiable(kl)
+        return (kl * mask).sum() / den, kl
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_kl):
+        d = ctx.d
+        if d is None:
+            raise RuntimeError("the fused OPD loss holds its gradient once: backward cannot run twice")
+        ctx.d = None
+        ops.scale_rows_inplace(d, g_loss.reshape(1).to(torch.float32).contiguous())
+        return d.view(ctx.shape), None, None
+
+
+def opd_loss_full_vocab(batch: dict, student_logits: torch.Tensor, teacher_logits: torch.Tensor):
+    """``reduce_opd_loss(batch, compute_opd_kl_full_vocab(student, teacher))`` in a single kernel launch
+    (opd_utils.py:1165-1169 + :1355-1365).  Returns ``(loss, per_token_kl)``; differentiable w.r.t. the student."""
+    dev = student_logits.device
+    mask = torch.cat([m.reshape(-1) for m in batch["loss_masks"]]).to(device=dev, dtype=torch.float32)
+    rows = student_logits.reshape(-1, student_logits.size(-1))
+    if mask.numel() != rows.size(0):
+        raise ValueError(f"loss masks cover {mask.numel()} tokens, logits have {rows.size(0)} rows")
+    if not (torch.is_grad_enabled() and student_logits.requires_grad):
+        kl = compute_opd_kl_full_vocab(student_logits, teacher_logits)
+        return reduce_opd_loss(batch, kl), kl
+    return _FusedOpdLoss.apply(student_logits, teacher_logits.detach(), mask)

@@ -363,6 +363,27 @@ def reverse_kl_bwd(s, t, kl, ls, lt, g, grad_scale: float = 1.0, grad_scale_dev=
     return d
 
 
+def reverse_kl_step_fused(student, teacher, g, grad_scale: float = 1.0):
+    """One launch: (kl, lse_s, lse_t, dstudent) with ``dstudent = g[t] * grad_scale * d kl[t] / d student``."""
+    _need_gpu(student, teacher, g)
+    s, t = _rows(student), _rows(teacher)
+    if s.shape != t.shape or s.dtype != t.dtype:
+        raise ValueError(f"student {tuple(s.shape)}/{s.dtype} and teacher {tuple(t.shape)}/{t.dtype} must match")
+    if s.size(0) > 1 and (s.stride(0) != s.size(1) or t.stride(0) != t.size(1)):
+        s, t = s.contiguous(), t.contiguous()
+    n = s.size(0)
+    g = _f32(g)
+    if g.numel() != n:
+        raise ValueError(f"g has {g.numel()} entries for {n} token rows")
+    kw = dict(dtype=torch.float32, device=s.device)
+    kl, ls, lt = torch.empty(n, **kw), torch.empty(n, **kw), torch.empty(n, **kw)
+    d = torch.empty_like(s)
+    with _timed("reverse_kl_step_fused"):
+        check(lib.relax_amd_reverse_kl_step_fused(_p(s), _p(t), _code(s), n, s.size(1), s.size(1), _p(g),
+                                                  float(grad_scale), _p(kl), _p(ls), _p(lt), _p(d), _stream()))
+    return kl, ls, lt, d
+
+
 class ReverseKL(torch.autograd.Function):
     """(student logits [R,V], teacher logits [R,V]) -> per-token KL(student || teacher) [R]; teacher gets no grad."""
 

@@ -179,6 +179,55 @@ def test_full_vocab_reverse_kl_vs_oracle(n, v, dtype, tol):
     assert same.abs().max().item() < 1e-5
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,v,dtype,tol", [
+    (33, 1000, torch.float32, 3e-5),        # scalar tail, 256-thread variant
+    (64, 151936, torch.bfloat16, 2e-3),     # the production vocabulary, 1024-thread variant
+    (17, 32003, torch.float16, 2e-3),       # rows that are not 16-byte aligned
+])
+def test_fused_opd_loss_matches_oracle_and_two_launch_path(n, v, dtype, tol):
+    """One-launch forward + backward of the masked token-mean reverse KL: same loss, per-token KL and student
+    gradient as the oracle and as the separate forward / backward launches; an upstream gradient other than 1 is
+    applied to the stored gradient."""
+    from relax_amd.opd_utils import compute_opd_kl_full_vocab, opd_loss_full_vocab, reduce_opd_loss
+
+    dev = require_gpu()
+    announce("fused OPD loss", n, v, dtype)
+    g = torch.Generator().manual_seed(n + v)
+    s = (torch.randn(n, v, generator=g) * 3).to(dtype)
+    t = (s.float() + torch.randn(n, v, generator=g)).to(dtype)
+    lens = [n // 3, n - n // 3]
+    masks = [(torch.rand(k, generator=g) > 0.3).float() for k in lens]
+    sc = s.clone().requires_grad_()
+    want = D.full_vocab_reverse_kl(sc, t)
+    want_loss = D.reduce_token_mean(want, lens, masks)
+    (2.5 * want_loss).backward()
+    batch = {"response_lengths": lens, "loss_masks": [m.to(dev) for m in masks]}
+    sd = s.to(dev).requires_grad_()
+    loss, kl = opd_loss_full_vocab(batch, sd, t.to(dev))
+    (2.5 * loss).backward()
+    torch.testing.assert_close(kl.cpu(), want.detach(), atol=tol, rtol=0)
+    assert abs(loss.item() - want_loss.item()) < tol
+    assert sd.grad.dtype == dtype and sd.grad.shape == s.shape
+    ulp = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 1e-5}[dtype]
+    torch.testing.assert_close(sd.grad.float().cpu(), sc.grad.float(), atol=tol, rtol=ulp)
+    # masked tokens: zero gradient rows, KL still reported
+    dead = torch.cat(masks) == 0
+    assert dead.any() and (sd.grad[dead.to(dev)] == 0).all()
+    # against the two-launch path on the same device
+    s2 = s.to(dev).requires_grad_()
+    kl2 = compute_opd_kl_full_vocab(s2, t.to(dev))
+    loss2 = reduce_opd_loss(batch, kl2)
+    (2.5 * loss2).backward()
+    torch.testing.assert_close(kl, kl2.detach(), atol=2e-6 if dtype == torch.float32 else 1e-5, rtol=1e-6)
+    torch.testing.assert_close(sd.grad.float(), s2.grad.float(), atol=tol * 1e-2, rtol=2 * ulp)
+    # no-grad call falls back to the forward-only kernel
+    with torch.no_grad():
+        loss3, kl3 = opd_loss_full_vocab(batch, s.to(dev), t.to(dev))
+    assert abs(loss3.item() - loss2.item()) < 1e-6
+    assert torch.equal(kl3, kl2.detach())
+
+
 def test_opd_token_mean_literal(literals):
     from relax_amd.opd_utils import compute_opd_kl, reduce_opd_loss
 
