@@ -39,6 +39,10 @@ enum { RELAX_AMD_LOSS_PPO = 0, RELAX_AMD_LOSS_GSPO = 1, RELAX_AMD_LOSS_CISPO = 2
 enum { RELAX_AMD_KL_NONE = 0, RELAX_AMD_KL_K1 = 1, RELAX_AMD_KL_K2 = 2, RELAX_AMD_KL_K3 = 3, RELAX_AMD_KL_LOW_VAR = 4 };
 /* group reward normalisation (relax/utils/utils.py:199-238) */
 enum { RELAX_AMD_GROUP_CENTER = 0, RELAX_AMD_GROUP_CENTER_STD = 1, RELAX_AMD_GROUP_RLOO = 2 };
+/* top-K distillation signal: the JSD family (jsd_alpha 0 = reverse KL, 1 = forward KL) or the element-wise k3 sum */
+enum { RELAX_AMD_OPD_JSD = 0, RELAX_AMD_OPD_LOW_VAR = 1 };
+/* opd_norm_mode: append the tail bin log(1 - sum p), renormalise over the K entries, or use them as they are */
+enum { RELAX_AMD_OPD_NORM_TAIL = 0, RELAX_AMD_OPD_NORM_NORM = 1, RELAX_AMD_OPD_NORM_TRUNC = 2 };
 
 /* slots of the metrics vector written by relax_amd_policy_loss */
 enum {
@@ -221,6 +225,43 @@ int relax_amd_reverse_kl_bwd(const void* student, const void* teacher, int dtype
 int relax_amd_reverse_kl_step_fused(const void* student, const void* teacher, int dtype, int64_t n_tokens,
                                     int64_t vocab, int64_t row_stride, const float* g, float grad_scale, float* kl,
                                     float* lse_s, float* lse_t, void* dstudent, void* stream);
+
+/*
+ * Log-probs of K given vocabulary ids per token: compute_log_probs_on_topk_token_ids
+ * (relax/utils/opd/opd_utils.py:1022-1094) on one rank.
+ *   topk_ids      int64 [n_tokens, k]; ids < 0 are sentinels (-inf out, no gradient), ids >= vocab read as a zero
+ *                 logit (the reference's fill for ids outside the rank's vocabulary slice)
+ *   row_ids       int32 [n_tokens] logits row of each token, or NULL (row t = token t)
+ *   lse_in        fp32 [n_tokens] log-sum-exp of each token's row (as written by relax_amd_logprob_entropy_fwd), or
+ *                 NULL: the kernel scans the row itself and writes lse_out (if not NULL)
+ *   topk_log_prob fp32 [n_tokens, k] out = logits[row, id] * inv_temperature - lse
+ * bwd: dlogits[row, v] = inv_temperature * ( sum_k g[t,k] * [v == id_k] - p[v] * sum_{k: id_k >= 0} g[t,k] ),
+ *   every row written once (rows with token_of_row < 0 or an all-zero g are zero-filled without a read).
+ */
+int relax_amd_topk_logprob_fwd(const void* logits, int dtype, int64_t n_tokens, int64_t vocab, int64_t row_stride,
+                               const int32_t* row_ids, const int64_t* topk_ids, int64_t k, float inv_temperature,
+                               const float* lse_in, float* topk_log_prob, float* lse_out, void* stream);
+int relax_amd_topk_logprob_bwd(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                               const int32_t* token_of_row, const int64_t* topk_ids, int64_t k, float inv_temperature,
+                               const float* lse, const float* g, void* dlogits, int64_t d_stride, void* stream);
+
+/*
+ * Per-token distillation signal on [n_rows, k] top-K log-probs: compute_opd_kl_topk / compute_opd_kl
+ * (relax/utils/opd/opd_utils.py:1097-1228).
+ *   mask          uint8 [n_rows, k] (non-zero = valid) for the union path's padded rows, or NULL.  With a mask the
+ *                 padded entries are excluded and, as in the reference, the tail bin is cut off as well.
+ *   kl_mode       RELAX_AMD_OPD_JSD (jsd_alpha in [0, 1]) or RELAX_AMD_OPD_LOW_VAR
+ *   norm_mode     RELAX_AMD_OPD_NORM_* (JSD family only)
+ *   has_clamp / log_prob_min_clamp   clamp both inputs from below first (opd_log_prob_min_clamp)
+ *   k             1..2048
+ * bwd: d_student_lp[r, j] = g[r] * d kl[r] / d student_lp[r, j]  (the teacher is detached)
+ */
+int relax_amd_opd_kl_topk_fwd(const float* student_lp, const float* teacher_lp, const uint8_t* mask, int64_t n_rows,
+                              int64_t k, int kl_mode, int norm_mode, float jsd_alpha, int has_clamp,
+                              float log_prob_min_clamp, float* kl, void* stream);
+int relax_amd_opd_kl_topk_bwd(const float* student_lp, const float* teacher_lp, const uint8_t* mask, int64_t n_rows,
+                              int64_t k, int kl_mode, int norm_mode, float jsd_alpha, int has_clamp,
+                              float log_prob_min_clamp, const float* g, float* d_student_lp, void* stream);
 
 /*
  * Fused actor step: log-prob + entropy forward, the per-token terms of relax_amd_policy_loss and the dlogits backward

@@ -16,16 +16,22 @@ def _with_tail(lp):
     return torch.cat([lp, torch.log(-torch.expm1(ls))], dim=-1)
 
 
-def opd_kl(s_lp, t_lp, kl_type="reverse_kl", jsd_alpha=0.5, norm_mode="tail", min_clamp=None):
-    """opd_utils.py:1097-1187 without the union-path padding mask."""
+def opd_kl(s_lp, t_lp, kl_type="reverse_kl", jsd_alpha=0.5, norm_mode="tail", min_clamp=None, mask=None):
+    """opd_utils.py:1097-1187.  ``mask`` (bool [R, K], True = valid) is the union path's padding mask (:1121-1127):
+    padded entries are set to -inf after the clamp, and the summed terms are cut back to the first K columns and
+    zeroed at the padding -- which also drops the tail bin (:1158-1186)."""
     s, t = s_lp.float(), t_lp.float()
     if min_clamp is not None:
         s, t = s.clamp_min(min_clamp), t.clamp_min(min_clamp)
+    if mask is not None:
+        s, t = s.masked_fill(~mask, float("-inf")), t.masked_fill(~mask, float("-inf"))
     d = s - t
     if kl_type == "reverse_kl":
         return d
     if kl_type == "low_var_kl":
         per = torch.exp(-d) - 1.0 + d
+        if mask is not None:
+            per = per.masked_fill(~mask, 0.0)
         return per.sum(dim=-1) if per.dim() > 1 else per
     if kl_type != "jsd":
         raise ValueError(f"Unknown opd_kl_type: {kl_type}.")
@@ -36,23 +42,43 @@ def opd_kl(s_lp, t_lp, kl_type="reverse_kl", jsd_alpha=0.5, norm_mode="tail", mi
     elif norm_mode == "norm":
         s = s - torch.logsumexp(s, dim=-1, keepdim=True)
         t = t - torch.logsumexp(t, dim=-1, keepdim=True)
+
+    def total(terms):
+        if mask is not None:
+            terms = terms[..., : mask.size(-1)].masked_fill(~mask, 0.0)
+        return terms.sum(dim=-1)
+
     if jsd_alpha == 0.0:
-        return (s.exp() * (s - t)).sum(dim=-1)
+        return total(s.exp() * (s - t))
     if jsd_alpha == 1.0:
-        return (t.exp() * (t - s)).sum(dim=-1)
+        return total(t.exp() * (t - s))
     l1 = torch.log(torch.tensor(1.0 - jsd_alpha, dtype=s.dtype))
     la = torch.log(torch.tensor(jsd_alpha, dtype=s.dtype))
     mix = torch.logsumexp(torch.stack([s + l1, t + la]), dim=0)
-    return (1.0 - jsd_alpha) * (s.exp() * (s - mix)).sum(-1) + jsd_alpha * (t.exp() * (t - mix)).sum(-1)
+    return (1.0 - jsd_alpha) * total(s.exp() * (s - mix)) + jsd_alpha * total(t.exp() * (t - mix))
 
 
-def opd_kl_topk(s_lp, t_lp, kl_type="reverse_kl", jsd_alpha=0.5, norm_mode="tail", min_clamp=None):
+def opd_kl_topk(s_lp, t_lp, kl_type="reverse_kl", jsd_alpha=0.5, norm_mode="tail", min_clamp=None, mask=None):
     """opd_utils.py:1190-1228: reverse/forward KL are the alpha = 0 / 1 ends of the JSD family."""
     if kl_type in ("reverse_kl", "forward_kl", "jsd"):
         alpha = {"reverse_kl": 0.0, "forward_kl": 1.0}.get(kl_type, float(jsd_alpha))
-        return opd_kl(s_lp, t_lp, "jsd", alpha, norm_mode, min_clamp)
-    per = opd_kl(s_lp, t_lp, kl_type, min_clamp=min_clamp)
+        return opd_kl(s_lp, t_lp, "jsd", alpha, norm_mode, min_clamp, mask)
+    per = opd_kl(s_lp, t_lp, kl_type, min_clamp=min_clamp, mask=mask)
     return per.sum(dim=-1) if per.dim() > 1 else per
+
+
+def log_probs_on_topk_ids(logits, ids):
+    """compute_log_probs_on_topk_token_ids (opd_utils.py:1022-1094) on one rank: ``logits[ids] - logsumexp(logits)``
+    per row; ids < 0 are sentinels and give -inf, ids >= V read as logit 0 (the reference's out-of-slice fill)."""
+    if logits.size(0) == 0:
+        return logits.new_zeros((0, ids.size(-1)))
+    x = logits
+    lse = torch.logsumexp(x.float(), dim=-1, keepdim=True).to(x.dtype)
+    ids = ids.to(torch.long)
+    safe = ids.clamp(min=0)
+    inside = safe < x.size(-1)
+    got = torch.gather(x, -1, safe.clamp(max=x.size(-1) - 1)).masked_fill(~inside, 0.0)
+    return (got - lse).masked_fill(ids < 0, float("-inf"))
 
 
 def full_vocab_reverse_kl(student_logits, teacher_logits, norm_mode="tail"):

@@ -24,6 +24,7 @@ F32, BF16, F16, F64 = 0, 1, 2, 3
 LOSS_KINDS = {"ppo": 0, "gspo": 1, "cispo": 2, "rloo": 3, "sapo": 4}
 KL_KINDS = {None: 0, "k1": 1, "k2": 2, "k3": 3, "low_var_kl": 4}
 GROUP_MODES = {"center": 0, "center_std": 1, "rloo": 2}
+OPD_JSD, OPD_LOW_VAR = 0, 1
 METRIC_SLOTS = [
     "loss", "pg_loss", "entropy_loss", "pg_clipfrac", "ppo_kl", "kl_loss", "train_rollout_logprob_abs_diff",
     "train_rollout_prob_abs_diff", "ois", "tis", "tis_clipfrac", "tis_abs", "mismatch_kl", "mismatch_k3_kl",
@@ -75,6 +76,14 @@ SIGNATURES = {
     "relax_amd_lmhead_dlogits_t": (
         C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _vp]),
     "relax_amd_reverse_kl_bwd": (C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp]),
+    "relax_amd_topk_logprob_fwd": (
+        C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _i64, _f32, _vp, _vp, _vp, _vp]),
+    "relax_amd_topk_logprob_bwd": (
+        C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _i64, _f32, _vp, _vp, _vp, _i64, _vp]),
+    "relax_amd_opd_kl_topk_fwd": (
+        C.c_int, [_vp, _vp, _vp, _i64, _i64, C.c_int, C.c_int, _f32, C.c_int, _f32, _vp, _vp]),
+    "relax_amd_opd_kl_topk_bwd": (
+        C.c_int, [_vp, _vp, _vp, _i64, _i64, C.c_int, C.c_int, _f32, C.c_int, _f32, _vp, _vp, _vp]),
     "relax_amd_reverse_kl_step_fused": (
         C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _vp, _f32, _vp, _vp, _vp, _vp, _vp]),
 }

@@ -9,8 +9,13 @@ from __future__ import annotations
 
 import torch
 
-from . import ops
+from . import _lib, ops
+from ._lib import check, lib
 from .cp_utils import _cu
+from .ops import _code, _f32, _need_gpu, _p, _rows, _stream
+
+OPD_KL_TYPES = ("reverse_kl", "forward_kl", "jsd", "low_var_kl")
+_NORM_MODES = {"tail": 0, "norm": 1, "trunc": 2}
 
 
 def compute_opd_kl_full_vocab(student_logits: torch.Tensor, teacher_logits: torch.Tensor) -> torch.Tensor:
@@ -19,17 +24,141 @@ def compute_opd_kl_full_vocab(student_logits: torch.Tensor, teacher_logits: torc
     return ops.ReverseKL.apply(student_logits, teacher_logits.detach())
 
 
-def compute_opd_kl(student_log_probs, teacher_log_probs, kl_type: str = "reverse_kl", **_):
-    """Sampled-token (1-D) signals of opd_utils.py:1133-1141, evaluated by the policy-loss kernel's KL estimators."""
+class TopKLogProbs(torch.autograd.Function):
+    """(logits [N, V], ids int64 [N, K]) -> log-probs [N, K] fp32 at the given vocabulary ids.  Saves the logits
+    reference, the ids and one float per row; the backward writes the dense [N, V] gradient in one streaming pass."""
+
+    @staticmethod
+    def forward(ctx, logits, ids, inv_temperature, lse):
+        x = _rows(logits)
+        n, k = ids.shape
+        out = torch.empty((n, k), dtype=torch.float32, device=x.device)
+        lse_out = lse if lse is not None else torch.empty(n, dtype=torch.float32, device=x.device)
+        stride = x.stride(0) if n > 1 else x.size(1)
+        with ops._timed("topk_logprob_fwd"):
+            check(lib.relax_amd_topk_logprob_fwd(_p(x), _code(x), n, x.size(1), stride, None, _p(ids), k,
+                                                 float(inv_temperature), _p(lse), _p(out),
+                                                 None if lse is not None else _p(lse_out), _stream()))
+        ctx.save_for_backward(x, ids, lse_out)
+        ctx.inv_temperature = float(inv_temperature)
+        ctx.shape = logits.shape
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        x, ids, lse = ctx.saved_tensors
+        n, k = ids.shape
+        d = torch.empty((n, x.size(1)), dtype=x.dtype, device=x.device)
+        stride = x.stride(0) if n > 1 else x.size(1)
+        g = _f32(g).reshape(n, k).contiguous()
+        with ops._timed("topk_logprob_bwd"):
+            check(lib.relax_amd_topk_logprob_bwd(_p(x), _code(x), n, x.size(1), stride, None, _p(ids), k,
+                                                 ctx.inv_temperature, _p(lse), _p(g), _p(d), d.size(1), _stream()))
+        return d.view(ctx.shape), None, None, None
+
+
+def compute_log_probs_on_topk_token_ids(logits: torch.Tensor, topk_token_ids: torch.Tensor, process_group=None,
+                                        temperature: float = 1.0, lse: torch.Tensor | None = None) -> torch.Tensor:
+    """``[S, K]`` log-probabilities of the given (global) vocabulary ids, opd_utils.py:1022-1094 on one rank: ids
+    ``< 0`` are sentinels and yield ``-inf``.  ``lse`` (fp32 ``[S]``, the row log-sum-exps a log-prob forward already
+    produced) turns the call into K loads per row; without it the kernel scans each row once.  Gradient flows to
+    ``logits`` through both the gather and the log-sum-exp."""
+    if process_group is not None and torch.distributed.is_initialized() and \
+            torch.distributed.get_world_size(process_group) > 1:
+        raise NotImplementedError("vocab-parallel top-K gather (tensor-parallel size > 1) is not supported")
+    if logits.dim() != 2 or topk_token_ids.dim() != 2 or topk_token_ids.size(0) != logits.size(0):
+        raise ValueError(f"expected logits [S, V] and ids [S, K], got {tuple(logits.shape)} and "
+                         f"{tuple(topk_token_ids.shape)}")
+    if logits.size(0) == 0:
+        return logits.new_zeros((0, topk_token_ids.size(-1)))
+    _need_gpu(logits)
+    ids = topk_token_ids.to(device=logits.device, dtype=torch.long).contiguous()
+    if ids.size(1) == 0:
+        return torch.zeros((logits.size(0), 0), dtype=torch.float32, device=logits.device)
+    if lse is not None:
+        lse = _f32(lse).reshape(-1)
+        if lse.numel() != logits.size(0):
+            raise ValueError(f"lse has {lse.numel()} entries for {logits.size(0)} rows")
+    return TopKLogProbs.apply(logits, ids, 1.0 / float(temperature), lse)
+
+
+class _OpdKlTopk(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, s, t, mask, mode, norm, alpha, clamp):
+        n, k = s.shape
+        kl = torch.empty(n, dtype=torch.float32, device=s.device)
+        has_clamp, cval = (0, 0.0) if clamp is None else (1, float(clamp))
+        check(lib.relax_amd_opd_kl_topk_fwd(_p(s), _p(t), _p(mask), n, k, mode, norm, alpha, has_clamp, cval, _p(kl),
+                                            _stream()))
+        ctx.save_for_backward(s, t, mask)
+        ctx.cfg = (mode, norm, alpha, has_clamp, cval)
+        return kl
+
+    @staticmethod
+    def backward(ctx, g):
+        s, t, mask = ctx.saved_tensors
+        mode, norm, alpha, has_clamp, cval = ctx.cfg
+        n, k = s.shape
+        d = torch.empty_like(s)
+        g = _f32(g).reshape(-1).contiguous()
+        check(lib.relax_amd_opd_kl_topk_bwd(_p(s), _p(t), _p(mask), n, k, mode, norm, alpha, has_clamp, cval, _p(g),
+                                            _p(d), _stream()))
+        return d, None, None, None, None, None, None
+
+
+def compute_opd_kl_topk(student_topk_lp: torch.Tensor, teacher_topk_lp: torch.Tensor, kl_type: str = "reverse_kl",
+                        jsd_alpha: float = 0.5, norm_mode: str = "tail", log_prob_min_clamp: float | None = None,
+                        mask: torch.Tensor | None = None) -> torch.Tensor:
+    """Per-token KL ``[R]`` (fp32) from ``[R, K]`` top-K log-probs, opd_utils.py:1190-1228: reverse / forward KL are
+    the ``jsd_alpha`` = 0 / 1 ends of the JSD family, ``low_var_kl`` is summed element-wise over K.  ``mask`` (bool
+    ``[R, K]``, True = valid) is the union path's padding mask.  Differentiable w.r.t. the student log-probs."""
+    if kl_type not in OPD_KL_TYPES:
+        raise ValueError(f"Unknown opd_kl_type: {kl_type}. Choose one of {OPD_KL_TYPES}.")
+    if kl_type == "low_var_kl":
+        mode, alpha = _lib.OPD_LOW_VAR, 0.0
+    else:
+        mode = _lib.OPD_JSD
+        alpha = {"reverse_kl": 0.0, "forward_kl": 1.0}.get(kl_type, float(jsd_alpha))
+        if not (0.0 <= alpha <= 1.0):
+            raise ValueError(f"jsd_alpha must be in [0, 1], got {jsd_alpha}")
+    if norm_mode not in _NORM_MODES:
+        raise ValueError(f"Unknown opd_norm_mode: {norm_mode}. Choose one of {tuple(_NORM_MODES)}.")
+    if student_topk_lp.dim() != 2 or student_topk_lp.shape != teacher_topk_lp.shape:
+        raise ValueError(f"expected matching [R, K] inputs, got {tuple(student_topk_lp.shape)} and "
+                         f"{tuple(teacher_topk_lp.shape)}")
+    _need_gpu(student_topk_lp)
+    dev = student_topk_lp.device
+    s = student_topk_lp.to(torch.float32).contiguous()
+    t = teacher_topk_lp.detach().to(device=dev, dtype=torch.float32).contiguous()
+    if mask is not None:
+        if mask.shape != s.shape:
+            raise ValueError(f"mask {tuple(mask.shape)} does not match the inputs {tuple(s.shape)}")
+        mask = mask.to(device=dev, dtype=torch.uint8).contiguous()
+    if s.size(0) == 0:
+        return s.sum(dim=-1)
+    return _OpdKlTopk.apply(s, t, mask, mode, _NORM_MODES[norm_mode], alpha, log_prob_min_clamp)
+
+
+def compute_opd_kl(student_log_probs, teacher_log_probs, kl_type: str = "reverse_kl", jsd_alpha: float = 0.5,
+                   norm_mode: str = "tail", log_prob_min_clamp: float | None = None, mask=None):
+    """Per-token OPD signal (opd_utils.py:1097-1187).  1-D sampled-token inputs: ``reverse_kl`` (k1) and
+    ``low_var_kl`` (k3), evaluated by the policy-loss kernel's KL estimators.  2-D ``[R, K]`` inputs: ``jsd`` and
+    ``low_var_kl`` through the top-K kernel."""
     from .ppo_utils import compute_approx_kl
 
-    if student_log_probs.dim() != 1:
-        raise NotImplementedError("[R, K] top-K inputs: use compute_opd_kl_full_vocab on logits for K = vocab")
+    if student_log_probs.dim() == 2:
+        if kl_type in ("jsd", "low_var_kl"):
+            return compute_opd_kl_topk(student_log_probs, teacher_log_probs, kl_type, jsd_alpha, norm_mode,
+                                       log_prob_min_clamp, mask)
+        raise NotImplementedError("element-wise [R, K] log-ratios are not a loss signal; use compute_opd_kl_topk")
+    s, t = student_log_probs, teacher_log_probs
+    if log_prob_min_clamp is not None:
+        s, t = s.clamp_min(log_prob_min_clamp), t.clamp_min(log_prob_min_clamp)
     if kl_type == "reverse_kl":
-        return compute_approx_kl(student_log_probs, teacher_log_probs, "k1")
+        return compute_approx_kl(s, t, "k1")
     if kl_type == "low_var_kl":
-        return compute_approx_kl(student_log_probs, teacher_log_probs, "k3")
-    raise ValueError(f"Unknown opd_kl_type: {kl_type}.")
+        return compute_approx_kl(s, t, "k3")
+    raise ValueError(f"Unknown opd_kl_type: {kl_type}. Choose one of {OPD_KL_TYPES}.")
 
 
 class _TokenMean(torch.autograd.Function):

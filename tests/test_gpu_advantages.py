@@ -240,3 +240,101 @@ def test_opd_token_mean_literal(literals):
     torch.testing.assert_close(compute_opd_kl(s, t, "reverse_kl"), s - t)
     d = s - t
     torch.testing.assert_close(compute_opd_kl(s, t, "low_var_kl"), torch.exp(-d) - 1 + d, atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("n,v,k,dtype,tol", [
+    (19, 1003, 7, torch.float32, 3e-5),
+    (8, 151936, 32, torch.bfloat16, 2e-3),
+    (5, 4104, 300, torch.float16, 2e-3),      # K larger than a workgroup pass, repeated ids
+])
+def test_topk_log_probs_vs_oracle(n, v, k, dtype, tol):
+    """compute_log_probs_on_topk_token_ids: values, sentinels, out-of-range ids, repeated ids and the dense gradient."""
+    from relax_amd.opd_utils import compute_log_probs_on_topk_token_ids
+    from relax_amd.ppo_utils import calculate_log_probs_and_entropy
+
+    dev = require_gpu()
+    announce("top-K log-probs", n, v, k, dtype)
+    g = torch.Generator().manual_seed(n * k)
+    x = (torch.randn(n, v, generator=g) * 3).to(dtype)
+    ids = torch.randint(0, v, (n, k), generator=g)
+    ids[0, 0] = -1                      # sentinel
+    ids[1, 1] = v + 5                   # outside the vocabulary
+    ids[2, 2] = ids[2, 3]               # repeated id: both gradients land on the same logit
+    up = torch.randn(n, k, generator=g)
+    up[3] = 0.0                         # a row without incoming gradient
+    xc = x.clone().float().requires_grad_()
+    want = D.log_probs_on_topk_ids(xc, ids)
+    (want.masked_fill(ids < 0, 0.0) * up).sum().backward()
+    xd = x.to(dev).requires_grad_()
+    got = compute_log_probs_on_topk_token_ids(xd, ids.to(dev), None)
+    assert got.dtype == torch.float32 and got.shape == (n, k)
+    assert torch.isinf(got[0, 0]) and got[0, 0] < 0
+    fin = ids >= 0
+    torch.testing.assert_close(got.cpu()[fin], want.detach()[fin], atol=tol, rtol=0)
+    (got.masked_fill((ids < 0).to(dev), 0.0) * up.to(dev)).sum().backward()
+    ulp = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 1e-5}[dtype]
+    torch.testing.assert_close(xd.grad.float().cpu(), xc.grad, atol=tol, rtol=2 * ulp)
+    assert (xd.grad[3] == 0).all()
+    # reusing the log-sum-exp of a log-prob forward gives the same values without a row scan
+    from relax_amd import ops
+    _, _, lse, _ = ops.logprob_entropy_fwd(x.to(dev), torch.zeros(n, dtype=torch.long, device=dev), with_entropy=False)
+    again = compute_log_probs_on_topk_token_ids(x.to(dev), ids.to(dev), None, lse=lse)
+    torch.testing.assert_close(again[fin.to(dev)], got.detach()[fin.to(dev)], atol=2e-6, rtol=0)
+    assert compute_log_probs_on_topk_token_ids(x[:0].to(dev), ids[:0].to(dev), None).shape == (0, k)
+
+
+@pytest.mark.parametrize("kl_type,alpha", [("reverse_kl", 0.5), ("forward_kl", 0.5), ("jsd", 0.3), ("jsd", 0.0),
+                                           ("jsd", 1.0), ("low_var_kl", 0.5)])
+@pytest.mark.parametrize("norm_mode", ["tail", "norm", "trunc"])
+@pytest.mark.parametrize("masked,clamp", [(False, None), (True, None), (False, -6.0), (True, -6.0)])
+def test_opd_kl_topk_vs_oracle(kl_type, alpha, norm_mode, masked, clamp):
+    """compute_opd_kl_topk on [R, K] log-probs: every KL type x normalisation x union mask x clamp, values and
+    gradient w.r.t. the student log-probs."""
+    from relax_amd.opd_utils import compute_opd_kl_topk
+
+    dev = require_gpu()
+    r, k, v = 37, 70, 400
+    g = torch.Generator().manual_seed(7)
+    full_s = torch.log_softmax(torch.randn(r, v, generator=g) * 2, -1)
+    full_t = torch.log_softmax(torch.randn(r, v, generator=g) * 2, -1)
+    s, t = full_s[:, :k].contiguous(), full_t[:, :k].contiguous()
+    mask = None
+    if masked:
+        ksz = torch.randint(1, k + 1, (r,), generator=g)
+        mask = torch.arange(k).unsqueeze(0) < ksz.unsqueeze(1)
+    up = torch.randn(r, generator=g)
+    sc = s.clone().requires_grad_()
+    if mask is None:
+        want = D.opd_kl_topk(sc, t, kl_type, alpha, norm_mode, clamp)
+    else:
+        # Row by row on the valid prefix, where the mask is a no-op and (the tail bin being cut off with the
+        # padding) "tail" reads as "trunc".  The masked formulation itself is pinned against this one on the CPU; its
+        # autograd gradient is NaN for "norm" (0 * (-inf - -inf) reaches the log-sum-exp), which no kernel should copy.
+        mode = "trunc" if norm_mode == "tail" else norm_mode
+        want = torch.cat([D.opd_kl_topk(sc[i:i + 1, :n], t[i:i + 1, :n], kl_type, alpha, mode, clamp)
+                          for i, n in enumerate(ksz.tolist())])
+        torch.testing.assert_close(want.detach(), D.opd_kl_topk(s, t, kl_type, alpha, norm_mode, clamp, mask),
+                                   atol=1e-5, rtol=1e-5)
+    (want * up).sum().backward()
+    sd = s.to(dev).requires_grad_()
+    got = compute_opd_kl_topk(sd, t.to(dev), kl_type, alpha, norm_mode, clamp, None if mask is None else mask.to(dev))
+    (got * up.to(dev)).sum().backward()
+    scale = max(1.0, want.detach().abs().max().item())
+    torch.testing.assert_close(got.detach().cpu(), want.detach(), atol=2e-5 * scale, rtol=2e-5)
+    gscale = max(1.0, sc.grad.abs().max().item())
+    torch.testing.assert_close(sd.grad.cpu(), sc.grad, atol=2e-5 * gscale, rtol=2e-4)
+
+
+def test_opd_kl_topk_argument_checks():
+    from relax_amd.opd_utils import compute_opd_kl, compute_opd_kl_topk
+
+    dev = require_gpu()
+    s = torch.zeros(3, 4, device=dev) - 2.0
+    with pytest.raises(ValueError, match="Unknown opd_kl_type"):
+        compute_opd_kl_topk(s, s, "nope")
+    with pytest.raises(ValueError, match="jsd_alpha"):
+        compute_opd_kl_topk(s, s, "jsd", 1.5)
+    assert compute_opd_kl_topk(s[:0], s[:0]).shape == (0,)
+    # identical distributions: zero divergence in every mode
+    for kt in ("reverse_kl", "forward_kl", "jsd", "low_var_kl"):
+        assert compute_opd_kl(s, s, "jsd" if kt != "low_var_kl" else kt).abs().max().item() < 1e-6

@@ -134,6 +134,49 @@ def test_opd_sampled_token_forms_and_tail_bin():
     torch.testing.assert_close(got, (pt * (pt.log() - ps.log())).sum(-1), atol=1e-6, rtol=0)
 
 
+def test_opd_union_mask_and_jsd_closed_forms():
+    """The union path's padding mask: padded entries drop out, the tail bin is cut off with them, and the masked
+    result equals the unmasked one on the row's valid prefix; JSD against its textbook definition."""
+    torch.manual_seed(3)
+    s = torch.log_softmax(torch.randn(4, 12), -1)[:, :6]
+    t = torch.log_softmax(torch.randn(4, 12), -1)[:, :6]
+    ksz = torch.tensor([6, 4, 1, 3])
+    mask = torch.arange(6).unsqueeze(0) < ksz.unsqueeze(1)
+    for kl_type, alpha in (("reverse_kl", 0.0), ("forward_kl", 1.0), ("jsd", 0.25), ("low_var_kl", 0.0)):
+        for mode in ("norm", "trunc"):
+            got = D.opd_kl_topk(s, t, kl_type, alpha, mode, None, mask)
+            for i, n in enumerate(ksz.tolist()):
+                want = D.opd_kl_topk(s[i:i + 1, :n], t[i:i + 1, :n], kl_type, alpha, mode)
+                torch.testing.assert_close(got[i:i + 1], want, atol=1e-6, rtol=1e-6)
+        # with a mask the tail bin does not contribute: "tail" degenerates to "trunc"
+        torch.testing.assert_close(D.opd_kl_topk(s, t, kl_type, alpha, "tail", None, mask),
+                                   D.opd_kl_topk(s, t, kl_type, alpha, "trunc", None, mask))
+    # generalised JSD on complete distributions: (1-a) KL(p || m) + a KL(q || m), m = (1-a) p + a q
+    p, q = torch.softmax(torch.randn(5, 9).double(), -1), torch.softmax(torch.randn(5, 9).double(), -1)
+    a = 0.3
+    m = (1 - a) * p + a * q
+    want = (1 - a) * (p * (p / m).log()).sum(-1) + a * (q * (q / m).log()).sum(-1)
+    got = D.opd_kl_topk(p.log().float(), q.log().float(), "jsd", a, "trunc")
+    torch.testing.assert_close(got.double(), want, atol=1e-6, rtol=1e-5)
+    # clamping from below bounds the log-ratio
+    lo = D.opd_kl(torch.tensor([-50.0]), torch.tensor([-1.0]), "reverse_kl", min_clamp=-10.0)
+    assert lo.item() == -9.0
+
+
+def test_log_probs_on_topk_ids_against_log_softmax():
+    torch.manual_seed(5)
+    x = torch.randn(7, 40) * 3
+    ids = torch.randint(0, 40, (7, 5))
+    ids[0, 0], ids[1, 1] = -1, 45
+    got = D.log_probs_on_topk_ids(x, ids)
+    ref = torch.log_softmax(x.double(), -1)
+    ok = (ids >= 0) & (ids < 40)
+    torch.testing.assert_close(got[ok].double(), ref.gather(-1, ids.clamp(0, 39))[ok], atol=2e-6, rtol=0)
+    assert got[0, 0] == float("-inf")
+    torch.testing.assert_close(got[1, 1].double(), -torch.logsumexp(x[1].double(), -1), atol=2e-6, rtol=0)
+    assert D.log_probs_on_topk_ids(x[:0], ids[:0]).shape == (0, 5)
+
+
 def test_response_slicing_literal_and_bruteforce(literals):
     fx = literals["response_slicing"]
     logits = torch.tensor(fx["logits"])
