@@ -227,6 +227,28 @@ int relax_amd_reverse_kl_step_fused(const void* student, const void* teacher, in
                                     float* lse_s, float* lse_t, void* dstudent, void* stream);
 
 /*
+ * Log-prob + entropy with a vocabulary keep mask: the log_prob_keep_mask branch of
+ * _VocabParallelLogProbEntropy.forward / .backward (relax/utils/training/ppo_utils.py:546-567, 597-629).  The
+ * log-prob's softmax runs over the entries whose mask byte is non-zero plus the target; the entropy over the whole row.
+ *   keep_mask  uint8 [n_tokens, vocab] indexed by token (row stride keep_stride >= vocab)
+ *   lse_kept   fp32 [n_tokens] out: log-sum-exp over kept entries (needed by the backward)
+ *   entropy, lse_full, spx   fp32 [n_tokens] out, may be NULL when no entropy is wanted
+ * bwd: dlogits = g_lp*(onehot - keep'*p_kept)/T + g_ent*p_full*(spx - x/T)/T, keep' = keep or target; every row
+ *      is written once.
+ */
+int relax_amd_logprob_entropy_masked_fwd(const void* logits, int dtype, int64_t n_tokens, int64_t vocab,
+                                         int64_t row_stride, const int32_t* row_ids, const int64_t* targets,
+                                         const uint8_t* keep_mask, int64_t keep_stride, float inv_temperature,
+                                         float* log_prob, float* entropy, float* lse_kept, float* lse_full, float* spx,
+                                         void* stream);
+int relax_amd_logprob_entropy_masked_bwd(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
+                                         int64_t row_stride, const int32_t* token_of_row, const int64_t* targets,
+                                         const uint8_t* keep_mask, int64_t keep_stride, const float* lse_kept,
+                                         const float* lse_full, const float* spx, const float* g_lp,
+                                         const float* g_ent, float grad_scale, float inv_temperature, void* dlogits,
+                                         int64_t d_row_stride, void* stream);
+
+/*
  * Log-probs of K given vocabulary ids per token: compute_log_probs_on_topk_token_ids
  * (relax/utils/opd/opd_utils.py:1022-1094) on one rank.
  *   topk_ids      int64 [n_tokens, k]; ids < 0 are sentinels (-inf out, no gradient), ids >= vocab read as a zero

@@ -166,6 +166,54 @@ class LogProbEntropy(torch.autograd.Function):
         return d, None, None, None, None, None, None
 
 
+class LogProbEntropyMasked(torch.autograd.Function):
+    """(logits [R,V], targets [R], keep mask bool [R,V]) -> (log_prob [R], entropy [R]): the log-prob's softmax is
+    restricted to the kept vocabulary entries (plus the target), the entropy uses the whole row."""
+
+    @staticmethod
+    def forward(ctx, logits, targets, keep, inv_temperature, with_entropy, with_entropy_grad):
+        with_entropy_grad = bool(with_entropy and with_entropy_grad)
+        x = _rows(logits)
+        n, v = x.shape
+        if targets.dtype != torch.int64 or not targets.is_contiguous():
+            targets = targets.to(torch.int64).contiguous()
+        kw = dict(dtype=torch.float32, device=x.device)
+        lp, lk = torch.empty(n, **kw), torch.empty(n, **kw)
+        ent = torch.empty(n, **kw) if with_entropy else None
+        lf = torch.empty(n, **kw) if with_entropy else None
+        spx = torch.empty(n, **kw) if with_entropy else None
+        stride = x.stride(0) if n > 1 else v
+        check(lib.relax_amd_logprob_entropy_masked_fwd(_p(x), _code(x), n, v, stride, None, _p(targets), _p(keep), v,
+                                                       float(inv_temperature), _p(lp), _p(ent), _p(lk), _p(lf),
+                                                       _p(spx), _stream()))
+        ctx.save_for_backward(x, targets, keep, lk, lf if with_entropy_grad else None,
+                              spx if with_entropy_grad else None)
+        ctx.inv_temperature = inv_temperature
+        ctx.with_entropy_grad = with_entropy_grad
+        if ent is None:
+            ent = lp.new_zeros((0,))
+        if not with_entropy_grad:
+            ctx.mark_non_differentiable(ent)
+        return lp, ent
+
+    @staticmethod
+    def backward(ctx, g_lp, g_ent):
+        x, targets, keep, lk, lf, spx = ctx.saved_tensors
+        if g_lp is None:
+            raise RuntimeError("LogProbEntropyMasked expected a materialized grad_log_prob")
+        if not ctx.with_entropy_grad or g_ent is None or g_ent.numel() == 0:
+            g_ent = None
+        n, v = x.shape
+        d = torch.empty((n, v), dtype=x.dtype, device=x.device)
+        stride = x.stride(0) if n > 1 else v
+        g_lp = _f32(g_lp.reshape(-1))
+        g_ent = None if g_ent is None else _f32(g_ent.reshape(-1))
+        check(lib.relax_amd_logprob_entropy_masked_bwd(_p(x), _code(x), n, v, stride, None, _p(targets), _p(keep), v,
+                                                       _p(lk), _p(lf), _p(spx), _p(g_lp), _p(g_ent), 1.0,
+                                                       float(ctx.inv_temperature), _p(d), v, _stream()))
+        return d, None, None, None, None, None
+
+
 # ------------------------------------------------------------------------------------------------------- row maps
 
 

@@ -41,10 +41,17 @@ def calculate_log_probs_and_entropy(
     holds no [chunk, V] temporaries, so there is nothing to chunk.  Results do not depend on it.
     """
     _single_rank(tp_group)
-    if log_prob_keep_mask is not None:
-        raise NotImplementedError("log_prob_keep_mask is not supported by the fused kernel (no production caller)")
     if logits.size(0) == 0:
         return logits.new_zeros((0,)), (logits.new_zeros((0,)) if with_entropy else None)
+    if log_prob_keep_mask is not None:
+        # the log-prob's softmax only sees the kept vocabulary entries (and the target); the entropy sees the row
+        if log_prob_keep_mask.shape != logits.shape:
+            raise ValueError(f"log_prob_keep_mask {tuple(log_prob_keep_mask.shape)} must match the logits "
+                             f"{tuple(logits.shape)}")
+        keep = log_prob_keep_mask.to(device=logits.device, dtype=torch.uint8).contiguous()
+        lp, ent = ops.LogProbEntropyMasked.apply(logits, tokens, keep, 1.0, bool(with_entropy),
+                                                 bool(with_entropy_grad))
+        return lp.unsqueeze(-1), (ent if with_entropy else None)
     lp, ent = ops.LogProbEntropy.apply(logits, tokens, None, None, 1.0, bool(with_entropy), bool(with_entropy_grad))
     return lp.unsqueeze(-1), (ent if with_entropy else None)
 

@@ -87,6 +87,59 @@ def test_forward_backward_vs_oracle(n, v, dtype, scale, tol, inv_t):
     torch.testing.assert_close(lp3, lp, atol=1e-6, rtol=0)
 
 
+def test_keep_mask_reference_literal_and_random_rows(literals):
+    """log_prob_keep_mask: the reference test's literal case, then random rows in every dtype (the target is kept
+    whatever the mask says; entropy ignores the mask), values and gradients against the oracle."""
+    import relax_amd
+
+    dev = require_gpu()
+    fx = literals["logprob_single_rank"]
+    announce("keep mask literal")
+    keep = torch.tensor(fx["keep_mask"])
+    wl, we = torch.tensor(fx["logprob_weights"]), torch.tensor(fx["entropy_weights"])
+    xc = torch.tensor(fx["logits"], requires_grad=True)
+    tok = torch.tensor(fx["tokens"])
+    lp, ent = O.calculate_log_probs_and_entropy(xc, tok, None, with_entropy=True, log_prob_keep_mask=keep)
+    ((lp.squeeze(-1) * wl).sum() + (ent * we).sum()).backward()
+    xd = torch.tensor(fx["logits"], device=dev, requires_grad=True)
+    glp, gent = relax_amd.calculate_log_probs_and_entropy(xd, tok.to(dev), None, with_entropy=True,
+                                                          log_prob_keep_mask=keep.to(dev))
+    ((glp.squeeze(-1) * wl.to(dev)).sum() + (gent * we.to(dev)).sum()).backward()
+    torch.testing.assert_close(glp.cpu(), lp.detach(), atol=2e-6, rtol=0)
+    torch.testing.assert_close(gent.cpu(), ent.detach(), atol=2e-6, rtol=0)
+    torch.testing.assert_close(xd.grad.cpu(), xc.grad, atol=2e-6, rtol=0)
+    for n, v, dtype, tol in ((9, 1003, torch.float32, 3e-5), (6, 151936, torch.bfloat16, 2e-3),
+                             (7, 4104, torch.float16, 2e-3)):
+        announce("keep mask", n, v, dtype)
+        g = torch.Generator().manual_seed(v)
+        x = (torch.randn(n, v, generator=g) * 3).to(dtype)
+        tok = torch.randint(0, v, (n,), generator=g)
+        keep = torch.rand(n, v, generator=g) < 0.3
+        keep[0] = True                       # nothing masked: must equal the unmasked path
+        keep[1] = False                      # everything masked: only the target survives, log-prob 0
+        wl, we = torch.randn(n, generator=g), torch.randn(n, generator=g)
+        xc = x.clone().float().requires_grad_()
+        lp, ent = O.calculate_log_probs_and_entropy(xc, tok, None, with_entropy=True, log_prob_keep_mask=keep)
+        ((lp.squeeze(-1) * wl).sum() + (ent * we).sum()).backward()
+        xd = x.to(dev).requires_grad_()
+        glp, gent = relax_amd.calculate_log_probs_and_entropy(xd, tok.to(dev), None, with_entropy=True,
+                                                              log_prob_keep_mask=keep.to(dev))
+        ((glp.squeeze(-1) * wl.to(dev)).sum() + (gent * we.to(dev)).sum()).backward()
+        torch.testing.assert_close(glp.cpu(), lp.detach(), atol=tol, rtol=0)
+        torch.testing.assert_close(gent.cpu(), ent.detach(), atol=tol, rtol=0)
+        ulp = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 1e-5}[dtype]
+        torch.testing.assert_close(xd.grad.float().cpu(), xc.grad, atol=tol, rtol=ulp)
+        assert abs(glp[1].item()) < 1e-6
+        plain, _ = relax_amd.calculate_log_probs_and_entropy(x.to(dev), tok.to(dev), None, with_entropy=False)
+        assert abs(plain[0].item() - glp[0].item()) < 1e-5
+        # metric-only entropy: no entropy gradient reaches the logits
+        xd2 = x.to(dev).requires_grad_()
+        l2, e2 = relax_amd.calculate_log_probs_and_entropy(xd2, tok.to(dev), None, with_entropy=True,
+                                                           log_prob_keep_mask=keep.to(dev), with_entropy_grad=False)
+        assert not e2.requires_grad
+        l2.sum().backward()
+
+
 def test_autograd_function_semantics(literals):
     import relax_amd
 
