@@ -10,6 +10,7 @@ first 20 % of every sequence masked out.
 Prints ONE JSON line (metric, value, roofline of the dominant kernel, CPU baseline of the same arithmetic).
 
 ``--workload`` selects the other configurations of the same path, each printed in the same format:
+``cfg1`` (GRPO plumbing case: 512 responses x 256 tokens, fp32 logits [131072, 32000], rewards -> advantages -> loss),
 ``lmhead`` (fused LM-head + log-prob/entropy forward and dhidden/dweight backward, hidden [32768, 4096], MFMA-bound),
 ``reverse_kl`` (on-policy distillation, student/teacher [16384, 151936], forward + student dlogits),
 ``varlen_gspo`` / ``varlen_cispo`` (8 packed sequences of 2k-32k tokens, RLOO advantages, sequence-level losses).
@@ -156,7 +157,8 @@ def emit(a, n_tokens, wall, workload, config, roofline, cpu):
     print(json.dumps({
         "metric": METRIC, "value": n_tokens / (wall / a.steps), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": wall * 1e3 / a.steps, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": {"workload": workload, **config},
+        "vs_baseline": None, "dtype": config.pop("logits_dtype", "bf16"), "data": "synthetic",
+        "config": {"workload": workload, **config},
         "roofline": roofline, "cpu_baseline": cpu,
     }))
 
@@ -294,6 +296,87 @@ def run_reverse_kl(a, dev) -> None:
          None)
 
 
+def run_cfg1(a, dev) -> None:
+    """GRPO plumbing case: 64 prompts x group 8 = 512 responses x 256 tokens, fp32 logits [131072, 32000] ~ N(0, 2),
+    rewards ~ Bernoulli(0.4), group-normalised advantages (mean / std, eps 1e-6), trailing pad of 0..63 masked tokens
+    per response, PPO-clip 0.2, old = lp + N(0, 0.05), token-mean.  One step = policy loss forward + backward to fp32
+    dlogits; reward post-processing + advantage broadcast run once before and are timed separately."""
+    import relax_amd
+    from relax_amd import utils as U
+
+    prompts, group, resp_len, v = 64, 8, 256, 32000
+    seqs = prompts * group
+    n = seqs * resp_len
+    cpu = torch.Generator().manual_seed(0)
+    g = torch.Generator(device=dev).manual_seed(0)
+    logits = torch.empty((1, n, v), dtype=torch.float32, device=dev)
+    for s in range(0, n, 4096):
+        logits[0, s:s + 4096] = torch.randn((min(4096, n - s), v), device=dev, generator=g) * 2.0
+    rewards = torch.bernoulli(torch.full((seqs,), 0.4), generator=cpu).tolist()
+    pads = torch.randint(0, 64, (seqs,), generator=cpu).tolist()
+    masks = []
+    for p in pads:
+        m = torch.ones(resp_len, device=dev)
+        if p:
+            m[resp_len - p:] = 0.0
+        masks.append(m)
+    args = make_args()
+    args.eps_clip_high = 0.2
+    args.use_kl_loss = False
+    args.rewards_normalization = True
+    args.grpo_std_normalization = True
+    args.n_samples_per_prompt = group
+    args.global_batch_size = seqs
+    samples = [SimpleNamespace(group_index=i // group, get_reward_value=(lambda _a, r=r: r)) for i, r in enumerate(rewards)]
+    total_unmasked = float(sum(resp_len - p for p in pads))
+    batch = dict(
+        unconcat_tokens=[torch.randint(0, v, (resp_len,), device=dev, generator=g) for _ in range(seqs)],
+        total_lengths=[resp_len] * seqs, response_lengths=[resp_len] * seqs, loss_masks=masks,
+        relax_amd_sample_denominators=torch.full((seqs,), total_unmasked, device=dev),
+    )
+    args.use_kl_loss = False
+    batch["advantages"] = [torch.zeros(resp_len, device=dev) for _ in range(seqs)]
+    attach_old_and_ref(batch, logits, args, g)
+    batch.pop("ref_log_probs")
+    logits.requires_grad_()
+
+    # Rewards -> group-normalised advantages happen once per rollout, not per optimisation step: timed on their own
+    # (second call, warm) and reported in config.advantages_ms.
+    adv_ms = 0.0
+    for _ in range(2):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        _, normed = U.post_process_rewards(args, samples, device=dev)
+        data = dict(log_probs=batch["log_probs"], rewards=normed, loss_masks=masks)
+        relax_amd.compute_advantages_and_returns(args, data)
+        torch.cuda.synchronize()
+        adv_ms = (time.perf_counter() - t0) * 1e3
+    batch["advantages"] = data["advantages"]
+
+    def step():
+        logits.grad = None
+        loss, _ = relax_amd.policy_loss_function(args, batch, logits, None)
+        loss.backward()
+        return loss
+
+    wall, kernel_ms, _, loss = timed_steps(step, a.warmup, a.steps)
+    row_bytes = float(v * 4) * n
+    dom = kernel_ms["actor_step_fused"]
+    achieved = 3.0 * row_bytes / (dom * 1e-3) / 1e9
+    out_cpu = None
+    if a.cpu_rows > 0:
+        out_cpu = cpu_baseline(args, a.cpu_rows, v)
+    emit(a, n, wall,
+         f"GRPO plumbing: {prompts} prompts x {group} = {seqs} responses x {resp_len} tokens = {n} rows x V={v} fp32 "
+         f"logits, group-normalised advantages, PPO-clip 0.2, token-mean, fwd + bwd to dlogits",
+         {"rows": n, "vocab": v, "loss": float(loss.item()), "logits_dtype": "f32", "advantages_ms": adv_ms},
+         {"bound": "hbm", "kernel": "actor_step_fused_kernel<float, true, 512>", "achieved": achieved,
+          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+          "algorithmic_bytes_per_launch": 3.0 * row_bytes, "avg_launch_ms": dom, "kernel_ms": kernel_ms,
+          "step_algorithmic_GBs": 3.0 * row_bytes / (wall / a.steps) / 1e9},
+         out_cpu)
+
+
 def run_varlen(a, dev, loss_kind: str) -> None:
     """8 packed sequences with lengths ~ U[2k, 32k], 3-6 masked tool-output spans (~30 % of tokens) per sequence,
     RLOO advantages from rewards ~ U[0, 1] over the group of 8, GSPO (clip 3e-4/4e-4) or CISPO loss,
@@ -367,7 +450,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="actor_step",
-                    choices=["actor_step", "lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo"])
+                    choices=["actor_step", "cfg1", "lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo"])
     ap.add_argument("--seqs", type=int, default=SEQS)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
     ap.add_argument("--vocab", type=int, default=VOCAB)
@@ -392,6 +475,8 @@ def main() -> int:
     torch.cuda.set_device(dev)
     if a.workload == "actor_step":
         run_actor_step(a, dev)
+    elif a.workload == "cfg1":
+        run_cfg1(a, dev)
     elif a.workload == "lmhead":
         run_lmhead(a, dev)
     elif a.workload == "reverse_kl":

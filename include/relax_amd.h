@@ -121,6 +121,18 @@ int relax_amd_build_row_maps(const int64_t* row_begin, const int64_t* cu_resp, i
                              void* stream);
 
 /*
+ * Packed target ids of the response tokens in one launch: the per-sample `tokens[-response_length:]` of get_responses
+ * (loss.py:103-125) and the shifted, zero-padded `tokens[1:]` of the SFT layout (relax/utils/sft_utils.py:23-40).
+ *   tokens     int64, every sample's token ids back to back
+ *   src_begin  [n_samples] int64 position in `tokens` of sample i's first target
+ *   src_end    [n_samples] int64 end of sample i's tokens; targets past it read as 0
+ *   cu_resp    [n_samples+1] int64 exclusive prefix sum of response lengths
+ *   targets    [n_tokens] out int64
+ */
+int relax_amd_gather_targets(const int64_t* tokens, const int64_t* src_begin, const int64_t* src_end,
+                             const int64_t* cu_resp, int64_t n_samples, int64_t* targets, void* stream);
+
+/*
  * Per-token policy loss, KL penalty, masked per-sample aggregation and the
  * gradient coefficients d loss / d log_prob, d loss / d entropy.  Replaces the
  * arithmetic of policy_loss_function (loss.py:961-1134) with

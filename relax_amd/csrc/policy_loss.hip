@@ -137,9 +137,37 @@ __global__ __launch_bounds__(256) void row_maps_kernel(const int64_t* __restrict
   }
 }
 
+// Target ids of the packed response tokens, gathered from the packed token ids: sample i's j-th target sits at
+// src_begin[i] + j of `tokens`, or is 0 when that position is past src_end[i] (the SFT layout's final pad).
+__global__ __launch_bounds__(256) void gather_targets_kernel(const int64_t* __restrict__ tokens,
+                                                             const int64_t* __restrict__ src_begin,
+                                                             const int64_t* __restrict__ src_end,
+                                                             const int64_t* __restrict__ cu,
+                                                             int64_t* __restrict__ targets) {
+  const int64_t i = blockIdx.x;
+  const int64_t beg = cu[i], len = cu[i + 1] - cu[i], s0 = src_begin[i], s1 = src_end[i];
+  for (int64_t j = threadIdx.x; j < len; j += 256) targets[beg + j] = (s0 + j < s1) ? tokens[s0 + j] : 0;
+}
+
 }  // namespace relax_amd
 
 using namespace relax_amd;
+
+extern "C" int relax_amd_gather_targets(const int64_t* tokens, const int64_t* src_begin, const int64_t* src_end,
+                                        const int64_t* cu_resp, int64_t n_samples, int64_t* targets, void* stream) {
+  if (n_samples < 0 || n_samples > 2147483647LL) {
+    set_error("gather_targets: bad n_samples=%lld", (long long)n_samples);
+    return RELAX_AMD_EINVAL;
+  }
+  if (n_samples == 0) return RELAX_AMD_OK;
+  if (!tokens || !src_begin || !src_end || !cu_resp || !targets) {
+    set_error("gather_targets: NULL argument");
+    return RELAX_AMD_EINVAL;
+  }
+  hipLaunchKernelGGL(gather_targets_kernel, dim3(static_cast<unsigned>(n_samples)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), tokens, src_begin, src_end, cu_resp, targets);
+  return check_launch("gather_targets");
+}
 
 extern "C" int relax_amd_policy_loss(const relax_amd_policy_loss_args* a, void* stream) {
   if (!a) {

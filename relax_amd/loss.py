@@ -95,17 +95,27 @@ class PackedLayout:
         cu = [0]
         for r in self.response_lengths:
             cu.append(cu[-1] + r)
-        dev = upload_int64(begins + cu, device)
-        self.row_begin, self.cu_resp = dev[: self.n_samples], dev[self.n_samples :]
+        # where each sample's targets sit in the back-to-back token ids: the last `response` tokens, or (SFT layout)
+        # the tokens shifted by one with a final zero
+        src_begin, src_end, pos = [], [], 0
+        for toks, is_sft, resp in zip(unconcat_tokens, sft, self.response_lengths, strict=False):
+            n_tok = int(toks.numel())
+            if resp > n_tok:
+                raise ValueError(f"response length {resp} exceeds the sample's {n_tok} tokens")
+            src_begin.append(pos + 1 if is_sft else pos + n_tok - resp)
+            src_end.append(pos + n_tok)
+            pos += n_tok
+        b = self.n_samples
+        dev = upload_int64(begins + cu + src_begin + src_end, device)
+        self.row_begin, self.cu_resp = dev[:b], dev[b : 2 * b + 1]
         self.row_ids, self.sample_ids, self.token_of_row = ops.build_row_maps(
             self.row_begin, self.cu_resp, self.n_tokens, n_rows, want_inverse=need_inverse
         )
-        parts = []
-        for toks, is_sft, resp in zip(unconcat_tokens, sft, self.response_lengths, strict=False):
-            parts.append(torch.nn.functional.pad(toks[1:], (0, 1), value=0) if is_sft else toks[-resp:] if resp else toks[:0])
-        self.targets = (
-            torch.cat(parts).to(device=device, dtype=torch.int64) if parts else torch.zeros(0, dtype=torch.int64, device=device)
-        )
+        self.targets = torch.empty(self.n_tokens, dtype=torch.int64, device=device)
+        if self.n_tokens:
+            packed = torch.cat([t.reshape(-1) for t in unconcat_tokens]) if b > 1 else unconcat_tokens[0].reshape(-1)
+            packed = packed.to(device=device, dtype=torch.int64)
+            ops.gather_targets(packed, dev[2 * b + 1 : 3 * b + 1], dev[3 * b + 1 :], self.cu_resp, self.targets)
 
     def split(self, flat: torch.Tensor) -> list[torch.Tensor]:
         return list(torch.split(flat, self.response_lengths))
@@ -217,10 +227,16 @@ def _single_pass_ok(args, flat, kw, needs_bwd) -> bool:
 
 
 def _cat_f32(parts, device):
+    """Per-sample tensors -> one packed fp32 vector on ``device`` (one concatenation, one conversion)."""
     if parts is None:
         return None
     if isinstance(parts, torch.Tensor):
         return parts.to(device=device, dtype=torch.float32).reshape(-1)
+    if len(parts) == 1:
+        return parts[0].reshape(-1).to(device=device, dtype=torch.float32)
+    first = parts[0]
+    if all(p.device == first.device and p.dtype == first.dtype and p.dim() == 1 for p in parts):
+        return torch.cat(parts).to(device=device, dtype=torch.float32)
     return torch.cat([p.to(device=device).reshape(-1) for p in parts]).to(torch.float32)
 
 

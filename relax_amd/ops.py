@@ -228,6 +228,14 @@ def build_row_maps(row_begin, cu_resp, n_tokens: int, n_rows: int, want_inverse:
     return row_ids, sample_ids, inv
 
 
+def gather_targets(packed_tokens, src_begin, src_end, cu_resp, out):
+    """out[cu[i] + j] = packed_tokens[src_begin[i] + j] if that position is before src_end[i] else 0."""
+    _need_gpu(packed_tokens, src_begin, src_end, cu_resp, out)
+    check(lib.relax_amd_gather_targets(_p(packed_tokens), _p(src_begin), _p(src_end), _p(cu_resp), src_begin.numel(),
+                                       _p(out), _stream()))
+    return out
+
+
 def segment_sum(mask, cu_resp, values=None):
     """fp64 [B]: per-sample sum of mask (or values*mask)."""
     dev = _need_gpu(mask, cu_resp)
