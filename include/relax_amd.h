@@ -213,6 +213,31 @@ int relax_amd_masked_whiten(const float* values, const float* mask, int64_t n, i
                             double* partials, float* stats, float* out, void* stream);
 
 /*
+ * Per-sequence reverse recurrences over the packed response layout (cu_resp [n_samples+1] int64), fp32 or fp64
+ * (dtype RELAX_AMD_F32 / RELAX_AMD_F64 applies to every data pointer of the call).  Each sequence is evaluated in the
+ * reference's sequential order, so results are bit-identical to its Python loops.
+ *
+ * relax_amd_reinforce_pp_returns: get_reinforce_plus_plus_returns (relax/utils/training/ppo_utils.py:708-804, one
+ *   context-parallel rank).  G_t = r_t + gamma * G_{t+1}, r_t = -kl_coef * kl[t] on mask != 0 tokens (0 elsewhere,
+ *   so masked NaN/inf never enter), rewards[i] added at the last valid token; 0 outside the mask.
+ * relax_amd_gae: get_advantages_and_returns / vanilla_gae (ppo_utils.py:846-906, 1026-1047).
+ *   delta_t = rewards[t] + gamma * values[t+1] - values[t], A_t = delta_t + gamma*lambd * A_{t+1}, returns = A + values.
+ */
+int relax_amd_reinforce_pp_returns(const void* kl, const void* mask, const void* rewards, int dtype,
+                                   const int64_t* cu_resp, int64_t n_samples, double kl_coef, double gamma,
+                                   void* returns, void* stream);
+int relax_amd_gae(const void* values, const void* rewards, int dtype, const int64_t* cu_resp, int64_t n_samples,
+                  double gamma, double lambd, void* advantages, void* returns, void* stream);
+
+/*
+ * REINFORCE++ advantage normaliser on one rank: distributed_masked_normalize (relax/utils/distributed_utils.py:161-213).
+ * Population mean / variance (ddof = 0) over mask != 0, out = (x - mean) * rsqrt(max(variance, variance_floor)) on
+ * the mask and 0 elsewhere.  stats [3] out (same dtype) = mean, variance, count.
+ */
+int relax_amd_masked_normalize(const void* values, const void* mask, int dtype, int64_t n, double variance_floor,
+                               void* out, void* stats, void* stream);
+
+/*
  * Full-vocab reverse KL(student || teacher) per token and its gradient w.r.t.
  * the student logits.  The K = vocab case of compute_opd_kl's jsd_alpha == 0
  * branch (relax/utils/opd/opd_utils.py:1165-1169) on complete log-softmax rows.

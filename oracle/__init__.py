@@ -38,6 +38,13 @@ live in ``tests/test_oracle_*.py``):
   textbook formulas).  The exact edge conventions the closed forms do not fix
   (CISPO ``A == 0`` branch, whiten Bessel switch at n < 2) are taken from
   reading the reference source; see DESIGN notes in each docstring.
+* ``advantages.reinforce_pp_returns`` / ``reinforce_pp_baseline_advantages``: the input cases of
+  tests/utils/training/test_reinforce_plus_plus.py:45-167 with expectations worked out by hand
+  (gamma = 1 reverse cumulative sums; the gamma = 0.5 case [0.20625, 0, 1.025]; masked NaN/inf).
+  ``advantages.gae``: the textbook sum A_t = sum_l (gamma*lambda)^l delta_{t+l} in fp64 and the shapes case
+  of tests/backends/megatron/test_ppo_gae_parity.py:41-60.  ``advantages.masked_normalize``: numpy
+  population moments.  ``opd.opd_kl`` union mask / ``log_probs_on_topk_ids``: closed forms (row-prefix
+  equivalence, textbook JSD, ``log_softmax`` gather).
 * ``reducers.seq_mean_token_sum``: the reference has no implementation of this
   aggregation (only the reducer plug-in point, loss.py:1062-1072)
   -- **parity unpinned**; defined here as sum_i sum_t x*m / B.

@@ -90,3 +90,61 @@ def advantages_and_returns(rewards, shapes_like: list, masks: list | None = None
         flat = masked_whiten(torch.cat(adv), torch.cat(masks))
         adv = list(torch.split(flat, [a.size(0) for a in adv]))
     return adv, returns
+
+
+def reinforce_pp_returns(rewards, kl: list, loss_masks: list, kl_coef: float, gamma: float) -> list:
+    """relax/utils/training/ppo_utils.py:708-804 on one context-parallel rank: token rewards ``-kl_coef * kl`` on
+    valid tokens (selected, not multiplied, so masked NaN cannot leak), the sequence reward on the last valid token,
+    ``G_t = r_t + gamma * G_{t+1}`` evaluated right to left, zero outside the mask and for fully masked sequences."""
+    if not (len(kl) == len(loss_masks) == len(rewards)):
+        raise ValueError("rewards, kl, loss_masks must contain the same number of responses.")
+    out = []
+    for i, (k, m) in enumerate(zip(kl, loss_masks)):
+        if k.shape != m.shape:
+            raise ValueError(f"KL and loss mask for response {i} must have the same shape")
+        valid = m != 0
+        if not bool(valid.any()):
+            out.append(torch.zeros_like(k))
+            continue
+        r = -kl_coef * torch.where(valid, k, torch.zeros_like(k))
+        r[int(valid.nonzero()[-1])] += rewards[i]
+        g = torch.zeros_like(r)
+        run = 0.0
+        for t in range(r.numel() - 1, -1, -1):
+            run = r[t] + gamma * run
+            g[t] = run
+        out.append(torch.where(valid, g, torch.zeros_like(g)))
+    return out
+
+
+def reinforce_pp_baseline_advantages(rewards, like: list, loss_masks: list) -> list:
+    """ppo_utils.py:807-843: the (already group-centred) reward on every valid token, zero elsewhere."""
+    return [torch.where(m != 0, torch.ones_like(k) * r, torch.zeros_like(k)) for k, r, m in zip(like, rewards, loss_masks)]
+
+
+def gae(values: torch.Tensor, rewards: torch.Tensor, gamma: float, lambd: float):
+    """ppo_utils.py:846-906 / vanilla_gae :1026-1047 for one response: ``delta_t = r_t + gamma V_{t+1} - V_t``,
+    ``A_t = delta_t + gamma*lambd*A_{t+1}`` right to left (V past the end = 0), returns = A + V."""
+    n = values.numel()
+    adv = torch.zeros_like(values)
+    last = torch.zeros((), dtype=values.dtype)
+    for t in range(n - 1, -1, -1):
+        nxt = values[t + 1] if t < n - 1 else 0.0
+        delta = rewards[t] + gamma * nxt - values[t]
+        last = delta + gamma * lambd * last
+        adv[t] = last
+    return adv, adv + values
+
+
+def masked_normalize(values: torch.Tensor, mask: torch.Tensor, variance_floor: float = 1e-8):
+    """relax/utils/distributed_utils.py:161-213 on one rank: population moments (ddof = 0) over mask != 0, output
+    zero outside the mask.  Returns (normalized, mean, variance, count)."""
+    work = torch.float64 if values.dtype == torch.float64 else torch.float32
+    v = values.to(work)
+    valid = mask != 0
+    count = valid.to(work).sum().clamp_min(1)
+    mean = torch.where(valid, v, torch.zeros_like(v)).sum() / count
+    centred = torch.where(valid, v - mean, torch.zeros_like(v))
+    var = (centred.square().sum() / count).clamp_min(0.0)
+    out = torch.where(valid, (v - mean) * torch.rsqrt(var.clamp_min(variance_floor)), torch.zeros_like(v))
+    return out, mean, var, valid.to(work).sum()

@@ -76,6 +76,9 @@ SIGNATURES = {
     "relax_amd_lmhead_dlogits_t": (
         C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _vp]),
     "relax_amd_reverse_kl_bwd": (C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp]),
+    "relax_amd_reinforce_pp_returns": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp, _i64, C.c_double, C.c_double, _vp, _vp]),
+    "relax_amd_gae": (C.c_int, [_vp, _vp, C.c_int, _vp, _i64, C.c_double, C.c_double, _vp, _vp, _vp]),
+    "relax_amd_masked_normalize": (C.c_int, [_vp, _vp, C.c_int, _i64, C.c_double, _vp, _vp, _vp]),
     "relax_amd_gather_targets": (C.c_int, [_vp, _vp, _vp, _vp, _i64, _vp, _vp]),
     "relax_amd_logprob_entropy_masked_fwd": (
         C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _f32, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -375,31 +375,81 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
 
 
 def compute_advantages_and_returns(args: Namespace, rollout_data: dict) -> None:
-    """GRPO-family branch of loss.py:532-738: broadcast the (already group-normalised) per-sample rewards over each
-    response, optionally whiten across the micro-batch.  Writes ``advantages`` / ``returns`` lists in place."""
-    from .distributed_utils import distributed_masked_whiten
+    """Counterpart of loss.py:532-738 on one GPU.  GRPO family: broadcast the (already group-normalised) per-sample
+    rewards over each response.  ``ppo``: token rewards ``-kl_coef * kl`` (+ the sequence reward on the last token)
+    through GAE.  ``reinforce_plus_plus``: discounted returns; ``reinforce_plus_plus_baseline``: masked broadcast.
+    With ``args.normalize_advantages`` the advantages are whitened (REINFORCE++: population-normalised, with the
+    reference's ``reinforce_pp_*`` statistics) across the micro-batch.  Writes ``advantages`` / ``returns`` in place."""
+    from .distributed_utils import distributed_masked_normalize, distributed_masked_whiten
+    from .ppo_utils import (compute_approx_kl, get_advantages_and_returns_batch,
+                            get_reinforce_plus_plus_baseline_advantages, get_reinforce_plus_plus_returns)
 
     log_probs = rollout_data.get("rollout_log_probs" if getattr(args, "use_rollout_logprobs", False) else "log_probs")
+    ref_log_probs = rollout_data.get("ref_log_probs")
     values = rollout_data.get("values")
     rewards = rollout_data.get("rewards")
     loss_masks = rollout_data.get("loss_masks")
-    if args.advantage_estimator not in GRPO_FAMILY:
-        raise NotImplementedError(f"advantage_estimator {args.advantage_estimator} is not supported. ")
+    est = args.advantage_estimator
+    if est not in GRPO_FAMILY + ("ppo", "reinforce_plus_plus", "reinforce_plus_plus_baseline"):
+        raise NotImplementedError(f"advantage_estimator {est} is not supported. ")
+    if getattr(args, "use_opd", False):
+        raise NotImplementedError("OPD advantage shaping (apply_opd_to_advantages) is outside the fused path")
     xs = log_probs if log_probs is not None else values
     if xs is None:
         return
     dev = xs[0].device
-    # kl only supplies shape / dtype / device for this estimator family (loss.py:574-591)
-    like = [torch.empty(x.shape, dtype=torch.float32, device=dev) for x in xs]
-    rw = torch.tensor(rewards, dtype=torch.float32, device=dev)
-    returns = get_grpo_returns(rw, like)
-    advantages = list(returns)
+    kl_coef = float(getattr(args, "kl_coef", 0.0) or 0.0)
+    if kl_coef == 0 or not log_probs:
+        # kl only supplies shape / dtype / device here (loss.py:574-577)
+        kl = [torch.zeros(x.shape, dtype=torch.float32, device=dev) for x in xs]
+    else:
+        lens = [int(x.numel()) for x in log_probs]
+        flat = compute_approx_kl(torch.cat([x.reshape(-1) for x in log_probs]),
+                                 torch.cat([x.reshape(-1) for x in ref_log_probs]).to(dev),
+                                 kl_loss_type=args.kl_loss_type)
+        kl = list(torch.split(flat, lens))
+    if est in GRPO_FAMILY:
+        rw = torch.tensor(rewards, dtype=torch.float32, device=dev)
+        returns = get_grpo_returns(rw, kl)
+        advantages = list(returns)
+    elif est == "ppo":
+        token_rewards = []
+        for reward, k in zip(rewards, kl, strict=False):
+            k = k * (-kl_coef)
+            k[-1] += reward
+            token_rewards.append(k)
+        advantages, returns = get_advantages_and_returns_batch(
+            rollout_data.get("total_lengths"), rollout_data.get("response_lengths"), values, token_rewards,
+            args.gamma, args.lambd)
+    elif est == "reinforce_plus_plus":
+        rw = torch.tensor(rewards, dtype=torch.float32, device=dev)
+        returns = get_reinforce_plus_plus_returns(
+            rewards=rw, kl=kl, loss_masks=loss_masks, response_lengths=rollout_data.get("response_lengths"),
+            total_lengths=rollout_data.get("total_lengths"), kl_coef=kl_coef, gamma=args.gamma)
+        advantages = list(returns)
+    else:
+        rw = torch.tensor(rewards, dtype=torch.float32, device=dev)
+        advantages = get_reinforce_plus_plus_baseline_advantages(rewards=rw, kl=kl, loss_masks=loss_masks)
+        returns = advantages
     if getattr(args, "normalize_advantages", False):
         flat = torch.cat(advantages)
         masks = torch.cat(loss_masks).to(dev)
         assert flat.size() == masks.size(), f"Shape mismatch before whitening: advantages {flat.size()}, masks {masks.size()}"
-        if masks.numel() > 0:
-            white = distributed_masked_whiten(flat, masks, process_group=None, shift_mean=True)
+        is_rpp = est in ("reinforce_plus_plus", "reinforce_plus_plus_baseline")
+        if is_rpp or masks.numel() > 0:
+            if is_rpp:
+                white, raw_mean, raw_var, count = distributed_masked_normalize(flat, masks, process_group=None)
+                floor = torch.tensor(1e-8, device=dev, dtype=raw_var.dtype)
+                norm_var = raw_var / torch.maximum(raw_var, floor)
+                k = len(advantages)
+                rollout_data["reinforce_pp_advantage_raw_mean"] = [raw_mean.detach()] * k
+                rollout_data["reinforce_pp_advantage_raw_std"] = [raw_var.sqrt().detach()] * k
+                rollout_data["reinforce_pp_advantage_normalized_mean"] = [torch.zeros_like(raw_mean)] * k
+                rollout_data["reinforce_pp_advantage_normalized_std"] = [norm_var.sqrt().detach()] * k
+                rollout_data["reinforce_pp_valid_token_count"] = [count.detach()] * k
+                rollout_data["reinforce_pp_zero_variance"] = [(raw_var == 0).to(dtype=raw_var.dtype).detach()] * k
+            else:
+                white = distributed_masked_whiten(flat, masks, process_group=None, shift_mean=True)
             advantages = list(torch.split(white, [a.size(0) for a in advantages]))
     rollout_data["advantages"] = advantages
     rollout_data["returns"] = returns

@@ -12,13 +12,19 @@ Reference lines (paths relative to the reference checkout):
   compute_opsm_mask                    :142-180
   get_grpo_returns                     :654-661
   compute_rloo_leave_one_out_rewards   :664-705
+  get_reinforce_plus_plus_returns / _baseline_advantages   :708-843
+  get_advantages_and_returns(_batch), vanilla_gae, chunked_gae   :846-1189
 """
 
 from __future__ import annotations
 
+from itertools import accumulate as _accumulate
+
 import torch
 
-from . import ops
+from . import _lib, ops
+from ._lib import check, lib
+from ._staging import upload_int64
 
 
 def _single_rank(tp_group) -> None:
@@ -226,6 +232,108 @@ def get_grpo_returns(rewards, kl):
     for piece, like in zip(torch.split(flat, lens), kl, strict=True):
         outs.append(piece.reshape(like.shape).to(like.dtype))
     return outs
+
+
+def _scan_dtype(t: torch.Tensor):
+    """(torch dtype, ABI code) the recurrences run in: fp64 stays fp64, everything else is evaluated in fp32."""
+    return (torch.float64, _lib.F64) if t.dtype == torch.float64 else (torch.float32, _lib.F32)
+
+
+def _pack(parts, dtype, dev):
+    return torch.cat([p.reshape(-1) for p in parts]).to(device=dev, dtype=dtype) if len(parts) > 1 else \
+        parts[0].reshape(-1).to(device=dev, dtype=dtype)
+
+
+def get_reinforce_plus_plus_returns(rewards, kl, loss_masks, response_lengths, total_lengths, kl_coef: float,
+                                    gamma: float):
+    """Discounted REINFORCE++ returns, one launch for the whole batch (ppo_utils.py:708-804, cp_size == 1):
+    ``G_t = r_t + gamma * G_{t+1}`` with ``r_t = -kl_coef * kl_t`` on valid tokens and the sequence reward added at
+    the last valid token; masked tokens (and fully masked sequences) get 0, and masked NaN/inf never leak."""
+    n = len(rewards)
+    if not (len(kl) == n and len(loss_masks) == n and len(response_lengths) == n and len(total_lengths) == n):
+        raise ValueError(
+            "rewards, kl, loss_masks, response_lengths, and total_lengths must contain the same number of responses.")
+    for i, (k, m) in enumerate(zip(kl, loss_masks)):
+        if k.shape != m.shape:
+            raise ValueError(f"KL and loss mask for response {i} must have the same shape, got {k.shape} and {m.shape}.")
+    if n == 0:
+        return []
+    dev = kl[0].device
+    ops._need_gpu(kl[0])
+    dtype, code = _scan_dtype(kl[0])
+    lens = [int(k.numel()) for k in kl]
+    cu = upload_int64([0] + list(_accumulate(lens)), dev)
+    flat_kl, flat_mask = _pack(kl, dtype, dev), _pack(loss_masks, dtype, dev)
+    rw = torch.as_tensor(rewards).to(device=dev, dtype=dtype).contiguous()
+    out = torch.empty_like(flat_kl)
+    check(lib.relax_amd_reinforce_pp_returns(ops._p(flat_kl), ops._p(flat_mask), ops._p(rw), code, ops._p(cu), n,
+                                             float(kl_coef), float(gamma), ops._p(out), ops._stream()))
+    return [piece.reshape(k.shape).to(k.dtype) for piece, k in zip(torch.split(out, lens), kl)]
+
+
+def get_reinforce_plus_plus_baseline_advantages(rewards, kl, loss_masks):
+    """``rewards[i]`` broadcast over sample i's valid tokens, 0 elsewhere (ppo_utils.py:807-843); ``kl`` only
+    supplies shapes, so non-finite values in it are harmless."""
+    if not (len(rewards) == len(kl) == len(loss_masks)):
+        raise ValueError("rewards, token shapes, and loss_masks must contain the same number of responses.")
+    for i, (k, m) in enumerate(zip(kl, loss_masks)):
+        if k.shape != m.shape:
+            raise ValueError(f"Token shape and loss mask for response {i} must match, got {k.shape} and {m.shape}.")
+    if len(kl) == 0:
+        return []
+    dev = kl[0].device
+    lens = [int(k.numel()) for k in kl]
+    rw = torch.as_tensor(rewards).to(dev)
+    if kl[0].dtype == torch.float64:
+        # the broadcast kernel is fp32; fp64 callers (the reference's own tests) keep every bit of the reward
+        flat = torch.repeat_interleave(rw.to(torch.float64), torch.tensor(lens, device=dev))
+    else:
+        flat = ops.broadcast_per_sample(rw.float(), upload_int64([0] + list(_accumulate(lens)), dev), sum(lens))
+    mask = torch.cat([m.reshape(-1) for m in loss_masks]).to(dev)
+    out = torch.where(mask != 0, flat, torch.zeros((), dtype=flat.dtype, device=dev))
+    return [piece.reshape(k.shape).to(k.dtype) for piece, k in zip(torch.split(out, lens), kl)]
+
+
+def get_advantages_and_returns_batch(total_lengths, response_lengths, values_list, rewards_list, gamma, lambd,
+                                     chunked: bool = True, padded_total_lengths=None):
+    """GAE for a batch of responses in one launch (ppo_utils.py:909-1023, cp_size == 1).  Every sequence is scanned in
+    the order of ``vanilla_gae``; ``chunked`` is accepted for signature compatibility (the reference's chunked scan is
+    a faster evaluation of the same recurrence and agrees with the sequential one to 1e-5)."""
+    b = len(response_lengths)
+    assert b == len(values_list)
+    assert b == len(rewards_list)
+    if b == 0:
+        return [], []
+    dev = values_list[0].device
+    ops._need_gpu(values_list[0])
+    dtype, code = _scan_dtype(values_list[0])
+    lens = [int(r) for r in response_lengths]
+    cu = upload_int64([0] + list(_accumulate(lens)), dev)
+    v = _pack([x[:n] for x, n in zip(values_list, lens)], dtype, dev)
+    r = _pack([x[:n] for x, n in zip(rewards_list, lens)], dtype, dev)
+    adv, ret = torch.empty_like(v), torch.empty_like(v)
+    check(lib.relax_amd_gae(ops._p(v), ops._p(r), code, ops._p(cu), b, float(gamma), float(lambd), ops._p(adv),
+                            ops._p(ret), ops._stream()))
+    out_dtype = values_list[0].dtype
+    return ([a.to(out_dtype) for a in torch.split(adv, lens)], [x.to(out_dtype) for x in torch.split(ret, lens)])
+
+
+def get_advantages_and_returns(total_len: int, response_len: int, values, rewards, gamma: float, lambd: float):
+    """One response (ppo_utils.py:846-906): ``(advantages.detach(), returns)``."""
+    adv, ret = get_advantages_and_returns_batch([total_len], [response_len], [values], [rewards], gamma, lambd)
+    return adv[0].detach(), ret[0]
+
+
+def vanilla_gae(rewards, values, gamma: float, lambd: float):
+    """``[B, T]`` padded form (ppo_utils.py:1026-1047): every row is one sequence of length T."""
+    b, t = rewards.shape
+    adv, ret = get_advantages_and_returns_batch([t] * b, [t] * b, list(values), list(rewards), gamma, lambd)
+    return torch.stack(adv), torch.stack(ret)
+
+
+def chunked_gae(rewards, values, gamma: float, lambd: float, chunk_size: int = 128):
+    """Same recurrence as :func:`vanilla_gae`; the chunk size has no effect here."""
+    return vanilla_gae(rewards, values, gamma, lambd)
 
 
 def compute_rloo_leave_one_out_rewards(group_rewards):

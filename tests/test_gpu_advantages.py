@@ -338,3 +338,122 @@ def test_opd_kl_topk_argument_checks():
     # identical distributions: zero divergence in every mode
     for kt in ("reverse_kl", "forward_kl", "jsd", "low_var_kl"):
         assert compute_opd_kl(s, s, "jsd" if kt != "low_var_kl" else kt).abs().max().item() < 1e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_reinforce_pp_returns_and_baseline_vs_oracle(dtype):
+    """One-launch REINFORCE++ returns: the reference test's cases, then random ragged sequences (longer than one
+    64-token chunk, fully masked ones, masked NaN/inf) -- bit-exact against the sequential oracle."""
+    from relax_amd.ppo_utils import get_reinforce_plus_plus_baseline_advantages, get_reinforce_plus_plus_returns
+
+    dev = require_gpu()
+    announce("REINFORCE++ returns", dtype)
+    got = get_reinforce_plus_plus_returns(
+        torch.tensor([1.0], dtype=dtype), [torch.tensor([0.5, 12345.0, -0.25], dtype=dtype, device=dev)],
+        [torch.tensor([1.0, 0.0, 1.0], dtype=dtype, device=dev)], [3], [3], 0.1, 0.5)
+    torch.testing.assert_close(got[0].cpu(), torch.tensor([0.20625, 0.0, 1.025], dtype=dtype), atol=1e-6, rtol=1e-6)
+    g = torch.Generator().manual_seed(11)
+    lens = [1, 63, 64, 65, 200, 5, 1000]
+    kls = [torch.randn(n, generator=g, dtype=dtype) for n in lens]
+    masks = [(torch.rand(n, generator=g) > 0.3).to(dtype) for n in lens]
+    masks[5] = torch.zeros(5, dtype=dtype)                     # fully masked sequence
+    kls[4][masks[4] == 0] = float("nan")                       # garbage outside the mask
+    kls[6][masks[6] == 0] = float("inf")
+    rewards = torch.randn(len(lens), generator=g, dtype=dtype)
+    for gamma in (1.0, 0.97):
+        want = A.reinforce_pp_returns(rewards, kls, masks, 0.05, gamma)
+        got = get_reinforce_plus_plus_returns(rewards, [k.to(dev) for k in kls], [m.to(dev) for m in masks], lens, lens,
+                                              0.05, gamma)
+        for a, b, k in zip(got, want, kls):
+            assert a.dtype == dtype and a.shape == k.shape
+            assert torch.equal(a.cpu(), b), (a.cpu() - b).abs().max()
+    base = get_reinforce_plus_plus_baseline_advantages(rewards, [k.to(dev) for k in kls], [m.to(dev) for m in masks])
+    for a, b in zip(base, A.reinforce_pp_baseline_advantages(rewards, kls, masks)):
+        assert torch.equal(a.cpu(), b)
+    with pytest.raises(ValueError, match="same number of responses"):
+        get_reinforce_plus_plus_returns(torch.tensor([0.0, 1.0]), [torch.ones(1, device=dev)], [torch.ones(1, device=dev)],
+                                        [1], [1], 0.1, 1.0)
+    with pytest.raises(ValueError, match="must have the same shape"):
+        get_reinforce_plus_plus_returns(torch.tensor([0.0]), [torch.ones(2, device=dev)], [torch.ones(1, device=dev)],
+                                        [1], [1], 0.1, 1.0)
+    with pytest.raises(ValueError, match="must match"):
+        get_reinforce_plus_plus_baseline_advantages(torch.tensor([1.0]), [torch.ones(2, device=dev)], [torch.ones(1, device=dev)])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_gae_vs_oracle_and_padded_forms(dtype):
+    from relax_amd.ppo_utils import (chunked_gae, get_advantages_and_returns, get_advantages_and_returns_batch,
+                                     vanilla_gae)
+
+    dev = require_gpu()
+    announce("GAE", dtype)
+    g = torch.Generator().manual_seed(5)
+    lens = [3, 2, 64, 65, 257, 1]
+    vals = [torch.randn(n, generator=g, dtype=dtype) for n in lens]
+    rews = [torch.randn(n, generator=g, dtype=dtype) for n in lens]
+    adv, ret = get_advantages_and_returns_batch([n + 3 for n in lens], lens, [v.to(dev) for v in vals],
+                                                [r.to(dev) for r in rews], 0.99, 0.95)
+    for a, r_, v, rw in zip(adv, ret, vals, rews):
+        wa, wr = A.gae(v, rw, 0.99, 0.95)
+        assert a.shape == v.shape and a.dtype == dtype
+        assert torch.equal(a.cpu(), wa) and torch.equal(r_.cpu(), wr)
+    a1, r1 = get_advantages_and_returns(6, 3, vals[0].to(dev), rews[0].to(dev), 0.99, 0.95)
+    assert torch.equal(a1, adv[0]) and torch.equal(r1, ret[0]) and not a1.requires_grad
+    # [B, T] padded forms: rows are independent sequences of length T
+    rw2, v2 = torch.randn(3, 257, generator=g, dtype=dtype), torch.randn(3, 257, generator=g, dtype=dtype)
+    av, rv = vanilla_gae(rw2.to(dev), v2.to(dev), 0.99, 0.95)
+    ac, rc = chunked_gae(rw2.to(dev), v2.to(dev), 0.99, 0.95, chunk_size=32)
+    for i in range(3):
+        wa, wr = A.gae(v2[i], rw2[i], 0.99, 0.95)
+        assert torch.equal(av[i].cpu(), wa) and torch.equal(rv[i].cpu(), wr)
+    assert torch.equal(av, ac) and torch.equal(rv, rc)
+
+
+def test_masked_normalize_and_estimator_dispatch():
+    """distributed_masked_normalize on one rank, and compute_advantages_and_returns for the ppo / REINFORCE++
+    estimators against the oracle's composition of the same pieces."""
+    import relax_amd
+    from relax_amd.distributed_utils import distributed_masked_normalize
+
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(5000, generator=g)
+    m = (torch.rand(5000, generator=g) > 0.4).float()
+    x[m == 0] = float("nan")
+    out, mean, var, cnt = distributed_masked_normalize(x.to(dev), m.to(dev))
+    wo, wm, wv, wc = A.masked_normalize(x, m)
+    assert cnt.item() == wc.item()
+    torch.testing.assert_close(mean.cpu(), wm, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(var.cpu(), wv, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(out.cpu(), wo, atol=2e-6, rtol=2e-6)
+    with pytest.raises(ValueError, match="same shape"):
+        distributed_masked_normalize(x[:3].to(dev), m[:2].to(dev))
+    lens = [4, 70, 9]
+    lps = [torch.randn(n, generator=g) * 0.1 - 1 for n in lens]
+    refs = [lp + 0.05 * torch.randn(n, generator=g) for lp, n in zip(lps, lens)]
+    masks = [(torch.rand(n, generator=g) > 0.2).float() for n in lens]
+    rewards = [0.5, -1.0, 2.0]
+    kl = [lp - rf for lp, rf in zip(lps, refs)]  # k1
+    args = SimpleNamespace(advantage_estimator="reinforce_plus_plus", use_rollout_logprobs=False, kl_coef=0.1,
+                           kl_loss_type="k1", gamma=0.9, lambd=0.95, normalize_advantages=True)
+    data = dict(log_probs=[t.to(dev) for t in lps], ref_log_probs=[t.to(dev) for t in refs], rewards=rewards,
+                loss_masks=[t.to(dev) for t in masks], response_lengths=lens, total_lengths=lens)
+    relax_amd.compute_advantages_and_returns(args, data)
+    want_ret = A.reinforce_pp_returns(torch.tensor(rewards), kl, masks, 0.1, 0.9)
+    for a, b in zip(data["returns"], want_ret):
+        torch.testing.assert_close(a.cpu(), b, atol=1e-6, rtol=1e-6)
+    white, wm, wv, wc = A.masked_normalize(torch.cat(want_ret), torch.cat(masks))
+    torch.testing.assert_close(torch.cat(data["advantages"]).cpu(), white, atol=2e-6, rtol=2e-5)
+    assert data["reinforce_pp_valid_token_count"][0].item() == wc.item() and len(data["reinforce_pp_zero_variance"]) == 3
+    args.advantage_estimator, args.normalize_advantages = "ppo", False
+    vals = [torch.randn(n, generator=g) for n in lens]
+    data = dict(log_probs=[t.to(dev) for t in lps], ref_log_probs=[t.to(dev) for t in refs], rewards=rewards,
+                values=[t.to(dev) for t in vals], loss_masks=[t.to(dev) for t in masks], response_lengths=lens,
+                total_lengths=lens)
+    relax_amd.compute_advantages_and_returns(args, data)
+    for i, n in enumerate(lens):
+        tok_r = -0.1 * kl[i]
+        tok_r[-1] += rewards[i]
+        wa, wr = A.gae(vals[i], tok_r, 0.9, 0.95)
+        torch.testing.assert_close(data["advantages"][i].cpu(), wa, atol=2e-6, rtol=2e-6)
+        torch.testing.assert_close(data["returns"][i].cpu(), wr, atol=2e-6, rtol=2e-6)

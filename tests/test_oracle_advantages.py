@@ -134,6 +134,65 @@ def test_opd_sampled_token_forms_and_tail_bin():
     torch.testing.assert_close(got, (pt * (pt.log() - ps.log())).sum(-1), atol=1e-6, rtol=0)
 
 
+def test_reinforce_pp_returns_reference_cases_by_hand():
+    """The input cases of the reference's own test (tests/utils/training/test_reinforce_plus_plus.py:45-127) with the
+    expected returns worked out by hand."""
+    kls = [torch.tensor([0.2], dtype=torch.float64), torch.tensor([0.1, 9999.0, -0.3], dtype=torch.float64),
+           torch.tensor([0.2, -0.4, 0.7, -8888.0, 0.5], dtype=torch.float64)]
+    masks = [torch.tensor([1.0], dtype=torch.float64), torch.tensor([1.0, 0.0, 1.0], dtype=torch.float64),
+             torch.tensor([1.0, 1.0, 1.0, 0.0, 1.0], dtype=torch.float64)]
+    got = A.reinforce_pp_returns(torch.tensor([1.5, -0.25, 2.0], dtype=torch.float64), kls, masks, 0.2, 1.0)
+    # gamma = 1: reverse cumulative sums of r = -0.2 * kl (valid tokens) with the reward on the last valid token
+    want = [[1.5 - 0.04], [-0.02 + (0.06 - 0.25), 0.0, 0.06 - 0.25],
+            [-0.04 + 0.08 - 0.14 + (2.0 - 0.1), 0.08 - 0.14 + 1.9, -0.14 + 1.9, 0.0, 1.9]]
+    for g, w in zip(got, want):
+        torch.testing.assert_close(g, torch.tensor(w, dtype=torch.float64), atol=1e-12, rtol=0)
+    # discounting, masked garbage in the middle: r = [-0.05, 0, 1.025]
+    got = A.reinforce_pp_returns(torch.tensor([1.0], dtype=torch.float64),
+                                 [torch.tensor([0.5, 12345.0, -0.25], dtype=torch.float64)],
+                                 [torch.tensor([1.0, 0.0, 1.0], dtype=torch.float64)], 0.1, 0.5)
+    torch.testing.assert_close(got[0], torch.tensor([0.20625, 0.0, 1.025], dtype=torch.float64), atol=1e-12, rtol=0)
+    # fully masked NaN / inf -> exact zeros; non-finite values outside the mask never leak
+    got = A.reinforce_pp_returns(torch.tensor([0.0]), [torch.tensor([float("nan"), float("inf")])], [torch.zeros(2)], 0.1, 1.0)
+    assert torch.equal(got[0], torch.zeros(2))
+    got = A.reinforce_pp_returns(torch.tensor([1.0], dtype=torch.float64),
+                                 [torch.tensor([0.5, float("nan"), -0.25, float("inf")], dtype=torch.float64)],
+                                 [torch.tensor([1.0, 0.0, 1.0, 0.0], dtype=torch.float64)], 0.1, 1.0)
+    torch.testing.assert_close(got[0], torch.tensor([-0.05 + 1.025, 0.0, 1.025, 0.0], dtype=torch.float64), atol=1e-12, rtol=0)
+    base = A.reinforce_pp_baseline_advantages(
+        torch.tensor([1.0, -1.0], dtype=torch.float64),
+        [torch.tensor([5.0, 9999.0, -7.0], dtype=torch.float64), torch.tensor([-123.0, float("nan")], dtype=torch.float64)],
+        [torch.tensor([1.0, 0.0, 1.0], dtype=torch.float64), torch.tensor([0.0, 1.0], dtype=torch.float64)])
+    assert base[0].tolist() == [1.0, 0.0, 1.0] and base[1].tolist() == [0.0, -1.0]
+
+
+def test_gae_textbook_sum_and_masked_normalize_moments():
+    torch.manual_seed(0)
+    r, v = torch.randn(37, dtype=torch.float64), torch.randn(37, dtype=torch.float64)
+    gamma, lam = 0.99, 0.95
+    adv, ret = A.gae(v, r, gamma, lam)
+    nxt = torch.cat([v[1:], torch.zeros(1, dtype=torch.float64)])
+    delta = r + gamma * nxt - v
+    want = torch.stack([sum((gamma * lam) ** l * delta[t + l] for l in range(37 - t)) for t in range(37)])
+    torch.testing.assert_close(adv, want, atol=1e-12, rtol=1e-12)
+    torch.testing.assert_close(ret, want + v, atol=1e-12, rtol=1e-12)
+    # lambda = 1, gamma = 1: advantage = reward-to-go minus the value
+    adv, _ = A.gae(v, r, 1.0, 1.0)
+    torch.testing.assert_close(adv, torch.flip(torch.cumsum(torch.flip(r, [0]), 0), [0]) - v, atol=1e-12, rtol=1e-12)
+    x = torch.randn(200)
+    m = (torch.rand(200) > 0.3).float()
+    x[m == 0] = float("nan")
+    out, mean, var, cnt = A.masked_normalize(x, m)
+    sel = x[m != 0].double().numpy()
+    assert cnt.item() == len(sel)
+    np.testing.assert_allclose(mean.item(), sel.mean(), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(var.item(), sel.var(ddof=0), rtol=1e-5)
+    np.testing.assert_allclose(out[m != 0].numpy(), (sel - sel.mean()) / np.sqrt(sel.var(ddof=0)), rtol=2e-5, atol=2e-5)
+    assert (out[m == 0] == 0).all()
+    const, _, var0, _ = A.masked_normalize(torch.full((5,), 3.0), torch.ones(5))
+    assert var0.item() == 0 and (const == 0).all()
+
+
 def test_opd_union_mask_and_jsd_closed_forms():
     """The union path's padding mask: padded entries drop out, the tail bin is cut off with them, and the masked
     result equals the unmasked one on the row's valid prefix; JSD against its textbook definition."""
