@@ -120,6 +120,16 @@ def policy_loss_function(args, batch, logits, reducer, pg_reducer=None):
     """Composition of loss.py:824-1185 (no OPD top-K, no M2PO, no CP).  Returns (loss, metrics dict)."""
     adv = torch.cat(batch["advantages"], dim=0) if isinstance(batch["advantages"], list) else batch["advantages"]
     resp, tot = batch["response_lengths"], batch["total_lengths"]
+    if args.advantage_estimator in ("reinforce_plus_plus", "reinforce_plus_plus_baseline"):
+        # loss.py:804-821, 864-865, 1056-1072: every reduction first selects the valid tokens, so a non-finite value
+        # at a masked position cannot leak through ``NaN * 0``
+        valid = torch.cat([m.reshape(-1) != 0 for m in batch["loss_masks"]], dim=0)
+
+        def _safe(inner):
+            return lambda values: inner(torch.where(valid, values, torch.zeros_like(values)))
+
+        reducer = _safe(reducer)
+        pg_reducer = _safe(pg_reducer) if pg_reducer is not None else None
     _, out = get_log_probs_and_entropy(
         logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=tot, response_lengths=resp,
         with_entropy=True,

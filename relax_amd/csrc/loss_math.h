@@ -194,6 +194,17 @@ __device__ __forceinline__ TokenResult token_terms(const relax_amd_policy_loss_a
     o.metric[RELAX_AMD_M_MISMATCH_K3] = (tis - log_ratio - 1.0f) * m;
   }
   o.metric[RELAX_AMD_M_OPSM_CLIPFRAC] = drop;
+  if (m == 0.f && mp == 0.f) {
+    // A fully masked token is selected out rather than multiplied by its zero mask, so a non-finite value sitting at
+    // a padded position cannot reach any sum or gradient: the mask-safe reducer the reference wraps around the
+    // REINFORCE++ estimators (loss.py:804-821), applied to every estimator here (finite inputs give the same result).
+#pragma unroll
+    for (int k = 0; k < RELAX_AMD_NUM_METRICS; ++k)
+      if (k != RELAX_AMD_M_OPSM_CLIPFRAC) o.metric[k] = 0.f;
+    o.coef_lp = 0.f;
+    o.coef_ent = 0.f;
+    o.g_seq = 0.f;
+  }
   return o;
 }
 

@@ -252,7 +252,7 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     flat = _check_logits(logits, args)
     dev = flat.device
     est = args.advantage_estimator
-    if est in ("m2po", "reinforce_plus_plus", "reinforce_plus_plus_baseline"):
+    if est == "m2po":
         raise NotImplementedError(f"advantage_estimator {est} is not part of the fused path")
     if getattr(args, "custom_tis_function_path", None) is not None or getattr(args, "custom_pg_loss_reducer_function_path", None) is not None:
         raise NotImplementedError("custom TIS / reducer callables cannot run inside the fused kernel")
@@ -292,7 +292,9 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         loss_mask=masks,
         sample_denom=None if denom is None else denom.to(device=dev, dtype=torch.float32),
         pg_sample_denom=None if pg_denom is None else pg_denom.to(device=dev, dtype=torch.float32),
-        loss_kind={"grpo": "ppo", "ppo": "ppo"}.get(est, est),
+        # REINFORCE++ trains with the PPO-clip surrogate; its mask-safe reduction is what the kernel does anyway
+        loss_kind={"grpo": "ppo", "ppo": "ppo", "reinforce_plus_plus": "ppo",
+                   "reinforce_plus_plus_baseline": "ppo"}.get(est, est),
         kl_kind=args.kl_loss_type if use_kl else None,
         unbiased_kl=bool(getattr(args, "use_unbiased_kl", False)) and use_kl,
         use_opsm=bool(getattr(args, "use_opsm", False)),

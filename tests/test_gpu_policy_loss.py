@@ -65,6 +65,9 @@ CASES = {
     "true_on_policy": dict(true_on_policy_mode=True),
     "use_rollout_logprobs": dict(use_rollout_logprobs=True),
     "temperature": dict(rollout_temperature=0.7, entropy_coef=0.01),
+    "reinforce_pp": dict(advantage_estimator="reinforce_plus_plus"),
+    "reinforce_pp_baseline_k2": dict(advantage_estimator="reinforce_plus_plus_baseline", use_kl_loss=True,
+                                     kl_loss_coef=0.1, kl_loss_type="k2"),
 }
 
 
@@ -97,6 +100,39 @@ def test_policy_loss_function_vs_oracle(name, dtype, tol, single_pass):
         assert abs(met[k].item() - float(w)) < tol * max(1.0, abs(float(w))), (k, met[k].item(), float(w))
     assert set(met) == set(want_m)
     torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, atol=tol, rtol=BF16_ULP if dtype == torch.bfloat16 else 0)
+
+
+@pytest.mark.parametrize("single_pass", ["auto", "off"])
+def test_reinforce_pp_masked_nonfinite_values_do_not_leak(single_pass):
+    """REINFORCE++ reduces with a mask-safe reducer: NaN / inf advantages and old log-probs at masked tokens leave the
+    loss, every metric and the gradient finite and equal to the oracle's."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("reinforce++ mask-safe", single_pass)
+    tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 264
+    logits, batch = _make_batch(23, tot, resp, v)
+    for key, bad in (("advantages", float("nan")), ("log_probs", float("inf")), ("ref_log_probs", float("nan"))):
+        batch[key] = [torch.where(m != 0, x, torch.full_like(x, bad)) for x, m in zip(batch[key], batch["loss_masks"])]
+    args = P.make_args(relax_amd_single_pass=single_pass, advantage_estimator="reinforce_plus_plus", use_kl_loss=True,
+                       kl_loss_coef=0.1, kl_loss_type="k2")
+    lo = logits.clone().requires_grad_()
+    want_loss, want_m = P.policy_loss_function(args, dict(batch), lo, R.make_reducer(resp, batch["loss_masks"]))
+    want_loss.backward()
+    assert torch.isfinite(want_loss)
+    # autograd still carries 0 * NaN into the logits rows of the masked tokens (the selected-out branch has a NaN local
+    # derivative); the kernel writes exact zeros there, which is what a finite optimiser step needs
+    clean = torch.isfinite(lo.grad[0]).all(-1)
+    assert not clean.all() and clean.any()
+    lg = logits.to(dev).requires_grad_()
+    loss, met = relax_amd.policy_loss_function(args, _to_dev(batch, dev), lg, None)
+    loss.backward()
+    assert abs(loss.item() - want_loss.item()) < 3e-5
+    for k, w in want_m.items():
+        assert abs(met[k].item() - float(w)) < 3e-5 * max(1.0, abs(float(w))), (k, met[k].item(), float(w))
+    got = lg.grad[0].cpu()
+    assert torch.isfinite(got).all() and (got[~clean] == 0).all()
+    torch.testing.assert_close(got[clean], lo.grad[0][clean], atol=3e-5, rtol=0)
 
 
 @pytest.mark.parametrize("v,dtype", [(151936, torch.bfloat16), (32000, torch.float32), (4096, torch.float16),
