@@ -5,6 +5,8 @@ Tolerances follow the reference's own chunked-LM-head test for bf16 operands
 (+ one bf16 ulp of output rounding for the bf16 gradients).
 """
 
+import math
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -115,3 +117,38 @@ def test_argument_errors():
     torch.testing.assert_close(lp, want, atol=2e-3, rtol=0)
     with pytest.raises(TypeError, match="bfloat16"):
         lm_head_log_probs_and_entropy(hid.float(), w, tok)
+
+
+def test_full_size_forward_and_gradient_properties():
+    """The benchmark shape (hidden [32768, 4096] x weight [151936, 4096]): sampled rows against a library fp32
+    matmul + log_softmax, range properties for every row, and gradient identities that hold at any size --
+    sum_v dlogits = 0 makes dhidden orthogonal to nothing in particular, but the weight gradient of a constant shift is
+    zero: sum_v dweight[v, :] = sum_n dlogits_rowsum[n] * hidden[n, :] = 0."""
+    from relax_amd.lm_head import lm_head_log_probs_and_entropy
+
+    dev = require_gpu()
+    n, h, v = 32768, 4096, 151936
+    announce("lmhead full size", n, h, v)
+    g = torch.Generator(device=dev).manual_seed(0)
+    hid = torch.randn(n, h, device=dev, generator=g).bfloat16().requires_grad_()
+    w = (torch.randn(v, h, device=dev, generator=g) * 0.02).bfloat16().requires_grad_()
+    tok = torch.randint(0, v, (n,), device=dev, generator=g)
+    lp, ent = lm_head_log_probs_and_entropy(hid, w, tok, 1.0, True, False)
+    assert torch.isfinite(lp).all() and (lp <= 0).all()
+    assert (ent >= 0).all() and (ent <= math.log(v) + 1e-3).all()
+    idx = torch.arange(0, n, n // 64, device=dev)
+    ref = torch.log_softmax(hid.detach()[idx].float() @ w.detach().float().t(), -1)
+    torch.testing.assert_close(lp.detach()[idx], ref[torch.arange(idx.numel(), device=dev), tok[idx]], atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent[idx], -(ref.exp() * ref).sum(-1), atol=2e-3, rtol=0)
+    del ref
+    adv = torch.randn(n, device=dev, generator=g) / n
+    (-(adv * lp)).sum().backward()
+    assert torch.isfinite(hid.grad).all() and torch.isfinite(w.grad).all()
+    # a uniform shift of every logit changes no log-prob: the weight gradient summed over the vocabulary vanishes
+    col = w.grad.float().sum(0)
+    assert col.abs().max().item() < 2e-3 * max(1.0, w.grad.float().abs().sum(0).max().item())
+    # sampled rows of dhidden against the closed form  dh_n = -adv_n * (w[tok_n] - sum_v p_v w_v)
+    pick = idx[:8]
+    p = torch.softmax(hid.detach()[pick].float() @ w.detach().float().t(), -1)
+    want = -adv[pick, None] * (w.detach()[tok[pick]].float() - p @ w.detach().float())
+    torch.testing.assert_close(hid.grad[pick].float(), want, atol=2e-3 * want.abs().max().item(), rtol=2 * BF16_ULP)

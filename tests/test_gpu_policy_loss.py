@@ -350,3 +350,70 @@ def test_reducers_vs_oracle_literals(literals):
     red = cp_utils.get_sum_of_sample_mean([4], [4], m, calculate_per_token_loss=True)
     assert red(torch.tensor(fx["values"], device=dev)).item() == fx["token_sum"]
     assert cp_utils.get_cp_local_num_tokens([4], [4], m).item() == fx["count"]
+
+
+def test_full_size_packed_varlen_gspo_and_cispo_properties():
+    """Packed variable-length batch at the benchmark's vocabulary (8 sequences, 2k-6k tokens here to bound the test's
+    memory; the kernels are per-row): sequence-level GSPO through the two-launch path and token-level CISPO through the
+    fused launch.  Checks that hold at any size: finite loss, every dlogits row sums to ~0, masked rows are exactly
+    zero, the CISPO loss is identical bit for bit on both paths, and GSPO's per-sequence ratio really is shared by the
+    sequence (scaling one token's old log-prob moves every gradient row of that sequence, and no other)."""
+    import relax_amd
+
+    dev = require_gpu()
+    v = 151936
+    cpu = torch.Generator().manual_seed(0)
+    lengths = [int(x) for x in torch.randint(2048, 6145, (8,), generator=cpu)]
+    n = sum(lengths)
+    announce("varlen full vocab", lengths)
+    g = torch.Generator(device=dev).manual_seed(0)
+    logits = (torch.randn((1, n, v), device=dev, generator=g) * 3.0).to(torch.bfloat16)
+    masks = []
+    for ln in lengths:
+        m = torch.ones(ln)
+        for _ in range(4):
+            w = int(0.075 * ln)
+            st = int(torch.randint(0, ln - w, (1,), generator=cpu))
+            m[st:st + w] = 0.0
+        masks.append(m.to(dev))
+    toks = [torch.randint(0, v, (ln,), device=dev, generator=g) for ln in lengths]
+    adv = torch.rand(8, generator=cpu) - 0.5
+    batch = dict(unconcat_tokens=toks, total_lengths=lengths, response_lengths=lengths, loss_masks=masks,
+                 advantages=[adv[i].to(dev).expand(ln).contiguous() for i, ln in enumerate(lengths)],
+                 relax_amd_sample_denominators=torch.full((8,), 8.0, device=dev))
+    base = P.make_args()
+    with torch.no_grad():
+        _, out = relax_amd.get_log_probs_and_entropy(logits, args=base, unconcat_tokens=toks, total_lengths=lengths,
+                                                     response_lengths=lengths, with_entropy=False)
+    batch["log_probs"] = [lp + 0.02 * torch.randn(lp.shape, device=dev, generator=g) for lp in out["log_probs"]]
+    flat_mask = torch.cat(masks)
+    results = {}
+    for name, kw in (("gspo", dict(advantage_estimator="gspo", eps_clip=3e-4, eps_clip_high=4e-4)),
+                     ("cispo", dict(advantage_estimator="cispo", eps_clip=0.2, eps_clip_high=0.28)),
+                     ("cispo_two_launch", dict(advantage_estimator="cispo", eps_clip=0.2, eps_clip_high=0.28,
+                                               relax_amd_single_pass="off"))):
+        lg = logits.clone().requires_grad_()
+        loss, met = relax_amd.policy_loss_function(P.make_args(**kw), batch, lg, None)
+        loss.backward()
+        assert torch.isfinite(loss) and all(torch.isfinite(x) for x in met.values())
+        d = lg.grad[0]
+        assert d.float().sum(-1).abs().max().item() < 2e-2
+        assert (d[flat_mask == 0] == 0).all()
+        results[name] = (loss.item(), d)
+    assert results["cispo"][0] == results["cispo_two_launch"][0]
+    torch.testing.assert_close(results["cispo"][1].float(), results["cispo_two_launch"][1].float(), atol=1e-6,
+                               rtol=2 * BF16_ULP)
+    # GSPO: perturb one token's old log-prob in sequence 3; only that sequence's gradient rows may change
+    lo = [x.clone() for x in batch["log_probs"]]
+    first_valid = int(torch.nonzero(masks[3])[0])
+    lo[3][first_valid] += 0.5
+    lg = logits.clone().requires_grad_()
+    loss2, _ = relax_amd.policy_loss_function(P.make_args(advantage_estimator="gspo", eps_clip=3e-4, eps_clip_high=4e-4),
+                                              dict(batch, log_probs=lo), lg, None)
+    loss2.backward()
+    changed = (lg.grad[0] != results["gspo"][1]).any(-1)
+    start = sum(lengths[:3])
+    inside = torch.zeros(n, dtype=torch.bool, device=dev)
+    inside[start:start + lengths[3]] = True
+    assert not changed[~inside].any()
+    assert changed[inside & (flat_mask != 0)].float().mean().item() > 0.99
