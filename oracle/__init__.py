@@ -37,7 +37,7 @@ live in ``tests/test_oracle_*.py``):
   the oracle code (explicit python loops / fp64 autograd / ``scipy``-style
   textbook formulas).  The exact edge conventions the closed forms do not fix
   (CISPO ``A == 0`` branch, whiten Bessel switch at n < 2) are taken from
-  reading the reference source; see DESIGN notes in each docstring.
+  reading the reference source; each docstring says which.
 * ``advantages.reinforce_pp_returns`` / ``reinforce_pp_baseline_advantages``: the input cases of
   tests/utils/training/test_reinforce_plus_plus.py:45-167 with expectations worked out by hand
   (gamma = 1 reverse cumulative sums; the gamma = 0.5 case [0.20625, 0, 1.025]; masked NaN/inf).
