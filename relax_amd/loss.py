@@ -143,8 +143,6 @@ def get_log_probs_and_entropy(
     """One packed launch over every response token; returns ``(empty, {"log_probs": [...], "entropy": [...]})``
     with per-sample ``[R_i]`` fp32 views, differentiable w.r.t. ``logits``."""
     assert non_loss_data
-    if with_topk or gather_topk_token_ids is not None:
-        raise NotImplementedError("top-K outputs are not part of the fused path")
     if lm_head_forward is not None:
         raise NotImplementedError("pass hidden states and the weight to relax_amd.lm_head instead of a callable")
     flat = _check_logits(logits, args)
@@ -162,7 +160,48 @@ def get_log_probs_and_entropy(
     res = {"log_probs": lay.split(lp)}
     if with_entropy:
         res["entropy"] = lay.split(ent)
+    if with_topk:
+        # diagnostic student-side top-K ids (loss.py:436-438): a library selection over each sample's own rows
+        k = topk_k if topk_k is not None else getattr(args, "opd_log_prob_top_k", 1)
+        k = min(max(int(k), 1), int(flat.size(-1)))
+        begins, _ = response_row_begins(total_lengths, response_lengths)
+        res["topk_token_ids"] = [torch.topk(flat[b:b + r], k=k, dim=-1).indices
+                                 for b, r in zip(begins, lay.response_lengths)]
+    if gather_topk_token_ids is not None:
+        res["topk_log_probs"] = _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t)
     return torch.empty((0,), device=logits.device), res
+
+
+def _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t):
+    """Per-sample ``[R_i, K_i]`` log-probs at the given vocabulary ids (compute_opd_topk_log_probs,
+    relax/utils/opd/opd_utils.py:1005-1019) in one packed launch: samples with fewer ids (the union path) are padded
+    with the -1 sentinel, which yields -inf and no gradient, and trimmed again afterwards."""
+    from .opd_utils import TopKLogProbs
+
+    dev = flat.device
+    per_sample, widths = [], []
+    for i, r in enumerate(lay.response_lengths):
+        ids = gather_topk_token_ids[i] if i < len(gather_topk_token_ids) else None
+        if ids is None or ids.numel() == 0:
+            per_sample.append(None)
+            widths.append(0)
+            continue
+        if ids.dim() != 2 or ids.size(0) != r:
+            raise ValueError(f"top-K ids of sample {i} must be [{r}, K], got {tuple(ids.shape)}")
+        per_sample.append(ids.to(device=dev, dtype=torch.long))
+        widths.append(int(ids.size(1)))
+    k_max = max(widths) if widths else 0
+    if k_max == 0 or lay.n_tokens == 0:
+        return [flat.new_zeros((r, 0)) for r in lay.response_lengths]
+    packed = torch.full((lay.n_tokens, k_max), -1, dtype=torch.long, device=dev)
+    pos = 0
+    for ids, r, w in zip(per_sample, lay.response_lengths, widths):
+        if w:
+            packed[pos:pos + r, :w] = ids
+        pos += r
+    out = TopKLogProbs.apply(flat, packed, inv_t, None, lay.row_ids, lay.token_of_row)
+    pieces = torch.split(out, lay.response_lengths)
+    return [p[:, :w] if w else flat.new_zeros((r, 0)) for p, r, w in zip(pieces, lay.response_lengths, widths)]
 
 
 # ------------------------------------------------------------------------------------------ fused policy loss

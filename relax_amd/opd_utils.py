@@ -25,36 +25,41 @@ def compute_opd_kl_full_vocab(student_logits: torch.Tensor, teacher_logits: torc
 
 
 class TopKLogProbs(torch.autograd.Function):
-    """(logits [N, V], ids int64 [N, K]) -> log-probs [N, K] fp32 at the given vocabulary ids.  Saves the logits
-    reference, the ids and one float per row; the backward writes the dense [N, V] gradient in one streaming pass."""
+    """(logits [T, V], ids int64 [N, K]) -> log-probs [N, K] fp32 at the given vocabulary ids.  ``row_ids`` /
+    ``token_of_row`` (int32, optional) map the N tokens to logits rows and back for the packed response layout; without
+    them token t is row t.  Saves the logits reference, the ids and one float per token; the backward writes the
+    dense [T, V] gradient in one streaming pass."""
 
     @staticmethod
-    def forward(ctx, logits, ids, inv_temperature, lse):
+    def forward(ctx, logits, ids, inv_temperature, lse, row_ids=None, token_of_row=None):
         x = _rows(logits)
         n, k = ids.shape
+        if row_ids is not None and token_of_row is None and logits.requires_grad:
+            raise RuntimeError("row_ids without token_of_row cannot be differentiated")
         out = torch.empty((n, k), dtype=torch.float32, device=x.device)
         lse_out = lse if lse is not None else torch.empty(n, dtype=torch.float32, device=x.device)
-        stride = x.stride(0) if n > 1 else x.size(1)
+        stride = x.stride(0) if x.size(0) > 1 else x.size(1)
         with ops._timed("topk_logprob_fwd"):
-            check(lib.relax_amd_topk_logprob_fwd(_p(x), _code(x), n, x.size(1), stride, None, _p(ids), k,
+            check(lib.relax_amd_topk_logprob_fwd(_p(x), _code(x), n, x.size(1), stride, _p(row_ids), _p(ids), k,
                                                  float(inv_temperature), _p(lse), _p(out),
                                                  None if lse is not None else _p(lse_out), _stream()))
-        ctx.save_for_backward(x, ids, lse_out)
+        ctx.save_for_backward(x, ids, lse_out, token_of_row)
         ctx.inv_temperature = float(inv_temperature)
         ctx.shape = logits.shape
         return out
 
     @staticmethod
     def backward(ctx, g):
-        x, ids, lse = ctx.saved_tensors
+        x, ids, lse, token_of_row = ctx.saved_tensors
         n, k = ids.shape
-        d = torch.empty((n, x.size(1)), dtype=x.dtype, device=x.device)
-        stride = x.stride(0) if n > 1 else x.size(1)
+        d = torch.empty((x.size(0), x.size(1)), dtype=x.dtype, device=x.device)
+        stride = x.stride(0) if x.size(0) > 1 else x.size(1)
         g = _f32(g).reshape(n, k).contiguous()
         with ops._timed("topk_logprob_bwd"):
-            check(lib.relax_amd_topk_logprob_bwd(_p(x), _code(x), n, x.size(1), stride, None, _p(ids), k,
-                                                 ctx.inv_temperature, _p(lse), _p(g), _p(d), d.size(1), _stream()))
-        return d.view(ctx.shape), None, None, None
+            check(lib.relax_amd_topk_logprob_bwd(_p(x), _code(x), x.size(0), x.size(1), stride, _p(token_of_row),
+                                                 _p(ids), k, ctx.inv_temperature, _p(lse), _p(g), _p(d), d.size(1),
+                                                 _stream()))
+        return d.view(ctx.shape), None, None, None, None, None
 
 
 def compute_log_probs_on_topk_token_ids(logits: torch.Tensor, topk_token_ids: torch.Tensor, process_group=None,

@@ -417,3 +417,55 @@ def test_full_size_packed_varlen_gspo_and_cispo_properties():
     inside[start:start + lengths[3]] = True
     assert not changed[~inside].any()
     assert changed[inside & (flat_mask != 0)].float().mean().item() > 0.99
+
+
+def test_get_log_probs_and_entropy_topk_outputs_vs_oracle():
+    """``gather_topk_token_ids`` (per-sample [R_i, K_i] ids, ragged K as on the union path, one sample without ids) and
+    ``with_topk`` through the packed launch: values per sample, and the gradient of a loss that mixes the sampled-token
+    log-probs with the gathered ones."""
+    import relax_amd
+    from oracle import opd as D
+
+    dev = require_gpu()
+    announce("packed top-K outputs")
+    tot, resp, v = [9, 6, 12, 7], [4, 6, 7, 5], 300   # sample 1 is SFT-shaped (response == total)
+    logits, batch = _make_batch(5, tot, resp, v)
+    g = torch.Generator().manual_seed(1)
+    widths = [5, 0, 3, 5]
+    ids = [torch.randint(0, v, (r, w), generator=g) if w else None for r, w in zip(resp, widths)]
+    ids[0][0, 0] = -1
+    up = [torch.randn(r, w, generator=g) for r, w in zip(resp, widths)]
+    args = P.make_args(rollout_temperature=0.8)
+    lo = logits.clone().requires_grad_()
+    want, loss_w = [], 0.0
+    for i, (chunk, targets) in enumerate(P.iter_responses(lo, batch["unconcat_tokens"], tot, resp)):
+        x = chunk / 0.8
+        lp = torch.log_softmax(x, -1).gather(-1, targets[:, None]).squeeze(-1)
+        loss_w = loss_w + lp.sum() * 0.01
+        if ids[i] is None:
+            want.append(torch.zeros(resp[i], 0))
+            continue
+        t = D.log_probs_on_topk_ids(x, ids[i])
+        want.append(t.detach())
+        loss_w = loss_w + (t.masked_fill(ids[i] < 0, 0.0) * up[i]).sum()
+    loss_w.backward()
+    lg = logits.to(dev).requires_grad_()
+    _, out = relax_amd.get_log_probs_and_entropy(
+        lg, args=args, unconcat_tokens=[t.to(dev) for t in batch["unconcat_tokens"]], total_lengths=tot,
+        response_lengths=resp, with_entropy=False, with_topk=True, topk_k=4,
+        gather_topk_token_ids=[None if x is None else x.to(dev) for x in ids])
+    loss = sum(lp.sum() for lp in out["log_probs"]) * 0.01
+    for i, t in enumerate(out["topk_log_probs"]):
+        assert t.shape == (resp[i], widths[i])
+        if widths[i]:
+            fin = ids[i] >= 0
+            torch.testing.assert_close(t.detach().cpu()[fin], want[i][fin], atol=3e-5, rtol=0)
+            loss = loss + (t.masked_fill((ids[i] < 0).to(dev), 0.0) * up[i].to(dev)).sum()
+    assert torch.isinf(out["topk_log_probs"][0][0, 0])
+    loss.backward()
+    torch.testing.assert_close(lg.grad.cpu(), lo.grad, atol=3e-5, rtol=1e-5)
+    for i, (chunk, _) in enumerate(P.iter_responses(logits, batch["unconcat_tokens"], tot, resp)):
+        got = out["topk_token_ids"][i].cpu()
+        assert got.shape == (resp[i], 4)
+        # same top-4 values (ties could permute the ids)
+        torch.testing.assert_close(chunk.gather(-1, got), torch.topk(chunk, 4, dim=-1).values)
