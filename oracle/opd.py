@@ -93,3 +93,46 @@ def reduce_token_mean(values, response_lengths, masks):
     parts = [c * m.to(c.dtype) for c, m in zip(torch.split(values, response_lengths, dim=0), masks, strict=False)]
     den = sum(m.to(values.dtype).sum() for m in masks)
     return torch.cat(parts, dim=0).sum() / torch.clamp_min(den, 1)
+
+
+def policy_opd_loss(args, batch, log_probs, old_log_probs, topk_log_probs):
+    """compute_policy_opd_loss, opd_utils.py:1368-1455: ``opd_loss_coef`` times the masked token mean of the per-token
+    distillation signal -- top-K (per sample, with the union path's length mask) or sampled-token -- after the
+    optional per-token clip and importance-ratio clip.  Returns (loss | None, metrics)."""
+    coef = float(getattr(args, "opd_loss_coef", 0.0))
+    if coef == 0.0:
+        return None, {}
+    kl_type, alpha = args.opd_kl_type, float(args.opd_jsd_alpha)
+    norm = getattr(args, "opd_norm_mode", "tail")
+    clamp = getattr(args, "opd_log_prob_min_clamp", None)
+    sel = args.opd_token_selection
+    teacher_topk = batch.get("opd_topk_teacher_log_probs")
+    if sel in ("student_topk", "teacher_topk", "union"):
+        if not (topk_log_probs and teacher_topk):
+            return None, {}
+        ksz = batch.get("opd_topk_ksz") if sel == "union" else None
+        parts = []
+        for i, s_lp in enumerate(topk_log_probs):
+            t_lp = teacher_topk[i].detach()
+            mask = None
+            if ksz is not None and i < len(ksz) and ksz[i] is not None:
+                mask = torch.arange(t_lp.size(-1)).unsqueeze(0) < ksz[i].unsqueeze(1)
+            parts.append(opd_kl_topk(s_lp, t_lp, kl_type, alpha, norm, clamp, mask))
+        per_token = torch.cat(parts, dim=0).to(log_probs.dtype)
+    else:
+        if batch.get("teacher_log_probs") is None:
+            return None, {}
+        teacher = torch.cat(batch["teacher_log_probs"], dim=0).to(log_probs.dtype).detach()
+        per_token = opd_kl(log_probs, teacher, kl_type, alpha, norm, clamp).to(log_probs.dtype)
+    metrics = {}
+    tau = getattr(args, "opd_per_token_clip", None)
+    if tau is not None:
+        before = per_token
+        per_token = torch.clamp(per_token, max=float(tau))
+        metrics["opd_per_token_clip_frac"] = (before > float(tau)).float().mean().detach()
+    clip = getattr(args, "opd_is_clip", None)
+    if clip is not None:
+        ratio = torch.exp(log_probs.detach() - old_log_probs.detach())
+        per_token = per_token * torch.clamp(ratio, max=float(clip)).to(per_token.dtype)
+        metrics["opd_is_clip_frac"] = (ratio > float(clip)).float().mean().detach()
+    return coef * reduce_token_mean(per_token, batch["response_lengths"], batch["loss_masks"]), metrics

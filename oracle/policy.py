@@ -38,6 +38,14 @@ DEFAULT_ARGS = dict(
     global_batch_size=1,
     loss_type="policy_loss",
     sft_logits_chunk_size=1024,
+    opd_loss_coef=0.0,
+    opd_kl_type="reverse_kl",
+    opd_jsd_alpha=0.5,
+    opd_norm_mode="tail",
+    opd_log_prob_min_clamp=None,
+    opd_token_selection="sampled",
+    opd_per_token_clip=None,
+    opd_is_clip=None,
 )
 
 
@@ -80,13 +88,17 @@ def iter_responses(logits, tokens_list, total_lengths, response_lengths, tempera
         yield chunk, targets
 
 
-def get_log_probs_and_entropy(logits, *, args, unconcat_tokens, total_lengths, response_lengths, with_entropy=False, **_):
-    """loss.py:290-463 without top-K / CP branches."""
+def get_log_probs_and_entropy(logits, *, args, unconcat_tokens, total_lengths, response_lengths, with_entropy=False,
+                              gather_topk_token_ids=None, **_):
+    """loss.py:290-463 without the CP branches; ``gather_topk_token_ids`` adds the per-sample ``topk_log_probs``
+    (:440-441, compute_opd_topk_log_probs)."""
+    from .opd import log_probs_on_topk_ids
+
     want_grad = with_entropy and getattr(args, "entropy_coef", 0.0) != 0  # :373
-    lps, ents = [], []
-    for chunk, targets in iter_responses(
+    lps, ents, topk = [], [], []
+    for i, (chunk, targets) in enumerate(iter_responses(
         logits, unconcat_tokens, total_lengths, response_lengths, args.rollout_temperature
-    ):
+    )):
         lp, ent = calculate_log_probs_and_entropy(
             chunk,
             targets,
@@ -97,9 +109,17 @@ def get_log_probs_and_entropy(logits, *, args, unconcat_tokens, total_lengths, r
         )
         lps.append(lp.squeeze(-1))
         ents.append(ent)
+        if gather_topk_token_ids is not None:
+            ids = gather_topk_token_ids[i] if i < len(gather_topk_token_ids) else None
+            if ids is None or ids.numel() == 0:
+                topk.append(chunk.new_zeros((chunk.size(0), 0)))
+            else:
+                topk.append(log_probs_on_topk_ids(chunk, ids))
     res = {"log_probs": lps}
     if with_entropy:
         res["entropy"] = ents
+    if gather_topk_token_ids is not None:
+        res["topk_log_probs"] = topk
     return torch.empty((0,)), res
 
 
@@ -130,9 +150,11 @@ def policy_loss_function(args, batch, logits, reducer, pg_reducer=None):
 
         reducer = _safe(reducer)
         pg_reducer = _safe(pg_reducer) if pg_reducer is not None else None
+    gather = batch.get("opd_topk_token_ids") if getattr(args, "opd_token_selection", None) in (
+        "student_topk", "teacher_topk", "union") else None  # resolve_opd_gather_topk_token_ids, opd_utils.py:999-1003
     _, out = get_log_probs_and_entropy(
         logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=tot, response_lengths=resp,
-        with_entropy=True,
+        with_entropy=True, gather_topk_token_ids=gather,
     )
     lps = out["log_probs"]
     if args.true_on_policy_mode:
@@ -185,6 +207,11 @@ def policy_loss_function(args, batch, logits, reducer, pg_reducer=None):
         kl = losses.approx_kl(lp, ref, args.kl_loss_type, ratio)
         kl_loss = reducer(kl)
         loss = loss + args.kl_loss_coef * kl_loss
+    from .opd import policy_opd_loss
+
+    opd_loss, opd_metrics = policy_opd_loss(args, batch, lp, old, out.get("topk_log_probs"))  # :1102-1110
+    if opd_loss is not None:
+        loss = loss + opd_loss
     if lp.numel() == 0:
         loss = loss + 0 * logits.sum()
     metrics.update(
@@ -194,6 +221,7 @@ def policy_loss_function(args, batch, logits, reducer, pg_reducer=None):
         pg_clipfrac=pg_clipfrac.detach().clone(),
         ppo_kl=kl_metric.detach().clone(),
     )
+    metrics.update(opd_metrics)
     if batch.get("rollout_log_probs") is not None:  # :1115-1134
         roll = torch.cat(batch["rollout_log_probs"], dim=0)
         if not args.use_rollout_logprobs:

@@ -295,8 +295,6 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         raise NotImplementedError(f"advantage_estimator {est} is not part of the fused path")
     if getattr(args, "custom_tis_function_path", None) is not None or getattr(args, "custom_pg_loss_reducer_function_path", None) is not None:
         raise NotImplementedError("custom TIS / reducer callables cannot run inside the fused kernel")
-    if float(getattr(args, "opd_loss_coef", 0.0) or 0.0) != 0.0:
-        raise NotImplementedError("the OPD loss term is provided by relax_amd.opd_utils, not the fused policy loss")
     response_lengths, total_lengths = batch["response_lengths"], batch["total_lengths"]
     needs_bwd = torch.is_grad_enabled() and logits.requires_grad
     lay = PackedLayout(dev, flat.size(0), batch["unconcat_tokens"], total_lengths, response_lengths, needs_bwd)
@@ -366,8 +364,27 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     def m(name):
         return mvec[_SLOT[name]]
 
+    opd_reported = {}
+    loss_metric = m("loss")
+    if float(getattr(args, "opd_loss_coef", 0.0) or 0.0) != 0.0:
+        # The distillation term (loss.py:1102-1110) needs log-probs that autograd can see, which the fused step keeps
+        # to itself: a second, differentiable log-prob launch (plus the top-K gather) feeds it.
+        from .opd_utils import compute_policy_opd_loss, resolve_opd_gather_topk_token_ids
+
+        _, lpe = get_log_probs_and_entropy(
+            logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=total_lengths,
+            response_lengths=response_lengths, with_entropy=False,
+            gather_topk_token_ids=resolve_opd_gather_topk_token_ids(args, batch))
+        old_for_opd = old if old is not None else lp.detach()
+        opd_loss, opd_reported = compute_policy_opd_loss(
+            args=args, batch=batch, log_probs=torch.cat(lpe["log_probs"]), old_log_probs=old_for_opd,
+            log_probs_and_entropy=lpe)
+        if opd_loss is not None:
+            loss = loss + opd_loss
+            loss_metric = loss.detach().clone()
+
     reported = {
-        "loss": m("loss"),
+        "loss": loss_metric,
         "pg_loss": m("pg_loss"),
         "entropy_loss": m("entropy_loss"),
         "pg_clipfrac": m("pg_clipfrac"),
@@ -381,6 +398,7 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     if mismatch:
         for k in ("ois", "tis", "tis_clipfrac", "tis_abs", "mismatch_kl", "mismatch_k3_kl"):
             reported[k] = m(k)
+    reported.update(opd_reported)
     if kw["use_opsm"]:
         reported["opsm_clipfrac"] = m("opsm_clipfrac")
     return loss, reported

@@ -225,3 +225,59 @@ def opd_loss_full_vocab(batch: dict, student_logits: torch.Tensor, teacher_logit
         kl = compute_opd_kl_full_vocab(student_logits, teacher_logits)
         return reduce_opd_loss(batch, kl), kl
     return _FusedOpdLoss.apply(student_logits, teacher_logits.detach(), mask)
+
+
+def resolve_opd_gather_topk_token_ids(args, batch):
+    """opd_utils.py:999-1003: the ids whose log-probs the forward must gather, for the top-K token selections."""
+    if getattr(args, "opd_token_selection", None) in ("student_topk", "teacher_topk", "union"):
+        return batch.get("opd_topk_token_ids", None)
+    return None
+
+
+def compute_policy_opd_loss(*, args, batch, log_probs, old_log_probs, log_probs_and_entropy):
+    """``opd_loss_coef`` times the masked token mean of the per-token distillation signal (opd_utils.py:1368-1455):
+    top-K (per sample, with the union path's length mask) or sampled-token, after the optional per-token clip and
+    importance-ratio clip.  Returns ``(loss | None, metrics)``; differentiable through ``log_probs`` and the gathered
+    ``topk_log_probs``."""
+    coef = float(getattr(args, "opd_loss_coef", 0.0) or 0.0)
+    if coef == 0.0:
+        return None, {}
+    kl_type = args.opd_kl_type
+    alpha = float(args.opd_jsd_alpha)
+    norm = getattr(args, "opd_norm_mode", "tail")
+    clamp = getattr(args, "opd_log_prob_min_clamp", None)
+    selection = args.opd_token_selection
+    dev = log_probs.device
+    if selection in ("student_topk", "teacher_topk", "union"):
+        student = log_probs_and_entropy.get("topk_log_probs")
+        teacher = batch.get("opd_topk_teacher_log_probs")
+        if not (student and teacher):
+            return None, {}
+        ksz = batch.get("opd_topk_ksz") if selection == "union" else None
+        parts = []
+        for i, s_lp in enumerate(student):
+            t_lp = teacher[i].to(device=dev).detach()
+            mask = None
+            if ksz is not None and i < len(ksz) and ksz[i] is not None:
+                mask = torch.arange(t_lp.size(-1), device=dev).unsqueeze(0) < ksz[i].to(dev).unsqueeze(1)
+            parts.append(compute_opd_kl_topk(s_lp, t_lp, kl_type, alpha, norm, clamp, mask))
+        per_token = torch.cat(parts, dim=0).to(log_probs.dtype)
+    else:
+        if batch.get("teacher_log_probs") is None:
+            return None, {}
+        teacher = torch.cat(batch["teacher_log_probs"], dim=0).to(device=dev, dtype=log_probs.dtype).detach()
+        per_token = compute_opd_kl(log_probs, teacher, kl_type, alpha, norm, clamp).to(log_probs.dtype)
+    reported = {}
+    tau = getattr(args, "opd_per_token_clip", None)
+    if tau is not None:
+        before = per_token
+        per_token = torch.clamp(per_token, max=float(tau))
+        with torch.no_grad():
+            reported["opd_per_token_clip_frac"] = (before > float(tau)).float().mean().clone().detach()
+    clip = getattr(args, "opd_is_clip", None)
+    if clip is not None:
+        ratio = torch.exp(log_probs.detach() - old_log_probs.detach())
+        per_token = per_token * torch.clamp(ratio, max=float(clip)).to(per_token.dtype)
+        with torch.no_grad():
+            reported["opd_is_clip_frac"] = (ratio > float(clip)).float().mean().clone().detach()
+    return coef * reduce_opd_loss(batch, per_token), reported

@@ -469,3 +469,45 @@ def test_get_log_probs_and_entropy_topk_outputs_vs_oracle():
         assert got.shape == (resp[i], 4)
         # same top-4 values (ties could permute the ids)
         torch.testing.assert_close(chunk.gather(-1, got), torch.topk(chunk, 4, dim=-1).values)
+
+
+@pytest.mark.parametrize("case", ["sampled_clips", "student_topk_forward", "union_jsd"])
+@pytest.mark.parametrize("single_pass", ["auto", "off"])
+def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
+    """``opd_loss_coef != 0``: the distillation term (sampled-token or top-K, union mask, per-token and
+    importance-ratio clips) added to the policy loss -- loss, metrics and dlogits against the oracle."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("policy loss + OPD", case, single_pass)
+    tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 264
+    logits, batch = _make_batch(31, tot, resp, v)
+    g = torch.Generator().manual_seed(2)
+    kw = dict(relax_amd_single_pass=single_pass, opd_loss_coef=0.7, use_kl_loss=True, kl_loss_coef=0.01,
+              kl_loss_type="k3")
+    if case == "sampled_clips":
+        kw.update(opd_token_selection="sampled", opd_kl_type="low_var_kl", opd_per_token_clip=0.02, opd_is_clip=1.01)
+        batch["teacher_log_probs"] = [lp + 0.2 * torch.randn(lp.shape, generator=g) for lp in batch["log_probs"]]
+    else:
+        k = 6
+        batch["opd_topk_token_ids"] = [torch.randint(0, v, (r, k), generator=g) for r in resp]
+        batch["opd_topk_teacher_log_probs"] = [torch.log_softmax(torch.randn(r, v, generator=g), -1)[:, :k].contiguous()
+                                               for r in resp]
+        if case == "student_topk_forward":
+            kw.update(opd_token_selection="student_topk", opd_kl_type="forward_kl", opd_norm_mode="tail")
+        else:
+            kw.update(opd_token_selection="union", opd_kl_type="jsd", opd_jsd_alpha=0.4, opd_norm_mode="trunc",
+                      opd_log_prob_min_clamp=-12.0)
+            batch["opd_topk_ksz"] = [torch.randint(1, k + 1, (r,), generator=g) for r in resp]
+    args = P.make_args(**kw)
+    lo = logits.clone().requires_grad_()
+    want_loss, want_m = P.policy_loss_function(args, dict(batch), lo, R.make_reducer(resp, batch["loss_masks"]))
+    want_loss.backward()
+    lg = logits.to(dev).requires_grad_()
+    loss, met = relax_amd.policy_loss_function(args, _to_dev(batch, dev), lg, None)
+    loss.backward()
+    assert abs(loss.item() - want_loss.item()) < 3e-5 * max(1.0, abs(want_loss.item()))
+    assert set(met) == set(want_m), (sorted(met), sorted(want_m))
+    for key, w in want_m.items():
+        assert abs(met[key].item() - float(w)) < 3e-5 * max(1.0, abs(float(w))), (key, met[key].item(), float(w))
+    torch.testing.assert_close(lg.grad.cpu(), lo.grad, atol=3e-5, rtol=1e-5)
