@@ -136,3 +136,34 @@ def policy_opd_loss(args, batch, log_probs, old_log_probs, topk_log_probs):
         per_token = per_token * torch.clamp(ratio, max=float(clip)).to(per_token.dtype)
         metrics["opd_is_clip_frac"] = (ratio > float(clip)).float().mean().detach()
     return coef * reduce_token_mean(per_token, batch["response_lengths"], batch["loss_masks"]), metrics
+
+
+def apply_to_advantages(args, rollout_data, advantages: list) -> None:
+    """apply_opd_to_advantages, opd_utils.py:1275-1351: ``advantages[i] -= opd_kl_coef * signal_i`` in place."""
+    if args.opd_kl_coef == 0.0:
+        return
+    kl_type, alpha = args.opd_kl_type, float(args.opd_jsd_alpha)
+    norm = getattr(args, "opd_norm_mode", "tail")
+    clamp = getattr(args, "opd_log_prob_min_clamp", None)
+    sel = args.opd_token_selection
+    if sel in ("student_topk", "teacher_topk", "union"):
+        student, teacher = rollout_data.get("opd_topk_student_log_probs"), rollout_data.get("opd_topk_teacher_log_probs")
+        if student is None or teacher is None:
+            return
+        ksz = rollout_data.get("opd_topk_ksz") if sel == "union" else None
+        for i, adv in enumerate(advantages):
+            mask = None
+            if ksz is not None and ksz[i] is not None:
+                mask = torch.arange(teacher[i].size(-1)).unsqueeze(0) < ksz[i].unsqueeze(1)
+            term = opd_kl_topk(student[i], teacher[i], kl_type, alpha, norm, clamp, mask).to(student[i].dtype)
+            tau = getattr(args, "opd_per_token_clip", None)
+            if tau is not None:
+                term = torch.clamp(term, max=float(tau))
+            advantages[i] = adv - args.opd_kl_coef * term.detach()
+        return
+    student, teacher = rollout_data.get("rollout_log_probs"), rollout_data.get("teacher_log_probs")
+    if student is None or teacher is None:
+        return
+    for i, adv in enumerate(advantages):
+        term = opd_kl(student[i], teacher[i], kl_type, alpha, norm, clamp).to(student[i].dtype)
+        advantages[i] = adv - args.opd_kl_coef * term.detach()

@@ -451,8 +451,6 @@ def compute_advantages_and_returns(args: Namespace, rollout_data: dict) -> None:
     est = args.advantage_estimator
     if est not in GRPO_FAMILY + ("ppo", "reinforce_plus_plus", "reinforce_plus_plus_baseline"):
         raise NotImplementedError(f"advantage_estimator {est} is not supported. ")
-    if getattr(args, "use_opd", False):
-        raise NotImplementedError("OPD advantage shaping (apply_opd_to_advantages) is outside the fused path")
     xs = log_probs if log_probs is not None else values
     if xs is None:
         return
@@ -490,6 +488,14 @@ def compute_advantages_and_returns(args: Namespace, rollout_data: dict) -> None:
         rw = torch.tensor(rewards, dtype=torch.float32, device=dev)
         advantages = get_reinforce_plus_plus_baseline_advantages(rewards=rw, kl=kl, loss_masks=loss_masks)
         returns = advantages
+    if getattr(args, "use_opd", False):
+        from .opd_utils import apply_opd_to_advantages
+
+        if getattr(args, "opd_only_reward", False):  # pure distillation: drop every non-OPD contribution first
+            advantages = [torch.zeros_like(a) for a in advantages]
+            returns = [torch.zeros_like(r) for r in returns]
+        advantages = list(advantages)
+        apply_opd_to_advantages(args, rollout_data, advantages)
     if getattr(args, "normalize_advantages", False):
         flat = torch.cat(advantages)
         masks = torch.cat(loss_masks).to(dev)

@@ -281,3 +281,44 @@ def compute_policy_opd_loss(*, args, batch, log_probs, old_log_probs, log_probs_
         with torch.no_grad():
             reported["opd_is_clip_frac"] = (ratio > float(clip)).float().mean().clone().detach()
     return coef * reduce_opd_loss(batch, per_token), reported
+
+
+def apply_opd_to_advantages(args, rollout_data, advantages: list) -> None:
+    """``advantages[i] -= opd_kl_coef * per_token_signal`` in place (opd_utils.py:1275-1351): the top-K signal from the
+    rollout's stored student / teacher top-K log-probs (with the union path's length mask and the per-token clip), or
+    the sampled-token signal from ``rollout_log_probs`` / ``teacher_log_probs``."""
+    if args.opd_kl_coef == 0.0:
+        return
+    kl_type = args.opd_kl_type
+    alpha = float(args.opd_jsd_alpha)
+    norm = getattr(args, "opd_norm_mode", "tail")
+    clamp = getattr(args, "opd_log_prob_min_clamp", None)
+    selection = args.opd_token_selection
+    if selection in ("student_topk", "teacher_topk", "union"):
+        student = rollout_data.get("opd_topk_student_log_probs")
+        teacher = rollout_data.get("opd_topk_teacher_log_probs")
+        if student is None or teacher is None:
+            return
+        ksz = rollout_data.get("opd_topk_ksz") if selection == "union" else None
+        tau = getattr(args, "opd_per_token_clip", None)
+        for i, adv in enumerate(advantages):
+            dev = adv.device
+            s_lp = student[i].to(dev) if i < len(student) and isinstance(student[i], torch.Tensor) else None
+            t_lp = teacher[i].to(dev) if i < len(teacher) and isinstance(teacher[i], torch.Tensor) else None
+            if s_lp is None or t_lp is None or s_lp.numel() == 0 or s_lp.shape != t_lp.shape:
+                raise ValueError(f"OPD per-token signal: token_selection={selection} but the required arms are missing.")
+            mask = None
+            if ksz is not None and i < len(ksz) and ksz[i] is not None:
+                mask = torch.arange(t_lp.size(-1), device=dev).unsqueeze(0) < ksz[i].to(dev).unsqueeze(1)
+            term = compute_opd_kl_topk(s_lp, t_lp, kl_type, alpha, norm, clamp, mask).to(s_lp.dtype)
+            if tau is not None:
+                term = torch.clamp(term, max=float(tau))
+            advantages[i] = adv - args.opd_kl_coef * term.detach()
+        return
+    student = rollout_data.get("rollout_log_probs")
+    teacher = rollout_data.get("teacher_log_probs")
+    if student is None or teacher is None:
+        return
+    for i, adv in enumerate(advantages):
+        term = compute_opd_kl(student[i], teacher[i].to(student[i].device), kl_type, alpha, norm, clamp)
+        advantages[i] = adv - args.opd_kl_coef * term.detach().to(student[i].dtype)

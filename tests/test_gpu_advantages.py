@@ -493,3 +493,36 @@ def test_full_size_reverse_kl_properties():
     torch.testing.assert_close(sd.grad.float(), s2.grad.float(), atol=1e-9, rtol=2.0 ** -6)
     same = compute_opd_kl_full_vocab(s[:256], s[:256])
     assert same.abs().max().item() < 1e-5
+
+
+@pytest.mark.parametrize("selection", ["sampled", "union"])
+def test_opd_advantage_shaping_vs_oracle(selection):
+    """compute_advantages_and_returns with ``use_opd``: the per-token distillation signal is subtracted from the GRPO
+    advantages (and replaces them entirely with ``opd_only_reward``)."""
+    import relax_amd
+
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(9)
+    lens, k = [5, 8, 3], 6
+    lps = [torch.randn(n, generator=g) * 0.1 - 1 for n in lens]
+    data = dict(log_probs=lps, rewards=[0.5, -1.0, 2.0], loss_masks=[torch.ones(n) for n in lens],
+                response_lengths=lens, total_lengths=lens,
+                rollout_log_probs=[lp + 0.01 * torch.randn(n, generator=g) for lp, n in zip(lps, lens)],
+                teacher_log_probs=[lp + 0.3 * torch.randn(n, generator=g) for lp, n in zip(lps, lens)],
+                opd_topk_student_log_probs=[torch.log_softmax(torch.randn(n, 40, generator=g), -1)[:, :k].contiguous() for n in lens],
+                opd_topk_teacher_log_probs=[torch.log_softmax(torch.randn(n, 40, generator=g), -1)[:, :k].contiguous() for n in lens],
+                opd_topk_ksz=[torch.randint(1, k + 1, (n,), generator=g) for n in lens])
+    for only in (False, True):
+        args = SimpleNamespace(advantage_estimator="grpo", use_rollout_logprobs=False, kl_coef=0.0, use_opd=True,
+                               opd_only_reward=only, opd_kl_coef=0.3, opd_kl_type="reverse_kl" if selection == "sampled" else "jsd",
+                               opd_jsd_alpha=0.3, opd_norm_mode="tail", opd_log_prob_min_clamp=None,
+                               opd_token_selection=selection, opd_per_token_clip=0.5, normalize_advantages=False)
+        want = [torch.zeros(n) if only else torch.full((n,), r) for n, r in zip(lens, data["rewards"])]
+        D.apply_to_advantages(args, data, want)
+        dd = {key: ([t.to(dev) for t in val] if isinstance(val, list) and isinstance(val[0], torch.Tensor) else val)
+              for key, val in data.items()}
+        relax_amd.compute_advantages_and_returns(args, dd)
+        for a, b in zip(dd["advantages"], want):
+            torch.testing.assert_close(a.cpu(), b, atol=2e-6, rtol=2e-6)
+        for r_, n, r in zip(dd["returns"], lens, data["rewards"]):
+            assert torch.equal(r_.cpu(), torch.zeros(n) if only else torch.full((n,), r))
