@@ -11,6 +11,8 @@ from .loss import (  # noqa: F401
     get_responses,
     loss_function,
     policy_loss_function,
+    sft_loss_function,
+    sft_loss_function_chunked,
 )
 from .ppo_utils import calculate_log_probs_and_entropy  # noqa: F401
 

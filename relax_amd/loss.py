@@ -144,7 +144,8 @@ def get_log_probs_and_entropy(
     with per-sample ``[R_i]`` fp32 views, differentiable w.r.t. ``logits``."""
     assert non_loss_data
     if lm_head_forward is not None:
-        raise NotImplementedError("pass hidden states and the weight to relax_amd.lm_head instead of a callable")
+        return _deferred_lm_head_log_probs(logits, args, unconcat_tokens, total_lengths, response_lengths,
+                                           with_entropy, lm_head_forward)
     flat = _check_logits(logits, args)
     want_grad = with_entropy and getattr(args, "entropy_coef", 0.0) != 0
     needs_bwd = torch.is_grad_enabled() and logits.requires_grad
@@ -170,6 +171,93 @@ def get_log_probs_and_entropy(
     if gather_topk_token_ids is not None:
         res["topk_log_probs"] = _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t)
     return torch.empty((0,), device=logits.device), res
+
+
+def lm_head_weight_of(lm_head_forward) -> torch.Tensor:
+    """The ``[V, H]`` weight behind a deferred LM head.  The reference hands the loss the captured
+    ``output_layer.forward`` (relax/backends/megatron/model.py:93-181) and calls it per 1024-row sub-chunk; a fused
+    kernel needs the operand itself, which a bound method, a module or a plain tensor all give up."""
+    if isinstance(lm_head_forward, torch.Tensor):
+        return lm_head_forward
+    owner = getattr(lm_head_forward, "__self__", lm_head_forward)
+    weight = getattr(owner, "weight", None)
+    if not isinstance(weight, torch.Tensor) or weight.dim() != 2:
+        raise NotImplementedError(
+            "lm_head_forward must expose the LM-head weight (a bound forward of a module with .weight, the module "
+            "itself, or the weight tensor): an opaque callable cannot be fused")
+    if getattr(owner, "bias", None) is not None:
+        raise NotImplementedError("a deferred LM head with a bias is not supported")
+    return weight
+
+
+def _deferred_lm_head_log_probs(hidden, args, unconcat_tokens, total_lengths, response_lengths, with_entropy,
+                                lm_head_forward):
+    """Deferred-LM-head branch of get_log_probs_and_entropy (loss.py:391-419): ``hidden`` is ``[1, T, H]`` (or
+    ``[T, H]``) and the ``[T, V]`` logits are never formed.  The response rows of all samples go through the fused
+    LM-head kernel in one launch; unlike the reference's chunked path entropy is available as well."""
+    from .lm_head import lm_head_log_probs_and_entropy
+
+    weight = lm_head_weight_of(lm_head_forward)
+    if hidden.dim() == 3:
+        if hidden.size(0) != 1:
+            raise ValueError(f"expected packed hidden states [1, T, H], got {tuple(hidden.shape)}")
+        rows = hidden[0]
+    else:
+        rows = hidden
+    if rows.dim() != 2 or rows.size(1) != weight.size(1):
+        raise ValueError(f"hidden states {tuple(hidden.shape)} do not match the LM-head weight {tuple(weight.shape)}")
+    if not rows.is_cuda:
+        raise RuntimeError("relax_amd kernels need ROCm device tensors (no CPU fallback)")
+    lay = PackedLayout(rows.device, rows.size(0), unconcat_tokens, total_lengths, response_lengths, False)
+    if lay.n_tokens == 0:
+        lp = rows.new_zeros((0,), dtype=torch.float32)
+        ent = lp
+    else:
+        picked = rows.index_select(0, lay.row_ids.to(torch.int64)).to(weight.dtype)  # [N, H]: megabytes, not [N, V]
+        want_grad = with_entropy and getattr(args, "entropy_coef", 0.0) != 0
+        lp, ent = lm_head_log_probs_and_entropy(picked, weight, lay.targets,
+                                                float(getattr(args, "rollout_temperature", 1.0)),
+                                                with_entropy=bool(with_entropy), with_entropy_grad=bool(want_grad))
+    res = {"log_probs": lay.split(lp)}
+    if with_entropy:
+        res["entropy"] = lay.split(ent)
+    return torch.empty((0,), device=hidden.device), res
+
+
+def sft_loss_function_chunked(args: Namespace, batch: dict, hidden_states: torch.Tensor, sum_of_sample_mean=None, *,
+                              lm_head_forward):
+    """SFT loss with the LM head deferred into the loss (loss.py:1386-1428): ``-sum_of_sample_mean(log_probs)`` with
+    the log-probs taken straight from hidden states and the LM-head weight.  ``sum_of_sample_mean`` may be None: the
+    reference's reducer is then rebuilt from the batch."""
+    _, out = get_log_probs_and_entropy(
+        hidden_states, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=batch["total_lengths"],
+        response_lengths=batch["response_lengths"], with_entropy=False, lm_head_forward=lm_head_forward)
+    log_probs = torch.cat(out["log_probs"], dim=0)
+    if sum_of_sample_mean is None:
+        sum_of_sample_mean = get_sum_of_sample_mean(
+            batch["total_lengths"], batch["response_lengths"], batch["loss_masks"],
+            bool(getattr(args, "calculate_per_token_loss", False)), sample_denoms=batch.get("sample_index_mask_sums"))
+    loss = -sum_of_sample_mean(log_probs)
+    if log_probs.numel() == 0:
+        loss = loss + 0 * hidden_states.sum()
+    return loss, {"loss": loss.clone().detach()}
+
+
+def sft_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum_of_sample_mean=None):
+    """Negative log-likelihood of the response tokens (loss.py:1247-1293): ``-sum_of_sample_mean(log_probs)`` from one
+    packed log-prob launch.  ``sum_of_sample_mean`` may be None: the reference's reducer is then rebuilt from the batch."""
+    _, out = get_log_probs_and_entropy(
+        logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=batch["total_lengths"],
+        response_lengths=batch["response_lengths"], with_entropy=False)
+    log_probs = torch.cat(out["log_probs"], dim=0)
+    if sum_of_sample_mean is None:
+        sum_of_sample_mean = get_sum_of_sample_mean(
+            batch["total_lengths"], batch["response_lengths"], batch["loss_masks"],
+            bool(getattr(args, "calculate_per_token_loss", False)), sample_denoms=batch.get("sample_index_mask_sums"))
+    loss = -sum_of_sample_mean(log_probs)
+    if log_probs.numel() == 0:
+        loss = loss + 0 * logits.sum()
+    return loss, {"loss": loss.clone().detach()}
 
 
 def _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t):
@@ -406,13 +494,23 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
 
 def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: torch.Tensor, *, lm_head_forward=None,
                   dp_world_size: int = 1):
-    """Counterpart of loss.py:1443-1620 for ``loss_type == "policy_loss"`` on one GPU: token count, fused loss,
-    Megatron gradient-accumulation scaling, and the ``{"keys", "values"}`` logging dict."""
-    if getattr(args, "loss_type", "policy_loss") != "policy_loss":
-        raise ValueError(f"Unknown loss type: {args.loss_type}") if args.loss_type not in ("value_loss", "sft", "custom_loss") \
-            else NotImplementedError(f"loss type {args.loss_type} is outside the fused policy path")
+    """Counterpart of loss.py:1443-1620 on one GPU: token count, the loss selected by ``args.loss_type``
+    (``policy_loss``; ``sft``, with the LM head deferred into the loss when ``args.sft_chunked_logits`` and an
+    ``lm_head_forward`` are given), Megatron gradient-accumulation scaling, and the ``{"keys", "values"}`` logging
+    dict."""
+    loss_type = getattr(args, "loss_type", "policy_loss")
+    if loss_type not in ("policy_loss", "sft"):
+        raise ValueError(f"Unknown loss type: {loss_type}") if loss_type not in ("value_loss", "custom_loss") \
+            else NotImplementedError(f"loss type {loss_type} is outside the fused policy path")
     num_tokens = get_cp_local_num_tokens(batch["total_lengths"], batch["response_lengths"], batch["loss_masks"])
-    loss, log = policy_loss_function(args, batch, logits, None)
+    if loss_type == "policy_loss":
+        loss, log = policy_loss_function(args, batch, logits, None)
+    elif getattr(args, "task_type", "causal_lm") == "seq_cls":
+        raise NotImplementedError("sequence-classification SFT is outside the fused policy path")
+    elif getattr(args, "sft_chunked_logits", False) and lm_head_forward is not None:
+        loss, log = sft_loss_function_chunked(args, batch, logits, None, lm_head_forward=lm_head_forward)
+    else:
+        loss, log = sft_loss_function(args, batch, logits, None)
     per_token = bool(getattr(args, "calculate_per_token_loss", False))
     is_dummy = batch.get("__is_dummy__", False)
     explicit = batch.get("__loss_scale__", None)

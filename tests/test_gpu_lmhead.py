@@ -152,3 +152,59 @@ def test_full_size_forward_and_gradient_properties():
     p = torch.softmax(hid.detach()[pick].float() @ w.detach().float().t(), -1)
     want = -adv[pick, None] * (w.detach()[tok[pick]].float() - p @ w.detach().float())
     torch.testing.assert_close(hid.grad[pick].float(), want, atol=2e-3 * want.abs().max().item(), rtol=2 * BF16_ULP)
+
+
+def test_sft_losses_plain_and_with_deferred_lm_head_vs_oracle():
+    """sft_loss_function on logits and sft_loss_function_chunked on hidden states + LM-head weight (handed over as a
+    module, a bound forward or the tensor) against the oracle's F.linear -> log-softmax -> sample-mean composition,
+    forward and gradients; loss_function dispatch for ``loss_type="sft"``."""
+    import relax_amd
+    from oracle import reducers as R
+
+    dev = require_gpu()
+    announce("sft losses")
+    g = torch.Generator().manual_seed(4)
+    tot, resp, h, v = [7, 12, 5], [7, 5, 5], 128, 300     # SFT-shaped and RL-shaped samples mixed
+    t = sum(tot)
+    hid = torch.randn(1, t, h, generator=g).bfloat16()
+    head = torch.nn.Linear(h, v, bias=False)
+    with torch.no_grad():
+        head.weight.copy_(torch.randn(v, h, generator=g) * 0.1)
+    head = head.bfloat16()
+    toks = [torch.randint(0, v, (n,), generator=g) for n in tot]
+    masks = [(torch.rand(r, generator=g) > 0.2).float() for r in resp]
+    batch = dict(unconcat_tokens=toks, total_lengths=tot, response_lengths=resp, loss_masks=masks)
+    args = P.make_args(loss_type="sft", sft_chunked_logits=True, rollout_temperature=0.9, global_batch_size=3)
+    # oracle: materialised logits in the weight dtype, fp32 log-softmax, sample mean
+    hc, wc = hid.clone().requires_grad_(), head.weight.detach().clone().requires_grad_()
+    lps = []
+    for (b, e, _), tk, r in zip(P.response_row_ranges(tot, resp), toks, resp):
+        tg = F.pad(tk[1:], (0, 1), value=0) if r == tk.numel() else tk[-r:]
+        lps.append(P.lm_head_log_probs(hc[0, b:e], wc, tg, temperature=0.9, sub_chunk=4))
+    want = -R.make_reducer(resp, masks)(torch.cat(lps))
+    want.backward()
+    dbatch = dict(unconcat_tokens=[x.to(dev) for x in toks], total_lengths=tot, response_lengths=resp,
+                  loss_masks=[m.to(dev) for m in masks])
+    dhead = torch.nn.Linear(h, v, bias=False).bfloat16().to(dev)
+    with torch.no_grad():
+        dhead.weight.copy_(head.weight)
+    for handle in (dhead, dhead.forward, dhead.weight):
+        hd = hid.to(dev).requires_grad_()
+        dhead.weight.grad = None
+        loss, log = relax_amd.sft_loss_function_chunked(args, dbatch, hd, None, lm_head_forward=handle)
+        loss.backward()
+        # the oracle rounds the logits to bf16 before the softmax (as F.linear in the weight dtype does); the kernel
+        # keeps fp32 accumulators: 2e-3 per sample mean, three samples summed
+        assert abs(loss.item() - want.item()) < 2e-3 * len(resp) and abs(log["loss"].item() - loss.item()) == 0
+        torch.testing.assert_close(hd.grad.float().cpu(), hc.grad.float(), atol=5e-3, rtol=2 * BF16_ULP)
+        torch.testing.assert_close(dhead.weight.grad.float().cpu(), wc.grad.float(), atol=5e-3, rtol=2 * BF16_ULP)
+    # the same loss from materialised logits
+    logits = (hid[0].to(dev) @ dhead.weight.detach().t()).float().unsqueeze(0).requires_grad_()
+    loss2, _ = relax_amd.sft_loss_function(args, dbatch, logits, None)
+    assert abs(loss2.item() - want.item()) < 2e-3 * len(resp)
+    # loss_function: Megatron scaling (num_microbatches / global_batch_size) and the logging dict
+    hd = hid.to(dev).requires_grad_()
+    scaled, normalizer, logd = relax_amd.loss_function(args, dbatch, 2, hd, lm_head_forward=dhead.forward)
+    assert abs(scaled.item() - want.item() * 2 / 3) < 2e-3 * len(resp) and logd["keys"] == ["loss"] and int(normalizer) == 1
+    with pytest.raises(NotImplementedError, match="expose the LM-head weight"):
+        relax_amd.sft_loss_function_chunked(args, dbatch, hd, None, lm_head_forward=lambda x: x)
