@@ -31,6 +31,7 @@ VOCAB = 151936
 SEQS, SEQ_LEN = 16, 4096
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+PEAK_SCLK_MHZ = 2400.0  # the shader clock the published matrix-core peak is quoted at
 METRIC = "tokens/s fused logprob+entropy+loss fwd+bwd @V=151936 bf16; % HBM/MFMA peak"
 # HBM bytes one actor_step_fused launch moves at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # at the L2 <-> fabric boundary (profiles/actor_step_fused_bf16_v151936_n65536.md): 26 780 743 KiB fetched
@@ -129,6 +130,50 @@ def cpu_baseline(args, rows: int, vocab: int, budget_s: float = 12.0, max_reps: 
     }
 
 
+class ClockSampler:
+    """Samples the shader clock and the board power from sysfs while a timed region runs (a reading every 20 ms from a
+    host thread; no effect on the GPU).  Matrix-core kernels on dense random operands run into the board's power limit
+    and the clock drops well below the 2.4 GHz the published peak assumes, so the bench reports what it saw."""
+
+    def __init__(self):
+        import glob
+        self.sclk = (glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk") or [None])[0]
+        self.power = (glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") or [None])[0]
+        self.samples, self._stop, self._thread = [], False, None
+
+    def _run(self):
+        while not self._stop:
+            try:
+                cur = [ln for ln in open(self.sclk).read().splitlines() if "*" in ln]
+                mhz = float(cur[0].split()[1].lower().replace("mhz", ""))
+                watts = float(open(self.power).read()) / 1e6 if self.power else float("nan")
+                self.samples.append((time.perf_counter(), mhz, watts))
+            except (OSError, ValueError, IndexError):
+                return
+            time.sleep(0.02)
+
+    def __enter__(self):
+        if self.sclk:
+            import threading
+            self._thread = threading.Thread(target=self._run, daemon=True)
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        if self._thread:
+            self._thread.join()
+
+    def summary(self):
+        """Mean over the second half of the region (the clock takes ~0.3 s to settle under load), or None."""
+        if len(self.samples) < 4:
+            return None
+        t0, t1 = self.samples[0][0], self.samples[-1][0]
+        tail = [s for s in self.samples if s[0] >= t0 + 0.5 * (t1 - t0)]
+        return {"sclk_mhz": sum(s[1] for s in tail) / len(tail), "power_w": sum(s[2] for s in tail) / len(tail),
+                "samples": len(tail)}
+
+
 def timed_steps(step, warmup: int, steps: int):
     """``warmup`` untimed steps, then exactly ``steps`` timed ones bracketed by device synchronisation; returns
     (wall seconds, {kernel name: mean HIP-event ms per launch, launches per step}, last step's result)."""
@@ -222,29 +267,45 @@ def run_lmhead(a, dev) -> None:
     tokens = torch.randint(0, v, (n,), device=dev, generator=g)
     adv = torch.randn(n, device=dev, generator=g) / n
 
+    if a.lmhead_operands == "zeros":  # diagnostic: same kernels and addresses, no switching activity in the operands
+        with torch.no_grad():
+            hidden.zero_()
+            weight.zero_()
+
     def step():
         hidden.grad = None
         weight.grad = None
-        lp, ent = lm_head_log_probs_and_entropy(hidden, weight, tokens, 1.0, True, False)
+        if a.forward_only:  # diagnostic: the clock / power samples then belong to the forward kernel alone
+            with torch.no_grad():
+                lp, ent = lm_head_log_probs_and_entropy(hidden, weight, tokens, 1.0, True, False)
+            return -(adv * lp).sum()
+        lp, ent = lm_head_log_probs_and_entropy(hidden, weight, tokens, 1.0, True, False, keep_logits=a.keep_logits)
         loss = -(adv * lp).sum()
         loss.backward()
         return loss
 
-    wall, kernel_ms, launches, loss = timed_steps(step, a.warmup, a.steps)
+    with ClockSampler() as clock:
+        wall, kernel_ms, launches, loss = timed_steps(step, a.warmup, a.steps)
+    clk = clock.summary()
     # the timed forward region holds the target-logit gather, the MFMA kernel and the split combine; the MFMA kernel
     # is > 99 % of it (see the rocprofv3 summary), so its event time stands for lmhead_fwd_kernel
     dom = kernel_ms["lmhead_logprob_fwd"]
     flops = 2.0 * n * h * v
     achieved = flops / (dom * 1e-3) / 1e12
     emit(a, n, wall,
-         f"fused LM-head + log-prob/entropy: hidden bf16 [{n}, {h}], weight bf16 [{v}, {h}], fwd (no logits in HBM) + "
-         f"bwd to dhidden/dweight from a scalar loss",
-         {"rows": n, "hidden": h, "vocab": v, "loss": float(loss.item())},
+         f"fused LM-head + log-prob/entropy: hidden bf16 [{n}, {h}], weight bf16 [{v}, {h}], fwd "
+         + ("(bf16 logits kept for the backward pass)" if a.keep_logits else "(no logits in HBM)")
+         + (" only [diagnostic]" if a.forward_only else " + bwd to dhidden/dweight from a scalar loss")
+         + (" [diagnostic: all-zero operands]" if a.lmhead_operands == "zeros" else ""),
+         {"rows": n, "hidden": h, "vocab": v, "keep_logits": bool(a.keep_logits), "loss": float(loss.item())},
          {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
           "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
           "algorithmic_flops_per_launch": flops, "avg_launch_ms": dom, "kernel_ms": kernel_ms,
           "launches_per_step": launches,
-          "step_TFLOPs_credited_6NHV": 6.0 * n * h * v / (wall / a.steps) / 1e12},
+          "step_TFLOPs_credited_6NHV": 6.0 * n * h * v / (wall / a.steps) / 1e12,
+          # shader clock / board power seen during the timed steps, and the fraction of the peak rescaled to that clock
+          "clock": clk, "frac_at_measured_clock":
+              (achieved / (MFMA_BF16_PEAK_TFLOPS * clk["sclk_mhz"] / PEAK_SCLK_MHZ)) if clk else None},
          None)
 
 
@@ -457,6 +518,13 @@ def main() -> int:
     ap.add_argument("--rows", type=int, default=0, help="token rows of the lmhead / reverse_kl workloads (0 = default)")
     ap.add_argument("--hidden", type=int, default=4096, help="hidden size of the lmhead workload")
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the CPU baseline slab (0 = skip)")
+    ap.add_argument("--keep-logits", action="store_true",
+                    help="lmhead workload: keep a [V, N] bf16 copy of the logits for the backward pass instead of "
+                         "projecting a second time (10 GB at the default size)")
+    ap.add_argument("--forward-only", action="store_true",
+                    help="lmhead workload, diagnostic: time the forward pass alone (clock samples of that kernel only)")
+    ap.add_argument("--lmhead-operands", choices=["random", "zeros"], default="random",
+                    help="lmhead workload, diagnostic: all-zero operands show the kernel without the board power limit")
     ap.add_argument("--two-launch", action="store_true",
                     help="use the separate forward / backward launches (the path GSPO takes) instead of the fused step")
     ap.add_argument("--calibrate-copy", action="store_true",

@@ -376,6 +376,29 @@ int relax_amd_lmhead_dlogits_t(const void* hidden, const void* weight, int dtype
                                const float* g_ent, const float* grad_scale_dev, float inv_temperature, void* d_t,
                                int64_t d_stride, void* stream);
 
+/*
+ * The same forward pass that also keeps the logits: logits_t [vocab, l_stride] bf16 (token contiguous, l_stride >=
+ * n_tokens) receives bf16(hidden @ weight^T), and the softmax statistics and the target logit are taken from those
+ * rounded values -- the reference's own numerics, whose F.linear runs in the weight dtype before .float()
+ * (relax/backends/megatron/loss.py:405-409).  For callers that would rather spend vocab * n_tokens * 2 bytes of HBM
+ * than recompute the projection in the backward pass (the reference's non-deferred path keeps the logits too).
+ */
+int relax_amd_lmhead_logprob_fwd_keep(const void* hidden, const void* weight, int dtype, int64_t n_tokens,
+                                      int64_t hidden_size, int64_t vocab, int64_t h_stride, int64_t w_stride,
+                                      const int64_t* targets, float inv_temperature, void* workspace, float* log_prob,
+                                      float* entropy, float* lse, float* spx, void* logits_t, int64_t l_stride,
+                                      void* stream);
+/*
+ * Backward from kept logits: overwrites logits_t in place with the d_t of relax_amd_lmhead_dlogits_t (same formula,
+ * x = the stored bf16 logit), one read and one write of the slab instead of a second projection
+ * (_VocabParallelLogProbEntropy.backward, ppo_utils.py:591-629, applied to the stored logits).
+ * l_stride must be a multiple of 8 and logits_t 16-byte aligned; columns n_tokens..l_stride-1 are left undefined.
+ */
+int relax_amd_lmhead_dlogits_from_logits_t(void* logits_t, int64_t n_tokens, int64_t vocab, int64_t l_stride,
+                                           const int64_t* targets, const float* lse, const float* spx,
+                                           const float* g_lp, const float* g_ent, const float* grad_scale_dev,
+                                           float inv_temperature, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -310,9 +310,92 @@ __device__ __forceinline__ void lm_absorb_block(const floatx16& blk, int vbase, 
   }
 }
 
+// Writes accumulator blocks, as bf16, into a [vocab, token] matrix (token contiguous).  Addresses are a wave-uniform
+// tile base plus one 32-bit lane offset plus a uniform per-store offset, so the 256 stores of a tile cost one vector add
+// each and no 64-bit lane arithmetic.  Neighbouring lanes hold neighbouring tokens of the same vocabulary rows: with
+// PAIRS an even/odd lane pair swaps one value per two rows and each lane writes two tokens with one 4-byte store, half
+// the store instructions of the 2-byte form (needs an even row stride and a 4-byte aligned matrix).  Tiles that cross
+// the end of the vocabulary or of the tokens take a checked 2-byte path.
+struct LmSlabWriter {
+  uint16_t* matrix;
+  int64_t stride, vocab, n_tokens, tok0;
+  unsigned char* tile;  // element (v0, tok0) of the current tile
+  int64_t v0;
+  uint32_t lane_off, lane_off_pair, stride_b;
+  int wv, wt, lane;
+  bool interior;
+
+  __device__ __forceinline__ void init(uint16_t* m, int64_t stride_, int64_t vocab_, int64_t n_tokens_, int64_t tok0_,
+                                       int wv_, int wt_, int lane_) {
+    matrix = m, stride = stride_, vocab = vocab_, n_tokens = n_tokens_, tok0 = tok0_;
+    wv = wv_, wt = wt_, lane = lane_;
+    stride_b = uint32_t(stride * 2);
+    const uint32_t row = uint32_t(wv * 128 + 4 * (lane >> 5)), col = uint32_t(wt * 128 + (lane & 31));
+    lane_off = row * stride_b + col * 2;
+    lane_off_pair = (row + (lane & 1)) * stride_b + (col & ~1u) * 2;
+  }
+  __device__ __forceinline__ void set_tile(int64_t v0_) {
+    v0 = v0_;
+    tile = reinterpret_cast<unsigned char*>(matrix + v0 * stride + tok0);
+    interior = v0 + kLmTile <= vocab && tok0 + kLmTile <= n_tokens;
+  }
+  // block (i, j) of the wave's 4 x 4 accumulator blocks; d[r] = value of accumulator register r
+  template <bool PAIRS>
+  __device__ __forceinline__ void store(const float (&d)[16], int i, int j) const {
+    using gptr32 = __attribute__((address_space(1))) uint32_t*;
+    using gptr16 = __attribute__((address_space(1))) uint16_t*;
+    if (interior) {
+      uint64_t base = reinterpret_cast<uint64_t>(tile);
+      asm volatile("" : "+s"(base));
+      const uint32_t block_off = uint32_t(i * 32) * stride_b + uint32_t(j * 64);
+      if (PAIRS) {
+        uint32_t lo = lane_off_pair;
+        asm volatile("" : "+v"(lo));
+        const bool odd = lane & 1;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const float send = odd ? d[2 * q] : d[2 * q + 1];
+          // quad_perm [1, 0, 3, 2]: exchange with the neighbouring lane
+          const float recv =
+              __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send), 0xB1, 0xF, 0xF, true));
+          const uint32_t word = odd ? pack_bf16(recv, d[2 * q + 1]) : pack_bf16(d[2 * q], recv);
+          const uint32_t row_even = uint32_t(8 * ((2 * q) >> 2) + ((2 * q) & 3));
+          *(gptr32)(base + uint64_t(lo + (block_off + row_even * stride_b))) = word;
+        }
+      } else {
+        uint32_t lo = lane_off;
+        asm volatile("" : "+v"(lo));
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          const uint32_t pk = pack_bf16(d[r], d[r + 1]);
+          const uint32_t row = uint32_t(8 * (r >> 2) + (r & 3));
+          *(gptr16)(base + uint64_t(lo + (block_off + row * stride_b))) = uint16_t(pk);
+          *(gptr16)(base + uint64_t(lo + (block_off + (row + 1) * stride_b))) = uint16_t(pk >> 16);
+        }
+      }
+    } else {
+      const int64_t tok = tok0 + wt * 128 + j * 32 + (lane & 31);
+      const int64_t vb = v0 + wv * 128 + i * 32 + 4 * (lane >> 5);
+      if (tok < n_tokens) {
+        uint16_t* p = matrix + vb * stride + tok;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = 8 * (r >> 2) + (r & 3);
+          if (vb + row < vocab) p[row * stride] = uint16_t(f32_to_bf16_bits(d[r]));
+        }
+      }
+    }
+  }
+};
+
+// STORE: also writes the logits, rounded to bf16, into l_t [vocab, l_stride] (token contiguous), and takes the softmax
+// statistics from the rounded values (what the reference's bf16 F.linear hands to its fp32 log-softmax), so that a
+// backward pass reading l_t sees exactly the distribution the forward pass normalised.
+template <bool STORE, bool PAIRS>
 __global__ __launch_bounds__(kLmThreads, 1) void lmhead_fwd_kernel(const uint16_t* __restrict__ hidden,
                                                                    const uint16_t* __restrict__ weight, LmGeom g,
-                                                                   float c, float* __restrict__ partial) {
+                                                                   float c, float* __restrict__ partial,
+                                                                   uint16_t* __restrict__ l_t, int64_t l_stride) {
   __shared__ __attribute__((aligned(1024))) unsigned char w0[kLmOperandBytes];
   __shared__ __attribute__((aligned(1024))) unsigned char h0[kLmOperandBytes];
   __shared__ __attribute__((aligned(1024))) unsigned char w1[kLmOperandBytes];
@@ -331,27 +414,35 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_fwd_kernel(const uint16_
   }
   const int vt_begin = split * g.tiles_per_split;
   const int vt_end = min(g.n_tiles, vt_begin + g.tiles_per_split);
+  LmSlabWriter writer;
+  if (STORE) writer.init(l_t, l_stride, g.vocab, g.n_tokens, tok0, wv, wt, lane);
   lm_pipeline(LmLds{w0, h0, w1, h1}, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
     const int limit = int(min<int64_t>(g.vocab - v0, kLmTile));
-    if (limit < kLmTile) {  // ragged last tile: entries past the vocabulary are masked out
+    if (STORE) writer.set_tile(v0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-        {
-          lm_absorb_block<true>(acc[i][j], wv * 128 + i * 32 + 4 * (lane >> 5), limit, c, m[j], s[j], t[j]);
-          __builtin_amdgcn_sched_barrier(0);
+      for (int j = 0; j < 4; ++j) {
+        // one 16-value block at a time: without the barrier all 256 accumulators are copied out of the AGPRs first
+        floatx16 blk = acc[i][j];
+        if (STORE) {
+          float x[16];
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            x[r] = blk[r];
+            x[r + 1] = blk[r + 1];
+            const uint32_t pk = pack_bf16(x[r], x[r + 1]);
+            blk[r] = bf16_lo(pk);
+            blk[r + 1] = bf16_hi(pk);
+          }
+          writer.template store<PAIRS>(x, i, j);
         }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          // one 16-value block at a time: without the barrier all 256 accumulators are copied out of the AGPRs first
-          lm_absorb_block<false>(acc[i][j], 0, 0, c, m[j], s[j], t[j]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-    }
+        if (limit < kLmTile)  // ragged last tile: entries past the vocabulary are masked out
+          lm_absorb_block<true>(blk, wv * 128 + i * 32 + 4 * (lane >> 5), limit, c, m[j], s[j], t[j]);
+        else
+          lm_absorb_block<false>(blk, 0, 0, c, m[j], s[j], t[j]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
   });
   // merge the two lane halves (same tokens, different vocab rows), then the two waves sharing the tokens
   float* red = reinterpret_cast<float*>(smem);  // [2 (wv)][256 tokens][3]
@@ -436,9 +527,76 @@ __global__ __launch_bounds__(256) void lmhead_combine_kernel(const float* __rest
   if (spx_out) spx_out[tok] = spx;
 }
 
+// Target logit read back from the stored bf16 logits (so log_prob uses the very value the statistics saw).
+__global__ __launch_bounds__(256) void lmhead_target_from_logits_kernel(const uint16_t* __restrict__ l_t,
+                                                                        int64_t l_stride, int64_t n_tokens,
+                                                                        int64_t vocab,
+                                                                        const int64_t* __restrict__ targets,
+                                                                        float* __restrict__ x_target) {
+  const int64_t tok = blockIdx.x * 256LL + threadIdx.x;
+  if (tok >= n_tokens) return;
+  const int64_t tg = targets[tok];
+  x_target[tok] = (tg < 0 || tg >= vocab) ? __builtin_nanf("") : bf16_lo(l_t[tg * l_stride + tok]);
+}
+
+// Backward from stored logits: overwrites l_t [vocab, stride] (bf16 logits, token contiguous) with the gradient
+// dT[v, n] = inv_T * ( g_lp*(onehot - p) + g_H * p * (spx - x) ),  p = exp(x - lse)  -- the same expression the
+// recomputing kernel evaluates on its accumulators.  A thread owns eight neighbouring tokens (one 16-byte access per
+// vocabulary row) and keeps their per-token coefficients in registers while it walks `rows_per_block` rows.
+constexpr int kLmInplaceThreads = 256;
+__global__ __launch_bounds__(kLmInplaceThreads) void lmhead_dlogits_inplace_kernel(
+    uint16_t* __restrict__ l_t, int64_t stride, int64_t n_tokens, int64_t vocab, int rows_per_block, float c,
+    float inv_t, const int64_t* __restrict__ targets, const float* __restrict__ lse, const float* __restrict__ spx,
+    const float* __restrict__ g_lp, const float* __restrict__ g_ent, const float* __restrict__ grad_scale_dev) {
+  const int64_t tok8 = (int64_t(blockIdx.x) * kLmInplaceThreads + threadIdx.x) * 8;
+  if (tok8 >= n_tokens) return;
+  const float gs = grad_scale_dev ? *grad_scale_dev : 1.0f;
+  float k0[8], a0[8], a1[8], hot[8];
+  int64_t tg[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int64_t tk = tok8 + k < n_tokens ? tok8 + k : n_tokens - 1;
+    const float glp = g_lp[tk] * gs, gh = g_ent ? g_ent[tk] * gs : 0.f;
+    const float b = gh * inv_t;
+    k0[k] = -lse[tk] * kLog2e;
+    a0[k] = -glp * inv_t + (g_ent ? b * spx[tk] : 0.f);
+    a1[k] = -b * inv_t;
+    hot[k] = glp * inv_t;
+    tg[k] = tok8 + k < n_tokens ? targets[tk] : -1;
+  }
+  const int64_t v_begin = int64_t(blockIdx.y) * rows_per_block;
+  const int64_t v_end = min<int64_t>(vocab, v_begin + rows_per_block);
+  // four rows in flight per thread: the loads of a group are issued before its first store (in place, so the compiler
+  // must not be asked to reorder them itself)
+  for (int64_t v = v_begin; v < v_end; v += 4) {
+    u32x4 raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (v + u < v_end) raw[u] = *reinterpret_cast<const u32x4*>(l_t + (v + u) * stride + tok8);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (v + u >= v_end) break;
+      float x[8], d[8];
+      Row<bf16_t>::unpack(raw[u], x);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        d[k] = fast_exp2(fmaf(x[k], c, k0[k])) * fmaf(x[k], a1[k], a0[k]);
+        if (v + u == tg[k]) d[k] += hot[k];
+      }
+      u32x4 o;
+      o.x = pack_bf16(d[0], d[1]);
+      o.y = pack_bf16(d[2], d[3]);
+      o.z = pack_bf16(d[4], d[5]);
+      o.w = pack_bf16(d[6], d[7]);
+      *reinterpret_cast<u32x4*>(l_t + (v + u) * stride + tok8) = o;
+    }
+  }
+}
+
 // Backward helper: recompute one [chunk, V] slab of logits on the matrix cores and emit, transposed, the bf16
 // gradient w.r.t. the logits  dT[v, n] = inv_T * ( g_lp*(onehot - p) + g_H * p * (spx - x) ),  p = exp(x - lse).
 // dT is [vocab, chunk] (token-contiguous) so a lane's 32 neighbours write one 64-byte segment.
+template <bool PAIRS>
 __global__ __launch_bounds__(kLmThreads, 1) void lmhead_dlogits_kernel(
     const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ weight, LmGeom g, float c, float inv_t,
     const int64_t* __restrict__ targets, const float* __restrict__ lse, const float* __restrict__ spx,
@@ -469,24 +627,24 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_dlogits_kernel(
   }
   const int vt_begin = split * g.tiles_per_split;
   const int vt_end = min(g.n_tiles, vt_begin + g.tiles_per_split);
+  LmSlabWriter writer;
+  writer.init(d_t, d_stride, g.vocab, g.n_tokens, tok0, wv, wt, lane);
   lm_pipeline(LmLds{w0, h0, w1, h1}, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
+    writer.set_tile(v0);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        if (tokj[j] >= g.n_tokens) continue;
         const int64_t vb = v0 + wv * 128 + i * 32 + 4 * (lane >> 5);
         const floatx16 blk = acc[i][j];
+        float d[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int64_t v = vb + 8 * (r >> 2) + (r & 3);
-          if (v < g.vocab) {
-            const float x = blk[r];
-            float d = fast_exp2(fmaf(x, c, k0[j])) * fmaf(x, a1[j], a0[j]);
-            if (v == tg[j]) d += hot[j];
-            d_t[v * d_stride + tokj[j]] = uint16_t(f32_to_bf16_bits(d));
-          }
+          const float x = blk[r];
+          d[r] = fast_exp2(fmaf(x, c, k0[j])) * fmaf(x, a1[j], a0[j]);
+          if (vb + 8 * (r >> 2) + (r & 3) == tg[j]) d[r] += hot[j];
         }
+        writer.template store<PAIRS>(d, i, j);
         __builtin_amdgcn_sched_barrier(0);
       }
   });
@@ -538,17 +696,27 @@ extern "C" int64_t relax_amd_lmhead_workspace_bytes(int64_t n_tokens) {
   return (8 * 3 + 1) * n_tokens * int64_t(sizeof(float));
 }
 
-extern "C" int relax_amd_lmhead_logprob_fwd(const void* hidden, const void* weight, int dtype, int64_t n_tokens,
-                                            int64_t hidden_size, int64_t vocab, int64_t h_stride, int64_t w_stride,
-                                            const int64_t* targets, float inv_temperature, void* workspace,
-                                            float* log_prob, float* entropy, float* lse, float* spx, void* stream) {
-  if (n_tokens == 0) return RELAX_AMD_OK;
+// 4-byte paired stores need an even row stride and a 4-byte aligned base
+static bool lm_pairs_ok(const void* p, int64_t stride) {
+  return stride % 2 == 0 && reinterpret_cast<uintptr_t>(p) % 4 == 0;
+}
+// the slab writer keeps byte offsets inside a 256-row tile in 32 bits
+static int lm_slab_stride_ok(const char* what, int64_t stride) {
+  if (int64_t(kLmTile + 1) * stride * 2 >= (1LL << 31)) {
+    set_error("%s: slab row stride %lld too large", what, (long long)stride);
+    return RELAX_AMD_EUNSUPPORTED;
+  }
+  return RELAX_AMD_OK;
+}
+
+static int lm_forward(const char* what, const void* hidden, const void* weight, int dtype, int64_t n_tokens,
+                      int64_t hidden_size, int64_t vocab, int64_t h_stride, int64_t w_stride, const int64_t* targets,
+                      float inv_temperature, void* workspace, float* log_prob, float* entropy, float* lse, float* spx,
+                      uint16_t* l_t, int64_t l_stride, void* stream) {
   LmGeom g;
-  if (int rc = lm_geometry("lmhead_logprob_fwd", dtype, n_tokens, hidden_size, vocab, h_stride, w_stride, hidden,
-                           weight, g))
-    return rc;
+  if (int rc = lm_geometry(what, dtype, n_tokens, hidden_size, vocab, h_stride, w_stride, hidden, weight, g)) return rc;
   if (!targets || !workspace || !log_prob || !(inv_temperature > 0.f)) {
-    set_error("lmhead_logprob_fwd: NULL argument or non-positive inv_temperature");
+    set_error("%s: NULL argument or non-positive inv_temperature", what);
     return RELAX_AMD_EINVAL;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -556,15 +724,81 @@ extern "C" int relax_amd_lmhead_logprob_fwd(const void* hidden, const void* weig
   float* x_target = partial + 8 * 3 * n_tokens;
   const uint16_t* h = static_cast<const uint16_t*>(hidden);
   const uint16_t* w = static_cast<const uint16_t*>(weight);
-  hipLaunchKernelGGL(lmhead_target_logit_kernel, dim3(unsigned((n_tokens + 3) / 4)), dim3(256), 0, s, h, w, g, targets,
-                     x_target);
-  if (int rc = check_launch("lmhead_target_logit")) return rc;
-  hipLaunchKernelGGL(lmhead_fwd_kernel, dim3(lm_grid(g)), dim3(kLmThreads), 0, s, h, w, g,
-                     inv_temperature * kLog2e, partial);
+  const float c = inv_temperature * kLog2e;
+  const dim3 grid(lm_grid(g)), block(kLmThreads);
+  if (!l_t) {
+    hipLaunchKernelGGL(lmhead_target_logit_kernel, dim3(unsigned((n_tokens + 3) / 4)), dim3(256), 0, s, h, w, g,
+                       targets, x_target);
+    if (int rc = check_launch("lmhead_target_logit")) return rc;
+    hipLaunchKernelGGL((lmhead_fwd_kernel<false, false>), grid, block, 0, s, h, w, g, c, partial, nullptr, int64_t(0));
+  } else if (lm_pairs_ok(l_t, l_stride)) {
+    hipLaunchKernelGGL((lmhead_fwd_kernel<true, true>), grid, block, 0, s, h, w, g, c, partial, l_t, l_stride);
+  } else {
+    hipLaunchKernelGGL((lmhead_fwd_kernel<true, false>), grid, block, 0, s, h, w, g, c, partial, l_t, l_stride);
+  }
   if (int rc = check_launch("lmhead_fwd")) return rc;
+  if (l_t) {
+    hipLaunchKernelGGL(lmhead_target_from_logits_kernel, dim3(unsigned((n_tokens + 255) / 256)), dim3(256), 0, s, l_t,
+                       l_stride, n_tokens, vocab, targets, x_target);
+    if (int rc = check_launch("lmhead_target_from_logits")) return rc;
+  }
   hipLaunchKernelGGL(lmhead_combine_kernel, dim3(unsigned((n_tokens + 255) / 256)), dim3(256), 0, s, partial, x_target,
                      n_tokens, g.splits, inv_temperature, log_prob, entropy, lse, spx);
   return check_launch("lmhead_combine");
+}
+
+extern "C" int relax_amd_lmhead_logprob_fwd(const void* hidden, const void* weight, int dtype, int64_t n_tokens,
+                                            int64_t hidden_size, int64_t vocab, int64_t h_stride, int64_t w_stride,
+                                            const int64_t* targets, float inv_temperature, void* workspace,
+                                            float* log_prob, float* entropy, float* lse, float* spx, void* stream) {
+  if (n_tokens == 0) return RELAX_AMD_OK;
+  return lm_forward("lmhead_logprob_fwd", hidden, weight, dtype, n_tokens, hidden_size, vocab, h_stride, w_stride,
+                    targets, inv_temperature, workspace, log_prob, entropy, lse, spx, nullptr, 0, stream);
+}
+
+extern "C" int relax_amd_lmhead_logprob_fwd_keep(const void* hidden, const void* weight, int dtype, int64_t n_tokens,
+                                                 int64_t hidden_size, int64_t vocab, int64_t h_stride,
+                                                 int64_t w_stride, const int64_t* targets, float inv_temperature,
+                                                 void* workspace, float* log_prob, float* entropy, float* lse,
+                                                 float* spx, void* logits_t, int64_t l_stride, void* stream) {
+  if (n_tokens == 0) return RELAX_AMD_OK;
+  if (!logits_t || l_stride < n_tokens) {
+    set_error("lmhead_logprob_fwd_keep: NULL logits_t or l_stride < n_tokens");
+    return RELAX_AMD_EINVAL;
+  }
+  if (int rc = lm_slab_stride_ok("lmhead_logprob_fwd_keep", l_stride)) return rc;
+  return lm_forward("lmhead_logprob_fwd_keep", hidden, weight, dtype, n_tokens, hidden_size, vocab, h_stride,
+                    w_stride, targets, inv_temperature, workspace, log_prob, entropy, lse, spx,
+                    static_cast<uint16_t*>(logits_t), l_stride, stream);
+}
+
+extern "C" int relax_amd_lmhead_dlogits_from_logits_t(void* logits_t, int64_t n_tokens, int64_t vocab,
+                                                      int64_t l_stride, const int64_t* targets, const float* lse,
+                                                      const float* spx, const float* g_lp, const float* g_ent,
+                                                      const float* grad_scale_dev, float inv_temperature,
+                                                      void* stream) {
+  if (n_tokens == 0 || vocab == 0) return RELAX_AMD_OK;
+  if (n_tokens < 0 || vocab < 0 || !logits_t || !targets || !lse || !g_lp || (g_ent && !spx) ||
+      !(inv_temperature > 0.f)) {
+    set_error("lmhead_dlogits_from_logits_t: NULL argument, negative size or non-positive inv_temperature");
+    return RELAX_AMD_EINVAL;
+  }
+  if (l_stride % 8 != 0 || l_stride < n_tokens || !aligned16(logits_t)) {
+    set_error("lmhead_dlogits_from_logits_t: l_stride must be a multiple of 8 and >= n_tokens, base 16-byte aligned");
+    return RELAX_AMD_EUNSUPPORTED;
+  }
+  constexpr int kRows = 64;
+  const int64_t col_blocks = (n_tokens + 8LL * kLmInplaceThreads - 1) / (8LL * kLmInplaceThreads);
+  const int64_t row_blocks = (vocab + kRows - 1) / kRows;
+  if (row_blocks > 65535 || col_blocks > 2147483647LL) {
+    set_error("lmhead_dlogits_from_logits_t: vocab=%lld too large", (long long)vocab);
+    return RELAX_AMD_EUNSUPPORTED;
+  }
+  hipLaunchKernelGGL(lmhead_dlogits_inplace_kernel, dim3(unsigned(col_blocks), unsigned(row_blocks)),
+                     dim3(kLmInplaceThreads), 0, static_cast<hipStream_t>(stream), static_cast<uint16_t*>(logits_t),
+                     l_stride, n_tokens, vocab, kRows, inv_temperature * kLog2e, inv_temperature, targets, lse, spx,
+                     g_lp, g_ent, grad_scale_dev);
+  return check_launch("lmhead_dlogits_inplace");
 }
 
 extern "C" int relax_amd_lmhead_dlogits_t(const void* hidden, const void* weight, int dtype, int64_t n_tokens,
@@ -581,10 +815,17 @@ extern "C" int relax_amd_lmhead_dlogits_t(const void* hidden, const void* weight
     set_error("lmhead_dlogits_t: NULL argument, short d_stride or non-positive inv_temperature");
     return RELAX_AMD_EINVAL;
   }
+  if (int rc = lm_slab_stride_ok("lmhead_dlogits_t", d_stride)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(lmhead_dlogits_kernel, dim3(lm_grid(g)), dim3(kLmThreads), 0, s,
-                     static_cast<const uint16_t*>(hidden), static_cast<const uint16_t*>(weight), g,
-                     inv_temperature * kLog2e, inv_temperature, targets, lse, spx, g_lp, g_ent, grad_scale_dev,
-                     static_cast<uint16_t*>(d_t), d_stride);
+  if (lm_pairs_ok(d_t, d_stride))
+    hipLaunchKernelGGL(lmhead_dlogits_kernel<true>, dim3(lm_grid(g)), dim3(kLmThreads), 0, s,
+                       static_cast<const uint16_t*>(hidden), static_cast<const uint16_t*>(weight), g,
+                       inv_temperature * kLog2e, inv_temperature, targets, lse, spx, g_lp, g_ent, grad_scale_dev,
+                       static_cast<uint16_t*>(d_t), d_stride);
+  else
+    hipLaunchKernelGGL(lmhead_dlogits_kernel<false>, dim3(lm_grid(g)), dim3(kLmThreads), 0, s,
+                       static_cast<const uint16_t*>(hidden), static_cast<const uint16_t*>(weight), g,
+                       inv_temperature * kLog2e, inv_temperature, targets, lse, spx, g_lp, g_ent, grad_scale_dev,
+                       static_cast<uint16_t*>(d_t), d_stride);
   return check_launch("lmhead_dlogits");
 }

@@ -21,6 +21,11 @@ from .ops import _need_gpu, _p, _stream
 # sized for 288 GB of HBM, so the usual micro-batch is one slab and dweight needs no cross-slab accumulation)
 BACKWARD_SLAB = 32768
 
+# Largest [V, N] bf16 logits slab (bytes) the forward pass may keep for the backward pass when the caller leaves
+# ``keep_logits`` undecided.  0 = never: the logits stay out of HBM and the backward pass projects a second time.
+# Keeping them trades V * N * 2 bytes (10 GB at V = 151936, N = 32768) for one of the four GEMM-sized kernels of a step.
+KEEP_LOGITS_MAX_BYTES = 0
+
 
 def _bf16_rows(t: torch.Tensor, what: str) -> torch.Tensor:
     if t.dim() != 2:
@@ -33,8 +38,10 @@ def _bf16_rows(t: torch.Tensor, what: str) -> torch.Tensor:
     return t
 
 
-def lmhead_logprob_fwd(hidden, weight, targets, inv_temperature: float = 1.0, with_entropy: bool = True):
-    """Returns (log_prob, entropy | None, lse, spx | None), fp32 [N]."""
+def lmhead_logprob_fwd(hidden, weight, targets, inv_temperature: float = 1.0, with_entropy: bool = True,
+                       logits_t=None):
+    """Returns (log_prob, entropy | None, lse, spx | None), fp32 [N].  ``logits_t`` ([V, >= N] bf16, token contiguous),
+    when given, receives the bf16 logits and the statistics are taken from those rounded values."""
     dev = _need_gpu(hidden, weight, targets)
     n, h = hidden.shape
     v = weight.size(0)
@@ -48,10 +55,29 @@ def lmhead_logprob_fwd(hidden, weight, targets, inv_temperature: float = 1.0, wi
         return lp, ent, lse, spx
     ws = torch.empty(lib.relax_amd_lmhead_workspace_bytes(n), dtype=torch.uint8, device=dev)
     with ops._timed("lmhead_logprob_fwd"):
-        check(lib.relax_amd_lmhead_logprob_fwd(_p(hidden), _p(weight), _lib.BF16, n, h, v, hidden.stride(0),
-                                               weight.stride(0), _p(targets), float(inv_temperature), _p(ws), _p(lp),
-                                               _p(ent), _p(lse), _p(spx), _stream()))
+        if logits_t is None:
+            check(lib.relax_amd_lmhead_logprob_fwd(_p(hidden), _p(weight), _lib.BF16, n, h, v, hidden.stride(0),
+                                                   weight.stride(0), _p(targets), float(inv_temperature), _p(ws),
+                                                   _p(lp), _p(ent), _p(lse), _p(spx), _stream()))
+        else:
+            if logits_t.dtype != torch.bfloat16 or logits_t.dim() != 2 or logits_t.size(0) != v \
+                    or logits_t.size(1) < n or logits_t.stride(1) != 1:
+                raise ValueError(f"logits_t must be bf16 [V={v}, >= {n}] with contiguous tokens, "
+                                 f"got {logits_t.dtype} {tuple(logits_t.shape)} strides {logits_t.stride()}")
+            check(lib.relax_amd_lmhead_logprob_fwd_keep(_p(hidden), _p(weight), _lib.BF16, n, h, v, hidden.stride(0),
+                                                        weight.stride(0), _p(targets), float(inv_temperature), _p(ws),
+                                                        _p(lp), _p(ent), _p(lse), _p(spx), _p(logits_t),
+                                                        logits_t.stride(0), _stream()))
     return lp, ent, lse, spx
+
+
+def lmhead_dlogits_from_logits_t(logits_t, n, targets, lse, spx, g_lp, g_ent, inv_temperature: float):
+    """Turns the kept bf16 logits ``[V, >= n]`` into d loss / d logits in place and returns the ``[V, n]`` view."""
+    with ops._timed("lmhead_dlogits_inplace"):
+        check(lib.relax_amd_lmhead_dlogits_from_logits_t(_p(logits_t), n, logits_t.size(0), logits_t.stride(0),
+                                                         _p(targets), _p(lse), _p(spx), _p(g_lp), _p(g_ent), None,
+                                                         float(inv_temperature), _stream()))
+    return logits_t[:, :n]
 
 
 def lmhead_dlogits_t(hidden, weight, targets, lse, spx, g_lp, g_ent, inv_temperature: float, out=None):
@@ -72,16 +98,22 @@ class FusedLMHeadLogProb(torch.autograd.Function):
 
     Backward recomputes the logits slab by slab on the matrix cores, emits d loss / d logits for the slab in bf16
     (never the full [N, V] tensor) and contracts it with the weight (dhidden) and the hidden states (dweight) with
-    plain library GEMMs; dweight is accumulated in fp32 across slabs.
+    plain library GEMMs; dweight is accumulated in fp32 across slabs.  With ``keep_logits`` the forward pass writes
+    the bf16 logits, transposed, into the slab the backward pass needs anyway, and the backward pass turns them into
+    the gradient in place instead of projecting again (one backward pass only: the slab is consumed).
     """
 
     @staticmethod
-    def forward(ctx, hidden, weight, targets, inv_temperature, with_entropy, with_entropy_grad):
+    def forward(ctx, hidden, weight, targets, inv_temperature, with_entropy, with_entropy_grad, keep_logits=False):
         with_entropy_grad = bool(with_entropy and with_entropy_grad)
         hidden, weight = _bf16_rows(hidden, "hidden"), _bf16_rows(weight, "weight")
         if targets.dtype != torch.int64 or not targets.is_contiguous():
             targets = targets.to(torch.int64).contiguous()
-        lp, ent, lse, spx = lmhead_logprob_fwd(hidden, weight, targets, inv_temperature, with_entropy)
+        n, v = hidden.size(0), weight.size(0)
+        ctx.logits_t = None
+        if keep_logits and n > 0 and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]):
+            ctx.logits_t = torch.empty((v, (n + 7) // 8 * 8), dtype=torch.bfloat16, device=hidden.device)
+        lp, ent, lse, spx = lmhead_logprob_fwd(hidden, weight, targets, inv_temperature, with_entropy, ctx.logits_t)
         ctx.save_for_backward(hidden, weight, targets, lse, spx if with_entropy_grad else None)
         ctx.inv_temperature = inv_temperature
         ctx.with_entropy_grad = with_entropy_grad
@@ -106,6 +138,20 @@ class FusedLMHeadLogProb(torch.autograd.Function):
         need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         d_hidden = torch.empty_like(hidden) if need_h else None
         d_weight32 = None
+        if ctx.logits_t is not None:
+            if ctx.logits_t is False:
+                raise RuntimeError("FusedLMHeadLogProb(keep_logits=True) supports one backward pass: the kept logits "
+                                   "were overwritten with their gradient by the first one")
+            d_t = lmhead_dlogits_from_logits_t(ctx.logits_t, n, targets, lse, spx, g_lp, g_ent, ctx.inv_temperature)
+            ctx.logits_t = False
+            if need_h:
+                with ops._timed("lmhead_dhidden_gemm"):
+                    torch.mm(d_t.t(), weight, out=d_hidden)
+            d_weight = None
+            if need_w:
+                with ops._timed("lmhead_dweight_gemm"):
+                    d_weight = torch.mm(d_t, hidden)
+            return d_hidden, d_weight, None, None, None, None, None
         slab = torch.empty((v, min(n, BACKWARD_SLAB)), dtype=torch.bfloat16, device=hidden.device)
         for s in range(0, n, BACKWARD_SLAB):
             e = min(n, s + BACKWARD_SLAB)
@@ -119,17 +165,20 @@ class FusedLMHeadLogProb(torch.autograd.Function):
                 with ops._timed("lmhead_dweight_gemm"):
                     part = torch.mm(d_t, hidden[s:e])
                 if s == 0 and e == n:
-                    return d_hidden, part, None, None, None, None
+                    return d_hidden, part, None, None, None, None, None
                 if d_weight32 is None:
                     d_weight32 = part.to(torch.float32)
                 else:
                     d_weight32.add_(part)
-        return d_hidden, (d_weight32.to(weight.dtype) if need_w else None), None, None, None, None
+        return d_hidden, (d_weight32.to(weight.dtype) if need_w else None), None, None, None, None, None
 
 
 def lm_head_log_probs_and_entropy(hidden, weight, tokens, temperature: float = 1.0, with_entropy: bool = False,
-                                  with_entropy_grad: bool = True):
+                                  with_entropy_grad: bool = True, keep_logits: bool | None = None):
     """``(log_prob [N] fp32, entropy [N] fp32 | None)`` of ``log_softmax(hidden @ weight.T / temperature)``.
+
+    ``keep_logits``: True keeps a ``[V, N]`` bf16 copy of the logits between forward and backward (faster backward,
+    V * N * 2 bytes), False never does, None decides by ``KEEP_LOGITS_MAX_BYTES``.
 
     The kernels consume the hidden size in pairs of 64-wide slices; other sizes are zero-padded here (zeros add nothing to
     the logits, and autograd through the padding returns gradients of the original shapes)."""
@@ -137,6 +186,8 @@ def lm_head_log_probs_and_entropy(hidden, weight, tokens, temperature: float = 1
     if pad:
         hidden = torch.nn.functional.pad(hidden, (0, pad))
         weight = torch.nn.functional.pad(weight, (0, pad))
+    if keep_logits is None:
+        keep_logits = 2 * hidden.size(0) * weight.size(0) <= KEEP_LOGITS_MAX_BYTES
     lp, ent = FusedLMHeadLogProb.apply(hidden, weight, tokens, 1.0 / float(temperature), bool(with_entropy),
-                                       bool(with_entropy_grad))
+                                       bool(with_entropy_grad), bool(keep_logits))
     return lp, (ent if with_entropy else None)

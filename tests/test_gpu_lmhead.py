@@ -43,6 +43,7 @@ def _oracle(hid, w, tok, wl, we, temperature):
     (300, 128, 1000, 0.7),      # ragged tokens and ragged vocabulary
     (1024, 256, 5000, 1.0),     # several vocab tiles and splits
     (70, 4096, 1030, 1.0),      # production hidden size
+    (301, 128, 700, 1.0),       # odd token count: odd slab stride, 2-byte stores in the backward slab
 ])
 def test_forward_backward_vs_oracle(n, h, v, temperature):
     from relax_amd.lm_head import lm_head_log_probs_and_entropy
@@ -67,6 +68,88 @@ def test_forward_backward_vs_oracle(n, h, v, temperature):
     # deterministic
     lp2, _ = lm_head_log_probs_and_entropy(hid.to(dev), w.to(dev), tok.to(dev), temperature, with_entropy=True)
     assert torch.equal(lp2, lp.detach())
+
+
+def _oracle_bf16_logits(hid, w, tok, wl, we, temperature):
+    """The reference's numerics: F.linear in bf16 (logits rounded to bf16), then fp32 log-softmax
+    (relax/backends/megatron/loss.py:405-409); gradients flow through the rounding unchanged."""
+    h32 = hid.float().requires_grad_()
+    w32 = w.float().requires_grad_()
+    raw = F.linear(h32, w32)
+    logits = (raw + (raw.bfloat16().float() - raw).detach()) / temperature
+    ls = torch.log_softmax(logits, -1)
+    lp = ls[torch.arange(hid.size(0)), tok]
+    ent = -(ls.exp() * ls).sum(-1)
+    ((lp * wl).sum() + (ent * we).sum()).backward()
+    return lp.detach(), ent.detach(), h32.grad, w32.grad
+
+
+@pytest.mark.parametrize("n,h,v,temperature", [
+    (256, 64, 256, 1.0),
+    (301, 128, 1000, 0.7),      # ragged vocabulary, odd token count (a half-filled token pair at the end)
+    (1024, 256, 5000, 1.0),
+    (70, 4096, 1030, 1.0),
+])
+def test_keep_logits_forward_backward_vs_bf16_logit_oracle(n, h, v, temperature):
+    from relax_amd.lm_head import lm_head_log_probs_and_entropy
+
+    dev = require_gpu()
+    announce("lmhead keep_logits", n, h, v, temperature)
+    hid, w, tok, g = _inputs(n, h, v, seed=3 * n + v, w_scale=0.3 if h < 1024 else 0.05)
+    wl, we = torch.randn(n, generator=g) / 16, torch.randn(n, generator=g) / 32
+    rlp, rent, rgh, rgw = _oracle_bf16_logits(hid, w, tok, wl, we, temperature)
+    hd, wd = hid.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    lp, ent = lm_head_log_probs_and_entropy(hd, wd, tok.to(dev), temperature, with_entropy=True, keep_logits=True)
+    # a logit whose fp32 value sits on a bf16 rounding boundary may round the other way than on the CPU (different
+    # summation order): one bf16 ulp of that logit, which only shows where it is the target or carries most of the mass
+    close = lambda a, b, tol: ((a - b).abs() <= tol).float().mean().item()
+    assert close(lp.detach().cpu(), rlp, 2e-3) >= 0.995, (lp.detach().cpu() - rlp).abs().max()
+    torch.testing.assert_close(lp.detach().cpu(), rlp, atol=4e-2, rtol=0)
+    torch.testing.assert_close(ent.detach().cpu(), rent, atol=2e-3, rtol=0)
+    loss = (lp * wl.to(dev)).sum() + (ent * we.to(dev)).sum()
+    loss.backward(retain_graph=True)
+    torch.testing.assert_close(hd.grad.float().cpu(), rgh, atol=5e-3, rtol=2 * BF16_ULP)
+    torch.testing.assert_close(wd.grad.float().cpu(), rgw, atol=5e-3, rtol=2 * BF16_ULP)
+    with pytest.raises(RuntimeError, match="one backward pass"):
+        loss.backward()
+
+
+def test_kept_logits_slab_is_the_bf16_projection_and_stride_parity():
+    """The slab the forward pass keeps equals bf16(hidden @ weight^T) transposed; an odd row stride (2-byte stores)
+    and an even one (paired 4-byte stores) give the same bytes; the in-place backward equals the recomputing one
+    evaluated on the same (rounded) logits to one bf16 ulp."""
+    from relax_amd.lm_head import lmhead_dlogits_from_logits_t, lmhead_logprob_fwd
+
+    dev = require_gpu()
+    announce("lmhead kept slab")
+    n, h, v = 333, 256, 777
+    hid, w, tok, g = _inputs(n, h, v, seed=5, w_scale=0.2)
+    hd, wd, td = hid.to(dev), w.to(dev), tok.to(dev)
+    even = torch.full((v, 336), float("nan"), dtype=torch.bfloat16, device=dev)
+    odd = torch.full((v, 335), float("nan"), dtype=torch.bfloat16, device=dev)
+    out_e = lmhead_logprob_fwd(hd, wd, td, 1.0, True, logits_t=even)
+    out_o = lmhead_logprob_fwd(hd, wd, td, 1.0, True, logits_t=odd)
+    assert torch.equal(even[:, :n].view(torch.int16), odd[:, :n].view(torch.int16))
+    assert torch.isnan(even[:, n:]).all() and torch.isnan(odd[:, n:]).all()  # padding columns untouched
+    for a, b in zip(out_e, out_o):
+        assert torch.equal(a, b)
+    ref = F.linear(hid.float(), w.float())
+    got = even[:, :n].t().float().cpu()
+    assert ((got - ref).abs() <= ref.abs() * 2.0 ** -8 + 1e-5).all()  # half a bf16 ulp + fp32 summation order
+    assert (got == ref.bfloat16().float()).float().mean() > 0.999
+    # statistics of the rounded logits
+    lp, ent, lse, spx = out_e
+    ls = torch.log_softmax(got, -1)
+    torch.testing.assert_close(lp.cpu(), ls[torch.arange(n), tok], atol=1e-4, rtol=0)
+    torch.testing.assert_close(ent.cpu(), -(ls.exp() * ls).sum(-1), atol=1e-4, rtol=0)
+    # in-place gradient against the closed form on the stored logits
+    g_lp = (torch.randn(n, generator=g) / 8).to(dev)
+    g_ent = (torch.randn(n, generator=g) / 8).to(dev)
+    d_t = lmhead_dlogits_from_logits_t(even, n, td, lse, spx, g_lp, g_ent, 1.0)
+    p = ls.exp()
+    onehot = F.one_hot(tok, v).float()
+    want = g_lp.cpu()[:, None] * (onehot - p) + g_ent.cpu()[:, None] * p * ((p * got).sum(-1, keepdim=True) - got)
+    torch.testing.assert_close(d_t.t().float().cpu(), want, atol=1e-5, rtol=2 * BF16_ULP)
 
 
 def test_reference_shaped_case_temperature_and_labels():
