@@ -399,6 +399,15 @@ int relax_amd_lmhead_dlogits_from_logits_t(void* logits_t, int64_t n_tokens, int
                                            const float* g_lp, const float* g_ent, const float* grad_scale_dev,
                                            float inv_temperature, void* stream);
 
+/*
+ * out[c, r] = in[r, c] for 16-bit elements (bf16 / fp16), row strides in elements.  The layout change
+ * `x.t().contiguous()` makes; the LM-head backward uses it to give the library GEMMs of dhidden / dweight
+ * contraction-contiguous operands (autograd of F.linear in relax/backends/megatron/loss.py:405 leaves the choice of
+ * layout to the BLAS library).  16-byte accesses when the strides are multiples of 8 and the bases 16-byte aligned.
+ */
+int relax_amd_transpose_16bit(const void* in, int64_t rows, int64_t cols, int64_t in_stride, void* out,
+                              int64_t out_stride, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -93,6 +93,25 @@ def lmhead_dlogits_t(hidden, weight, targets, lse, spx, g_lp, g_ent, inv_tempera
     return out
 
 
+def transpose_16bit(x: torch.Tensor) -> torch.Tensor:
+    """``x.t().contiguous()`` for a 2-D bf16 / fp16 tensor with contiguous rows, through the tiled HIP kernel."""
+    if x.dim() != 2 or x.element_size() != 2 or x.stride(1) != 1:
+        raise ValueError(f"transpose_16bit needs a 2-D 16-bit tensor with contiguous rows, got {x.dtype} "
+                         f"{tuple(x.shape)} strides {x.stride()}")
+    _need_gpu(x)
+    out = torch.empty((x.size(1), x.size(0)), dtype=x.dtype, device=x.device)
+    check(lib.relax_amd_transpose_16bit(_p(x), x.size(0), x.size(1), x.stride(0), _p(out), out.stride(0), _stream()))
+    return out
+
+
+def _k_contiguous(b: torch.Tensor) -> torch.Tensor:
+    """``b`` ([K, M], the right-hand operand of ``a @ b``) re-laid so that the contraction index is the contiguous one
+    (a transposed copy, returned as a [K, M] view of it).  The library GEMMs of these shapes measured 10 - 15 % faster
+    with both operands contraction-contiguous (dweight 30.6 -> 26.0 ms, dhidden 34.0 -> 30.5 ms at N = 32768,
+    V = 151936, H = 4096); the copy costs well under a millisecond."""
+    return transpose_16bit(b).t()
+
+
 class FusedLMHeadLogProb(torch.autograd.Function):
     """(hidden [N,H] bf16, weight [V,H] bf16, targets [N]) -> (log_prob [N], entropy [N]).
 
@@ -146,12 +165,13 @@ class FusedLMHeadLogProb(torch.autograd.Function):
             ctx.logits_t = False
             if need_h:
                 with ops._timed("lmhead_dhidden_gemm"):
-                    torch.mm(d_t.t(), weight, out=d_hidden)
+                    torch.mm(d_t.t(), _k_contiguous(weight), out=d_hidden)
             d_weight = None
             if need_w:
                 with ops._timed("lmhead_dweight_gemm"):
-                    d_weight = torch.mm(d_t, hidden)
+                    d_weight = torch.mm(d_t, _k_contiguous(hidden))
             return d_hidden, d_weight, None, None, None, None, None
+        weight_k = _k_contiguous(weight) if need_h else None
         slab = torch.empty((v, min(n, BACKWARD_SLAB)), dtype=torch.bfloat16, device=hidden.device)
         for s in range(0, n, BACKWARD_SLAB):
             e = min(n, s + BACKWARD_SLAB)
@@ -160,10 +180,10 @@ class FusedLMHeadLogProb(torch.autograd.Function):
                              g_lp[s:e], None if g_ent is None else g_ent[s:e], ctx.inv_temperature, out=d_t)
             if need_h:
                 with ops._timed("lmhead_dhidden_gemm"):
-                    torch.mm(d_t.t(), weight, out=d_hidden[s:e])
+                    torch.mm(d_t.t(), weight_k, out=d_hidden[s:e])
             if need_w:
                 with ops._timed("lmhead_dweight_gemm"):
-                    part = torch.mm(d_t, hidden[s:e])
+                    part = torch.mm(d_t, _k_contiguous(hidden[s:e]))
                 if s == 0 and e == n:
                     return d_hidden, part, None, None, None, None, None
                 if d_weight32 is None:

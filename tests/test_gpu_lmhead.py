@@ -291,3 +291,25 @@ def test_sft_losses_plain_and_with_deferred_lm_head_vs_oracle():
     assert abs(scaled.item() - want.item() * 2 / 3) < 2e-3 * len(resp) and logd["keys"] == ["loss"] and int(normalizer) == 1
     with pytest.raises(NotImplementedError, match="expose the LM-head weight"):
         relax_amd.sft_loss_function_chunked(args, dbatch, hd, None, lm_head_forward=lambda x: x)
+
+
+@pytest.mark.parametrize("rows,cols,row_pad", [
+    (64, 64, 0), (1000, 200, 0), (77, 4096, 0), (129, 65, 3), (8, 1, 0), (300, 301, 5), (4096, 1030, 8),
+])
+def test_transpose_16bit_is_exact(rows, cols, row_pad):
+    """Bit-exact against torch's own transposed copy, for ragged tiles and for row strides that rule out 16-byte
+    accesses on either side."""
+    from relax_amd.lm_head import transpose_16bit
+
+    dev = require_gpu()
+    announce("transpose", rows, cols, row_pad)
+    g = torch.Generator().manual_seed(rows * 7 + cols)
+    full = torch.randn(rows, cols + row_pad, generator=g).bfloat16().to(dev)
+    x = full[:, :cols]
+    got = transpose_16bit(x)
+    assert got.shape == (cols, rows) and got.is_contiguous()
+    assert torch.equal(got.view(torch.int16), x.t().contiguous().view(torch.int16))
+    with pytest.raises(ValueError):
+        transpose_16bit(x.t())
+    with pytest.raises(ValueError):
+        transpose_16bit(x.float())
