@@ -272,9 +272,17 @@ def run_lmhead(a, dev) -> None:
             hidden.zero_()
             weight.zero_()
 
+    vendor_out = torch.empty((min(n, 8192), v), dtype=torch.bfloat16, device=dev) if a.vendor_gemm else None
+
     def step():
         hidden.grad = None
         weight.grad = None
+        if a.vendor_gemm:  # diagnostic: the library's plain GEMM of the same shape, logits written, 8192 rows at a time
+            from relax_amd import ops
+            with torch.no_grad(), ops._timed("lmhead_logprob_fwd"):
+                for s0 in range(0, n, 8192):
+                    torch.matmul(hidden[s0:s0 + 8192], weight.t(), out=vendor_out[: min(n, s0 + 8192) - s0])
+            return vendor_out[0, 0].float()
         if a.forward_only:  # diagnostic: the clock / power samples then belong to the forward kernel alone
             with torch.no_grad():
                 lp, ent = lm_head_log_probs_and_entropy(hidden, weight, tokens, 1.0, True, False)
@@ -296,9 +304,12 @@ def run_lmhead(a, dev) -> None:
          f"fused LM-head + log-prob/entropy: hidden bf16 [{n}, {h}], weight bf16 [{v}, {h}], fwd "
          + ("(bf16 logits kept for the backward pass)" if a.keep_logits else "(no logits in HBM)")
          + (" only [diagnostic]" if a.forward_only else " + bwd to dhidden/dweight from a scalar loss")
-         + (" [diagnostic: all-zero operands]" if a.lmhead_operands == "zeros" else ""),
+         + (" [diagnostic: all-zero operands]" if a.lmhead_operands == "zeros" else "")
+         + (" [diagnostic: NOT the fused kernel -- hipBLASLt GEMM of the forward shape, logits written]"
+            if a.vendor_gemm else ""),
          {"rows": n, "hidden": h, "vocab": v, "keep_logits": bool(a.keep_logits), "loss": float(loss.item())},
-         {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
+         {"bound": "mfma", "kernel": "hipBLASLt GEMM (diagnostic)" if a.vendor_gemm else "lmhead_fwd_kernel",
+          "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
           "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
           "algorithmic_flops_per_launch": flops, "avg_launch_ms": dom, "kernel_ms": kernel_ms,
           "launches_per_step": launches,
@@ -523,6 +534,9 @@ def main() -> int:
                          "projecting a second time (10 GB at the default size)")
     ap.add_argument("--forward-only", action="store_true",
                     help="lmhead workload, diagnostic: time the forward pass alone (clock samples of that kernel only)")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="lmhead workload, diagnostic: time the library's plain GEMM of the forward shape instead of "
+                         "the fused kernel (same operands, logits written to HBM), for comparison")
     ap.add_argument("--lmhead-operands", choices=["random", "zeros"], default="random",
                     help="lmhead workload, diagnostic: all-zero operands show the kernel without the board power limit")
     ap.add_argument("--two-launch", action="store_true",
