@@ -320,6 +320,47 @@ def run_lmhead(a, dev) -> None:
          None)
 
 
+def run_mfma_ceiling(a, dev) -> None:
+    """Diagnostic, not a workload of the path: bf16 32x32x16 MFMAs on register-resident N(0, 1) operand fragments, one
+    wave per SIMD on every CU, no memory traffic.  What this sustains under the board's power limit is the practical
+    ceiling for the LM-head kernels on this box.  A "step" is one launch of 256 workgroups x 20000 iterations."""
+    import ctypes as C
+    from relax_amd import ops
+    from relax_amd._lib import check, lib
+
+    blocks, iters = 256, 20000
+    g = torch.Generator(device=dev).manual_seed(0)
+    src = torch.randn(4096 * 8, device=dev, generator=g).bfloat16()
+    if a.lmhead_operands == "zeros":
+        src.zero_()
+    out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def step():
+        with ops._timed("diag_mfma_loop"):
+            check(lib.relax_amd_diag_mfma_loop(C.c_void_p(src.data_ptr()), C.c_void_p(out.data_ptr()), blocks, iters,
+                                               stream))
+        return out
+
+    with ClockSampler() as clock:
+        wall, kernel_ms, launches, _ = timed_steps(step, a.warmup, a.steps)
+    clk = clock.summary()
+    flops = blocks * 4 * iters * 64 * 32768.0
+    achieved = flops / (kernel_ms["diag_mfma_loop"] * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "TFLOP/s of register-fed bf16 MFMAs [diagnostic ceiling, not the headline metric]", "value": achieved,
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": wall * 1e3 / a.steps,
+        "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "mfma_ceiling: 256 workgroups x 4 waves x 20000 x 64 MFMA 32x32x16 bf16, operands "
+                               + ("all zero" if a.lmhead_operands == "zeros" else "N(0, 1)") + ", no memory traffic"},
+        "roofline": {"bound": "mfma", "kernel": "diag_mfma_loop_kernel", "achieved": achieved,
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": None, "avg_launch_ms": kernel_ms["diag_mfma_loop"], "clock": clk,
+                     "frac_at_measured_clock":
+                         (achieved / (MFMA_BF16_PEAK_TFLOPS * clk["sclk_mhz"] / PEAK_SCLK_MHZ)) if clk else None},
+        "cpu_baseline": None}))
+
+
 def run_reverse_kl(a, dev) -> None:
     """student / teacher bf16 logits [N, V], teacher = student + N(0, 1); per-token full-vocabulary reverse KL with a
     15 % zero loss mask, token-mean reduction, backward to the student's dlogits."""
@@ -522,7 +563,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="actor_step",
-                    choices=["actor_step", "cfg1", "lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo"])
+                    choices=["actor_step", "cfg1", "lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "mfma_ceiling"])
     ap.add_argument("--seqs", type=int, default=SEQS)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
     ap.add_argument("--vocab", type=int, default=VOCAB)
@@ -561,6 +602,8 @@ def main() -> int:
         run_cfg1(a, dev)
     elif a.workload == "lmhead":
         run_lmhead(a, dev)
+    elif a.workload == "mfma_ceiling":
+        run_mfma_ceiling(a, dev)
     elif a.workload == "reverse_kl":
         run_reverse_kl(a, dev)
     else:

@@ -408,6 +408,14 @@ int relax_amd_lmhead_dlogits_from_logits_t(void* logits_t, int64_t n_tokens, int
 int relax_amd_transpose_16bit(const void* in, int64_t rows, int64_t cols, int64_t in_stride, void* out,
                               int64_t out_stride, void* stream);
 
+/*
+ * Measurement aid with no counterpart in the reference: `blocks` workgroups of four waves each run `iters` iterations
+ * of 64 independent bf16 32x32x16 MFMAs per wave on operand fragments read once from src (4096 x 16 bytes of bf16),
+ * i.e. blocks * 4 * iters * 64 * 32768 FLOP with no memory traffic.  bench.py uses it to report what the matrix cores
+ * sustain on a given box under its power limit.  out receives blocks * 256 floats (a checksum that keeps the loop alive).
+ */
+int relax_amd_diag_mfma_loop(const void* src, float* out, int blocks, int iters, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
