@@ -511,3 +511,30 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
     for key, w in want_m.items():
         assert abs(met[key].item() - float(w)) < 3e-5 * max(1.0, abs(float(w))), (key, met[key].item(), float(w))
     torch.testing.assert_close(lg.grad.cpu(), lo.grad, atol=3e-5, rtol=1e-5)
+
+
+def test_outputs_leave_as_one_packed_copy_in_the_reference_wire_format():
+    """What the forward-only pass returns goes to the data system as jagged nested tensors on the host
+    (relax/backends/megatron/actor.py:2351-2363): the per-sample lists are views of one packed vector, so the packed
+    vector is what crosses PCIe, and the result equals the list-based construction of the reference."""
+    import relax_amd
+    from relax_amd import data_fields as DF
+
+    dev = require_gpu()
+    announce("wire format of forward-only outputs")
+    tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 1000
+    logits, batch = _make_batch(5, tot, resp, v, torch.bfloat16)
+    db = _to_dev(batch, dev)
+    ids = [torch.randint(0, v, (r, 3), device=dev) for r in resp]
+    with torch.no_grad():
+        _, out = relax_amd.get_log_probs_and_entropy(
+            logits.to(dev), args=P.make_args(), unconcat_tokens=db["unconcat_tokens"], total_lengths=tot,
+            response_lengths=resp, with_entropy=True, gather_topk_token_ids=ids)
+    assert DF._packed_parent(out["log_probs"]) is not None and DF._packed_parent(out["entropy"]) is not None
+    payload = DF.to_transfer_payload(out)
+    for key, items in out.items():
+        want = torch.nested.as_nested_tensor([t.cpu() for t in items], layout=torch.jagged)
+        got = payload[key]
+        assert got.is_nested and got.layout == torch.jagged and got.device.type == "cpu"
+        for a, b in zip(got.unbind(), want.unbind()):
+            assert a.dtype == b.dtype and torch.equal(a, b)
