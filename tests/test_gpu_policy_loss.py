@@ -538,3 +538,58 @@ def test_outputs_leave_as_one_packed_copy_in_the_reference_wire_format():
         assert got.is_nested and got.layout == torch.jagged and got.device.type == "cpu"
         for a, b in zip(got.unbind(), want.unbind()):
             assert a.dtype == b.dtype and torch.equal(a, b)
+
+
+def test_callable_from_worker_threads_and_under_activation_checkpointing():
+    """The reference runs this path from worker threads (ActorFwd / Advantages services: threading.Thread,
+    asyncio.to_thread; relax/components/actor_fwd.py:56-66) and may wrap the loss in torch.utils.checkpoint
+    (relax/backends/megatron/loss.py:1535-1543, the forward then runs twice): results must not depend on the calling
+    thread, concurrent callers must not disturb each other, and the recomputed forward must be deterministic."""
+    import threading
+
+    import relax_amd
+    from torch.utils.checkpoint import checkpoint
+
+    dev = require_gpu()
+    announce("worker threads + checkpoint")
+    tot, resp, v = [40, 25, 33, 18], [20, 11, 30, 9], 3000
+    logits, batch = _make_batch(31, tot, resp, v, torch.bfloat16)
+    db = _to_dev(batch, dev)
+    args = P.make_args(eps_clip_high=0.28, use_kl_loss=True, kl_loss_coef=1e-3, kl_loss_type="k3", entropy_coef=0.01)
+    from relax_amd.cp_utils import get_sum_of_sample_mean
+
+    red = get_sum_of_sample_mean(tot, resp, db["loss_masks"])
+
+    def run():
+        lg = logits.to(dev).requires_grad_()
+        loss, metrics = relax_amd.policy_loss_function(args, db, lg, red)
+        loss.backward()
+        return loss.detach().clone(), lg.grad.clone(), {k: m.clone() for k, m in metrics.items()}
+
+    want = run()
+    results, errors = {}, []
+
+    def worker(i):
+        try:
+            with torch.cuda.stream(torch.cuda.Stream(device=dev)):  # default priority; each thread its own stream
+                for _ in range(5):
+                    results[i] = run()
+                torch.cuda.current_stream().synchronize()
+        except Exception as exc:  # surfaced below: an exception inside a thread would otherwise be lost
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(3)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(3):
+        loss, grad, metrics = results[i]
+        assert torch.equal(loss, want[0]) and torch.equal(grad, want[1])
+        assert all(torch.equal(metrics[k], want[2][k]) for k in want[2])
+
+    lg = logits.to(dev).requires_grad_()
+    loss = checkpoint(lambda x: relax_amd.policy_loss_function(args, db, x, red)[0], lg, use_reentrant=False)
+    loss.backward()
+    assert torch.equal(loss.detach(), want[0]) and torch.equal(lg.grad, want[1])
