@@ -313,3 +313,59 @@ def test_transpose_16bit_is_exact(rows, cols, row_pad):
         transpose_16bit(x.t())
     with pytest.raises(ValueError):
         transpose_16bit(x.float())
+
+
+def test_model_forward_under_bypass_feeds_the_fused_loss_end_to_end():
+    """A small model run under ``bypass_output_layer`` returns hidden states; ``loss_function`` with the yielded handle
+    gives the loss and the gradients (LM-head weight and the layers below it) of the same model run normally with
+    materialised logits, to the bf16 tolerances of the reference's chunked-LM-head test."""
+    import relax_amd
+    from relax_amd.model import bypass_output_layer
+
+    dev = require_gpu()
+    announce("bypass end to end")
+
+    class Head(torch.nn.Module):
+        def __init__(self, h, v):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.randn(v, h) * 0.1)
+
+        def forward(self, input_, weight=None, runtime_gather_output=None):
+            return F.linear(input_, self.weight if weight is None else weight), None
+
+    class Tiny(torch.nn.Module):
+        def __init__(self, v, h):
+            super().__init__()
+            self.embed = torch.nn.Embedding(v, h)
+            self.mix = torch.nn.Linear(h, h)
+            self.output_layer = Head(h, v)
+
+        def forward(self, tokens):
+            x = torch.tanh(self.mix(self.embed(tokens)))
+            return self.output_layer(x)[0]
+
+    torch.manual_seed(3)
+    v, h, tot, resp = 300, 128, [9, 14, 6], [9, 6, 6]
+    model = Tiny(v, h).bfloat16().to(dev)
+    g = torch.Generator().manual_seed(8)
+    toks = [torch.randint(0, v, (n,), generator=g).to(dev) for n in tot]
+    masks = [(torch.rand(r, generator=g) > 0.2).float().to(dev) for r in resp]
+    batch = dict(unconcat_tokens=toks, total_lengths=tot, response_lengths=resp, loss_masks=masks)
+    args = P.make_args(loss_type="sft", sft_chunked_logits=True, global_batch_size=3)
+    packed = torch.cat(toks).unsqueeze(0)
+
+    logits = model(packed).float()
+    want, _, _ = relax_amd.loss_function(P.make_args(loss_type="sft", global_batch_size=3), batch, 1, logits)
+    want.backward()
+    ref_grads = {k: p.grad.clone() for k, p in model.named_parameters()}
+    model.zero_grad()
+
+    with bypass_output_layer(model) as head:
+        hidden = model(packed)
+        assert hidden.shape == (1, sum(tot), h) and hidden.dtype == torch.bfloat16
+        loss, _, log = relax_amd.loss_function(args, batch, 1, hidden, lm_head_forward=head)
+    loss.backward()
+    assert abs(loss.item() - want.item()) < 2e-3 * len(resp)
+    for k, p in model.named_parameters():
+        torch.testing.assert_close(p.grad.float(), ref_grads[k].float(), atol=5e-3, rtol=4 * BF16_ULP, msg=k)
+    assert torch.equal(model(packed).float(), logits)  # the layer projects again once the block is left
