@@ -526,3 +526,28 @@ def test_opd_advantage_shaping_vs_oracle(selection):
             torch.testing.assert_close(a.cpu(), b, atol=2e-6, rtol=2e-6)
         for r_, n, r in zip(dd["returns"], lens, data["rewards"]):
             assert torch.equal(r_.cpu(), torch.zeros(n) if only else torch.full((n,), r))
+
+
+def test_reinforce_pp_baseline_wiring_literals():
+    """The literal case of the reference's wiring test
+    (tests/backends/megatron/test_reinforce_plus_plus_wiring.py:45-79): rewards [1, -1], masks [[1, 0], [1, 1]],
+    gamma 1, no KL, normalisation on."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("reinforce++ baseline wiring literals")
+    args = SimpleNamespace(use_rollout_logprobs=False, kl_coef=0.0, kl_loss_type="k2",
+                           advantage_estimator="reinforce_plus_plus_baseline", gamma=1.0, use_opd=False,
+                           normalize_advantages=True)
+    data = {"log_probs": [torch.zeros(2, device=dev), torch.zeros(2, device=dev)], "ref_log_probs": None,
+            "rewards": [1.0, -1.0], "values": None, "response_lengths": [2, 2],
+            "loss_masks": [torch.tensor([1.0, 0.0], device=dev), torch.tensor([1.0, 1.0], device=dev)],
+            "total_lengths": [2, 2]}
+    relax_amd.compute_advantages_and_returns(args, data)
+    for got, want in zip(data["returns"], [[1.0, 0.0], [-1.0, -1.0]]):
+        torch.testing.assert_close(got.cpu(), torch.tensor(want), atol=1e-6, rtol=1e-6)
+    for got, want in zip(data["advantages"], [[2.0 ** 0.5, 0.0], [-(0.5 ** 0.5), -(0.5 ** 0.5)]]):
+        torch.testing.assert_close(got.cpu(), torch.tensor(want), atol=1e-6, rtol=1e-6)
+    assert data["reinforce_pp_valid_token_count"][0].item() == 3
+    assert data["reinforce_pp_zero_variance"][0].item() == 0
+    assert isinstance(data["reinforce_pp_advantage_raw_mean"][0], torch.Tensor)
