@@ -145,3 +145,15 @@ def test_transfer_payload_and_advantages_payload():
     pay = DF.advantages_payload(adv, adv)
     assert pay["advantages"].is_nested and [t.shape for t in pay["returns"].unbind()] == [t.shape for t in adv]
     assert all(torch.equal(x, y) for x, y in zip(pay["advantages"].unbind(), adv))
+
+
+def test_ppl_metrics_literals():
+    """tests/engine/sft/eval/test_ppl.py:14-33: totals 10.0 over 6 tokens; an empty evaluation gives zeros."""
+    import math
+
+    from relax_amd.sft_eval import compute_ppl_metrics
+
+    m = compute_ppl_metrics(total_neg_log_prob=10.0, total_tokens=6)
+    assert math.isclose(m["eval/loss"], 10.0 / 6.0, rel_tol=1e-6)
+    assert math.isclose(m["eval/ppl"], math.exp(10.0 / 6.0), rel_tol=1e-5) and m["eval/num_tokens"] == 6
+    assert compute_ppl_metrics(0.0, 0) == {"eval/loss": 0.0, "eval/ppl": 0.0, "eval/num_tokens": 0}

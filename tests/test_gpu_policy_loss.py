@@ -593,3 +593,29 @@ def test_callable_from_worker_threads_and_under_activation_checkpointing():
     loss = checkpoint(lambda x: relax_amd.policy_loss_function(args, db, x, red)[0], lg, use_reentrant=False)
     loss.backward()
     assert torch.equal(loss.detach(), want[0]) and torch.equal(lg.grad, want[1])
+
+
+def test_sft_eval_step_sums_and_counts_vs_oracle():
+    """The SFT evaluation callback (relax/engine/sft/eval/ppl.py:24-92): masked sum of negative log-probs and the
+    exact token count per micro-batch, in the shapes and dtypes the forward-only harness stacks."""
+    from relax_amd.sft_eval import compute_ppl_metrics, compute_sft_eval_step
+
+    dev = require_gpu()
+    announce("sft eval step")
+    tot, resp, v = [9, 6, 12], [9, 3, 12], 500     # SFT-shaped samples (response == total) and one RL-shaped
+    logits, batch = _make_batch(9, tot, resp, v, torch.bfloat16, int_masks=True)
+    db = _to_dev(batch, dev)
+    empty, out = compute_sft_eval_step(logits.to(dev), args=P.make_args(), unconcat_tokens=db["unconcat_tokens"],
+                                       total_lengths=tot, response_lengths=resp, loss_masks=db["loss_masks"],
+                                       dynamic_cp_size=None, dynamic_cp_rank=None, max_seq_lens=None)
+    assert empty.shape == (0,) and empty.device.type == "cuda"
+    s, n = out["sum_neg_log_prob"][0], out["num_tokens"][0]
+    assert s.shape == (1,) and s.dtype == torch.float32 and n.shape == (1,) and n.dtype == torch.long
+    _, ref = P.get_log_probs_and_entropy(logits.float(), args=P.make_args(), unconcat_tokens=batch["unconcat_tokens"],
+                                         total_lengths=tot, response_lengths=resp)
+    masks = torch.cat([m.float() for m in batch["loss_masks"]])
+    want = -(torch.cat(ref["log_probs"]) * masks).sum()
+    assert n.item() == int(masks.sum().item())
+    assert abs(s.item() - want.item()) < 2e-3 * max(1, n.item())
+    m = compute_ppl_metrics(s.item(), n.item())
+    assert abs(m["eval/loss"] - want.item() / masks.sum().item()) < 2e-3
