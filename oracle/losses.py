@@ -105,3 +105,18 @@ def vanilla_tis(pg_loss, train_lp, rollout_lp, clip_low: float, clip_high: float
         "mismatch_k3_kl": (tis - log_ratio - 1).detach(),
     }
     return pg_loss * w, metrics
+
+
+def icepop(pg_loss, train_lp, rollout_lp, clip_low: float, clip_high: float):
+    """relax/backends/megatron/loss.py:772-801: importance ratios outside [clip_low, clip_high] get weight zero."""
+    log_ratio = train_lp - rollout_lp
+    tis = torch.exp(log_ratio)
+    w = torch.where((tis >= clip_low) & (tis <= clip_high), tis, torch.zeros_like(tis))
+    metrics = {
+        "tis": tis.detach().clone(),
+        "tis_clipfrac": (w != tis).float(),
+        "tis_abs": (tis - 1).abs().detach(),
+        "mismatch_kl": (-log_ratio).detach(),
+        "mismatch_k3_kl": (tis - log_ratio - 1).detach(),
+    }
+    return pg_loss * w, metrics

@@ -136,8 +136,14 @@ def lm_head_log_probs(hidden, weight, targets, temperature=1.0, sub_chunk=1024):
     return torch.cat(out, dim=0) if out else hidden.new_zeros((0,), dtype=torch.float32)
 
 
-def policy_loss_function(args, batch, logits, reducer, pg_reducer=None):
-    """Composition of loss.py:824-1185 (no OPD top-K, no M2PO, no CP).  Returns (loss, metrics dict)."""
+def policy_loss_function(args, batch, logits, reducer, pg_reducer=None, tis_fn=None, rebuild_reducer=None,
+                         pg_reducer_factory=None):
+    """Composition of loss.py:824-1185 (no M2PO, no CP).  Returns (loss, metrics dict).
+
+    Plug-in points: ``tis_fn(pg_loss, train_lp, rollout_lp, masks) -> (pg_loss, masks, metrics)`` stands for
+    ``--custom-tis-function-path`` (:1036-1040); when it is given, ``rebuild_reducer(masks)`` builds the reducer used
+    after it (:1044-1059) while the importance-sampling metrics keep the original one (:1007-1014);
+    ``pg_reducer_factory(masks)`` stands for ``--custom-pg-loss-reducer-function-path`` (:1062-1072)."""
     adv = torch.cat(batch["advantages"], dim=0) if isinstance(batch["advantages"], list) else batch["advantages"]
     resp, tot = batch["response_lengths"], batch["total_lengths"]
     if args.advantage_estimator in ("reinforce_plus_plus", "reinforce_plus_plus_baseline"):
@@ -186,13 +192,23 @@ def policy_loss_function(args, batch, logits, reducer, pg_reducer=None):
         pg = pg * om
 
     tis_metrics = None
-    if args.get_mismatch_metrics or args.use_tis:  # :1006-1059 with the vanilla weights, masks unchanged
+    metric_reducer = reducer
+    pg_masks = batch["loss_masks"]
+    if args.get_mismatch_metrics or args.use_tis:  # :1006-1059
         ois = (-ppo_kl).exp()
         train_side = torch.cat([x.detach() for x in lps]) if args.true_on_policy_mode else torch.cat(batch["log_probs"])
-        pg, tis_metrics = losses.vanilla_tis(
-            pg, train_side, torch.cat(batch["rollout_log_probs"]), args.tis_clip_low, args.tis_clip
-        )
+        if tis_fn is None:
+            pg, tis_metrics = losses.vanilla_tis(
+                pg, train_side, torch.cat(batch["rollout_log_probs"]), args.tis_clip_low, args.tis_clip
+            )
+        else:
+            pg, pg_masks, tis_metrics = tis_fn(pg, train_side, torch.cat(batch["rollout_log_probs"]), pg_masks)
+            reducer = rebuild_reducer(pg_masks)
 
+    if pg_reducer_factory is not None:
+        pg_reducer = pg_reducer_factory(pg_masks)
+        if args.advantage_estimator in ("reinforce_plus_plus", "reinforce_plus_plus_baseline"):
+            pg_reducer = _safe(pg_reducer)  # :1070-1071
     pg_red = pg_reducer if pg_reducer is not None else reducer
     pg_loss = pg_red(pg)
     pg_clipfrac = reducer(clipfrac)
@@ -235,9 +251,9 @@ def policy_loss_function(args, batch, logits, reducer, pg_reducer=None):
     if args.use_kl_loss:
         metrics["kl_loss"] = kl_loss.detach().clone()
     if tis_metrics is not None:
-        metrics["ois"] = reducer(ois).detach().clone()
+        metrics["ois"] = metric_reducer(ois).detach().clone()
         for k, v in tis_metrics.items():
-            metrics[k] = reducer(v)
+            metrics[k] = metric_reducer(v)
     if args.use_opsm:
         metrics["opsm_clipfrac"] = opsm_frac
     return loss, metrics

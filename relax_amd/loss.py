@@ -367,6 +367,175 @@ def _cat_f32(parts, device):
     return torch.cat([p.to(device=device).reshape(-1) for p in parts]).to(torch.float32)
 
 
+def load_function(path: str):
+    """``"pkg.module.fn"`` -> the function object (relax/utils/misc.py:30-38)."""
+    import importlib
+
+    module_path, _, attr = path.rpartition(".")
+    return getattr(importlib.import_module(module_path), attr)
+
+
+def _tis_terms(args, pg_loss, train_log_probs, rollout_log_probs):
+    ratio_log = torch.cat(train_log_probs, dim=0) - torch.cat(rollout_log_probs, dim=0)
+    tis = torch.exp(ratio_log)
+    metrics = {"tis": tis, "tis_abs": (tis - 1).abs(), "mismatch_kl": -ratio_log, "mismatch_k3_kl": tis - ratio_log - 1}
+    return tis, metrics
+
+
+def vanilla_tis_function(args, *, pg_loss, train_log_probs, rollout_log_probs, loss_masks, **kwargs):
+    """Truncated importance sampling, loss.py:741-769: weights ``clamp(exp(train - rollout), tis_clip_low, tis_clip)``.
+    Returns ``(pg_loss * weights, loss_masks, per-token metrics)``; the plug-in signature of
+    ``--custom-tis-function-path``."""
+    tis, metrics = _tis_terms(args, pg_loss, train_log_probs, rollout_log_probs)
+    weights = torch.clamp(tis, min=args.tis_clip_low, max=args.tis_clip)
+    metrics["tis_clipfrac"] = (weights != tis).float()
+    return pg_loss * weights, loss_masks, {k: v.clone().detach() for k, v in metrics.items()}
+
+
+def icepop_function(args, *, pg_loss, train_log_probs, rollout_log_probs, loss_masks, **kwargs):
+    """loss.py:772-801: like the truncated weights, but ratios outside ``[tis_clip_low, tis_clip]`` are zeroed."""
+    tis, metrics = _tis_terms(args, pg_loss, train_log_probs, rollout_log_probs)
+    weights = torch.where((tis >= args.tis_clip_low) & (tis <= args.tis_clip), tis, torch.zeros_like(tis))
+    metrics["tis_clipfrac"] = (weights != tis).float()
+    return pg_loss * weights, loss_masks, {k: v.clone().detach() for k, v in metrics.items()}
+
+
+def _mask_safe(reducer, loss_masks):
+    """REINFORCE++ reductions select the valid tokens first (loss.py:804-821), so a non-finite value under a zero mask
+    cannot reach the sum as ``NaN * 0``."""
+    valid = torch.cat([m.reshape(-1) != 0 for m in loss_masks], dim=0)
+
+    def reduce_valid_tokens(values):
+        v = valid.to(device=values.device)
+        if values.shape[0] != v.numel():
+            raise ValueError("REINFORCE++ reducer expected one value per response token, "
+                             f"got {values.shape[0]} values for {v.numel()} mask elements.")
+        return reducer(torch.where(v, values, torch.zeros_like(values)))
+
+    return reduce_valid_tokens
+
+
+def _composed_policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum_of_sample_mean=None):
+    """The policy loss as the reference composes it (loss.py:824-1185), step by step, for the configurations that hand
+    per-token tensors to user code: ``--custom-tis-function-path`` (importance weights / rejection masks) and
+    ``--custom-pg-loss-reducer-function-path``.  The ``[N, V]`` work is still one packed log-prob / entropy launch
+    (forward) and one dlogits launch (backward); everything between them acts on ``[N]`` vectors through the
+    differentiable token-loss kernels of ``ppo_utils`` and plain tensor arithmetic, so arbitrary Python can sit in the
+    middle."""
+    from . import ppo_utils as PU
+    from .opd_utils import compute_policy_opd_loss, resolve_opd_gather_topk_token_ids
+
+    est = args.advantage_estimator
+    pp = est in ("reinforce_plus_plus", "reinforce_plus_plus_baseline")
+    response_lengths, total_lengths = batch["response_lengths"], batch["total_lengths"]
+    masks = batch["loss_masks"]
+    per_token = bool(getattr(args, "calculate_per_token_loss", False))
+
+    def reducer_for(loss_masks):
+        red = get_sum_of_sample_mean(total_lengths, response_lengths, loss_masks, per_token,
+                                     sample_denoms=batch.get("sample_index_mask_sums"))
+        return _mask_safe(red, loss_masks) if pp else red
+
+    reduce = sum_of_sample_mean if sum_of_sample_mean is not None else reducer_for(masks)
+    if pp and sum_of_sample_mean is not None:
+        reduce = _mask_safe(reduce, masks)
+    dev = logits.device
+    adv = batch["advantages"]
+    adv = adv.to(dev).float() if isinstance(adv, torch.Tensor) else torch.cat([a.to(dev) for a in adv]).float()
+    _, out = get_log_probs_and_entropy(
+        logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=total_lengths,
+        response_lengths=response_lengths, with_entropy=True,
+        gather_topk_token_ids=resolve_opd_gather_topk_token_ids(args, batch))
+    lps = out["log_probs"]
+    true_on_policy = getattr(args, "true_on_policy_mode", False)
+    if true_on_policy:
+        olds = [x.detach() for x in lps]
+    else:
+        olds = [x.to(dev) for x in (batch["rollout_log_probs"] if args.use_rollout_logprobs else batch["log_probs"])]
+    masks_dev = [m.to(dev) for m in masks]
+    adv_list = list(torch.split(adv, response_lengths))
+    if getattr(args, "use_opsm", False):
+        opsm_mask, opsm_clipfrac = PU.compute_opsm_mask(args, lps, olds, adv_list, masks_dev)
+    lp, old = torch.cat(lps), torch.cat(olds).float()
+    ppo_kl = PU.compute_gspo_kl(lps, olds, lps, masks_dev) if est == "gspo" else old - lp
+    if est == "sapo":
+        pg_loss, pg_clipfrac = PU.compute_sapo_loss(ppo_kl, adv, args.sapo_tau_pos, args.sapo_tau_neg)
+    elif est == "cispo":
+        pg_loss, pg_clipfrac = PU.compute_cispo_loss(lp, ppo_kl, adv, args.eps_clip, args.eps_clip_high)
+    elif est == "rloo":
+        pg_loss, pg_clipfrac = PU.compute_rloo_loss(lp, adv)
+    elif est in ("grpo", "gspo", "ppo") or pp:
+        pg_loss, pg_clipfrac = PU.compute_policy_loss(ppo_kl, adv, args.eps_clip, args.eps_clip_high)
+    else:
+        raise NotImplementedError(f"advantage_estimator {est} is not supported. ")
+    if getattr(args, "use_opsm", False):
+        pg_loss = pg_loss * opsm_mask
+
+    mismatch = bool(getattr(args, "get_mismatch_metrics", False) or getattr(args, "use_tis", False))
+    tis_metrics, metric_reduce = None, reduce
+    pg_masks = masks
+    if mismatch:
+        assert "rollout_log_probs" in batch, "rollout_log_probs must be provided for TIS"
+        ois = (-ppo_kl).exp()
+        train = [x.detach() for x in lps] if true_on_policy else [x.to(dev) for x in batch["log_probs"]]
+        path = getattr(args, "custom_tis_function_path", None)
+        tis_func = load_function(path) if path is not None else vanilla_tis_function
+        pg_loss, pg_masks, tis_metrics = tis_func(
+            args=args, pg_loss=pg_loss, train_log_probs=train,
+            rollout_log_probs=[x.to(dev) for x in batch["rollout_log_probs"]], loss_masks=masks_dev,
+            total_lengths=total_lengths, response_lengths=response_lengths)
+        reduce = reducer_for(pg_masks)  # rejection masks change the numerators; denominators stay per logical sample
+    path = getattr(args, "custom_pg_loss_reducer_function_path", None)
+    if path is not None:
+        pg_reduce = load_function(path)(total_lengths, response_lengths, pg_masks, per_token)
+        if pp:
+            pg_reduce = _mask_safe(pg_reduce, pg_masks)
+    else:
+        pg_reduce = reduce
+
+    pg_loss = pg_reduce(pg_loss)
+    pg_clipfrac = reduce(pg_clipfrac)
+    kl_metric = reduce(ppo_kl)
+    entropy_loss = reduce(torch.cat(out["entropy"], dim=0))
+    loss = pg_loss - args.entropy_coef * entropy_loss
+    use_kl = bool(getattr(args, "use_kl_loss", False))
+    if use_kl:
+        ref = torch.cat([x.to(dev) for x in batch["ref_log_probs"]], dim=0).float()
+        ratio = torch.exp(lp - old) if getattr(args, "use_unbiased_kl", False) else None
+        kl_loss = reduce(PU.compute_approx_kl(lp, ref, args.kl_loss_type, ratio))
+        loss = loss + args.kl_loss_coef * kl_loss
+    opd_loss, opd_reported = compute_policy_opd_loss(args=args, batch=batch, log_probs=lp, old_log_probs=old,
+                                                     log_probs_and_entropy=out)
+    if opd_loss is not None:
+        loss = loss + opd_loss
+    if lp.numel() == 0:
+        loss = loss + 0 * logits.sum()
+
+    reported = {"loss": loss.clone().detach(), "pg_loss": pg_loss.clone().detach(),
+                "entropy_loss": entropy_loss.clone().detach(), "pg_clipfrac": pg_clipfrac.clone().detach(),
+                "ppo_kl": kl_metric.clone().detach()}
+    reported.update(opd_reported)
+    if batch.get("rollout_log_probs") is not None:
+        rollout = torch.cat([x.to(dev) for x in batch["rollout_log_probs"]], dim=0).float()
+        if not args.use_rollout_logprobs:
+            side = old
+        elif batch.get("log_probs"):
+            side = torch.cat([x.to(dev) for x in batch["log_probs"]], dim=0).float()
+        else:
+            side = lp.detach()
+        reported["train_rollout_logprob_abs_diff"] = reduce((side - rollout).abs()).clone().detach()
+        reported["train_rollout_prob_abs_diff"] = reduce((side.exp() - rollout.exp()).abs()).clone().detach()
+    if use_kl:
+        reported["kl_loss"] = kl_loss.clone().detach()
+    if tis_metrics is not None:
+        reported["ois"] = metric_reduce(ois).clone().detach()
+        for k, v in tis_metrics.items():
+            reported[k] = metric_reduce(v)  # over the tokens valid before any rejection (loss.py:1007-1014)
+    if getattr(args, "use_opsm", False):
+        reported["opsm_clipfrac"] = opsm_clipfrac
+    return loss, reported
+
+
 def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum_of_sample_mean=None):
     """Fused counterpart of loss.py:824-1185.  Returns ``(loss, metrics)`` with the reference's metric keys.
 
@@ -374,15 +543,19 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     ``sample_index_mask_sums`` denominators, or the masked token sum when ``args.calculate_per_token_loss``) is
     evaluated inside the kernel from ``batch``.  A caller-specific reducer can be passed as
     ``batch["relax_amd_sample_denominators"]`` (per-sample divisors) or, for pg_loss only,
-    ``batch["relax_amd_pg_sample_denominators"]``.
+    ``batch["relax_amd_pg_sample_denominators"]``.  With ``args.custom_tis_function_path`` or
+    ``args.custom_pg_loss_reducer_function_path`` set, the loss is composed step by step around the user's callables
+    (``_composed_policy_loss_function``) instead of being evaluated inside one kernel.
     """
     flat = _check_logits(logits, args)
     dev = flat.device
     est = args.advantage_estimator
     if est == "m2po":
         raise NotImplementedError(f"advantage_estimator {est} is not part of the fused path")
-    if getattr(args, "custom_tis_function_path", None) is not None or getattr(args, "custom_pg_loss_reducer_function_path", None) is not None:
-        raise NotImplementedError("custom TIS / reducer callables cannot run inside the fused kernel")
+    if getattr(args, "custom_tis_function_path", None) is not None \
+            or getattr(args, "custom_pg_loss_reducer_function_path", None) is not None:
+        _check_logits(logits, args)
+        return _composed_policy_loss_function(args, batch, logits, None)  # user code acts on per-token tensors
     response_lengths, total_lengths = batch["response_lengths"], batch["total_lengths"]
     needs_bwd = torch.is_grad_enabled() and logits.requires_grad
     lay = PackedLayout(dev, flat.size(0), batch["unconcat_tokens"], total_lengths, response_lengths, needs_bwd)
@@ -499,12 +672,17 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
     ``lm_head_forward`` are given), Megatron gradient-accumulation scaling, and the ``{"keys", "values"}`` logging
     dict."""
     loss_type = getattr(args, "loss_type", "policy_loss")
-    if loss_type not in ("policy_loss", "sft"):
-        raise ValueError(f"Unknown loss type: {loss_type}") if loss_type not in ("value_loss", "custom_loss") \
+    if loss_type not in ("policy_loss", "sft", "custom_loss"):
+        raise ValueError(f"Unknown loss type: {loss_type}") if loss_type != "value_loss" \
             else NotImplementedError(f"loss type {loss_type} is outside the fused policy path")
     num_tokens = get_cp_local_num_tokens(batch["total_lengths"], batch["response_lengths"], batch["loss_masks"])
     if loss_type == "policy_loss":
         loss, log = policy_loss_function(args, batch, logits, None)
+    elif loss_type == "custom_loss":  # loss.py:1530-1531: the plug-in gets the reducer the built-in losses use
+        reducer = get_sum_of_sample_mean(batch["total_lengths"], batch["response_lengths"], batch["loss_masks"],
+                                         bool(getattr(args, "calculate_per_token_loss", False)),
+                                         sample_denoms=batch.get("sample_index_mask_sums"))
+        loss, log = load_function(args.custom_loss_function_path)(args, batch, logits, reducer)
     elif getattr(args, "task_type", "causal_lm") == "seq_cls":
         raise NotImplementedError("sequence-classification SFT is outside the fused policy path")
     elif getattr(args, "sft_chunked_logits", False) and lm_head_forward is not None:

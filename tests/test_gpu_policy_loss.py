@@ -619,3 +619,95 @@ def test_sft_eval_step_sums_and_counts_vs_oracle():
     assert abs(s.item() - want.item()) < 2e-3 * max(1, n.item())
     m = compute_ppl_metrics(s.item(), n.item())
     assert abs(m["eval/loss"] - want.item() / masks.sum().item()) < 2e-3
+
+
+@pytest.mark.parametrize("case", ["vanilla_vs_fused", "icepop", "rejecting_tis_and_token_mean", "reinforce_pp_custom_reducer"])
+def test_custom_tis_and_reducer_hooks(case):
+    """``--custom-tis-function-path`` / ``--custom-pg-loss-reducer-function-path`` (loss.py:1036-1072): the loss is
+    composed around the user's callables.  With the library's own ``vanilla_tis_function`` named as the custom
+    function the composed path must reproduce the single-kernel path; the other cases are checked against the oracle's
+    composition with the same plug-ins."""
+    import relax_amd
+    from oracle import losses as L
+
+    dev = require_gpu()
+    announce("custom hooks", case)
+    tot, resp, v = [11, 8, 14, 9], [6, 5, 9, 4], 700
+    logits, batch = _make_batch(41, tot, resp, v, torch.float32)
+    db = _to_dev(batch, dev)
+    base = dict(use_tis=True, tis_clip=1.05, tis_clip_low=0.95, use_kl_loss=True, kl_loss_coef=0.05, kl_loss_type="k3",
+                entropy_coef=0.01, custom_tis_function_path=None, custom_pg_loss_reducer_function_path=None)
+    oracle_kw = {}
+    if case == "vanilla_vs_fused":
+        args = P.make_args(**{**base, "custom_tis_function_path": "relax_amd.loss.vanilla_tis_function"})
+    elif case == "icepop":
+        args = P.make_args(**{**base, "custom_tis_function_path": "relax_amd.loss.icepop_function"})
+        oracle_kw = dict(
+            tis_fn=lambda pg, tr, ro, masks: (*L.icepop(pg, tr, ro, 0.95, 1.05)[:1], masks, L.icepop(pg, tr, ro, 0.95, 1.05)[1]),
+            rebuild_reducer=lambda masks: R.make_reducer(resp, masks))
+    elif case == "rejecting_tis_and_token_mean":
+        from tests import custom_hooks as H
+
+        args = P.make_args(**{**base, "custom_tis_function_path": "tests.custom_hooks.rejecting_tis",
+                              "custom_pg_loss_reducer_function_path": "tests.custom_hooks.token_mean_reducer"})
+
+        def tis_fn(pg, tr, ro, masks):
+            return H.rejecting_tis(None, pg_loss=pg, train_log_probs=[tr], rollout_log_probs=[ro], loss_masks=masks)
+
+        oracle_kw = dict(tis_fn=tis_fn, rebuild_reducer=lambda masks: R.make_reducer(resp, masks),
+                         pg_reducer_factory=lambda masks: H.token_mean_reducer(tot, resp, masks, False))
+    else:
+        from tests import custom_hooks as H
+
+        args = P.make_args(**{**base, "use_tis": False, "advantage_estimator": "reinforce_plus_plus",
+                              "custom_pg_loss_reducer_function_path": "tests.custom_hooks.token_mean_reducer"})
+        oracle_kw = dict(pg_reducer_factory=lambda masks: H.token_mean_reducer(tot, resp, masks, False))
+
+    lg = logits.to(dev).requires_grad_()
+    loss, metrics = relax_amd.policy_loss_function(args, db, lg, None)
+    loss.backward()
+
+    if case == "vanilla_vs_fused":
+        fused_args = P.make_args(**base)
+        lg2 = logits.to(dev).requires_grad_()
+        want_loss, want_metrics = relax_amd.policy_loss_function(fused_args, db, lg2, None)
+        want_loss.backward()
+        want_grad = lg2.grad.cpu()
+        want_metrics = {k: m.cpu() for k, m in want_metrics.items()}
+        want_loss = want_loss.detach().cpu()
+    else:
+        lref = logits.clone().requires_grad_()
+        want_loss, want_metrics = P.policy_loss_function(args, batch, lref, R.make_reducer(resp, batch["loss_masks"]),
+                                                         **oracle_kw)
+        want_loss.backward()
+        want_grad, want_loss = lref.grad, want_loss.detach()
+    assert set(metrics) == set(want_metrics), (sorted(metrics), sorted(want_metrics))
+    torch.testing.assert_close(loss.detach().cpu(), want_loss, atol=3e-5, rtol=1e-5)
+    for k in want_metrics:
+        torch.testing.assert_close(metrics[k].cpu().float(), want_metrics[k].float(), atol=3e-5, rtol=1e-4, msg=k)
+    torch.testing.assert_close(lg.grad.cpu(), want_grad, atol=3e-5, rtol=1e-4)
+
+
+def test_custom_loss_function_path_dispatch():
+    """``--loss-type custom_loss --custom-loss-function-path`` (loss.py:1530-1531): the plug-in is loaded by dotted path
+    and called with the library's reducer; scaling and the logging dict are those of the built-in losses."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("custom loss dispatch")
+    tot, resp, v = [11, 8, 14], [6, 5, 9], 400
+    logits, batch = _make_batch(43, tot, resp, v, torch.float32)
+    db = _to_dev(batch, dev)
+    args = P.make_args(loss_type="custom_loss", custom_loss_function_path="tests.custom_hooks.negative_log_likelihood",
+                       global_batch_size=3)
+    lg = logits.to(dev).requires_grad_()
+    loss, norm, log = relax_amd.loss_function(args, db, 2, lg)
+    loss.backward()
+    lref = logits.clone().requires_grad_()
+    _, out = P.get_log_probs_and_entropy(lref, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=tot,
+                                         response_lengths=resp)
+    want = -R.make_reducer(resp, batch["loss_masks"])(torch.cat(out["log_probs"])) * 2 / 3
+    want.backward()
+    torch.testing.assert_close(loss.detach().cpu(), want.detach(), atol=3e-5, rtol=1e-5)
+    torch.testing.assert_close(lg.grad.cpu(), lref.grad, atol=3e-5, rtol=1e-4)
+    assert log["keys"] == ["loss"] and int(norm) == 1
