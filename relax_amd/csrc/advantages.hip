@@ -163,7 +163,9 @@ extern "C" int relax_amd_broadcast_per_sample(const float* per_sample, const int
   return check_launch("broadcast_per_sample");
 }
 
-extern "C" int64_t relax_amd_whiten_partials(int64_t n) { return n <= 0 ? 0 : (n + kWhitenPerBlock - 1) / kWhitenPerBlock; }
+extern "C" int64_t relax_amd_whiten_partials(int64_t n) {
+  return n <= 0 ? 0 : (n + kWhitenPerBlock - 1) / kWhitenPerBlock;
+}
 
 extern "C" int relax_amd_masked_whiten(const float* values, const float* mask, int64_t n, int32_t shift_mean,
                                        float epsilon, double* partials, float* stats, float* out, void* stream) {

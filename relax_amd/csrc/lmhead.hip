@@ -10,9 +10,10 @@
 // 16-byte vector and the wave's 64 vectors land contiguously, i.e. 8 rows x 128 B per instruction.  The LDS has 64
 // four-byte banks and serves 16 lanes of a 16-byte read per clock, so the fragment reads of 16 consecutive rows (same
 // k offset) must hit 16 distinct bank quads: with 128-byte rows the bank quad is (row parity, slot), hence lane
-// (row r, slot v) fetches global vector v ^ ((r >> 1) & 7) and fragment reads apply the same XOR (no padding).  The copy of slice k+1 (or of the next vocabulary tile's
-// first slice) is issued before the MFMAs of slice k and awaited after them, so global latency hides behind 64 MFMAs
-// per wave; fragments for the next 16-wide k-step are fetched from LDS while the current 16 MFMAs issue.
+// (row r, slot v) fetches global vector v ^ ((r >> 1) & 7) and fragment reads apply the same XOR (no padding).
+// The 16 copies of slice k+1 (or of the next vocabulary tile's first slice) are slotted between the 64 MFMAs of slice
+// k, one per two MFMAs, and awaited at the slice boundary; fragments for the next 16-wide k-step are fetched from LDS
+// while the current 16 MFMAs issue.
 //
 // The MFMA "A" operand is the WEIGHT tile and "B" the HIDDEN tile, so in the 32x32 accumulator layout a lane's column
 // is a TOKEN and its 16 registers are 16 vocabulary entries: the online softmax over the vocabulary is then a
@@ -20,6 +21,8 @@
 // and one cross-wave merge at the very end.  Each wave computes 128 vocab x 128 tokens = 4x4 MFMA tiles (256 fp32
 // accumulators per lane, held in AGPRs).  Vocabulary ranges are split over workgroups (flash-decoding style) and
 // merged by a small combine kernel; the target logit comes from a gather-dot kernel (one wave per token).
+// The same pipeline drives the backward's recompute kernel, whose epilogue turns each accumulator block into the
+// gradient w.r.t. the logits and stores it transposed in bf16, and the forward variant that keeps the bf16 logits.
 //
 // Workgroup -> (XCD, row block, vocab split) mapping: hardware places consecutive workgroup ids round-robin on the
 // 8 XCDs; the 32 workgroups resident on one XCD are arranged as (32/S) row blocks x S vocab splits so that hidden
@@ -53,14 +56,14 @@ __device__ __forceinline__ bool lm_block_coords(const LmGeom& g, int& rb, int& s
   return rb < g.row_blocks;
 }
 
+// s_waitcnt immediates, issued through the builtin so that the compiler's own wait-count bookkeeping sees them:
+// "all vector-memory operations done" (vmcnt = 0, expcnt and lgkmcnt left at their maxima), and vmcnt = lgkmcnt = 0.
+constexpr int kLmWaitCopies = 0x0F70;
+constexpr int kLmWaitEverything = 0x0070;
+
 // Asynchronous global -> LDS copy of one 256-row x 64-col bf16 slice of an operand.  Thread t covers row t/8 of each
 // 32-row pass and LDS slot t%8; it fetches global vector (t%8) ^ ((row >> 1) & 7) of that row (the same value for
 // every pass).  Rows past the ragged edge re-read the last valid row; their results are discarded by the caller.
-// s_waitcnt immediate for "all vector-memory operations done" (vmcnt = 0, expcnt and lgkmcnt left at their maxima).
-// Issued through the builtin so that the compiler's own wait-count bookkeeping sees it.
-constexpr int kLmWaitCopies = 0x0F70;
-constexpr int kLmWaitEverything = 0x0070;  // vmcnt = 0 and lgkmcnt = 0
-
 struct LmCopier {
   const unsigned char* base;  // first row of the tile (wave-uniform, lives in scalar registers)
   uint32_t off[kLmPasses];    // byte offset of this thread's vector in each pass, k-slice 0
@@ -311,11 +314,11 @@ __device__ __forceinline__ void lm_absorb_block(const floatx16& blk, int vbase, 
 }
 
 // Writes accumulator blocks, as bf16, into a [vocab, token] matrix (token contiguous).  Addresses are a wave-uniform
-// tile base plus one 32-bit lane offset plus a uniform per-store offset, so the 256 stores of a tile cost one vector add
-// each and no 64-bit lane arithmetic.  Neighbouring lanes hold neighbouring tokens of the same vocabulary rows: with
-// PAIRS an even/odd lane pair swaps one value per two rows and each lane writes two tokens with one 4-byte store, half
-// the store instructions of the 2-byte form (needs an even row stride and a 4-byte aligned matrix).  Tiles that cross
-// the end of the vocabulary or of the tokens take a checked 2-byte path.
+// tile base plus one 32-bit lane offset plus a uniform per-store offset, so the 256 stores of a tile cost one vector
+// add each and no 64-bit lane arithmetic.  Neighbouring lanes hold neighbouring tokens of the same vocabulary rows:
+// with PAIRS an even/odd lane pair swaps one value per two rows and each lane writes two tokens with one 4-byte store,
+// half the store instructions of the 2-byte form (needs an even row stride and a 4-byte aligned matrix).  Tiles that
+// cross the end of the vocabulary or of the tokens take a checked 2-byte path.
 struct LmSlabWriter {
   uint16_t* matrix;
   int64_t stride, vocab, n_tokens, tok0;

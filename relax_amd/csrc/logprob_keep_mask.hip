@@ -198,11 +198,14 @@ extern "C" int relax_amd_logprob_entropy_masked_fwd(const void* logits, int dtyp
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
     case RELAX_AMD_F32:
-      return launch_masked_fwd<float>(logits, n_tokens, vocab, row_stride, row_ids, targets, keep_mask, keep_stride, inv_temperature, log_prob, entropy, lse_kept, lse_full, spx, s);
+      return launch_masked_fwd<float>(logits, n_tokens, vocab, row_stride, row_ids, targets, keep_mask, keep_stride,
+          inv_temperature, log_prob, entropy, lse_kept, lse_full, spx, s);
     case RELAX_AMD_BF16:
-      return launch_masked_fwd<bf16_t>(logits, n_tokens, vocab, row_stride, row_ids, targets, keep_mask, keep_stride, inv_temperature, log_prob, entropy, lse_kept, lse_full, spx, s);
+      return launch_masked_fwd<bf16_t>(logits, n_tokens, vocab, row_stride, row_ids, targets, keep_mask, keep_stride,
+          inv_temperature, log_prob, entropy, lse_kept, lse_full, spx, s);
     case RELAX_AMD_F16:
-      return launch_masked_fwd<f16_t>(logits, n_tokens, vocab, row_stride, row_ids, targets, keep_mask, keep_stride, inv_temperature, log_prob, entropy, lse_kept, lse_full, spx, s);
+      return launch_masked_fwd<f16_t>(logits, n_tokens, vocab, row_stride, row_ids, targets, keep_mask, keep_stride,
+          inv_temperature, log_prob, entropy, lse_kept, lse_full, spx, s);
     default: set_error("logprob_entropy_masked_fwd: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
   }
 }
@@ -226,11 +229,14 @@ extern "C" int relax_amd_logprob_entropy_masked_bwd(const void* logits, int dtyp
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
     case RELAX_AMD_F32:
-      return launch_masked_bwd<float>(logits, n_rows, vocab, row_stride, token_of_row, targets, keep_mask, keep_stride, lse_kept, lse_full, spx, g_lp, g_ent, grad_scale, inv_temperature, dlogits, d_row_stride, s);
+      return launch_masked_bwd<float>(logits, n_rows, vocab, row_stride, token_of_row, targets, keep_mask,
+          keep_stride, lse_kept, lse_full, spx, g_lp, g_ent, grad_scale, inv_temperature, dlogits, d_row_stride, s);
     case RELAX_AMD_BF16:
-      return launch_masked_bwd<bf16_t>(logits, n_rows, vocab, row_stride, token_of_row, targets, keep_mask, keep_stride, lse_kept, lse_full, spx, g_lp, g_ent, grad_scale, inv_temperature, dlogits, d_row_stride, s);
+      return launch_masked_bwd<bf16_t>(logits, n_rows, vocab, row_stride, token_of_row, targets, keep_mask,
+          keep_stride, lse_kept, lse_full, spx, g_lp, g_ent, grad_scale, inv_temperature, dlogits, d_row_stride, s);
     case RELAX_AMD_F16:
-      return launch_masked_bwd<f16_t>(logits, n_rows, vocab, row_stride, token_of_row, targets, keep_mask, keep_stride, lse_kept, lse_full, spx, g_lp, g_ent, grad_scale, inv_temperature, dlogits, d_row_stride, s);
+      return launch_masked_bwd<f16_t>(logits, n_rows, vocab, row_stride, token_of_row, targets, keep_mask,
+          keep_stride, lse_kept, lse_full, spx, g_lp, g_ent, grad_scale, inv_temperature, dlogits, d_row_stride, s);
     default: set_error("logprob_entropy_masked_bwd: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
   }
 }

@@ -161,7 +161,8 @@ __device__ __forceinline__ void opd_entry(float s, float t, float alpha, float l
 
 // One wave per row; `sv`/`tv` are the row's clamped + masked log-probs staged in LDS (k is a run-time size).
 template <bool BWD>
-__global__ __launch_bounds__(256) void opd_kl_topk_kernel(const float* __restrict__ s_lp, const float* __restrict__ t_lp,
+__global__ __launch_bounds__(256) void opd_kl_topk_kernel(const float* __restrict__ s_lp,
+    const float* __restrict__ t_lp,
                                                           const uint8_t* __restrict__ mask, int64_t n_rows, int k_ids,
                                                           OpdParams p, const float* __restrict__ g,
                                                           float* __restrict__ out, float* __restrict__ d_s) {
@@ -307,11 +308,14 @@ extern "C" int relax_amd_topk_logprob_fwd(const void* logits, int dtype, int64_t
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
     case RELAX_AMD_F32:
-      return launch_topk_fwd<float>(logits, n_tokens, vocab, row_stride, row_ids, topk_ids, int(k), inv_temperature, lse_in, topk_log_prob, lse_out, s);
+      return launch_topk_fwd<float>(logits, n_tokens, vocab, row_stride, row_ids, topk_ids, int(k), inv_temperature,
+          lse_in, topk_log_prob, lse_out, s);
     case RELAX_AMD_BF16:
-      return launch_topk_fwd<bf16_t>(logits, n_tokens, vocab, row_stride, row_ids, topk_ids, int(k), inv_temperature, lse_in, topk_log_prob, lse_out, s);
+      return launch_topk_fwd<bf16_t>(logits, n_tokens, vocab, row_stride, row_ids, topk_ids, int(k), inv_temperature,
+          lse_in, topk_log_prob, lse_out, s);
     case RELAX_AMD_F16:
-      return launch_topk_fwd<f16_t>(logits, n_tokens, vocab, row_stride, row_ids, topk_ids, int(k), inv_temperature, lse_in, topk_log_prob, lse_out, s);
+      return launch_topk_fwd<f16_t>(logits, n_tokens, vocab, row_stride, row_ids, topk_ids, int(k), inv_temperature,
+          lse_in, topk_log_prob, lse_out, s);
     default: set_error("topk_logprob_fwd: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
   }
 }
@@ -329,11 +333,14 @@ extern "C" int relax_amd_topk_logprob_bwd(const void* logits, int dtype, int64_t
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
     case RELAX_AMD_F32:
-      return launch_topk_bwd<float>(logits, n_rows, vocab, row_stride, token_of_row, topk_ids, int(k), inv_temperature, lse, g, dlogits, d_stride, s);
+      return launch_topk_bwd<float>(logits, n_rows, vocab, row_stride, token_of_row, topk_ids, int(k),
+          inv_temperature, lse, g, dlogits, d_stride, s);
     case RELAX_AMD_BF16:
-      return launch_topk_bwd<bf16_t>(logits, n_rows, vocab, row_stride, token_of_row, topk_ids, int(k), inv_temperature, lse, g, dlogits, d_stride, s);
+      return launch_topk_bwd<bf16_t>(logits, n_rows, vocab, row_stride, token_of_row, topk_ids, int(k),
+          inv_temperature, lse, g, dlogits, d_stride, s);
     case RELAX_AMD_F16:
-      return launch_topk_bwd<f16_t>(logits, n_rows, vocab, row_stride, token_of_row, topk_ids, int(k), inv_temperature, lse, g, dlogits, d_stride, s);
+      return launch_topk_bwd<f16_t>(logits, n_rows, vocab, row_stride, token_of_row, topk_ids, int(k),
+          inv_temperature, lse, g, dlogits, d_stride, s);
     default: set_error("topk_logprob_bwd: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
   }
 }
@@ -358,7 +365,8 @@ extern "C" int relax_amd_opd_kl_topk_fwd(const float* student_lp, const float* t
                                          int64_t n_rows, int64_t k, int kl_mode, int norm_mode, float jsd_alpha,
                                          int has_clamp, float log_prob_min_clamp, float* kl, void* stream) {
   OpdParams p;
-  if (int rc = opd_params("opd_kl_topk_fwd", kl_mode, norm_mode, jsd_alpha, has_clamp, log_prob_min_clamp, n_rows, k, p))
+  if (int rc = opd_params("opd_kl_topk_fwd", kl_mode, norm_mode, jsd_alpha, has_clamp, log_prob_min_clamp, n_rows, k,
+      p))
     return rc;
   if (n_rows == 0) return RELAX_AMD_OK;
   if (!student_lp || !teacher_lp || !kl) {
@@ -377,7 +385,8 @@ extern "C" int relax_amd_opd_kl_topk_bwd(const float* student_lp, const float* t
                                          int has_clamp, float log_prob_min_clamp, const float* g, float* d_student_lp,
                                          void* stream) {
   OpdParams p;
-  if (int rc = opd_params("opd_kl_topk_bwd", kl_mode, norm_mode, jsd_alpha, has_clamp, log_prob_min_clamp, n_rows, k, p))
+  if (int rc = opd_params("opd_kl_topk_bwd", kl_mode, norm_mode, jsd_alpha, has_clamp, log_prob_min_clamp, n_rows, k,
+      p))
     return rc;
   if (n_rows == 0) return RELAX_AMD_OK;
   if (!student_lp || !teacher_lp || !g || !d_student_lp) {

@@ -415,7 +415,8 @@ extern "C" int relax_amd_reverse_kl_fwd(const void* student, const void* teacher
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
     case RELAX_AMD_F32: return launch_kl_fwd<float>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, s);
-    case RELAX_AMD_BF16: return launch_kl_fwd<bf16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, s);
+    case RELAX_AMD_BF16: return launch_kl_fwd<bf16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t,
+        s);
     case RELAX_AMD_F16: return launch_kl_fwd<f16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, s);
     default: set_error("reverse_kl_fwd: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
   }
@@ -434,11 +435,14 @@ extern "C" int relax_amd_reverse_kl_bwd(const void* student, const void* teacher
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
     case RELAX_AMD_F32:
-      return launch_kl_bwd<float>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, g, grad_scale, grad_scale_dev, dstudent, s);
+      return launch_kl_bwd<float>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, g, grad_scale,
+          grad_scale_dev, dstudent, s);
     case RELAX_AMD_BF16:
-      return launch_kl_bwd<bf16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, g, grad_scale, grad_scale_dev, dstudent, s);
+      return launch_kl_bwd<bf16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, g, grad_scale,
+          grad_scale_dev, dstudent, s);
     case RELAX_AMD_F16:
-      return launch_kl_bwd<f16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, g, grad_scale, grad_scale_dev, dstudent, s);
+      return launch_kl_bwd<f16_t>(student, teacher, n_tokens, vocab, row_stride, kl, lse_s, lse_t, g, grad_scale,
+          grad_scale_dev, dstudent, s);
     default: set_error("reverse_kl_bwd: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
   }
 }
@@ -455,11 +459,14 @@ extern "C" int relax_amd_reverse_kl_step_fused(const void* student, const void* 
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
     case RELAX_AMD_F32:
-      return launch_kl_step<float>(student, teacher, n_tokens, vocab, row_stride, g, grad_scale, kl, lse_s, lse_t, dstudent, s);
+      return launch_kl_step<float>(student, teacher, n_tokens, vocab, row_stride, g, grad_scale, kl, lse_s, lse_t,
+          dstudent, s);
     case RELAX_AMD_BF16:
-      return launch_kl_step<bf16_t>(student, teacher, n_tokens, vocab, row_stride, g, grad_scale, kl, lse_s, lse_t, dstudent, s);
+      return launch_kl_step<bf16_t>(student, teacher, n_tokens, vocab, row_stride, g, grad_scale, kl, lse_s, lse_t,
+          dstudent, s);
     case RELAX_AMD_F16:
-      return launch_kl_step<f16_t>(student, teacher, n_tokens, vocab, row_stride, g, grad_scale, kl, lse_s, lse_t, dstudent, s);
+      return launch_kl_step<f16_t>(student, teacher, n_tokens, vocab, row_stride, g, grad_scale, kl, lse_s, lse_t,
+          dstudent, s);
     default: set_error("reverse_kl_step_fused: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
   }
 }

@@ -7,7 +7,8 @@
 // Both recurrences are y_t = x_t + a * y_{t+1}.  One wave owns one sequence and walks it from the end in 64-token
 // chunks: the chunk is loaded coalesced, lane 0 runs the 64 dependent steps in the reference's order (a multiply and
 // an add, each rounded on its own, so the result is bit-identical to the sequential Python loop), and the chunk is
-// stored coalesced.  The data is a few hundred KB; what matters is one launch instead of one Python iteration per token.
+// stored coalesced.  The data is a few hundred KB; what matters is one launch instead of one Python iteration per
+// token.
 #include "device_utils.h"
 #include "relax_amd.h"
 
