@@ -328,32 +328,36 @@ def run_mfma_ceiling(a, dev) -> None:
     from relax_amd import ops
     from relax_amd._lib import check, lib
 
-    blocks, iters = 256, 20000
+    shape = 1 if a.mfma_shape == "16x16x32" else 0
+    blocks, iters = 256, (10000 if shape else 20000)  # the same FLOP per launch for both shapes
     g = torch.Generator(device=dev).manual_seed(0)
     src = torch.randn(4096 * 8, device=dev, generator=g).bfloat16()
     if a.lmhead_operands == "zeros":
         src.zero_()
-    out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+    out = torch.empty(blocks * 512, dtype=torch.float32, device=dev)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
     def step():
         with ops._timed("diag_mfma_loop"):
             check(lib.relax_amd_diag_mfma_loop(C.c_void_p(src.data_ptr()), C.c_void_p(out.data_ptr()), blocks, iters,
-                                               stream))
+                                               shape, stream))
         return out
 
     with ClockSampler() as clock:
         wall, kernel_ms, launches, _ = timed_steps(step, a.warmup, a.steps)
     clk = clock.summary()
-    flops = blocks * 4 * iters * 64 * 32768.0
+    flops = blocks * (8 * iters * 128 * 16384.0 if shape else 4 * iters * 64 * 32768.0)
     achieved = flops / (kernel_ms["diag_mfma_loop"] * 1e-3) / 1e12
     print(json.dumps({
         "metric": "TFLOP/s of register-fed bf16 MFMAs [diagnostic ceiling, not the headline metric]", "value": achieved,
         "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": wall * 1e3 / a.steps,
         "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "mfma_ceiling: 256 workgroups x 4 waves x 20000 x 64 MFMA 32x32x16 bf16, operands "
+        "config": {"workload": "mfma_ceiling: 256 workgroups x "
+                               + ("8 waves (two per SIMD) x 10000 x 128 MFMA 16x16x32" if shape else
+                                  "4 waves (one per SIMD) x 20000 x 64 MFMA 32x32x16") + " bf16, operands "
                                + ("all zero" if a.lmhead_operands == "zeros" else "N(0, 1)") + ", no memory traffic"},
-        "roofline": {"bound": "mfma", "kernel": "diag_mfma_loop_kernel", "achieved": achieved,
+        "roofline": {"bound": "mfma", "kernel": "diag_mfma_loop16_kernel" if shape else "diag_mfma_loop_kernel",
+                     "achieved": achieved,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": None, "avg_launch_ms": kernel_ms["diag_mfma_loop"], "clock": clk,
                      "frac_at_measured_clock":
@@ -575,6 +579,8 @@ def main() -> int:
                          "projecting a second time (10 GB at the default size)")
     ap.add_argument("--forward-only", action="store_true",
                     help="lmhead workload, diagnostic: time the forward pass alone (clock samples of that kernel only)")
+    ap.add_argument("--mfma-shape", choices=["32x32x16", "16x16x32"], default="32x32x16",
+                    help="mfma_ceiling workload: instruction shape (16x16x32 runs two waves per SIMD)")
     ap.add_argument("--vendor-gemm", action="store_true",
                     help="lmhead workload, diagnostic: time the library's plain GEMM of the forward shape instead of "
                          "the fused kernel (same operands, logits written to HBM), for comparison")

@@ -43,16 +43,57 @@ __global__ __launch_bounds__(256, 1) void diag_mfma_loop_kernel(const diag_bf16x
   out[blockIdx.x * 256 + lane] = sum;
 }
 
+// The same measurement for the 16x16x32 shape.  One wave per SIMD cannot issue these four-pass instructions back to
+// back (measured 66 % of the issue slots), so this variant runs two waves per SIMD with 32 four-register accumulators
+// each: 128 MFMAs of 16x16x32 per iteration and wave, i.e. the same FLOP per iteration as the 32x32x16 loop.
+typedef float diag_floatx4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(512, 1) void diag_mfma_loop16_kernel(const diag_bf16x8* __restrict__ src,
+                                                                  float* __restrict__ out, int iters) {
+  const int lane = threadIdx.x & 255;
+  diag_bf16x8 a[8], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = src[i * 256 + lane];
+    b[i] = src[(i + 8) * 256 + lane];
+  }
+  diag_floatx4 acc[4][8] = {};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          acc[i][j] =
+              __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[(i + ks) & 7], b[(j + 3 * ks) & 7], acc[i][j], 0, 0, 0);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sum += acc[i][j][r];
+  out[blockIdx.x * 512 + threadIdx.x] = sum;
+}
+
 }  // namespace relax_amd
 
 using namespace relax_amd;
 
-extern "C" int relax_amd_diag_mfma_loop(const void* src, float* out, int blocks, int iters, void* stream) {
-  if (!src || !out || blocks <= 0 || iters < 0 || !aligned16(src)) {
-    set_error("diag_mfma_loop: src (4096 x 16 bytes, 16-byte aligned) and out (blocks x 256 floats) are required");
+extern "C" int relax_amd_diag_mfma_loop(const void* src, float* out, int blocks, int iters, int shape, void* stream) {
+  if (!src || !out || blocks <= 0 || iters < 0 || !aligned16(src) || (shape != 0 && shape != 1)) {
+    set_error("diag_mfma_loop: src (4096 x 16 bytes, 16-byte aligned), out (blocks x 512 floats) and shape 0 "
+              "(32x32x16, one wave per SIMD) or 1 (16x16x32, two waves per SIMD) are required");
     return RELAX_AMD_EINVAL;
   }
-  hipLaunchKernelGGL(diag_mfma_loop_kernel, dim3(unsigned(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const diag_bf16x8*>(src), out, iters);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (shape == 0)
+    hipLaunchKernelGGL(diag_mfma_loop_kernel, dim3(unsigned(blocks)), dim3(256), 0, s,
+                       static_cast<const diag_bf16x8*>(src), out, iters);
+  else
+    hipLaunchKernelGGL(diag_mfma_loop16_kernel, dim3(unsigned(blocks)), dim3(512), 0, s,
+                       static_cast<const diag_bf16x8*>(src), out, iters);
   return check_launch("diag_mfma_loop");
 }
