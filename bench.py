@@ -365,6 +365,42 @@ def run_mfma_ceiling(a, dev) -> None:
         "cpu_baseline": None}))
 
 
+def run_hbm_ceiling(a, dev) -> None:
+    """Diagnostic, not a workload of the path: plain read / write / copy streams over a buffer of the actor step's
+    logits size (65536 x 151936 bf16 = 19.9 GB), 16-byte accesses.  What these sustain is the practical ceiling for the
+    bandwidth-bound kernels on this box.  A "step" is one read, one write and one copy launch."""
+    import ctypes as C
+    from relax_amd import ops
+    from relax_amd._lib import check, lib
+
+    nbytes = 65536 * 151936 * 2
+    src = torch.ones(nbytes // 2, dtype=torch.bfloat16, device=dev)
+    dst = torch.empty_like(src)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    p = lambda t: C.c_void_p(t.data_ptr())
+
+    def step():
+        for mode, name in ((0, "diag_stream_read"), (1, "diag_stream_write"), (2, "diag_stream_copy")):
+            with ops._timed(name):
+                check(lib.relax_amd_diag_stream(mode, p(src), p(dst), nbytes, p(sink), stream))
+        return dst
+
+    wall, kernel_ms, launches, _ = timed_steps(step, a.warmup, a.steps)
+    rates = {"read_GBs": nbytes / kernel_ms["diag_stream_read"] / 1e6,
+             "write_GBs": nbytes / kernel_ms["diag_stream_write"] / 1e6,
+             "copy_GBs": 2 * nbytes / kernel_ms["diag_stream_copy"] / 1e6}
+    print(json.dumps({
+        "metric": "GB/s of plain HBM streams [diagnostic ceiling, not the headline metric]", "value": rates["read_GBs"],
+        "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": wall * 1e3 / a.steps,
+        "higher_is_better": True, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "hbm_ceiling: read, write and copy of 19.9 GB with 16-byte accesses", **rates},
+        "roofline": {"bound": "hbm", "kernel": "diag_stream_kernel<0> (read)", "achieved": rates["read_GBs"],
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": rates["read_GBs"] / HBM_PEAK_GBS, "traffic": None,
+                     "kernel_ms": kernel_ms},
+        "cpu_baseline": None}))
+
+
 def run_reverse_kl(a, dev) -> None:
     """student / teacher bf16 logits [N, V], teacher = student + N(0, 1); per-token full-vocabulary reverse KL with a
     15 % zero loss mask, token-mean reduction, backward to the student's dlogits."""
@@ -567,7 +603,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="actor_step",
-                    choices=["actor_step", "cfg1", "lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "mfma_ceiling"])
+                    choices=["actor_step", "cfg1", "lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "mfma_ceiling", "hbm_ceiling"])
     ap.add_argument("--seqs", type=int, default=SEQS)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
     ap.add_argument("--vocab", type=int, default=VOCAB)
@@ -610,6 +646,8 @@ def main() -> int:
         run_lmhead(a, dev)
     elif a.workload == "mfma_ceiling":
         run_mfma_ceiling(a, dev)
+    elif a.workload == "hbm_ceiling":
+        run_hbm_ceiling(a, dev)
     elif a.workload == "reverse_kl":
         run_reverse_kl(a, dev)
     else:

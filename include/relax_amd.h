@@ -418,6 +418,13 @@ int relax_amd_transpose_16bit(const void* in, int64_t rows, int64_t cols, int64_
  */
 int relax_amd_diag_mfma_loop(const void* src, float* out, int blocks, int iters, int shape, void* stream);
 
+/*
+ * Measurement aid with no counterpart in the reference: one plain HBM stream over `bytes` (a multiple of 65536) with
+ * 16-byte accesses.  mode 0 reads src (sink: 4 bytes of device memory, practically never written), mode 1 writes dst,
+ * mode 2 copies src to dst.  bench.py uses it to report the box's streaming ceilings next to the bandwidth-bound kernels.
+ */
+int relax_amd_diag_stream(int mode, const void* src, void* dst, int64_t bytes, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

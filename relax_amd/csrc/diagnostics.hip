@@ -1,4 +1,6 @@
-// Measurement aid, not part of the loss path: the matrix cores fed from registers, with no memory traffic at all.
+// Measurement aids, not part of the loss path.
+//
+// (1) The matrix cores fed from registers, with no memory traffic at all.
 //
 // The published bf16 peak assumes the 2.4 GHz boost clock.  On dense operands with the statistics of real activations
 // the board reaches its power limit long before that, so the number a GEMM-shaped kernel can be held against on a
@@ -78,9 +80,61 @@ __global__ __launch_bounds__(512, 1) void diag_mfma_loop16_kernel(const diag_bf1
   out[blockIdx.x * 512 + threadIdx.x] = sum;
 }
 
+// Plain HBM streams, for the ceiling the bandwidth-bound kernels can be held against on a given box: 16-byte accesses,
+// four in flight per thread, grid-stride over the buffer.  mode 0 reads, 1 writes, 2 copies.
+template <int MODE>
+__global__ __launch_bounds__(1024) void diag_stream_kernel(const u32x4* __restrict__ in, u32x4* __restrict__ out,
+                                                           int64_t n, unsigned* __restrict__ sink) {
+  constexpr int kUnroll = 4;
+  int64_t i = int64_t(blockIdx.x) * 1024 * kUnroll + threadIdx.x;
+  const int64_t stride = int64_t(gridDim.x) * 1024 * kUnroll;
+  unsigned acc = 0;
+  for (; i + 1024 * (kUnroll - 1) < n; i += stride) {
+    u32x4 v[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      if (MODE == 1)
+        v[u] = u32x4{unsigned(i), 2u, 3u, 4u};
+      else
+        v[u] = __builtin_nontemporal_load(in + i + u * 1024);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      if (MODE == 0)
+        acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+      else
+        __builtin_nontemporal_store(v[u], out + i + u * 1024);
+    }
+  }
+  if (MODE == 0 && acc == 0x12345678u) sink[0] = acc;  // keeps the loads alive; practically never true
+}
+
 }  // namespace relax_amd
 
 using namespace relax_amd;
+
+extern "C" int relax_amd_diag_stream(int mode, const void* src, void* dst, int64_t bytes, void* sink, void* stream) {
+  if (mode < 0 || mode > 2 || bytes < 0 || bytes % (16 * 4096) != 0 || (mode != 1 && !src) || (mode != 0 && !dst) ||
+      (mode == 0 && !sink) || !aligned16(src) || !aligned16(dst)) {
+    set_error("diag_stream: mode 0 (read: src, sink) / 1 (write: dst) / 2 (copy: src, dst); bytes a multiple of 65536; "
+              "16-byte aligned buffers");
+    return RELAX_AMD_EINVAL;
+  }
+  if (bytes == 0) return RELAX_AMD_OK;
+  const int64_t n = bytes / 16;
+  const int64_t groups = n / 4096;
+  const dim3 grid(unsigned(groups < 65536 ? groups : 65536)), block(1024);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const u32x4* in = static_cast<const u32x4*>(src);
+  u32x4* out = static_cast<u32x4*>(dst);
+  if (mode == 0)
+    hipLaunchKernelGGL(diag_stream_kernel<0>, grid, block, 0, s, in, out, n, static_cast<unsigned*>(sink));
+  else if (mode == 1)
+    hipLaunchKernelGGL(diag_stream_kernel<1>, grid, block, 0, s, in, out, n, static_cast<unsigned*>(sink));
+  else
+    hipLaunchKernelGGL(diag_stream_kernel<2>, grid, block, 0, s, in, out, n, static_cast<unsigned*>(sink));
+  return check_launch("diag_stream");
+}
 
 extern "C" int relax_amd_diag_mfma_loop(const void* src, float* out, int blocks, int iters, int shape, void* stream) {
   if (!src || !out || blocks <= 0 || iters < 0 || !aligned16(src) || (shape != 0 && shape != 1)) {
