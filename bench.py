@@ -33,10 +33,23 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 PEAK_SCLK_MHZ = 2400.0  # the shader clock the published matrix-core peak is quoted at
 METRIC = "tokens/s fused logprob+entropy+loss fwd+bwd @V=151936 bf16; % HBM/MFMA peak"
-# HBM bytes one actor_step_fused launch moves at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# at the L2 <-> fabric boundary (profiles/actor_step_fused_bf16_v151936_n65536.md): 26 780 743 KiB fetched
-# (counter x 2.000) + 19 464 492 KiB written.
+# HBM bytes one launch of the fused actor step moves at the default workload, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE at the L2 <-> fabric boundary (counter x 2.000 for FETCH_SIZE): the register-resident kernel
+# (profiles/actor_step_resident_bf16_v151936_n65536.md) fetches 15 664 908 KiB and writes 19 469 551 KiB; the two-walk
+# kernel (profiles/actor_step_fused_bf16_v151936_n65536.md, RELAX_AMD_FUSED_STEP_KERNEL=cached) 26 780 743 + 19 464 492.
+MEASURED_TRAFFIC_RESIDENT = (15664908 + 19469551) * 1024.0
 MEASURED_TRAFFIC_FUSED = (26780743 + 19464492) * 1024.0
+
+
+def fused_step_kernel_name(vocab: int) -> str:
+    """Which kernel relax_amd_actor_step_fused runs for bf16 rows of ``vocab`` entries (the library's own rule)."""
+    nvec = vocab // 8
+    shape = (nvec // 1024, nvec % 1024 != 0)
+    if vocab % 8 == 0 and shape in ((18, True), (15, True), (16, False), (12, True)) \
+            and os.environ.get("RELAX_AMD_FUSED_STEP_KERNEL") != "cached":
+        return f"actor_step_resident_kernel<bf16_t, {shape[0]}, {str(shape[1]).lower()}>"
+    threads = 1024 if nvec >= 8192 else 512 if nvec >= 2048 else 256
+    return f"actor_step_fused_kernel<bf16_t, true, {threads}>"
 
 
 def make_args():
@@ -238,8 +251,11 @@ def run_actor_step(a, dev) -> None:
     if "actor_step_fused" in kernel_ms:
         # one launch does the forward scan and the dlogits backward: 3*V*s algorithmic bytes per token (forward read,
         # backward read, dlogits write); its second read is served by cache, see "traffic"
-        dom, dom_name, dom_bytes = kernel_ms["actor_step_fused"], "actor_step_fused_kernel<bf16_t, true, 1024>", 3.0 * row_bytes
-        traffic = MEASURED_TRAFFIC_FUSED if (a.vocab, n_tokens) == (VOCAB, SEQS * SEQ_LEN) else None
+        dom, dom_bytes = kernel_ms["actor_step_fused"], 3.0 * row_bytes
+        dom_name = fused_step_kernel_name(a.vocab)
+        traffic = None
+        if (a.vocab, n_tokens) == (VOCAB, SEQS * SEQ_LEN):
+            traffic = MEASURED_TRAFFIC_RESIDENT if "resident" in dom_name else MEASURED_TRAFFIC_FUSED
     else:
         dom, dom_name, dom_bytes = kernel_ms["logprob_entropy_bwd"], "logprob_entropy_bwd_kernel<bf16_t, true>", 2.0 * row_bytes
         traffic = None
@@ -590,7 +606,8 @@ def run_varlen(a, dev, loss_kind: str) -> None:
          f"packed varlen: {seqs} sequences {lengths} = {n} rows x V={v} bf16 logits, ~30 % masked spans, RLOO "
          f"advantages, {loss_kind.upper()} loss, sequence-mean-token-sum, fwd + bwd to dlogits",
          {"rows": n, "vocab": v, "loss": float(loss.item()), "lengths": lengths},
-         {"bound": "hbm", "kernel": name + "_kernel<bf16_t>", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+         {"bound": "hbm", "kernel": fused_step_kernel_name(v) if name == "actor_step_fused" else name + "_kernel<bf16_t>",
+          "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
           "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": dom_bytes,
           "avg_launch_ms": dom, "kernel_ms": kernel_ms,
           "step_algorithmic_GBs": 3.0 * row_bytes / (wall / a.steps) / 1e9},

@@ -36,9 +36,21 @@ def sources() -> list[str]:
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
+def _file_flags(src: str) -> list[str]:
+    """Extra compiler flags a source file asks for itself, on ``// hipcc-flags: ...`` lines of its leading comment."""
+    flags: list[str] = []
+    with open(src) as f:
+        for line in f:
+            if not line.startswith("//"):
+                break
+            if line.startswith("// hipcc-flags:"):
+                flags += line[len("// hipcc-flags:"):].split()
+    return flags
+
+
 def _compile(src: str) -> str:
     obj = os.path.join(BUILD_DIR, os.path.basename(src)[:-4] + ".o")
-    cmd = [HIPCC, *FLAGS, "-c", src, "-o", obj]
+    cmd = [HIPCC, *FLAGS, *_file_flags(src), "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")

@@ -25,6 +25,11 @@
 #include "relax_amd.h"
 #include "row_scan.h"
 
+#include <cstdlib>
+#include <cstring>
+
+#include "actor_step_resident.h"
+
 namespace relax_amd {
 
 template <typename T, bool VEC, int THREADS>
@@ -169,6 +174,22 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
   }
 }
 
+// RELAX_AMD_FUSED_STEP_KERNEL = "cached" forces the two-walk kernel (second walk out of cache); unset or anything
+// else lets the row lengths the register-resident kernel is built for take that one.  Read at every launch; meant for
+// measurements.
+static bool fused_step_force_cached() {
+  const char* e = getenv("RELAX_AMD_FUSED_STEP_KERNEL");
+  return e && strcmp(e, "cached") == 0;
+}
+
+static int device_compute_units() {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    return 256;
+  return cus;
+}
+
 template <typename T>
 static int dispatch_fused(const void* logits, int64_t n_rows, int64_t vocab, int64_t stride,
                           const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets, float inv_t,
@@ -179,6 +200,11 @@ static int dispatch_fused(const void* logits, int64_t n_rows, int64_t vocab, int
   const T* x = static_cast<const T*>(logits);
   T* d = static_cast<T*>(dlogits);
   dim3 grid(static_cast<unsigned>(n_rows));
+  if (vec && !fused_step_force_cached()) {
+    const int rc = launch_actor_step_resident<T>(x, stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t, a,
+                                                 grad_scale, lp, ent, lse, spx, d, d_stride, device_compute_units(), s);
+    if (rc != RELAX_AMD_EUNSUPPORTED) return rc;  // launched (or failed to): otherwise the row length is not built
+  }
 #define RELAX_AMD_FUSED(V, TH)                                                                                     \
   hipLaunchKernelGGL((actor_step_fused_kernel<T, V, TH>), grid, dim3(TH), 0, s, x, stride, vocab, token_of_row,       \
                      sample_ids, targets, inv_t * kLog2e, inv_t, a, grad_scale, lp, ent, lse, spx, d, d_stride)

@@ -1,0 +1,342 @@
+// Register-resident fused actor step: the same computation as actor_step_fused_kernel (log-prob + entropy forward,
+// per-token policy-loss coefficients, dlogits backward, one launch) for long 16-bit rows of the common vocabulary sizes.
+//
+// A 1024-thread workgroup holds a whole row in its vector registers (V = 151936 bf16 is 18992 16-byte vectors = 19 per
+// thread = 76 registers), so HBM sees exactly one read and one write per row and the second walk over the row costs no
+// cache or fabric traffic at all.  One such workgroup fits a CU; to keep loads, arithmetic and stores of different rows
+// overlapped the workgroups are persistent (one per CU, rows b, b + grid, ...) and roll the next row in behind the
+// stores of the current one: as soon as a vector's gradient has been stored, its registers receive the same vector of
+// the workgroup's next live row, and a few vectors behind the loads the next row's softmax scan follows.  No workgroup
+// waits for another; the loop bound is the only exit condition.
+//
+// The number of vectors per thread is a template parameter (full vector positions NVF, plus one partially filled
+// position when PARTIAL), so the store / load loop is straight-line code without per-lane bounds checks.  That matters
+// for more than instruction count: the compiler can only count how many loads and stores may stay in flight at each
+// later use when no branch separates them; behind bounds checks it waits for all of them, stores included, several times
+// per row.  Row lengths without an instantiation take the two-walk kernel.
+//
+// The scan over the registers repeats scan_row()'s grouping and order exactly (four vectors absorbed together while a
+// thread has four to go, then single vectors; waves merged in index order), so log-probs stay bit-identical to the
+// forward-only kernel's, which Relax's step-0 check (ppo_kl == 0 for identical weights) relies on.
+//
+// Replaces, like the two-walk kernel, _VocabParallelLogProbEntropy.forward + .backward
+// (relax/utils/training/ppo_utils.py:481-629) and the per-token part of policy_loss_function
+// (relax/backends/megatron/loss.py:961-1100) for one micro-batch.
+//
+// The kernels sit at the edge of the register file (76 of 128 registers hold the row).  With the scheduler's generic
+// register-pressure tracking the allocator ends up parking parts of the row in scratch memory; with the AMDGPU
+// trackers it does not:
+// hipcc-flags: -mllvm -amdgpu-use-amdgpu-trackers=1
+#include "actor_step_resident.h"
+
+#include "device_utils.h"
+#include "loss_math.h"
+#include "row_scan.h"
+
+namespace relax_amd {
+
+constexpr int kResThreads = 1024;
+constexpr int kResLag = 4;  // vector positions between a load and the scan step that uses it
+
+// scan_absorb() over the values of kScanUnroll raw vectors, without holding them all unpacked
+template <typename T>
+__device__ __forceinline__ void absorb_raw_group(const u32x4* raw, float c, SoftmaxAcc& st) {
+  constexpr int VN = Row<T>::kPerVec;
+  float vmax = 0.f;
+#pragma unroll
+  for (int u = 0; u < kScanUnroll; ++u) {
+    float v[VN];
+    Row<T>::unpack(raw[u], v);
+#pragma unroll
+    for (int k = 0; k < VN; ++k) vmax = (u == 0 && k == 0) ? v[0] : fmaxf(vmax, v[k]);
+    __builtin_amdgcn_sched_barrier(0);  // one vector's worth of temporaries at a time (see the callers)
+  }
+  const float mc = __fmul_rn(vmax, c);
+  if (mc > st.m) {
+    const float sc = fast_exp2(__fsub_rn(st.m, mc));
+    st.s = __fmul_rn(st.s, sc);
+    st.t = __fmul_rn(st.t, sc);
+    st.m = mc;
+  }
+#pragma unroll
+  for (int u = 0; u < kScanUnroll; ++u) {
+    // unpack again from an opaque copy of the raw vector: the 32 values of the first walk kept alive (which is what
+    // common-subexpression elimination would do) do not fit the register file next to the resident row
+    u32x4 r = raw[u];
+    asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w));
+    float v[VN];
+    Row<T>::unpack(r, v);
+#pragma unroll
+    for (int k = 0; k < VN; ++k) {
+      const float e = fast_exp2(fmaf(v[k], c, -st.m));
+      st.s = __fadd_rn(st.s, e);
+      st.t = fmaf(e, v[k], st.t);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// What thread 0 needs of a token before it can evaluate the loss terms.
+struct ResidentTokenData {
+  TokenInputs in;
+  float x_target, den, pg_den;
+  int64_t tg;
+};
+
+template <typename T, int NVF, bool PARTIAL>
+__global__ __launch_bounds__(kResThreads, 4) void actor_step_resident_kernel(
+    const T* __restrict__ logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
+    const int32_t* __restrict__ token_of_row, const int32_t* __restrict__ sample_ids,
+    const int64_t* __restrict__ targets, float c, float inv_t, relax_amd_policy_loss_args a, float grad_scale,
+    float* __restrict__ log_prob, float* __restrict__ entropy, float* __restrict__ lse_out,
+    float* __restrict__ spx_out, T* __restrict__ dlogits, int64_t d_stride) {
+  constexpr int THREADS = kResThreads, LAG = kResLag, kU = kScanUnroll;
+  constexpr int VN = Row<T>::kPerVec;
+  constexpr int NV = NVF + (PARTIAL ? 1 : 0);  // vector positions per thread
+  constexpr int kGroups = (NV + kU - 1) / kU;
+  __shared__ float wave_state[THREADS / kWave][3];
+  __shared__ float bc[5];
+  __shared__ int64_t bc_target;
+  const int tid = threadIdx.x;
+  const bool wave0 = __builtin_amdgcn_readfirstlane(tid) < kWave;  // scalar: other waves branch around thread 0's work
+  const int rem = int(vocab / VN) - NVF * THREADS;  // lanes that hold a vector at the partial position (host-checked)
+  u32x4 reg[NV];
+
+  // does this lane hold a vector at position j?  A compile-time answer except at the partial position.
+  auto has = [&](int j) -> bool { return j < NVF || (PARTIAL && j == NVF && tid < rem); };
+
+  // token of a row, or -1 when the row scores nothing or both of its masks are zero (uniform over the workgroup)
+  auto live_token = [&](int64_t row) -> int64_t {
+    if (row >= n_rows) return -1;
+    const int64_t tok = token_of_row ? int64_t(token_of_row[row]) : row;
+    if (tok < 0) return -1;
+    const float m = a.loss_mask[tok];
+    const float mp = a.pg_loss_mask ? a.pg_loss_mask[tok] : m;
+    return (m == 0.f && mp == 0.f) ? -1 : tok;
+  };
+  auto fetch_token = [&](int64_t row, int64_t tok) {
+    ResidentTokenData td{};
+    td.tg = -1;
+    if (wave0 && tok >= 0) {
+      if (tid == 0) {
+        td.in = load_token_inputs(a, tok);
+        td.tg = targets[tok];
+        if (td.tg >= 0 && td.tg < vocab) td.x_target = Row<T>::load1(logits + row * row_stride + td.tg);
+        const int32_t sid = sample_ids ? sample_ids[tok] : 0;
+        td.den = a.sample_denom ? a.sample_denom[sid] : 1.0f;
+        td.pg_den = a.pg_sample_denom ? a.pg_sample_denom[sid] : td.den;
+      }
+    }
+    return td;
+  };
+  // group g of the resident row into st, following scan_row(): four vectors together while this thread still has
+  // four to go, single vectors afterwards (g is a compile-time constant at every call site)
+  auto absorb_group = [&](int g, SoftmaxAcc& st, bool& grouped) {
+    if (grouped && kU * g + kU - 1 < NV && has(kU * g + kU - 1)) {
+      absorb_raw_group<T>(&reg[kU * g < NV - kU ? kU * g : NV - kU], c, st);
+    } else {
+      grouped = false;
+#pragma unroll
+      for (int u = 0; u < kU; ++u)
+        if (kU * g + u < NV && has(kU * g + u)) {
+          float v[VN];
+          Row<T>::unpack(reg[kU * g + u < NV ? kU * g + u : NV - 1], v);
+          scan_absorb(v, c, st);
+        }
+    }
+    // The state is only needed once the whole row is in; without a use here the compiler moves the scan of every
+    // group behind the store loop and spills the vectors it was meant to consume on the way.
+    asm volatile("" : "+v"(st.m), "+v"(st.s), "+v"(st.t));
+    __builtin_amdgcn_sched_barrier(0);  // and one group at a time: hoisting the next group's unpacking spills too
+  };
+  // writes zeros to the per-token outputs of rows that score a token whose masks are both zero, and zero rows
+  auto zero_row = [&](int64_t row) {
+    const int64_t t0 = token_of_row ? int64_t(token_of_row[row]) : row;
+    if (t0 >= 0 && tid == 0) {
+      log_prob[t0] = 0.f;
+      entropy[t0] = 0.f;
+      lse_out[t0] = 0.f;
+      spx_out[t0] = 0.f;
+      a.coef_log_prob[t0] = 0.f;
+      if (a.coef_entropy) a.coef_entropy[t0] = 0.f;
+    }
+    u32x4* dv = reinterpret_cast<u32x4*>(dlogits + row * d_stride);
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+      if (has(j)) store_stream(dv + tid + j * THREADS, u32x4{0u, 0u, 0u, 0u});
+  };
+  // this workgroup's first live row at or after `row` (n_rows or more: none); the dead rows passed on the way are
+  // zero-filled here, so the main loop only ever sees live rows
+  auto advance = [&](int64_t row) -> int64_t {
+    while (row < n_rows && live_token(row) < 0) {
+      zero_row(row);
+      row += gridDim.x;
+    }
+    return row;
+  };
+
+  // prologue: the first live row is loaded and scanned on its own
+  int64_t row = advance(blockIdx.x);
+  if (row >= n_rows) return;
+  int64_t tok = live_token(row);
+  SoftmaxAcc st{kNegHuge, 0.f, 0.f};
+  {
+    const u32x4* xv = reinterpret_cast<const u32x4*>(logits + row * row_stride);
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+      if (has(j)) reg[j] = load_stream(xv + tid + j * THREADS);
+    bool grouped = true;
+#pragma unroll
+    for (int g = 0; g < kGroups; ++g) absorb_group(g, st, grouped);
+  }
+
+  while (true) {
+    const int64_t next = advance(row + gridDim.x);
+    const bool has_next = next < n_rows;
+    const int64_t next_tok = has_next ? live_token(next) : -1;
+
+    // Thread 0's view of the token.  The per-token vectors are a few hundred KB and stay in cache, so fetching them
+    // here, behind the merge of the waves' partial states, costs less than carrying them through the scan in
+    // registers that every wave would have to set aside.
+    const ResidentTokenData td = fetch_token(row, tok);
+    scan_block_merge<THREADS>(st, wave_state);
+    if (wave0) {
+      if (tid == 0) {
+        float lse, spx, ent, lp;
+        scan_finish(st, td.x_target, td.tg >= 0 && td.tg < vocab, inv_t, lse, spx, ent, lp);
+        log_prob[tok] = lp;
+        entropy[tok] = ent;
+        lse_out[tok] = lse;
+        spx_out[tok] = spx;
+        relax_amd_policy_loss_args al = a;
+        // opaque copies: derived constants (1 + eps, ...) would otherwise be hoisted out of the row loop into vector
+        // registers that every wave has to keep for thread 0's sake
+        asm volatile("" : "+s"(al.eps_clip), "+s"(al.eps_clip_high), "+s"(al.eps_clip_c), "+s"(al.entropy_coef),
+                     "+s"(al.kl_coef), "+s"(al.tis_lo), "+s"(al.tis_hi), "+s"(al.tau_pos), "+s"(al.tau_neg));
+        const TokenResult tr = token_terms(al, td.in, lp, ent, false, 0.f, td.den, td.pg_den);
+        a.coef_log_prob[tok] = tr.coef_lp;
+        if (a.coef_entropy) a.coef_entropy[tok] = tr.coef_ent;
+        const float glp = tr.coef_lp * grad_scale, gh = tr.coef_ent * grad_scale;
+        const float b = gh * inv_t;
+        bc[0] = -lse * kLog2e;           // k0: p = exp2(x*c + k0)
+        bc[1] = -glp * inv_t + b * spx;  // a0
+        bc[2] = -b * inv_t;              // a1: d = p * (a0 + a1*x)
+        bc[3] = glp * inv_t;             // added at the target
+        bc[4] = (glp == 0.f && gh == 0.f) ? 1.f : 0.f;
+        bc_target = td.tg;
+      }
+    }
+    // the barrier's fence also waits for this wave's outstanding loads and stores; all of this row's data is in
+    // registers by now, so that costs at most the drain of the previous row's last stores
+    __syncthreads();
+    const float k0 = bc[0], a0 = bc[1], a1 = bc[2], hot = bc[3];
+    const int64_t tg = bc_target;
+    const bool emit_zero = bc[4] != 0.f;  // both gradient coefficients vanish: a zero row, whatever the logits hold
+
+    // The gradient of this row goes out vector by vector; each vector's registers then receive the same vector of
+    // the next live row, and LAG positions behind the loads the next row's scan follows.
+    u32x4* dv = reinterpret_cast<u32x4*>(dlogits + row * d_stride);
+    const u32x4* nxv = reinterpret_cast<const u32x4*>(logits + (has_next ? next : row) * row_stride);
+    const int tvec = (tg >= 0 && tg < vocab) ? int(tg / VN) : -1;
+    const int tsub = int(tg % VN);
+    st = SoftmaxAcc{kNegHuge, 0.f, 0.f};
+    bool grouped = true;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      int lane_id = tid;
+      asm volatile("" : "+v"(lane_id));  // recomputed per vector: 19 loop-invariant index registers would not fit
+      const int idx = lane_id + j * THREADS;
+      float v[VN];
+      Row<T>::unpack(reg[j], v);
+#pragma unroll
+      for (int k = 0; k < VN; ++k) {
+        v[k] = fast_exp2(fmaf(v[k], c, k0)) * fmaf(v[k], a1, a0);
+        // half a vector in flight at a time: with all eight interleaved the temporaries push parts of the resident
+        // row out to scratch (four waves per SIMD cover the latency of the exponentials)
+        if (k == VN / 2 - 1) __builtin_amdgcn_sched_barrier(0);
+      }
+      if (idx == tvec) {  // one lane of the workgroup per row; no memory operation inside, so waits stay countable
+#pragma unroll
+        for (int k = 0; k < VN; ++k)
+          if (k == tsub) v[k] += hot;
+      }
+      u32x4 out = Row<T>::pack(v);
+      if (emit_zero) out = u32x4{0u, 0u, 0u, 0u};
+      if (has(j)) {
+        store_stream(dv + idx, out);
+        // without a next row the row itself is read again: a branch here would cost the precise wait counts, and
+        // the last row of a workgroup is one in hundreds
+        reg[j] = load_stream(nxv + idx);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // one vector at a time: hoisting the next one's unpacking spills
+      if (j - LAG - (kU - 1) >= 0 && (j - LAG - (kU - 1)) % kU == 0)
+        absorb_group((j - LAG - (kU - 1)) / kU, st, grouped);
+    }
+    if (!has_next) return;
+#pragma unroll
+    for (int g = 0; g < kGroups; ++g)
+      if (kU * g + kU - 1 + LAG > NV - 1) absorb_group(g, st, grouped);
+    row = next;
+    tok = next_tok;
+  }
+}
+
+template <typename T>
+struct ResidentSupported {
+  static constexpr bool value = false;
+};
+template <>
+struct ResidentSupported<bf16_t> {
+  static constexpr bool value = true;
+};
+template <>
+struct ResidentSupported<f16_t> {
+  static constexpr bool value = true;
+};
+
+template <typename T>
+int launch_actor_step_resident(const T* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
+                               const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,
+                               float inv_t, const relax_amd_policy_loss_args& a, float grad_scale, float* log_prob,
+                               float* entropy, float* lse, float* spx, T* dlogits, int64_t d_stride,
+                               int compute_units, hipStream_t stream) {
+  if constexpr (!ResidentSupported<T>::value) {
+    return RELAX_AMD_EUNSUPPORTED;
+  } else {
+    constexpr int VN = Row<T>::kPerVec;
+    if (vocab % VN != 0 || scan_threads(vocab, VN) != kResThreads) return RELAX_AMD_EUNSUPPORTED;
+    const int64_t nvec = vocab / VN;
+    const int full = int(nvec / kResThreads);
+    const bool partial = nvec % kResThreads != 0;
+    const int64_t blocks = n_rows < compute_units ? n_rows : compute_units;
+    const dim3 grid(static_cast<unsigned>(blocks)), block(kResThreads);
+#define RELAX_AMD_RESIDENT(NVF, PARTIAL)                                                                             \
+  if (full == NVF && partial == PARTIAL) {                                                                            \
+    hipLaunchKernelGGL((actor_step_resident_kernel<T, NVF, PARTIAL>), grid, block, 0, stream, logits, row_stride,    \
+                       vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a, grad_scale,       \
+                       log_prob, entropy, lse, spx, dlogits, d_stride);                                              \
+    return check_launch("actor_step_resident");                                                                      \
+  }
+    // vocabularies of 151936 / 152064 (18992 / 19008 vectors), 128256 / 129280 (16032 / 16160), 131072 (16384),
+    // 100352 / 102400 (12544 / 12800) entries
+    RELAX_AMD_RESIDENT(18, true)
+    RELAX_AMD_RESIDENT(15, true)
+    RELAX_AMD_RESIDENT(16, false)
+    RELAX_AMD_RESIDENT(12, true)
+#undef RELAX_AMD_RESIDENT
+    return RELAX_AMD_EUNSUPPORTED;
+  }
+}
+
+template int launch_actor_step_resident<float>(const float*, int64_t, int64_t, int64_t, const int32_t*, const int32_t*,
+                                               const int64_t*, float, const relax_amd_policy_loss_args&, float, float*,
+                                               float*, float*, float*, float*, int64_t, int, hipStream_t);
+template int launch_actor_step_resident<bf16_t>(const bf16_t*, int64_t, int64_t, int64_t, const int32_t*,
+                                                const int32_t*, const int64_t*, float,
+                                                const relax_amd_policy_loss_args&, float, float*, float*, float*,
+                                                float*, bf16_t*, int64_t, int, hipStream_t);
+template int launch_actor_step_resident<f16_t>(const f16_t*, int64_t, int64_t, int64_t, const int32_t*, const int32_t*,
+                                               const int64_t*, float, const relax_amd_policy_loss_args&, float, float*,
+                                               float*, float*, float*, f16_t*, int64_t, int, hipStream_t);
+
+}  // namespace relax_amd

@@ -711,3 +711,40 @@ def test_custom_loss_function_path_dispatch():
     torch.testing.assert_close(loss.detach().cpu(), want.detach(), atol=3e-5, rtol=1e-5)
     torch.testing.assert_close(lg.grad.cpu(), lref.grad, atol=3e-5, rtol=1e-4)
     assert log["keys"] == ["loss"] and int(norm) == 1
+
+
+@pytest.mark.parametrize("v,dtype,n_samples", [(100352, torch.bfloat16, 18), (128256, torch.float16, 18),
+                                                (131072, torch.bfloat16, 18), (151936, torch.bfloat16, 18),
+                                                (65536, torch.bfloat16, 18)])
+def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples):
+    """More logits rows than persistent workgroups, so every workgroup of the register-resident kernel rolls several
+    rows through its registers (prompt rows, fully masked samples and masked tokens in between), for every row shape
+    the kernel is built for (12 / 15 / 18 full vectors per thread plus a partial one, 16 exactly) and one it is not
+    (65536: two-walk kernel): same loss bits as the two-launch path, gradients equal to it and to the oracle."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("register-resident step, many rows", v, dtype, n_samples)
+    g = torch.Generator().manual_seed(v + n_samples)
+    tot = [int(x) for x in torch.randint(20, 60, (n_samples,), generator=g)]
+    resp = [int(torch.randint(1, t, (1,), generator=g)) for t in tot]
+    logits, batch = _make_batch(29, tot, resp, v, dtype)
+    batch["loss_masks"][3] = torch.zeros_like(batch["loss_masks"][3])
+    assert sum(tot) > 600
+    db = _to_dev(batch, dev)
+    kw = dict(eps_clip_high=0.28, use_kl_loss=True, kl_loss_coef=1e-3, kl_loss_type="k3", entropy_coef=0.01)
+    outs = {}
+    for mode in ("auto", "off"):
+        lg = logits.to(dev).requires_grad_()
+        loss, met = relax_amd.policy_loss_function(P.make_args(relax_amd_single_pass=mode, **kw), db, lg, None)
+        loss.backward()
+        outs[mode] = (loss.detach(), met, lg.grad)
+    assert torch.equal(outs["auto"][0], outs["off"][0])
+    ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    torch.testing.assert_close(outs["auto"][2].float(), outs["off"][2].float(), atol=1e-6, rtol=ulp)
+    lo = logits.float().clone().requires_grad_()
+    want, _ = P.policy_loss_function(P.make_args(**kw), dict(batch), lo, R.make_reducer(resp, batch["loss_masks"]))
+    want.backward()
+    tol = 2e-3
+    assert abs(outs["auto"][0].item() - want.item()) < tol * max(1.0, abs(want.item()))
+    torch.testing.assert_close(outs["auto"][2].float().cpu(), lo.grad, atol=tol, rtol=max(ulp, 1e-5))
