@@ -748,3 +748,63 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
     tol = 2e-3
     assert abs(outs["auto"][0].item() - want.item()) < tol * max(1.0, abs(want.item()))
     torch.testing.assert_close(outs["auto"][2].float().cpu(), lo.grad, atol=tol, rtol=max(ulp, 1e-5))
+
+
+@pytest.mark.parametrize("pattern", ["all_dead", "one_live_last", "few_live", "random", "all_live_no_map",
+                                     "zero_advantage"])
+def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, monkeypatch):
+    """The two kernels behind relax_amd_actor_step_fused, switched with RELAX_AMD_FUSED_STEP_KERNEL, on row / token
+    layouts that stress the persistent loop of the register-resident one: no live row at all, a single live row at
+    the very end, fewer live rows than workgroups, random prompt rows and masked tokens over several rows per
+    workgroup, no row map (every row scores its own token), and tokens whose gradient coefficients vanish (zero
+    rows without a look at the logits).  Every output must be bit-identical."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("resident vs two-walk", pattern)
+    v, n_rows = 100352, 700  # 12 full vectors per thread + a partial one
+    g = torch.Generator().manual_seed(len(pattern))
+    logits = (torch.randn(n_rows, v, generator=g) * 2).bfloat16().to(dev)
+    if pattern == "all_live_no_map":
+        token_of_row, n_tok = None, n_rows
+    else:
+        scores = torch.rand(n_rows, generator=g) > 0.25
+        idx = torch.cumsum(scores.int(), 0) - 1
+        token_of_row = torch.where(scores, idx, torch.full_like(idx, -1)).int().to(dev)
+        n_tok = int(scores.sum())
+    mask = (torch.rand(n_tok, generator=g) > 0.2).float()
+    if pattern == "all_dead":
+        mask.zero_()
+    elif pattern == "one_live_last":
+        mask.zero_()
+        mask[-1] = 1.0
+    elif pattern == "few_live":
+        mask.zero_()
+        mask[torch.randperm(n_tok, generator=g)[:37]] = 1.0
+    adv = torch.randn(n_tok, generator=g)
+    if pattern == "zero_advantage":
+        adv[::3] = 0.0  # PPO-clip without KL or entropy terms: coefficient exactly zero
+    base = -2.0 + 0.3 * torch.randn(n_tok, generator=g)
+    lens = [n_tok // 3, n_tok - n_tok // 3]
+    cu = torch.tensor([0, lens[0], n_tok], dtype=torch.int64, device=dev)
+    sample_ids = torch.cat([torch.full((n,), i, dtype=torch.int32) for i, n in enumerate(lens)]).to(dev)
+    kw = dict(advantages=adv.to(dev), loss_mask=mask.to(dev), cu_resp=cu, old_log_prob=base.to(dev),
+              sample_denom=torch.tensor([max(1.0, mask[:lens[0]].sum().item()), max(1.0, mask[lens[0]:].sum().item())],
+                                        device=dev),
+              loss_kind="ppo", eps_clip=0.2, eps_clip_high=0.28)
+    if pattern != "zero_advantage":
+        kw.update(ref_log_prob=(base + 0.1 * torch.randn(n_tok, generator=g)).to(dev), kl_kind="k3", kl_coef=1e-3,
+                  entropy_coef=0.01)
+    targets = torch.randint(0, v, (n_tok,), generator=g).to(dev)
+    results = {}
+    for kind in ("cached", "resident"):
+        monkeypatch.setenv("RELAX_AMD_FUSED_STEP_KERNEL", kind)
+        out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, token_of_row, sample_ids, n_tok, 1.0, 1.0, **kw)
+        torch.cuda.synchronize()
+        results[kind] = dict(lp=lp, ent=ent, lse=lse, spx=spx, d=d.view(torch.int16), coef=out["coef_log_prob"],
+                             coef_ent=out["coef_entropy"], metrics=out["metrics"])
+    for key, want in results["cached"].items():
+        got = results["resident"][key]
+        assert torch.equal(got, want), (pattern, key, (got.float() - want.float()).abs().max())
+    if pattern == "all_dead":
+        assert not results["resident"]["d"].any()
