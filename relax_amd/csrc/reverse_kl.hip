@@ -8,54 +8,13 @@
 // Backward: d KL / d x_s[v] = p_s[v] * ((log p_s[v] - log p_t[v]) - KL); reads both rows once, writes one.
 #include "device_utils.h"
 #include "relax_amd.h"
+#include "reverse_kl_math.h"
+#include "reverse_kl_resident.h"
+
+#include <cstdlib>
+#include <cstring>
 
 namespace relax_amd {
-
-constexpr int kKlThreads = 256;
-constexpr int kKlUnroll = 2;
-
-struct KlState {
-  float ms, ss, us, mt, st;
-};
-
-template <int K>
-__device__ __forceinline__ void absorb_pair(const float (&xs)[K], const float (&xt)[K], KlState& q) {
-  float smax = xs[0], tmax = xt[0];
-#pragma unroll
-  for (int i = 1; i < K; ++i) {
-    smax = fmaxf(smax, xs[i]);
-    tmax = fmaxf(tmax, xt[i]);
-  }
-  const float sm = smax * kLog2e, tm = tmax * kLog2e;
-  if (sm > q.ms) {
-    const float sc = fast_exp2(q.ms - sm);
-    q.ss *= sc;
-    q.us *= sc;
-    q.ms = sm;
-  }
-  if (tm > q.mt) {
-    q.st *= fast_exp2(q.mt - tm);
-    q.mt = tm;
-  }
-#pragma unroll
-  for (int i = 0; i < K; ++i) {
-    const float es = fast_exp2(fmaf(xs[i], kLog2e, -q.ms));
-    const float et = fast_exp2(fmaf(xt[i], kLog2e, -q.mt));
-    q.ss += es;
-    q.us = fmaf(es, xs[i] - xt[i], q.us);
-    q.st += et;
-  }
-}
-
-__device__ __forceinline__ void merge_kl(KlState& a, const KlState& b) {
-  const float ms = fmaxf(a.ms, b.ms), mt = fmaxf(a.mt, b.mt);
-  const float fa = fast_exp2(a.ms - ms), fb = fast_exp2(b.ms - ms);
-  a.ss = a.ss * fa + b.ss * fb;
-  a.us = a.us * fa + b.us * fb;
-  a.st = a.st * fast_exp2(a.mt - mt) + b.st * fast_exp2(b.mt - mt);
-  a.ms = ms;
-  a.mt = mt;
-}
 
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kKlThreads) void reverse_kl_fwd_kernel(const T* __restrict__ student,
@@ -347,6 +306,16 @@ static int launch_kl_step(const void* s, const void* t, int64_t n, int64_t vocab
                           float scale, float* kl, float* ls, float* lt, void* d, hipStream_t st) {
   const bool vec = aligned16(s) && aligned16(t) && aligned16(d) && (stride * int64_t(sizeof(T))) % 16 == 0;
   dim3 grid(static_cast<unsigned>(n));
+  const char* forced = getenv("RELAX_AMD_FUSED_STEP_KERNEL");  // "cached": two-walk kernel for every row length
+  if (vec && !(forced && strcmp(forced, "cached") == 0)) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    const int rc = launch_reverse_kl_resident<T>(static_cast<const T*>(s), static_cast<const T*>(t), stride, vocab, n,
+                                                 g, scale, kl, ls, lt, static_cast<T*>(d), cus, st);
+    if (rc != RELAX_AMD_EUNSUPPORTED) return rc;  // launched (or failed to): otherwise the row length is not built
+  }
 #define RELAX_AMD_KL_STEP(V, TH)                                                                                   \
   hipLaunchKernelGGL((reverse_kl_step_kernel<T, V, TH>), grid, dim3(TH), 0, st, static_cast<const T*>(s),            \
                      static_cast<const T*>(t), stride, vocab, g, scale, kl, ls, lt, static_cast<T*>(d))

@@ -228,6 +228,50 @@ def test_fused_opd_loss_matches_oracle_and_two_launch_path(n, v, dtype, tol):
     assert torch.equal(kl3, kl2.detach())
 
 
+@pytest.mark.parametrize("v,dtype,n", [(151936, torch.bfloat16, 700), (152064, torch.float16, 300),
+                                       (128256, torch.bfloat16, 520), (131072, torch.float16, 515),
+                                       (100352, torch.bfloat16, 1030), (102400, torch.bfloat16, 40)])
+def test_register_resident_reverse_kl_step_equals_two_walk_kernel_bitwise(v, dtype, n, monkeypatch):
+    """The two kernels behind relax_amd_reverse_kl_step_fused, switched with RELAX_AMD_FUSED_STEP_KERNEL, for every
+    row shape the register-resident one is built for (partial and full last vector positions), with more rows than
+    workgroups (several rows per persistent workgroup, uneven counts), fewer rows than workgroups, and rows without
+    gradient (zero rows, KL still reported) scattered and in runs.  KL, both log-sum-exps and the gradient must be
+    bit-identical, and a few rows are checked against the oracle."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("resident reverse KL vs two-walk", v, dtype, n)
+    gen = torch.Generator(device=dev).manual_seed(v + n)
+    s = (torch.randn((n, v), device=dev, generator=gen) * 3).to(dtype)
+    t = (s.float() + torch.randn((n, v), device=dev, generator=gen)).to(dtype)
+    s[1, 7] = 40.0       # a row dominated by one entry
+    t[2] = s[2]          # KL == 0
+    g = (torch.rand(n, device=dev, generator=gen) > 0.2).float() * torch.rand(n, device=dev, generator=gen)
+    g[n // 2:n // 2 + 9] = 0.0
+    g[-1] = 0.0
+    results = {}
+    for kind in ("cached", "resident"):
+        monkeypatch.setenv("RELAX_AMD_FUSED_STEP_KERNEL", kind)
+        kl, ls, lt, d = ops.reverse_kl_step_fused(s, t, g, 0.75)
+        torch.cuda.synchronize()
+        results[kind] = dict(kl=kl, lse_s=ls, lse_t=lt, d=d.view(torch.int16))
+    for key, want in results["cached"].items():
+        got = results["resident"][key]
+        assert torch.equal(got, want), (key, (got.float() - want.float()).abs().max())
+    d = results["resident"]["d"].view(dtype)
+    live = g != 0
+    live[2] = False  # identical rows: every gradient entry is p_s * 0
+    assert (d[g == 0] == 0).all() and d[live].float().abs().sum(-1).min().item() > 0
+    assert abs(results["resident"]["kl"][2].item()) < 1e-5
+    rows = [0, 1, 2, n - 2]
+    sc = s[rows].cpu().requires_grad_()
+    want = D.full_vocab_reverse_kl(sc, t[rows].cpu())
+    (want * (0.75 * g[rows].cpu())).sum().backward()
+    torch.testing.assert_close(results["resident"]["kl"][rows].cpu(), want.detach(), atol=2e-3, rtol=0)
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    torch.testing.assert_close(d[rows].float().cpu(), sc.grad.float(), atol=2e-3, rtol=ulp)
+
+
 def test_opd_token_mean_literal(literals):
     from relax_amd.opd_utils import compute_opd_kl, reduce_opd_loss
 
