@@ -257,7 +257,10 @@ int relax_amd_reverse_kl_bwd(const void* student, const void* teacher, int dtype
  * known before the forward runs: the masked token mean of reduce_opd_loss (relax/utils/opd/opd_utils.py:1355-1365),
  * g[t] = mask[t] / clamp_min(sum mask, 1).  Same outputs as relax_amd_reverse_kl_fwd followed by
  * relax_amd_reverse_kl_bwd (dstudent row stride = row_stride); each workgroup re-reads its two rows out of cache, so
- * HBM moves 3*V*s bytes per token instead of 5*V*s.
+ * HBM moves 3*V*s bytes per token instead of 5*V*s.  Two kernels sit behind it, with bit-identical results: 16-bit
+ * rows of the built vocabulary shapes (12 / 15 / 18 full 16-byte vectors per thread of a 1024-thread workgroup plus
+ * a partial one, or 16 exactly) keep the student row in registers and stream the teacher row past it twice; other
+ * rows, and every row when RELAX_AMD_FUSED_STEP_KERNEL=cached is in the environment, walk both rows twice.
  */
 int relax_amd_reverse_kl_step_fused(const void* student, const void* teacher, int dtype, int64_t n_tokens,
                                     int64_t vocab, int64_t row_stride, const float* g, float grad_scale, float* kl,

@@ -30,7 +30,10 @@
 namespace relax_amd {
 
 constexpr int kKlResThreads = 1024;
-constexpr int kKlResDepth = 4;  // teacher vectors in flight ahead of their use (two pairs)
+// Teacher vectors in flight ahead of their use.  The slots freed by a pass's last positions take the next pass's first
+// vectors in rotated order, starting with vector NV % depth; the depth is chosen so that vector 0, needed first, is not
+// the one requested last (which would make the next pass wait for everything in flight).
+constexpr int kl_ring_depth(int nv) { return nv % 4 == 1 ? 5 : 4; }
 
 // absorb_pair() over the values of kKlUnroll raw vector pairs, without holding them all unpacked
 // marks a raw vector as changed without touching it: what is unpacked from it afterwards is a new value to the
@@ -103,11 +106,12 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
     const T* __restrict__ student, const T* __restrict__ teacher, int64_t stride, int64_t vocab, int64_t n_rows,
     const float* __restrict__ g, float grad_scale, float* __restrict__ kl, float* __restrict__ lse_s,
     float* __restrict__ lse_t, T* __restrict__ dstudent) {
-  constexpr int THREADS = kKlResThreads, D = kKlResDepth, kU = kKlUnroll;
+  constexpr int THREADS = kKlResThreads, kU = kKlUnroll;
   constexpr int VN = Row<T>::kPerVec;
   constexpr int NV = NVF + (PARTIAL ? 1 : 0);  // vector positions per thread
+  constexpr int D = kl_ring_depth(NV);
   constexpr int kGroups = (NV + kU - 1) / kU;
-  static_assert(kU == 2 && D >= kU, "the teacher ring is refilled pair by pair");
+  static_assert(kU == 2 && D >= kU && D <= NVF, "the teacher ring is refilled pair by pair");
   __shared__ float lds[THREADS / kWave][5];
   __shared__ float bc[2];
   const int tid = threadIdx.x;
@@ -125,6 +129,9 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
 #pragma unroll
     for (int j = 0; j < NV; ++j)
       if (has(j)) srow[j] = load_stream(row_vec(sv, tid + j * THREADS));
+    const u32x4* tv0 = reinterpret_cast<const u32x4*>(teacher + row * stride);
+#pragma unroll
+    for (int j = 0; j < D; ++j) ring[j] = *row_vec(tv0, tid + j * THREADS);
   }
 
   while (true) {
@@ -133,13 +140,15 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
     const float gt = g[row] * grad_scale;
     const u32x4* tv = reinterpret_cast<const u32x4*>(teacher + row * stride);
 
-    // ---- scan: both online softmaxes and sum e_s * (x_s - x_t); the teacher row streams through the ring (ordinary
-    // loads: it is read again in a moment)
-    int fill_id = tid;
-    asm volatile("" : "+v"(fill_id));  // recomputed per row, like the indices below
-#pragma unroll
-    for (int j = 0; j < D; ++j)
-      if (j < NV && has(j)) ring[j] = *row_vec(tv, fill_id + j * THREADS);
+    // a token without gradient (g == 0) gets a zero row; the second pass's teacher loads then all go to the row's
+    // first vector, which costs nothing, so that the instruction stream -- and with it the wait counts -- stays the same
+    const bool emit_zero = gt == 0.f;
+    const int tscale = emit_zero ? 0 : 1;
+
+    // ---- scan: both online softmaxes and sum e_s * (x_s - x_t).  The teacher row streams through the ring (ordinary
+    // loads: it is read again in a moment); its first D vectors are already on their way (requested during the previous
+    // row's gradient pass), and the slots freed by the last D positions take the first vectors of the second pass, which
+    // land during the merge.
     KlState q{kNegHuge, 0.f, 0.f, kNegHuge, 0.f};
     bool grouped = true;
 #pragma unroll
@@ -162,10 +171,17 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
             absorb_pair(a, b, q);
           }
       }
-      // the ring slots just consumed take the vectors D positions further on
+      // the ring slots just consumed take the vectors D positions further on, or the second pass's first ones
 #pragma unroll
-      for (int u = 0; u < kU; ++u)
-        if (j0 + u + D < NV && has(j0 + u + D)) ring[(j0 + u) % D] = *row_vec(tv, lane_id + (j0 + u + D) * THREADS);
+      for (int u = 0; u < kU; ++u) {
+        const int j = j0 + u;
+        if (j >= NV) continue;
+        if (j + D < NV) {
+          if (has(j + D)) ring[j % D] = *row_vec(tv, lane_id + (j + D) * THREADS);
+        } else {
+          ring[j % D] = load_stream(row_vec(tv, (lane_id + (j % D) * THREADS) * tscale));
+        }
+      }
       asm volatile("" : "+v"(q.ss), "+v"(q.us), "+v"(q.st));  // keeps each group's work where it is written
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -205,17 +221,11 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
     const float k0 = bc[0], k1 = bc[1];
 
     // ---- gradient: d = p_s * g * ((x_s - x_t) + lse_t - lse_s - KL), the teacher row a second time (last use:
-    // non-temporal), and behind each stored vector the same vector of the next row's student.  A token without
-    // gradient (g == 0) gets a zero row; its teacher loads all go to the row's first vector, which costs nothing, so
-    // that the instruction stream -- and with it the wait counts -- stays the same.
-    const bool emit_zero = gt == 0.f;
-    const int tscale = emit_zero ? 0 : 1;
+    // non-temporal), and behind each stored vector the same vector of the next row's student; the ring slots freed by
+    // the last D positions take the first teacher vectors of the next row.
     u32x4* dv = reinterpret_cast<u32x4*>(dstudent + row * stride);
     const u32x4* nsv = reinterpret_cast<const u32x4*>(student + (has_next ? next : row) * stride);
-    asm volatile("" : "+v"(fill_id));
-#pragma unroll
-    for (int j = 0; j < D; ++j)
-      if (j < NV && has(j)) ring[j] = load_stream(row_vec(tv, (fill_id + j * THREADS) * tscale));
+    const u32x4* ntv = reinterpret_cast<const u32x4*>(teacher + (has_next ? next : row) * stride);
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       int lane_id = tid;
@@ -225,26 +235,29 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
       // one 32-bit word of the vector at a time: a whole vector of both rows unpacked does not fit
       const uint32_t sw[4] = {srow[j].x, srow[j].y, srow[j].z, srow[j].w};
       const uint32_t tw[4] = {ring[j % D].x, ring[j % D].y, ring[j % D].z, ring[j % D].w};
-      uint32_t ow[4];
+      uint32_t ow[4] = {0u, 0u, 0u, 0u};
+      if (!emit_zero) {  // the same answer in every lane of the workgroup: a jump, not a mask
 #pragma unroll
-      for (int h = 0; h < 4; ++h) {
-        float a[VN], b[VN];
-        Row<T>::unpack(u32x4{sw[h], 0u, 0u, 0u}, a);
-        Row<T>::unpack(u32x4{tw[h], 0u, 0u, 0u}, b);
+        for (int h = 0; h < 4; ++h) {
+          float a[VN], b[VN];
+          Row<T>::unpack(u32x4{sw[h], 0u, 0u, 0u}, a);
+          Row<T>::unpack(u32x4{tw[h], 0u, 0u, 0u}, b);
 #pragma unroll
-        for (int k = 0; k < VN / 4; ++k) a[k] = fast_exp2(fmaf(a[k], kLog2e, k0)) * fmaf(a[k] - b[k], gt, k1);
-        ow[h] = Row<T>::pack(a).x;
-        if (h == 1) __builtin_amdgcn_sched_barrier(0);
+          for (int k = 0; k < VN / 4; ++k) a[k] = fast_exp2(fmaf(a[k], kLog2e, k0)) * fmaf(a[k] - b[k], gt, k1);
+          ow[h] = Row<T>::pack(a).x;
+          if (h == 1) __builtin_amdgcn_sched_barrier(0);
+        }
       }
-      u32x4 out{ow[0], ow[1], ow[2], ow[3]};
-      if (emit_zero) out = u32x4{0u, 0u, 0u, 0u};
-      if (has(j)) {
-        store_stream(row_vec(dv, idx), out);
-        // without a next row the row itself is read again: a branch here would cost the precise wait counts, and
-        // the last row of a workgroup is one in dozens
-        srow[j] = load_stream(row_vec(nsv, idx));
+      const u32x4 out{ow[0], ow[1], ow[2], ow[3]};
+      if (has(j)) store_stream(row_vec(dv, idx), out);
+      // without a next row the row itself is read again, and a lane without a vector at the partial position reads
+      // its first vector again (never used): branches here would cost the precise wait counts
+      srow[j] = load_stream(row_vec(nsv, has(j) ? idx : lane_id));
+      if (j + D < NV) {
+        if (has(j + D)) ring[j % D] = load_stream(row_vec(tv, (idx + D * THREADS) * tscale));
+      } else {
+        ring[j % D] = *row_vec(ntv, lane_id + (j % D) * THREADS);  // the row itself again when there is no next one
       }
-      if (j + D < NV && has(j + D)) ring[j % D] = load_stream(row_vec(tv, (idx + D * THREADS) * tscale));
       __builtin_amdgcn_sched_barrier(0);  // one vector at a time: hoisting the next one's unpacking spills
     }
     if (!has_next) return;
