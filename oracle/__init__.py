@@ -45,6 +45,11 @@ live in ``tests/test_oracle_*.py``):
   of tests/backends/megatron/test_ppo_gae_parity.py:41-60.  ``advantages.masked_normalize``: numpy
   population moments.  ``opd.opd_kl`` union mask / ``log_probs_on_topk_ids``: closed forms (row-prefix
   equivalence, textbook JSD, ``log_softmax`` gather).
+* ``losses.m2po*`` (second-moment trust region): no reference test or fixture; ``m2po_solve_tau`` is pinned by
+  enumeration (every data value tried as the cap: the chosen one is the largest whose capped sum stays below the
+  budget, and the reported moment is that capped sum / n), the harmful-token set, the within-budget, no-harmful-token
+  and all-equal cases by closed forms, the loss by ``policy_clip`` with the solved margins.  The reference's quirk that
+  a stop at the first element reports the uncapped moment is kept (read from ppo_utils.py:417-418).
 * ``reducers.seq_mean_token_sum``: the reference has no implementation of this
   aggregation (only the reducer plug-in point, loss.py:1062-1072)
   -- **parity unpinned**; defined here as sum_i sum_t x*m / B.

@@ -302,6 +302,19 @@ class _FusedPolicyLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, flat, lay, inv_t, kw):
         lp, ent, lse, spx = ops.logprob_entropy_fwd(flat, lay.targets, lay.row_ids, inv_t, True)
+        m2po = kw.get("m2po")
+        if m2po is not None:
+            # M2PO (loss.py:990-993): the clip margins are solved from this micro-batch's log-ratios, which exist only
+            # now; the PPO-clip kernel then runs with them
+            from .ppo_utils import m2po_clip_margins
+
+            old = kw["old_log_prob"]
+            ppo_kl = old - lp if old is not None else torch.zeros_like(lp)
+            eps_low, eps_high, m2_now, m2_after = m2po_clip_margins(
+                ppo_kl, kw["advantages"], m2po["kl2_budget"], m2po["miniclip_low"], m2po["miniclip_high"])
+            m2po["scalars"] = (m2_now, m2_after, eps_low, eps_high)
+            kw = {k: v for k, v in kw.items() if k != "m2po"}
+            kw["eps_clip"], kw["eps_clip_high"] = eps_low, eps_high
         out = ops.policy_loss(log_prob=lp, entropy=ent, cu_resp=lay.cu_resp, **kw)
         metrics = out["metrics"]
         entropy_grad = kw.get("entropy_coef", 0.0) != 0
@@ -350,6 +363,8 @@ def _single_pass_ok(args, flat, kw, needs_bwd) -> bool:
         return False
     if kw["loss_kind"] == "gspo" or kw["use_opsm"]:
         return False  # sequence-coupled gradients need the per-sequence reduction between forward and backward
+    if kw.get("m2po") is not None:
+        return False  # the clip margins depend on every token's log-prob: they are solved between the two launches
     return True
 
 
@@ -464,6 +479,9 @@ def _composed_policy_loss_function(args: Namespace, batch: dict, logits: torch.T
         pg_loss, pg_clipfrac = PU.compute_cispo_loss(lp, ppo_kl, adv, args.eps_clip, args.eps_clip_high)
     elif est == "rloo":
         pg_loss, pg_clipfrac = PU.compute_rloo_loss(lp, adv)
+    elif est == "m2po":
+        pg_loss, pg_clipfrac, *m2po_scalars = PU.compute_m2po_loss(
+            ppo_kl, adv, args.m2po_kl2_budget, args.m2po_miniclip_low, args.m2po_miniclip_high)
     elif est in ("grpo", "gspo", "ppo") or pp:
         pg_loss, pg_clipfrac = PU.compute_policy_loss(ppo_kl, adv, args.eps_clip, args.eps_clip_high)
     else:
@@ -533,7 +551,17 @@ def _composed_policy_loss_function(args: Namespace, batch: dict, logits: torch.T
             reported[k] = metric_reduce(v)  # over the tokens valid before any rejection (loss.py:1007-1014)
     if getattr(args, "use_opsm", False):
         reported["opsm_clipfrac"] = opsm_clipfrac
+    if est == "m2po":
+        reported.update(_m2po_reported(m2po_scalars, dev))
     return loss, reported
+
+
+_M2PO_KEYS = ("ppo_kl_m2_before", "ppo_kl_m2_after", "m2po_eps_low", "m2po_eps_high")
+
+
+def _m2po_reported(scalars, device) -> dict:
+    """(M2 before, M2 after, eps_low, eps_high) -> the reference's four metric entries (loss.py:1179-1183)."""
+    return {key: torch.tensor(value, device=device).detach() for key, value in zip(_M2PO_KEYS, scalars, strict=True)}
 
 
 def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum_of_sample_mean=None):
@@ -550,8 +578,6 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     flat = _check_logits(logits, args)
     dev = flat.device
     est = args.advantage_estimator
-    if est == "m2po":
-        raise NotImplementedError(f"advantage_estimator {est} is not part of the fused path")
     if getattr(args, "custom_tis_function_path", None) is not None \
             or getattr(args, "custom_pg_loss_reducer_function_path", None) is not None:
         _check_logits(logits, args)
@@ -591,8 +617,9 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         sample_denom=None if denom is None else denom.to(device=dev, dtype=torch.float32),
         pg_sample_denom=None if pg_denom is None else pg_denom.to(device=dev, dtype=torch.float32),
         # REINFORCE++ trains with the PPO-clip surrogate; its mask-safe reduction is what the kernel does anyway
+        # M2PO is the PPO-clip surrogate with margins solved per micro-batch (set in _FusedPolicyLoss.forward)
         loss_kind={"grpo": "ppo", "ppo": "ppo", "reinforce_plus_plus": "ppo",
-                   "reinforce_plus_plus_baseline": "ppo"}.get(est, est),
+                   "reinforce_plus_plus_baseline": "ppo", "m2po": "ppo"}.get(est, est),
         kl_kind=args.kl_loss_type if use_kl else None,
         unbiased_kl=bool(getattr(args, "use_unbiased_kl", False)) and use_kl,
         use_opsm=bool(getattr(args, "use_opsm", False)),
@@ -611,6 +638,9 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     )
     if kw["loss_kind"] not in ("ppo", "gspo", "cispo", "rloo", "sapo"):
         raise NotImplementedError(f"advantage_estimator {est} is not supported. ")
+    if est == "m2po":
+        kw["m2po"] = dict(kl2_budget=float(args.m2po_kl2_budget), miniclip_low=float(args.m2po_miniclip_low),
+                          miniclip_high=float(args.m2po_miniclip_high))
     inv_t = 1.0 / float(getattr(args, "rollout_temperature", 1.0))
     if lay.n_tokens == 0:
         loss = 0 * logits.sum()
@@ -618,6 +648,9 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         metrics = {k: zero.clone() for k in ("loss", "pg_loss", "entropy_loss", "pg_clipfrac", "ppo_kl")}
         if use_kl:
             metrics["kl_loss"] = zero.clone()
+        if est == "m2po":  # no token is harmful: no adaptive clip, the margins are the wide defaults
+            metrics.update(_m2po_reported((0.0, 0.0, max(1.0, kw["m2po"]["miniclip_low"]),
+                                           max(99999.0, kw["m2po"]["miniclip_high"])), dev))
         return loss, metrics
     fn = _SinglePassPolicyLoss if _single_pass_ok(args, flat, kw, needs_bwd) else _FusedPolicyLoss
     loss, mvec, lp, ent = fn.apply(flat, lay, inv_t, kw)
@@ -662,6 +695,8 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     reported.update(opd_reported)
     if kw["use_opsm"]:
         reported["opsm_clipfrac"] = m("opsm_clipfrac")
+    if est == "m2po":
+        reported.update(_m2po_reported(kw["m2po"]["scalars"], dev))
     return loss, reported
 
 
@@ -690,6 +725,12 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
     else:
         loss, log = sft_loss_function(args, batch, logits, None)
     per_token = bool(getattr(args, "calculate_per_token_loss", False))
+    if per_token and getattr(args, "advantage_estimator", None) == "m2po":
+        # the M2PO scalars are global, not per-token sums: pre-multiplied so that the logger's division by the token
+        # count gives them back (loss.py:1547-1552)
+        for key in _M2PO_KEYS:
+            if key in log:
+                log[key] = log[key] * num_tokens
     is_dummy = batch.get("__is_dummy__", False)
     explicit = batch.get("__loss_scale__", None)
     gbs = batch.get("dynamic_global_batch_size", getattr(args, "global_batch_size", 1))
