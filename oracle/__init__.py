@@ -50,6 +50,8 @@ live in ``tests/test_oracle_*.py``):
   budget, and the reported moment is that capped sum / n), the harmful-token set, the within-budget, no-harmful-token
   and all-equal cases by closed forms, the loss by ``policy_clip`` with the solved margins.  The reference's quirk that
   a stop at the first element reports the uncapped moment is kept (read from ppo_utils.py:417-418).
+* ``policy.value_loss_function`` / ``policy.get_values``: a three-token case worked by hand (clipped and unclipped
+  branches of the maximum, the clip fraction, the response-row slicing).
 * ``reducers.seq_mean_token_sum``: the reference has no implementation of this
   aggregation (only the reducer plug-in point, loss.py:1062-1072)
   -- **parity unpinned**; defined here as sum_i sum_t x*m / B.

@@ -284,3 +284,25 @@ def loss_function(args, batch, num_microbatches, logits, dp_world: int = 1, func
     vals = torch.stack([denom] + [v if isinstance(v, torch.Tensor) else torch.tensor(v) for v in log.values()])
     norm = ntok if args.calculate_per_token_loss else torch.tensor(1)
     return loss, norm, {"keys": list(log.keys()), "values": vals}
+
+
+def get_values(logits, total_lengths, response_lengths):
+    """loss.py:466-518: the value head's [1, T, 1] output over each sample's response rows (same slicing as the
+    log-prob path, no temperature), squeezed to [R_i]."""
+    assert logits.dim() == 3 and logits.size(0) == 1 and logits.size(-1) == 1
+    flat = logits.squeeze(0)
+    return [flat[b:e].squeeze(-1) for b, e, _sft in response_row_ranges(total_lengths, response_lengths)]
+
+
+def value_loss_function(args, batch, logits, reducer):
+    """loss.py:1188-1244: clipped value loss and its two metrics."""
+    old = torch.cat(batch["values"], dim=0)
+    values = torch.cat([v.flatten() for v in get_values(logits, batch["total_lengths"], batch["response_lengths"])])
+    returns = torch.cat(batch["returns"], dim=0)
+    clipfrac = torch.abs(values - old) > args.value_clip
+    clipped = old + (values - old).clamp(-args.value_clip, args.value_clip)
+    loss = reducer(torch.max((clipped - returns) ** 2, (values - returns) ** 2))
+    frac = reducer(clipfrac.float())
+    if values.numel() == 0:
+        loss = loss + 0 * values.sum()
+    return loss, {"value_loss": loss.clone().detach(), "value_clipfrac": frac.clone().detach()}

@@ -9,10 +9,12 @@ from .loss import (  # noqa: F401
     compute_advantages_and_returns,
     get_log_probs_and_entropy,
     get_responses,
+    get_values,
     loss_function,
     policy_loss_function,
     sft_loss_function,
     sft_loss_function_chunked,
+    value_loss_function,
 )
 from .ppo_utils import calculate_log_probs_and_entropy  # noqa: F401
 

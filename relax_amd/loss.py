@@ -700,6 +700,46 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     return loss, reported
 
 
+def get_values(logits: torch.Tensor, *, args: Namespace, unconcat_tokens, total_lengths, response_lengths,
+               with_entropy: bool = False, non_loss_data: bool = True, max_seq_lens=None, padded_total_lengths=None,
+               **_: Any):
+    """Counterpart of loss.py:466-518: the value head's output ``[1, T, 1]`` at every response token, as per-sample
+    ``[R_i]`` views of one packed gather (the same row map as the log-prob path; no temperature), differentiable
+    w.r.t. ``logits``.  Returns ``(empty, {"values": [...]})``."""
+    assert logits.dim() == 3 and logits.size(0) == 1 and logits.size(-1) == 1, f"{logits.shape}"
+    flat = logits.reshape(-1)
+    lay = PackedLayout(flat.device, flat.size(0), unconcat_tokens, total_lengths, response_lengths, False)
+    values = flat.index_select(0, lay.row_ids.to(torch.int64)) if lay.n_tokens else flat[:0]
+    return torch.empty((0,), device=flat.device), {"values": lay.split(values)}
+
+
+def value_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum_of_sample_mean=None):
+    """Counterpart of loss.py:1188-1244: PPO's clipped value loss ``max((v_clipped - R)^2, (v - R)^2)`` with
+    ``v_clipped = v_old + clamp(v - v_old, +-value_clip)``, reduced like the policy loss; metrics ``value_loss`` and
+    ``value_clipfrac``.  The work is ``[N]``-sized (one value per response token); the reduction is the masked
+    per-sample kernel behind ``get_sum_of_sample_mean`` when no reducer is passed in."""
+    dev = logits.device
+    old_values = _cat_f32(batch["values"], dev)
+    _, out = get_values(logits, args=args, unconcat_tokens=batch["unconcat_tokens"],
+                        total_lengths=batch["total_lengths"], response_lengths=batch["response_lengths"],
+                        max_seq_lens=batch.get("max_seq_lens"), padded_total_lengths=batch.get("padded_total_lengths"))
+    values = torch.cat([v.flatten() for v in out["values"]], dim=0)
+    returns = _cat_f32(batch["returns"], dev)
+    if sum_of_sample_mean is None:
+        sum_of_sample_mean = get_sum_of_sample_mean(
+            batch["total_lengths"], batch["response_lengths"], [m.to(dev) for m in batch["loss_masks"]],
+            bool(getattr(args, "calculate_per_token_loss", False)), sample_denoms=batch.get("sample_index_mask_sums"))
+    clip = float(args.value_clip)
+    clipfrac = torch.abs(values - old_values) > clip
+    clipped = old_values + (values - old_values).clamp(-clip, clip)
+    loss = torch.max((clipped - returns) ** 2, (values - returns) ** 2)
+    loss = sum_of_sample_mean(loss)
+    clipfrac = sum_of_sample_mean(clipfrac.float())
+    if values.numel() == 0:
+        loss = loss + 0 * values.sum()
+    return loss, {"value_loss": loss.clone().detach(), "value_clipfrac": clipfrac.clone().detach()}
+
+
 def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: torch.Tensor, *, lm_head_forward=None,
                   dp_world_size: int = 1):
     """Counterpart of loss.py:1443-1620 on one GPU: token count, the loss selected by ``args.loss_type``
@@ -707,12 +747,13 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
     ``lm_head_forward`` are given), Megatron gradient-accumulation scaling, and the ``{"keys", "values"}`` logging
     dict."""
     loss_type = getattr(args, "loss_type", "policy_loss")
-    if loss_type not in ("policy_loss", "sft", "custom_loss"):
-        raise ValueError(f"Unknown loss type: {loss_type}") if loss_type != "value_loss" \
-            else NotImplementedError(f"loss type {loss_type} is outside the fused policy path")
+    if loss_type not in ("policy_loss", "value_loss", "sft", "custom_loss"):
+        raise ValueError(f"Unknown loss type: {loss_type}")
     num_tokens = get_cp_local_num_tokens(batch["total_lengths"], batch["response_lengths"], batch["loss_masks"])
     if loss_type == "policy_loss":
         loss, log = policy_loss_function(args, batch, logits, None)
+    elif loss_type == "value_loss":
+        loss, log = value_loss_function(args, batch, logits, None)
     elif loss_type == "custom_loss":  # loss.py:1530-1531: the plug-in gets the reducer the built-in losses use
         reducer = get_sum_of_sample_mean(batch["total_lengths"], batch["response_lengths"], batch["loss_masks"],
                                          bool(getattr(args, "calculate_per_token_loss", False)),

@@ -393,6 +393,68 @@ def test_m2po_scalars_survive_the_per_token_logging_division():
     assert met["ppo_kl_m2_after"].item() <= 30.0 < met["ppo_kl_m2_before"].item()  # an interior cap was solved
 
 
+@pytest.mark.parametrize("per_token", [False, True])
+def test_value_loss_function_vs_oracle_and_closed_forms(per_token):
+    """The critic's loss (``--loss-type value_loss``): value-head output [1, T, 1] sliced to the response rows, clipped
+    squared error, per-sample masked mean.  Against the oracle (values, loss, both metrics, gradient w.r.t. the value
+    head's output, which is zero outside the response rows and under a zero mask), through ``loss_function``'s
+    dispatch, and against two closed forms: a clip wider than every deviation gives the plain squared error with
+    gradient 2 (v - R) m / denominator, and with old values equal to the new ones nothing is clipped."""
+    import relax_amd
+    from relax_amd.loss import loss_function
+
+    dev = require_gpu()
+    announce("value loss", per_token)
+    tot, resp = [9, 6, 12, 7], [4, 3, 7, 5]
+    _, batch = _make_batch(5, tot, resp, 8)
+    g = torch.Generator().manual_seed(77)
+    n = sum(resp)
+    head = torch.randn(1, sum(tot), 1, generator=g)
+    batch["values"] = list(torch.split(torch.randn(n, generator=g), resp))
+    batch["returns"] = list(torch.split(torch.randn(n, generator=g), resp))
+    args = P.make_args(loss_type="value_loss", value_clip=0.4, calculate_per_token_loss=per_token)
+    red = R.make_reducer(resp, batch["loss_masks"], per_token)
+    ho = head.clone().requires_grad_()
+    want_loss, want_m = P.value_loss_function(args, batch, ho, red)
+    want_loss.backward()
+    bd = _to_dev(batch, dev)
+    hd = head.to(dev).requires_grad_()
+    _, vals = relax_amd.get_values(hd, args=args, unconcat_tokens=bd["unconcat_tokens"], total_lengths=tot,
+                                   response_lengths=resp)
+    for got, want in zip(vals["values"], P.get_values(head, tot, resp)):
+        assert torch.equal(got.detach().cpu(), want)
+    loss, met = relax_amd.value_loss_function(args, bd, hd, None)
+    loss.backward()
+    assert abs(loss.item() - want_loss.item()) < 3e-6 * max(1.0, abs(want_loss.item()))
+    assert set(met) == {"value_loss", "value_clipfrac"}
+    for k, w in want_m.items():
+        assert abs(met[k].item() - float(w)) < 3e-6 * max(1.0, abs(float(w))), k
+    assert 0 < want_m["value_clipfrac"].item()  # the case does clip
+    torch.testing.assert_close(hd.grad.cpu(), ho.grad, atol=1e-6, rtol=1e-5)
+    loss2, normalizer, log = loss_function(args, bd, 1, head.to(dev))
+    assert log["keys"] == ["value_loss", "value_clipfrac"]
+    scale = 1.0 if per_token else 1.0 / args.global_batch_size
+    assert abs(loss2.item() - want_loss.item() * scale) < 3e-6 * max(1.0, abs(want_loss.item()))
+    # closed forms
+    wide = P.make_args(loss_type="value_loss", value_clip=1e9, calculate_per_token_loss=per_token)
+    hd2 = head.to(dev).requires_grad_()
+    loss3, met3 = relax_amd.value_loss_function(wide, bd, hd2, None)
+    loss3.backward()
+    rows = torch.cat([torch.arange(b, e) for b, e, _ in P.response_row_ranges(tot, resp)])
+    v = head.reshape(-1)[rows]
+    ret, mask = torch.cat(batch["returns"]), torch.cat(batch["loss_masks"])
+    den = torch.cat([torch.full((r,), 1.0 if per_token else max(float(m.sum()), 1.0))
+                     for r, m in zip(resp, batch["loss_masks"])])
+    assert abs(loss3.item() - float((((v - ret) ** 2) * mask / den).sum())) < 1e-5
+    assert met3["value_clipfrac"].item() == 0
+    want_grad = torch.zeros(sum(tot))
+    want_grad[rows] = 2 * (v - ret) * mask / den
+    torch.testing.assert_close(hd2.grad.reshape(-1).cpu(), want_grad, atol=1e-6, rtol=1e-5)
+    bd_same = dict(bd, values=[x.detach().clone() for x in vals["values"]])
+    _, met4 = relax_amd.value_loss_function(args, bd_same, head.to(dev), None)
+    assert met4["value_clipfrac"].item() == 0
+
+
 def test_reducers_vs_oracle_literals(literals):
     from relax_amd import cp_utils
 

@@ -272,3 +272,21 @@ def test_m2po_special_cases():
     assert torch.equal(frac, want_frac)
     _pg, _frac, _n, _a, eps_low, eps_high = L.m2po(kl, adv, 0.1)  # default floors 0.3 / 0.5 win over 0.26 / 0.35
     assert (eps_low, eps_high) == (0.3, 0.5)
+
+
+def test_value_loss_hand_computed():
+    """Clipped value loss, worked by hand for clip 0.5 and old values 0: (v, R) = (1, 0) -> clipped to 0.5, max(0.25, 1)
+    = 1, counted as clipped; (0.2, 0) -> 0.04, not clipped; (1, 2) -> max((0.5 - 2)^2, (1 - 2)^2) = 2.25, clipped.
+    One sample of three response tokens after a two-token prompt: the values sit on head rows 1..3."""
+    from types import SimpleNamespace
+
+    from oracle import policy as P
+
+    head = torch.tensor([9.0, 1.0, 0.2, 1.0, 9.0]).reshape(1, 5, 1)
+    batch = dict(values=[torch.zeros(3)], returns=[torch.tensor([0.0, 0.0, 2.0])], total_lengths=[5],
+                 response_lengths=[3], loss_masks=[torch.ones(3)])
+    assert torch.equal(P.get_values(head, [5], [3])[0], torch.tensor([1.0, 0.2, 1.0]))
+    red = R.make_reducer([3], batch["loss_masks"], False)
+    loss, met = P.value_loss_function(SimpleNamespace(value_clip=0.5), batch, head, red)
+    assert abs(loss.item() - (1 + 0.04 + 2.25) / 3) < 1e-6
+    assert abs(met["value_clipfrac"].item() - 2 / 3) < 1e-6 and abs(met["value_loss"].item() - loss.item()) < 1e-7
