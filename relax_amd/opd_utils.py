@@ -155,7 +155,17 @@ def compute_opd_kl(student_log_probs, teacher_log_probs, kl_type: str = "reverse
         if kl_type in ("jsd", "low_var_kl"):
             return compute_opd_kl_topk(student_log_probs, teacher_log_probs, kl_type, jsd_alpha, norm_mode,
                                        log_prob_min_clamp, mask)
-        raise NotImplementedError("element-wise [R, K] log-ratios are not a loss signal; use compute_opd_kl_topk")
+        if kl_type != "reverse_kl":
+            raise ValueError(f"Unknown opd_kl_type: {kl_type}. Choose one of {OPD_KL_TYPES}.")
+        # opd_utils.py:1126-1138: for [R, K] inputs "reverse_kl" is the element-wise log-ratio itself (padding of a
+        # union mask gives -inf - -inf there, as in the reference); callers that want the summed KL use
+        # compute_opd_kl_topk
+        s, t = student_log_probs.float(), teacher_log_probs.float()
+        if log_prob_min_clamp is not None:
+            s, t = s.clamp_min(log_prob_min_clamp), t.clamp_min(log_prob_min_clamp)
+        if mask is not None:
+            s, t = s.masked_fill(~mask, float("-inf")), t.masked_fill(~mask, float("-inf"))
+        return s - t
     s, t = student_log_probs, teacher_log_probs
     if log_prob_min_clamp is not None:
         s, t = s.clamp_min(log_prob_min_clamp), t.clamp_min(log_prob_min_clamp)

@@ -20,7 +20,14 @@ def post_process_rewards(args: Any, samples: list, device=None):
     reference: missing group index, wrong group size and (RLOO) non-finite rewards raise ``ValueError``.
     """
     if getattr(args, "custom_reward_post_process_path", None) is not None:
-        raise NotImplementedError("custom reward post-processing callables run outside relax_amd")
+        # relax/utils/utils.py:186-192: the user's function decides; a 2-tuple is (raw, processed), anything else is
+        # the processed rewards alone
+        from .loss import load_function
+
+        processed = load_function(args.custom_reward_post_process_path)(args, samples)
+        if isinstance(processed, tuple) and len(processed) == 2:
+            return processed
+        return [s.get_reward_value(args) for s in samples], processed
     raw = [s.get_reward_value(args) for s in samples]
     if getattr(args, "agentic_custom_advantage_path", None) is not None:
         return raw, [s.custom_advantage for s in samples]

@@ -1,7 +1,7 @@
 """User-side plug-ins for the tests of the dotted-path hooks (``--custom-tis-function-path``,
 ``--custom-pg-loss-reducer-function-path``, ``--custom-loss-function-path``): plain tensor code of the kind a user of
 the reference writes, with the reference's plug-in signatures (relax/backends/megatron/loss.py:1026-1040, 1062-1072,
-1530-1531)."""
+1530-1531; ``--custom-reward-post-process-path``: relax/utils/utils.py:186-192)."""
 
 import torch
 
@@ -36,3 +36,15 @@ def negative_log_likelihood(args, batch, logits, sum_of_sample_mean):
         response_lengths=batch["response_lengths"], with_entropy=False)
     loss = -sum_of_sample_mean(torch.cat(out["log_probs"]))
     return loss, {"loss": loss.clone().detach()}
+
+
+def halved_rewards(args, samples):
+    """A reward post-processor that returns the processed rewards only."""
+    return [0.5 * s.get_reward_value(args) for s in samples]
+
+
+def raw_and_centred_rewards(args, samples):
+    """A reward post-processor that returns the (raw, processed) pair itself."""
+    raw = [s.get_reward_value(args) for s in samples]
+    mean = sum(raw) / len(raw)
+    return raw, [r - mean for r in raw]

@@ -157,3 +157,25 @@ def test_ppl_metrics_literals():
     assert math.isclose(m["eval/loss"], 10.0 / 6.0, rel_tol=1e-6)
     assert math.isclose(m["eval/ppl"], math.exp(10.0 / 6.0), rel_tol=1e-5) and m["eval/num_tokens"] == 6
     assert compute_ppl_metrics(0.0, 0) == {"eval/loss": 0.0, "eval/ppl": 0.0, "eval/num_tokens": 0}
+
+
+def test_custom_reward_post_process_hook():
+    """``--custom-reward-post-process-path`` (relax/utils/utils.py:186-192): the named function replaces the built-in
+    processing; a 2-tuple is taken as (raw, processed), anything else as the processed rewards next to the raw ones."""
+    from types import SimpleNamespace
+
+    from relax_amd.utils import post_process_rewards
+
+    class S:
+        def __init__(self, r):
+            self.r, self.group_index = r, 0
+
+        def get_reward_value(self, args):
+            return self.r
+
+    samples = [S(1.0), S(2.0), S(6.0)]
+    args = SimpleNamespace(custom_reward_post_process_path="tests.custom_hooks.halved_rewards",
+                           advantage_estimator="grpo", rewards_normalization=True)
+    assert post_process_rewards(args, samples) == ([1.0, 2.0, 6.0], [0.5, 1.0, 3.0])
+    args.custom_reward_post_process_path = "tests.custom_hooks.raw_and_centred_rewards"
+    assert post_process_rewards(args, samples) == ([1.0, 2.0, 6.0], [-2.0, -1.0, 3.0])

@@ -369,6 +369,26 @@ def test_opd_kl_topk_vs_oracle(kl_type, alpha, norm_mode, masked, clamp):
     torch.testing.assert_close(sd.grad.cpu(), sc.grad, atol=2e-5 * gscale, rtol=2e-4)
 
 
+def test_opd_kl_two_dimensional_reverse_kl_is_the_elementwise_log_ratio():
+    """compute_opd_kl on [R, K] inputs with ``reverse_kl`` returns s - t element by element (opd_utils.py:1126-1138),
+    after the lower clamp, with -inf - -inf = NaN at the padding of a union mask like the reference."""
+    from relax_amd.opd_utils import compute_opd_kl
+
+    dev = require_gpu()
+    announce("opd kl 2-D reverse_kl")
+    g = torch.Generator().manual_seed(3)
+    s = (-torch.rand(5, 7, generator=g) * 9).to(dev)
+    t = (-torch.rand(5, 7, generator=g) * 9).to(dev)
+    assert torch.equal(compute_opd_kl(s, t, "reverse_kl"), s - t)
+    assert torch.equal(compute_opd_kl(s.bfloat16(), t, "reverse_kl", log_prob_min_clamp=-4.0),
+                       s.bfloat16().float().clamp_min(-4.0) - t.clamp_min(-4.0))
+    mask = torch.rand(5, 7, generator=g).to(dev) > 0.3
+    got = compute_opd_kl(s, t, "reverse_kl", mask=mask)
+    assert torch.equal(got[mask], (s - t)[mask]) and torch.isnan(got[~mask]).all()
+    with pytest.raises(ValueError, match="Unknown opd_kl_type"):
+        compute_opd_kl(s, t, "forward_kl")
+
+
 def test_opd_kl_topk_argument_checks():
     from relax_amd.opd_utils import compute_opd_kl, compute_opd_kl_topk
 
