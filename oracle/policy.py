@@ -58,8 +58,9 @@ def make_args(**kw):
     return SimpleNamespace(**d)
 
 
-def response_row_ranges(total_lengths, response_lengths):
-    """Index arithmetic of relax/backends/megatron/loss.py:103-125 (cp_size == 1, thd).
+def response_row_ranges(total_lengths, response_lengths, max_seq_lens=None):
+    """Index arithmetic of relax/backends/megatron/loss.py:103-125 (cp_size == 1; packed "thd" layout, or with
+    ``max_seq_lens`` the padded "bshd" layout flattened to rows, where sample i begins at max_seq_lens[i] * i).
 
     Returns per sample (row_begin, row_end, sft) where logits rows [row_begin, row_end) score the response
     tokens.  RL samples use the previous position's logits (start-1 .. end-1); the SFT convention
@@ -67,8 +68,8 @@ def response_row_ranges(total_lengths, response_lengths):
     """
     out = []
     end = 0
-    for total, resp in zip(total_lengths, response_lengths, strict=False):
-        end += total
+    for i, (total, resp) in enumerate(zip(total_lengths, response_lengths, strict=False)):
+        end = max_seq_lens[i] * i + total if max_seq_lens is not None else end + total  # :112-117
         start = end - resp
         if resp == total:
             out.append((start, end, True))

@@ -32,23 +32,32 @@ _SLOT = {k: i for i, k in enumerate(METRIC_SLOTS)}
 GRPO_FAMILY = ("grpo", "gspo", "sapo", "cispo", "m2po", "rloo")
 
 
-def _check_logits(logits: torch.Tensor, args) -> torch.Tensor:
-    """[1, T, V] -> [T, V].  fp32 is what stock Megatron hands over; bf16 / fp16 logits are accepted as well."""
+def _check_logits(logits: torch.Tensor, args, max_seq_lens=None) -> torch.Tensor:
+    """[1, T, V] (packed, "thd") or [B, S, V] (padded, "bshd") -> [rows, V] (loss.py:94-99).  fp32 is what stock
+    Megatron hands over; bf16 / fp16 logits are accepted as well."""
     assert logits.dtype in (torch.float32, torch.bfloat16, torch.float16), f"{logits.dtype}"
     assert len(logits.shape) == 3, f"{logits.shape}"
-    if getattr(args, "qkv_format", "thd") != "thd":
-        raise NotImplementedError("relax_amd handles the packed 'thd' layout only")
-    assert logits.size(0) == 1, f"{logits.shape}"
-    return logits.squeeze(0)
+    if getattr(args, "qkv_format", "thd") == "thd":
+        assert logits.size(0) == 1, f"{logits.shape}"
+        return logits.squeeze(0)
+    assert max_seq_lens is not None
+    return logits.reshape(-1, logits.size(-1))
 
 
-def response_row_begins(total_lengths, response_lengths) -> tuple[list[int], list[bool]]:
+def _padded_starts(args, max_seq_lens):
+    """``max_seq_lens`` when the batch is in the padded "bshd" layout (sample i starts at row max_seq_lens[i] * i),
+    None for the packed layout, where a sample starts where the previous one ends."""
+    return None if getattr(args, "qkv_format", "thd") == "thd" else max_seq_lens
+
+
+def response_row_begins(total_lengths, response_lengths, max_seq_lens=None) -> tuple[list[int], list[bool]]:
     """First logits row of each sample's response (loss.py:103-125): RL samples are scored by the previous
-    position's logits (start - 1); the SFT convention (response == total) uses start (sft_utils.py:23-40)."""
+    position's logits (start - 1); the SFT convention (response == total) uses start (sft_utils.py:23-40).  With
+    ``max_seq_lens`` (padded layout, loss.py:112-114) sample i's rows begin at ``max_seq_lens[i] * i``."""
     begins, sft = [], []
     end = 0
-    for total, resp in zip(total_lengths, response_lengths, strict=False):
-        end += total
+    for i, (total, resp) in enumerate(zip(total_lengths, response_lengths, strict=False)):
+        end = max_seq_lens[i] * i + total if max_seq_lens is not None else end + total
         start = end - resp
         is_sft = resp == total
         begins.append(start if is_sft else start - 1)
@@ -71,8 +80,8 @@ def get_responses(
 ) -> Iterator[tuple[torch.Tensor, torch.Tensor]]:
     """Yields per-sample ``(logits rows [R, V], target ids [R])`` views.  Kept for callers that want the slices;
     the fused functions below do not iterate samples.  Temperature is applied per chunk like the reference."""
-    flat = _check_logits(logits, args)
-    begins, sft = response_row_begins(total_lengths, response_lengths)
+    flat = _check_logits(logits, args, max_seq_lens)
+    begins, sft = response_row_begins(total_lengths, response_lengths, _padded_starts(args, max_seq_lens))
     for b, is_sft, toks, resp in zip(begins, sft, unconcat_tokens, response_lengths, strict=False):
         chunk = flat[b : b + resp]
         targets = torch.nn.functional.pad(toks[1:], (0, 1), value=0) if is_sft else toks[-resp:]
@@ -84,11 +93,12 @@ def get_responses(
 class PackedLayout:
     """Device-side description of one packed micro-batch: response offsets, row maps and packed target ids."""
 
-    def __init__(self, device, n_rows: int, unconcat_tokens, total_lengths, response_lengths, need_inverse: bool):
+    def __init__(self, device, n_rows: int, unconcat_tokens, total_lengths, response_lengths, need_inverse: bool,
+                 max_seq_lens=None):
         self.response_lengths = [int(r) for r in response_lengths]
         self.n_samples = len(self.response_lengths)
         self.n_tokens = sum(self.response_lengths)
-        begins, sft = response_row_begins(total_lengths, response_lengths)
+        begins, sft = response_row_begins(total_lengths, response_lengths, max_seq_lens)
         for b, r in zip(begins, self.response_lengths):
             if r > 0 and (b < 0 or b + r > n_rows):
                 raise IndexError(f"response rows [{b}, {b + r}) fall outside the {n_rows} logits rows")
@@ -145,11 +155,12 @@ def get_log_probs_and_entropy(
     assert non_loss_data
     if lm_head_forward is not None:
         return _deferred_lm_head_log_probs(logits, args, unconcat_tokens, total_lengths, response_lengths,
-                                           with_entropy, lm_head_forward)
-    flat = _check_logits(logits, args)
+                                           with_entropy, lm_head_forward, max_seq_lens)
+    flat = _check_logits(logits, args, max_seq_lens)
     want_grad = with_entropy and getattr(args, "entropy_coef", 0.0) != 0
     needs_bwd = torch.is_grad_enabled() and logits.requires_grad
-    lay = PackedLayout(flat.device, flat.size(0), unconcat_tokens, total_lengths, response_lengths, needs_bwd)
+    lay = PackedLayout(flat.device, flat.size(0), unconcat_tokens, total_lengths, response_lengths, needs_bwd,
+                       _padded_starts(args, max_seq_lens))
     inv_t = 1.0 / float(getattr(args, "rollout_temperature", 1.0))
     if lay.n_tokens == 0:
         lp = flat.new_zeros((0,), dtype=torch.float32)
@@ -165,7 +176,7 @@ def get_log_probs_and_entropy(
         # diagnostic student-side top-K ids (loss.py:436-438): a library selection over each sample's own rows
         k = topk_k if topk_k is not None else getattr(args, "opd_log_prob_top_k", 1)
         k = min(max(int(k), 1), int(flat.size(-1)))
-        begins, _ = response_row_begins(total_lengths, response_lengths)
+        begins, _ = response_row_begins(total_lengths, response_lengths, _padded_starts(args, max_seq_lens))
         res["topk_token_ids"] = [torch.topk(flat[b:b + r], k=k, dim=-1).indices
                                  for b, r in zip(begins, lay.response_lengths)]
     if gather_topk_token_ids is not None:
@@ -191,14 +202,17 @@ def lm_head_weight_of(lm_head_forward) -> torch.Tensor:
 
 
 def _deferred_lm_head_log_probs(hidden, args, unconcat_tokens, total_lengths, response_lengths, with_entropy,
-                                lm_head_forward):
+                                lm_head_forward, max_seq_lens=None):
     """Deferred-LM-head branch of get_log_probs_and_entropy (loss.py:391-419): ``hidden`` is ``[1, T, H]`` (or
     ``[T, H]``) and the ``[T, V]`` logits are never formed.  The response rows of all samples go through the fused
     LM-head kernel in one launch; unlike the reference's chunked path entropy is available as well."""
     from .lm_head import lm_head_log_probs_and_entropy
 
     weight = lm_head_weight_of(lm_head_forward)
-    if hidden.dim() == 3:
+    padded = _padded_starts(args, max_seq_lens)
+    if hidden.dim() == 3 and padded is not None:
+        rows = hidden.reshape(-1, hidden.size(-1))  # [B, S, H]: sample i starts at row max_seq_lens[i] * i
+    elif hidden.dim() == 3:
         if hidden.size(0) != 1:
             raise ValueError(f"expected packed hidden states [1, T, H], got {tuple(hidden.shape)}")
         rows = hidden[0]
@@ -208,7 +222,7 @@ def _deferred_lm_head_log_probs(hidden, args, unconcat_tokens, total_lengths, re
         raise ValueError(f"hidden states {tuple(hidden.shape)} do not match the LM-head weight {tuple(weight.shape)}")
     if not rows.is_cuda:
         raise RuntimeError("relax_amd kernels need ROCm device tensors (no CPU fallback)")
-    lay = PackedLayout(rows.device, rows.size(0), unconcat_tokens, total_lengths, response_lengths, False)
+    lay = PackedLayout(rows.device, rows.size(0), unconcat_tokens, total_lengths, response_lengths, False, padded)
     if lay.n_tokens == 0:
         lp = rows.new_zeros((0,), dtype=torch.float32)
         ent = lp
@@ -231,7 +245,8 @@ def sft_loss_function_chunked(args: Namespace, batch: dict, hidden_states: torch
     reference's reducer is then rebuilt from the batch."""
     _, out = get_log_probs_and_entropy(
         hidden_states, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=batch["total_lengths"],
-        response_lengths=batch["response_lengths"], with_entropy=False, lm_head_forward=lm_head_forward)
+        response_lengths=batch["response_lengths"], with_entropy=False, lm_head_forward=lm_head_forward,
+        max_seq_lens=batch.get("max_seq_lens"))
     log_probs = torch.cat(out["log_probs"], dim=0)
     if sum_of_sample_mean is None:
         sum_of_sample_mean = get_sum_of_sample_mean(
@@ -248,7 +263,7 @@ def sft_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum_of
     packed log-prob launch.  ``sum_of_sample_mean`` may be None: the reference's reducer is then rebuilt from the batch."""
     _, out = get_log_probs_and_entropy(
         logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=batch["total_lengths"],
-        response_lengths=batch["response_lengths"], with_entropy=False)
+        response_lengths=batch["response_lengths"], with_entropy=False, max_seq_lens=batch.get("max_seq_lens"))
     log_probs = torch.cat(out["log_probs"], dim=0)
     if sum_of_sample_mean is None:
         sum_of_sample_mean = get_sum_of_sample_mean(
@@ -459,7 +474,7 @@ def _composed_policy_loss_function(args: Namespace, batch: dict, logits: torch.T
     adv = adv.to(dev).float() if isinstance(adv, torch.Tensor) else torch.cat([a.to(dev) for a in adv]).float()
     _, out = get_log_probs_and_entropy(
         logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=total_lengths,
-        response_lengths=response_lengths, with_entropy=True,
+        response_lengths=response_lengths, with_entropy=True, max_seq_lens=batch.get("max_seq_lens"),
         gather_topk_token_ids=resolve_opd_gather_topk_token_ids(args, batch))
     lps = out["log_probs"]
     true_on_policy = getattr(args, "true_on_policy_mode", False)
@@ -575,16 +590,16 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     ``args.custom_pg_loss_reducer_function_path`` set, the loss is composed step by step around the user's callables
     (``_composed_policy_loss_function``) instead of being evaluated inside one kernel.
     """
-    flat = _check_logits(logits, args)
+    flat = _check_logits(logits, args, batch.get("max_seq_lens"))
     dev = flat.device
     est = args.advantage_estimator
     if getattr(args, "custom_tis_function_path", None) is not None \
             or getattr(args, "custom_pg_loss_reducer_function_path", None) is not None:
-        _check_logits(logits, args)
         return _composed_policy_loss_function(args, batch, logits, None)  # user code acts on per-token tensors
     response_lengths, total_lengths = batch["response_lengths"], batch["total_lengths"]
     needs_bwd = torch.is_grad_enabled() and logits.requires_grad
-    lay = PackedLayout(dev, flat.size(0), batch["unconcat_tokens"], total_lengths, response_lengths, needs_bwd)
+    lay = PackedLayout(dev, flat.size(0), batch["unconcat_tokens"], total_lengths, response_lengths, needs_bwd,
+                       _padded_starts(args, batch.get("max_seq_lens")))
 
     true_on_policy = getattr(args, "true_on_policy_mode", False)
     use_rollout = getattr(args, "use_rollout_logprobs", False)
@@ -667,7 +682,7 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
 
         _, lpe = get_log_probs_and_entropy(
             logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=total_lengths,
-            response_lengths=response_lengths, with_entropy=False,
+            response_lengths=response_lengths, with_entropy=False, max_seq_lens=batch.get("max_seq_lens"),
             gather_topk_token_ids=resolve_opd_gather_topk_token_ids(args, batch))
         old_for_opd = old if old is not None else lp.detach()
         opd_loss, opd_reported = compute_policy_opd_loss(
@@ -706,9 +721,11 @@ def get_values(logits: torch.Tensor, *, args: Namespace, unconcat_tokens, total_
     """Counterpart of loss.py:466-518: the value head's output ``[1, T, 1]`` at every response token, as per-sample
     ``[R_i]`` views of one packed gather (the same row map as the log-prob path; no temperature), differentiable
     w.r.t. ``logits``.  Returns ``(empty, {"values": [...]})``."""
-    assert logits.dim() == 3 and logits.size(0) == 1 and logits.size(-1) == 1, f"{logits.shape}"
+    assert logits.dim() == 3 and logits.size(-1) == 1, f"{logits.shape}"
+    padded = _padded_starts(args, max_seq_lens)
+    assert logits.size(0) == 1 or padded is not None, f"{logits.shape}"
     flat = logits.reshape(-1)
-    lay = PackedLayout(flat.device, flat.size(0), unconcat_tokens, total_lengths, response_lengths, False)
+    lay = PackedLayout(flat.device, flat.size(0), unconcat_tokens, total_lengths, response_lengths, False, padded)
     values = flat.index_select(0, lay.row_ids.to(torch.int64)) if lay.n_tokens else flat[:0]
     return torch.empty((0,), device=flat.device), {"values": lay.split(values)}
 

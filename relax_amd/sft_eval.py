@@ -14,7 +14,7 @@ import torch
 
 
 def compute_sft_eval_step(logits: torch.Tensor, *, args, unconcat_tokens, total_lengths, response_lengths,
-                          with_entropy: bool = False, loss_masks=None, lm_head_forward=None, **_):
+                          with_entropy: bool = False, loss_masks=None, lm_head_forward=None, max_seq_lens=None, **_):
     """``(empty tensor, {"sum_neg_log_prob": [fp32 [1]], "num_tokens": [int64 [1]]})`` (ppl.py:24-92).  ``logits`` may
     be hidden states when ``lm_head_forward`` is given, as for ``get_log_probs_and_entropy``."""
     from .cp_utils import get_sum_of_sample_mean
@@ -24,7 +24,8 @@ def compute_sft_eval_step(logits: torch.Tensor, *, args, unconcat_tokens, total_
     with torch.no_grad():
         _, res = get_log_probs_and_entropy(logits, args=args, unconcat_tokens=unconcat_tokens,
                                            total_lengths=total_lengths, response_lengths=response_lengths,
-                                           with_entropy=False, lm_head_forward=lm_head_forward)
+                                           with_entropy=False, lm_head_forward=lm_head_forward,
+                                           max_seq_lens=max_seq_lens)
         flat = torch.cat(res["log_probs"], dim=0)
         token_sum = get_sum_of_sample_mean(total_lengths, response_lengths, loss_masks, calculate_per_token_loss=True)
         sum_neg_lp = -token_sum(flat)

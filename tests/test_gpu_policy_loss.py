@@ -455,6 +455,60 @@ def test_value_loss_function_vs_oracle_and_closed_forms(per_token):
     assert met4["value_clipfrac"].item() == 0
 
 
+@pytest.mark.parametrize("case", ["ppo_k3_entropy", "gspo", "m2po_interior"])
+def test_padded_bshd_layout_equals_packed_layout(case):
+    """``qkv_format="bshd"``: logits [B, S, V] padded to S = max_seq_len rows per sample (loss.py:94-117).  The same
+    samples laid out packed and padded give the same loss and metrics bit for bit, the same gradient on every real
+    row and exact zeros on the padding; the response rows are the ones brute-force enumeration names."""
+    import relax_amd
+    from relax_amd.loss import response_row_begins
+
+    dev = require_gpu()
+    announce("bshd layout", case)
+    tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 264
+    s_max = 13
+    logits, batch = _make_batch(17, tot, resp, v)
+    begins, _ = response_row_begins(tot, resp, [s_max] * 4)
+    want_rows = [s_max * i + t - r - 1 for i, (t, r) in enumerate(zip(tot, resp))]  # previous position scores a token
+    assert begins == want_rows
+    assert [b for b, _e, _s in P.response_row_ranges(tot, resp, [s_max] * 4)] == want_rows
+    padded = torch.full((4, s_max, v), 7.0)  # padding rows hold junk that must not matter
+    off = 0
+    for i, t in enumerate(tot):
+        padded[i, :t] = logits[0, off:off + t]
+        off += t
+    bd = _to_dev(batch, dev)
+    args = P.make_args(**CASES[case])
+    lg = logits.to(dev).requires_grad_()
+    loss, met = relax_amd.policy_loss_function(args, bd, lg, None)
+    loss.backward()
+    args_b = P.make_args(qkv_format="bshd", **CASES[case])
+    bd_b = dict(bd, max_seq_lens=[s_max] * 4)
+    pg = padded.to(dev).requires_grad_()
+    loss_b, met_b = relax_amd.policy_loss_function(args_b, bd_b, pg, None)
+    loss_b.backward()
+    assert loss_b.item() == loss.item()
+    for k in met:
+        assert met_b[k].item() == met[k].item(), k
+    assert pg.grad.shape == padded.shape
+    off = 0
+    for i, t in enumerate(tot):
+        assert torch.equal(pg.grad[i, :t], lg.grad[0, off:off + t])
+        assert not pg.grad[i, t:].any()
+        off += t
+    _, out = relax_amd.get_log_probs_and_entropy(padded.to(dev), args=args_b, unconcat_tokens=bd["unconcat_tokens"],
+                                                 total_lengths=tot, response_lengths=resp, with_entropy=True,
+                                                 max_seq_lens=[s_max] * 4)
+    _, ref = relax_amd.get_log_probs_and_entropy(logits.to(dev), args=args, unconcat_tokens=bd["unconcat_tokens"],
+                                                 total_lengths=tot, response_lengths=resp, with_entropy=True)
+    for a, b in zip(out["log_probs"] + out["entropy"], ref["log_probs"] + ref["entropy"]):
+        assert torch.equal(a, b)
+    chunks = list(relax_amd.get_responses(padded.to(dev), args=args_b, unconcat_tokens=bd["unconcat_tokens"],
+                                          total_lengths=tot, response_lengths=resp, max_seq_lens=[s_max] * 4))
+    for (chunk, _tk), b, r in zip(chunks, want_rows, resp):
+        assert torch.equal(chunk.cpu(), padded.reshape(-1, v)[b:b + r])
+
+
 def test_reducers_vs_oracle_literals(literals):
     from relax_amd import cp_utils
 
