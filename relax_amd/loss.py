@@ -757,6 +757,14 @@ def value_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum_
     return loss, {"value_loss": loss.clone().detach(), "value_clipfrac": clipfrac.clone().detach()}
 
 
+def mtp_only_loss_function(args: Namespace, batch: dict, hidden_states: torch.Tensor, sum_of_sample_mean=None):
+    """loss.py:1431-1440: no language loss of its own; a zero that keeps the graph (and the multi-token-prediction
+    auxiliary loss attached to it) alive."""
+    del args, batch, sum_of_sample_mean
+    loss = 0.0 * hidden_states.sum()
+    return loss, {"loss": loss.detach()}
+
+
 def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: torch.Tensor, *, lm_head_forward=None,
                   dp_world_size: int = 1):
     """Counterpart of loss.py:1443-1620 on one GPU: token count, the loss selected by ``args.loss_type``
@@ -767,21 +775,34 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
     if loss_type not in ("policy_loss", "value_loss", "sft", "custom_loss"):
         raise ValueError(f"Unknown loss type: {loss_type}")
     num_tokens = get_cp_local_num_tokens(batch["total_lengths"], batch["response_lengths"], batch["loss_masks"])
-    if loss_type == "policy_loss":
-        loss, log = policy_loss_function(args, batch, logits, None)
+    reducer = None
+    if getattr(args, "mtp_only_training", False):
+        func = mtp_only_loss_function
+    elif loss_type == "policy_loss":
+        func = policy_loss_function
     elif loss_type == "value_loss":
-        loss, log = value_loss_function(args, batch, logits, None)
+        func = value_loss_function
     elif loss_type == "custom_loss":  # loss.py:1530-1531: the plug-in gets the reducer the built-in losses use
         reducer = get_sum_of_sample_mean(batch["total_lengths"], batch["response_lengths"], batch["loss_masks"],
                                          bool(getattr(args, "calculate_per_token_loss", False)),
                                          sample_denoms=batch.get("sample_index_mask_sums"))
-        loss, log = load_function(args.custom_loss_function_path)(args, batch, logits, reducer)
+        func = load_function(args.custom_loss_function_path)
     elif getattr(args, "task_type", "causal_lm") == "seq_cls":
         raise NotImplementedError("sequence-classification SFT is outside the fused policy path")
     elif getattr(args, "sft_chunked_logits", False) and lm_head_forward is not None:
-        loss, log = sft_loss_function_chunked(args, batch, logits, None, lm_head_forward=lm_head_forward)
+        from functools import partial
+
+        func = partial(sft_loss_function_chunked, lm_head_forward=lm_head_forward)
     else:
-        loss, log = sft_loss_function(args, batch, logits, None)
+        func = sft_loss_function
+    if getattr(args, "recompute_loss_function", False):
+        # loss.py:1535-1543: the loss is evaluated again during backward instead of keeping what it saved
+        from torch.utils.checkpoint import checkpoint
+
+        loss, log = checkpoint(func, args, batch, logits, reducer,
+                               use_reentrant=getattr(args, "recompute_loss_function_use_reentrant", True))
+    else:
+        loss, log = func(args, batch, logits, reducer)
     per_token = bool(getattr(args, "calculate_per_token_loss", False))
     if per_token and getattr(args, "advantage_estimator", None) == "m2po":
         # the M2PO scalars are global, not per-token sums: pre-multiplied so that the logger's division by the token

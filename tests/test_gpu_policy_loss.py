@@ -221,6 +221,53 @@ def test_loss_function_scaling_and_exact_token_count():
     assert n.dtype == torch.int64 and n.item() == R.num_tokens(batch["loss_masks"]).item()
 
 
+@pytest.mark.parametrize("loss_type", ["policy_loss", "sft", "value_loss"])
+@pytest.mark.parametrize("reentrant", [True, False])
+def test_loss_function_recompute_gives_the_same_loss_and_gradient(loss_type, reentrant):
+    """``--recompute-loss-function`` (loss.py:1535-1543): the loss runs under ``torch.utils.checkpoint`` -- once
+    without autograd, once more during backward -- and must return the same loss, logging values and gradient, bit
+    for bit, as the direct call."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("loss_function recompute", loss_type, reentrant)
+    tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 264
+    logits, batch = _make_batch(41, tot, resp, v)
+    n = sum(resp)
+    g = torch.Generator().manual_seed(1)
+    batch["values"] = list(torch.split(torch.randn(n, generator=g), resp))
+    batch["returns"] = list(torch.split(torch.randn(n, generator=g), resp))
+    x = torch.randn(1, sum(tot), 1, generator=g) if loss_type == "value_loss" else logits
+    bd = _to_dev(batch, dev)
+    results = []
+    for recompute in (False, True):
+        args = P.make_args(loss_type=loss_type, value_clip=0.3, global_batch_size=4, use_kl_loss=True,
+                           kl_loss_coef=0.01, kl_loss_type="k3", entropy_coef=0.01,
+                           recompute_loss_function=recompute, recompute_loss_function_use_reentrant=reentrant)
+        xd = x.to(dev).requires_grad_()
+        loss, _norm, log = relax_amd.loss_function(args, bd, 2, xd)
+        loss.backward()
+        results.append((loss.detach(), log["keys"], log["values"], xd.grad))
+    (l0, k0, v0, g0), (l1, k1, v1, g1) = results
+    assert k0 == k1 and torch.equal(l0, l1) and torch.equal(v0, v1) and torch.equal(g0, g1)
+    assert g0.abs().sum().item() > 0
+
+
+def test_mtp_only_training_dispatch():
+    """``args.mtp_only_training`` (loss.py:1431-1440, 1512-1513): a zero loss that stays attached to its input."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("mtp only")
+    tot, resp, v = [9, 6], [4, 3], 64
+    logits, batch = _make_batch(4, tot, resp, v)
+    args = P.make_args(mtp_only_training=True, global_batch_size=2)
+    hd = torch.randn(1, sum(tot), 16).to(dev).requires_grad_()
+    loss, _norm, log = relax_amd.loss_function(args, _to_dev(batch, dev), 1, hd)
+    loss.backward()
+    assert loss.item() == 0 and log["keys"] == ["loss"] and not hd.grad.any() and hd.grad.shape == hd.shape
+
+
 def test_get_log_probs_and_entropy_forward_only_matches_training_forward_bitwise():
     """The forward-only pass and the training forward must give identical log-probs for identical inputs."""
     import relax_amd
