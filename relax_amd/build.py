@@ -72,7 +72,29 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
     if verbose:
         print(f"built {LIB_PATH} from {len(srcs)} sources")
+    build_abi_client(verbose)
     return LIB_PATH
+
+
+ABI_CLIENT_SRC = os.path.join(os.path.dirname(HERE), "tests", "abi_client.c")
+ABI_CLIENT = os.path.join(BUILD_DIR, "abi_client")
+
+
+def build_abi_client(verbose: bool = True) -> str | None:
+    """The plain-C client of the library used by the GPU tests (no Python, no PyTorch in the process): compiled as C
+    against ``include/relax_amd.h`` and the HIP runtime API, linked to the library just built."""
+    if not os.path.exists(ABI_CLIENT_SRC):
+        return None
+    rocm = os.path.dirname(os.path.dirname(HIPCC))
+    cmd = ["gcc", "-std=c11", "-O1", "-Wall", "-D__HIP_PLATFORM_AMD__", f"-I{INCLUDE}", f"-I{rocm}/include",
+           ABI_CLIENT_SRC, "-o", ABI_CLIENT, f"-L{HERE}", "-lrelax_amd", f"-L{rocm}/lib", "-lamdhip64", "-lm",
+           f"-Wl,-rpath,{HERE}", "-Wl,-rpath,$ORIGIN/../..", f"-Wl,-rpath,{rocm}/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"building the C client failed:\n{r.stdout}\n{r.stderr}")
+    if verbose:
+        print(f"built {ABI_CLIENT}")
+    return ABI_CLIENT
 
 
 if __name__ == "__main__":
