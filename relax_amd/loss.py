@@ -258,9 +258,40 @@ def sft_loss_function_chunked(args: Namespace, batch: dict, hidden_states: torch
     return loss, {"loss": loss.clone().detach()}
 
 
+def _sft_single_pass(args: Namespace, batch: dict, logits: torch.Tensor):
+    """The SFT loss as one launch of the fused step: ``-sum_of_sample_mean(lp)`` is the REINFORCE surrogate
+    ``-A * lp`` with unit advantages and no KL or entropy term, so forward scan and dlogits share one pass over the
+    logits (one HBM read and one write per row instead of two reads and a write)."""
+    flat = _check_logits(logits, args, batch.get("max_seq_lens"))
+    dev = flat.device
+    lay = PackedLayout(dev, flat.size(0), batch["unconcat_tokens"], batch["total_lengths"], batch["response_lengths"],
+                       True, _padded_starts(args, batch.get("max_seq_lens")))
+    if lay.n_tokens == 0:
+        return None
+    per_token = bool(getattr(args, "calculate_per_token_loss", False))
+    masks = [m.to(dev) for m in batch["loss_masks"]]
+    denom = None if per_token else sample_denominators(masks, lay, batch.get("sample_index_mask_sums"))
+    kw = dict(
+        old_log_prob=None, ref_log_prob=None, train_log_prob=None, rollout_log_prob=None,
+        advantages=torch.ones(lay.n_tokens, dtype=torch.float32, device=dev), loss_mask=_cat_f32(masks, dev),
+        sample_denom=denom, pg_sample_denom=None, loss_kind="rloo", kl_kind=None, unbiased_kl=False, use_opsm=False,
+        use_tis=False, mismatch_metrics=False, abs_diff_from_old=2, eps_clip=0.2, eps_clip_high=0.2, entropy_coef=0.0,
+        kl_coef=0.0, tis_lo=0.0, tis_hi=2.0, opsm_delta=1e-4, tau_pos=1.0, tau_neg=1.05)
+    inv_t = 1.0 / float(getattr(args, "rollout_temperature", 1.0))
+    loss, _metrics, _lp, _ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw)
+    return loss
+
+
 def sft_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum_of_sample_mean=None):
-    """Negative log-likelihood of the response tokens (loss.py:1247-1293): ``-sum_of_sample_mean(log_probs)`` from one
-    packed log-prob launch.  ``sum_of_sample_mean`` may be None: the reference's reducer is then rebuilt from the batch."""
+    """Negative log-likelihood of the response tokens (loss.py:1247-1293): ``-sum_of_sample_mean(log_probs)``.
+    ``sum_of_sample_mean`` may be None: the reference's reducer is then rebuilt from the batch, and when a gradient
+    is wanted the whole loss runs as one launch (``args.relax_amd_single_pass = "off"`` keeps the separate log-prob
+    forward / backward launches)."""
+    if sum_of_sample_mean is None and torch.is_grad_enabled() and logits.requires_grad \
+            and getattr(args, "relax_amd_single_pass", "auto") not in (False, "off"):
+        loss = _sft_single_pass(args, batch, logits)
+        if loss is not None:
+            return loss, {"loss": loss.clone().detach()}
     _, out = get_log_probs_and_entropy(
         logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=batch["total_lengths"],
         response_lengths=batch["response_lengths"], with_entropy=False, max_seq_lens=batch.get("max_seq_lens"))

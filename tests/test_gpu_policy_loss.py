@@ -830,6 +830,46 @@ def test_callable_from_worker_threads_and_under_activation_checkpointing():
     assert torch.equal(loss.detach(), want[0]) and torch.equal(lg.grad, want[1])
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-5), (torch.bfloat16, 2e-3)])
+@pytest.mark.parametrize("per_token", [False, True])
+def test_sft_loss_single_launch_equals_two_launch_path_and_oracle(dtype, tol, per_token):
+    """sft_loss_function with a gradient wanted runs as one launch of the fused step (REINFORCE surrogate with unit
+    advantages); ``relax_amd_single_pass="off"`` keeps the separate forward / backward launches.  Both against the
+    oracle's -sum_of_sample_mean(log_probs), SFT-shaped (response == total) and RL-shaped samples mixed, a
+    temperature other than 1, an upstream gradient other than 1; no-grad calls return the same loss."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("sft single launch", dtype, per_token)
+    tot, resp, v = [7, 12, 5, 9], [7, 5, 5, 4], 264
+    logits, batch = _make_batch(19, tot, resp, v, dtype)
+    lo = logits.float().clone().requires_grad_()
+    oargs = P.make_args(loss_type="sft", rollout_temperature=0.8, calculate_per_token_loss=per_token)
+    _, out = P.get_log_probs_and_entropy(lo, args=oargs, unconcat_tokens=batch["unconcat_tokens"], total_lengths=tot,
+                                         response_lengths=resp)
+    want = -R.make_reducer(resp, batch["loss_masks"], per_token)(torch.cat(out["log_probs"]))
+    (1.7 * want).backward()
+    bd = _to_dev(batch, dev)
+    got = {}
+    for mode in ("auto", "off"):
+        args = P.make_args(loss_type="sft", rollout_temperature=0.8, calculate_per_token_loss=per_token,
+                           relax_amd_single_pass=mode)
+        lg = logits.to(dev).requires_grad_()
+        loss, log = relax_amd.sft_loss_function(args, bd, lg, None)
+        (1.7 * loss).backward()
+        assert list(log) == ["loss"] and log["loss"].item() == loss.item()
+        assert abs(loss.item() - want.item()) < tol * max(1.0, abs(want.item())), (mode, loss.item(), want.item())
+        assert lg.grad.dtype == dtype
+        torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, atol=tol, rtol=BF16_ULP if dtype == torch.bfloat16 else 0)
+        got[mode] = (loss.item(), lg.grad)
+        with torch.no_grad():
+            quiet, _ = relax_amd.sft_loss_function(args, bd, logits.to(dev), None)
+        assert abs(quiet.item() - loss.item()) < 1e-6 * max(1.0, abs(loss.item()))
+    assert abs(got["auto"][0] - got["off"][0]) < 1e-6 * max(1.0, abs(want.item()))
+    torch.testing.assert_close(got["auto"][1].float(), got["off"][1].float(), atol=tol * 1e-2,
+                               rtol=2 * BF16_ULP if dtype == torch.bfloat16 else 1e-5)
+
+
 def test_sft_eval_step_sums_and_counts_vs_oracle():
     """The SFT evaluation callback (relax/engine/sft/eval/ppl.py:24-92): masked sum of negative log-probs and the
     exact token count per micro-batch, in the shapes and dtypes the forward-only harness stacks."""
