@@ -657,6 +657,8 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_dlogits_kernel(
 
 using namespace relax_amd;
 
+static int lm_max_splits(int64_t n_tokens);
+
 static int lm_geometry(const char* what, int dtype, int64_t n, int64_t hidden, int64_t vocab, int64_t h_stride,
                        int64_t w_stride, const void* h, const void* w, LmGeom& g) {
   if (dtype != RELAX_AMD_BF16) {
@@ -681,11 +683,28 @@ static int lm_geometry(const char* what, int dtype, int64_t n, int64_t hidden, i
   g.w_stride = w_stride;
   g.row_blocks = int((n + kLmTile - 1) / kLmTile);
   g.n_tiles = int((vocab + kLmTile - 1) / kLmTile);
-  int s = 1;
-  while (s < 8 && g.row_blocks * s < 512 && s * 2 <= g.n_tiles) s *= 2;
+  int s = lm_max_splits(n);
+  while (s > 1 && s > g.n_tiles) s /= 2;
   g.splits = s;
   g.tiles_per_split = (g.n_tiles + s - 1) / s;
   return RELAX_AMD_OK;
+}
+
+// Vocabulary splits per row block as far as the token count decides (the workspace is sized from it): enough to put
+// two workgroups on every CU while that takes at most 8 splits, and for short inputs up to 32 (one row block per XCD)
+// as long as fewer than 256 workgroups would otherwise have work.
+static int lm_max_splits(int64_t n_tokens) {
+  const int64_t row_blocks = (n_tokens + kLmTile - 1) / kLmTile;
+  int s = 1;
+  while (s < 8 && row_blocks * s < 512) s *= 2;
+  while (s < kLmPerXcd && row_blocks * s < 256) s *= 2;
+  return s;
+}
+
+// floats of per-split softmax partials in the workspace (three per token and split)
+static int64_t lm_partial_floats(int64_t n_tokens) {
+  const int s = lm_max_splits(n_tokens);
+  return int64_t(s < 8 ? 8 : s) * 3 * n_tokens;
 }
 
 static unsigned lm_grid(const LmGeom& g) {
@@ -696,7 +715,7 @@ static unsigned lm_grid(const LmGeom& g) {
 
 extern "C" int64_t relax_amd_lmhead_workspace_bytes(int64_t n_tokens) {
   if (n_tokens <= 0) return 0;
-  return (8 * 3 + 1) * n_tokens * int64_t(sizeof(float));
+  return (lm_partial_floats(n_tokens) + n_tokens) * int64_t(sizeof(float));
 }
 
 // 4-byte paired stores need an even row stride and a 4-byte aligned base
@@ -724,7 +743,7 @@ static int lm_forward(const char* what, const void* hidden, const void* weight, 
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* partial = static_cast<float*>(workspace);
-  float* x_target = partial + 8 * 3 * n_tokens;
+  float* x_target = partial + lm_partial_floats(n_tokens);
   const uint16_t* h = static_cast<const uint16_t*>(hidden);
   const uint16_t* w = static_cast<const uint16_t*>(weight);
   const float c = inv_temperature * kLog2e;

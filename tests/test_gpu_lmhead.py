@@ -44,6 +44,8 @@ def _oracle(hid, w, tok, wl, we, temperature):
     (1024, 256, 5000, 1.0),     # several vocab tiles and splits
     (70, 4096, 1030, 1.0),      # production hidden size
     (301, 128, 700, 1.0),       # odd token count: odd slab stride, 2-byte stores in the backward slab
+    (300, 128, 9000, 1.0),      # few tokens, 36 vocabulary tiles: 32 vocabulary splits per row block
+    (600, 128, 5000, 0.9),      # 20 tiles: 16 splits, the last ones short or empty
 ])
 def test_forward_backward_vs_oracle(n, h, v, temperature):
     from relax_amd.lm_head import lm_head_log_probs_and_entropy
@@ -89,6 +91,7 @@ def _oracle_bf16_logits(hid, w, tok, wl, we, temperature):
     (301, 128, 1000, 0.7),      # ragged vocabulary, odd token count (a half-filled token pair at the end)
     (1024, 256, 5000, 1.0),
     (70, 4096, 1030, 1.0),
+    (300, 128, 9000, 1.0),      # 32 vocabulary splits per row block
 ])
 def test_keep_logits_forward_backward_vs_bf16_logit_oracle(n, h, v, temperature):
     from relax_amd.lm_head import lm_head_log_probs_and_entropy
