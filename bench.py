@@ -427,6 +427,45 @@ def run_hbm_ceiling(a, dev) -> None:
         "cpu_baseline": None}))
 
 
+def run_actor_fwd_topk(a, dev) -> None:
+    """The forward-only pass the actor runs when it also collects the student's top-K ids for on-policy distillation
+    (compute_log_prob(collect_topk=True)): log-probs + entropy and ``topk_token_ids`` of every response row of the
+    actor-step logits, no gradient.  ``--vendor-topk`` times torch.topk on the same rows instead of the library's
+    selection kernel (the rest of the pass unchanged)."""
+    import relax_amd
+    from relax_amd import ops
+
+    args = make_args()
+    args.opd_log_prob_top_k = a.topk
+    logits, batch, _ = make_workload(dev, a.seqs, a.seq_len, a.vocab)
+    n_tokens = a.seqs * a.seq_len
+    if a.vendor_topk:
+        ops.TOPK_ROWS_MAX_K = 0  # get_log_probs_and_entropy then selects with torch.topk, sample by sample
+
+    def step():
+        with torch.no_grad():
+            _, out = relax_amd.get_log_probs_and_entropy(
+                logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=batch["total_lengths"],
+                response_lengths=batch["response_lengths"], with_entropy=True, with_topk=True, topk_k=a.topk)
+        return out["topk_token_ids"][-1][-1, 0].float()
+
+    wall, kernel_ms, _, _ = timed_steps(step, a.warmup, a.steps)
+    row_bytes = float(a.vocab * logits.element_size()) * n_tokens
+    if "topk_rows" in kernel_ms:
+        # the selection reads every row (the second look at a row is served by the caches in part)
+        dom, dom_name = kernel_ms["topk_rows"], "topk_rows_fast_kernel<bf16_t, true>"
+    else:
+        dom, dom_name = kernel_ms["logprob_entropy_fwd"], "logprob_entropy_fwd_kernel<bf16_t, true, 1024>"
+    achieved = row_bytes / (dom * 1e-3) / 1e9
+    emit(a, n_tokens, wall,
+         f"actor forward-only pass with student top-{a.topk} ids: {a.seqs} seqs x {a.seq_len} tokens x V={a.vocab} bf16 "
+         f"logits, log-prob + entropy + top-K selection" + (" [torch.topk selection]" if a.vendor_topk else ""),
+         {"rows": n_tokens, "vocab": a.vocab, "k": a.topk},
+         {"bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+          "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": row_bytes,
+          "avg_launch_ms": dom, "kernel_ms": kernel_ms}, None)
+
+
 def run_reverse_kl(a, dev) -> None:
     """student / teacher bf16 logits [N, V], teacher = student + N(0, 1); per-token full-vocabulary reverse KL with a
     15 % zero loss mask, token-mean reduction, backward to the student's dlogits."""
@@ -630,7 +669,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="actor_step",
-                    choices=["actor_step", "cfg1", "lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "mfma_ceiling", "hbm_ceiling"])
+                    choices=["actor_step", "cfg1", "lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "actor_fwd_topk",
+                             "mfma_ceiling", "hbm_ceiling"])
     ap.add_argument("--seqs", type=int, default=SEQS)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
     ap.add_argument("--vocab", type=int, default=VOCAB)
@@ -649,6 +689,9 @@ def main() -> int:
                          "the fused kernel (same operands, logits written to HBM), for comparison")
     ap.add_argument("--lmhead-operands", choices=["random", "zeros"], default="random",
                     help="lmhead workload, diagnostic: all-zero operands show the kernel without the board power limit")
+    ap.add_argument("--topk", type=int, default=64, help="k of the actor_fwd_topk workload")
+    ap.add_argument("--vendor-topk", action="store_true",
+                    help="actor_fwd_topk: select with torch.topk instead of the library's kernel (comparison)")
     ap.add_argument("--two-launch", action="store_true",
                     help="use the separate forward / backward launches (the path GSPO takes) instead of the fused step")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -677,6 +720,8 @@ def main() -> int:
         run_hbm_ceiling(a, dev)
     elif a.workload == "reverse_kl":
         run_reverse_kl(a, dev)
+    elif a.workload == "actor_fwd_topk":
+        run_actor_fwd_topk(a, dev)
     else:
         run_varlen(a, dev, a.workload.split("_")[1])
     return 0

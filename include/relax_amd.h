@@ -326,6 +326,22 @@ int relax_amd_opd_kl_topk_bwd(const float* student_lp, const float* teacher_lp, 
                               float log_prob_min_clamp, const float* g, float* d_student_lp, void* stream);
 
 /*
+ * The k largest logits of each token's row and their vocabulary ids, largest first: torch.topk(logits_chunk, k=k,
+ * dim=-1) of get_log_probs_and_entropy (relax/backends/megatron/loss.py:434-436), for every response row in one
+ * launch.  NaN orders above +inf as in torch.topk; which of several equal values at the k-th place is returned is
+ * unspecified there and here.
+ *   row_ids  int32 [n_tokens] logits row of each token, or NULL (row t = token t)
+ *   values   fp32 [n_tokens, k] out (the logits as fp32), or NULL
+ *   indices  int64 [n_tokens, k] out
+ *   workspace n_tokens bytes of device memory (one flag per row: rows with long runs of equal values take a second,
+ *            general kernel)
+ * 1 <= k <= 512 and vocab <= 1000000, otherwise RELAX_AMD_EUNSUPPORTED.
+ */
+int relax_amd_topk_rows(const void* logits, int dtype, int64_t n_tokens, int64_t vocab, int64_t row_stride,
+                        const int32_t* row_ids, int k, float* values, int64_t* indices, uint8_t* workspace,
+                        void* stream);
+
+/*
  * Fused actor step: log-prob + entropy forward, the per-token terms of relax_amd_policy_loss and the dlogits backward
  * in one launch.  Each workgroup scans its row, derives the token's gradient constants and immediately walks the row
  * again to emit dlogits; the second walk is served by the L2 / memory-side cache, so HBM sees one read and one write

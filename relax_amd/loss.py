@@ -176,9 +176,14 @@ def get_log_probs_and_entropy(
         # diagnostic student-side top-K ids (loss.py:436-438): a library selection over each sample's own rows
         k = topk_k if topk_k is not None else getattr(args, "opd_log_prob_top_k", 1)
         k = min(max(int(k), 1), int(flat.size(-1)))
-        begins, _ = response_row_begins(total_lengths, response_lengths, _padded_starts(args, max_seq_lens))
-        res["topk_token_ids"] = [torch.topk(flat[b:b + r], k=k, dim=-1).indices
-                                 for b, r in zip(begins, lay.response_lengths)]
+        if lay.n_tokens and k <= ops.TOPK_ROWS_MAX_K and flat.size(-1) <= ops.TOPK_ROWS_MAX_VOCAB:
+            # one launch over every response row (the selection does not depend on the temperature)
+            _, ids = ops.topk_rows(flat, lay.row_ids, k, with_values=False)
+            res["topk_token_ids"] = lay.split(ids)
+        else:  # very large k: the library's selection, sample by sample like the reference
+            begins, _ = response_row_begins(total_lengths, response_lengths, _padded_starts(args, max_seq_lens))
+            res["topk_token_ids"] = [torch.topk(flat[b:b + r], k=k, dim=-1).indices
+                                     for b, r in zip(begins, lay.response_lengths)]
     if gather_topk_token_ids is not None:
         res["topk_log_probs"] = _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t)
     return torch.empty((0,), device=logits.device), res

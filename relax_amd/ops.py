@@ -337,6 +337,27 @@ def actor_step_fused(logits, targets, token_of_row, sample_ids, n_tokens: int, i
     return out, lp, ent, lse, spx, dlogits
 
 
+TOPK_ROWS_MAX_K = 512
+TOPK_ROWS_MAX_VOCAB = 1000000
+
+
+def topk_rows(logits, row_ids, k: int, with_values: bool = True):
+    """The ``k`` largest logits of each token's row, largest first: ``(values fp32 [n, k] | None, indices int64
+    [n, k])``.  ``row_ids`` (int32 [n]) names the logits row of each token; None scores every row."""
+    dev = _need_gpu(logits)
+    logits = _rows(logits)
+    n = int(row_ids.numel()) if row_ids is not None else logits.size(0)
+    k = int(k)
+    values = torch.empty((n, k), dtype=torch.float32, device=dev) if with_values else None
+    indices = torch.empty((n, k), dtype=torch.int64, device=dev)
+    flags = torch.empty(max(n, 1), dtype=torch.uint8, device=dev)
+    stride = logits.stride(0) if logits.size(0) > 1 else logits.size(1)
+    with _timed("topk_rows"):
+        check(lib.relax_amd_topk_rows(_p(logits), _code(logits), n, logits.size(1), stride, _p(row_ids), k, _p(values),
+                                      _p(indices), _p(flags), _stream()))
+    return values, indices
+
+
 def scale_rows_inplace(data, factor_dev):
     data2 = data.reshape(-1, data.size(-1))
     stride = data2.stride(0) if data2.size(0) > 1 else data2.size(1)

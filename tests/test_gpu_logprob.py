@@ -235,3 +235,97 @@ def test_full_size_properties_headline_shape():
     rlp, rent = O.calculate_log_probs_and_entropy(xs, tok[idx].cpu(), None, with_entropy=True)
     torch.testing.assert_close(lp[idx].cpu(), rlp.squeeze(-1), atol=2e-3, rtol=0)
     torch.testing.assert_close(ent[idx].cpu(), rent, atol=2e-3, rtol=0)
+
+
+# ------------------------------------------------------------------------------------------------- top-K selection
+
+
+def _check_topk_rows(x, k, row_ids=None):
+    """values equal torch.topk's exactly and are sorted; every index is valid, distinct and points at its value;
+    where a value is strictly greater than the k-th value the index must be among torch's."""
+    from relax_amd import ops
+
+    vals, idx = ops.topk_rows(x, row_ids, k)
+    rows = x if row_ids is None else x[row_ids.long()]
+    want = torch.topk(rows.float(), k, dim=-1)
+    got_v, want_v = vals, want.values
+    same = (got_v == want_v) | (torch.isnan(got_v) & torch.isnan(want_v))
+    assert same.all(), (got_v[~same][:5], want_v[~same][:5])
+    assert idx.dtype == torch.int64 and (idx >= 0).all() and (idx < x.size(1)).all()
+    gathered = torch.gather(rows.float(), 1, idx)
+    ok = (gathered == got_v) | (torch.isnan(gathered) & torch.isnan(got_v))
+    assert ok.all()
+    assert (torch.sort(idx, dim=1).values.diff(dim=1) > 0).all() or k == 1  # distinct
+    kth = want_v[:, -1:]
+    strict = got_v > kth
+    for r in range(min(rows.size(0), 64)):  # set equality above the threshold (ties at the threshold may differ)
+        assert set(idx[r][strict[r]].tolist()) == set(want.indices[r][want_v[r] > kth[r]].tolist())
+    return vals, idx
+
+
+@pytest.mark.parametrize("n,v,k,dtype", [
+    (64, 151936, 64, torch.bfloat16),    # the production vocabulary: many equal bf16 values around the threshold
+    (33, 151936, 8, torch.float32),      # what stock Megatron hands over
+    (50, 32003, 100, torch.float16),     # rows that are not 16-byte aligned (scalar loads)
+    (40, 4104, 512, torch.float32),      # the largest k
+    (17, 1000, 1, torch.bfloat16),       # k = 1: the arg-max
+    (9, 700, 700, torch.float32),        # k = vocabulary: a full sort... of at most 512 -> uses 512 below
+])
+def test_topk_rows_equals_torch_topk(n, v, k, dtype):
+    dev = require_gpu()
+    announce("topk rows", n, v, k, dtype)
+    k = min(k, 512)
+    g = torch.Generator(device=dev).manual_seed(n + v + k)
+    x = (torch.randn((n, v), device=dev, generator=g) * 3).to(dtype)
+    _check_topk_rows(x, k)
+    # through a row map: the last rows first, some rows twice
+    row_ids = torch.cat([torch.arange(n - 1, -1, -2, device=dev), torch.tensor([0, 0], device=dev)]).int()
+    _check_topk_rows(x, k, row_ids)
+
+
+def test_topk_rows_on_degenerate_rows():
+    """Rows that defeat the first histogram: all values equal (every key shares all 32 bits), two distinct values,
+    values that differ only in their low mantissa bits (three refinement passes), infinities, NaN (ordered above
+    +inf as torch does), signed zeros, and a row whose k-th value is shared by thousands of entries."""
+    dev = require_gpu()
+    announce("topk rows degenerate")
+    v, k = 20000, 50
+    g = torch.Generator(device=dev).manual_seed(7)
+    rows = [
+        torch.full((v,), 1.25, device=dev),
+        (torch.rand(v, device=dev, generator=g) > 0.999).float() * 3 - 1,
+        1.0 + torch.arange(v, device=dev).float() * 2.0 ** -22,
+        torch.randn(v, device=dev, generator=g),
+        torch.randn(v, device=dev, generator=g),
+        torch.zeros(v, device=dev),
+        torch.randn(v, device=dev, generator=g).round(),
+    ]
+    rows[3][5], rows[3][77], rows[3][4000] = float("inf"), float("-inf"), float("inf")
+    rows[4][123], rows[4][19999] = float("nan"), float("nan")
+    rows[5][::2] = -0.0
+    x = torch.stack(rows)
+    vals, idx = _check_topk_rows(x, k)
+    assert torch.isnan(vals[4, :2]).all() and set(idx[4, :2].tolist()) == {123, 19999}
+    assert set(idx[3, :2].tolist()) == {5, 4000}
+    assert (vals[0] == 1.25).all() and (vals[2] == x[2, -k:].flip(0)).all()
+    _check_topk_rows(x.bfloat16(), k)
+    _check_topk_rows(x, 512)
+
+
+def test_get_log_probs_and_entropy_with_topk_uses_one_launch_and_matches_torch():
+    """``with_topk=True`` (loss.py:434-446): per-sample ``topk_token_ids`` [R_i, k], the rows' k largest logits."""
+    import relax_amd
+    from oracle import policy as P
+
+    dev = require_gpu()
+    announce("with_topk")
+    tot, resp, v, k = [9, 6, 12], [4, 3, 7], 3000, 5
+    g = torch.Generator().manual_seed(12)
+    logits = (torch.randn(1, sum(tot), v, generator=g) * 2).to(dev)
+    toks = [torch.randint(0, v, (n,), generator=g).to(dev) for n in tot]
+    args = P.make_args(rollout_temperature=0.7, opd_log_prob_top_k=k)
+    _, out = relax_amd.get_log_probs_and_entropy(logits, args=args, unconcat_tokens=toks, total_lengths=tot,
+                                                 response_lengths=resp, with_topk=True)
+    assert [tuple(t.shape) for t in out["topk_token_ids"]] == [(r, k) for r in resp]
+    for (b, e, _), ids in zip(P.response_row_ranges(tot, resp), out["topk_token_ids"]):
+        assert torch.equal(ids, torch.topk(logits[0, b:e], k, dim=-1).indices)
