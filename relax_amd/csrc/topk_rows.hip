@@ -281,53 +281,63 @@ __global__ __launch_bounds__(kTkThreads) void topk_rows_kernel(const T* __restri
   uint64_t* const list = reinterpret_cast<uint64_t*>(hist_words);
   const int tid = threadIdx.x, wave = tid / kWave;
 
-  for (int64_t tok = blockIdx.x; tok < n_tokens; tok += gridDim.x) {
-    if (!needs_general[tok]) continue;  // the same answer in every thread
-    const int64_t row = row_ids ? int64_t(row_ids[tok]) : tok;
-    const T* x = logits + row * stride;
-    uint32_t prefix = 0, need = uint32_t(k);
-    int prefix_bits = 0;
-    while (true) {
-      const int db = 32 - prefix_bits < kTkDigitBits ? 32 - prefix_bits : kTkDigitBits;
-      for (int i = tid; i < kTkWaves * kTkBins / 2; i += kTkThreads) hist_words[i] = 0u;
-      __syncthreads();
-      tk_for_each<T, VEC, false>(x, vocab, [&](uint32_t, float v) {
+  // this workgroup's rows are blockIdx.x, blockIdx.x + gridDim.x, ...; their flags are fetched 1024 at a time, one per
+  // thread, so that a launch with nothing to do costs one load instead of a chain of them
+  __shared__ uint8_t flagged[kTkThreads];
+  for (int64_t chunk = blockIdx.x; chunk < n_tokens; chunk += int64_t(kTkThreads) * gridDim.x) {
+    const int64_t mine = chunk + int64_t(tid) * gridDim.x;
+    __syncthreads();  // the previous chunk's flags have been walked
+    flagged[tid] = mine < n_tokens ? needs_general[mine] : uint8_t(0);
+    if (!__syncthreads_or(flagged[tid])) continue;  // nothing flagged among these rows (the usual case)
+    for (int slot = 0; slot < kTkThreads; ++slot) {
+      if (!flagged[slot]) continue;  // the same answer in every thread
+      const int64_t tok = chunk + int64_t(slot) * gridDim.x;
+      const int64_t row = row_ids ? int64_t(row_ids[tok]) : tok;
+      const T* x = logits + row * stride;
+      uint32_t prefix = 0, need = uint32_t(k);
+      int prefix_bits = 0;
+      while (true) {
+        const int db = 32 - prefix_bits < kTkDigitBits ? 32 - prefix_bits : kTkDigitBits;
+        for (int i = tid; i < kTkWaves * kTkBins / 2; i += kTkThreads) hist_words[i] = 0u;
+        __syncthreads();
+        tk_for_each<T, VEC, false>(x, vocab, [&](uint32_t, float v) {
+          const uint32_t key = tk_key(v);
+          if (prefix_bits == 0 || (key >> (32 - prefix_bits)) == prefix) {
+            const uint32_t digit = (key << prefix_bits) >> (32 - db);
+            atomicAdd(&hist[wave][digit >> 1], (digit & 1u) ? 0x10000u : 1u);
+          }
+        });
+        __syncthreads();
+        for (int d = tid; d < kTkBins; d += kTkThreads) {
+          uint32_t sum = 0;
+  #pragma unroll
+          for (int w = 0; w < kTkWaves; ++w) sum += (hist[w][d >> 1] >> ((d & 1) * 16)) & 0xFFFFu;
+          tot[d] = sum;
+        }
+        __syncthreads();
+        tk_locate(tot, wave_part, found, need);
+        const uint32_t digit = found[0], above = found[1], inside = found[2];
+        prefix = (prefix_bits == 0 ? 0u : prefix << db) | digit;
+        prefix_bits += db;
+        need -= above;  // how many of the prefix-sharing keys are still wanted: at least one
+        if (inside <= uint32_t(kTkCap) || prefix_bits >= 32) break;
+      }
+      if (tid == 0) counters[0] = counters[1] = 0u;
+      __syncthreads();  // also: every thread is done with the histogram, whose memory now holds the list
+      tk_for_each<T, VEC, true>(x, vocab, [&](uint32_t idx, float v) {
         const uint32_t key = tk_key(v);
-        if (prefix_bits == 0 || (key >> (32 - prefix_bits)) == prefix) {
-          const uint32_t digit = (key << prefix_bits) >> (32 - db);
-          atomicAdd(&hist[wave][digit >> 1], (digit & 1u) ? 0x10000u : 1u);
+        const uint32_t top = prefix_bits >= 32 ? key : key >> (32 - prefix_bits);
+        bool take = top > prefix;
+        if (top == prefix) take = atomicAdd(&counters[1], 1u) < uint32_t(kTkCap);
+        if (take) {
+          const uint32_t slot = atomicAdd(&counters[0], 1u);
+          if (slot < uint32_t(kTkList)) list[slot] = (uint64_t(key) << 32) | uint64_t(0xFFFFFFFFu - idx);
         }
       });
       __syncthreads();
-      for (int d = tid; d < kTkBins; d += kTkThreads) {
-        uint32_t sum = 0;
-#pragma unroll
-        for (int w = 0; w < kTkWaves; ++w) sum += (hist[w][d >> 1] >> ((d & 1) * 16)) & 0xFFFFu;
-        tot[d] = sum;
-      }
-      __syncthreads();
-      tk_locate(tot, wave_part, found, need);
-      const uint32_t digit = found[0], above = found[1], inside = found[2];
-      prefix = (prefix_bits == 0 ? 0u : prefix << db) | digit;
-      prefix_bits += db;
-      need -= above;  // how many of the prefix-sharing keys are still wanted: at least one
-      if (inside <= uint32_t(kTkCap) || prefix_bits >= 32) break;
+      tk_sort_emit(list, counters[0], kTkList, k, tok, out_values, out_indices);
+      __syncthreads();  // the list is read to the end before the next row's histogram overwrites it
     }
-    if (tid == 0) counters[0] = counters[1] = 0u;
-    __syncthreads();  // also: every thread is done with the histogram, whose memory now holds the list
-    tk_for_each<T, VEC, true>(x, vocab, [&](uint32_t idx, float v) {
-      const uint32_t key = tk_key(v);
-      const uint32_t top = prefix_bits >= 32 ? key : key >> (32 - prefix_bits);
-      bool take = top > prefix;
-      if (top == prefix) take = atomicAdd(&counters[1], 1u) < uint32_t(kTkCap);
-      if (take) {
-        const uint32_t slot = atomicAdd(&counters[0], 1u);
-        if (slot < uint32_t(kTkList)) list[slot] = (uint64_t(key) << 32) | uint64_t(0xFFFFFFFFu - idx);
-      }
-    });
-    __syncthreads();
-    tk_sort_emit(list, counters[0], kTkList, k, tok, out_values, out_indices);
-    __syncthreads();  // the list is read to the end before the next row's histogram overwrites it
   }
 }
 
