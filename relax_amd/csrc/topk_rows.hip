@@ -5,9 +5,9 @@
 //
 // One 1024-thread workgroup per row, working on order-preserving 32-bit keys of the fp32 values.  Usually a shortcut
 // suffices: the k-th largest of the 1024 per-thread maxima is a lower bound of the row's k-th largest value, the few
-// hundred elements at or above (the 12-bit bin of) that bound are collected in a second pass over the row (served by
-// the caches in good part) and sorted in LDS.  Rows where that leaves too many candidates (long runs of equal or
-// nearly equal values) take the general way, a radix select:
+// hundred elements at or above (the 12-bit bin of) that bound are collected in a second look that skips every group
+// of eight vectors whose maximum, noted during the first look, lies below the bound, and are ranked in LDS.  Rows where
+// that leaves too many candidates (long runs of equal or nearly equal values) take the general way, a radix select:
 //   1. histogram of the keys' leading 12 bits (wave-private 16-bit counters in LDS, so that a wave's atomics only
 //      meet that wave's own conflicts), totals per bin, a workgroup-wide suffix scan from the top bin down: the bin
 //      that holds the K-th largest key, how many keys lie above it and how many inside;
@@ -15,7 +15,8 @@
 //      values), the same again on the next 12 bits of the keys that share the prefix found so far;
 //   3. one more pass over the row collects (key, index) of everything above the final prefix plus the keys that share
 //      it (at most kTkCap of them; with every bit consumed they are exact ties and any of them will do);
-//   4. a bitonic sort of that short list in LDS (key descending, then index ascending); the first K entries leave.
+//   4. that short list is ordered in LDS (key descending, then index ascending: by counting ranks up to 512 entries,
+//      by a bitonic sort beyond); the first K entries leave.
 // NaN orders above +inf (as torch.topk does); -0 orders below +0; which of several equal
 // values at the threshold is taken is unspecified in torch as well -- here the list order decides.
 #include "device_utils.h"
@@ -28,6 +29,7 @@ constexpr int kTkDigitBits = 12, kTkBins = 1 << kTkDigitBits;
 constexpr int kTkCap = 4096;   // keys sharing the final prefix that are kept for the sort
 constexpr int kTkMaxK = 512;
 constexpr int kTkList = 8192;  // >= kTkMaxK + kTkCap entries, a power of two
+constexpr int kTkRankMax = 512;  // lists up to this length are ranked by counting instead of sorted
 static_assert(kTkList >= kTkMaxK + kTkCap && (kTkList & (kTkList - 1)) == 0, "list capacity");
 static_assert(kTkList * 8 <= kTkWaves * kTkBins * 2, "the list reuses the histogram's memory");
 static_assert(kTkBins == 4 * kTkThreads, "the suffix scan gives every thread four bins");
@@ -109,11 +111,36 @@ __device__ __forceinline__ void tk_locate(const uint32_t* tot, uint32_t* wave_pa
 // list[0 .. len) holds (key << 32 | ~index) of every element of the top k and not many more (complete and visible):
 // bitonic sort, key descending then index ascending, and the first k entries leave.  `capacity` is a power of two.
 __device__ __forceinline__ void tk_sort_emit(uint64_t* list, uint32_t len, uint32_t capacity, int k, int64_t tok,
-                                             float* __restrict__ out_values, int64_t* __restrict__ out_indices) {
+                                             float* __restrict__ out_values, int64_t* __restrict__ out_indices,
+                                             uint32_t* rank) {
   const uint32_t tid = threadIdx.x;
   if (len > capacity) len = capacity;
   uint32_t padded = 2;
   while (padded < len) padded <<= 1;
+  if (padded <= uint32_t(kTkRankMax)) {
+    // a short list (the usual case) is ranked instead of sorted: an entry's place is the number of entries above it
+    // (entries are distinct: the index is part of them).  The 1024 threads split the len^2 comparisons, `padded`
+    // entries by 1024 / padded stretches of the list; three barriers instead of dozens.
+    const uint32_t stretches = kTkThreads / padded, mine = tid % padded, part = tid / padded;
+    if (tid < uint32_t(kTkRankMax)) rank[tid] = 0u;
+    __syncthreads();
+    if (mine < len) {
+      const uint64_t me = list[mine];
+      const uint32_t per = (len + stretches - 1) / stretches;
+      const uint32_t begin = part * per, end = begin + per < len ? begin + per : len;
+      uint32_t above = 0;
+      for (uint32_t i = begin; i < end; ++i) above += list[i] > me ? 1u : 0u;
+      if (above) atomicAdd(&rank[mine], above);
+    }
+    __syncthreads();
+    if (tid < len && rank[tid] < uint32_t(k)) {
+      const uint64_t entry = list[tid];
+      const uint32_t at = rank[tid];
+      out_indices[tok * k + at] = int64_t(0xFFFFFFFFu - uint32_t(entry));
+      if (out_values) out_values[tok * k + at] = tk_value(uint32_t(entry >> 32));
+    }
+    return;
+  }
   for (uint32_t i = len + tid; i < padded; i += kTkThreads) list[i] = 0ull;  // below every real entry
   __syncthreads();
   for (uint32_t span = 2; span <= padded; span <<= 1)
@@ -154,6 +181,7 @@ __global__ __launch_bounds__(kTkThreads, 8) void topk_rows_fast_kernel(const T* 
   __shared__ uint64_t list[kTkFastList];
   __shared__ uint32_t tot[kTkBins];
   __shared__ uint32_t group_best[kTkGroups];  // largest key of every group of eight consecutive 16-byte vectors
+  __shared__ uint32_t rank[kTkRankMax];
   __shared__ uint32_t wave_part[kTkWaves];
   __shared__ uint32_t found[3];
   __shared__ uint32_t count;
@@ -171,31 +199,38 @@ __global__ __launch_bounds__(kTkThreads, 8) void topk_rows_fast_kernel(const T* 
   uint32_t best = 0u;  // below the key of every value
   if (by_group) {
     const u32x4* xv = reinterpret_cast<const u32x4*>(x);
+    // A ring of kTkFastBatch vectors in flight: each slot is refilled as soon as its vector has been looked at.
+    // Loads past the row's end are clamped to its last vector instead of being skipped (their result is ignored):
+    // without a branch around the loads the compiler can count how many may stay in flight at each use.
+    const int64_t last = nvec - 1;
+    u32x4 raw[kTkFastBatch];
+#pragma unroll
+    for (int u = 0; u < kTkFastBatch; ++u) {
+      const int64_t i = int64_t(tid) + int64_t(u) * kTkThreads;
+      raw[u] = xv[i < last ? i : last];
+    }
     for (int64_t i0 = tid; i0 - tid < nvec; i0 += int64_t(kTkFastBatch) * kTkThreads) {  // whole waves stay together
-      u32x4 raw[kTkFastBatch];
+      // the ring's loads are awaited here, once per turn (vmcnt(0)): inside the turn every slot is then known to be
+      // complete, and the refills issued during it have the rest of the turn to land
+      __builtin_amdgcn_s_waitcnt(0x0F70);
 #pragma unroll
       for (int u = 0; u < kTkFastBatch; ++u) {
         const int64_t i = i0 + int64_t(u) * kTkThreads;
-        if (i < nvec) raw[u] = xv[i];
-      }
+        // the largest of the vector's values by a float maximum (which passes over NaN) and a NaN flag: one key
+        // conversion per vector instead of one per element
+        float v[VN];
+        Row<T>::unpack(raw[u], v);
+        const int64_t ahead = i + int64_t(kTkFastBatch) * kTkThreads;
+        raw[u] = xv[ahead < last ? ahead : last];
+        float vmax = v[0];
+        bool nan = v[0] != v[0];
 #pragma unroll
-      for (int u = 0; u < kTkFastBatch; ++u) {
-        const int64_t i = i0 + int64_t(u) * kTkThreads;
-        uint32_t top = 0u;
-        if (i < nvec) {
-          // the largest of the vector's values by a float maximum (which passes over NaN) and a NaN flag: one
-          // key conversion per vector instead of one per element
-          float v[VN];
-          Row<T>::unpack(raw[u], v);
-          float vmax = v[0];
-          bool nan = v[0] != v[0];
-#pragma unroll
-          for (int e = 1; e < VN; ++e) {
-            vmax = fmaxf(vmax, v[e]);
-            nan |= v[e] != v[e];
-          }
-          top = nan ? 0xFFFFFFFFu : tk_key(vmax);
+        for (int e = 1; e < VN; ++e) {
+          vmax = fmaxf(vmax, v[e]);
+          nan |= v[e] != v[e];
         }
+        uint32_t top = nan ? 0xFFFFFFFFu : tk_key(vmax);
+        top = i < nvec ? top : 0u;
         best = top > best ? top : best;
 #pragma unroll
         for (int o = 1; o < 8; o <<= 1) {
@@ -261,7 +296,7 @@ __global__ __launch_bounds__(kTkThreads, 8) void topk_rows_fast_kernel(const T* 
   const uint32_t len = count;
   if (tid == 0) needs_general[tok] = len > uint32_t(kTkFastList) ? 1 : 0;
   if (len > uint32_t(kTkFastList)) return;  // the whole workgroup
-  tk_sort_emit(list, len, kTkFastList, k, tok, out_values, out_indices);
+  tk_sort_emit(list, len, kTkFastList, k, tok, out_values, out_indices, rank);
 }
 
 // The general way, for the rows the shortcut flagged (long runs of equal or nearly equal values): radix select, 12
@@ -277,6 +312,7 @@ __global__ __launch_bounds__(kTkThreads) void topk_rows_kernel(const T* __restri
   __shared__ uint32_t wave_part[kTkWaves];
   __shared__ uint32_t found[3];
   __shared__ uint32_t counters[2];  // list length, prefix-sharing keys seen
+  __shared__ uint32_t rank[kTkRankMax];
   uint32_t* const hist_words = &hist[0][0];
   uint64_t* const list = reinterpret_cast<uint64_t*>(hist_words);
   const int tid = threadIdx.x, wave = tid / kWave;
@@ -335,7 +371,7 @@ __global__ __launch_bounds__(kTkThreads) void topk_rows_kernel(const T* __restri
         }
       });
       __syncthreads();
-      tk_sort_emit(list, counters[0], kTkList, k, tok, out_values, out_indices);
+      tk_sort_emit(list, counters[0], kTkList, k, tok, out_values, out_indices, rank);
       __syncthreads();  // the list is read to the end before the next row's histogram overwrites it
     }
   }
