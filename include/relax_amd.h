@@ -326,6 +326,17 @@ int relax_amd_opd_kl_topk_bwd(const float* student_lp, const float* teacher_lp, 
                               float log_prob_min_clamp, const float* g, float* d_student_lp, void* stream);
 
 /*
+ * dlogits[row_ids[t], ids[t, j]] += values[t, j] * scale for j < k, and dlogits[row_ids[t], targets[t]] +=
+ * target_values[t] * scale: the sparse part of the gradient of gathered log-probs (the scatter of
+ * compute_log_probs_on_topk_token_ids' backward, relax/utils/opd/opd_utils.py:1022-1094) when its dense part, a
+ * multiple of the row's softmax, has been folded into the dlogits launch of the log-prob backward.  Ids outside
+ * [0, vocab) and zero values are skipped; targets / target_values may be NULL; row_ids NULL = row t.
+ */
+int relax_amd_sparse_row_add(void* dlogits, int dtype, int64_t n_tokens, int64_t vocab, int64_t row_stride,
+                             const int32_t* row_ids, const int64_t* ids, const float* values, int64_t k,
+                             const int64_t* targets, const float* target_values, float scale, void* stream);
+
+/*
  * The k largest logits of each token's row and their vocabulary ids, largest first: torch.topk(logits_chunk, k=k,
  * dim=-1) of get_log_probs_and_entropy (relax/backends/megatron/loss.py:434-436), for every response row in one
  * launch.  NaN orders above +inf as in torch.topk; which of several equal values at the k-th place is returned is

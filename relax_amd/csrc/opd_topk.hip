@@ -251,9 +251,67 @@ __global__ __launch_bounds__(256) void opd_kl_topk_kernel(const float* __restric
   }
 }
 
+// dlogits[row(t), id] += value * scale for the K (id, value) pairs of token t plus one pair at its target id: the
+// sparse part of a gradient whose dense part (a multiple of the row's softmax) another kernel has already written.
+// One thread walks all pairs of a token one after the other, so two pairs on the same element (a gathered id that
+// equals the target) cannot race; ids outside [0, vocab) are skipped.
+template <typename T>
+__global__ __launch_bounds__(256) void sparse_row_add_kernel(T* __restrict__ dlogits, int64_t stride, int64_t vocab,
+                                                             const int32_t* __restrict__ row_ids,
+                                                             const int64_t* __restrict__ ids,
+                                                             const float* __restrict__ values, int k,
+                                                             const int64_t* __restrict__ targets,
+                                                             const float* __restrict__ target_values, float scale,
+                                                             int64_t n_tokens) {
+  const int64_t tok = blockIdx.x * 256LL + threadIdx.x;
+  if (tok >= n_tokens) return;
+  T* d = dlogits + (row_ids ? int64_t(row_ids[tok]) : tok) * stride;
+  for (int j = 0; j < k; ++j) {
+    const int64_t id = ids[tok * k + j];
+    const float v = values[tok * k + j];
+    if (id >= 0 && id < vocab && v != 0.f) Row<T>::store1(d + id, Row<T>::load1(d + id) + v * scale);
+  }
+  if (targets) {
+    const int64_t id = targets[tok];
+    const float v = target_values[tok];
+    if (id >= 0 && id < vocab && v != 0.f) Row<T>::store1(d + id, Row<T>::load1(d + id) + v * scale);
+  }
+}
+
 }  // namespace relax_amd
 
 using namespace relax_amd;
+
+extern "C" int relax_amd_sparse_row_add(void* dlogits, int dtype, int64_t n_tokens, int64_t vocab, int64_t row_stride,
+                                        const int32_t* row_ids, const int64_t* ids, const float* values, int64_t k,
+                                        const int64_t* targets, const float* target_values, float scale,
+                                        void* stream) {
+  if (n_tokens == 0) return RELAX_AMD_OK;
+  if (n_tokens < 0 || vocab <= 0 || row_stride < vocab || k < 0 || k > (1 << 20) || !dlogits ||
+      (k > 0 && (!ids || !values)) || (targets && !target_values)) {
+    set_error("sparse_row_add: NULL argument or bad shape n=%lld vocab=%lld row_stride=%lld k=%lld",
+              (long long)n_tokens, (long long)vocab, (long long)row_stride, (long long)k);
+    return RELAX_AMD_EINVAL;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>((n_tokens + 255) / 256)), block(256);
+  switch (dtype) {
+    case RELAX_AMD_F32:
+      hipLaunchKernelGGL(sparse_row_add_kernel<float>, grid, block, 0, s, static_cast<float*>(dlogits), row_stride,
+                         vocab, row_ids, ids, values, int(k), targets, target_values, scale, n_tokens);
+      break;
+    case RELAX_AMD_BF16:
+      hipLaunchKernelGGL(sparse_row_add_kernel<bf16_t>, grid, block, 0, s, static_cast<bf16_t*>(dlogits), row_stride,
+                         vocab, row_ids, ids, values, int(k), targets, target_values, scale, n_tokens);
+      break;
+    case RELAX_AMD_F16:
+      hipLaunchKernelGGL(sparse_row_add_kernel<f16_t>, grid, block, 0, s, static_cast<f16_t*>(dlogits), row_stride,
+                         vocab, row_ids, ids, values, int(k), targets, target_values, scale, n_tokens);
+      break;
+    default: set_error("sparse_row_add: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
+  }
+  return check_launch("sparse_row_add");
+}
 
 static int topk_check(const char* what, int64_t n, int64_t vocab, int64_t stride, int64_t k) {
   if (n < 0 || n > 2147483647LL || vocab <= 0 || stride < vocab || k < 0 || k > (1 << 20)) {

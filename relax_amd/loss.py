@@ -311,12 +311,9 @@ def sft_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum_of
     return loss, {"loss": loss.clone().detach()}
 
 
-def _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t):
-    """Per-sample ``[R_i, K_i]`` log-probs at the given vocabulary ids (compute_opd_topk_log_probs,
-    relax/utils/opd/opd_utils.py:1005-1019) in one packed launch: samples with fewer ids (the union path) are padded
-    with the -1 sentinel, which yields -inf and no gradient, and trimmed again afterwards."""
-    from .opd_utils import TopKLogProbs
-
+def _pack_topk_ids(flat, lay, gather_topk_token_ids):
+    """Per-sample ``[R_i, K_i]`` id tensors -> (one ``[N, K_max]`` int64 tensor padded with the -1 sentinel, the
+    per-sample widths); ``(None, widths)`` when there is nothing to gather."""
     dev = flat.device
     per_sample, widths = [], []
     for i, r in enumerate(lay.response_lengths):
@@ -331,16 +328,33 @@ def _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t):
         widths.append(int(ids.size(1)))
     k_max = max(widths) if widths else 0
     if k_max == 0 or lay.n_tokens == 0:
-        return [flat.new_zeros((r, 0)) for r in lay.response_lengths]
+        return None, widths
     packed = torch.full((lay.n_tokens, k_max), -1, dtype=torch.long, device=dev)
     pos = 0
     for ids, r, w in zip(per_sample, lay.response_lengths, widths):
         if w:
             packed[pos:pos + r, :w] = ids
         pos += r
-    out = TopKLogProbs.apply(flat, packed, inv_t, None, lay.row_ids, lay.token_of_row)
+    return packed, widths
+
+
+def _trim_topk(out, flat, lay, widths):
+    """``[N, K_max]`` gathered log-probs -> per-sample ``[R_i, K_i]`` views."""
+    if out is None:
+        return [flat.new_zeros((r, 0)) for r in lay.response_lengths]
     pieces = torch.split(out, lay.response_lengths)
     return [p[:, :w] if w else flat.new_zeros((r, 0)) for p, r, w in zip(pieces, lay.response_lengths, widths)]
+
+
+def _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t):
+    """Per-sample ``[R_i, K_i]`` log-probs at the given vocabulary ids (compute_opd_topk_log_probs,
+    relax/utils/opd/opd_utils.py:1005-1019) in one packed launch: samples with fewer ids (the union path) are padded
+    with the -1 sentinel, which yields -inf and no gradient, and trimmed again afterwards."""
+    from .opd_utils import TopKLogProbs
+
+    packed, widths = _pack_topk_ids(flat, lay, gather_topk_token_ids)
+    out = None if packed is None else TopKLogProbs.apply(flat, packed, inv_t, None, lay.row_ids, lay.token_of_row)
+    return _trim_topk(out, flat, lay, widths)
 
 
 # ------------------------------------------------------------------------------------------ fused policy loss
@@ -353,6 +367,9 @@ class _FusedPolicyLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, flat, lay, inv_t, kw):
         lp, ent, lse, spx = ops.logprob_entropy_fwd(flat, lay.targets, lay.row_ids, inv_t, True)
+        lp_visible = bool(kw.get("lp_requires_grad", False))
+        gather_ids = kw.get("gather_topk_ids")
+        kw = {k: v for k, v in kw.items() if k not in ("lp_requires_grad", "gather_topk_ids")}
         m2po = kw.get("m2po")
         if m2po is not None:
             # M2PO (loss.py:990-993): the clip margins are solved from this micro-batch's log-ratios, which exist only
@@ -369,18 +386,51 @@ class _FusedPolicyLoss(torch.autograd.Function):
         out = ops.policy_loss(log_prob=lp, entropy=ent, cu_resp=lay.cu_resp, **kw)
         metrics = out["metrics"]
         entropy_grad = kw.get("entropy_coef", 0.0) != 0
+        if gather_ids is not None:
+            # log-probs at the given vocabulary ids (the top-K distillation term): K loads per row next to the
+            # log-sum-exp just computed; their gradient comes back to this function's one dlogits launch
+            topk_lp = torch.empty(gather_ids.shape, dtype=torch.float32, device=flat.device)
+            stride = flat.stride(0) if flat.size(0) > 1 else flat.size(1)
+            ops.check(ops.lib.relax_amd_topk_logprob_fwd(
+                ops._p(flat), ops._code(flat), gather_ids.size(0), flat.size(1), stride, ops._p(lay.row_ids),
+                ops._p(gather_ids), gather_ids.size(1), float(inv_t), ops._p(lse), ops._p(topk_lp), None,
+                ops._stream()))
+        else:
+            topk_lp = lp.new_zeros(0)
         ctx.save_for_backward(flat, lay.targets, lse, spx if entropy_grad else None, out["coef_log_prob"],
-                              out["coef_entropy"] if entropy_grad else None, lay.token_of_row)
+                              out["coef_entropy"] if entropy_grad else None, lay.token_of_row, gather_ids,
+                              lay.row_ids if gather_ids is not None else None)
         ctx.inv_t = inv_t
-        ctx.mark_non_differentiable(metrics, lp, ent)
-        return metrics[_SLOT["loss"]].clone(), metrics, lp, ent
+        # ``lp_requires_grad``: further loss terms built on the returned log-probs (the distillation term) send their
+        # gradient back here, where it joins the policy loss's coefficient before the one dlogits launch
+        hidden = [metrics, ent] + ([] if lp_visible else [lp]) + ([] if gather_ids is not None else [topk_lp])
+        ctx.mark_non_differentiable(*hidden)
+        return metrics[_SLOT["loss"]].clone(), metrics, lp, ent, topk_lp
 
     @staticmethod
-    def backward(ctx, g_loss, _gm, _glp, _gent):
-        flat, targets, lse, spx, c_lp, c_ent, token_of_row = ctx.saved_tensors
+    def backward(ctx, g_loss, _gm, g_lp, _gent, g_topk):
+        flat, targets, lse, spx, c_lp, c_ent, token_of_row, gather_ids, row_ids = ctx.saved_tensors
         scale = g_loss.reshape(1).to(torch.float32).contiguous()
+        sparse = None
+        if gather_ids is None:
+            g_topk = None
+        if g_lp is not None or g_topk is not None:
+            c_lp = c_lp * scale
+            c_ent = None if c_ent is None else c_ent * scale
+            scale = None
+            if g_lp is not None:
+                c_lp = c_lp + g_lp.reshape(-1).to(torch.float32)
+            if g_topk is not None:
+                # d log p[id_k] / d logits = onehot(id_k) - p: the -p parts of all K join the log-prob coefficient
+                # (whose own onehot, at the target, is taken back below); the onehots are K sparse additions
+                g_k = torch.where(gather_ids >= 0, g_topk.to(torch.float32), torch.zeros((), device=flat.device))
+                total = g_k.sum(dim=-1)
+                c_lp = c_lp + total
+                sparse = (g_k, -total)
         d = ops.logprob_entropy_bwd(flat, targets, lse, spx, c_lp, c_ent, token_of_row=token_of_row,
                                     grad_scale_dev=scale, inv_temperature=ctx.inv_t)
+        if sparse is not None:
+            ops.sparse_row_add(d, row_ids, gather_ids, sparse[0], targets, sparse[1], scale=ctx.inv_t)
         return d, None, None, None
 
 
@@ -703,27 +753,51 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
             metrics.update(_m2po_reported((0.0, 0.0, max(1.0, kw["m2po"]["miniclip_low"]),
                                            max(99999.0, kw["m2po"]["miniclip_high"])), dev))
         return loss, metrics
-    fn = _SinglePassPolicyLoss if _single_pass_ok(args, flat, kw, needs_bwd) else _FusedPolicyLoss
-    loss, mvec, lp, ent = fn.apply(flat, lay, inv_t, kw)
+    opd_on = float(getattr(args, "opd_loss_coef", 0.0) or 0.0) != 0.0
+    opd_gather = None
+    if opd_on:
+        from .opd_utils import compute_policy_opd_loss, resolve_opd_gather_topk_token_ids
+
+        opd_gather = resolve_opd_gather_topk_token_ids(args, batch)
+    # a sampled-token distillation term needs nothing but this step's log-probs: it is built on the two-launch
+    # function's output, and its gradient joins the policy loss's before the single dlogits launch
+    # the same holds for the top-K selections: the log-probs at the given ids are K loads per row next to the row's
+    # log-sum-exp, and their gradient is a multiple of the softmax plus K sparse additions
+    opd_on_lp = opd_on and needs_bwd
+    topk_widths = None
+    if opd_on_lp:
+        kw["lp_requires_grad"] = True
+        if opd_gather is not None:
+            kw["gather_topk_ids"], topk_widths = _pack_topk_ids(flat, lay, opd_gather)
+    if not opd_on_lp and _single_pass_ok(args, flat, kw, needs_bwd):
+        loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw)
+        topk_lp = None
+    else:
+        loss, mvec, lp, ent, topk_lp = _FusedPolicyLoss.apply(flat, lay, inv_t, kw)
 
     def m(name):
         return mvec[_SLOT[name]]
 
     opd_reported = {}
     loss_metric = m("loss")
-    if float(getattr(args, "opd_loss_coef", 0.0) or 0.0) != 0.0:
-        # The distillation term (loss.py:1102-1110) needs log-probs that autograd can see, which the fused step keeps
-        # to itself: a second, differentiable log-prob launch (plus the top-K gather) feeds it.
-        from .opd_utils import compute_policy_opd_loss, resolve_opd_gather_topk_token_ids
-
-        _, lpe = get_log_probs_and_entropy(
-            logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=total_lengths,
-            response_lengths=response_lengths, with_entropy=False, max_seq_lens=batch.get("max_seq_lens"),
-            gather_topk_token_ids=resolve_opd_gather_topk_token_ids(args, batch))
+    if opd_on:
+        # The distillation term (loss.py:1102-1110) needs log-probs that autograd can see: the two-launch function's
+        # own outputs when a gradient is wanted, a separate log-prob launch (with the top-K gather) otherwise.
+        if opd_on_lp:
+            lpe = {"log_probs": lay.split(lp)}
+            if opd_gather is not None:
+                lpe["topk_log_probs"] = _trim_topk(topk_lp if kw.get("gather_topk_ids") is not None else None, flat,
+                                                   lay, topk_widths)
+            opd_lp = lp
+        else:
+            _, lpe = get_log_probs_and_entropy(
+                logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=total_lengths,
+                response_lengths=response_lengths, with_entropy=False, max_seq_lens=batch.get("max_seq_lens"),
+                gather_topk_token_ids=opd_gather)
+            opd_lp = torch.cat(lpe["log_probs"])
         old_for_opd = old if old is not None else lp.detach()
         opd_loss, opd_reported = compute_policy_opd_loss(
-            args=args, batch=batch, log_probs=torch.cat(lpe["log_probs"]), old_log_probs=old_for_opd,
-            log_probs_and_entropy=lpe)
+            args=args, batch=batch, log_probs=opd_lp, old_log_probs=old_for_opd, log_probs_and_entropy=lpe)
         if opd_loss is not None:
             loss = loss + opd_loss
             loss_metric = loss.detach().clone()

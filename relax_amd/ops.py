@@ -337,6 +337,19 @@ def actor_step_fused(logits, targets, token_of_row, sample_ids, n_tokens: int, i
     return out, lp, ent, lse, spx, dlogits
 
 
+def sparse_row_add(dlogits, row_ids, ids, values, targets=None, target_values=None, scale: float = 1.0):
+    """``dlogits[row_ids[t], ids[t, j]] += values[t, j] * scale`` (and the same at ``targets[t]`` with
+    ``target_values[t]``), in place; ids outside the vocabulary are skipped."""
+    _need_gpu(dlogits, ids)
+    d = dlogits.reshape(-1, dlogits.size(-1))
+    n, k = ids.shape
+    stride = d.stride(0) if d.size(0) > 1 else d.size(1)
+    check(lib.relax_amd_sparse_row_add(_p(d), _code(d), n, d.size(1), stride, _p(row_ids), _p(ids.contiguous()),
+                                       _p(_f32(values)), k, _p(targets), _p(_f32(target_values)), float(scale),
+                                       _stream()))
+    return dlogits
+
+
 TOPK_ROWS_MAX_K = 512
 TOPK_ROWS_MAX_VOCAB = 1000000
 

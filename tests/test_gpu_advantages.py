@@ -389,6 +389,39 @@ def test_opd_kl_two_dimensional_reverse_kl_is_the_elementwise_log_ratio():
         compute_opd_kl(s, t, "forward_kl")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_sparse_row_add_patches_rows_in_place(dtype):
+    """The sparse half of the gathered log-probs' gradient: K (id, value) pairs per token plus one at the target are
+    added to the token's logits row in place; an id equal to the target gets both additions, ids outside the vocabulary
+    (sentinels, ids of another shard) and zero values are skipped, other rows and elements are untouched."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("sparse row add", dtype)
+    g = torch.Generator().manual_seed(5)
+    rows, v, n, k = 9, 50, 6, 4
+    d0 = torch.randn(rows, v, generator=g).to(dtype)
+    row_ids = torch.tensor([7, 0, 3, 4, 8, 1], dtype=torch.int32)
+    ids = torch.randint(0, v, (n, k), generator=g)
+    ids[0, 1], ids[2, 0], ids[3, 3] = -1, v + 5, -1
+    targets = torch.randint(0, v, (n,), generator=g)
+    ids[4, 2] = targets[4]  # a gathered id that equals the target
+    vals = torch.randn(n, k, generator=g)
+    vals[5, 0] = 0.0
+    tvals = torch.randn(n, generator=g)
+    want = d0.float().clone()
+    for t in range(n):
+        for j in range(k):
+            if 0 <= ids[t, j] < v:
+                r, c = row_ids[t], ids[t, j]
+                want[r, c] = (want[r, c] + vals[t, j] * 0.5).to(dtype).float()
+        r, c = row_ids[t], targets[t]
+        want[r, c] = (want[r, c] + tvals[t] * 0.5).to(dtype).float()
+    d = d0.to(dev)
+    ops.sparse_row_add(d, row_ids.to(dev), ids.to(dev), vals.to(dev), targets.to(dev), tvals.to(dev), scale=0.5)
+    assert torch.equal(d.float().cpu(), want)
+
+
 def test_opd_kl_topk_argument_checks():
     from relax_amd.opd_utils import compute_opd_kl, compute_opd_kl_topk
 
