@@ -162,9 +162,14 @@ def get_log_probs_and_entropy(
     lay = PackedLayout(flat.device, flat.size(0), unconcat_tokens, total_lengths, response_lengths, needs_bwd,
                        _padded_starts(args, max_seq_lens))
     inv_t = 1.0 / float(getattr(args, "rollout_temperature", 1.0))
+    lse = None
     if lay.n_tokens == 0:
         lp = flat.new_zeros((0,), dtype=torch.float32)
         ent = lp
+    elif not needs_bwd:
+        # forward-only (the ActorFwd / Reference passes): the launch's log-sum-exps stay at hand, so that a top-K gather
+        # below costs K loads per row instead of another scan of the logits
+        lp, ent, lse, _ = ops.logprob_entropy_fwd(ops._rows(flat), lay.targets, lay.row_ids, inv_t, bool(with_entropy))
     else:
         lp, ent = ops.LogProbEntropy.apply(
             flat, lay.targets, lay.row_ids, lay.token_of_row, inv_t, bool(with_entropy), bool(want_grad)
@@ -185,7 +190,7 @@ def get_log_probs_and_entropy(
             res["topk_token_ids"] = [torch.topk(flat[b:b + r], k=k, dim=-1).indices
                                      for b, r in zip(begins, lay.response_lengths)]
     if gather_topk_token_ids is not None:
-        res["topk_log_probs"] = _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t)
+        res["topk_log_probs"] = _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t, lse)
     return torch.empty((0,), device=logits.device), res
 
 
@@ -346,14 +351,15 @@ def _trim_topk(out, flat, lay, widths):
     return [p[:, :w] if w else flat.new_zeros((r, 0)) for p, r, w in zip(pieces, lay.response_lengths, widths)]
 
 
-def _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t):
+def _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t, lse=None):
     """Per-sample ``[R_i, K_i]`` log-probs at the given vocabulary ids (compute_opd_topk_log_probs,
     relax/utils/opd/opd_utils.py:1005-1019) in one packed launch: samples with fewer ids (the union path) are padded
-    with the -1 sentinel, which yields -inf and no gradient, and trimmed again afterwards."""
+    with the -1 sentinel, which yields -inf and no gradient, and trimmed again afterwards.  ``lse`` (the rows'
+    log-sum-exps from a log-prob launch over the same rows) spares the gather its own scan of the logits."""
     from .opd_utils import TopKLogProbs
 
     packed, widths = _pack_topk_ids(flat, lay, gather_topk_token_ids)
-    out = None if packed is None else TopKLogProbs.apply(flat, packed, inv_t, None, lay.row_ids, lay.token_of_row)
+    out = None if packed is None else TopKLogProbs.apply(flat, packed, inv_t, lse, lay.row_ids, lay.token_of_row)
     return _trim_topk(out, flat, lay, widths)
 
 

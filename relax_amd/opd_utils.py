@@ -34,7 +34,7 @@ class TopKLogProbs(torch.autograd.Function):
     def forward(ctx, logits, ids, inv_temperature, lse, row_ids=None, token_of_row=None):
         x = _rows(logits)
         n, k = ids.shape
-        if row_ids is not None and token_of_row is None and logits.requires_grad:
+        if row_ids is not None and token_of_row is None and ctx.needs_input_grad[0]:
             raise RuntimeError("row_ids without token_of_row cannot be differentiated")
         out = torch.empty((n, k), dtype=torch.float32, device=x.device)
         lse_out = lse if lse is not None else torch.empty(n, dtype=torch.float32, device=x.device)

@@ -1083,3 +1083,28 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, monkey
         assert torch.equal(got, want), (pattern, key, (got.float() - want.float()).abs().max())
     if pattern == "all_dead":
         assert not results["resident"]["d"].any()
+
+
+def test_forward_only_topk_gather_on_logits_that_require_grad():
+    """The ActorFwd pass runs under ``torch.no_grad()`` on logits that may still carry ``requires_grad``: the top-K
+    gather then reuses the log-prob launch's log-sum-exps and returns the same values as the differentiable path."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("forward-only top-K gather")
+    tot, resp, v, k = [9, 6, 12], [4, 3, 7], 3000, 6
+    g = torch.Generator().manual_seed(21)
+    logits = (torch.randn(1, sum(tot), v, generator=g) * 2).to(dev).requires_grad_()
+    toks = [torch.randint(0, v, (n,), generator=g).to(dev) for n in tot]
+    ids = [torch.randint(0, v, (r, k), generator=g).to(dev) for r in resp]
+    args = P.make_args(rollout_temperature=0.8)
+    kw = dict(args=args, unconcat_tokens=toks, total_lengths=tot, response_lengths=resp, with_entropy=True,
+              gather_topk_token_ids=ids)
+    with torch.no_grad():
+        _, quiet = relax_amd.get_log_probs_and_entropy(logits, **kw)
+    _, loud = relax_amd.get_log_probs_and_entropy(logits, **kw)
+    for key in ("log_probs", "entropy", "topk_log_probs"):
+        for a, b in zip(quiet[key], loud[key]):
+            assert not a.requires_grad
+            torch.testing.assert_close(a, b.detach(), atol=1e-6, rtol=1e-6)
+    assert loud["topk_log_probs"][0].requires_grad
