@@ -359,7 +359,8 @@ def _gathered_topk_log_probs(flat, lay, gather_topk_token_ids, inv_t, lse=None):
     from .opd_utils import TopKLogProbs
 
     packed, widths = _pack_topk_ids(flat, lay, gather_topk_token_ids)
-    out = None if packed is None else TopKLogProbs.apply(flat, packed, inv_t, lse, lay.row_ids, lay.token_of_row)
+    out = None if packed is None else TopKLogProbs.apply(flat, packed, inv_t, lse, lay.row_ids, lay.token_of_row,
+                                                         torch.is_grad_enabled() and flat.requires_grad)
     return _trim_topk(out, flat, lay, widths)
 
 

@@ -31,10 +31,12 @@ class TopKLogProbs(torch.autograd.Function):
     dense [T, V] gradient in one streaming pass."""
 
     @staticmethod
-    def forward(ctx, logits, ids, inv_temperature, lse, row_ids=None, token_of_row=None):
+    def forward(ctx, logits, ids, inv_temperature, lse, row_ids=None, token_of_row=None, differentiable=True):
         x = _rows(logits)
         n, k = ids.shape
-        if row_ids is not None and token_of_row is None and ctx.needs_input_grad[0]:
+        # (``differentiable`` is the caller's word: inside a Function's forward the grad mode is always off, and the
+        # inputs report requires_grad under torch.no_grad() as well)
+        if row_ids is not None and token_of_row is None and differentiable:
             raise RuntimeError("row_ids without token_of_row cannot be differentiated")
         out = torch.empty((n, k), dtype=torch.float32, device=x.device)
         lse_out = lse if lse is not None else torch.empty(n, dtype=torch.float32, device=x.device)
@@ -59,7 +61,7 @@ class TopKLogProbs(torch.autograd.Function):
             check(lib.relax_amd_topk_logprob_bwd(_p(x), _code(x), x.size(0), x.size(1), stride, _p(token_of_row),
                                                  _p(ids), k, ctx.inv_temperature, _p(lse), _p(g), _p(d), d.size(1),
                                                  _stream()))
-        return d.view(ctx.shape), None, None, None, None, None
+        return d.view(ctx.shape), None, None, None, None, None, None
 
 
 def compute_log_probs_on_topk_token_ids(logits: torch.Tensor, topk_token_ids: torch.Tensor, process_group=None,
