@@ -194,7 +194,7 @@ __global__ __launch_bounds__(kTkThreads, 8) void topk_rows_fast_kernel(const T* 
   // With 16-byte loads, eight neighbouring lanes read eight neighbouring vectors (128 bytes): the first look also
   // notes each such group's largest key, and the second look skips the groups that lie below the bound -- all but a
   // few per cent of the row.
-  const bool by_group = VEC && nvec <= int64_t(8) * kTkGroups;
+  const bool by_group = VEC && nvec > 0 && nvec <= int64_t(8) * kTkGroups;
 
   uint32_t best = 0u;  // below the key of every value
   if (by_group) {

@@ -283,6 +283,17 @@ def test_topk_rows_equals_torch_topk(n, v, k, dtype):
     _check_topk_rows(x, k, row_ids)
 
 
+def test_topk_rows_on_tiny_vocabularies():
+    """Rows shorter than one 16-byte vector, with a row stride that still allows vector loads: nothing may be read
+    outside the row."""
+    dev = require_gpu()
+    announce("topk rows tiny")
+    g = torch.Generator(device=dev).manual_seed(3)
+    for v, k, dtype in ((5, 3, torch.bfloat16), (3, 3, torch.float32), (1, 1, torch.bfloat16), (9, 4, torch.float16)):
+        wide = (torch.randn((12, 16), device=dev, generator=g) * 2).to(dtype)
+        _check_topk_rows(wide[:, :v], k)  # row stride 16 elements: 16-byte aligned rows of v elements
+
+
 def test_topk_rows_on_degenerate_rows():
     """Rows that defeat the first histogram: all values equal (every key shares all 32 bits), two distinct values,
     values that differ only in their low mantissa bits (three refinement passes), infinities, NaN (ordered above
