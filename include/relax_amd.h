@@ -176,6 +176,11 @@ typedef struct relax_amd_policy_loss_args {
   float* kl_tok;
   float* sample_partials;        /* workspace [n_samples * RELAX_AMD_NUM_METRICS] */
   float* metrics;                /* [RELAX_AMD_NUM_METRICS] */
+  /* optional input, last so that the fields above keep their offsets: [n_tokens] added to d loss / d log_prob of every
+   * token whose masks are not both zero -- the gradient of a caller's loss term that is linear in the log-probs, such
+   * as opd_loss_coef * token_mean(log_prob - teacher_log_prob) (relax/utils/opd/opd_utils.py:1368-1455 with the
+   * sampled-token reverse_kl signal), so that term's gradient leaves in the same dlogits launch.  NULL = none. */
+  const float* extra_coef_log_prob;
 } relax_amd_policy_loss_args;
 
 int relax_amd_policy_loss(const relax_amd_policy_loss_args* args, void* stream);

@@ -49,6 +49,7 @@ class PolicyLossArgs(C.Structure):
         ("tis_lo", _f32), ("tis_hi", _f32), ("opsm_delta", _f32), ("tau_pos", _f32), ("tau_neg", _f32),
         ("coef_log_prob", _vp), ("coef_entropy", _vp), ("pg_loss_tok", _vp), ("clipfrac_tok", _vp),
         ("ppo_kl_tok", _vp), ("kl_tok", _vp), ("sample_partials", _vp), ("metrics", _vp),
+        ("extra_coef_log_prob", _vp),
     ]
 
 

@@ -103,6 +103,7 @@ struct TokenResult {
 // Per-token inputs of the loss, fetched ahead of time so their latency can hide behind other work.
 struct TokenInputs {
   float old_lp, ref_lp, train_lp, rollout_lp, adv, m, mp;
+  float extra_lp;  // caller-supplied addition to d loss / d log_prob (0 when there is none)
   bool has_old, has_train;
 };
 
@@ -117,6 +118,7 @@ __device__ __forceinline__ TokenInputs load_token_inputs(const relax_amd_policy_
   in.adv = a.advantages[t];
   in.m = a.loss_mask[t];
   in.mp = a.pg_loss_mask ? a.pg_loss_mask[t] : in.m;
+  in.extra_lp = a.extra_coef_log_prob ? a.extra_coef_log_prob[t] : 0.f;
   return in;
 }
 
@@ -177,6 +179,7 @@ __device__ __forceinline__ TokenResult token_terms(const relax_amd_policy_loss_a
     o.metric[RELAX_AMD_M_KL_LOSS] = kl * m;
     o.coef_lp += a.kl_coef * (m / den) * dkl;
   }
+  o.coef_lp += in.extra_lp;
   if (a.rollout_log_prob) {
     const float roll = in.rollout_lp;
     float side = lp;

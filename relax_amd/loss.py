@@ -448,12 +448,21 @@ class _SinglePassPolicyLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, flat, lay, inv_t, kw):
+        # kw["linear_lp_term"] = (weights [N], offsets [N]) adds sum_t weights[t] * (lp[t] - offsets[t]) to the loss:
+        # its gradient w.r.t. each log-prob is weights[t], known before the launch, so it leaves in the same dlogits
+        linear = kw.get("linear_lp_term")
+        kw = {k: v for k, v in kw.items() if k != "linear_lp_term"}
+        if linear is not None:
+            kw["extra_coef_log_prob"] = linear[0]
         out, lp, ent, _lse, _spx, dlogits = ops.actor_step_fused(
             flat, lay.targets, lay.token_of_row, lay.sample_ids, lay.n_tokens, inv_t, 1.0, cu_resp=lay.cu_resp, **kw)
         metrics = out["metrics"]
         ctx.dlogits = dlogits
         ctx.mark_non_differentiable(metrics, lp, ent)
-        return metrics[_SLOT["loss"]].clone(), metrics, lp, ent
+        loss = metrics[_SLOT["loss"]].clone()
+        if linear is not None:
+            loss = loss + (linear[0] * (lp - linear[1])).sum()
+        return loss, metrics, lp, ent
 
     @staticmethod
     def backward(ctx, g_loss, _gm, _glp, _gent):
@@ -463,6 +472,28 @@ class _SinglePassPolicyLoss(torch.autograd.Function):
         ctx.dlogits = None
         ops.scale_rows_inplace(d, g_loss.reshape(1).to(torch.float32).contiguous())
         return d, None, None, None
+
+
+def _linear_opd_term(args, batch, loss_mask, dev):
+    """(weights, teacher log-probs), both [N], when the distillation loss term is linear in this step's log-probs:
+    sampled-token selection with the ``reverse_kl`` signal (lp - teacher) and no clamp, per-token clip or
+    importance-ratio clip (relax/utils/opd/opd_utils.py:1368-1455).  Then the term is
+    ``sum_t weights[t] * (lp[t] - teacher[t])`` with ``weights = opd_loss_coef * mask / clamp_min(sum mask, 1)``.
+    None in every other configuration."""
+    if getattr(args, "opd_token_selection", "sampled") in ("student_topk", "teacher_topk", "union"):
+        return None
+    if getattr(args, "opd_kl_type", "reverse_kl") != "reverse_kl":
+        return None
+    if any(getattr(args, k, None) is not None for k in ("opd_log_prob_min_clamp", "opd_per_token_clip", "opd_is_clip")):
+        return None
+    teacher = batch.get("teacher_log_probs")
+    if teacher is None:
+        return None
+    teacher = torch.cat([t.reshape(-1) for t in teacher]).to(device=dev, dtype=torch.float32)
+    if teacher.numel() != loss_mask.numel():
+        return None
+    weights = loss_mask * (float(args.opd_loss_coef) / torch.clamp_min(loss_mask.sum(), 1))
+    return weights, teacher
 
 
 def _single_pass_ok(args, flat, kw, needs_bwd) -> bool:
@@ -776,7 +807,17 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         kw["lp_requires_grad"] = True
         if opd_gather is not None:
             kw["gather_topk_ids"], topk_widths = _pack_topk_ids(flat, lay, opd_gather)
-    if not opd_on_lp and _single_pass_ok(args, flat, kw, needs_bwd):
+    opd_linear = None
+    if opd_on_lp and opd_gather is None and _single_pass_ok(args, flat, kw, needs_bwd):
+        opd_linear = _linear_opd_term(args, batch, kw["loss_mask"], dev)
+    if opd_linear is not None:
+        # the sampled-token reverse-KL signal without clips is coef * token_mean(lp - teacher): linear in the
+        # log-probs, so the single launch carries its gradient and the term's value follows from the launch's lp
+        kw.pop("lp_requires_grad", None)
+        loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, dict(kw, linear_lp_term=opd_linear))
+        topk_lp = None
+        reported_loss = loss.detach().clone()
+    elif not opd_on_lp and _single_pass_ok(args, flat, kw, needs_bwd):
         loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw)
         topk_lp = None
     else:
@@ -787,7 +828,9 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
 
     opd_reported = {}
     loss_metric = m("loss")
-    if opd_on:
+    if opd_linear is not None:
+        loss_metric = reported_loss
+    elif opd_on:
         # The distillation term (loss.py:1102-1110) needs log-probs that autograd can see: the two-launch function's
         # own outputs when a gradient is wanted, a separate log-prob launch (with the top-K gather) otherwise.
         if opd_on_lp:

@@ -253,8 +253,11 @@ def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_pr
                  pg_sample_denom=None, loss_kind="ppo", kl_kind=None, unbiased_kl=False, use_opsm=False,
                  use_tis=False, mismatch_metrics=False, abs_diff_from_old=1, eps_clip=0.2, eps_clip_high=0.2,
                  eps_clip_c=None, entropy_coef=0.0, kl_coef=0.0, tis_lo=0.0, tis_hi=2.0, opsm_delta=1e-4,
-                 tau_pos=1.0, tau_neg=1.05, per_token_outputs=False, want_coef_entropy=False):
-    """Fills a ``relax_amd_policy_loss_args`` block; returns (struct, outputs dict holding every live tensor)."""
+                 tau_pos=1.0, tau_neg=1.05, per_token_outputs=False, want_coef_entropy=False,
+                 extra_coef_log_prob=None):
+    """Fills a ``relax_amd_policy_loss_args`` block; returns (struct, outputs dict holding every live tensor).
+    ``extra_coef_log_prob`` [n]: added to d loss / d log_prob of every unmasked token (the gradient of a caller's loss
+    term that is linear in the log-probs)."""
     dev = _need_gpu(advantages, loss_mask, cu_resp)
     b = int(cu_resp.numel()) - 1
     if loss_kind not in _lib.LOSS_KINDS:
@@ -265,7 +268,8 @@ def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_pr
         raise TypeError("cu_resp must be int64")
     keep = [_f32(t) for t in (log_prob, old_log_prob, ref_log_prob, train_log_prob, rollout_log_prob, advantages,
                                loss_mask, pg_loss_mask, entropy, sample_denom, pg_sample_denom)]
-    for t in keep[:9]:
+    extra = _f32(extra_coef_log_prob)
+    for t in keep[:9] + [extra]:
         if t is not None and t.numel() != n:
             raise ValueError(f"per-token tensor has {t.numel()} elements, expected {n}")
     for t in keep[9:]:
@@ -302,7 +306,8 @@ def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_pr
         setattr(a, k, None if t is None else t.data_ptr())
     a.sample_partials = partials.data_ptr()
     a.metrics = out["metrics"].data_ptr()
-    out["_keepalive"] = (keep, partials, cu_resp)
+    a.extra_coef_log_prob = None if extra is None else extra.data_ptr()
+    out["_keepalive"] = (keep, partials, cu_resp, extra)
     return a, out
 
 

@@ -706,7 +706,7 @@ def test_get_log_probs_and_entropy_topk_outputs_vs_oracle():
         torch.testing.assert_close(chunk.gather(-1, got), torch.topk(chunk, 4, dim=-1).values)
 
 
-@pytest.mark.parametrize("case", ["sampled_clips", "student_topk_forward", "union_jsd"])
+@pytest.mark.parametrize("case", ["sampled_plain", "sampled_clips", "student_topk_forward", "union_jsd"])
 @pytest.mark.parametrize("single_pass", ["auto", "off"])
 def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
     """``opd_loss_coef != 0``: the distillation term (sampled-token or top-K, union mask, per-token and
@@ -720,7 +720,10 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
     g = torch.Generator().manual_seed(2)
     kw = dict(relax_amd_single_pass=single_pass, opd_loss_coef=0.7, use_kl_loss=True, kl_loss_coef=0.01,
               kl_loss_type="k3")
-    if case == "sampled_clips":
+    if case == "sampled_plain":  # linear in the log-probs: its gradient leaves with the single launch
+        kw.update(opd_token_selection="sampled", opd_kl_type="reverse_kl")
+        batch["teacher_log_probs"] = [lp + 0.2 * torch.randn(lp.shape, generator=g) for lp in batch["log_probs"]]
+    elif case == "sampled_clips":
         kw.update(opd_token_selection="sampled", opd_kl_type="low_var_kl", opd_per_token_clip=0.02, opd_is_clip=1.01)
         batch["teacher_log_probs"] = [lp + 0.2 * torch.randn(lp.shape, generator=g) for lp in batch["log_probs"]]
     else:
@@ -746,6 +749,32 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
     for key, w in want_m.items():
         assert abs(met[key].item() - float(w)) < 3e-5 * max(1.0, abs(float(w))), (key, met[key].item(), float(w))
     torch.testing.assert_close(lg.grad.cpu(), lo.grad, atol=3e-5, rtol=1e-5)
+
+
+def test_linear_opd_term_rides_the_single_launch(monkeypatch):
+    """Sampled-token reverse_kl distillation without clips: one fused launch, no separate log-prob or dlogits launch;
+    with a clip configured the two-launch path is taken."""
+    import relax_amd
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("linear OPD term: launches")
+    tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 264
+    logits, batch = _make_batch(32, tot, resp, v)
+    g = torch.Generator().manual_seed(4)
+    batch["teacher_log_probs"] = [lp + 0.2 * torch.randn(lp.shape, generator=g) for lp in batch["log_probs"]]
+    calls = []
+    for name in ("actor_step_fused", "logprob_entropy_fwd", "logprob_entropy_bwd"):
+        real = getattr(ops, name)
+        monkeypatch.setattr(ops, name, lambda *a, _n=name, _r=real, **k: (calls.append(_n), _r(*a, **k))[1])
+    for clip, want in ((None, ["actor_step_fused"]), (0.02, ["logprob_entropy_fwd", "logprob_entropy_bwd"])):
+        calls.clear()
+        args = P.make_args(opd_loss_coef=0.7, opd_token_selection="sampled", opd_kl_type="reverse_kl",
+                           opd_per_token_clip=clip)
+        lg = logits.to(dev).requires_grad_()
+        loss, _ = relax_amd.policy_loss_function(args, _to_dev(batch, dev), lg, None)
+        loss.backward()
+        assert calls == want, (clip, calls)
 
 
 def test_outputs_leave_as_one_packed_copy_in_the_reference_wire_format():
