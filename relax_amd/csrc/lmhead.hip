@@ -1064,7 +1064,7 @@ static int lm_forward(const char* what, const void* hidden, const void* weight, 
                        targets, x_target);
     if (int rc = check_launch("lmhead_target_logit")) return rc;
     // RELAX_AMD_LMHEAD_FWD=mfma16 selects the 8-wave 16x16x32 shape (same results to rounding, same speed on
-    // random operands: it holds a higher clock under the power limit and loses it again to LDS bandwidth)
+    // random operands: it holds a higher clock under the power limit and leaves the matrix cores idle more often)
     const char* shape = getenv("RELAX_AMD_LMHEAD_FWD");
     if (shape && !strcmp(shape, "mfma16"))
       hipLaunchKernelGGL(lmhead_fwd16_kernel, grid, dim3(kLm16Threads), 0, s, h, w, g, c, partial);
