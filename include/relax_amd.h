@@ -181,6 +181,15 @@ typedef struct relax_amd_policy_loss_args {
    * as opd_loss_coef * token_mean(log_prob - teacher_log_prob) (relax/utils/opd/opd_utils.py:1368-1455 with the
    * sampled-token reverse_kl signal), so that term's gradient leaves in the same dlogits launch.  NULL = none. */
   const float* extra_coef_log_prob;
+  /* optional: the sampled-token distillation signal of compute_policy_opd_loss (opd_utils.py:1368-1455) when it is
+   * not linear.  With distill_teacher_log_prob [n_tokens] set, extra_coef_log_prob[t] is the weight of token t's
+   * signal in the loss (opd_loss_coef * mask / clamp_min(sum mask, 1)) and the kernel multiplies it by the signal's
+   * derivative: both log-probs clamped from below at distill_min_clamp, estimator distill_kl_kind (RELAX_AMD_KL_K1
+   * for "reverse_kl", RELAX_AMD_KL_K3 for "low_var_kl"), signal clipped from above at distill_token_clip, times
+   * min(exp(log_prob - old_log_prob), distill_is_clip) taken as a constant.  A NaN switches a clamp / clip off. */
+  const float* distill_teacher_log_prob;
+  int32_t distill_kl_kind;
+  float distill_min_clamp, distill_token_clip, distill_is_clip;
 } relax_amd_policy_loss_args;
 
 int relax_amd_policy_loss(const relax_amd_policy_loss_args* args, void* stream);

@@ -50,6 +50,8 @@ class PolicyLossArgs(C.Structure):
         ("coef_log_prob", _vp), ("coef_entropy", _vp), ("pg_loss_tok", _vp), ("clipfrac_tok", _vp),
         ("ppo_kl_tok", _vp), ("kl_tok", _vp), ("sample_partials", _vp), ("metrics", _vp),
         ("extra_coef_log_prob", _vp),
+        ("distill_teacher_log_prob", _vp), ("distill_kl_kind", _i32),
+        ("distill_min_clamp", _f32), ("distill_token_clip", _f32), ("distill_is_clip", _f32),
     ]
 
 

@@ -241,6 +241,10 @@ extern "C" int relax_amd_actor_step_fused(const void* logits, int dtype, int64_t
     set_error("actor_step_fused: NULL argument");
     return RELAX_AMD_EINVAL;
   }
+  if (const char* why = distill_args_error(*loss)) {
+    set_error("actor_step_fused: %s", why);
+    return RELAX_AMD_EINVAL;
+  }
   if (!(inv_temperature > 0.f)) {
     set_error("actor_step_fused: inv_temperature must be > 0");
     return RELAX_AMD_EINVAL;

@@ -93,6 +93,15 @@ __device__ __forceinline__ void kl_term(int kind, float lp, float ref, float& kl
 }
 
 
+// Host-side check of the optional distillation fields; NULL when they are consistent.
+inline const char* distill_args_error(const relax_amd_policy_loss_args& a) {
+  if (!a.distill_teacher_log_prob) return nullptr;
+  if (!a.extra_coef_log_prob) return "distill_teacher_log_prob needs extra_coef_log_prob (the signal's weights)";
+  if (a.distill_kl_kind != RELAX_AMD_KL_K1 && a.distill_kl_kind != RELAX_AMD_KL_K3)
+    return "distill_kl_kind must be RELAX_AMD_KL_K1 or RELAX_AMD_KL_K3";
+  return nullptr;
+}
+
 struct TokenResult {
   float metric[RELAX_AMD_NUM_METRICS];  // this token's masked contribution to every per-sample sum
   float pg, clipfrac, ppo_kl, kl;       // un-masked per-token values
@@ -103,7 +112,8 @@ struct TokenResult {
 // Per-token inputs of the loss, fetched ahead of time so their latency can hide behind other work.
 struct TokenInputs {
   float old_lp, ref_lp, train_lp, rollout_lp, adv, m, mp;
-  float extra_lp;  // caller-supplied addition to d loss / d log_prob (0 when there is none)
+  float extra_lp;    // caller-supplied addition to d loss / d log_prob (0 when there is none)
+  float teacher_lp;  // teacher log-prob of the sampled-token distillation signal (when that is configured)
   bool has_old, has_train;
 };
 
@@ -119,6 +129,7 @@ __device__ __forceinline__ TokenInputs load_token_inputs(const relax_amd_policy_
   in.m = a.loss_mask[t];
   in.mp = a.pg_loss_mask ? a.pg_loss_mask[t] : in.m;
   in.extra_lp = a.extra_coef_log_prob ? a.extra_coef_log_prob[t] : 0.f;
+  in.teacher_lp = a.distill_teacher_log_prob ? a.distill_teacher_log_prob[t] : 0.f;
   return in;
 }
 
@@ -179,7 +190,25 @@ __device__ __forceinline__ TokenResult token_terms(const relax_amd_policy_loss_a
     o.metric[RELAX_AMD_M_KL_LOSS] = kl * m;
     o.coef_lp += a.kl_coef * (m / den) * dkl;
   }
-  o.coef_lp += in.extra_lp;
+  float extra = in.extra_lp;
+  if (a.distill_teacher_log_prob) {
+    // extra_lp is the weight of this token's distillation signal in the loss; the signal's own derivative follows
+    // the chain clamp_min -> estimator -> clamp(max = token clip) -> x min(ratio, clip) with the ratio detached
+    float s = lp, t = in.teacher_lp, pass = 1.f;
+    if (a.distill_min_clamp == a.distill_min_clamp) {  // set (not NaN)
+      if (s < a.distill_min_clamp) {
+        s = a.distill_min_clamp;
+        pass = 0.f;
+      }
+      t = fmaxf(t, a.distill_min_clamp);
+    }
+    float sig, dsig;
+    kl_term(a.distill_kl_kind, s, t, sig, dsig);
+    if (a.distill_token_clip == a.distill_token_clip && sig > a.distill_token_clip) pass = 0.f;
+    if (a.distill_is_clip == a.distill_is_clip) pass *= fminf(expf(lp - old), a.distill_is_clip);
+    extra *= pass * dsig;
+  }
+  o.coef_lp += extra;
   if (a.rollout_log_prob) {
     const float roll = in.rollout_lp;
     float side = lp;

@@ -186,6 +186,10 @@ extern "C" int relax_amd_policy_loss(const relax_amd_policy_loss_args* a, void* 
     set_error("policy_loss: log_prob, advantages, loss_mask and coef_log_prob must not be NULL");
     return RELAX_AMD_EINVAL;
   }
+  if (const char* why = distill_args_error(*a)) {
+    set_error("policy_loss: %s", why);
+    return RELAX_AMD_EINVAL;
+  }
   if (a->loss_kind < RELAX_AMD_LOSS_PPO || a->loss_kind > RELAX_AMD_LOSS_SAPO) {
     set_error("policy_loss: unknown loss_kind %d", a->loss_kind);
     return RELAX_AMD_EINVAL;

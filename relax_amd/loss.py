@@ -448,21 +448,12 @@ class _SinglePassPolicyLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, flat, lay, inv_t, kw):
-        # kw["linear_lp_term"] = (weights [N], offsets [N]) adds sum_t weights[t] * (lp[t] - offsets[t]) to the loss:
-        # its gradient w.r.t. each log-prob is weights[t], known before the launch, so it leaves in the same dlogits
-        linear = kw.get("linear_lp_term")
-        kw = {k: v for k, v in kw.items() if k != "linear_lp_term"}
-        if linear is not None:
-            kw["extra_coef_log_prob"] = linear[0]
         out, lp, ent, _lse, _spx, dlogits = ops.actor_step_fused(
             flat, lay.targets, lay.token_of_row, lay.sample_ids, lay.n_tokens, inv_t, 1.0, cu_resp=lay.cu_resp, **kw)
         metrics = out["metrics"]
         ctx.dlogits = dlogits
         ctx.mark_non_differentiable(metrics, lp, ent)
-        loss = metrics[_SLOT["loss"]].clone()
-        if linear is not None:
-            loss = loss + (linear[0] * (lp - linear[1])).sum()
-        return loss, metrics, lp, ent
+        return metrics[_SLOT["loss"]].clone(), metrics, lp, ent
 
     @staticmethod
     def backward(ctx, g_loss, _gm, _glp, _gent):
@@ -474,17 +465,16 @@ class _SinglePassPolicyLoss(torch.autograd.Function):
         return d, None, None, None
 
 
-def _linear_opd_term(args, batch, loss_mask, dev):
-    """(weights, teacher log-probs), both [N], when the distillation loss term is linear in this step's log-probs:
-    sampled-token selection with the ``reverse_kl`` signal (lp - teacher) and no clamp, per-token clip or
-    importance-ratio clip (relax/utils/opd/opd_utils.py:1368-1455).  Then the term is
-    ``sum_t weights[t] * (lp[t] - teacher[t])`` with ``weights = opd_loss_coef * mask / clamp_min(sum mask, 1)``.
-    None in every other configuration."""
+def _sampled_opd_kernel_args(args, batch, loss_mask, dev):
+    """(kernel arguments, teacher log-probs [N]) that put the gradient of the sampled-token distillation term
+    (relax/utils/opd/opd_utils.py:1368-1455: ``opd_loss_coef * token_mean(signal)``) into the single launch, or None
+    when the term is not of that kind (top-K selections, no teacher log-probs).  ``extra_coef_log_prob`` holds each
+    token's weight ``opd_loss_coef * mask / clamp_min(sum mask, 1)``; the plain ``reverse_kl`` signal (lp - teacher)
+    has derivative 1 and needs nothing else, ``low_var_kl`` and the clamp / clips are applied by the kernel."""
     if getattr(args, "opd_token_selection", "sampled") in ("student_topk", "teacher_topk", "union"):
         return None
-    if getattr(args, "opd_kl_type", "reverse_kl") != "reverse_kl":
-        return None
-    if any(getattr(args, k, None) is not None for k in ("opd_log_prob_min_clamp", "opd_per_token_clip", "opd_is_clip")):
+    kl_type = getattr(args, "opd_kl_type", "reverse_kl")
+    if kl_type not in ("reverse_kl", "low_var_kl"):
         return None
     teacher = batch.get("teacher_log_probs")
     if teacher is None:
@@ -492,8 +482,17 @@ def _linear_opd_term(args, batch, loss_mask, dev):
     teacher = torch.cat([t.reshape(-1) for t in teacher]).to(device=dev, dtype=torch.float32)
     if teacher.numel() != loss_mask.numel():
         return None
-    weights = loss_mask * (float(args.opd_loss_coef) / torch.clamp_min(loss_mask.sum(), 1))
-    return weights, teacher
+    clamp, tau, is_clip = (getattr(args, k, None) for k in ("opd_log_prob_min_clamp", "opd_per_token_clip",
+                                                            "opd_is_clip"))
+    if (tau is not None or is_clip is not None) and bool((loss_mask == 0).any()):
+        # the clip-fraction metrics are plain means over every response token, masked ones included, and the single
+        # launch does not read the rows of masked tokens: their log-probs come from the two-launch path
+        return None
+    out = {"extra_coef_log_prob": loss_mask * (float(args.opd_loss_coef) / torch.clamp_min(loss_mask.sum(), 1))}
+    if kl_type != "reverse_kl" or any(v is not None for v in (clamp, tau, is_clip)):
+        out["distill"] = dict(teacher=teacher, kl_kind="k1" if kl_type == "reverse_kl" else "k3", min_clamp=clamp,
+                              token_clip=tau, is_clip=is_clip)
+    return out, teacher
 
 
 def _single_pass_ok(args, flat, kw, needs_bwd) -> bool:
@@ -807,16 +806,16 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         kw["lp_requires_grad"] = True
         if opd_gather is not None:
             kw["gather_topk_ids"], topk_widths = _pack_topk_ids(flat, lay, opd_gather)
-    opd_linear = None
+    opd_in_kernel = None
     if opd_on_lp and opd_gather is None and _single_pass_ok(args, flat, kw, needs_bwd):
-        opd_linear = _linear_opd_term(args, batch, kw["loss_mask"], dev)
-    if opd_linear is not None:
-        # the sampled-token reverse-KL signal without clips is coef * token_mean(lp - teacher): linear in the
-        # log-probs, so the single launch carries its gradient and the term's value follows from the launch's lp
+        opd_in_kernel = _sampled_opd_kernel_args(args, batch, kw["loss_mask"], dev)
+    if opd_in_kernel is not None:
+        # the sampled-token term's gradient w.r.t. each log-prob is a per-token weight times the signal's derivative,
+        # which the kernel evaluates next to the policy loss's: one launch; the term's value and metrics follow from
+        # the launch's log-probs on [N] vectors
         kw.pop("lp_requires_grad", None)
-        loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, dict(kw, linear_lp_term=opd_linear))
+        loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, dict(kw, **opd_in_kernel[0]))
         topk_lp = None
-        reported_loss = loss.detach().clone()
     elif not opd_on_lp and _single_pass_ok(args, flat, kw, needs_bwd):
         loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw)
         topk_lp = None
@@ -828,8 +827,16 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
 
     opd_reported = {}
     loss_metric = m("loss")
-    if opd_linear is not None:
-        loss_metric = reported_loss
+    if opd_in_kernel is not None:
+        with torch.no_grad():
+            if "distill" in opd_in_kernel[0]:
+                opd_value, opd_reported = compute_policy_opd_loss(
+                    args=args, batch=batch, log_probs=lp, old_log_probs=old if old is not None else lp,
+                    log_probs_and_entropy={})
+            else:  # plain reverse_kl: the term is the weighted sum of lp - teacher, and reports nothing of its own
+                opd_value = (opd_in_kernel[0]["extra_coef_log_prob"] * (lp - opd_in_kernel[1])).sum()
+        loss = loss + opd_value
+        loss_metric = loss.detach().clone()
     elif opd_on:
         # The distillation term (loss.py:1102-1110) needs log-probs that autograd can see: the two-launch function's
         # own outputs when a gradient is wanted, a separate log-prob launch (with the top-K gather) otherwise.

@@ -254,10 +254,12 @@ def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_pr
                  use_tis=False, mismatch_metrics=False, abs_diff_from_old=1, eps_clip=0.2, eps_clip_high=0.2,
                  eps_clip_c=None, entropy_coef=0.0, kl_coef=0.0, tis_lo=0.0, tis_hi=2.0, opsm_delta=1e-4,
                  tau_pos=1.0, tau_neg=1.05, per_token_outputs=False, want_coef_entropy=False,
-                 extra_coef_log_prob=None):
+                 extra_coef_log_prob=None, distill=None):
     """Fills a ``relax_amd_policy_loss_args`` block; returns (struct, outputs dict holding every live tensor).
     ``extra_coef_log_prob`` [n]: added to d loss / d log_prob of every unmasked token (the gradient of a caller's loss
-    term that is linear in the log-probs)."""
+    term that is linear in the log-probs).  ``distill`` = dict(teacher [n], kl_kind "k1" | "k3", min_clamp, token_clip,
+    is_clip; None = off): ``extra_coef_log_prob`` then holds the weights of the sampled-token distillation signal and
+    the kernel applies the signal's own derivative."""
     dev = _need_gpu(advantages, loss_mask, cu_resp)
     b = int(cu_resp.numel()) - 1
     if loss_kind not in _lib.LOSS_KINDS:
@@ -307,7 +309,17 @@ def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_pr
     a.sample_partials = partials.data_ptr()
     a.metrics = out["metrics"].data_ptr()
     a.extra_coef_log_prob = None if extra is None else extra.data_ptr()
-    out["_keepalive"] = (keep, partials, cu_resp, extra)
+    teacher = None
+    if distill is not None:
+        teacher = _f32(distill["teacher"])
+        if extra is None or teacher.numel() != n:
+            raise ValueError("distill needs extra_coef_log_prob and a teacher log-prob per token")
+        a.distill_teacher_log_prob = teacher.data_ptr()
+        a.distill_kl_kind = _lib.KL_KINDS[distill["kl_kind"]]
+        nan = float("nan")
+        a.distill_min_clamp, a.distill_token_clip, a.distill_is_clip = (
+            nan if distill.get(k) is None else float(distill[k]) for k in ("min_clamp", "token_clip", "is_clip"))
+    out["_keepalive"] = (keep, partials, cu_resp, extra, teacher)
     return a, out
 
 

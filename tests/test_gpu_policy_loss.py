@@ -706,7 +706,8 @@ def test_get_log_probs_and_entropy_topk_outputs_vs_oracle():
         torch.testing.assert_close(chunk.gather(-1, got), torch.topk(chunk, 4, dim=-1).values)
 
 
-@pytest.mark.parametrize("case", ["sampled_plain", "sampled_clips", "student_topk_forward", "union_jsd"])
+@pytest.mark.parametrize("case", ["sampled_plain", "sampled_clips", "sampled_clamped", "sampled_clips_all_tokens",
+                                  "sampled_clamped_all_tokens", "student_topk_forward", "union_jsd"])
 @pytest.mark.parametrize("single_pass", ["auto", "off"])
 def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
     """``opd_loss_coef != 0``: the distillation term (sampled-token or top-K, union mask, per-token and
@@ -720,8 +721,17 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
     g = torch.Generator().manual_seed(2)
     kw = dict(relax_amd_single_pass=single_pass, opd_loss_coef=0.7, use_kl_loss=True, kl_loss_coef=0.01,
               kl_loss_type="k3")
+    if case.endswith("_all_tokens"):
+        # no masked token: the clipped signals' derivative is evaluated inside the single launch (with masked tokens
+        # their clip-fraction metrics need log-probs the single launch does not produce, and two launches run)
+        batch["loss_masks"] = [torch.ones_like(m) for m in batch["loss_masks"]]
+        case = case[:-len("_all_tokens")]
     if case == "sampled_plain":  # linear in the log-probs: its gradient leaves with the single launch
         kw.update(opd_token_selection="sampled", opd_kl_type="reverse_kl")
+        batch["teacher_log_probs"] = [lp + 0.2 * torch.randn(lp.shape, generator=g) for lp in batch["log_probs"]]
+    elif case == "sampled_clamped":  # clamp from below on both log-probs, ratio clip, no old log-probs in the batch
+        kw.update(opd_token_selection="sampled", opd_kl_type="reverse_kl", opd_log_prob_min_clamp=-1.5,
+                  opd_is_clip=1.02, opd_per_token_clip=0.1)
         batch["teacher_log_probs"] = [lp + 0.2 * torch.randn(lp.shape, generator=g) for lp in batch["log_probs"]]
     elif case == "sampled_clips":
         kw.update(opd_token_selection="sampled", opd_kl_type="low_var_kl", opd_per_token_clip=0.02, opd_is_clip=1.01)
@@ -752,8 +762,8 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
 
 
 def test_linear_opd_term_rides_the_single_launch(monkeypatch):
-    """Sampled-token reverse_kl distillation without clips: one fused launch, no separate log-prob or dlogits launch;
-    with a clip configured the two-launch path is taken."""
+    """Sampled-token distillation signals (plain reverse_kl: linear in the log-probs; low_var_kl or clipped: derivative
+    evaluated by the kernel): one fused launch, no separate log-prob or dlogits launch."""
     import relax_amd
     from relax_amd import ops
 
@@ -767,14 +777,19 @@ def test_linear_opd_term_rides_the_single_launch(monkeypatch):
     for name in ("actor_step_fused", "logprob_entropy_fwd", "logprob_entropy_bwd"):
         real = getattr(ops, name)
         monkeypatch.setattr(ops, name, lambda *a, _n=name, _r=real, **k: (calls.append(_n), _r(*a, **k))[1])
-    for clip, want in ((None, ["actor_step_fused"]), (0.02, ["logprob_entropy_fwd", "logprob_entropy_bwd"])):
+    two = ["logprob_entropy_fwd", "logprob_entropy_bwd"]
+    ones = [torch.ones_like(m) for m in batch["loss_masks"]]
+    for kl_type, clip, masks, want in (
+            ("reverse_kl", None, None, ["actor_step_fused"]), ("low_var_kl", None, None, ["actor_step_fused"]),
+            ("reverse_kl", 0.02, ones, ["actor_step_fused"]), ("reverse_kl", 0.02, None, two)):
         calls.clear()
-        args = P.make_args(opd_loss_coef=0.7, opd_token_selection="sampled", opd_kl_type="reverse_kl",
+        case_batch = batch if masks is None else dict(batch, loss_masks=masks)
+        args = P.make_args(opd_loss_coef=0.7, opd_token_selection="sampled", opd_kl_type=kl_type,
                            opd_per_token_clip=clip)
         lg = logits.to(dev).requires_grad_()
-        loss, _ = relax_amd.policy_loss_function(args, _to_dev(batch, dev), lg, None)
+        loss, _ = relax_amd.policy_loss_function(args, _to_dev(case_batch, dev), lg, None)
         loss.backward()
-        assert calls == want, (clip, calls)
+        assert calls == want, (kl_type, clip, calls)
 
 
 def test_outputs_leave_as_one_packed_copy_in_the_reference_wire_format():
