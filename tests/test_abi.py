@@ -26,16 +26,22 @@ def test_struct_layout_matches_c_header(tmp_path):
     src = tmp_path / "layout.c"
     src.write_text(
         '#include <stdio.h>\n#include <stddef.h>\n#include "relax_amd.h"\n'
-        "int main(void){printf(\"%zu %zu %zu %zu %d\\n\", sizeof(relax_amd_policy_loss_args),"
+        "int main(void){printf(\"%zu %zu %zu %zu %d %zu %zu %zu\\n\", sizeof(relax_amd_policy_loss_args),"
         " offsetof(relax_amd_policy_loss_args, n_samples), offsetof(relax_amd_policy_loss_args, eps_clip),"
-        " offsetof(relax_amd_policy_loss_args, metrics), RELAX_AMD_NUM_METRICS);return 0;}\n"
+        " offsetof(relax_amd_policy_loss_args, metrics), RELAX_AMD_NUM_METRICS,"
+        " offsetof(relax_amd_policy_loss_args, extra_coef_log_prob),"
+        " offsetof(relax_amd_policy_loss_args, distill_kl_kind),"
+        " offsetof(relax_amd_policy_loss_args, distill_is_clip));return 0;}\n"
     )
     exe = tmp_path / "layout"
     subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
-    size, off_n, off_eps, off_metrics, nmet = map(int, subprocess.check_output([str(exe)]).split())
+    size, off_n, off_eps, off_metrics, nmet, off_extra, off_kind, off_is = map(
+        int, subprocess.check_output([str(exe)]).split())
     S = _lib.PolicyLossArgs
     assert C.sizeof(S) == size
     assert S.n_samples.offset == off_n and S.eps_clip.offset == off_eps and S.metrics.offset == off_metrics
+    assert S.extra_coef_log_prob.offset == off_extra and S.distill_kl_kind.offset == off_kind
+    assert S.distill_is_clip.offset == off_is
     assert nmet == _lib.NUM_METRICS
 
 
@@ -48,6 +54,13 @@ def test_argument_validation_reports_errors_without_touching_the_gpu():
     rc = L.relax_amd_logprob_entropy_fwd(C.c_void_p(16), 9, 4, 8, 8, None, C.c_void_p(16), 1.0, C.c_void_p(16), None, None, None, None)
     assert rc == -1 and b"dtype" in L.relax_amd_last_error()
     assert L.relax_amd_logprob_entropy_fwd(None, 0, 0, 8, 8, None, None, 1.0, None, None, None, None, None) == 0
+    # the distillation fields of the policy-loss block are checked before anything is launched
+    a = _lib.PolicyLossArgs()
+    a.metrics = a.sample_partials = a.cu_resp = 16
+    a.distill_teacher_log_prob = 16
+    assert L.relax_amd_policy_loss(C.byref(a), None) == -1 and b"extra_coef_log_prob" in L.relax_amd_last_error()
+    a.extra_coef_log_prob, a.distill_kl_kind = 16, _lib.KL_KINDS["k2"]
+    assert L.relax_amd_policy_loss(C.byref(a), None) == -1 and b"distill_kl_kind" in L.relax_amd_last_error()
     rc = L.relax_amd_group_rewards(None, 0, None, 4, 7, None, None, None)
     assert rc == -1 and b"mode" in L.relax_amd_last_error()
     rc = L.relax_amd_masked_whiten(None, None, 0, 1, 1e-8, None, None, None, None)
