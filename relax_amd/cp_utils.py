@@ -80,6 +80,37 @@ def get_sum_of_sample_mean(
     return reducer
 
 
+class PerSampleDivisorReducer:
+    """Reducer ``x [N] -> sum_i (x_i * m_i).sum() / divisor_i`` that also carries its divisors.
+
+    A function named by ``--custom-pg-loss-reducer-function-path`` (loss.py:1062-1072) may return one of these instead
+    of an opaque callable: ``policy_loss_function`` then reads ``sample_divisors`` and evaluates the pg_loss reduction
+    inside its fused launch; any other code can still call the object like the closure the reference expects."""
+
+    def __init__(self, response_lengths, loss_masks, sample_divisors):
+        self.response_lengths = [int(r) for r in response_lengths]
+        self.loss_masks = loss_masks
+        self.sample_divisors = torch.as_tensor(sample_divisors, dtype=torch.float32).reshape(-1)
+        if self.sample_divisors.numel() != len(self.response_lengths):
+            raise ValueError(f"{self.sample_divisors.numel()} divisors for {len(self.response_lengths)} samples")
+        self._state = None
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        if self._state is None or self._state[0].device != x.device:
+            dev = x.device
+            mask = torch.cat([m.reshape(-1) for m in self.loss_masks]).to(device=dev, dtype=torch.float32)
+            self._state = (mask, _cu(self.response_lengths, dev), 1.0 / self.sample_divisors.to(dev))
+        return _MaskedSampleReduce.apply(x, *self._state)
+
+
+def get_seq_mean_token_sum_reducer(total_lengths, response_lengths, loss_masks, calculate_per_token_loss=False):
+    """``--custom-pg-loss-reducer-function-path relax_amd.cp_utils.get_seq_mean_token_sum_reducer``: every sequence's
+    masked token sum, averaged over the B sequences of the micro-batch (sequence-mean of token-sums; a fully masked
+    sequence still counts in B).  Signature of the reference's plug-in point, loss.py:1066-1068."""
+    b = len(response_lengths)
+    return PerSampleDivisorReducer(response_lengths, loss_masks, torch.full((b,), float(max(b, 1))))
+
+
 def get_cp_local_mask_sums(total_lengths, response_lengths, loss_masks, qkv_format="thd", max_seq_lens=None,
                            padded_total_lengths=None, dynamic_cp_size=None, dynamic_cp_rank=None) -> torch.Tensor:
     return _mask_sums(loss_masks)

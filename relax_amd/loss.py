@@ -25,7 +25,8 @@ import torch
 from . import ops
 from ._lib import METRIC_SLOTS
 from ._staging import upload_int64
-from .cp_utils import get_cp_local_num_tokens, get_sum_of_sample_mean, sample_denominators
+from .cp_utils import (PerSampleDivisorReducer, get_cp_local_num_tokens, get_sum_of_sample_mean,
+                       sample_denominators)
 from .ppo_utils import get_grpo_returns
 
 _SLOT = {k: i for i, k in enumerate(METRIC_SLOTS)}
@@ -716,10 +717,19 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     flat = _check_logits(logits, args, batch.get("max_seq_lens"))
     dev = flat.device
     est = args.advantage_estimator
-    if getattr(args, "custom_tis_function_path", None) is not None \
-            or getattr(args, "custom_pg_loss_reducer_function_path", None) is not None:
-        return _composed_policy_loss_function(args, batch, logits, None)  # user code acts on per-token tensors
     response_lengths, total_lengths = batch["response_lengths"], batch["total_lengths"]
+    if getattr(args, "custom_tis_function_path", None) is not None:
+        return _composed_policy_loss_function(args, batch, logits, None)  # user code acts on per-token tensors
+    hook_pg_denom = None
+    reducer_path = getattr(args, "custom_pg_loss_reducer_function_path", None)
+    if reducer_path is not None:
+        # the built-in importance weights leave the loss masks as they are, so the masks the reference hands the
+        # hook (loss.py:1065) are the batch's own in every case that reaches this point
+        hook_reducer = load_function(reducer_path)(total_lengths, response_lengths, batch["loss_masks"],
+                                                   bool(getattr(args, "calculate_per_token_loss", False)))
+        if not isinstance(hook_reducer, PerSampleDivisorReducer):
+            return _composed_policy_loss_function(args, batch, logits, None)  # an opaque callable: [N] tensors
+        hook_pg_denom = hook_reducer.sample_divisors
     needs_bwd = torch.is_grad_enabled() and logits.requires_grad
     lay = PackedLayout(dev, flat.size(0), batch["unconcat_tokens"], total_lengths, response_lengths, needs_bwd,
                        _padded_starts(args, batch.get("max_seq_lens")))
@@ -743,7 +753,7 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     denom = batch.get("relax_amd_sample_denominators")
     if denom is None and not per_token:
         denom = sample_denominators(batch["loss_masks"], lay, batch.get("sample_index_mask_sums"))
-    pg_denom = batch.get("relax_amd_pg_sample_denominators")
+    pg_denom = hook_pg_denom if hook_pg_denom is not None else batch.get("relax_amd_pg_sample_denominators")
     use_kl = bool(getattr(args, "use_kl_loss", False))
     kw = dict(
         old_log_prob=old,

@@ -110,6 +110,101 @@ def test_policy_loss_function_vs_oracle(name, dtype, tol, single_pass):
     torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, atol=tol, rtol=BF16_ULP if dtype == torch.bfloat16 else 0)
 
 
+AGG_CASES = {
+    "gspo": dict(advantage_estimator="gspo", eps_clip=3e-4, eps_clip_high=4e-4),
+    "gspo_wide_kl": dict(advantage_estimator="gspo", eps_clip=0.2, eps_clip_high=0.2, entropy_coef=0.02,
+                         use_kl_loss=True, kl_loss_coef=0.05, kl_loss_type="k3"),
+    "cispo": dict(advantage_estimator="cispo", eps_clip=0.2, eps_clip_high=0.28),
+    "cispo_tis": dict(advantage_estimator="cispo", eps_clip=0.2, eps_clip_high=0.28, use_tis=True, tis_clip=1.02,
+                      tis_clip_low=0.97, entropy_coef=0.01),
+    "ppo_per_token": dict(calculate_per_token_loss=True, use_kl_loss=True, kl_loss_coef=0.1, kl_loss_type="k1"),
+}
+
+
+@pytest.mark.parametrize("name", sorted(AGG_CASES))
+@pytest.mark.parametrize("route", ["all_terms", "pg_only_batch_key", "pg_only_reference_hook"])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-5), (torch.bfloat16, 2e-3)])
+@pytest.mark.parametrize("single_pass", ["auto", "off"])
+def test_seq_mean_token_sum_aggregation_vs_oracle(name, route, dtype, tol, single_pass):
+    """Sequence-mean-token-sum aggregation (every sequence's masked token sum, averaged over the B sequences) against
+    ``oracle.reducers.seq_mean_token_sum``: loss, every metric and dlogits.  ``all_terms`` divides every reduced term
+    by B (``relax_amd_sample_denominators``); the two ``pg_only`` routes reduce pg_loss that way and leave the other
+    terms on the reference's sample-mean reducer, as ``--custom-pg-loss-reducer-function-path`` does
+    (loss.py:1062-1076): once through the batch key, once through the reference's own hook returning a reducer that
+    carries its divisors (which keeps the step on the fused launch)."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("seq_mean_token_sum", name, route, dtype, single_pass)
+    tot, resp, v = [9, 6, 12, 7, 15], [4, 3, 7, 5, 11], 264
+    logits, batch = _make_batch(29, tot, resp, v, dtype)
+    b = len(resp)
+    per_token = bool(AGG_CASES[name].get("calculate_per_token_loss", False))
+    if route == "all_terms" and per_token:
+        pytest.skip("token-sum mode has no per-sample divisors for the other terms")
+    kw = dict(relax_amd_single_pass=single_pass, **AGG_CASES[name])
+    if route == "pg_only_reference_hook":
+        kw["custom_pg_loss_reducer_function_path"] = "relax_amd.cp_utils.get_seq_mean_token_sum_reducer"
+    args = P.make_args(**kw)
+    masks = batch["loss_masks"]
+    lo = logits.float().clone().requires_grad_()
+    if route == "all_terms":
+        want_loss, want_m = P.policy_loss_function(args, dict(batch), lo, R.seq_mean_token_sum(resp, masks))
+    else:
+        want_loss, want_m = P.policy_loss_function(args, dict(batch), lo, R.make_reducer(resp, masks, per_token),
+                                                   pg_reducer_factory=lambda m: R.seq_mean_token_sum(resp, m))
+    want_loss.backward()
+    db = _to_dev(batch, dev)
+    if route == "all_terms":
+        db["relax_amd_sample_denominators"] = torch.full((b,), float(b), device=dev)
+    elif route == "pg_only_batch_key":
+        db["relax_amd_pg_sample_denominators"] = torch.full((b,), float(b), device=dev)
+    lg = logits.to(dev).requires_grad_()
+    calls = []
+    if route == "pg_only_reference_hook":  # the hook must not push the step onto the composed path
+        import relax_amd.loss as RL
+
+        orig = RL._composed_policy_loss_function
+        RL._composed_policy_loss_function = lambda *a, **k: calls.append(1) or orig(*a, **k)
+    try:
+        loss, met = relax_amd.policy_loss_function(args, db, lg, None)
+    finally:
+        if route == "pg_only_reference_hook":
+            RL._composed_policy_loss_function = orig
+    assert not calls
+    loss.backward()
+    assert abs(loss.item() - want_loss.item()) < tol * max(1.0, abs(want_loss.item()))
+    assert set(met) == set(want_m)
+    for k, w in want_m.items():
+        assert abs(met[k].item() - float(w)) < tol * max(1.0, abs(float(w))), (k, met[k].item(), float(w))
+    torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, atol=tol, rtol=BF16_ULP if dtype == torch.bfloat16 else 0)
+    # the aggregation is not the sample mean in disguise: pg_loss differs from the reference reducer's
+    lo2 = logits.float().clone().requires_grad_()
+    _, plain = P.policy_loss_function(P.make_args(**AGG_CASES[name]), dict(batch), lo2,
+                                      R.make_reducer(resp, masks, per_token))
+    assert abs(float(plain["pg_loss"]) - float(want_m["pg_loss"])) > 10 * tol
+
+
+def test_divisor_reducer_called_as_plain_closure_matches_token_loop():
+    """The reducer object the hook returns is still the callable the reference expects (``reducer(x) -> scalar``)."""
+    from relax_amd.cp_utils import get_seq_mean_token_sum_reducer
+
+    dev = require_gpu()
+    announce("divisor reducer as closure")
+    g = torch.Generator().manual_seed(3)
+    resp = [5, 1, 8, 3]
+    masks = [(torch.rand(n, generator=g) > 0.4).float() for n in resp]
+    masks[1] = torch.zeros(1)
+    x = torch.randn(sum(resp), generator=g)
+    want = R.seq_mean_token_sum(resp, masks)(x.double())
+    red = get_seq_mean_token_sum_reducer([n + 2 for n in resp], resp, [m.to(dev) for m in masks], False)
+    xd = x.to(dev).requires_grad_()
+    got = red(xd)
+    got.backward()
+    assert abs(got.item() - want.item()) < 1e-6
+    torch.testing.assert_close(xd.grad.cpu(), torch.cat(masks) / len(resp), atol=1e-7, rtol=0)
+
+
 @pytest.mark.parametrize("single_pass", ["auto", "off"])
 def test_reinforce_pp_masked_nonfinite_values_do_not_leak(single_pass):
     """REINFORCE++ reduces with a mask-safe reducer: NaN / inf advantages and old log-probs at masked tokens leave the
