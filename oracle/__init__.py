@@ -52,7 +52,15 @@ live in ``tests/test_oracle_*.py``):
   a stop at the first element reports the uncapped moment is kept (read from ppo_utils.py:417-418).
 * ``policy.value_loss_function`` / ``policy.get_values``: a three-token case worked by hand (clipped and unclipped
   branches of the maximum, the clip fraction, the response-row slicing).
-* ``reducers.seq_mean_token_sum``: the reference has no implementation of this
-  aggregation (only the reducer plug-in point, loss.py:1062-1072)
-  -- **parity unpinned**; defined here as sum_i sum_t x*m / B.
+* ``losses.opsm_mask`` (ppo_utils.py:142-180): scalar per-sequence / per-token Python loops on a hand-worked case
+  (sequence KL exactly at delta is kept, ``A == 0`` kept, a fully masked sequence divides by one, the dropped-token
+  count includes masked tokens) and on random ragged batches.  ``losses.icepop`` (loss.py:772-801): brute force per
+  token with ratios exactly on either closed bound and one ulp outside, every metric, gradient = weight.
+  ``losses.sapo`` (ppo_utils.py:212-270): scalar loops over random ratios with both advantage signs and ``A == 0``
+  (takes ``tau_neg``), the gradient ``4 s (1 - s) r A`` against fp64 autograd, the clip-fraction threshold from the
+  closed form ``4 s (1 - s) = sech^2(x / 2) < 0.9  <=>  |x| > 2 atanh(sqrt 0.1)``.
+* ``reducers.seq_mean_token_sum``: the reference has no implementation of this aggregation (only the reducer plug-in
+  point, loss.py:1062-1072; the example file its help text names is not in the tree), so there is nothing of the
+  reference's to be at parity with; the definition used here, sum_i sum_t x*m / B, is pinned by a token loop, a
+  hand-sized case and its gradient m_t / B.
 """

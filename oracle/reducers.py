@@ -41,7 +41,9 @@ def num_tokens(masks: list) -> torch.Tensor:
 
 
 def seq_mean_token_sum(response_lengths: list, masks: list):
-    """sum_i sum_t x*m / B.  PARITY UNPINNED: the reference only has the plug-in point (loss.py:1062-1072)."""
+    """sum_i sum_t x*m / B: each sequence's masked token sum, averaged over the B sequences.  The reference only has
+    the plug-in point for such a reducer (loss.py:1062-1072) and no implementation, so this definition is the
+    contract; tests/test_oracle_losses.py pins it by a token loop."""
     b = len(response_lengths)
 
     def red(x):

@@ -177,7 +177,10 @@ def test_seq_mean_token_sum_aggregation_vs_oracle(name, route, dtype, tol, singl
     assert set(met) == set(want_m)
     for k, w in want_m.items():
         assert abs(met[k].item() - float(w)) < tol * max(1.0, abs(float(w))), (k, met[k].item(), float(w))
-    torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, atol=tol, rtol=BF16_ULP if dtype == torch.bfloat16 else 0)
+    # dividing token sums by B instead of by the token count leaves gradient entries of magnitude ~100 on the wide-clip
+    # GSPO case (sequence ratios far from one): fp32 rounding of those is relative, 1e-5 of the value
+    torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, atol=tol,
+                               rtol=BF16_ULP if dtype == torch.bfloat16 else 1e-5)
     # the aggregation is not the sample mean in disguise: pg_loss differs from the reference reducer's
     lo2 = logits.float().clone().requires_grad_()
     _, plain = P.policy_loss_function(P.make_args(**AGG_CASES[name]), dict(batch), lo2,
