@@ -410,6 +410,21 @@ int relax_amd_lmhead_logprob_fwd(const void* hidden, const void* weight, int dty
                                  const int64_t* targets, float inv_temperature, void* workspace, float* log_prob,
                                  float* entropy, float* lse, float* spx, void* stream);
 /*
+ * The same forward pass for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Identical to
+ * relax_amd_lmhead_logprob_fwd except that the workspace is a fixed array inside the library (one copy per GPU,
+ * RELAX_AMD_LMHEAD_STATIC_SCRATCH_BYTES, held until the process ends), so the call allocates and frees nothing.
+ * n_tokens above RELAX_AMD_LMHEAD_STATIC_MAX_TOKENS returns RELAX_AMD_EUNSUPPORTED.  All calls on one GPU share
+ * that GPU's array: calls that overlap in time on one GPU (different streams or threads) race; serialise them.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress); make it outside graph capture.
+ */
+#define RELAX_AMD_LMHEAD_STATIC_MAX_TOKENS 32768
+#define RELAX_AMD_LMHEAD_STATIC_SCRATCH_BYTES (25 * 4 * RELAX_AMD_LMHEAD_STATIC_MAX_TOKENS)
+int relax_amd_lmhead_logprob_fwd_static(const void* hidden, const void* weight, int dtype, int64_t n_tokens,
+                                        int64_t hidden_size, int64_t vocab, int64_t h_stride, int64_t w_stride,
+                                        const int64_t* targets, float inv_temperature, float* log_prob,
+                                        float* entropy, float* lse, float* spx, void* stream);
+/*
  * Backward helper of the fused LM head: recomputes the logits of n_tokens rows on the matrix cores and writes the
  * gradient w.r.t. the logits, transposed and in bf16:
  *   d_t[v, n] = inv_T * ( g_lp[n]*(onehot(target[n]) - p) + g_ent[n] * p * (spx[n] - x) ),  p = exp(x - lse[n])

@@ -76,6 +76,8 @@ SIGNATURES = {
     "relax_amd_lmhead_workspace_bytes": (_i64, [_i64]),
     "relax_amd_lmhead_logprob_fwd": (
         C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _i64, _i64, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "relax_amd_lmhead_logprob_fwd_static": (
+        C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _i64, _i64, _vp, _f32, _vp, _vp, _vp, _vp, _vp]),
     "relax_amd_lmhead_dlogits_t": (
         C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _vp]),
     "relax_amd_lmhead_logprob_fwd_keep": (

@@ -29,6 +29,7 @@
 // tiles are shared by S workgroups and weight tiles by 32/S workgroups inside that XCD's L2.
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "device_utils.h"
 #include "relax_amd.h"
@@ -1094,6 +1095,61 @@ extern "C" int relax_amd_lmhead_logprob_fwd(const void* hidden, const void* weig
   if (n_tokens == 0) return RELAX_AMD_OK;
   return lm_forward("lmhead_logprob_fwd", hidden, weight, dtype, n_tokens, hidden_size, vocab, h_stride, w_stride,
                     targets, inv_temperature, workspace, log_prob, entropy, lse, spx, nullptr, 0, stream);
+}
+
+// Scratch of the allocation-free entry point: the per-split softmax partials and the target logits of up to
+// RELAX_AMD_LMHEAD_STATIC_MAX_TOKENS tokens.  One copy per GPU, held until the process ends.  The name is a host-side
+// stand-in, not a device address: host code only ever uses the pointer hipGetSymbolAddress returns for the current
+// device.
+static __device__ __align__(256) float lm_static_scratch[RELAX_AMD_LMHEAD_STATIC_SCRATCH_BYTES / sizeof(float)];
+
+namespace {
+constexpr int kLmMaxDevices = 64;
+std::mutex lm_static_mutex;
+void* lm_static_ptr[kLmMaxDevices] = {};
+}  // namespace
+
+// The current device's copy of lm_static_scratch (looked up once per device, with that device current).
+static int lm_static_workspace(const char* what, void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kLmMaxDevices) {
+    set_error("%s: no usable current device (%s)", what, e == hipSuccess ? "index out of range" : hipGetErrorString(e));
+    return RELAX_AMD_EINVAL;
+  }
+  std::lock_guard<std::mutex> lock(lm_static_mutex);
+  if (!lm_static_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(lm_static_scratch));
+    if (e != hipSuccess || !p) {
+      set_error("%s: hipGetSymbolAddress failed on device %d: %s", what, dev, hipGetErrorString(e));
+      return RELAX_AMD_ELAUNCH;
+    }
+    lm_static_ptr[dev] = p;
+  }
+  *out = lm_static_ptr[dev];
+  return RELAX_AMD_OK;
+}
+
+extern "C" int relax_amd_lmhead_logprob_fwd_static(const void* hidden, const void* weight, int dtype,
+                                                   int64_t n_tokens, int64_t hidden_size, int64_t vocab,
+                                                   int64_t h_stride, int64_t w_stride, const int64_t* targets,
+                                                   float inv_temperature, float* log_prob, float* entropy, float* lse,
+                                                   float* spx, void* stream) {
+  if (n_tokens == 0) return RELAX_AMD_OK;
+  if (n_tokens < 0 || n_tokens > RELAX_AMD_LMHEAD_STATIC_MAX_TOKENS ||
+      relax_amd_lmhead_workspace_bytes(n_tokens) > int64_t(RELAX_AMD_LMHEAD_STATIC_SCRATCH_BYTES)) {
+    set_error("lmhead_logprob_fwd_static: n_tokens=%lld is outside 0..%d, the size the built-in scratch holds; use "
+              "relax_amd_lmhead_logprob_fwd with a caller workspace", (long long)n_tokens,
+              RELAX_AMD_LMHEAD_STATIC_MAX_TOKENS);
+    return RELAX_AMD_EUNSUPPORTED;
+  }
+  void* workspace = nullptr;
+  if (int rc = lm_static_workspace("lmhead_logprob_fwd_static", &workspace)) return rc;
+  // every partial and target logit the combine kernel reads is written by this call's own launches first, so the
+  // contents a previous call left behind need no clearing
+  return lm_forward("lmhead_logprob_fwd_static", hidden, weight, dtype, n_tokens, hidden_size, vocab, h_stride,
+                    w_stride, targets, inv_temperature, workspace, log_prob, entropy, lse, spx, nullptr, 0, stream);
 }
 
 extern "C" int relax_amd_lmhead_logprob_fwd_keep(const void* hidden, const void* weight, int dtype, int64_t n_tokens,
