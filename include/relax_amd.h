@@ -390,8 +390,10 @@ int relax_amd_actor_step_fused(const void* logits, int dtype, int64_t n_rows, in
                                float inv_temperature, const relax_amd_policy_loss_args* loss, float grad_scale,
                                float* log_prob, float* entropy, float* lse, float* spx, void* dlogits,
                                int64_t d_row_stride, void* stream);
-/* data[row, :] *= *factor_dev in place; returns immediately on the device when the factor is exactly 1.  Lets an
- * autograd backward apply an upstream scalar that differs from the grad_scale assumed above without a host read. */
+/* data[row, :] *= *factor_dev in place; returns immediately on the device when the factor is 1 to within 2^-20 (a
+ * product of fp32 factors that equals the assumed scale mathematically may differ from it in the last bits).  Lets an
+ * autograd backward apply upstream / grad_scale when the upstream scalar turns out to differ from the grad_scale
+ * assumed above, without a host read. */
 int relax_amd_scale_rows_inplace(void* data, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                                  const float* factor_dev, void* stream);
 

@@ -270,20 +270,45 @@ def policy_loss_function(args, batch, logits, reducer, pg_reducer=None, tis_fn=N
     return loss, metrics
 
 
+def sft_loss_function(args, batch, logits, reducer):
+    """loss.py:1247-1293: negative reduced log-probability of the response tokens."""
+    _, out = get_log_probs_and_entropy(logits, args=args, unconcat_tokens=batch["unconcat_tokens"],
+                                       total_lengths=batch["total_lengths"], response_lengths=batch["response_lengths"])
+    log_probs = torch.cat(out["log_probs"], dim=0)
+    loss = -reducer(log_probs)
+    if log_probs.numel() == 0:
+        loss = loss + 0 * logits.sum()
+    return loss, {"loss": loss.clone().detach()}
+
+
 def loss_function(args, batch, num_microbatches, logits, dp_world: int = 1, func=None):
-    """Scaling tail of loss.py:1488-1620 at cp = 1: returns (loss, normalizer, {"keys", "values"})."""
+    """Scaling tail of loss.py:1488-1620 at cp = 1: returns (loss, normalizer, {"keys", "values"}).  The loss is
+    picked by ``args.loss_type`` (:1515-1533) unless ``func`` is given; dummy micro-batches and an explicit
+    ``__loss_scale__`` follow :1565-1586."""
     ntok = reducers.num_tokens(batch["loss_masks"])
     red = reducers.make_reducer(
         batch["response_lengths"], batch["loss_masks"], args.calculate_per_token_loss,
         batch.get("sample_index_mask_sums"),
     )
-    func = func or policy_loss_function
+    if func is None:
+        func = {"policy_loss": policy_loss_function, "sft": sft_loss_function,
+                "value_loss": value_loss_function}[getattr(args, "loss_type", "policy_loss")]
     loss, log = func(args, batch, logits, red)
-    if not args.calculate_per_token_loss:
-        loss = loss * num_microbatches / args.global_batch_size * dp_world
-    denom = ntok if args.calculate_per_token_loss else torch.zeros_like(ntok)
+    dummy = batch.get("__is_dummy__", False)
+    if dummy:
+        loss = 0.0 * loss
+    elif not args.calculate_per_token_loss:
+        explicit = batch.get("__loss_scale__", None)
+        if explicit is not None:
+            loss = loss * explicit
+        else:
+            loss = loss * num_microbatches / batch.get("dynamic_global_batch_size", args.global_batch_size) * dp_world
+    eff = torch.zeros_like(ntok) if dummy else ntok
+    denom = eff if args.calculate_per_token_loss else torch.zeros_like(ntok)
     vals = torch.stack([denom] + [v if isinstance(v, torch.Tensor) else torch.tensor(v) for v in log.values()])
-    norm = ntok if args.calculate_per_token_loss else torch.tensor(1)
+    if dummy:
+        vals = torch.zeros_like(vals)
+    norm = eff if args.calculate_per_token_loss else torch.tensor(1)
     return loss, norm, {"keys": list(log.keys()), "values": vals}
 
 

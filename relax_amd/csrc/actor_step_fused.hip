@@ -284,29 +284,43 @@ extern "C" int relax_amd_actor_step_fused(const void* logits, int dtype, int64_t
   }
 }
 
-// dlogits *= (*factor) in place, skipped entirely (one compare per workgroup) when the factor is exactly 1: lets the
-// autograd backward of the fused step honour an upstream gradient that differs from the scale assumed at forward time
-// without a host read-back.
-__global__ __launch_bounds__(256) void rescale_rows_kernel(uint16_t* __restrict__ p16, float* __restrict__ p32,
-                                                           int64_t stride, int64_t vocab, int is_bf16,
+// dlogits *= (*factor) in place.  Skipped entirely (one compare per workgroup) when the factor is 1 to within 2^-20:
+// the autograd backward of the fused step passes upstream / assumed here, and a chain of fp32 multiplications that
+// mathematically equals the assumed scale may differ from it in the last bits; a relative 1e-6 is far below the
+// rounding of the stored gradients.  Lets the backward honour an upstream gradient that differs from the scale
+// assumed at forward time without a host read-back.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void rescale_rows_kernel(T* __restrict__ data, int64_t stride, int64_t vocab,
                                                            const float* __restrict__ factor) {
   const float f = *factor;
-  if (f == 1.0f) return;
-  const int64_t row = blockIdx.x;
-  if (p32) {
-    float* r = p32 + row * stride;
-    for (int64_t e = threadIdx.x; e < vocab; e += 256) r[e] *= f;
-  } else {
-    uint16_t* r = p16 + row * stride;
-    for (int64_t e = threadIdx.x; e < vocab; e += 256) {
-      if (is_bf16) {
-        r[e] = uint16_t(f32_to_bf16_bits(__uint_as_float(uint32_t(r[e]) << 16) * f));
-      } else {
-        _Float16 h = __builtin_bit_cast(_Float16, r[e]);
-        r[e] = __builtin_bit_cast(uint16_t, _Float16(float(h) * f));
-      }
+  if (fabsf(f - 1.0f) <= 0x1p-20f) return;
+  T* r = data + int64_t(blockIdx.x) * stride;
+  if constexpr (VEC) {
+    constexpr int kPer = Row<T>::kPerVec;
+    u32x4* rv = reinterpret_cast<u32x4*>(r);
+    const int64_t nvec = vocab / kPer;
+    for (int64_t i = threadIdx.x; i < nvec; i += 256) {
+      float x[kPer];
+      Row<T>::unpack(rv[i], x);
+#pragma unroll
+      for (int k = 0; k < kPer; ++k) x[k] *= f;
+      rv[i] = Row<T>::pack(x);
     }
+    for (int64_t e = nvec * kPer + threadIdx.x; e < vocab; e += 256) Row<T>::store1(r + e, Row<T>::load1(r + e) * f);
+  } else {
+    for (int64_t e = threadIdx.x; e < vocab; e += 256) Row<T>::store1(r + e, Row<T>::load1(r + e) * f);
   }
+}
+
+template <typename T>
+static void launch_rescale(void* data, int64_t n_rows, int64_t vocab, int64_t stride, const float* factor,
+                           hipStream_t s) {
+  const bool vec = aligned16(data) && (stride * int64_t(sizeof(T))) % 16 == 0;
+  const dim3 grid(static_cast<unsigned>(n_rows)), block(256);
+  if (vec)
+    hipLaunchKernelGGL((rescale_rows_kernel<T, true>), grid, block, 0, s, static_cast<T*>(data), stride, vocab, factor);
+  else
+    hipLaunchKernelGGL((rescale_rows_kernel<T, false>), grid, block, 0, s, static_cast<T*>(data), stride, vocab, factor);
 }
 
 extern "C" int relax_amd_scale_rows_inplace(void* data, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
@@ -320,9 +334,9 @@ extern "C" int relax_amd_scale_rows_inplace(void* data, int dtype, int64_t n_row
     return RELAX_AMD_EINVAL;
   }
   if (n_rows == 0) return RELAX_AMD_OK;
-  hipLaunchKernelGGL(rescale_rows_kernel, dim3(static_cast<unsigned>(n_rows)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), dtype == RELAX_AMD_F32 ? nullptr : static_cast<uint16_t*>(data),
-                     dtype == RELAX_AMD_F32 ? static_cast<float*>(data) : nullptr, row_stride, vocab,
-                     int(dtype == RELAX_AMD_BF16), factor_dev);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == RELAX_AMD_F32) launch_rescale<float>(data, n_rows, vocab, row_stride, factor_dev, s);
+  else if (dtype == RELAX_AMD_BF16) launch_rescale<bf16_t>(data, n_rows, vocab, row_stride, factor_dev, s);
+  else launch_rescale<f16_t>(data, n_rows, vocab, row_stride, factor_dev, s);
   return check_launch("rescale_rows");
 }

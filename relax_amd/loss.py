@@ -289,7 +289,7 @@ def _sft_single_pass(args: Namespace, batch: dict, logits: torch.Tensor):
         use_tis=False, mismatch_metrics=False, abs_diff_from_old=2, eps_clip=0.2, eps_clip_high=0.2, entropy_coef=0.0,
         kl_coef=0.0, tis_lo=0.0, tis_hi=2.0, opsm_delta=1e-4, tau_pos=1.0, tau_neg=1.05)
     inv_t = 1.0 / float(getattr(args, "rollout_temperature", 1.0))
-    loss, _metrics, _lp, _ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw)
+    loss, _metrics, _lp, _ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw, expected_grad_scale(batch))
     return loss
 
 
@@ -442,17 +442,34 @@ class _FusedPolicyLoss(torch.autograd.Function):
         return d, None, None, None
 
 
+GRAD_SCALE_KEY = "relax_amd_grad_scale"
+
+
+def expected_grad_scale(batch) -> float:
+    """The upstream gradient the loss is expected to receive in backward (``batch["relax_amd_grad_scale"]``, set by
+    ``loss_function`` from its own scaling; 1 when the loss is differentiated as returned)."""
+    hint = batch.get(GRAD_SCALE_KEY)
+    if hint is None:
+        return 1.0
+    hint = float(hint)
+    return hint if (hint == hint and hint != 0.0 and abs(hint) != float("inf")) else 1.0
+
+
 class _SinglePassPolicyLoss(torch.autograd.Function):
     """logits [T, V] -> scalar loss, single-launch form: each workgroup scans its row and at once walks it again
-    (out of cache) to write dlogits for an upstream gradient of 1, so HBM sees one read and one write per row.  The
-    backward multiplies by the actual upstream gradient on the device (a no-op kernel when it is exactly 1)."""
+    (out of registers or cache) to write dlogits for the upstream gradient ``assumed_scale`` the caller expects, so
+    HBM sees one read and one write per row.  The backward compares the actual upstream gradient with the assumed one
+    on the device: a no-op kernel when they agree, one more pass over dlogits (and a second rounding of 16-bit
+    gradients) when they do not."""
 
     @staticmethod
-    def forward(ctx, flat, lay, inv_t, kw):
+    def forward(ctx, flat, lay, inv_t, kw, assumed_scale=1.0):
         out, lp, ent, _lse, _spx, dlogits = ops.actor_step_fused(
-            flat, lay.targets, lay.token_of_row, lay.sample_ids, lay.n_tokens, inv_t, 1.0, cu_resp=lay.cu_resp, **kw)
+            flat, lay.targets, lay.token_of_row, lay.sample_ids, lay.n_tokens, inv_t, float(assumed_scale),
+            cu_resp=lay.cu_resp, **kw)
         metrics = out["metrics"]
         ctx.dlogits = dlogits
+        ctx.assumed_scale = float(assumed_scale)
         ctx.mark_non_differentiable(metrics, lp, ent)
         return metrics[_SLOT["loss"]].clone(), metrics, lp, ent
 
@@ -462,8 +479,11 @@ class _SinglePassPolicyLoss(torch.autograd.Function):
         if d is None:
             raise RuntimeError("the single-pass policy loss holds its gradient once: backward cannot run twice")
         ctx.dlogits = None
-        ops.scale_rows_inplace(d, g_loss.reshape(1).to(torch.float32).contiguous())
-        return d, None, None, None
+        factor = g_loss.reshape(1).to(torch.float32)
+        if ctx.assumed_scale != 1.0:
+            factor = factor / ctx.assumed_scale
+        ops.scale_rows_inplace(d, factor.contiguous())
+        return d, None, None, None, None
 
 
 def _sampled_opd_kernel_args(args, batch, loss_mask, dev):
@@ -824,10 +844,11 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         # which the kernel evaluates next to the policy loss's: one launch; the term's value and metrics follow from
         # the launch's log-probs on [N] vectors
         kw.pop("lp_requires_grad", None)
-        loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, dict(kw, **opd_in_kernel[0]))
+        loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, dict(kw, **opd_in_kernel[0]),
+                                                          expected_grad_scale(batch))
         topk_lp = None
     elif not opd_on_lp and _single_pass_ok(args, flat, kw, needs_bwd):
-        loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw)
+        loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw, expected_grad_scale(batch))
         topk_lp = None
     else:
         loss, mvec, lp, ent, topk_lp = _FusedPolicyLoss.apply(flat, lay, inv_t, kw)
@@ -942,6 +963,40 @@ def mtp_only_loss_function(args: Namespace, batch: dict, hidden_states: torch.Te
     return loss, {"loss": loss.detach()}
 
 
+def _upstream_scale_hint(args, batch, num_microbatches, dp_world_size):
+    """The gradient the loss returned by ``loss_function``'s inner function will receive in backward, as far as it
+    is known on the host: this function's own factor (loss.py:1572-1586: ``__loss_scale__``, or
+    ``num_microbatches / global_batch_size * dp_world_size``; none in per-token mode) times the factor the training
+    schedule applies to the returned loss before ``backward()``.  The latter is ``args.relax_amd_schedule_loss_scale``
+    when set; otherwise ``1 / num_microbatches`` in sample-mean mode (Megatron's ``forward_step_calc_loss`` divides
+    the loss by the returned normalizer, 1, and by the number of micro-batches) and 1 in per-token mode (Megatron
+    normalises the gradients by the token count later).  None when unknown without a device read; a wrong value
+    costs one rescaling pass in backward, never correctness."""
+    if batch.get("__is_dummy__", False):
+        return None
+    per_token = bool(getattr(args, "calculate_per_token_loss", False))
+    own = 1.0
+    if not per_token:
+        explicit = batch.get("__loss_scale__", None)
+        if explicit is not None:
+            if isinstance(explicit, torch.Tensor):
+                if explicit.is_cuda or explicit.numel() != 1:
+                    return None
+                explicit = explicit.item()
+            own = float(explicit)
+        else:
+            gbs = batch.get("dynamic_global_batch_size", getattr(args, "global_batch_size", 1))
+            if isinstance(gbs, torch.Tensor):
+                if gbs.is_cuda:
+                    return None
+                gbs = gbs.item()
+            own = float(num_microbatches) / float(gbs) * float(dp_world_size)
+    schedule = getattr(args, "relax_amd_schedule_loss_scale", None)
+    if schedule is None:
+        schedule = 1.0 if per_token else 1.0 / max(int(num_microbatches), 1)
+    return own * float(schedule)
+
+
 def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: torch.Tensor, *, lm_head_forward=None,
                   dp_world_size: int = 1):
     """Counterpart of loss.py:1443-1620 on one GPU: token count, the loss selected by ``args.loss_type``
@@ -972,6 +1027,12 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
         func = partial(sft_loss_function_chunked, lm_head_forward=lm_head_forward)
     else:
         func = sft_loss_function
+    hint = _upstream_scale_hint(args, batch, num_microbatches, dp_world_size)
+    if hint is not None and func in (policy_loss_function, sft_loss_function):
+        # the single-launch losses write dlogits during their forward pass, already multiplied by the upstream
+        # gradient they expect; telling them the scale applied below saves a rescaling pass over dlogits in backward
+        batch = dict(batch)
+        batch[GRAD_SCALE_KEY] = hint
     if getattr(args, "recompute_loss_function", False):
         # loss.py:1535-1543: the loss is evaluated again during backward instead of keeping what it saved
         from torch.utils.checkpoint import checkpoint

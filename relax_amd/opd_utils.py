@@ -203,15 +203,17 @@ class _FusedOpdLoss(torch.autograd.Function):
     """student logits [N, V] -> (masked token-mean reverse KL, per-token KL), one launch: the gradient of the token
     mean w.r.t. each token's KL (mask / clamp_min(sum mask, 1)) is known before the forward, so the kernel writes the
     student gradient for an upstream gradient of 1 while the rows are still in cache; the backward multiplies by the
-    actual upstream gradient on the device (a no-op kernel when it is exactly 1)."""
+    actual upstream gradient over the assumed one (``batch["relax_amd_grad_scale"]``, default 1) on the device: a
+    no-op kernel when they agree."""
 
     @staticmethod
-    def forward(ctx, student, teacher, mask):
+    def forward(ctx, student, teacher, mask, assumed_scale=1.0):
         den = torch.clamp_min(mask.sum(), 1)
         g = mask / den
-        kl, _ls, _lt, d = ops.reverse_kl_step_fused(student, teacher, g)
+        kl, _ls, _lt, d = ops.reverse_kl_step_fused(student, teacher, g if assumed_scale == 1.0 else g * assumed_scale)
         ctx.d = d
         ctx.shape = student.shape
+        ctx.assumed_scale = float(assumed_scale)
         ctx.mark_non_differentiable(kl)
         return (kl * mask).sum() / den, kl
 
@@ -221,8 +223,11 @@ class _FusedOpdLoss(torch.autograd.Function):
         if d is None:
             raise RuntimeError("the fused OPD loss holds its gradient once: backward cannot run twice")
         ctx.d = None
-        ops.scale_rows_inplace(d, g_loss.reshape(1).to(torch.float32).contiguous())
-        return d.view(ctx.shape), None, None
+        factor = g_loss.reshape(1).to(torch.float32)
+        if ctx.assumed_scale != 1.0:
+            factor = factor / ctx.assumed_scale
+        ops.scale_rows_inplace(d, factor.contiguous())
+        return d.view(ctx.shape), None, None, None
 
 
 def opd_loss_full_vocab(batch: dict, student_logits: torch.Tensor, teacher_logits: torch.Tensor):
@@ -236,7 +241,9 @@ def opd_loss_full_vocab(batch: dict, student_logits: torch.Tensor, teacher_logit
     if not (torch.is_grad_enabled() and student_logits.requires_grad):
         kl = compute_opd_kl_full_vocab(student_logits, teacher_logits)
         return reduce_opd_loss(batch, kl), kl
-    return _FusedOpdLoss.apply(student_logits, teacher_logits.detach(), mask)
+    from .loss import expected_grad_scale
+
+    return _FusedOpdLoss.apply(student_logits, teacher_logits.detach(), mask, expected_grad_scale(batch))
 
 
 def resolve_opd_gather_topk_token_ids(args, batch):

@@ -319,6 +319,71 @@ def test_loss_function_scaling_and_exact_token_count():
     assert n.dtype == torch.int64 and n.item() == R.num_tokens(batch["loss_masks"]).item()
 
 
+@pytest.mark.parametrize("loss_type", ["policy_loss", "sft"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("schedule", ["megatron", "as_returned", "explicit_scale", "per_token"])
+def test_loss_function_scale_reaches_the_single_launch(loss_type, dtype, schedule, monkeypatch):
+    """``loss_function`` multiplies the loss by ``num_microbatches / global_batch_size * dp`` (or ``__loss_scale__``)
+    and the training schedule divides by the number of micro-batches, so the upstream gradient of the fused
+    single-launch loss is never 1 in training.  The scale is handed to the launch, which writes dlogits already
+    multiplied by it: backward must find nothing left to rescale (factor 1) and the gradient must equal the
+    two-launch path's, which applies the scale in its dlogits kernel, to one rounding of the output dtype.  When the
+    schedule does something else than announced, backward rescales and the gradient is still right."""
+    import relax_amd
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("loss_function scale into the single launch", loss_type, dtype, schedule)
+    tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 4096
+    logits, batch = _make_batch(53, tot, resp, v, dtype)
+    if loss_type == "sft":
+        tot = resp = [9, 6, 12, 7]
+        logits, batch = _make_batch(53, tot, resp, v, dtype)
+    nm, gbs, dp = 4, 32, 2
+    kw = dict(loss_type=loss_type, global_batch_size=gbs, use_kl_loss=True, kl_loss_coef=0.01, kl_loss_type="k3",
+              entropy_coef=0.01, calculate_per_token_loss=(schedule == "per_token"))
+    bd = _to_dev(batch, dev)
+    if schedule == "explicit_scale":
+        bd["__loss_scale__"] = 0.3
+    post = {"megatron": 1.0 / nm, "as_returned": 1.0, "explicit_scale": 1.0 / nm, "per_token": 1.0}[schedule]
+    if schedule == "as_returned":
+        kw["relax_amd_schedule_loss_scale"] = 1.0
+    factors = []
+    real = ops.scale_rows_inplace
+    monkeypatch.setattr(ops, "scale_rows_inplace", lambda d, f: factors.append(f.clone()) or real(d, f))
+    grads = {}
+    for mode in ("auto", "off"):
+        args = P.make_args(relax_amd_single_pass=mode, **kw)
+        lg = logits.to(dev).requires_grad_()
+        loss, _norm, _log = relax_amd.loss_function(args, bd, nm, lg, dp_world_size=dp)
+        (loss * post).backward()
+        grads[mode] = lg.grad.clone()
+    assert len(factors) == 1  # only the single-launch path goes through the in-place rescale
+    assert abs(factors[0].item() - 1.0) <= 2.0 ** -20, factors[0].item()
+    ulp = {torch.float32: 2e-6, torch.bfloat16: 2.0 ** -8}[dtype]
+    torch.testing.assert_close(grads["auto"].float(), grads["off"].float(), atol=1e-9, rtol=ulp)
+    assert grads["auto"].abs().sum().item() > 0
+    # oracle, same scaling
+    lo = logits.float().clone().requires_grad_()
+    oargs = P.make_args(**kw)
+    ob = dict(batch)
+    if schedule == "explicit_scale":
+        ob["__loss_scale__"] = 0.3
+    want, _, _ = P.loss_function(oargs, ob, nm, lo, dp_world=dp)
+    (want * post).backward()
+    tol = 3e-5 if dtype == torch.float32 else 2e-3
+    torch.testing.assert_close(grads["auto"].float().cpu(), lo.grad, atol=tol, rtol=max(ulp, 1e-5))
+    # a schedule that does not do what was announced: the backward rescales, the result is still right
+    factors.clear()
+    args = P.make_args(relax_amd_single_pass="auto", **kw)
+    lg = logits.to(dev).requires_grad_()
+    loss, _norm, _log = relax_amd.loss_function(args, bd, nm, lg, dp_world_size=dp)
+    (loss * post * 7.0).backward()
+    assert len(factors) == 1 and abs(factors[0].item() - 7.0) < 1e-5
+    torch.testing.assert_close(lg.grad.float().cpu(), lo.grad * 7.0, atol=7 * tol,
+                               rtol=max(2 * ulp, 1e-5))
+
+
 @pytest.mark.parametrize("loss_type", ["policy_loss", "sft", "value_loss"])
 @pytest.mark.parametrize("reentrant", [True, False])
 def test_loss_function_recompute_gives_the_same_loss_and_gradient(loss_type, reentrant):
