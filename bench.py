@@ -33,12 +33,49 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 PEAK_SCLK_MHZ = 2400.0  # the shader clock the published matrix-core peak is quoted at
 METRIC = "tokens/s fused logprob+entropy+loss fwd+bwd @V=151936 bf16; % HBM/MFMA peak"
-# HBM bytes one launch of the fused actor step moves at the default workload, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE at the L2 <-> fabric boundary (counter x 2.000 for FETCH_SIZE): the register-resident kernel
-# (profiles/actor_step_resident_bf16_v151936_n65536.md) fetches 15 664 908 KiB and writes 19 469 551 KiB; the two-walk
-# kernel (profiles/actor_step_fused_bf16_v151936_n65536.md, RELAX_AMD_FUSED_STEP_KERNEL=cached) 26 780 743 + 19 464 492.
-MEASURED_TRAFFIC_RESIDENT = (15664908 + 19469551) * 1024.0
-MEASURED_TRAFFIC_FUSED = (26780743 + 19464492) * 1024.0
+PROFILES_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles")
+
+
+def measured_traffic(kernel: str, rows: int, vocab: int):
+    """(HBM bytes per launch, source file) for ``kernel`` on ``rows`` x ``vocab``, from the rocprofv3 --pmc summaries
+    under profiles/: a line ``counters: kernel=<name> rows=<n> vocab=<v> FETCH_SIZE_KiB=<a> fetch_scale=<f>
+    WRITE_SIZE_KiB=<b> write_scale=<g>`` gives (a * f + b * g) KiB, the per-dispatch counter readings scaled by what
+    the same counters read for a plain copy of known size.  (None, None) when no summary covers this launch: the
+    counters need the profiler and are not collected by this run."""
+    import glob
+    import re
+
+    for path in sorted(glob.glob(os.path.join(PROFILES_DIR, "*.md"))):
+        for line in open(path, errors="replace"):
+            if not line.startswith("counters:"):
+                continue
+            m = re.match(r"counters: kernel=(.+?) rows=(\d+) vocab=(\d+) FETCH_SIZE_KiB=([\d.]+) fetch_scale=([\d.]+) "
+                         r"WRITE_SIZE_KiB=([\d.]+) write_scale=([\d.]+)", line.strip())
+            if m and m.group(1) == kernel and int(m.group(2)) == rows and int(m.group(3)) == vocab:
+                kib = float(m.group(4)) * float(m.group(5)) + float(m.group(6)) * float(m.group(7))
+                return kib * 1024.0, "profiles/" + os.path.basename(path)
+    return None, None
+
+
+def hbm_roofline(kernel: str, launch_ms: float, necessary_bytes: float, rows: int, vocab: int, kernel_ms: dict,
+                 ms_per_step: float, survey_bytes: float | None = None) -> dict:
+    """Roofline block of a bandwidth-bound launch.  ``achieved`` = the bytes the launch has to move (every input row
+    it needs read once, every output row written once) / its HIP-event time; ``frac`` = achieved / 8 TB/s, a true
+    fraction.  ``survey_bytes`` (the forward-read + backward-read + write count of a two-pass implementation) is kept
+    beside it as ``two_pass_*``: a kernel that keeps the row on chip moves fewer bytes than that, so the figure can
+    exceed the memory system's peak and is not a roofline fraction."""
+    achieved = necessary_bytes / (launch_ms * 1e-3) / 1e9
+    frac = achieved / HBM_PEAK_GBS
+    assert frac <= 1.0, f"roofline fraction {frac} > 1: the byte count does not describe the launch"
+    traffic, source = measured_traffic(kernel, rows, vocab)
+    out = {"bound": "hbm", "kernel": kernel, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": frac,
+           "traffic": traffic, "traffic_source": source, "algorithmic_bytes_per_launch": necessary_bytes,
+           "avg_launch_ms": launch_ms, "kernel_ms": kernel_ms,
+           "step_GBs": necessary_bytes / (ms_per_step * 1e-3) / 1e9}
+    if survey_bytes is not None:
+        out["two_pass_bytes_per_launch"] = survey_bytes
+        out["two_pass_GBs"] = survey_bytes / (launch_ms * 1e-3) / 1e9
+    return out
 
 
 def fused_step_kernel_name(vocab: int) -> str:
@@ -231,20 +268,30 @@ def emit(a, n_tokens, wall, workload, config, roofline, cpu):
     }))
 
 
+def live_rows(batch) -> int:
+    """Response tokens whose loss mask is not zero: the rows a step has to read (a masked token's gradient row is
+    all zeros whatever its logits hold)."""
+    return int(sum(int((m != 0).sum().item()) for m in batch["loss_masks"]))
+
+
 def run_actor_step(a, dev) -> None:
     import relax_amd
 
     args = make_args()
+    args.loss_type = "policy_loss"
     logits, batch, g = make_workload(dev, a.seqs, a.seq_len, a.vocab)
     attach_old_and_ref(batch, logits, args, g)
     logits.requires_grad_()
     n_tokens = a.seqs * a.seq_len
     if a.two_launch:
         args.relax_amd_single_pass = "off"
+    # the step as the training loop runs it: loss_function applies Megatron's gradient-accumulation scaling
+    # (num_microbatches / global_batch_size * dp = 1 / 16 here), so the loss's upstream gradient is not 1
+    num_microbatches = 1
 
     def step():
         logits.grad = None
-        loss, _ = relax_amd.policy_loss_function(args, batch, logits, None)
+        loss, _normalizer, _log = relax_amd.loss_function(args, batch, num_microbatches, logits)
         loss.backward()
         return loss
 
@@ -257,27 +304,21 @@ def run_actor_step(a, dev) -> None:
         del src, dst
     wall, kernel_ms, _, loss = timed_steps(step, a.warmup, a.steps)
     ms_per_step = wall * 1e3 / a.steps
-    row_bytes = float(a.vocab * logits.element_size()) * n_tokens
+    row_bytes = float(a.vocab * logits.element_size())
+    live = live_rows(batch)
+    # what the step must move: every live row read once, every dlogits row written once (masked rows: zeros)
+    necessary = row_bytes * (live + n_tokens)
     if "actor_step_fused" in kernel_ms:
-        # one launch does the forward scan and the dlogits backward: 3*V*s algorithmic bytes per token (forward read,
-        # backward read, dlogits write); its second read is served by cache, see "traffic"
-        dom, dom_bytes = kernel_ms["actor_step_fused"], 3.0 * row_bytes
-        dom_name = fused_step_kernel_name(a.vocab)
-        traffic = None
-        if (a.vocab, n_tokens) == (VOCAB, SEQS * SEQ_LEN):
-            traffic = MEASURED_TRAFFIC_RESIDENT if "resident" in dom_name else MEASURED_TRAFFIC_FUSED
-    else:
-        dom, dom_name, dom_bytes = kernel_ms["logprob_entropy_bwd"], "logprob_entropy_bwd_kernel<bf16_t, true>", 2.0 * row_bytes
-        traffic = None
-    achieved = dom_bytes / (dom * 1e-3) / 1e9
+        dom, dom_name = kernel_ms["actor_step_fused"], fused_step_kernel_name(a.vocab)
+    else:  # two launches: the backward (read live rows, write all rows) dominates; the forward read is its own launch
+        dom, dom_name = kernel_ms["logprob_entropy_bwd"], "logprob_entropy_bwd_kernel<bf16_t, true>"
     emit(a, n_tokens, wall,
          f"Qwen3-8B-shaped actor step: {a.seqs} seqs x {a.seq_len} tokens = {n_tokens} rows x V={a.vocab} bf16 "
-         f"logits, PPO-clip 0.2/0.28 + k3 KL 1e-3, fwd + bwd to dlogits",
-         {"rows": n_tokens, "vocab": a.vocab, "loss": float(loss.item())},
-         {"bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-          "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "algorithmic_bytes_per_launch": dom_bytes,
-          "avg_launch_ms": dom, "kernel_ms": kernel_ms,
-          "step_algorithmic_GBs": 3.0 * row_bytes / (ms_per_step * 1e-3) / 1e9},
+         f"logits, PPO-clip 0.2/0.28 + k3 KL 1e-3, loss_function (scale 1/{args.global_batch_size}) fwd + bwd to "
+         f"dlogits",
+         {"rows": n_tokens, "live_rows": live, "vocab": a.vocab, "loss": float(loss.item())},
+         hbm_roofline(dom_name, dom, necessary, n_tokens, a.vocab, kernel_ms, ms_per_step,
+                      survey_bytes=3.0 * row_bytes * n_tokens if "actor_step_fused" in kernel_ms else None),
          cpu_baseline(args, a.cpu_rows, a.vocab) if a.cpu_rows > 0 else None)
 
 
@@ -496,21 +537,19 @@ def run_reverse_kl(a, dev) -> None:
         return loss
 
     wall, kernel_ms, _, loss = timed_steps(step, a.warmup, a.steps)
-    row_bytes = float(v * 2) * n
+    row_bytes = float(v * 2)
     if "reverse_kl_step_fused" in kernel_ms:
-        # forward scan of both rows, second pass over both (out of registers / cache), write of the student gradient
-        dom, dom_name, dom_bytes = kernel_ms["reverse_kl_step_fused"], kl_step_kernel_name(v), 5.0 * row_bytes
+        # every token reports its KL, so both rows of every token are read once; one gradient row written per token
+        dom, dom_name, necessary = kernel_ms["reverse_kl_step_fused"], kl_step_kernel_name(v), 3.0 * row_bytes * n
+        survey = 5.0 * row_bytes * n  # forward read of both rows, backward re-read of both, gradient write
     else:
-        dom, dom_name, dom_bytes = kernel_ms["reverse_kl_bwd"], "reverse_kl_bwd_kernel<bf16_t, true>", 3.0 * row_bytes
-    achieved = dom_bytes / (dom * 1e-3) / 1e9
+        dom, dom_name, necessary = kernel_ms["reverse_kl_bwd"], "reverse_kl_bwd_kernel<bf16_t, true>", 3.0 * row_bytes * n
+        survey = None
     emit(a, n, wall,
          f"on-policy distillation: student/teacher bf16 logits [{n}, {v}], full-vocab reverse KL, token-mean, fwd + "
          f"student dlogits bwd",
          {"rows": n, "vocab": v, "loss": float(loss.item())},
-         {"bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS,
-          "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": dom_bytes,
-          "avg_launch_ms": dom, "kernel_ms": kernel_ms,
-          "step_algorithmic_GBs": 5.0 * row_bytes / (wall / a.steps) / 1e9},
+         hbm_roofline(dom_name, dom, necessary, n, v, kernel_ms, wall * 1e3 / a.steps, survey_bytes=survey),
          None)
 
 
@@ -578,20 +617,19 @@ def run_cfg1(a, dev) -> None:
         return loss
 
     wall, kernel_ms, _, loss = timed_steps(step, a.warmup, a.steps)
-    row_bytes = float(v * 4) * n
+    row_bytes = float(v * 4)
     dom = kernel_ms["actor_step_fused"]
-    achieved = 3.0 * row_bytes / (dom * 1e-3) / 1e9
+    live = live_rows(batch)
     out_cpu = None
     if a.cpu_rows > 0:
         out_cpu = cpu_baseline(args, a.cpu_rows, v)
     emit(a, n, wall,
          f"GRPO plumbing: {prompts} prompts x {group} = {seqs} responses x {resp_len} tokens = {n} rows x V={v} fp32 "
          f"logits, group-normalised advantages, PPO-clip 0.2, token-mean, fwd + bwd to dlogits",
-         {"rows": n, "vocab": v, "loss": float(loss.item()), "logits_dtype": "f32", "advantages_ms": adv_ms},
-         {"bound": "hbm", "kernel": "actor_step_fused_kernel<float, true, 512>", "achieved": achieved,
-          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-          "algorithmic_bytes_per_launch": 3.0 * row_bytes, "avg_launch_ms": dom, "kernel_ms": kernel_ms,
-          "step_algorithmic_GBs": 3.0 * row_bytes / (wall / a.steps) / 1e9},
+         {"rows": n, "live_rows": live, "vocab": v, "loss": float(loss.item()), "logits_dtype": "f32",
+          "advantages_ms": adv_ms},
+         hbm_roofline("actor_step_fused_kernel<float, true, 512>", dom, row_bytes * (live + n), n, v, kernel_ms,
+                      wall * 1e3 / a.steps, survey_bytes=3.0 * row_bytes * n),
          out_cpu)
 
 
@@ -633,9 +671,11 @@ def run_varlen(a, dev, loss_kind: str) -> None:
         unconcat_tokens=[torch.randint(0, v, (ln,), device=dev, generator=g) for ln in lengths],
         total_lengths=lengths, response_lengths=lengths, loss_masks=masks,
         advantages=[shaped[i].expand(ln).contiguous() for i, ln in enumerate(lengths)],
-        # sequence-mean-token-sum: every sample's masked token sum is divided by the number of sequences
-        relax_amd_sample_denominators=torch.full((seqs,), float(seqs), device=dev),
     )
+    # sequence-mean-token-sum aggregation of pg_loss through the reference's own reducer hook (loss.py:1062-1072):
+    # every sample's masked token sum divided by the number of sequences; the returned reducer carries its divisors,
+    # so the step stays on the fused launches
+    args.custom_pg_loss_reducer_function_path = "relax_amd.cp_utils.get_seq_mean_token_sum_reducer"
     attach_old_and_ref(batch, logits, args, g)
     logits.requires_grad_()
 
@@ -646,20 +686,18 @@ def run_varlen(a, dev, loss_kind: str) -> None:
         return loss
 
     wall, kernel_ms, _, loss = timed_steps(step, a.warmup, a.steps)
-    row_bytes = float(v * 2) * n
-    name = "actor_step_fused" if "actor_step_fused" in kernel_ms else "logprob_entropy_bwd"
+    row_bytes = float(v * 2)
+    live = live_rows(batch)
+    fused = "actor_step_fused" in kernel_ms
+    name = "actor_step_fused" if fused else "logprob_entropy_bwd"
     dom = kernel_ms[name]
-    dom_bytes = (3.0 if name == "actor_step_fused" else 2.0) * row_bytes
-    achieved = dom_bytes / (dom * 1e-3) / 1e9
     emit(a, n, wall,
          f"packed varlen: {seqs} sequences {lengths} = {n} rows x V={v} bf16 logits, ~30 % masked spans, RLOO "
          f"advantages, {loss_kind.upper()} loss, sequence-mean-token-sum, fwd + bwd to dlogits",
-         {"rows": n, "vocab": v, "loss": float(loss.item()), "lengths": lengths},
-         {"bound": "hbm", "kernel": fused_step_kernel_name(v) if name == "actor_step_fused" else name + "_kernel<bf16_t>",
-          "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-          "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": dom_bytes,
-          "avg_launch_ms": dom, "kernel_ms": kernel_ms,
-          "step_algorithmic_GBs": 3.0 * row_bytes / (wall / a.steps) / 1e9},
+         {"rows": n, "live_rows": live, "vocab": v, "loss": float(loss.item()), "lengths": lengths},
+         hbm_roofline(fused_step_kernel_name(v) if fused else name + "_kernel<bf16_t, true>", dom,
+                      row_bytes * (live + n), n, v, kernel_ms, wall * 1e3 / a.steps,
+                      survey_bytes=3.0 * row_bytes * n if fused else None),
          None)
 
 

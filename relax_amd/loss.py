@@ -1060,7 +1060,7 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
     values = torch.stack([denominator.to(torch.float32)] + [v.to(torch.float32) for v in log.values()])
     if is_dummy:
         values = torch.zeros_like(values)
-    normalizer = effective if per_token else torch.tensor(1, device=logits.device)
+    normalizer = effective if per_token else torch.ones((), dtype=torch.int64, device=logits.device)  # no host copy
     return loss, normalizer, {"keys": list(log.keys()), "values": values}
 
 
