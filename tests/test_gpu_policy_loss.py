@@ -817,6 +817,132 @@ def test_full_size_packed_varlen_gspo_and_cispo_properties():
     assert changed[inside & (flat_mask != 0)].float().mean().item() > 0.99
 
 
+def _cfg4_lengths():
+    """The benchmark's packed lengths: 8 draws from U[2048, 32768], the longest halved until the total fits 131072."""
+    cpu = torch.Generator().manual_seed(0)
+    lengths = [int(x) for x in torch.randint(2048, 32769, (8,), generator=cpu)]
+    while sum(lengths) > 131072:
+        lengths[lengths.index(max(lengths))] //= 2
+    return lengths, cpu
+
+
+@pytest.mark.parametrize("estimator", ["gspo", "cispo"])
+def test_cfg4_full_size_varlen_seq_mean_token_sum_vs_oracle(estimator):
+    """The agentic packed configuration at its stated size: 8 sequences of 2k-32k tokens (129 579 rows x 151 936 bf16
+    logits, 39.4 GB), 3-6 masked tool-output spans per sequence (~30 % of tokens), RLOO advantages over the group of
+    8, GSPO (clip 3e-4 / 4e-4) or CISPO, sequence-mean-token-sum aggregation through the reference's reducer hook.
+
+    Oracle comparison at full size: the per-token losses, the sequence-level ratio, the aggregation, every metric and
+    d loss / d log-prob come from the oracle on the [N] log-prob vector (log-probs and entropy themselves are checked
+    against the oracle's row arithmetic on sampled rows), and dlogits rows are checked on sampled rows against
+    d loss / d log-prob * (onehot - softmax) computed on the CPU.  Plus the size-independent properties: every
+    gradient row sums to zero, masked rows are exactly zero."""
+    import relax_amd
+    from oracle import advantages as OA
+    from oracle import logprob as O
+
+    dev = require_gpu()
+    v = 151936
+    lengths, cpu = _cfg4_lengths()
+    n = sum(lengths)
+    announce("cfg4 full size", estimator, lengths, n)
+    assert 100000 < n <= 131072 and min(lengths) >= 2048 and max(lengths) <= 32768
+    g = torch.Generator(device=dev).manual_seed(0)
+    logits = torch.empty((1, n, v), dtype=torch.bfloat16, device=dev)
+    for s0 in range(0, n, 2048):
+        e0 = min(n, s0 + 2048)
+        logits[0, s0:e0] = (torch.randn((e0 - s0, v), device=dev, generator=g) * 3.0).to(torch.bfloat16)
+    masks = []
+    for ln in lengths:
+        m = torch.ones(ln)
+        spans = int(torch.randint(3, 7, (1,), generator=cpu))
+        for _ in range(spans):
+            w = int(0.3 * ln / spans)
+            st = int(torch.randint(0, ln - w, (1,), generator=cpu))
+            m[st:st + w] = 0.0
+        masks.append(m)
+    frac_masked = 1.0 - sum(float(m.sum()) for m in masks) / n
+    assert 0.15 < frac_masked < 0.35
+    rewards = torch.rand(8, generator=cpu)
+    shaped = OA.rloo_leave_one_out(rewards)
+    toks = [torch.randint(0, v, (ln,), device=dev, generator=g) for ln in lengths]
+    kw = dict(advantage_estimator=estimator, custom_pg_loss_reducer_function_path=
+              "relax_amd.cp_utils.get_seq_mean_token_sum_reducer")
+    kw.update(dict(eps_clip=3e-4, eps_clip_high=4e-4) if estimator == "gspo" else dict(eps_clip=0.2, eps_clip_high=0.28))
+    args = P.make_args(**kw)
+    with torch.no_grad():
+        _, out = relax_amd.get_log_probs_and_entropy(logits, args=args, unconcat_tokens=toks, total_lengths=lengths,
+                                                     response_lengths=lengths, with_entropy=True)
+    lp_gpu = torch.cat(out["log_probs"])
+    ent_gpu = torch.cat(out["entropy"])
+    # old log-probs: a small per-sequence drift plus token noise, so that GSPO's sequence ratios straddle its clip range
+    drift = (torch.rand(8, generator=cpu) - 0.5) * 1.2e-3
+    old = [lp.cpu() + drift[i] + 0.02 * torch.randn(lp.shape, generator=cpu) for i, lp in enumerate(out["log_probs"])]
+    batch = dict(unconcat_tokens=toks, total_lengths=lengths, response_lengths=lengths,
+                 loss_masks=[m.to(dev) for m in masks],
+                 advantages=[shaped[i].to(dev).expand(ln).contiguous() for i, ln in enumerate(lengths)],
+                 log_probs=[o.to(dev) for o in old])
+    logits.requires_grad_()
+    loss, met = relax_amd.policy_loss_function(args, batch, logits, None)
+    loss.backward()
+    d = logits.grad[0]
+
+    # (1) log-probs / entropy of sampled rows against the oracle's row arithmetic
+    idx = torch.arange(0, n, 997, device=dev)
+    # response == total: the reference's SFT convention, row t scores token t + 1 and the last row token 0
+    all_toks = torch.cat([torch.cat([t[1:], t.new_zeros(1)]) for t in toks])
+    xs = logits.detach()[0][idx].cpu()
+    rlp, rent = O.calculate_log_probs_and_entropy(xs, all_toks[idx].cpu(), None, with_entropy=True)
+    torch.testing.assert_close(lp_gpu[idx].cpu(), rlp.squeeze(-1), atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent_gpu[idx].cpu(), rent, atol=2e-3, rtol=0)
+
+    # (2) the oracle's composition on the [N] vectors: loss, metrics, d loss / d log-prob
+    from oracle import losses as L
+
+    lp_cpu = lp_gpu.cpu().double().requires_grad_()
+    lps = list(torch.split(lp_cpu, lengths))
+    olds = [o.double() for o in old]
+    adv = torch.cat([shaped[i].double().expand(ln) for i, ln in enumerate(lengths)])
+    dmasks = [m.double() for m in masks]
+    if estimator == "gspo":
+        ppo_kl = L.gspo_seq_kl(lps, olds, dmasks)
+        pg, clipfrac = L.policy_clip(ppo_kl, adv, args.eps_clip, args.eps_clip_high)
+    else:
+        ppo_kl = torch.cat(olds) - lp_cpu
+        pg, clipfrac = L.cispo(lp_cpu, ppo_kl, adv, args.eps_clip, args.eps_clip_high)
+    sample_mean = R.make_reducer(lengths, dmasks)
+    want_pg = R.seq_mean_token_sum(lengths, dmasks)(pg)
+    want_ent = sample_mean(ent_gpu.cpu().double())
+    want_loss = want_pg - args.entropy_coef * want_ent
+    want_loss.backward()
+    want = {"loss": want_loss, "pg_loss": want_pg, "entropy_loss": want_ent, "pg_clipfrac": sample_mean(clipfrac),
+            "ppo_kl": sample_mean(ppo_kl)}
+    want = {k: float(w.detach()) for k, w in want.items()}
+    assert set(met) == set(want)
+    for k, w in want.items():
+        assert abs(met[k].item() - w) < 2e-3 * max(1.0, abs(w)), (k, met[k].item(), w)
+    assert abs(loss.item() - want["loss"]) < 2e-3 * max(1.0, abs(want["loss"]))
+    if estimator == "gspo":  # the case exercises both sides of the clip
+        assert 0.0 < want["pg_clipfrac"] / 8 < 1.0
+    dlp = lp_cpu.grad.float()
+
+    # (3) sampled dlogits rows: dlp_t * (onehot(target) - softmax(row)); rows of masked tokens are exactly zero
+    p = torch.softmax(xs.float(), dim=-1)
+    hot = torch.zeros_like(p)
+    hot[torch.arange(idx.numel()), all_toks[idx].cpu()] = 1.0
+    want_rows = dlp[idx.cpu()][:, None] * (hot - p)
+    got_rows = d[idx].float().cpu()
+    torch.testing.assert_close(got_rows, want_rows, atol=2e-3, rtol=BF16_ULP)
+    assert want_rows.abs().max().item() > 1e-3  # the comparison is not of zeros
+    flat_mask = torch.cat(masks).to(dev)
+    for s0 in range(0, n, 8192):
+        e0 = min(n, s0 + 8192)
+        blk = d[s0:e0]
+        assert (blk[flat_mask[s0:e0] == 0] == 0).all()
+        assert blk.float().sum(-1).abs().max().item() < 5e-2
+    assert torch.isfinite(loss)
+
+
 def test_get_log_probs_and_entropy_topk_outputs_vs_oracle():
     """``gather_topk_token_ids`` (per-sample [R_i, K_i] ids, ragged K as on the union path, one sample without ids) and
     ``with_topk`` through the packed launch: values per sample, and the gradient of a loss that mixes the sampled-token
