@@ -387,14 +387,35 @@ def run_lmhead(a, dev) -> None:
          None)
 
 
+def load_ceilings():
+    """(library, check) of the benchmark's own measurement kernels, relax_amd/libceilings.so (built by
+    relax_amd/build.py next to the product library, which does not contain them)."""
+    import ctypes as C
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "relax_amd", "libceilings.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: run python relax_amd/build.py")
+    lib = C.CDLL(path)
+    lib.ceiling_mfma_loop.restype = C.c_int
+    lib.ceiling_mfma_loop.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    lib.ceiling_stream.restype = C.c_int
+    lib.ceiling_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
+
+    def check(rc):
+        if rc != 0:
+            raise RuntimeError(f"measurement kernel failed: code {rc}")
+
+    return lib, check
+
+
 def run_mfma_ceiling(a, dev) -> None:
     """Diagnostic, not a workload of the path: bf16 32x32x16 MFMAs on register-resident N(0, 1) operand fragments, one
     wave per SIMD on every CU, no memory traffic.  What this sustains under the board's power limit is the practical
     ceiling for the LM-head kernels on this box.  A "step" is one launch of 256 workgroups x 20000 iterations."""
     import ctypes as C
     from relax_amd import ops
-    from relax_amd._lib import check, lib
 
+    lib, check = load_ceilings()
     shape = 1 if a.mfma_shape == "16x16x32" else 0
     blocks, iters = 256, (10000 if shape else 20000)  # the same FLOP per launch for both shapes
     g = torch.Generator(device=dev).manual_seed(0)
@@ -406,7 +427,7 @@ def run_mfma_ceiling(a, dev) -> None:
 
     def step():
         with ops._timed("diag_mfma_loop"):
-            check(lib.relax_amd_diag_mfma_loop(C.c_void_p(src.data_ptr()), C.c_void_p(out.data_ptr()), blocks, iters,
+            check(lib.ceiling_mfma_loop(C.c_void_p(src.data_ptr()), C.c_void_p(out.data_ptr()), blocks, iters,
                                                shape, stream))
         return out
 
@@ -438,8 +459,8 @@ def run_hbm_ceiling(a, dev) -> None:
     bandwidth-bound kernels on this box.  A "step" is one read, one write and one copy launch."""
     import ctypes as C
     from relax_amd import ops
-    from relax_amd._lib import check, lib
 
+    lib, check = load_ceilings()
     nbytes = 65536 * 151936 * 2
     src = torch.ones(nbytes // 2, dtype=torch.bfloat16, device=dev)
     dst = torch.empty_like(src)
@@ -450,7 +471,7 @@ def run_hbm_ceiling(a, dev) -> None:
     def step():
         for mode, name in ((0, "diag_stream_read"), (1, "diag_stream_write"), (2, "diag_stream_copy")):
             with ops._timed(name):
-                check(lib.relax_amd_diag_stream(mode, p(src), p(dst), nbytes, p(sink), stream))
+                check(lib.ceiling_stream(mode, p(src), p(dst), nbytes, p(sink), stream))
         return dst
 
     wall, kernel_ms, launches, _ = timed_steps(step, a.warmup, a.steps)

@@ -472,23 +472,6 @@ int relax_amd_lmhead_dlogits_from_logits_t(void* logits_t, int64_t n_tokens, int
 int relax_amd_transpose_16bit(const void* in, int64_t rows, int64_t cols, int64_t in_stride, void* out,
                               int64_t out_stride, void* stream);
 
-/*
- * Measurement aid with no counterpart in the reference: `blocks` workgroups run `iters` iterations of independent bf16
- * MFMAs on operand fragments read once from src (4096 x 16 bytes of bf16), with no memory traffic.  shape 0: four waves
- * per workgroup (one per SIMD), 64 MFMAs 32x32x16 per wave and iteration = blocks * 4 * iters * 64 * 32768 FLOP;
- * shape 1: eight waves (two per SIMD), 128 MFMAs 16x16x32 per wave and iteration = blocks * 8 * iters * 128 * 16384
- * FLOP, i.e. twice the FLOP of shape 0 per iteration.  bench.py uses it to report what the matrix cores sustain on a
- * given box under its power limit.  out receives blocks * 512 floats (a checksum that keeps the loop alive).
- */
-int relax_amd_diag_mfma_loop(const void* src, float* out, int blocks, int iters, int shape, void* stream);
-
-/*
- * Measurement aid with no counterpart in the reference: one plain HBM stream over `bytes` (a multiple of 65536) with
- * 16-byte accesses.  mode 0 reads src (sink: 4 bytes of device memory, practically never written), mode 1 writes dst,
- * mode 2 copies src to dst.  bench.py uses it to report the box's streaming ceilings next to the bandwidth-bound kernels.
- */
-int relax_amd_diag_stream(int mode, const void* src, void* dst, int64_t bytes, void* sink, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -1,4 +1,6 @@
-// Measurement aids, not part of the loss path.
+// Measurement aids, not part of the loss path and not part of the product library: built into their own small
+// library (libceilings.so), which only the benchmark loads.  Entry points return 0, -1 for bad arguments, or the HIP
+// error code of a failed launch.
 //
 // (1) The matrix cores fed from registers, with no memory traffic at all.
 //
@@ -8,7 +10,6 @@
 // SIMD, operand fragments loaded once from `src` and rotated between the MFMAs so that consecutive instructions see
 // different operands, as they do in the LM-head kernels.
 #include "device_utils.h"
-#include "relax_amd.h"
 
 namespace relax_amd {
 
@@ -113,14 +114,12 @@ __global__ __launch_bounds__(1024) void diag_stream_kernel(const u32x4* __restri
 
 using namespace relax_amd;
 
-extern "C" int relax_amd_diag_stream(int mode, const void* src, void* dst, int64_t bytes, void* sink, void* stream) {
+extern "C" int ceiling_stream(int mode, const void* src, void* dst, int64_t bytes, void* sink, void* stream) {
   if (mode < 0 || mode > 2 || bytes < 0 || bytes % (16 * 4096) != 0 || (mode != 1 && !src) || (mode != 0 && !dst) ||
       (mode == 0 && !sink) || !aligned16(src) || !aligned16(dst)) {
-    set_error("diag_stream: mode 0 (read: src, sink) / 1 (write: dst) / 2 (copy: src, dst); bytes a multiple of 65536; "
-              "16-byte aligned buffers");
-    return RELAX_AMD_EINVAL;
+    return -1;
   }
-  if (bytes == 0) return RELAX_AMD_OK;
+  if (bytes == 0) return 0;
   const int64_t n = bytes / 16;
   const int64_t groups = n / 4096;
   const dim3 grid(unsigned(groups < 65536 ? groups : 65536)), block(1024);
@@ -133,14 +132,12 @@ extern "C" int relax_amd_diag_stream(int mode, const void* src, void* dst, int64
     hipLaunchKernelGGL(diag_stream_kernel<1>, grid, block, 0, s, in, out, n, static_cast<unsigned*>(sink));
   else
     hipLaunchKernelGGL(diag_stream_kernel<2>, grid, block, 0, s, in, out, n, static_cast<unsigned*>(sink));
-  return check_launch("diag_stream");
+  return int(hipGetLastError());
 }
 
-extern "C" int relax_amd_diag_mfma_loop(const void* src, float* out, int blocks, int iters, int shape, void* stream) {
+extern "C" int ceiling_mfma_loop(const void* src, float* out, int blocks, int iters, int shape, void* stream) {
   if (!src || !out || blocks <= 0 || iters < 0 || !aligned16(src) || (shape != 0 && shape != 1)) {
-    set_error("diag_mfma_loop: src (4096 x 16 bytes, 16-byte aligned), out (blocks x 512 floats) and shape 0 "
-              "(32x32x16, one wave per SIMD) or 1 (16x16x32, two waves per SIMD) are required");
-    return RELAX_AMD_EINVAL;
+    return -1;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (shape == 0)
@@ -149,5 +146,5 @@ extern "C" int relax_amd_diag_mfma_loop(const void* src, float* out, int blocks,
   else
     hipLaunchKernelGGL(diag_mfma_loop16_kernel, dim3(unsigned(blocks)), dim3(512), 0, s,
                        static_cast<const diag_bf16x8*>(src), out, iters);
-  return check_launch("diag_mfma_loop");
+  return int(hipGetLastError());
 }
