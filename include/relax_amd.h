@@ -441,6 +441,28 @@ int relax_amd_lmhead_dlogits_t(const void* hidden, const void* weight, int dtype
                                int64_t d_stride, void* stream);
 
 /*
+ * The two contractions of the gradient slab d_t [vocab, n_tokens] (bf16, token contiguous: what
+ * relax_amd_lmhead_dlogits_t / relax_amd_lmhead_dlogits_from_logits_t produce) that autograd through F.linear performs
+ * in the deferred-LM-head branch (relax/backends/megatron/loss.py:391-419, model.py:151-166), on the matrix cores:
+ *   relax_amd_lmhead_dhidden:  d_hidden[n, h] = sum_v d_t[v, n] * weight[v, h]
+ *   relax_amd_lmhead_dweight:  d_weight[v, h] = sum_n d_t[v, n] * hidden[n, h]
+ * Operands are read in the layouts they have (no transposed copies).  Reads past an operand's end are clamped and
+ * rely on zeros in d_t: d_t must be allocated with d_rows >= ceil128(vocab) rows of d_stride >= ceil128(n_tokens)
+ * elements, holding zeros in rows >= vocab and columns >= n_tokens up to those rounded sizes (the producers above
+ * never write there, so clearing the padding once after allocation is enough).  hidden_size and all row strides must
+ * be multiples of 8, bases 16-byte aligned.
+ *   out_mode  RELAX_AMD_GEMM_OUT_BF16: out is bf16; _F32: out is fp32; _F32_ACCUMULATE: out (fp32) += the product
+ *             (accumulation of d_weight over several slabs of tokens)
+ */
+enum { RELAX_AMD_GEMM_OUT_BF16 = 0, RELAX_AMD_GEMM_OUT_F32 = 1, RELAX_AMD_GEMM_OUT_F32_ACCUMULATE = 2 };
+int relax_amd_lmhead_dhidden(const void* d_t, int64_t d_rows, int64_t d_stride, const void* weight, int64_t w_stride,
+                             int64_t n_tokens, int64_t hidden_size, int64_t vocab, void* d_hidden, int64_t dh_stride,
+                             int out_mode, void* stream);
+int relax_amd_lmhead_dweight(const void* d_t, int64_t d_stride, const void* hidden, int64_t h_stride,
+                             int64_t n_tokens, int64_t hidden_size, int64_t vocab, void* d_weight, int64_t dw_stride,
+                             int out_mode, void* stream);
+
+/*
  * The same forward pass that also keeps the logits: logits_t [vocab, l_stride] bf16 (token contiguous, l_stride >=
  * n_tokens) receives bf16(hidden @ weight^T), and the softmax statistics and the target logit are taken from those
  * rounded values -- the reference's own numerics, whose F.linear runs in the weight dtype before .float()
@@ -462,15 +484,6 @@ int relax_amd_lmhead_dlogits_from_logits_t(void* logits_t, int64_t n_tokens, int
                                            const int64_t* targets, const float* lse, const float* spx,
                                            const float* g_lp, const float* g_ent, const float* grad_scale_dev,
                                            float inv_temperature, void* stream);
-
-/*
- * out[c, r] = in[r, c] for 16-bit elements (bf16 / fp16), row strides in elements.  The layout change
- * `x.t().contiguous()` makes; the LM-head backward uses it to give the library GEMMs of dhidden / dweight
- * contraction-contiguous operands (autograd of F.linear in relax/backends/megatron/loss.py:405 leaves the choice of
- * layout to the BLAS library).  16-byte accesses when the strides are multiples of 8 and the bases 16-byte aligned.
- */
-int relax_amd_transpose_16bit(const void* in, int64_t rows, int64_t cols, int64_t in_stride, void* out,
-                              int64_t out_stride, void* stream);
 
 #ifdef __cplusplus
 }

@@ -80,11 +80,12 @@ SIGNATURES = {
         C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _i64, _i64, _vp, _f32, _vp, _vp, _vp, _vp, _vp]),
     "relax_amd_lmhead_dlogits_t": (
         C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _vp]),
+    "relax_amd_lmhead_dhidden": (C.c_int, [_vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, C.c_int, _vp]),
+    "relax_amd_lmhead_dweight": (C.c_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, C.c_int, _vp]),
     "relax_amd_lmhead_logprob_fwd_keep": (
         C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _i64, _i64, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     "relax_amd_lmhead_dlogits_from_logits_t": (
         C.c_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp]),
-    "relax_amd_transpose_16bit": (C.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _vp]),
     "relax_amd_reverse_kl_bwd": (C.c_int, [_vp, _vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp]),
     "relax_amd_reinforce_pp_returns": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp, _i64, C.c_double, C.c_double, _vp, _vp]),
     "relax_amd_gae": (C.c_int, [_vp, _vp, C.c_int, _vp, _i64, C.c_double, C.c_double, _vp, _vp, _vp]),

@@ -93,23 +93,49 @@ def lmhead_dlogits_t(hidden, weight, targets, lse, spx, g_lp, g_ent, inv_tempera
     return out
 
 
-def transpose_16bit(x: torch.Tensor) -> torch.Tensor:
-    """``x.t().contiguous()`` for a 2-D bf16 / fp16 tensor with contiguous rows, through the tiled HIP kernel."""
-    if x.dim() != 2 or x.element_size() != 2 or x.stride(1) != 1:
-        raise ValueError(f"transpose_16bit needs a 2-D 16-bit tensor with contiguous rows, got {x.dtype} "
-                         f"{tuple(x.shape)} strides {x.stride()}")
-    _need_gpu(x)
-    out = torch.empty((x.size(1), x.size(0)), dtype=x.dtype, device=x.device)
-    check(lib.relax_amd_transpose_16bit(_p(x), x.size(0), x.size(1), x.stride(0), _p(out), out.stride(0), _stream()))
+def _ceil128(x: int) -> int:
+    return (x + 127) // 128 * 128
+
+
+def alloc_slab(vocab: int, n_tokens: int, device) -> torch.Tensor:
+    """The bf16 gradient slab ``[ceil128(vocab), ceil128(n_tokens)]`` the backward GEMMs read, with its padding rows
+    and columns cleared (the kernels that fill it never write there); ``slab[:vocab, :n_tokens]`` is the payload."""
+    slab = torch.empty((_ceil128(vocab), _ceil128(n_tokens)), dtype=torch.bfloat16, device=device)
+    if slab.size(0) > vocab:
+        slab[vocab:].zero_()
+    if slab.size(1) > n_tokens:
+        slab[:, n_tokens:].zero_()
+    return slab
+
+
+GEMM_OUT_BF16, GEMM_OUT_F32, GEMM_OUT_F32_ACCUMULATE = 0, 1, 2
+
+
+def _gemm_out(out: torch.Tensor, accumulate: bool) -> int:
+    if out.dtype == torch.bfloat16 and not accumulate:
+        return GEMM_OUT_BF16
+    if out.dtype == torch.float32:
+        return GEMM_OUT_F32_ACCUMULATE if accumulate else GEMM_OUT_F32
+    raise TypeError(f"output must be bfloat16, or float32 (required to accumulate), got {out.dtype}")
+
+
+def lmhead_dhidden(slab: torch.Tensor, n_tokens: int, weight: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out[n, h] = sum_v slab[v, n] * weight[v, h]`` on the matrix cores; ``slab`` as ``alloc_slab`` lays it out."""
+    v, h = weight.shape
+    with ops._timed("lmhead_dhidden_gemm"):
+        check(lib.relax_amd_lmhead_dhidden(_p(slab), slab.size(0), slab.stride(0), _p(weight), weight.stride(0),
+                                           n_tokens, h, v, _p(out), out.stride(0), _gemm_out(out, False), _stream()))
     return out
 
 
-def _k_contiguous(b: torch.Tensor) -> torch.Tensor:
-    """``b`` ([K, M], the right-hand operand of ``a @ b``) re-laid so that the contraction index is the contiguous one
-    (a transposed copy, returned as a [K, M] view of it).  The library GEMMs of these shapes measured 10 - 15 % faster
-    with both operands contraction-contiguous (dweight 30.6 -> 26.0 ms, dhidden 34.0 -> 30.5 ms at N = 32768,
-    V = 151936, H = 4096); the copy costs well under a millisecond."""
-    return transpose_16bit(b).t()
+def lmhead_dweight(slab: torch.Tensor, n_tokens: int, hidden: torch.Tensor, vocab: int, out: torch.Tensor,
+                   accumulate: bool = False) -> torch.Tensor:
+    """``out[v, h] (+)= sum_n slab[v, n] * hidden[n, h]`` on the matrix cores."""
+    with ops._timed("lmhead_dweight_gemm"):
+        check(lib.relax_amd_lmhead_dweight(_p(slab), slab.stride(0), _p(hidden), hidden.stride(0), n_tokens,
+                                           hidden.size(1), vocab, _p(out), out.stride(0), _gemm_out(out, accumulate),
+                                           _stream()))
+    return out
 
 
 class FusedLMHeadLogProb(torch.autograd.Function):
@@ -117,7 +143,8 @@ class FusedLMHeadLogProb(torch.autograd.Function):
 
     Backward recomputes the logits slab by slab on the matrix cores, emits d loss / d logits for the slab in bf16
     (never the full [N, V] tensor) and contracts it with the weight (dhidden) and the hidden states (dweight) with
-    plain library GEMMs; dweight is accumulated in fp32 across slabs.  With ``keep_logits`` the forward pass writes
+    the library's own matrix-core kernels, which read the slab, the weight and the hidden states in the layouts they
+    have; dweight is accumulated in fp32 across slabs.  With ``keep_logits`` the forward pass writes
     the bf16 logits, transposed, into the slab the backward pass needs anyway, and the backward pass turns them into
     the gradient in place instead of projecting again (one backward pass only: the slab is consumed).
     """
@@ -131,8 +158,9 @@ class FusedLMHeadLogProb(torch.autograd.Function):
         n, v = hidden.size(0), weight.size(0)
         ctx.logits_t = None
         if keep_logits and n > 0 and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]):
-            ctx.logits_t = torch.empty((v, (n + 7) // 8 * 8), dtype=torch.bfloat16, device=hidden.device)
-        lp, ent, lse, spx = lmhead_logprob_fwd(hidden, weight, targets, inv_temperature, with_entropy, ctx.logits_t)
+            ctx.logits_t = alloc_slab(v, n, hidden.device)
+        lp, ent, lse, spx = lmhead_logprob_fwd(hidden, weight, targets, inv_temperature, with_entropy,
+                                               None if ctx.logits_t is None else ctx.logits_t[:v])
         ctx.save_for_backward(hidden, weight, targets, lse, spx if with_entropy_grad else None)
         ctx.inv_temperature = inv_temperature
         ctx.with_entropy_grad = with_entropy_grad
@@ -156,41 +184,42 @@ class FusedLMHeadLogProb(torch.autograd.Function):
         v = weight.size(0)
         need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         d_hidden = torch.empty_like(hidden) if need_h else None
-        d_weight32 = None
+        if n == 0:  # an empty micro-batch: nothing flows back
+            return d_hidden, (torch.zeros_like(weight) if need_w else None), None, None, None, None, None
         if ctx.logits_t is not None:
             if ctx.logits_t is False:
                 raise RuntimeError("FusedLMHeadLogProb(keep_logits=True) supports one backward pass: the kept logits "
                                    "were overwritten with their gradient by the first one")
-            d_t = lmhead_dlogits_from_logits_t(ctx.logits_t, n, targets, lse, spx, g_lp, g_ent, ctx.inv_temperature)
+            slab = ctx.logits_t
+            lmhead_dlogits_from_logits_t(slab[:v], n, targets, lse, spx, g_lp, g_ent, ctx.inv_temperature)
+            if slab.size(1) > n:
+                slab[:, n:].zero_()  # the in-place kernel works on whole 16-byte vectors of tokens
             ctx.logits_t = False
             if need_h:
-                with ops._timed("lmhead_dhidden_gemm"):
-                    torch.mm(d_t.t(), _k_contiguous(weight), out=d_hidden)
-            d_weight = None
-            if need_w:
-                with ops._timed("lmhead_dweight_gemm"):
-                    d_weight = torch.mm(d_t, _k_contiguous(hidden))
+                lmhead_dhidden(slab, n, weight, d_hidden)
+            d_weight = lmhead_dweight(slab, n, hidden, v, torch.empty_like(weight)) if need_w else None
             return d_hidden, d_weight, None, None, None, None, None
-        weight_k = _k_contiguous(weight) if need_h else None
-        slab = torch.empty((v, min(n, BACKWARD_SLAB)), dtype=torch.bfloat16, device=hidden.device)
+        slab = alloc_slab(v, min(n, BACKWARD_SLAB), hidden.device)
+        single = n <= BACKWARD_SLAB
+        d_weight = None
+        if need_w:  # accumulated in fp32 when the micro-batch spans several slabs
+            d_weight = torch.empty_like(weight) if single else torch.empty(weight.shape, dtype=torch.float32,
+                                                                            device=weight.device)
         for s in range(0, n, BACKWARD_SLAB):
             e = min(n, s + BACKWARD_SLAB)
-            d_t = slab[:, : e - s]
+            cnt = e - s
+            if s > 0 and cnt < slab.size(1):
+                slab[:, cnt:_ceil128(cnt)].zero_()  # a shorter last slab: its padding columns hold the previous one
             lmhead_dlogits_t(hidden[s:e], weight, targets[s:e], lse[s:e], None if spx is None else spx[s:e],
-                             g_lp[s:e], None if g_ent is None else g_ent[s:e], ctx.inv_temperature, out=d_t)
+                             g_lp[s:e], None if g_ent is None else g_ent[s:e], ctx.inv_temperature,
+                             out=slab[:v, :cnt])
             if need_h:
-                with ops._timed("lmhead_dhidden_gemm"):
-                    torch.mm(d_t.t(), weight_k, out=d_hidden[s:e])
+                lmhead_dhidden(slab, cnt, weight, d_hidden[s:e])
             if need_w:
-                with ops._timed("lmhead_dweight_gemm"):
-                    part = torch.mm(d_t, _k_contiguous(hidden[s:e]))
-                if s == 0 and e == n:
-                    return d_hidden, part, None, None, None, None, None
-                if d_weight32 is None:
-                    d_weight32 = part.to(torch.float32)
-                else:
-                    d_weight32.add_(part)
-        return d_hidden, (d_weight32.to(weight.dtype) if need_w else None), None, None, None, None, None
+                lmhead_dweight(slab, cnt, hidden[s:e], v, d_weight, accumulate=s > 0)
+        if need_w and not single:
+            d_weight = d_weight.to(weight.dtype)
+        return d_hidden, d_weight, None, None, None, None, None
 
 
 def lm_head_log_probs_and_entropy(hidden, weight, tokens, temperature: float = 1.0, with_entropy: bool = False,

@@ -183,6 +183,86 @@ def test_kept_logits_slab_is_the_bf16_projection_and_stride_parity():
     torch.testing.assert_close(d_t.t().float().cpu(), want, atol=1e-5, rtol=2 * BF16_ULP)
 
 
+@pytest.mark.parametrize("n,h,v", [
+    (256, 256, 256),       # one tile, two k-slice pairs
+    (300, 128, 1000),      # ragged in every dimension, hidden size of half a tile
+    (777, 384, 1111),      # one and a half tiles of hidden units; odd extents
+    (1500, 512, 5000),     # several tiles either way
+    (64, 4096, 640),       # production hidden size, fewer tokens than one k-slice pair
+    (2048, 256, 8),        # a vocabulary shorter than one k-slice
+])
+def test_backward_gemms_vs_fp32_matmul(n, h, v):
+    """relax_amd_lmhead_dhidden / relax_amd_lmhead_dweight (the two contractions of the gradient slab autograd runs
+    through F.linear) against fp32 matmuls of the same bf16 operands: bf16 outputs to one rounding, fp32 outputs and
+    fp32 accumulation to accumulation-order noise."""
+    from relax_amd import lm_head as LM
+
+    dev = require_gpu()
+    announce("lmhead backward gemms", n, h, v)
+    g = torch.Generator().manual_seed(n + 3 * v)
+    hid = torch.randn(n, h, generator=g).bfloat16().to(dev)
+    w = (torch.randn(v, h, generator=g) * 0.5).bfloat16().to(dev)
+    d = (torch.randn(v, n, generator=g) * 0.25).bfloat16().to(dev)
+    slab = LM.alloc_slab(v, n, dev)
+    assert slab.shape == ((v + 127) // 128 * 128, (n + 127) // 128 * 128)
+    slab[:v, :n] = d
+    want_dh = d.float().t() @ w.float()
+    want_dw = d.float() @ hid.float()
+    # poisoned outputs: every element must be written, nothing beyond the valid extent
+    dh = torch.full((n + 3, h + 8), 7.0, dtype=torch.bfloat16, device=dev)
+    LM.lmhead_dhidden(slab, n, w, dh[:n, :h])
+    assert (dh[n:] == 7).all() and (dh[:, h:] == 7).all()
+    torch.testing.assert_close(dh[:n, :h].float(), want_dh, atol=1e-2 * want_dh.abs().max().item() * BF16_ULP,
+                               rtol=BF16_ULP)
+    dw = torch.full((v + 3, h + 8), 7.0, dtype=torch.bfloat16, device=dev)
+    LM.lmhead_dweight(slab, n, hid, v, dw[:v, :h])
+    assert (dw[v:] == 7).all() and (dw[:, h:] == 7).all()
+    torch.testing.assert_close(dw[:v, :h].float(), want_dw, atol=1e-2 * want_dw.abs().max().item() * BF16_ULP,
+                               rtol=BF16_ULP)
+    # fp32 output, then accumulation of a second product on top of it
+    dw32 = torch.full((v, h), float("nan"), dtype=torch.float32, device=dev)
+    LM.lmhead_dweight(slab, n, hid, v, dw32)
+    scale = max(1.0, want_dw.abs().max().item())
+    torch.testing.assert_close(dw32, want_dw, atol=2e-5 * scale, rtol=1e-5)
+    LM.lmhead_dweight(slab, n, hid, v, dw32, accumulate=True)
+    torch.testing.assert_close(dw32, 2 * want_dw, atol=4e-5 * scale, rtol=1e-5)
+    dh32 = torch.full((n, h), float("nan"), dtype=torch.float32, device=dev)
+    LM.lmhead_dhidden(slab, n, w, dh32)
+    torch.testing.assert_close(dh32, want_dh, atol=2e-5 * max(1.0, want_dh.abs().max().item()), rtol=1e-5)
+    # clamped reads are multiplied by the slab's zero padding: non-finite values next to the operands' ends in memory
+    # must not reach the result (the operands here are views into larger poisoned buffers)
+    big_w = torch.full((v + 130, h), float("nan"), dtype=torch.bfloat16, device=dev)
+    big_w[:v] = w
+    big_h = torch.full((n + 130, h), float("inf"), dtype=torch.bfloat16, device=dev)
+    big_h[:n] = hid
+    LM.lmhead_dhidden(slab, n, big_w[:v], dh32)
+    LM.lmhead_dweight(slab, n, big_h[:n], v, dw32)
+    assert torch.isfinite(dh32).all() and torch.isfinite(dw32).all()
+    torch.testing.assert_close(dw32, want_dw, atol=2e-5 * scale, rtol=1e-5)
+
+
+def test_backward_gemm_argument_errors():
+    from relax_amd import lm_head as LM
+    from relax_amd._lib import KernelError
+
+    dev = require_gpu()
+    announce("lmhead backward gemm errors")
+    w = torch.zeros(300, 128, dtype=torch.bfloat16, device=dev)
+    hid = torch.zeros(200, 128, dtype=torch.bfloat16, device=dev)
+    out_h = torch.zeros(200, 128, dtype=torch.bfloat16, device=dev)
+    out_w = torch.zeros(300, 128, dtype=torch.bfloat16, device=dev)
+    tight = torch.zeros(300, 200, dtype=torch.bfloat16, device=dev)  # neither rows nor columns padded to 128
+    with pytest.raises(KernelError, match="ceil128"):
+        LM.lmhead_dhidden(tight, 200, w, out_h)
+    with pytest.raises(KernelError, match="ceil128"):
+        LM.lmhead_dweight(tight, 200, hid, 300, out_w)
+    slab = LM.alloc_slab(300, 200, dev)
+    with pytest.raises(TypeError):
+        LM.lmhead_dweight(slab, 200, hid, 300, out_w, accumulate=True)  # accumulation needs an fp32 output
+    with pytest.raises(KernelError, match="ceil128"):
+        LM.lmhead_dhidden(slab[:300], 200, w, out_h)  # rows not padded
+
+
 def test_reference_shaped_case_temperature_and_labels():
     """Shape of the reference's own deferred-LM-head test (T=256, H=32, V=64, weight*0.02, temperature 0.7)."""
     from relax_amd.lm_head import lm_head_log_probs_and_entropy
@@ -322,28 +402,6 @@ def test_sft_losses_plain_and_with_deferred_lm_head_vs_oracle():
     assert abs(scaled.item() - want.item() * 2 / 3) < 2e-3 * len(resp) and logd["keys"] == ["loss"] and int(normalizer) == 1
     with pytest.raises(NotImplementedError, match="expose the LM-head weight"):
         relax_amd.sft_loss_function_chunked(args, dbatch, hd, None, lm_head_forward=lambda x: x)
-
-
-@pytest.mark.parametrize("rows,cols,row_pad", [
-    (64, 64, 0), (1000, 200, 0), (77, 4096, 0), (129, 65, 3), (8, 1, 0), (300, 301, 5), (4096, 1030, 8),
-])
-def test_transpose_16bit_is_exact(rows, cols, row_pad):
-    """Bit-exact against torch's own transposed copy, for ragged tiles and for row strides that rule out 16-byte
-    accesses on either side."""
-    from relax_amd.lm_head import transpose_16bit
-
-    dev = require_gpu()
-    announce("transpose", rows, cols, row_pad)
-    g = torch.Generator().manual_seed(rows * 7 + cols)
-    full = torch.randn(rows, cols + row_pad, generator=g).bfloat16().to(dev)
-    x = full[:, :cols]
-    got = transpose_16bit(x)
-    assert got.shape == (cols, rows) and got.is_contiguous()
-    assert torch.equal(got.view(torch.int16), x.t().contiguous().view(torch.int16))
-    with pytest.raises(ValueError):
-        transpose_16bit(x.t())
-    with pytest.raises(ValueError):
-        transpose_16bit(x.float())
 
 
 def test_model_forward_under_bypass_feeds_the_fused_loss_end_to_end():
