@@ -18,7 +18,10 @@
 // What bounds it: the board's power limit.  With every operand read served from cache the dhidden shape runs at
 // 0.63 - 0.65 of the published bf16 peak; streaming the operands from memory (60 GB per launch cross the L2 <-> fabric
 // boundary, the floor for 32 workgroups per XCD sharing 4 + 8 panels) costs both matrix-core cycles and clock and
-// leaves 0.54 - 0.57.
+// leaves 0.54 - 0.57.  The same loop on v_mfma_f32_16x16x32_bf16 (8 x 8 tiles per wave) was built and measured: the
+// clock rises from 1.5 - 1.65 to 1.9 - 2.1 GHz, but a single wave per SIMD cannot issue its fragment reads, copies and
+// address arithmetic between 16-cycle matrix instructions, the matrix cores idle a third of the time and the launch
+// takes longer (31.9 / 39.2 ms against 28.6 / 30.0 ms).
 //
 // Reads beyond an operand's extent are clamped to its last row / chunk, never out of bounds; the products stay exact
 // because d_t is zero-padded: the caller allocates it with ceil128(vocab) rows of ceil128(tokens) columns and zeros
