@@ -27,8 +27,6 @@
 // Workgroup -> (XCD, row block, vocab split) mapping: hardware places consecutive workgroup ids round-robin on the
 // 8 XCDs; the 32 workgroups resident on one XCD are arranged as (32/S) row blocks x S vocab splits so that hidden
 // tiles are shared by S workgroups and weight tiles by 32/S workgroups inside that XCD's L2.
-#include <cstdlib>
-#include <cstring>
 #include <mutex>
 
 #include "device_utils.h"
@@ -114,314 +112,6 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_fwd_kernel(const uint16_
   __syncthreads();
   const int64_t tok = tok0 + threadIdx.x;
   if (tok < g.n_tokens) {
-    const float* a = red + threadIdx.x * 3;
-    const float* b = red + (kLmTile + threadIdx.x) * 3;
-    const float mn = fmaxf(a[0], b[0]);
-    const float fa = fast_exp2(a[0] - mn), fb = fast_exp2(b[0] - mn);
-    float* o = partial + (int64_t(split) * g.n_tokens + tok) * 3;
-    o[0] = mn;
-    o[1] = a[1] * fa + b[1] * fb;
-    o[2] = a[2] * fa + b[2] * fb;
-  }
-}
-
-// ---------------------------------------------------------------------------------------------------------------
-// Forward pass without stored logits, second shape (opt-in): 512 threads = 8 wave64, two per SIMD, on
-// v_mfma_f32_16x16x32_bf16.  Same workgroup tile, LDS layout, copies and split / combine scheme as above; a wave owns
-// 128 vocab x 64 tokens (8 x 4 MFMA tiles of 16 x 16, 128 fp32 accumulators per lane, so two waves fit a SIMD's
-// register file).  Per flop the 16x16x32 instruction moves half the accumulator values of the 32x32x16 one and draws
-// less power, so under the board's power limit the clock settles higher (1.82 - 1.95 against 1.7 GHz); the eight waves
-// in turn keep the matrix cores busy in a smaller share of the cycles (76 % against 83 % by counters; 1.5 x the
-// fragment reads, twice the waves at every barrier), and measured end to end the two shapes take the same time.
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-constexpr int kLm16Threads = 512;
-constexpr int kLm16Passes = 4;  // 16-byte copies per thread per operand slice (64 rows per pass)
-
-// As LmCopier, for 512 threads: thread t covers row t/8 of each 64-row pass and LDS slot t%8.
-struct Lm16Copier {
-  const unsigned char* base;
-  uint32_t off0, off_last, pass_step;  // pass p reads at min(off0 + p * pass_step, off_last): two registers, not four
-
-  __device__ __forceinline__ void init(const uint16_t* matrix, int64_t stride, int64_t row0, int64_t row_limit) {
-    const int r = threadIdx.x >> 3, v = threadIdx.x & 7;
-    base = reinterpret_cast<const unsigned char*>(matrix + row0 * stride);
-    const int last = int(row_limit - row0);
-    const uint32_t col = uint32_t((v ^ ((r >> 1) & 7)) * 16);
-    off0 = uint32_t(min(r, last)) * uint32_t(stride * 2) + col;
-    off_last = uint32_t(last) * uint32_t(stride * 2) + col;
-    pass_step = 64u * uint32_t(stride * 2);
-  }
-  __device__ __forceinline__ void issue_pass(unsigned char* tile, int kslice, int p) const {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    uint64_t slice = reinterpret_cast<uint64_t>(base) + uint64_t(kslice) * (kLmBK * 2);
-    asm volatile("" : "+s"(slice));
-    uint32_t lane_off = min(off0 + uint32_t(p) * pass_step, off_last);
-    asm volatile("" : "+v"(lane_off));
-    const unsigned char* src = reinterpret_cast<const unsigned char*>(slice + uint64_t(lane_off));
-    unsigned char* dst = tile + (p * 64 + wave * 8) * (kLmBK * 2);  // wave-uniform; lane l lands at dst + 16*l
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src),
-                                     (__attribute__((address_space(3))) void*)(dst), 16, 0, 0);
-  }
-  __device__ __forceinline__ void issue(unsigned char* tile, int kslice) const {
-#pragma unroll
-    for (int p = 0; p < kLm16Passes; ++p) issue_pass(tile, kslice, p);
-  }
-};
-
-// Fragment of a 16-row sub-tile for 32-wide k-step `ks` (0 or 1): row (lane & 15), global vector 4*ks + (lane >> 4).
-__device__ __forceinline__ int lm16_frag_offset(int lane, int ks) {
-  const int row = lane & 15;
-  return row * (kLmBK * 2) + (((4 * ks + (lane >> 4)) ^ ((row >> 1) & 7)) * 16);
-}
-
-// A 32-wide k-step is multiplied in two quarters of the slice's 64 MFMAs: weight fragments 0..3 against the four
-// hidden fragments, then weight fragments 4..7 against the same four.  Two weight sets and two hidden sets are live
-// at a time (64 registers; whole k-steps double-buffered would take 96, and with 128 accumulators and two waves per
-// SIMD that spills into the loop).
-struct Lm16A {
-  bf16x8 a[4];
-};
-struct Lm16B {
-  bf16x8 b[4];
-};
-
-__device__ __forceinline__ void lm16_load_a(const LmStage& st, int lane, int ks, int half, int n, Lm16A& f) {
-  f.a[n] = *reinterpret_cast<const bf16x8*>(st.w + (half * 4 + n) * 16 * (kLmBK * 2) + lm16_frag_offset(lane, ks));
-}
-__device__ __forceinline__ void lm16_load_b(const LmStage& st, int lane, int ks, int n, Lm16B& f) {
-  f.b[n] = *reinterpret_cast<const bf16x8*>(st.h + n * 16 * (kLmBK * 2) + lm16_frag_offset(lane, ks));
-}
-
-// 16 MFMAs: weight fragments `fa` (rows 64 * HALF .. + 64 of the wave's 128) x hidden fragments `fb`; `between(n)` is
-// emitted right after MFMA n and pinned there.
-template <int HALF, typename Between>
-__device__ __forceinline__ void lm16_quarter(const Lm16A& fa, const Lm16B& fb, floatx4 (&acc)[8][4],
-                                             Between&& between) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      acc[HALF * 4 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa.a[i], fb.b[j], acc[HALF * 4 + i][j], 0, 0, 0);
-      between(i * 4 + j);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-}
-
-__device__ __forceinline__ void lm16_zero_acc(floatx4 (&acc)[8][4]) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
-}
-
-// Copies landed, fragment reads returned, then the workgroup barrier: the stage overwritten next is no longer read.
-__device__ __forceinline__ void lm16_slice_sync() {
-  __builtin_amdgcn_s_waitcnt(kLmWaitEverything);
-  __syncthreads();
-}
-
-// The registers of the pipeline: weight sets a0 / a1 and hidden sets b0 / b1.
-struct Lm16Regs {
-  Lm16A a0, a1;
-  Lm16B b0, b1;
-};
-
-// Quarters 0..2 of the slice in `st`.  On entry a0 / b0 hold (or are receiving) the low weight fragments and the
-// hidden fragments of k-step 0; on exit a1 / b1 hold the high weight fragments and the hidden fragments of k-step 1,
-// whose MFMAs are left to the caller (they run after the next barrier).  copy(4..7) are issued under quarter 0.
-template <typename Copy>
-__device__ __forceinline__ void lm16_slice_body(const LmStage& st, int lane, Lm16Regs& f, floatx4 (&acc)[8][4],
-                                                Copy&& copy) {
-  lm16_quarter<0>(f.a0, f.b0, acc, [&](int n) {
-    if (n < 4) lm16_load_a(st, lane, 0, 1, n, f.a1);
-    if ((n & 3) == 3) copy(4 + (n >> 2));
-  });
-  lm16_quarter<1>(f.a1, f.b0, acc, [&](int n) {
-    if (n < 4) lm16_load_a(st, lane, 1, 0, n, f.a0);
-    else if (n < 8) lm16_load_b(st, lane, 1, n - 4, f.b1);
-  });
-  lm16_quarter<0>(f.a0, f.b1, acc, [&](int n) {
-    if (n < 4) lm16_load_a(st, lane, 1, 1, n, f.a1);
-  });
-}
-
-// The previous slice's last quarter (a1 / b1) while the first fragments of the slice in `st` load into a0 / b0;
-// copy(0..3) are issued under it.
-template <typename Copy>
-__device__ __forceinline__ void lm16_slice_head(const LmStage& st, int lane, Lm16Regs& f, floatx4 (&acc)[8][4],
-                                                Copy&& copy) {
-  lm16_quarter<1>(f.a1, f.b1, acc, [&](int n) {
-    if (n < 4) lm16_load_a(st, lane, 0, 0, n, f.a0);
-    else if (n < 8) lm16_load_b(st, lane, 0, n - 4, f.b0);
-    if ((n & 3) == 3) copy(n >> 2);
-  });
-}
-
-// The 16x16x32 counterpart of lm_pipeline: same walk over (tile, k-slice), four quarters of 16 MFMAs per slice.
-template <typename Epilogue>
-__device__ __forceinline__ void lm16_pipeline(const LmLds lds, const uint16_t* hidden, const uint16_t* weight,
-                                              const LmGeom& g, int64_t tok0, int vt_begin, int vt_end,
-                                              Epilogue&& epilogue) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wv = wave >> 2, wt = wave & 3;
-  const int nk = int(g.hidden / kLmBK);  // even
-  const LmStage st0 = {lds.w0 + wv * 128 * (kLmBK * 2), lds.h0 + wt * 64 * (kLmBK * 2)};
-  const LmStage st1 = {lds.w1 + wv * 128 * (kLmBK * 2), lds.h1 + wt * 64 * (kLmBK * 2)};
-  Lm16Copier hc, wc;
-  hc.init(hidden, g.h_stride, tok0, g.n_tokens - 1);
-  floatx4 acc[8][4];
-  lm16_zero_acc(acc);
-  if (vt_begin >= vt_end) return;
-  wc.init(weight, g.w_stride, int64_t(vt_begin) * kLmTile, g.vocab - 1);
-  wc.issue(lds.w0, 0);
-  hc.issue(lds.h0, 0);
-  lm16_slice_sync();
-  Lm16Regs f;
-  for (int vt = vt_begin; vt < vt_end; ++vt) {
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_waitcnt(kLmWaitEverything);
-    __builtin_amdgcn_sched_barrier(0);
-    // slice 0 (stage 0): nothing to multiply yet, so its first fragments are waited for in the open
-#pragma unroll
-    for (int n = 0; n < 4; ++n) lm16_load_a(st0, lane, 0, 0, n, f.a0);
-#pragma unroll
-    for (int n = 0; n < 4; ++n) lm16_load_b(st0, lane, 0, n, f.b0);
-    wc.issue(lds.w1, 1);
-    hc.issue(lds.h1, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    lm16_slice_body(st0, lane, f, acc, [](int) {});
-    lm16_slice_sync();
-    for (int s = 1; s + 1 < nk; s += 2) {  // odd slices live in stage 1, even slices in stage 0
-      auto copy_to_0 = [&](int n) {
-        if (n < 4) {
-          wc.issue_pass(lds.w0, s + 1, n);
-        } else {
-          hc.issue_pass(lds.h0, s + 1, n - 4);
-        }
-      };
-      auto copy_to_1 = [&](int n) {
-        if (n < 4) {
-          wc.issue_pass(lds.w1, s + 2, n);
-        } else {
-          hc.issue_pass(lds.h1, s + 2, n - 4);
-        }
-      };
-      lm16_slice_head(st1, lane, f, acc, copy_to_0);
-      lm16_slice_body(st1, lane, f, acc, copy_to_0);
-      lm16_slice_sync();
-      lm16_slice_head(st0, lane, f, acc, copy_to_1);
-      lm16_slice_body(st0, lane, f, acc, copy_to_1);
-      lm16_slice_sync();
-    }
-    // last slice of the tile (stage 1); its copies fetch the next tile's first slice (after the last tile: this
-    // tile's first slice again, which nobody reads)
-    if (vt + 1 < vt_end) wc.init(weight, g.w_stride, int64_t(vt + 1) * kLmTile, g.vocab - 1);
-    auto copy_next_tile = [&](int n) {
-      if (n < 4) {
-        wc.issue_pass(lds.w0, 0, n);
-      } else {
-        hc.issue_pass(lds.h0, 0, n - 4);
-      }
-    };
-    lm16_slice_head(st1, lane, f, acc, copy_next_tile);
-    lm16_slice_body(st1, lane, f, acc, copy_next_tile);
-    lm16_quarter<1>(f.a1, f.b1, acc, [](int) {});
-    epilogue(acc, int64_t(vt) * kLmTile);
-    lm16_zero_acc(acc);
-    lm16_slice_sync();
-  }
-}
-
-// Online-softmax update of one token column with this lane's 32 logits of it (8 MFMA tiles x 4 registers): vocabulary
-// entry vbase + 16 * i + r of the workgroup's tile, `limit` = number of valid entries (masked variant only).
-template <bool MASKED>
-__device__ __forceinline__ void lm16_absorb_column(const floatx4 (&acc)[8][4], int j, int vbase, int limit, float c,
-                                                   float& m, float& s, float& t) {
-  float x[32];
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      x[i * 4 + r] = acc[i][j][r];
-      if (MASKED && vbase + 16 * i + r >= limit) x[i * 4 + r] = kNegHuge;
-    }
-  float vmax = x[0];
-#pragma unroll
-  for (int q = 1; q < 32; ++q) vmax = fmaxf(vmax, x[q]);
-  const float mc = fmaxf(vmax * c, kNegHuge);
-  if (mc > m) {
-    const float sc = fast_exp2(m - mc);
-    s *= sc;
-    t *= sc;
-    m = mc;
-  }
-#pragma unroll
-  for (int q = 0; q < 32; ++q) {
-    const float e = fast_exp2(fmaf(x[q], c, -m));
-    s += e;
-    t = fmaf(e, (MASKED && x[q] <= kNegHuge) ? 0.f : x[q], t);
-  }
-}
-
-__global__ __launch_bounds__(kLm16Threads, 1) void lmhead_fwd16_kernel(const uint16_t* __restrict__ hidden,
-                                                                       const uint16_t* __restrict__ weight, LmGeom g,
-                                                                       float c, float* __restrict__ partial) {
-  __shared__ __attribute__((aligned(1024))) unsigned char w0[kLmOperandBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char h0[kLmOperandBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char w1[kLmOperandBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char h1[kLmOperandBytes];
-  unsigned char* smem = w0;
-  int rb, split;
-  if (!lm_block_coords(g, rb, split)) return;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wv = wave >> 2, wt = wave & 3;
-  const int64_t tok0 = int64_t(rb) * kLmTile;
-  float m[4], s[4], t[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    m[j] = kNegHuge;
-    s[j] = 0.f;
-    t[j] = 0.f;
-  }
-  const int vt_begin = split * g.tiles_per_split;
-  const int vt_end = min(g.n_tiles, vt_begin + g.tiles_per_split);
-  lm16_pipeline(LmLds{w0, h0, w1, h1}, hidden, weight, g, tok0, vt_begin, vt_end,
-                [&](floatx4 (&acc)[8][4], int64_t v0) {
-                  const int limit = int(min<int64_t>(g.vocab - v0, kLmTile));
-                  const int vbase = wv * 128 + 4 * (lane >> 4);
-#pragma unroll
-                  for (int j = 0; j < 4; ++j) {
-                    if (limit < kLmTile)  // ragged last tile
-                      lm16_absorb_column<true>(acc, j, vbase, limit, c, m[j], s[j], t[j]);
-                    else
-                      lm16_absorb_column<false>(acc, j, 0, 0, c, m[j], s[j], t[j]);
-                    __builtin_amdgcn_sched_barrier(0);
-                  }
-                });
-  // merge the four lane groups (same tokens, different vocab rows), then the two waves sharing the tokens
-  float* red = reinterpret_cast<float*>(smem);  // [2 (wv)][256 tokens][3]
-  __syncthreads();
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-#pragma unroll
-    for (int d = 16; d <= 32; d *= 2) {
-      const float m2 = __shfl_xor(m[j], d, kWave), s2 = __shfl_xor(s[j], d, kWave), t2 = __shfl_xor(t[j], d, kWave);
-      const float mn = fmaxf(m[j], m2);
-      const float fa = fast_exp2(m[j] - mn), fb = fast_exp2(m2 - mn);
-      s[j] = s[j] * fa + s2 * fb;
-      t[j] = t[j] * fa + t2 * fb;
-      m[j] = mn;
-    }
-    if (lane < 16) {
-      float* o = red + (wv * kLmTile + wt * 64 + j * 16 + lane) * 3;
-      o[0] = m[j];
-      o[1] = s[j];
-      o[2] = t[j];
-    }
-  }
-  __syncthreads();
-  const int64_t tok = tok0 + threadIdx.x;
-  if (threadIdx.x < kLmTile && tok < g.n_tokens) {
     const float* a = red + threadIdx.x * 3;
     const float* b = red + (kLmTile + threadIdx.x) * 3;
     const float mn = fmaxf(a[0], b[0]);
@@ -706,14 +396,7 @@ static int lm_forward(const char* what, const void* hidden, const void* weight, 
     hipLaunchKernelGGL(lmhead_target_logit_kernel, dim3(unsigned((n_tokens + 3) / 4)), dim3(256), 0, s, h, w, g,
                        targets, x_target);
     if (int rc = check_launch("lmhead_target_logit")) return rc;
-    // RELAX_AMD_LMHEAD_FWD=mfma16 selects the 8-wave 16x16x32 shape (same results to rounding, same speed on
-    // random operands: it holds a higher clock under the power limit and leaves the matrix cores idle more often)
-    const char* shape = getenv("RELAX_AMD_LMHEAD_FWD");
-    if (shape && !strcmp(shape, "mfma16"))
-      hipLaunchKernelGGL(lmhead_fwd16_kernel, grid, dim3(kLm16Threads), 0, s, h, w, g, c, partial);
-    else
-      hipLaunchKernelGGL((lmhead_fwd_kernel<false, false>), grid, block, 0, s, h, w, g, c, partial, nullptr,
-                         int64_t(0));
+    hipLaunchKernelGGL((lmhead_fwd_kernel<false, false>), grid, block, 0, s, h, w, g, c, partial, nullptr, int64_t(0));
   } else if (lm_pairs_ok(l_t, l_stride)) {
     hipLaunchKernelGGL((lmhead_fwd_kernel<true, true>), grid, block, 0, s, h, w, g, c, partial, l_t, l_stride);
   } else {
