@@ -400,6 +400,8 @@ def load_ceilings():
     lib.ceiling_mfma_loop.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
     lib.ceiling_stream.restype = C.c_int
     lib.ceiling_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
+    lib.ceiling_row_copy.restype = C.c_int
+    lib.ceiling_row_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_void_p]
 
     def check(rc):
         if rc != 0:
@@ -472,17 +474,24 @@ def run_hbm_ceiling(a, dev) -> None:
         for mode, name in ((0, "diag_stream_read"), (1, "diag_stream_write"), (2, "diag_stream_copy")):
             with ops._timed(name):
                 check(lib.ceiling_stream(mode, p(src), p(dst), nbytes, p(sink), stream))
+        with ops._timed("diag_row_copy"):  # the same copy, one persistent workgroup per CU walking whole rows
+            check(lib.ceiling_row_copy(p(src), p(dst), 65536, 151936 * 2, 256, stream))
+        with ops._timed("memset"):
+            dst.view(torch.int32).zero_()
         return dst
 
     wall, kernel_ms, launches, _ = timed_steps(step, a.warmup, a.steps)
     rates = {"read_GBs": nbytes / kernel_ms["diag_stream_read"] / 1e6,
              "write_GBs": nbytes / kernel_ms["diag_stream_write"] / 1e6,
-             "copy_GBs": 2 * nbytes / kernel_ms["diag_stream_copy"] / 1e6}
+             "copy_GBs": 2 * nbytes / kernel_ms["diag_stream_copy"] / 1e6,
+             "row_copy_GBs": 2 * nbytes / kernel_ms["diag_row_copy"] / 1e6,
+             "torch_zero_fill_GBs": nbytes / kernel_ms["memset"] / 1e6}
     print(json.dumps({
         "metric": "GB/s of plain HBM streams [diagnostic ceiling, not the headline metric]", "value": rates["read_GBs"],
         "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": wall * 1e3 / a.steps,
         "higher_is_better": True, "dtype": "u8", "data": "synthetic",
-        "config": {"workload": "hbm_ceiling: read, write and copy of 19.9 GB with 16-byte accesses", **rates},
+        "config": {"workload": "hbm_ceiling: read, write, copy, row-wise copy (65536 rows of 303872 bytes, 256 persistent "
+                               "workgroups) and zero fill of 19.9 GB with 16-byte accesses", **rates},
         "roofline": {"bound": "hbm", "kernel": "diag_stream_kernel<0> (read)", "achieved": rates["read_GBs"],
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": rates["read_GBs"] / HBM_PEAK_GBS, "traffic": None,
                      "kernel_ms": kernel_ms},
