@@ -522,8 +522,11 @@ def run_actor_fwd_topk(a, dev) -> None:
 
     wall, kernel_ms, _, _ = timed_steps(step, a.warmup, a.steps)
     row_bytes = float(a.vocab * logits.element_size()) * n_tokens
-    if "topk_rows" in kernel_ms:
-        # the selection reads every row (the second look at a row is served by the caches in part)
+    if "logprob_entropy_topk_fwd" in kernel_ms:
+        # one read of every row serves the softmax scan and the selection (whose second, sparse look finds the row
+        # in cache)
+        dom, dom_name = kernel_ms["logprob_entropy_topk_fwd"], "logprob_topk_fwd_kernel<bf16_t>"
+    elif "topk_rows" in kernel_ms:
         dom, dom_name = kernel_ms["topk_rows"], "topk_rows_fast_kernel<bf16_t, true>"
     else:
         dom, dom_name = kernel_ms["logprob_entropy_fwd"], "logprob_entropy_fwd_kernel<bf16_t, true, 1024>"

@@ -367,6 +367,19 @@ int relax_amd_topk_rows(const void* logits, int dtype, int64_t n_tokens, int64_t
                         void* stream);
 
 /*
+ * relax_amd_logprob_entropy_fwd and relax_amd_topk_rows over the same response rows from one read of the logits: what
+ * get_log_probs_and_entropy(..., with_topk=True) computes per sample (relax/backends/megatron/loss.py:373-446: the
+ * log-probs / entropy of the response tokens and torch.topk of the same logits rows).  Arguments as in those two
+ * functions; log_prob / entropy / lse / spx are bit-identical to relax_amd_logprob_entropy_fwd's, values / indices
+ * follow relax_amd_topk_rows' contract (the selection does not depend on the temperature).  Rows that are not whole
+ * 16-byte vectors in groups of eight, or shorter than 8192 vectors, run the two passes one after the other.
+ */
+int relax_amd_logprob_entropy_topk_fwd(const void* logits, int dtype, int64_t n_tokens, int64_t vocab,
+                                       int64_t row_stride, const int32_t* row_ids, const int64_t* targets,
+                                       float inv_temperature, int k, float* log_prob, float* entropy, float* lse,
+                                       float* spx, float* values, int64_t* indices, uint8_t* workspace, void* stream);
+
+/*
  * Fused actor step: log-prob + entropy forward, the per-token terms of relax_amd_policy_loss and the dlogits backward
  * in one launch.  Each workgroup scans its row, derives the token's gradient constants and immediately walks the row
  * again to emit dlogits; the second walk is served by the L2 / memory-side cache, so HBM sees one read and one write

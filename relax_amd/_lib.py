@@ -99,6 +99,8 @@ SIGNATURES = {
     "relax_amd_sparse_row_add": (
         C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _f32, _vp]),
     "relax_amd_topk_rows": (C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, C.c_int, _vp, _vp, _vp, _vp]),
+    "relax_amd_logprob_entropy_topk_fwd": (
+        C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _f32, C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "relax_amd_topk_logprob_fwd": (
         C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _i64, _f32, _vp, _vp, _vp, _vp]),
     "relax_amd_topk_logprob_bwd": (

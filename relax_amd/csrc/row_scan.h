@@ -15,8 +15,9 @@ struct SoftmaxAcc {
   float m, s, t;  // max of x*c, sum exp2(x*c - m), sum exp2(x*c - m) * x     (c = log2(e) / temperature)
 };
 
+// Returns the largest of the K values (a float maximum: NaN passes unnoticed here and shows in st.s instead).
 template <int K>
-__device__ __forceinline__ void scan_absorb(const float (&v)[K], float c, SoftmaxAcc& st) {
+__device__ __forceinline__ float scan_absorb(const float (&v)[K], float c, SoftmaxAcc& st) {
   float vmax = v[0];
 #pragma unroll
   for (int i = 1; i < K; ++i) vmax = fmaxf(vmax, v[i]);
@@ -33,6 +34,7 @@ __device__ __forceinline__ void scan_absorb(const float (&v)[K], float c, Softma
     st.s = __fadd_rn(st.s, e);
     st.t = fmaf(e, v[i], st.t);
   }
+  return vmax;
 }
 
 __device__ __forceinline__ void scan_merge(SoftmaxAcc& a, float m2, float s2, float t2) {
@@ -43,11 +45,18 @@ __device__ __forceinline__ void scan_merge(SoftmaxAcc& a, float m2, float s2, fl
   a.m = mn;
 }
 
+// Optional observer of the scan: is told the largest value of every batch of elements a lane absorbs (kScanUnroll
+// vectors at a stride of THREADS vectors while that many remain, then single vectors, then single tail elements), in
+// the order scan_row() takes them, without touching the softmax arithmetic or its order.
+struct ScanNoHook {
+  __device__ __forceinline__ void absorbed(float) const {}
+};
+
 // Per-lane state over one row.  VEC: 16-byte loads (row base and stride 16-byte aligned) for the whole vectors and
 // scalar loads for the tail; otherwise scalar loads throughout.  STREAM selects non-temporal loads (row not needed
 // again soon) or ordinary cached loads (a second pass over the row follows immediately); it does not change results.
-template <typename T, bool VEC, bool STREAM, int THREADS>
-__device__ __forceinline__ SoftmaxAcc scan_row(const T* __restrict__ x, int64_t vocab, float c) {
+template <typename T, bool VEC, bool STREAM, int THREADS, typename Hook = ScanNoHook>
+__device__ __forceinline__ SoftmaxAcc scan_row(const T* __restrict__ x, int64_t vocab, float c, Hook&& hook = Hook()) {
   SoftmaxAcc st{kNegHuge, 0.f, 0.f};
   if (VEC) {
     constexpr int VN = Row<T>::kPerVec;
@@ -67,21 +76,21 @@ __device__ __forceinline__ SoftmaxAcc scan_row(const T* __restrict__ x, int64_t 
 #pragma unroll
         for (int k = 0; k < VN; ++k) v[u * VN + k] = part[k];
       }
-      scan_absorb(v, c, st);
+      hook.absorbed(scan_absorb(v, c, st));
     }
     for (; i < nvec; i += THREADS) {
       float v[VN];
       Row<T>::unpack(STREAM ? load_stream(xv + i) : xv[i], v);
-      scan_absorb(v, c, st);
+      hook.absorbed(scan_absorb(v, c, st));
     }
     for (int64_t e = nvec * VN + threadIdx.x; e < vocab; e += THREADS) {
       float v[1] = {Row<T>::load1(x + e)};
-      scan_absorb(v, c, st);
+      hook.absorbed(scan_absorb(v, c, st));
     }
   } else {
     for (int64_t e = threadIdx.x; e < vocab; e += THREADS) {
       float v[1] = {Row<T>::load1(x + e)};
-      scan_absorb(v, c, st);
+      hook.absorbed(scan_absorb(v, c, st));
     }
   }
   return st;

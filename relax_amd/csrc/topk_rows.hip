@@ -21,6 +21,7 @@
 // values at the threshold is taken is unspecified in torch as well -- here the list order decides.
 #include "device_utils.h"
 #include "relax_amd.h"
+#include "row_scan.h"
 
 namespace relax_amd {
 
@@ -172,6 +173,44 @@ __device__ __forceinline__ void tk_sort_emit(uint64_t* list, uint32_t len, uint3
 constexpr int kTkFastList = 2048;
 constexpr int kTkFastBatch = 6;  // loads in flight per thread within 64 registers (two workgroups per CU)
 constexpr int kTkGroups = 8192;  // groups of eight vectors the shortcut keeps a maximum for (vocab <= 524288 at 16 bit)
+// The shortcut's bound, shared by the selection kernel and the fused log-prob + selection kernel: `best` is each
+// thread's largest key.  Returns, as a float, the lower end of the 12-bit bin that holds the k-th largest of the thread
+// maxima (at most the 1024-th): !(v < bound) holds for every value whose key is at or above that bin (and for NaN, and
+// for -0 against a bound of +0: a few candidates more never hurt).  Clears *count for the collection that follows.
+__device__ __forceinline__ float tk_fast_floor(uint32_t best, int k, uint32_t* tot, uint32_t* wave_part,
+                                               uint32_t* found, uint32_t* count) {
+  const int tid = threadIdx.x;
+  for (int d = tid; d < kTkBins; d += kTkThreads) tot[d] = 0u;
+  if (tid == 0) *count = 0u;
+  __syncthreads();
+  atomicAdd(&tot[best >> (32 - kTkDigitBits)], 1u);
+  __syncthreads();
+  tk_locate(tot, wave_part, found, uint32_t(k) < uint32_t(kTkThreads) ? uint32_t(k) : uint32_t(kTkThreads));
+  return tk_value(found[0] << (32 - kTkDigitBits));
+}
+
+// One candidate of the shortcut's second look: kept when it is not below the bound.
+__device__ __forceinline__ void tk_fast_consider(uint32_t idx, float v, float floor_value, uint64_t* list,
+                                                 uint32_t* count) {
+  if (!(v < floor_value)) {
+    const uint32_t key = tk_key(v);
+    const uint32_t slot = atomicAdd(count, 1u);
+    if (slot < uint32_t(kTkFastList)) list[slot] = (uint64_t(key) << 32) | uint64_t(0xFFFFFFFFu - idx);
+  }
+}
+
+// After the second look: ranks the candidates and emits the first k, or flags the row for the general kernel when the
+// candidates did not fit the list.
+__device__ __forceinline__ void tk_fast_finish(uint64_t* list, const uint32_t* count, int k, int64_t tok,
+                                               float* __restrict__ out_values, int64_t* __restrict__ out_indices,
+                                               uint8_t* __restrict__ needs_general, uint32_t* rank) {
+  __syncthreads();
+  const uint32_t len = *count;
+  if (threadIdx.x == 0) needs_general[tok] = len > uint32_t(kTkFastList) ? 1 : 0;
+  if (len > uint32_t(kTkFastList)) return;  // the whole workgroup
+  tk_sort_emit(list, len, kTkFastList, k, tok, out_values, out_indices, rank);
+}
+
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kTkThreads, 8) void topk_rows_fast_kernel(const T* __restrict__ logits, int64_t stride,
                                                                     int64_t vocab, const int32_t* __restrict__ row_ids,
@@ -250,23 +289,9 @@ __global__ __launch_bounds__(kTkThreads, 8) void topk_rows_fast_kernel(const T* 
       best = key > best ? key : best;
     });
   }
-  for (int d = tid; d < kTkBins; d += kTkThreads) tot[d] = 0u;
-  if (tid == 0) count = 0u;
-  __syncthreads();
-  atomicAdd(&tot[best >> (32 - kTkDigitBits)], 1u);
-  __syncthreads();
-  tk_locate(tot, wave_part, found, uint32_t(k) < uint32_t(kTkThreads) ? uint32_t(k) : uint32_t(kTkThreads));
+  const float floor_value = tk_fast_floor(best, k, tot, wave_part, found, &count);
   const uint32_t floor_key = found[0] << (32 - kTkDigitBits);
-  // as a float comparison: !(v < bound) holds for every value whose key is >= floor_key (and for NaN, and for -0
-  // against a bound of +0: a few candidates more never hurt)
-  const float floor_value = tk_value(floor_key);
-  auto consider = [&](uint32_t idx, float v) {
-    if (!(v < floor_value)) {
-      const uint32_t key = tk_key(v);
-      const uint32_t slot = atomicAdd(&count, 1u);
-      if (slot < uint32_t(kTkFastList)) list[slot] = (uint64_t(key) << 32) | uint64_t(0xFFFFFFFFu - idx);
-    }
-  };
+  auto consider = [&](uint32_t idx, float v) { tk_fast_consider(idx, v, floor_value, list, &count); };
   if (by_group) {
     const u32x4* xv = reinterpret_cast<const u32x4*>(x);
     for (int64_t i0 = tid; i0 < nvec; i0 += int64_t(kTkFastBatch) * kTkThreads) {
@@ -292,11 +317,102 @@ __global__ __launch_bounds__(kTkThreads, 8) void topk_rows_fast_kernel(const T* 
   } else {
     tk_for_each<T, VEC, true>(x, vocab, consider);
   }
+  tk_fast_finish(list, &count, k, tok, out_values, out_indices, needs_general, rank);
+}
+
+// Log-prob + entropy and the top-K ids of a row from ONE read of it (the forward-only pass of an actor that also
+// collects its top-K ids, relax/backends/megatron/loss.py:373-446): the softmax scan is scan_row() itself, same
+// workgroup width and order as the forward-only kernel, so log-probs and entropy are bit-identical to that kernel's.
+// The scan already takes the maximum of every batch of elements a lane absorbs (it rescales its sums by it); its
+// observer keeps those maxima, one LDS word per lane and batch, and nothing else is added to the scan.  A lane's
+// largest is its thread maximum for the shortcut's bound, and the second look is lane-private: each lane walks its own
+// batches in the scan's order and reads again only those whose maximum reaches the bound (a few per cent of the row,
+// found in cache).  A row that holds NaN or +inf (its sum of exponentials is NaN) goes to the general kernel.
+// Built for rows of whole 16-byte vectors whose length selects the 1024-thread scan.
+constexpr int kTkScanSlots = 12;  // batches a lane may absorb: vocab / (kScanUnroll * 1024 * elements per vector) + 3
+
+struct TkScanHook {
+  float* slot;  // this lane's word of the next batch
+  float best;
+  __device__ __forceinline__ void absorbed(float vmax) {
+    *slot = vmax;
+    slot += kTkThreads;
+    best = fmaxf(best, vmax);
+  }
+};
+
+template <typename T>
+__global__ __launch_bounds__(kTkThreads, 8) void logprob_topk_fwd_kernel(
+    const T* __restrict__ logits, int64_t stride, int64_t vocab, const int32_t* __restrict__ row_ids,
+    const int64_t* __restrict__ targets, float c, float inv_t, int k, float* __restrict__ log_prob,
+    float* __restrict__ entropy, float* __restrict__ lse_out, float* __restrict__ spx_out,
+    float* __restrict__ out_values, int64_t* __restrict__ out_indices, uint8_t* __restrict__ needs_general) {
+  __shared__ uint64_t list[kTkFastList];  // the bound's histogram lives here before the candidates do
+  __shared__ float lane_max[kTkScanSlots * kTkThreads];
+  __shared__ uint32_t rank[kTkRankMax];
+  __shared__ uint32_t wave_part[kTkWaves];
+  __shared__ uint32_t found[3];
+  __shared__ uint32_t count;
+  __shared__ uint32_t odd_row;
+  __shared__ float wave_state[kTkWaves][3];
+  static_assert(sizeof(list) == sizeof(uint32_t) * kTkBins, "the histogram of the thread maxima fits the list");
+  uint32_t* tot = reinterpret_cast<uint32_t*>(list);
+  const int tid = threadIdx.x;
+  const int64_t tok = blockIdx.x;
+  const int64_t row = row_ids ? int64_t(row_ids[tok]) : tok;
+  const T* x = logits + row * stride;
+  constexpr int VN = Row<T>::kPerVec;
+  const int64_t nvec = vocab / VN;
+  float x_target = 0.f;
+  int64_t tg = -1;
+  if (tid == 0) {
+    tg = targets[tok];
+    if (tg >= 0 && tg < vocab) x_target = Row<T>::load1(x + tg);
+  }
+  TkScanHook hook{lane_max + tid, -__builtin_inff()};
+  SoftmaxAcc st = scan_row<T, true, false, kTkThreads>(x, vocab, c, hook);
+  scan_block_merge<kTkThreads>(st, wave_state);
+  if (tid == 0) {
+    float lse, spx, ent, lp;
+    scan_finish(st, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
+    log_prob[tok] = lp;
+    if (entropy) entropy[tok] = ent;
+    if (spx_out) spx_out[tok] = spx;
+    if (lse_out) lse_out[tok] = lse;
+    odd_row = st.s != st.s ? 1u : 0u;
+  }
   __syncthreads();
-  const uint32_t len = count;
-  if (tid == 0) needs_general[tok] = len > uint32_t(kTkFastList) ? 1 : 0;
-  if (len > uint32_t(kTkFastList)) return;  // the whole workgroup
-  tk_sort_emit(list, len, kTkFastList, k, tok, out_values, out_indices, rank);
+  if (odd_row) {  // the whole workgroup
+    if (tid == 0) needs_general[tok] = 1;
+    return;
+  }
+  const float floor_value = tk_fast_floor(tk_key(hook.best), k, tot, wave_part, found, &count);
+  // (tk_fast_floor ends with a barrier after the last reading of tot[]: the list may now overwrite it)
+  const u32x4* xv = reinterpret_cast<const u32x4*>(x);
+  const float* mine = lane_max + tid;
+  int64_t i = tid;
+  for (; i + int64_t(kScanUnroll - 1) * kTkThreads < nvec; i += int64_t(kScanUnroll) * kTkThreads, mine += kTkThreads) {
+    if (*mine < floor_value) continue;
+    u32x4 raw[kScanUnroll];
+#pragma unroll
+    for (int u = 0; u < kScanUnroll; ++u) raw[u] = load_stream(xv + i + int64_t(u) * kTkThreads);
+#pragma unroll
+    for (int u = 0; u < kScanUnroll; ++u) {
+      float v[VN];
+      Row<T>::unpack(raw[u], v);
+#pragma unroll
+      for (int e = 0; e < VN; ++e)
+        tk_fast_consider(uint32_t((i + int64_t(u) * kTkThreads) * VN + e), v[e], floor_value, list, &count);
+    }
+  }
+  for (; i < nvec; i += kTkThreads, mine += kTkThreads) {
+    if (*mine < floor_value) continue;
+    float v[VN];
+    Row<T>::unpack(load_stream(xv + i), v);
+#pragma unroll
+    for (int e = 0; e < VN; ++e) tk_fast_consider(uint32_t(i * VN + e), v[e], floor_value, list, &count);
+  }
+  tk_fast_finish(list, &count, k, tok, out_values, out_indices, needs_general, rank);
 }
 
 // The general way, for the rows the shortcut flagged (long runs of equal or nearly equal values): radix select, 12
@@ -432,5 +548,75 @@ extern "C" int relax_amd_topk_rows(const void* logits, int dtype, int64_t n_toke
     case RELAX_AMD_BF16: return launch_topk_rows<bf16_t>(logits, n_tokens, vocab, row_stride, row_ids, k, values, indices, workspace, s);
     case RELAX_AMD_F16: return launch_topk_rows<f16_t>(logits, n_tokens, vocab, row_stride, row_ids, k, values, indices, workspace, s);
     default: set_error("topk_rows: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
+  }
+}
+
+template <typename T>
+static bool topk_fusable(const void* logits, int64_t vocab, int64_t stride) {
+  constexpr int per_vec = 16 / int(sizeof(T));
+  const int64_t nvec = vocab / per_vec;
+  return aligned16(logits) && (stride * int64_t(sizeof(T))) % 16 == 0 && vocab % per_vec == 0 &&
+         nvec / (int64_t(kScanUnroll) * kTkThreads) + 3 <= kTkScanSlots && scan_threads(vocab, per_vec) == kTkThreads;
+}
+
+template <typename T>
+static int launch_logprob_topk(const void* logits, int64_t n_tokens, int64_t vocab, int64_t stride,
+                               const int32_t* row_ids, const int64_t* targets, float inv_t, int k, float* log_prob,
+                               float* entropy, float* lse, float* spx, float* values, int64_t* indices, uint8_t* flags,
+                               hipStream_t s) {
+  const T* x = static_cast<const T*>(logits);
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  hipLaunchKernelGGL((logprob_topk_fwd_kernel<T>), dim3(static_cast<unsigned>(n_tokens)), dim3(kTkThreads), 0, s, x,
+                     stride, vocab, row_ids, targets, inv_t * kLog2e, inv_t, k, log_prob, entropy, lse, spx, values,
+                     indices, flags);
+  if (int rc = check_launch("logprob_topk_fwd")) return rc;
+  hipLaunchKernelGGL((topk_rows_kernel<T, true>), dim3(static_cast<unsigned>(n_tokens < cus ? n_tokens : cus)),
+                     dim3(kTkThreads), 0, s, x, stride, vocab, row_ids, n_tokens, k, values, indices, flags);
+  return check_launch("topk_rows");
+}
+
+extern "C" int relax_amd_logprob_entropy_topk_fwd(const void* logits, int dtype, int64_t n_tokens, int64_t vocab,
+                                                  int64_t row_stride, const int32_t* row_ids, const int64_t* targets,
+                                                  float inv_temperature, int k, float* log_prob, float* entropy,
+                                                  float* lse, float* spx, float* values, int64_t* indices,
+                                                  uint8_t* workspace, void* stream) {
+  if (n_tokens == 0) return RELAX_AMD_OK;
+  if (n_tokens < 0 || n_tokens > 0x7FFFFFFFLL || vocab <= 0 || row_stride < vocab || !logits || !targets ||
+      !log_prob || !indices || !workspace || k < 1 || k > vocab || !(inv_temperature > 0.f)) {
+    set_error("logprob_entropy_topk_fwd: NULL argument, bad size, k outside [1, vocab] or non-positive inv_temperature");
+    return RELAX_AMD_EINVAL;
+  }
+  if (k > kTkMaxK || vocab > 1000000) {
+    set_error("logprob_entropy_topk_fwd: k > %d or vocab > 1000000 is not built", kTkMaxK);
+    return RELAX_AMD_EUNSUPPORTED;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  bool fused = false;
+  switch (dtype) {
+    case RELAX_AMD_F32: fused = topk_fusable<float>(logits, vocab, row_stride); break;
+    case RELAX_AMD_BF16: fused = topk_fusable<bf16_t>(logits, vocab, row_stride); break;
+    case RELAX_AMD_F16: fused = topk_fusable<f16_t>(logits, vocab, row_stride); break;
+    default: set_error("logprob_entropy_topk_fwd: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
+  }
+  if (!fused) {  // other row shapes: the two passes one after the other, same results
+    if (int rc = relax_amd_logprob_entropy_fwd(logits, dtype, n_tokens, vocab, row_stride, row_ids, targets,
+                                               inv_temperature, log_prob, entropy, lse, spx, stream))
+      return rc;
+    return relax_amd_topk_rows(logits, dtype, n_tokens, vocab, row_stride, row_ids, k, values, indices, workspace,
+                               stream);
+  }
+  switch (dtype) {
+    case RELAX_AMD_F32:
+      return launch_logprob_topk<float>(logits, n_tokens, vocab, row_stride, row_ids, targets, inv_temperature, k,
+                                        log_prob, entropy, lse, spx, values, indices, workspace, s);
+    case RELAX_AMD_BF16:
+      return launch_logprob_topk<bf16_t>(logits, n_tokens, vocab, row_stride, row_ids, targets, inv_temperature, k,
+                                         log_prob, entropy, lse, spx, values, indices, workspace, s);
+    default:
+      return launch_logprob_topk<f16_t>(logits, n_tokens, vocab, row_stride, row_ids, targets, inv_temperature, k,
+                                        log_prob, entropy, lse, spx, values, indices, workspace, s);
   }
 }

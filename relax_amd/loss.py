@@ -154,6 +154,7 @@ def get_log_probs_and_entropy(
     """One packed launch over every response token; returns ``(empty, {"log_probs": [...], "entropy": [...]})``
     with per-sample ``[R_i]`` fp32 views, differentiable w.r.t. ``logits``."""
     assert non_loss_data
+    topk_k_arg = topk_k
     if lm_head_forward is not None:
         return _deferred_lm_head_log_probs(logits, args, unconcat_tokens, total_lengths, response_lengths,
                                            with_entropy, lm_head_forward, max_seq_lens)
@@ -164,9 +165,19 @@ def get_log_probs_and_entropy(
                        _padded_starts(args, max_seq_lens))
     inv_t = 1.0 / float(getattr(args, "rollout_temperature", 1.0))
     lse = None
+    topk_ids = None
+    topk_k = None
+    if with_topk:
+        topk_k = topk_k_arg if topk_k_arg is not None else getattr(args, "opd_log_prob_top_k", 1)
+        topk_k = min(max(int(topk_k), 1), int(flat.size(-1)))
     if lay.n_tokens == 0:
         lp = flat.new_zeros((0,), dtype=torch.float32)
         ent = lp
+    elif not needs_bwd and with_topk and topk_k <= ops.TOPK_ROWS_MAX_K and flat.size(-1) <= ops.TOPK_ROWS_MAX_VOCAB:
+        # the actor's forward-only pass that also collects its top-K ids: one read of the logits serves the softmax
+        # scan and the selection (the selection does not depend on the temperature)
+        lp, ent, lse, _, _, topk_ids = ops.logprob_entropy_topk_fwd(ops._rows(flat), lay.targets, lay.row_ids, inv_t,
+                                                                    topk_k, bool(with_entropy))
     elif not needs_bwd:
         # forward-only (the ActorFwd / Reference passes): the launch's log-sum-exps stay at hand, so that a top-K gather
         # below costs K loads per row instead of another scan of the logits
@@ -180,9 +191,10 @@ def get_log_probs_and_entropy(
         res["entropy"] = lay.split(ent)
     if with_topk:
         # diagnostic student-side top-K ids (loss.py:436-438): a library selection over each sample's own rows
-        k = topk_k if topk_k is not None else getattr(args, "opd_log_prob_top_k", 1)
-        k = min(max(int(k), 1), int(flat.size(-1)))
-        if lay.n_tokens and k <= ops.TOPK_ROWS_MAX_K and flat.size(-1) <= ops.TOPK_ROWS_MAX_VOCAB:
+        k = topk_k
+        if topk_ids is not None:
+            res["topk_token_ids"] = lay.split(topk_ids)
+        elif lay.n_tokens and k <= ops.TOPK_ROWS_MAX_K and flat.size(-1) <= ops.TOPK_ROWS_MAX_VOCAB:
             # one launch over every response row (the selection does not depend on the temperature)
             _, ids = ops.topk_rows(flat, lay.row_ids, k, with_values=False)
             res["topk_token_ids"] = lay.split(ids)

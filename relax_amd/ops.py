@@ -388,6 +388,33 @@ def topk_rows(logits, row_ids, k: int, with_values: bool = True):
     return values, indices
 
 
+def logprob_entropy_topk_fwd(logits, targets, row_ids, inv_temperature: float, k: int, with_entropy: bool = True,
+                             with_values: bool = False):
+    """``logprob_entropy_fwd`` and ``topk_rows`` over the same rows from one read of the logits.  Returns
+    ``(log_prob, entropy | None, lse, spx | None, values | None, indices)``."""
+    dev = _need_gpu(logits, targets, row_ids)
+    logits = _rows(logits)
+    n = int(targets.numel())
+    if row_ids is None and n != logits.size(0):
+        raise ValueError(f"{n} targets for {logits.size(0)} logits rows")
+    if targets.dtype != torch.int64 or not targets.is_contiguous():
+        targets = targets.to(torch.int64).contiguous()
+    k = int(k)
+    kw = dict(dtype=torch.float32, device=dev)
+    lp, lse = torch.empty(n, **kw), torch.empty(n, **kw)
+    ent = torch.empty(n, **kw) if with_entropy else None
+    spx = torch.empty(n, **kw) if with_entropy else None
+    values = torch.empty((n, k), **kw) if with_values else None
+    indices = torch.empty((n, k), dtype=torch.int64, device=dev)
+    flags = torch.empty(max(n, 1), dtype=torch.uint8, device=dev)
+    stride = logits.stride(0) if logits.size(0) > 1 else logits.size(1)
+    with _timed("logprob_entropy_topk_fwd"):
+        check(lib.relax_amd_logprob_entropy_topk_fwd(
+            _p(logits), _code(logits), n, logits.size(1), stride, _p(row_ids), _p(targets), float(inv_temperature), k,
+            _p(lp), _p(ent), _p(lse), _p(spx), _p(values), _p(indices), _p(flags), _stream()))
+    return lp, ent, lse, spx, values, indices
+
+
 def scale_rows_inplace(data, factor_dev):
     data2 = data.reshape(-1, data.size(-1))
     stride = data2.stride(0) if data2.size(0) > 1 else data2.size(1)

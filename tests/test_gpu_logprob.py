@@ -283,6 +283,51 @@ def test_topk_rows_equals_torch_topk(n, v, k, dtype):
     _check_topk_rows(x, k, row_ids)
 
 
+@pytest.mark.parametrize("n,v,k,dtype,temperature", [
+    (96, 151936, 64, torch.bfloat16, 1.0),    # the production row: one read serves both
+    (40, 151936, 8, torch.float32, 0.7),      # fp32 rows of the same vocabulary
+    (50, 65536, 512, torch.float16, 1.0),     # the shortest row the fused kernel takes, the largest k
+    (50, 32003, 100, torch.float16, 1.0),     # rows that are not 16-byte aligned: the two passes run one after the other
+    (30, 4104, 16, torch.bfloat16, 1.3),      # a short row: likewise
+])
+def test_logprob_entropy_topk_one_read_equals_the_two_passes(n, v, k, dtype, temperature):
+    """``logprob_entropy_topk_fwd`` (log-probs, entropy and the top-K ids of the same rows from one read) against the
+    two separate launches: log-prob / entropy / lse / spx bit for bit, top-K values exactly, indices pointing at their
+    values; through a row map as well; rows with long runs of equal values or an infinite logit (which the shortcut
+    hands to the general kernel) included."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("logprob + topk one read", n, v, k, dtype, temperature)
+    g = torch.Generator(device=dev).manual_seed(n + v + k)
+    x = (torch.randn((n, v), device=dev, generator=g) * 3).to(dtype)
+    x[3] = 1.5        # a constant row: every element ties
+    x[5, : v // 2] = x[5, 0]  # half a row of equal values above most of the rest
+    x[5, 0: v // 2] = 9.0
+    x[7, 11] = float("inf")   # an infinite logit: log-prob and entropy are NaN in both kernels, the selection still exact
+    x[9, v // 3:] = float("-inf")  # most of a row at -inf
+    tok = torch.randint(0, v, (n,), device=dev, generator=g)
+    inv_t = 1.0 / temperature
+    for row_ids in (None, torch.cat([torch.arange(n - 1, -1, -2, device=dev), torch.tensor([0, 5, 5, 3], device=dev)]).int()):
+        t = tok if row_ids is None else tok[: row_ids.numel()]
+        lp, ent, lse, spx, vals, idx = ops.logprob_entropy_topk_fwd(x, t, row_ids, inv_t, k, True, with_values=True)
+        lp2, ent2, lse2, spx2 = ops.logprob_entropy_fwd(x, t, row_ids, inv_t, True)
+        for one, two in ((lp, lp2), (ent, ent2), (lse, lse2), (spx, spx2)):
+            assert torch.equal(one.isnan(), two.isnan()) and torch.equal(one.nan_to_num(), two.nan_to_num())
+        assert lp[~lp.isnan()].numel() >= lp.numel() - 3
+        vals2, idx2 = ops.topk_rows(x, row_ids, k)
+        rows = x if row_ids is None else x[row_ids.long()]
+        assert torch.equal(vals, vals2)
+        assert torch.equal(vals, torch.topk(rows.float(), k, dim=-1).values)
+        assert (idx >= 0).all() and (idx < v).all()
+        assert torch.equal(torch.gather(rows.float(), 1, idx), vals)
+        assert (torch.sort(idx, dim=1).values.diff(dim=1) > 0).all() or k == 1  # distinct
+    # without entropy and without values: the optional outputs are really optional
+    lp3, ent3, lse3, spx3, vals3, idx3 = ops.logprob_entropy_topk_fwd(x, tok, None, inv_t, k, False)
+    assert ent3 is None and spx3 is None and vals3 is None
+    assert torch.equal(lp3.nan_to_num(), ops.logprob_entropy_fwd(x, tok, None, inv_t, False)[0].nan_to_num())
+
+
 def test_topk_rows_on_tiny_vocabularies():
     """Rows shorter than one 16-byte vector, with a row stride that still allows vector loads: nothing may be read
     outside the row."""
