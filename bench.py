@@ -325,7 +325,7 @@ def run_actor_step(a, dev) -> None:
 def run_lmhead(a, dev) -> None:
     """hidden [N, 4096] ~ N(0, 1), weight [V, 4096] ~ N(0, 0.02), scalar PPO-style loss with advantages ~ N(0, 1):
     forward log-prob + entropy without materialised logits, backward to dhidden and dweight."""
-    from relax_amd.lm_head import lm_head_log_probs_and_entropy
+    from relax_amd.lm_head import lm_head_log_probs_and_entropy, lm_head_token_local_step
 
     n, h, v = a.rows or 32768, a.hidden, a.vocab
     g = torch.Generator(device=dev).manual_seed(0)
@@ -341,6 +341,9 @@ def run_lmhead(a, dev) -> None:
 
     vendor_out = torch.empty((min(n, 8192), v), dtype=torch.bfloat16, device=dev) if a.vendor_gemm else None
 
+    def surrogate(begin, end, lp, _ent):  # PPO's surrogate at ratio 1 (old log-probs = current ones): -A * lp
+        return -(adv[begin:end] * lp).sum()
+
     def step():
         hidden.grad = None
         weight.grad = None
@@ -354,8 +357,16 @@ def run_lmhead(a, dev) -> None:
             with torch.no_grad():
                 lp, ent = lm_head_log_probs_and_entropy(hidden, weight, tokens, 1.0, True, False)
             return -(adv * lp).sum()
-        lp, ent = lm_head_log_probs_and_entropy(hidden, weight, tokens, 1.0, True, False, keep_logits=a.keep_logits)
-        loss = -(adv * lp).sum()
+        if a.two_projections or a.keep_logits:
+            # log-probs / entropy handed to autograd; backward projects again (or reads the kept logits)
+            lp, ent = lm_head_log_probs_and_entropy(hidden, weight, tokens, 1.0, True, False,
+                                                    keep_logits=a.keep_logits)
+            loss = -(adv * lp).sum()
+        else:
+            # the step's default: the loss is token-local, so every slab of logits turns into its gradient as soon as
+            # its log-probs are known -- one projection, a[.lmhead_slab] rows of logits in HBM at a time
+            loss, lp, ent = lm_head_token_local_step(hidden, weight, tokens, surrogate, 1.0, with_entropy=True,
+                                                     slab_tokens=a.lmhead_slab)
         loss.backward()
         return loss
 
@@ -365,16 +376,20 @@ def run_lmhead(a, dev) -> None:
     # the timed forward region holds the target-logit gather, the MFMA kernel and the split combine; the MFMA kernel
     # is > 99 % of it (see the rocprofv3 summary), so its event time stands for lmhead_fwd_kernel
     dom = kernel_ms["lmhead_logprob_fwd"]
-    flops = 2.0 * n * h * v
+    flops = 2.0 * n * h * v / max(launches.get("lmhead_logprob_fwd", 1.0), 1.0)  # per launch: one slab of rows
     achieved = flops / (dom * 1e-3) / 1e12
     emit(a, n, wall,
          f"fused LM-head + log-prob/entropy: hidden bf16 [{n}, {h}], weight bf16 [{v}, {h}], fwd "
-         + ("(bf16 logits kept for the backward pass)" if a.keep_logits else "(no logits in HBM)")
+         + ("(bf16 logits kept for the backward pass)" if a.keep_logits else
+            "(no logits in HBM; backward projects a second time)" if a.two_projections else
+            f"(logits of {min(n, a.lmhead_slab)} rows at a time become their gradient in place)")
          + (" only [diagnostic]" if a.forward_only else " + bwd to dhidden/dweight from a scalar loss")
          + (" [diagnostic: all-zero operands]" if a.lmhead_operands == "zeros" else "")
          + (" [diagnostic: NOT the fused kernel -- hipBLASLt GEMM of the forward shape, logits written]"
             if a.vendor_gemm else ""),
-         {"rows": n, "hidden": h, "vocab": v, "keep_logits": bool(a.keep_logits), "loss": float(loss.item())},
+         {"rows": n, "hidden": h, "vocab": v, "keep_logits": bool(a.keep_logits),
+          "two_projections": bool(a.two_projections), "slab_rows": int(min(n, a.lmhead_slab)),
+          "loss": float(loss.item())},
          {"bound": "mfma", "kernel": "hipBLASLt GEMM (diagnostic)" if a.vendor_gemm else "lmhead_fwd_kernel",
           "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
           "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
@@ -751,6 +766,10 @@ def main() -> int:
     ap.add_argument("--keep-logits", action="store_true",
                     help="lmhead workload: keep a [V, N] bf16 copy of the logits for the backward pass instead of "
                          "projecting a second time (10 GB at the default size)")
+    ap.add_argument("--two-projections", action="store_true",
+                    help="lmhead: log-probs handed to autograd, the backward pass recomputes the projection")
+    ap.add_argument("--lmhead-slab", type=int, default=8192,
+                    help="lmhead: rows of logits that exist in HBM at a time in the one-projection step")
     ap.add_argument("--forward-only", action="store_true",
                     help="lmhead workload, diagnostic: time the forward pass alone (clock samples of that kernel only)")
     ap.add_argument("--mfma-shape", choices=["32x32x16", "16x16x32"], default="32x32x16",

@@ -361,24 +361,32 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_gemm_kernel(GemmOperand 
     float* c = static_cast<float*>(c_out);
     const int64_t bcol = b0 + wb * 128 + (lane & 31);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i) {
+      const int64_t arow = a0 + wa * 128 + i * 32 + 4 * (lane >> 5);
+      // accumulation: the 64 earlier values of this row of blocks are requested together, one memory round trip per
+      // row of blocks instead of one per block
+      float prev[4][16];
+      if (OUT == kGemmOutF32Accumulate) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int64_t a = arow + 8 * (r >> 2) + (r & 3), b = bcol + j * 32;
+            prev[j][r] = (a < ma && b < mb) ? c[a * c_stride + b] : 0.f;
+          }
+      }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const floatx16 blk = acc[i][j];
         const int64_t b = bcol + j * 32;
-        const int64_t arow = a0 + wa * 128 + i * 32 + 4 * (lane >> 5);
-        if (b < mb) {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int64_t a = arow + 8 * (r >> 2) + (r & 3);
-            if (a < ma) {
-              float* o = c + a * c_stride + b;
-              *o = OUT == kGemmOutF32Accumulate ? *o + blk[r] : blk[r];
-            }
-          }
+        for (int r = 0; r < 16; ++r) {
+          const int64_t a = arow + 8 * (r >> 2) + (r & 3);
+          if (a < ma && b < mb) c[a * c_stride + b] = OUT == kGemmOutF32Accumulate ? prev[j][r] + blk[r] : blk[r];
         }
-        __builtin_amdgcn_sched_barrier(0);
       }
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 }
 

@@ -240,3 +240,118 @@ def lm_head_log_probs_and_entropy(hidden, weight, tokens, temperature: float = 1
     lp, ent = FusedLMHeadLogProb.apply(hidden, weight, tokens, 1.0 / float(temperature), bool(with_entropy),
                                        bool(with_entropy_grad), bool(keep_logits))
     return lp, (ent if with_entropy else None)
+
+
+# tokens per slab of the no-recompute step below: the bf16 logits of one slab, [V, STEP_SLAB] (2.5 GB at V = 151936),
+# are the only logits in HBM at any time
+STEP_SLAB = 8192
+
+
+class _FusedLMHeadTokenLocalStep(torch.autograd.Function):
+    """(hidden [N,H] bf16, weight [V,H] bf16, targets [N]) -> (loss, log_prob [N], entropy [N]) for a loss that is a
+    sum of per-token terms whose weights do not depend on other tokens' log-probs (SFT, REINFORCE / PPO-clip with
+    fixed normalisers): the whole step runs inside forward, one slab of tokens at a time, and never projects twice.
+
+    Per slab: the forward kernel writes the slab's bf16 logits [V, slab] next to its log-probs / entropy; the caller's
+    ``token_loss`` turns those log-probs into the slab's share of the loss, whose derivative w.r.t. them (autograd over
+    [slab]-sized vectors) is the coefficient vector; the logits become d loss / d logits in place; dhidden of the slab
+    and the slab's addition to dweight (fp32 across slabs) follow on the matrix cores.  Backward only rescales the two
+    gradients when the upstream gradient differs from ``assumed_scale``.
+    """
+
+    @staticmethod
+    def forward(ctx, hidden, weight, targets, inv_temperature, with_entropy, token_loss, slab_tokens, assumed_scale):
+        hidden, weight = _bf16_rows(hidden, "hidden"), _bf16_rows(weight, "weight")
+        if targets.dtype != torch.int64 or not targets.is_contiguous():
+            targets = targets.to(torch.int64).contiguous()
+        n, v = hidden.size(0), weight.size(0)
+        need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        slab_tokens = max(128, _ceil128(min(int(slab_tokens), max(n, 1))))
+        dev = hidden.device
+        lp_all = torch.empty(n, dtype=torch.float32, device=dev)
+        ent_all = torch.empty(n if with_entropy else 0, dtype=torch.float32, device=dev)
+        loss = torch.zeros((), dtype=torch.float32, device=dev)
+        slab = alloc_slab(v, slab_tokens, dev) if (need_h or need_w) and n > 0 else None
+        d_hidden = torch.empty_like(hidden) if need_h else None
+        single = n <= slab_tokens
+        d_weight = None
+        if need_w:
+            d_weight = torch.zeros_like(weight) if n == 0 else (
+                torch.empty_like(weight) if single else torch.empty(weight.shape, dtype=torch.float32, device=dev))
+        for s in range(0, n, slab_tokens):
+            e = min(n, s + slab_tokens)
+            cnt = e - s
+            lp, ent, lse, spx = lmhead_logprob_fwd(hidden[s:e], weight, targets[s:e], inv_temperature, with_entropy,
+                                                   None if slab is None else slab[:v])
+            lp_all[s:e] = lp
+            if with_entropy:
+                ent_all[s:e] = ent
+            with torch.enable_grad():
+                lp_leaf = lp.detach().requires_grad_()
+                ent_leaf = ent.detach().requires_grad_() if with_entropy else None
+                part = token_loss(s, e, lp_leaf, ent_leaf)
+                if slab is not None:
+                    leaves = [lp_leaf] + ([ent_leaf] if with_entropy else [])
+                    grads = torch.autograd.grad(part, leaves, allow_unused=True)
+            loss = loss + part.detach().to(torch.float32)
+            if slab is None:
+                continue
+            g_lp = grads[0] if grads[0] is not None else torch.zeros_like(lp)
+            g_ent = grads[1] if with_entropy and grads[1] is not None else None
+            if assumed_scale != 1.0:
+                g_lp = g_lp * assumed_scale
+                g_ent = None if g_ent is None else g_ent * assumed_scale
+            g_lp = g_lp.to(torch.float32).contiguous()
+            g_ent = None if g_ent is None else g_ent.to(torch.float32).contiguous()
+            lmhead_dlogits_from_logits_t(slab[:v], cnt, targets[s:e], lse, spx if g_ent is not None else None, g_lp,
+                                         g_ent, inv_temperature)
+            if slab.size(1) > cnt:
+                slab[:, cnt:].zero_()  # the in-place kernel works on whole 16-byte vectors of tokens
+            if need_h:
+                lmhead_dhidden(slab, cnt, weight, d_hidden[s:e])
+            if need_w:
+                lmhead_dweight(slab, cnt, hidden[s:e], v, d_weight, accumulate=s > 0)
+        if need_w and n > 0 and not single:
+            d_weight = d_weight.to(weight.dtype)
+        ctx.grads = (d_hidden, d_weight)
+        ctx.assumed_scale = float(assumed_scale)
+        ctx.mark_non_differentiable(lp_all, ent_all)
+        return loss, lp_all, ent_all
+
+    @staticmethod
+    def backward(ctx, g_loss, _glp, _gent):
+        if ctx.grads is None:
+            raise RuntimeError("the fused LM-head step holds its gradients once: backward cannot run twice")
+        d_hidden, d_weight = ctx.grads
+        ctx.grads = None
+        factor = g_loss.reshape(1).to(torch.float32)
+        if ctx.assumed_scale != 1.0:
+            factor = factor / ctx.assumed_scale
+        factor = factor.contiguous()
+        for d in (d_hidden, d_weight):
+            if d is not None and d.numel():
+                ops.scale_rows_inplace(d, factor)  # a no-op launch when the upstream gradient is the assumed one
+        return d_hidden, d_weight, None, None, None, None, None, None
+
+
+def lm_head_token_local_step(hidden, weight, tokens, token_loss, temperature: float = 1.0, with_entropy: bool = False,
+                             slab_tokens: int | None = None, assumed_grad_scale: float = 1.0):
+    """``(loss, log_prob [N], entropy [N] | None)`` of a token-local loss over ``log_softmax(hidden @ weight.T / T)``
+    with the gradients w.r.t. ``hidden`` and ``weight`` produced inside this call (``loss.backward()`` then only hands
+    them on), never more than ``slab_tokens`` rows of logits in HBM and no second projection.
+
+    ``token_loss(begin, end, log_prob, entropy) -> 0-d tensor`` gives the share of rows ``[begin, end)`` in the loss,
+    built from differentiable ``[end - begin]``-sized vector operations on the two leaves it is handed; the shares add
+    up to the loss, so every normaliser inside it must be known up front (a token count, a per-sample mask sum: what
+    the reference's reducers divide by, relax/backends/megatron/cp_utils.py:125-162).  SFT's
+    ``-sum_of_sample_mean(log_probs)`` (loss.py:1386-1428) and a clipped policy-gradient surrogate with given old
+    log-probs and advantages are of this kind; GSPO's sequence-level ratio is not.
+    """
+    pad = (-hidden.size(-1)) % 128
+    if pad:
+        hidden = torch.nn.functional.pad(hidden, (0, pad))
+        weight = torch.nn.functional.pad(weight, (0, pad))
+    loss, lp, ent = _FusedLMHeadTokenLocalStep.apply(
+        hidden, weight, tokens, 1.0 / float(temperature), bool(with_entropy), token_loss,
+        int(slab_tokens or STEP_SLAB), float(assumed_grad_scale))
+    return loss, lp, (ent if with_entropy else None)

@@ -224,14 +224,9 @@ def lm_head_weight_of(lm_head_forward) -> torch.Tensor:
     return weight
 
 
-def _deferred_lm_head_log_probs(hidden, args, unconcat_tokens, total_lengths, response_lengths, with_entropy,
-                                lm_head_forward, max_seq_lens=None):
-    """Deferred-LM-head branch of get_log_probs_and_entropy (loss.py:391-419): ``hidden`` is ``[1, T, H]`` (or
-    ``[T, H]``) and the ``[T, V]`` logits are never formed.  The response rows of all samples go through the fused
-    LM-head kernel in one launch; unlike the reference's chunked path entropy is available as well."""
-    from .lm_head import lm_head_log_probs_and_entropy
-
-    weight = lm_head_weight_of(lm_head_forward)
+def _deferred_rows(hidden, weight, args, unconcat_tokens, total_lengths, response_lengths, max_seq_lens):
+    """``([T, H] rows of the hidden states, PackedLayout of their response tokens)`` for a deferred LM head: ``hidden``
+    is ``[1, T, H]`` packed, ``[B, S, H]`` padded, or ``[T, H]``."""
     padded = _padded_starts(args, max_seq_lens)
     if hidden.dim() == 3 and padded is not None:
         rows = hidden.reshape(-1, hidden.size(-1))  # [B, S, H]: sample i starts at row max_seq_lens[i] * i
@@ -246,6 +241,18 @@ def _deferred_lm_head_log_probs(hidden, args, unconcat_tokens, total_lengths, re
     if not rows.is_cuda:
         raise RuntimeError("relax_amd kernels need ROCm device tensors (no CPU fallback)")
     lay = PackedLayout(rows.device, rows.size(0), unconcat_tokens, total_lengths, response_lengths, False, padded)
+    return rows, lay
+
+
+def _deferred_lm_head_log_probs(hidden, args, unconcat_tokens, total_lengths, response_lengths, with_entropy,
+                                lm_head_forward, max_seq_lens=None):
+    """Deferred-LM-head branch of get_log_probs_and_entropy (loss.py:391-419): ``hidden`` is ``[1, T, H]`` (or
+    ``[T, H]``) and the ``[T, V]`` logits are never formed.  The response rows of all samples go through the fused
+    LM-head kernel in one launch; unlike the reference's chunked path entropy is available as well."""
+    from .lm_head import lm_head_log_probs_and_entropy
+
+    weight = lm_head_weight_of(lm_head_forward)
+    rows, lay = _deferred_rows(hidden, weight, args, unconcat_tokens, total_lengths, response_lengths, max_seq_lens)
     if lay.n_tokens == 0:
         lp = rows.new_zeros((0,), dtype=torch.float32)
         ent = lp
@@ -266,19 +273,53 @@ def sft_loss_function_chunked(args: Namespace, batch: dict, hidden_states: torch
     """SFT loss with the LM head deferred into the loss (loss.py:1386-1428): ``-sum_of_sample_mean(log_probs)`` with
     the log-probs taken straight from hidden states and the LM-head weight.  ``sum_of_sample_mean`` may be None: the
     reference's reducer is then rebuilt from the batch."""
+    if sum_of_sample_mean is None:
+        sum_of_sample_mean = get_sum_of_sample_mean(
+            batch["total_lengths"], batch["response_lengths"], batch["loss_masks"],
+            bool(getattr(args, "calculate_per_token_loss", False)), sample_denoms=batch.get("sample_index_mask_sums"))
+    if torch.is_grad_enabled() and getattr(args, "relax_amd_single_pass", "auto") not in (False, "off"):
+        loss = _sft_chunked_single_projection(args, batch, hidden_states, sum_of_sample_mean, lm_head_forward)
+        if loss is not None:
+            return loss, {"loss": loss.clone().detach()}
     _, out = get_log_probs_and_entropy(
         hidden_states, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=batch["total_lengths"],
         response_lengths=batch["response_lengths"], with_entropy=False, lm_head_forward=lm_head_forward,
         max_seq_lens=batch.get("max_seq_lens"))
     log_probs = torch.cat(out["log_probs"], dim=0)
-    if sum_of_sample_mean is None:
-        sum_of_sample_mean = get_sum_of_sample_mean(
-            batch["total_lengths"], batch["response_lengths"], batch["loss_masks"],
-            bool(getattr(args, "calculate_per_token_loss", False)), sample_denoms=batch.get("sample_index_mask_sums"))
     loss = -sum_of_sample_mean(log_probs)
     if log_probs.numel() == 0:
         loss = loss + 0 * hidden_states.sum()
     return loss, {"loss": loss.clone().detach()}
+
+
+def _sft_chunked_single_projection(args, batch, hidden_states, sum_of_sample_mean, lm_head_forward):
+    """The training step of the chunked SFT loss with one projection instead of two: the reducer is linear in the
+    log-probs (every reducer of cp_utils.py:125-162 is a sum of masked per-sample means or token sums), so each
+    token's weight in the loss is known before its log-prob is, and the LM-head step can turn every slab of logits
+    into its gradient straight away (``lm_head.lm_head_token_local_step``).  The weights are read off the reducer
+    itself, as its gradient; the value returned is the reducer's own.  None when nothing needs a gradient."""
+    from .lm_head import lm_head_token_local_step
+
+    weight = lm_head_weight_of(lm_head_forward)
+    if not (hidden_states.requires_grad or weight.requires_grad):
+        return None
+    rows, lay = _deferred_rows(hidden_states, weight, args, batch["unconcat_tokens"], batch["total_lengths"],
+                               batch["response_lengths"], batch.get("max_seq_lens"))
+    if lay.n_tokens == 0:
+        return None
+    probe = torch.zeros(lay.n_tokens, dtype=torch.float32, device=rows.device, requires_grad=True)
+    with torch.enable_grad():
+        token_weight, = torch.autograd.grad(sum_of_sample_mean(probe), probe)
+    picked = rows.index_select(0, lay.row_ids.to(torch.int64)).to(weight.dtype)  # [N, H]
+
+    def token_loss(begin, end, log_prob, _entropy):
+        return -(log_prob * token_weight[begin:end]).sum()
+
+    loss, log_probs, _ = lm_head_token_local_step(
+        picked, weight, lay.targets, token_loss, float(getattr(args, "rollout_temperature", 1.0)),
+        assumed_grad_scale=expected_grad_scale(batch))
+    # the value in the reducer's own order of summation; the gradient is the step's
+    return (-sum_of_sample_mean(log_probs)).detach().to(loss.dtype) + (loss - loss.detach())
 
 
 def _sft_single_pass(args: Namespace, batch: dict, logits: torch.Tensor):

@@ -72,6 +72,20 @@ def test_forward_backward_vs_oracle(n, h, v, temperature):
     assert torch.equal(lp2, lp.detach())
 
 
+def _oracle_bf16_logits(hid, w, tok, wl, we, temperature):
+    """The reference's numerics: F.linear in bf16 (logits rounded to bf16), then fp32 log-softmax
+    (relax/backends/megatron/loss.py:405-409); gradients flow through the rounding unchanged."""
+    h32 = hid.float().requires_grad_()
+    w32 = w.float().requires_grad_()
+    raw = F.linear(h32, w32)
+    logits = (raw + (raw.bfloat16().float() - raw).detach()) / temperature
+    ls = torch.log_softmax(logits, -1)
+    lp = ls[torch.arange(hid.size(0)), tok]
+    ent = -(ls.exp() * ls).sum(-1)
+    ((lp * wl).sum() + (ent * we).sum()).backward()
+    return lp.detach(), ent.detach(), h32.grad, w32.grad
+
+
 @pytest.mark.parametrize("n,h,v,temperature", [
     (256, 64, 256, 1.0),
     (301, 128, 1000, 0.7),      # ragged vocabulary, odd token count (a half-filled token pair at the end)
@@ -255,6 +269,113 @@ def test_slabbed_backward_accumulates_dweight(monkeypatch):
     torch.testing.assert_close(wd.grad.float().cpu(), rgw, atol=5e-3, rtol=2 * BF16_ULP)
 
 
+@pytest.mark.parametrize("n,h,v,temperature,slab,scale", [
+    (700, 64, 900, 1.0, 256, 1.0),       # three slabs, the last one short: dweight accumulated in fp32
+    (300, 128, 1000, 0.7, 8192, 1.0),    # one slab
+    (1100, 256, 5000, 1.0, 512, 0.25),   # the upstream gradient the caller announced
+    (513, 128, 700, 1.3, 384, 1.0),      # a last slab of one token
+])
+def test_token_local_step_vs_oracle(n, h, v, temperature, slab, scale):
+    """``lm_head_token_local_step`` (one projection: every slab's logits become their gradient in place, inside
+    forward) with a PPO-clip surrogate + entropy bonus as the token-local loss, against the oracle's F.linear ->
+    log-softmax -> same loss in fp32 autograd, and against the two-projection path of ``FusedLMHeadLogProb``."""
+    from relax_amd.lm_head import lm_head_log_probs_and_entropy, lm_head_token_local_step
+
+    dev = require_gpu()
+    announce("lmhead token-local step", n, h, v, temperature, slab, scale)
+    hid, w, tok, g = _inputs(n, h, v, seed=n + v, w_scale=0.3 if h < 1024 else 0.05)
+    adv = torch.randn(n, generator=g)
+    noise = torch.randn(n, generator=g) * 0.3      # a third of the tokens end up clipped
+    mask = (torch.rand(n, generator=g) > 0.2).float()
+    denom = mask.sum().clamp_min(1)
+
+    def surrogate(lp, ent, old, a, m, d):
+        ratio = torch.exp(lp - old)
+        pg = torch.maximum(-a * ratio, -a * ratio.clamp(0.8, 1.28))
+        return ((pg - 0.01 * ent) * m).sum() / d
+
+    # oracle, in the reference's numerics: logits rounded to bf16 (F.linear in the weight dtype), fp32 log-softmax
+    h32, w32 = hid.float().requires_grad_(), w.float().requires_grad_()
+    raw = F.linear(h32, w32)
+    lp_unrounded = torch.log_softmax(raw.detach() / temperature, -1)[torch.arange(n), tok]
+    ls = torch.log_softmax((raw + (raw.bfloat16().float() - raw).detach()) / temperature, -1)
+    rlp = ls[torch.arange(n), tok]
+    rent = -(ls.exp() * ls).sum(-1)
+    old = rlp.detach() + noise
+    want = surrogate(rlp, rent, old, adv, mask, denom)
+    (want * scale).backward()
+
+    old_d, adv_d, mask_d, denom_d = old.to(dev), adv.to(dev), mask.to(dev), denom.to(dev)
+
+    def token_loss(b, e, lp, ent):
+        return surrogate(lp, ent, old_d[b:e], adv_d[b:e], mask_d[b:e], denom_d)
+
+    hd, wd = hid.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    loss, lp, ent = lm_head_token_local_step(hd, wd, tok.to(dev), token_loss, temperature, with_entropy=True,
+                                             slab_tokens=slab, assumed_grad_scale=scale)
+    assert loss.requires_grad and not lp.requires_grad and not ent.requires_grad
+    torch.testing.assert_close(lp.cpu(), rlp.detach(), atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent.cpu(), rent.detach(), atol=2e-3, rtol=0)
+    assert abs(loss.item() - want.item()) < 2e-3
+    (loss * scale).backward()
+    torch.testing.assert_close(hd.grad.float().cpu(), h32.grad, atol=5e-3, rtol=2 * BF16_ULP)
+    torch.testing.assert_close(wd.grad.float().cpu(), w32.grad, atol=5e-3, rtol=2 * BF16_ULP)
+    with pytest.raises(RuntimeError, match="cannot run twice"):
+        (loss * scale).backward()
+
+    # the two-projection path, on a loss without clip boundaries (the two paths' log-probs differ by the bf16
+    # rounding of the kept logits, which moves tokens across a clip boundary): gradients equal up to that rounding
+    def smooth(lp, ent, a, m, d):
+        return ((-a * lp - 0.01 * ent) * m).sum() / d
+
+    h1, w1 = hid.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    loss1, _, _ = lm_head_token_local_step(
+        h1, w1, tok.to(dev), lambda b, e, lp, ent: smooth(lp, ent, adv_d[b:e], mask_d[b:e], denom_d), temperature,
+        with_entropy=True, slab_tokens=slab)
+    loss1.backward()
+    h2, w2 = hid.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    lp2, ent2 = lm_head_log_probs_and_entropy(h2, w2, tok.to(dev), temperature, with_entropy=True)
+    smooth(lp2, ent2, adv_d, mask_d, denom_d).backward()
+    torch.testing.assert_close(h1.grad.float(), h2.grad.float(), atol=5e-3, rtol=2 * BF16_ULP)
+    torch.testing.assert_close(w1.grad.float(), w2.grad.float(), atol=5e-3, rtol=2 * BF16_ULP)
+
+    # an upstream gradient other than the announced one: backward rescales what forward produced
+    h3, w3 = hid.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    loss3, _, _ = lm_head_token_local_step(h3, w3, tok.to(dev), token_loss, temperature, with_entropy=True,
+                                           slab_tokens=slab, assumed_grad_scale=scale)
+    (loss3 * (3.0 * scale)).backward()
+    torch.testing.assert_close(h3.grad.float(), 3.0 * hd.grad.float(), atol=1e-6, rtol=2 * BF16_ULP)
+    torch.testing.assert_close(w3.grad.float(), 3.0 * wd.grad.float(), atol=1e-6, rtol=2 * BF16_ULP)
+
+    # without gradients: the plain forward, no slab of logits (so nothing is rounded to bf16 on the way)
+    with torch.no_grad():
+        loss4, lp4, _ = lm_head_token_local_step(hid.to(dev), w.to(dev), tok.to(dev), token_loss, temperature,
+                                                 with_entropy=True, slab_tokens=slab)
+    assert not loss4.requires_grad and torch.isfinite(loss4)
+    torch.testing.assert_close(lp4.cpu(), lp_unrounded, atol=2e-3, rtol=0)
+
+
+def test_token_local_step_empty_input_and_weight_only_gradient():
+    from relax_amd.lm_head import lm_head_token_local_step
+
+    dev = require_gpu()
+    announce("lmhead token-local step: empty / weight-only")
+    hid, w, tok, g = _inputs(300, 128, 640, seed=11, w_scale=0.3)
+    coef = (torch.randn(300, generator=g) / 16).to(dev)
+    wd = w.to(dev).requires_grad_()
+    loss, lp, ent = lm_head_token_local_step(hid.to(dev)[:0], wd, tok.to(dev)[:0], lambda b, e, lp, _: lp.sum())
+    assert ent is None and lp.numel() == 0 and loss.item() == 0
+    loss.backward()
+    assert wd.grad is not None and not wd.grad.any()
+    # only the weight wants a gradient
+    wd.grad = None
+    loss, _, _ = lm_head_token_local_step(hid.to(dev), wd, tok.to(dev), lambda b, e, lp, _: (lp * coef[b:e]).sum(),
+                                          slab_tokens=128)
+    loss.backward()
+    _, _, _, rgw = _oracle(hid, w, tok, coef.cpu(), torch.zeros(300), 1.0)
+    torch.testing.assert_close(wd.grad.float().cpu(), rgw, atol=5e-3, rtol=2 * BF16_ULP)
+
+
 def test_argument_errors():
     from relax_amd.lm_head import lm_head_log_probs_and_entropy, lmhead_logprob_fwd
 
@@ -340,7 +461,10 @@ def test_sft_losses_plain_and_with_deferred_lm_head_vs_oracle():
     dhead = torch.nn.Linear(h, v, bias=False).bfloat16().to(dev)
     with torch.no_grad():
         dhead.weight.copy_(head.weight)
-    for handle in (dhead, dhead.forward, dhead.weight):
+    for handle, single in ((dhead, "auto"), (dhead.forward, "off"), (dhead.weight, "auto")):
+        # "auto": the one-projection step (each token's weight in the loss read off the reducer); "off": log-probs
+        # from the forward kernel, backward through a second projection
+        args.relax_amd_single_pass = single
         hd = hid.to(dev).requires_grad_()
         dhead.weight.grad = None
         loss, log = relax_amd.sft_loss_function_chunked(args, dbatch, hd, None, lm_head_forward=handle)
@@ -356,8 +480,12 @@ def test_sft_losses_plain_and_with_deferred_lm_head_vs_oracle():
     assert abs(loss2.item() - want.item()) < 2e-3 * len(resp)
     # loss_function: Megatron scaling (num_microbatches / global_batch_size) and the logging dict
     hd = hid.to(dev).requires_grad_()
+    dhead.weight.grad = None
     scaled, normalizer, logd = relax_amd.loss_function(args, dbatch, 2, hd, lm_head_forward=dhead.forward)
     assert abs(scaled.item() - want.item() * 2 / 3) < 2e-3 * len(resp) and logd["keys"] == ["loss"] and int(normalizer) == 1
+    scaled.backward()  # the step produced its gradients for the scale loss_function applies
+    torch.testing.assert_close(hd.grad.float().cpu(), hc.grad.float() * 2 / 3, atol=5e-3, rtol=2 * BF16_ULP)
+    torch.testing.assert_close(dhead.weight.grad.float().cpu(), wc.grad.float() * 2 / 3, atol=5e-3, rtol=2 * BF16_ULP)
     with pytest.raises(NotImplementedError, match="expose the LM-head weight"):
         relax_amd.sft_loss_function_chunked(args, dbatch, hd, None, lm_head_forward=lambda x: x)
 
