@@ -739,12 +739,18 @@ def run_varlen(a, dev, loss_kind: str) -> None:
     fused = "actor_step_fused" in kernel_ms
     name = "actor_step_fused" if fused else "logprob_entropy_bwd"
     dom = kernel_ms[name]
+    read_rows = live
+    if not fused:
+        # the separate backward launch knows every token's gradient coefficients before it starts and reads only the
+        # rows whose coefficients are not both zero (GSPO: every token of a sequence whose ratio is clipped has none)
+        read_rows = sum(int((logits.grad[0, s0:s0 + 4096] != 0).any(dim=1).sum().item()) for s0 in range(0, n, 4096))
     emit(a, n, wall,
          f"packed varlen: {seqs} sequences {lengths} = {n} rows x V={v} bf16 logits, ~30 % masked spans, RLOO "
          f"advantages, {loss_kind.upper()} loss, sequence-mean-token-sum, fwd + bwd to dlogits",
-         {"rows": n, "live_rows": live, "vocab": v, "loss": float(loss.item()), "lengths": lengths},
+         {"rows": n, "live_rows": live, "rows_read_by_the_launch": read_rows, "vocab": v, "loss": float(loss.item()),
+          "lengths": lengths},
          hbm_roofline(fused_step_kernel_name(v) if fused else name + "_kernel<bf16_t, true>", dom,
-                      row_bytes * (live + n), n, v, kernel_ms, wall * 1e3 / a.steps,
+                      row_bytes * (read_rows + n), n, v, kernel_ms, wall * 1e3 / a.steps,
                       survey_bytes=3.0 * row_bytes * n if fused else None),
          None)
 
