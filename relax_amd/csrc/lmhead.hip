@@ -63,7 +63,7 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_fwd_kernel(const uint16_
   const int vt_end = min(g.n_tiles, vt_begin + g.tiles_per_split);
   LmSlabWriter writer;
   if (STORE) writer.init(l_t, l_stride, g.vocab, g.n_tokens, tok0, wv, wt, lane);
-  lm_pipeline(LmLds{w0, h0, w1, h1}, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
+  lm_pipeline<STORE>(LmLds{w0, h0, w1, h1}, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
     const int limit = int(min<int64_t>(g.vocab - v0, kLmTile));
     if (STORE) writer.set_tile(v0);
 #pragma unroll
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_dlogits_kernel(
   const int vt_end = min(g.n_tiles, vt_begin + g.tiles_per_split);
   LmSlabWriter writer;
   writer.init(d_t, d_stride, g.vocab, g.n_tokens, tok0, wv, wt, lane);
-  lm_pipeline(LmLds{w0, h0, w1, h1}, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
+  lm_pipeline<true>(LmLds{w0, h0, w1, h1}, hidden, weight, g, tok0, vt_begin, vt_end, [&](floatx16 (&acc)[4][4], int64_t v0) {
     writer.set_tile(v0);
 #pragma unroll
     for (int i = 0; i < 4; ++i)

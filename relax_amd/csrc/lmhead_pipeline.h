@@ -36,6 +36,7 @@ __device__ __forceinline__ bool lm_block_coords(const LmGeom& g, int& rb, int& s
 // "all vector-memory operations done" (vmcnt = 0, expcnt and lgkmcnt left at their maxima), and vmcnt = lgkmcnt = 0.
 constexpr int kLmWaitCopies = 0x0F70;
 constexpr int kLmWaitEverything = 0x0070;
+constexpr int kLmWaitLdsAndScalar = 0xC07F;  // lgkmcnt = 0, vmcnt left at its maximum
 
 // Asynchronous global -> LDS copy of one 256-row x 64-col bf16 slice of an operand.  Thread t covers row t/8 of each
 // 32-row pass and LDS slot t%8; it fetches global vector (t%8) ^ ((row >> 1) & 7) of that row (the same value for
@@ -182,7 +183,13 @@ struct LmLds {
   unsigned char *w0, *h0, *w1, *h1;  // weight / hidden tile of stage 0 and of stage 1
 };
 
-template <typename Epilogue>
+//
+// EPILOGUE_STORES: the epilogue writes its tile to global memory (the kept logits, the gradient slab).  Vector-memory
+// operations retire in order, so a wait for the next slice's copies issued after those stores would also wait until
+// every store has been acknowledged by memory, once per tile.  In this form the copies of the next tile's first slice
+// (issued under the last slice, i.e. before the stores) are awaited before the epilogue instead, the tile boundary is
+// a bare barrier, and the stores drain under the next tile's first slice, whose closing wait finds them done.
+template <bool EPILOGUE_STORES = false, typename Epilogue>
 __device__ __forceinline__ void lm_pipeline(const LmLds lds, const uint16_t* hidden, const uint16_t* weight,
                                             const LmGeom& g, int64_t tok0, int vt_begin, int vt_end,
                                             Epilogue&& epilogue) {
@@ -204,7 +211,7 @@ __device__ __forceinline__ void lm_pipeline(const LmLds lds, const uint16_t* hid
     // Settle register reloads left over from the epilogue here, once per tile; otherwise the compiler waits for them
     // at their first use inside the steady-state loop, which also drains the copies issued just before.
     __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_waitcnt(kLmWaitEverything);
+    __builtin_amdgcn_s_waitcnt(EPILOGUE_STORES ? kLmWaitLdsAndScalar : kLmWaitEverything);
     __builtin_amdgcn_sched_barrier(0);
     // slice 0 (stage 0): nothing to multiply yet, so its first fragments are waited for in the open
 #pragma unroll
@@ -249,9 +256,22 @@ __device__ __forceinline__ void lm_pipeline(const LmLds lds, const uint16_t* hid
     lm_slice_head(st1, lane, f0, f1, acc, copy_next_tile);
     lm_slice_body(st1, lane, f0, f1, acc, copy_next_tile);
     lm_mma_group(f1, acc, [](int) {});
+    if (EPILOGUE_STORES) {
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(kLmWaitCopies);  // the next tile's first slice: issued a slice ago, before any store
+      __builtin_amdgcn_sched_barrier(0);
+    }
     epilogue(acc, int64_t(vt) * kLmTile);
     lm_zero_acc(acc);
-    lm_slice_sync();
+    if (EPILOGUE_STORES) {
+      // every wave has passed its own wait above, so all copies into stage 0 have landed, and every wave is done
+      // reading stage 1; no wait for the stores
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_barrier" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+    } else {
+      lm_slice_sync();
+    }
   }
 }
 
