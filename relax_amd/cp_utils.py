@@ -77,6 +77,7 @@ def get_sum_of_sample_mean(
     def reducer(x: torch.Tensor) -> torch.Tensor:
         return _MaskedSampleReduce.apply(x, mask, cu, inv)
 
+    reducer.relax_amd_linear = True  # a fixed weighted sum of its argument: callers may read the weights off it
     return reducer
 
 
@@ -86,6 +87,8 @@ class PerSampleDivisorReducer:
     A function named by ``--custom-pg-loss-reducer-function-path`` (loss.py:1062-1072) may return one of these instead
     of an opaque callable: ``policy_loss_function`` then reads ``sample_divisors`` and evaluates the pg_loss reduction
     inside its fused launch; any other code can still call the object like the closure the reference expects."""
+
+    relax_amd_linear = True  # a fixed weighted sum of its argument
 
     def __init__(self, response_lengths, loss_masks, sample_divisors):
         self.response_lengths = [int(r) for r in response_lengths]

@@ -277,7 +277,8 @@ def sft_loss_function_chunked(args: Namespace, batch: dict, hidden_states: torch
         sum_of_sample_mean = get_sum_of_sample_mean(
             batch["total_lengths"], batch["response_lengths"], batch["loss_masks"],
             bool(getattr(args, "calculate_per_token_loss", False)), sample_denoms=batch.get("sample_index_mask_sums"))
-    if torch.is_grad_enabled() and getattr(args, "relax_amd_single_pass", "auto") not in (False, "off"):
+    if torch.is_grad_enabled() and getattr(args, "relax_amd_single_pass", "auto") not in (False, "off") \
+            and getattr(sum_of_sample_mean, "relax_amd_linear", False):
         loss = _sft_chunked_single_projection(args, batch, hidden_states, sum_of_sample_mean, lm_head_forward)
         if loss is not None:
             return loss, {"loss": loss.clone().detach()}
@@ -294,7 +295,8 @@ def sft_loss_function_chunked(args: Namespace, batch: dict, hidden_states: torch
 
 def _sft_chunked_single_projection(args, batch, hidden_states, sum_of_sample_mean, lm_head_forward):
     """The training step of the chunked SFT loss with one projection instead of two: the reducer is linear in the
-    log-probs (every reducer of cp_utils.py:125-162 is a sum of masked per-sample means or token sums), so each
+    log-probs (every reducer of cp_utils.py:125-162 is a sum of masked per-sample means or token sums; this library's
+    reducers say so with ``relax_amd_linear``, any other callable keeps the two-projection path), so each
     token's weight in the loss is known before its log-prob is, and the LM-head step can turn every slab of logits
     into its gradient straight away (``lm_head.lm_head_token_local_step``).  The weights are read off the reducer
     itself, as its gradient; the value returned is the reducer's own.  None when nothing needs a gradient."""

@@ -433,6 +433,7 @@ def test_sft_losses_plain_and_with_deferred_lm_head_vs_oracle():
     forward and gradients; loss_function dispatch for ``loss_type="sft"``."""
     import relax_amd
     from oracle import reducers as R
+    from relax_amd.cp_utils import get_sum_of_sample_mean
 
     dev = require_gpu()
     announce("sft losses")
@@ -474,6 +475,16 @@ def test_sft_losses_plain_and_with_deferred_lm_head_vs_oracle():
         assert abs(loss.item() - want.item()) < 2e-3 * len(resp) and abs(log["loss"].item() - loss.item()) == 0
         torch.testing.assert_close(hd.grad.float().cpu(), hc.grad.float(), atol=5e-3, rtol=2 * BF16_ULP)
         torch.testing.assert_close(dhead.weight.grad.float().cpu(), wc.grad.float(), atol=5e-3, rtol=2 * BF16_ULP)
+    # a caller's own reducer (not known to be a fixed weighted sum) keeps log-probs-through-autograd: same results
+    args.relax_amd_single_pass = "auto"
+    lib_reducer = get_sum_of_sample_mean(tot, resp, dbatch["loss_masks"], False)
+    hd = hid.to(dev).requires_grad_()
+    dhead.weight.grad = None
+    loss, _ = relax_amd.sft_loss_function_chunked(args, dbatch, hd, lambda x: lib_reducer(x),
+                                                  lm_head_forward=dhead.forward)
+    loss.backward()
+    assert abs(loss.item() - want.item()) < 2e-3 * len(resp)
+    torch.testing.assert_close(hd.grad.float().cpu(), hc.grad.float(), atol=5e-3, rtol=2 * BF16_ULP)
     # the same loss from materialised logits
     logits = (hid[0].to(dev) @ dhead.weight.detach().t()).float().unsqueeze(0).requires_grad_()
     loss2, _ = relax_amd.sft_loss_function(args, dbatch, logits, None)
