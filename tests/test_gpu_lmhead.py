@@ -426,6 +426,30 @@ def test_full_size_forward_and_gradient_properties():
     want = -adv[pick, None] * (w.detach()[tok[pick]].float() - p @ w.detach().float())
     torch.testing.assert_close(hid.grad[pick].float(), want, atol=2e-3 * want.abs().max().item(), rtol=2 * BF16_ULP)
 
+    # the same step with one projection (four slabs of 8192 rows whose logits become their gradient in place): the
+    # same identities, and gradients that agree with the two-projection ones up to the bf16 rounding of the logits
+    from relax_amd.lm_head import lm_head_token_local_step
+
+    hid2, w2 = hid.detach().clone().requires_grad_(), w.detach().clone().requires_grad_()
+    loss, lp2, ent2 = lm_head_token_local_step(hid2, w2, tok, lambda b, e, lp_, _: -(adv[b:e] * lp_).sum(), 1.0,
+                                               with_entropy=True)
+    # its statistics come from the logits rounded to bf16 (the reference's numerics: F.linear in bf16, then .float())
+    ref = torch.log_softmax((hid.detach()[idx] @ w.detach().t()).float(), -1)
+    torch.testing.assert_close(lp2[idx], ref[torch.arange(idx.numel(), device=dev), tok[idx]], atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent2[idx], -(ref.exp() * ref).sum(-1), atol=2e-3, rtol=0)
+    del ref
+    assert (lp2 - lp.detach()).abs().max().item() < 4e-2  # one bf16 ulp of a target logit of magnitude < 8
+    assert abs(loss.item() + (adv * lp.detach()).sum().item()) < 2e-3
+    loss.backward()
+    col = w2.grad.float().sum(0)
+    assert col.abs().max().item() < 2e-3 * max(1.0, w2.grad.float().abs().sum(0).max().item())
+    torch.testing.assert_close(hid2.grad[pick].float(), want, atol=2e-3 * want.abs().max().item(), rtol=2 * BF16_ULP)
+    scale_h, scale_w = hid.grad.float().abs().max().item(), w.grad.float().abs().max().item()
+    torch.testing.assert_close(hid2.grad.float(), hid.grad.float(), atol=2e-2 * scale_h, rtol=4 * BF16_ULP)
+    for r0 in range(0, v, 16384):  # in pieces: a full fp32 copy of both weight gradients is 5 GB
+        torch.testing.assert_close(w2.grad[r0:r0 + 16384].float(), w.grad[r0:r0 + 16384].float(), atol=2e-2 * scale_w,
+                                   rtol=4 * BF16_ULP)
+
 
 def test_sft_losses_plain_and_with_deferred_lm_head_vs_oracle():
     """sft_loss_function on logits and sft_loss_function_chunked on hidden states + LM-head weight (handed over as a
