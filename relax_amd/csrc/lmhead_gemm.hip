@@ -219,9 +219,12 @@ __device__ __forceinline__ void gemm_slice_sync() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
-template <bool AKM, bool BKM>
+// `init_acc(acc)` gives the accumulators their starting values (zeros, or the earlier partial sums of an accumulating
+// product); it runs after the first three slices have been requested, so whatever it loads travels with them.
+template <bool AKM, bool BKM, typename InitAcc>
 __device__ __forceinline__ void gemm_pipeline(const GemmRing ring, const GemmOperand& A, const GemmOperand& B,
-                                              int64_t a0, int64_t b0, int nk, floatx16 (&acc)[4][4]) {
+                                              int64_t a0, int64_t b0, int nk, floatx16 (&acc)[4][4],
+                                              InitAcc&& init_acc) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wa = wave >> 1, wb = wave & 1;
   GemmCopier<AKM> ac;
   GemmCopier<BKM> bc;
@@ -282,10 +285,10 @@ __device__ __forceinline__ void gemm_pipeline(const GemmRing ring, const GemmOpe
     });
   };
 
-  lm_zero_acc(acc);
   copy_all(0, 0);
   copy_all(1, 1);
   copy_all(2, 2);
+  init_acc(acc);
   gemm_slice_sync();
 #pragma unroll
   for (int n = 0; n < kReads; ++n) read_one(0, 0, n, f0);
@@ -341,7 +344,31 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_gemm_kernel(GemmOperand 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wa = wave >> 1, wb = wave & 1;
   const int64_t a0 = int64_t(ta) * kLmTile, b0 = int64_t(tb) * kLmTile;
   floatx16 acc[4][4];
-  gemm_pipeline<AKM, BKM>(GemmRing{{a0s, a1s, a2s, a3s}, {b0s, b1s, b2s, b3s}}, A, B, a0, b0, nk, acc);
+  const GemmRing ring{{a0s, a1s, a2s, a3s}, {b0s, b1s, b2s, b3s}};
+  if (OUT == kGemmOutF32Accumulate) {
+    // the product is added to what c_out holds: the tile's earlier values are the accumulators' starting point, read
+    // while the first slices of the operands are on their way, and the epilogue is a plain store
+    const float* c = static_cast<const float*>(c_out);
+    gemm_pipeline<AKM, BKM>(ring, A, B, a0, b0, nk, acc, [&](floatx16 (&acc_)[4][4]) {
+      const int64_t bcol = b0 + wb * 128 + (lane & 31);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int64_t arow = a0 + wa * 128 + i * 32 + 4 * (lane >> 5);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int64_t a = arow + 8 * (r >> 2) + (r & 3), b = bcol + j * 32;
+            acc_[i][j][r] = (a < ma && b < mb) ? c[a * c_stride + b] : 0.f;
+          }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(kLmWaitCopies);  // everything requested so far, the three slices included
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  } else {
+    gemm_pipeline<AKM, BKM>(ring, A, B, a0, b0, nk, acc, [](floatx16 (&acc_)[4][4]) { lm_zero_acc(acc_); });
+  }
   if (OUT == kGemmOutBf16) {
     LmSlabWriter writer;
     writer.init(static_cast<uint16_t*>(c_out), c_stride, ma, mb, b0, wa, wb, lane);
@@ -361,32 +388,21 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_gemm_kernel(GemmOperand 
     float* c = static_cast<float*>(c_out);
     const int64_t bcol = b0 + wb * 128 + (lane & 31);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int64_t arow = a0 + wa * 128 + i * 32 + 4 * (lane >> 5);
-      // accumulation: the 64 earlier values of this row of blocks are requested together, one memory round trip per
-      // row of blocks instead of one per block
-      float prev[4][16];
-      if (OUT == kGemmOutF32Accumulate) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int64_t a = arow + 8 * (r >> 2) + (r & 3), b = bcol + j * 32;
-            prev[j][r] = (a < ma && b < mb) ? c[a * c_stride + b] : 0.f;
-          }
-      }
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const floatx16 blk = acc[i][j];
         const int64_t b = bcol + j * 32;
+        const int64_t arow = a0 + wa * 128 + i * 32 + 4 * (lane >> 5);
+        if (b < mb) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int64_t a = arow + 8 * (r >> 2) + (r & 3);
-          if (a < ma && b < mb) c[a * c_stride + b] = OUT == kGemmOutF32Accumulate ? prev[j][r] + blk[r] : blk[r];
+          for (int r = 0; r < 16; ++r) {
+            const int64_t a = arow + 8 * (r >> 2) + (r & 3);
+            if (a < ma) c[a * c_stride + b] = blk[r];
+          }
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
-    }
   }
 }
 
