@@ -174,19 +174,32 @@ constexpr int kTkFastList = 2048;
 constexpr int kTkFastBatch = 6;  // loads in flight per thread within 64 registers (two workgroups per CU)
 constexpr int kTkGroups = 8192;  // groups of eight vectors the shortcut keeps a maximum for (vocab <= 524288 at 16 bit)
 // The shortcut's bound, shared by the selection kernel and the fused log-prob + selection kernel: `best` is each
-// thread's largest key.  Returns, as a float, the lower end of the 12-bit bin that holds the k-th largest of the thread
-// maxima (at most the 1024-th): !(v < bound) holds for every value whose key is at or above that bin (and for NaN, and
-// for -0 against a bound of +0: a few candidates more never hurt).  Clears *count for the collection that follows.
+// thread's largest key.  Finds the k-th largest of the thread maxima (at most the 1024-th) to 24 bits -- the 12-bit bin
+// that holds it, then the 12-bit sub-bin inside that bin -- and returns the lower end of that sub-bin as a float:
+// !(v < bound) holds for every value whose key is at or above it (and for NaN, and for -0 against a bound of +0: a
+// few candidates more never hurt).  The first 12 bits alone (sign, exponent, three mantissa bits) would put the bound
+// up to an eighth below the value and triple the candidates of a Gaussian row.  *floor_key receives the bound as a
+// key; *count is cleared for the collection that follows.
 __device__ __forceinline__ float tk_fast_floor(uint32_t best, int k, uint32_t* tot, uint32_t* wave_part,
-                                               uint32_t* found, uint32_t* count) {
+                                               uint32_t* found, uint32_t* count, uint32_t* floor_key) {
   const int tid = threadIdx.x;
+  const uint32_t wanted = uint32_t(k) < uint32_t(kTkThreads) ? uint32_t(k) : uint32_t(kTkThreads);
   for (int d = tid; d < kTkBins; d += kTkThreads) tot[d] = 0u;
   if (tid == 0) *count = 0u;
   __syncthreads();
   atomicAdd(&tot[best >> (32 - kTkDigitBits)], 1u);
   __syncthreads();
-  tk_locate(tot, wave_part, found, uint32_t(k) < uint32_t(kTkThreads) ? uint32_t(k) : uint32_t(kTkThreads));
-  return tk_value(found[0] << (32 - kTkDigitBits));
+  tk_locate(tot, wave_part, found, wanted);
+  const uint32_t bin = found[0], still = wanted - found[1];  // the still-th largest inside the bin is the one
+  __syncthreads();  // everyone has read found[] and tot[]
+  for (int d = tid; d < kTkBins; d += kTkThreads) tot[d] = 0u;
+  __syncthreads();
+  if ((best >> (32 - kTkDigitBits)) == bin) atomicAdd(&tot[(best >> (32 - 2 * kTkDigitBits)) & (kTkBins - 1)], 1u);
+  __syncthreads();
+  tk_locate(tot, wave_part, found, still);
+  const uint32_t key = (bin << (32 - kTkDigitBits)) | (found[0] << (32 - 2 * kTkDigitBits));
+  *floor_key = key;
+  return tk_value(key);
 }
 
 // One candidate of the shortcut's second look: kept when it is not below the bound.
@@ -289,8 +302,8 @@ __global__ __launch_bounds__(kTkThreads, 8) void topk_rows_fast_kernel(const T* 
       best = key > best ? key : best;
     });
   }
-  const float floor_value = tk_fast_floor(best, k, tot, wave_part, found, &count);
-  const uint32_t floor_key = found[0] << (32 - kTkDigitBits);
+  uint32_t floor_key;
+  const float floor_value = tk_fast_floor(best, k, tot, wave_part, found, &count, &floor_key);
   auto consider = [&](uint32_t idx, float v) { tk_fast_consider(idx, v, floor_value, list, &count); };
   if (by_group) {
     const u32x4* xv = reinterpret_cast<const u32x4*>(x);
@@ -325,9 +338,9 @@ __global__ __launch_bounds__(kTkThreads, 8) void topk_rows_fast_kernel(const T* 
 // workgroup width and order as the forward-only kernel, so log-probs and entropy are bit-identical to that kernel's.
 // The scan already takes the maximum of every batch of elements a lane absorbs (it rescales its sums by it); its
 // observer keeps those maxima, one LDS word per lane and batch, and nothing else is added to the scan.  A lane's
-// largest is its thread maximum for the shortcut's bound, and the second look is lane-private: each lane walks its own
-// batches in the scan's order and reads again only those whose maximum reaches the bound (a few per cent of the row,
-// found in cache).  A row that holds NaN or +inf (its sum of exponentials is NaN) goes to the general kernel.
+// largest is its thread maximum for the shortcut's bound, and the second look is lane-private: each lane reads again
+// only those of its own batches whose maximum reaches the bound (a few per cent of the row, found in the memory-side
+// cache).  A row that holds NaN or +inf (its sum of exponentials is NaN) goes to the general kernel.
 // Built for rows of whole 16-byte vectors whose length selects the 1024-thread scan.
 constexpr int kTkScanSlots = 12;  // batches a lane may absorb: vocab / (kScanUnroll * 1024 * elements per vector) + 3
 
@@ -370,7 +383,7 @@ __global__ __launch_bounds__(kTkThreads, 8) void logprob_topk_fwd_kernel(
     if (tg >= 0 && tg < vocab) x_target = Row<T>::load1(x + tg);
   }
   TkScanHook hook{lane_max + tid, -__builtin_inff()};
-  SoftmaxAcc st = scan_row<T, true, false, kTkThreads>(x, vocab, c, hook);
+  SoftmaxAcc st = scan_row<T, true, true, kTkThreads>(x, vocab, c, hook);
   scan_block_merge<kTkThreads>(st, wave_state);
   if (tid == 0) {
     float lse, spx, ent, lp;
@@ -386,31 +399,61 @@ __global__ __launch_bounds__(kTkThreads, 8) void logprob_topk_fwd_kernel(
     if (tid == 0) needs_general[tok] = 1;
     return;
   }
-  const float floor_value = tk_fast_floor(tk_key(hook.best), k, tot, wave_part, found, &count);
+  uint32_t floor_key;
+  const float floor_value = tk_fast_floor(tk_key(hook.best), k, tot, wave_part, found, &count, &floor_key);
   // (tk_fast_floor ends with a barrier after the last reading of tot[]: the list may now overwrite it)
+  // Second look, lane-private.  A lane's batches are numbered in the scan's order: `nb` batches of kScanUnroll vectors
+  // at a stride of kTkThreads vectors, then single vectors.  Few lanes have a batch that reaches the bound and hardly
+  // any has more than two (a few hundred batches qualify in a row of 1024 lanes x 7), so the first two are found from
+  // the LDS words alone and their vectors requested together: one memory round trip instead of one per batch.
   const u32x4* xv = reinterpret_cast<const u32x4*>(x);
   const float* mine = lane_max + tid;
-  int64_t i = tid;
-  for (; i + int64_t(kScanUnroll - 1) * kTkThreads < nvec; i += int64_t(kScanUnroll) * kTkThreads, mine += kTkThreads) {
-    if (*mine < floor_value) continue;
-    u32x4 raw[kScanUnroll];
-#pragma unroll
-    for (int u = 0; u < kScanUnroll; ++u) raw[u] = load_stream(xv + i + int64_t(u) * kTkThreads);
-#pragma unroll
-    for (int u = 0; u < kScanUnroll; ++u) {
-      float v[VN];
-      Row<T>::unpack(raw[u], v);
-#pragma unroll
-      for (int e = 0; e < VN; ++e)
-        tk_fast_consider(uint32_t((i + int64_t(u) * kTkThreads) * VN + e), v[e], floor_value, list, &count);
+  const int nb = nvec >= int64_t(kScanUnroll - 1) * kTkThreads + tid + 1
+                     ? int((nvec - int64_t(kScanUnroll - 1) * kTkThreads - tid - 1) / (int64_t(kScanUnroll) * kTkThreads)) + 1
+                     : 0;
+  const int64_t single0 = int64_t(tid) + int64_t(nb) * kScanUnroll * kTkThreads;  // the lane's first single vector
+  const int ns = single0 < nvec ? int((nvec - single0 - 1) / kTkThreads) + 1 : 0;
+  auto slot_base = [&](int sl) -> int64_t {
+    return sl < nb ? int64_t(tid) + int64_t(sl) * kScanUnroll * kTkThreads : single0 + int64_t(sl - nb) * kTkThreads;
+  };
+  int hit0 = -1, hit1 = -1, resume = nb + ns;
+  for (int sl = 0; sl < nb + ns; ++sl) {
+    if (mine[sl * kTkThreads] < floor_value) continue;
+    if (hit0 < 0) {
+      hit0 = sl;
+    } else if (hit1 < 0) {
+      hit1 = sl;
+    } else {
+      resume = sl;
+      break;
     }
   }
-  for (; i < nvec; i += kTkThreads, mine += kTkThreads) {
-    if (*mine < floor_value) continue;
+  auto consider_vec = [&](const u32x4& raw, int64_t i) {
     float v[VN];
-    Row<T>::unpack(load_stream(xv + i), v);
+    Row<T>::unpack(raw, v);
 #pragma unroll
     for (int e = 0; e < VN; ++e) tk_fast_consider(uint32_t(i * VN + e), v[e], floor_value, list, &count);
+  };
+  if (hit0 >= 0) {  // a minority of the lanes
+    u32x4 raw0[kScanUnroll], raw1[kScanUnroll];
+    const int64_t b0 = slot_base(hit0), b1 = slot_base(hit1 >= 0 ? hit1 : hit0);
+    const int c0 = hit0 < nb ? kScanUnroll : 1, c1 = hit1 < 0 ? 0 : (hit1 < nb ? kScanUnroll : 1);
+#pragma unroll
+    for (int u = 0; u < kScanUnroll; ++u) {
+      if (u < c0) raw0[u] = load_stream(xv + b0 + int64_t(u) * kTkThreads);
+      if (u < c1) raw1[u] = load_stream(xv + b1 + int64_t(u) * kTkThreads);
+    }
+#pragma unroll
+    for (int u = 0; u < kScanUnroll; ++u) {
+      if (u < c0) consider_vec(raw0[u], b0 + int64_t(u) * kTkThreads);
+      if (u < c1) consider_vec(raw1[u], b1 + int64_t(u) * kTkThreads);
+    }
+    for (int sl = resume; sl < nb + ns; ++sl) {  // a third and further batches of one lane: one at a time
+      if (mine[sl * kTkThreads] < floor_value) continue;
+      const int64_t b = slot_base(sl);
+      const int c = sl < nb ? kScanUnroll : 1;
+      for (int u = 0; u < c; ++u) consider_vec(load_stream(xv + b + int64_t(u) * kTkThreads), b + int64_t(u) * kTkThreads);
+    }
   }
   tk_fast_finish(list, &count, k, tok, out_values, out_indices, needs_general, rank);
 }
