@@ -2,7 +2,10 @@
  * of include/relax_amd.h, no PyTorch.  It runs the log-prob / entropy forward and its dlogits backward on the
  * three-row case of the reference's tests/utils/training/test_ppo_logprob_entropy.py:174-263 (logits
  * [[1,2,3,4],[4,1,0.5,2],[-1,3,2,0]], tokens [3,0,1], weights [0.25,-0.5,1.5] / [0.55,-0.2,1.8]) and the reverse KL
- * of two rows, and compares with the closed forms evaluated here in double precision.  Exit status 0 = all good. */
+ * of two rows, and compares with the closed forms evaluated here in double precision; then the one-read log-prob +
+ * top-K entry point on the same rows (k = 2) and the group-normalised rewards of the reference's GRPO literal
+ * (tests/utils/training/test_rloo_advantages.py:160-172: rewards [0,1,0,1] in one group -> (r - 0.5) / (std + 1e-6)
+ * with the sample standard deviation) and its leave-one-out brute force.  Exit status 0 = all good. */
 #include <hip/hip_runtime_api.h>
 #include <math.h>
 #include <stdint.h>
@@ -108,6 +111,63 @@ int main(void) {
       const double p = exp(logits[i][v] - lse);
       const double want = w_lp[i] * ((v == tokens[i]) - p) + w_ent[i] * p * (px - logits[i][v]);
       ok &= close_enough("dlogits", i * V + v, grad[i][v], want, 2e-6);
+    }
+  }
+  /* log-probs + entropy + the two largest logits of every row from one entry point */
+  {
+    enum { K = 2 };
+    float *d_lp2 = to_device(NULL, N * sizeof(float)), *d_vals = to_device(NULL, N * K * sizeof(float));
+    int64_t* d_idx = to_device(NULL, N * K * sizeof(int64_t));
+    uint8_t* d_flags = to_device(NULL, N);
+    if (!d_lp2 || !d_vals || !d_idx || !d_flags) return 2;
+    CHECK_LIB(relax_amd_logprob_entropy_topk_fwd(d_logits, RELAX_AMD_F32, N, V, V, NULL, (const int64_t*)d_tokens, 1.0f,
+                                                 K, d_lp2, NULL, NULL, NULL, d_vals, d_idx, d_flags, stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    float lp2[N], vals[N][K];
+    int64_t idx[N][K];
+    CHECK_HIP(hipMemcpy(lp2, d_lp2, sizeof lp2, hipMemcpyDeviceToHost));
+    CHECK_HIP(hipMemcpy(vals, d_vals, sizeof vals, hipMemcpyDeviceToHost));
+    CHECK_HIP(hipMemcpy(idx, d_idx, sizeof idx, hipMemcpyDeviceToHost));
+    const int64_t want_idx[N][K] = {{3, 2}, {0, 3}, {1, 2}};
+    for (int i = 0; i < N; ++i) {
+      ok &= close_enough("topk log_prob", i, lp2[i], lp[i], 0.0);
+      for (int k = 0; k < K; ++k) {
+        ok &= close_enough("topk index", i * K + k, (double)idx[i][k], (double)want_idx[i][k], 0.0);
+        ok &= close_enough("topk value", i * K + k, vals[i][k], logits[i][want_idx[i][k]], 0.0);
+      }
+    }
+  }
+  /* group-normalised rewards: mean / sample-std normalisation and leave-one-out baselines of one group of four */
+  {
+    enum { G = 4 };
+    const float rewards[G] = {0, 1, 0, 1};
+    const int32_t group[G] = {0, 0, 0, 0};
+    void* d_r = to_device(rewards, sizeof rewards);
+    void* d_g = to_device(group, sizeof group);
+    float* d_out = to_device(NULL, sizeof rewards);
+    int32_t* d_cnt = to_device(NULL, sizeof group);
+    if (!d_r || !d_g || !d_out || !d_cnt) return 2;
+    float out[G];
+    int32_t cnt[G];
+    CHECK_LIB(relax_amd_group_rewards(d_r, RELAX_AMD_F32, (const int32_t*)d_g, G, RELAX_AMD_GROUP_CENTER_STD, d_out, d_cnt,
+                                      stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    CHECK_HIP(hipMemcpy(out, d_out, sizeof out, hipMemcpyDeviceToHost));
+    CHECK_HIP(hipMemcpy(cnt, d_cnt, sizeof cnt, hipMemcpyDeviceToHost));
+    const double sd = sqrt(4 * 0.25 / 3.0);  /* sample standard deviation of {0,1,0,1} */
+    for (int i = 0; i < G; ++i) {
+      ok &= close_enough("grpo reward", i, out[i], (rewards[i] - 0.5) / (sd + 1e-6), 1e-6);
+      ok &= close_enough("group size", i, cnt[i], G, 0.0);
+    }
+    CHECK_LIB(relax_amd_group_rewards(d_r, RELAX_AMD_F32, (const int32_t*)d_g, G, RELAX_AMD_GROUP_RLOO, d_out, d_cnt,
+                                      stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    CHECK_HIP(hipMemcpy(out, d_out, sizeof out, hipMemcpyDeviceToHost));
+    for (int i = 0; i < G; ++i) {
+      double others = 0;
+      for (int j = 0; j < G; ++j)
+        if (j != i) others += rewards[j];
+      ok &= close_enough("rloo reward", i, out[i], rewards[i] - others / (G - 1), 1e-6);
     }
   }
   /* error path: the library reports instead of launching */
