@@ -322,6 +322,17 @@ def test_logprob_entropy_topk_one_read_equals_the_two_passes(n, v, k, dtype, tem
         assert (idx >= 0).all() and (idx < v).all()
         assert torch.equal(torch.gather(rows.float(), 1, idx), vals)
         assert (torch.sort(idx, dim=1).values.diff(dim=1) > 0).all() or k == 1  # distinct
+    # rows that are views into a wider matrix (row stride > vocabulary, still 16-byte aligned)
+    wide = torch.full((n, v + 64), 50.0, device=dev, dtype=dtype)   # what lies beyond a row would win every selection
+    wide[:, :v] = x
+    lpw, entw, _, _, valsw, idxw = ops.logprob_entropy_topk_fwd(wide[:, :v], tok, None, inv_t, k, True, with_values=True)
+    lpc, entc, _, _, valsc, idxc = ops.logprob_entropy_topk_fwd(x, tok, None, inv_t, k, True, with_values=True)
+    assert torch.equal(lpw.nan_to_num(), lpc.nan_to_num()) and torch.equal(entw.nan_to_num(), entc.nan_to_num())
+    assert torch.equal(valsw, valsc)
+    plain = torch.ones(n, dtype=torch.bool, device=dev)
+    plain[[3, 5]] = False  # rows with tens of thousands of exact ties: which of the tied entries leave is not fixed
+    assert torch.equal(idxw[plain], idxc[plain])
+    assert torch.equal(torch.gather(x.float(), 1, idxw), valsw)
     # without entropy and without values: the optional outputs are really optional
     lp3, ent3, lse3, spx3, vals3, idx3 = ops.logprob_entropy_topk_fwd(x, tok, None, inv_t, k, False)
     assert ent3 is None and spx3 is None and vals3 is None
