@@ -545,14 +545,11 @@ def run_actor_fwd_topk(a, dev) -> None:
         dom, dom_name = kernel_ms["topk_rows"], "topk_rows_fast_kernel<bf16_t, true>"
     else:
         dom, dom_name = kernel_ms["logprob_entropy_fwd"], "logprob_entropy_fwd_kernel<bf16_t, true, 1024>"
-    achieved = row_bytes / (dom * 1e-3) / 1e9
     emit(a, n_tokens, wall,
          f"actor forward-only pass with student top-{a.topk} ids: {a.seqs} seqs x {a.seq_len} tokens x V={a.vocab} bf16 "
          f"logits, log-prob + entropy + top-K selection" + (" [torch.topk selection]" if a.vendor_topk else ""),
          {"rows": n_tokens, "vocab": a.vocab, "k": a.topk},
-         {"bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-          "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": row_bytes,
-          "avg_launch_ms": dom, "kernel_ms": kernel_ms}, None)
+         hbm_roofline(dom_name, dom, row_bytes, n_tokens, a.vocab, kernel_ms, wall * 1e3 / a.steps), None)
 
 
 def run_reverse_kl(a, dev) -> None:
