@@ -440,7 +440,7 @@ def test_sapo_temperature_pick_and_clip_fraction_threshold():
 
 
 def test_seq_mean_token_sum_token_loop():
-    # the aggregation of BASELINE config 4: every sequence's masked token SUM, averaged over the B sequences
+    # the aggregation of the packed varlen configuration: every sequence's masked token SUM, averaged over the B sequences
     # (fully masked sequences still count in B); the reference only has the plug-in point (loss.py:1062-1072)
     g = torch.Generator().manual_seed(5)
     lens = [5, 1, 8, 3, 4]
