@@ -127,26 +127,22 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
     const int64_t nvec = vocab / VN;
     const int64_t tvec = (tg >= 0 && tg < nvec * VN) ? tg / VN : -1;
     const int tsub = int(tg % VN);
-    int64_t i = tid;
-    for (; i + int64_t(kScanUnroll - 1) * THREADS < nvec; i += int64_t(kScanUnroll) * THREADS) {
-      u32x4 raw[kScanUnroll];
-#pragma unroll
-      for (int u = 0; u < kScanUnroll; ++u) raw[u] = load_stream(xv + i + int64_t(u) * THREADS);
-#pragma unroll
-      for (int u = 0; u < kScanUnroll; ++u) {
-        float v[VN];
-        Row<T>::unpack(raw[u], v);
-#pragma unroll
-        for (int k = 0; k < VN; ++k) v[k] = fast_exp2(fmaf(v[k], c, k0)) * fmaf(v[k], a1, a0);
-        if (i + int64_t(u) * THREADS == tvec) {
-#pragma unroll
-          for (int k = 0; k < VN; ++k)
-            if (k == tsub) v[k] += hot;
-        }
-        store_stream(dv + i + int64_t(u) * THREADS, Row<T>::pack(v));
-      }
+    // The row is walked from its end to its beginning: what the scan read last is what the caches still hold, so the
+    // second walk starts where the first one stopped.  The lane's share is the scan's: `nfull` batches of kScanUnroll
+    // vectors at a stride of THREADS, then `nsingle` single vectors, then tail elements.
+    const int64_t nfull = nvec > int64_t(kScanUnroll - 1) * THREADS + tid
+                              ? (nvec - int64_t(kScanUnroll - 1) * THREADS - tid - 1) / (int64_t(kScanUnroll) * THREADS) + 1
+                              : 0;
+    const int64_t single0 = int64_t(tid) + nfull * kScanUnroll * THREADS;
+    const int64_t nsingle = single0 < nvec ? (nvec - single0 - 1) / THREADS + 1 : 0;
+    for (int64_t e = nvec * VN + tid; e < vocab; e += THREADS) {
+      const float xe = Row<T>::load1(x + e);
+      float g = fast_exp2(fmaf(xe, c, k0)) * fmaf(xe, a1, a0);
+      if (e == tg) g += hot;
+      Row<T>::store1(d + e, g);
     }
-    for (; i < nvec; i += THREADS) {
+    for (int64_t q = nsingle - 1; q >= 0; --q) {
+      const int64_t i = single0 + q * THREADS;
       float v[VN];
       Row<T>::unpack(load_stream(xv + i), v);
 #pragma unroll
@@ -158,11 +154,24 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
       }
       store_stream(dv + i, Row<T>::pack(v));
     }
-    for (int64_t e = nvec * VN + tid; e < vocab; e += THREADS) {
-      const float xe = Row<T>::load1(x + e);
-      float g = fast_exp2(fmaf(xe, c, k0)) * fmaf(xe, a1, a0);
-      if (e == tg) g += hot;
-      Row<T>::store1(d + e, g);
+    for (int64_t b = nfull - 1; b >= 0; --b) {
+      const int64_t i = int64_t(tid) + b * kScanUnroll * THREADS;
+      u32x4 raw[kScanUnroll];
+#pragma unroll
+      for (int u = kScanUnroll - 1; u >= 0; --u) raw[u] = load_stream(xv + i + int64_t(u) * THREADS);
+#pragma unroll
+      for (int u = kScanUnroll - 1; u >= 0; --u) {
+        float v[VN];
+        Row<T>::unpack(raw[u], v);
+#pragma unroll
+        for (int k = 0; k < VN; ++k) v[k] = fast_exp2(fmaf(v[k], c, k0)) * fmaf(v[k], a1, a0);
+        if (i + int64_t(u) * THREADS == tvec) {
+#pragma unroll
+          for (int k = 0; k < VN; ++k)
+            if (k == tsub) v[k] += hot;
+        }
+        store_stream(dv + i + int64_t(u) * THREADS, Row<T>::pack(v));
+      }
     }
   } else {
     for (int64_t e = tid; e < vocab; e += THREADS) {
