@@ -267,16 +267,32 @@ __global__ __launch_bounds__(THREADS) void reverse_kl_step_kernel(
       const u32x4 z = {0u, 0u, 0u, 0u};
       for (int64_t i = tid; i < nvec; i += THREADS) store_stream(dv + i, z);
     } else {
-      int64_t i = tid;
-      for (; i + int64_t(kKlUnroll - 1) * THREADS < nvec; i += int64_t(kKlUnroll) * THREADS) {
+      // from the rows' end to their beginning: the second walk starts on what the caches still hold from the scan.
+      // The lane's share is the scan's: `nfull` batches of kKlUnroll vectors at a stride of THREADS, then singles.
+      const int64_t nfull = nvec > int64_t(kKlUnroll - 1) * THREADS + tid
+                                ? (nvec - int64_t(kKlUnroll - 1) * THREADS - tid - 1) / (int64_t(kKlUnroll) * THREADS) + 1
+                                : 0;
+      const int64_t single0 = int64_t(tid) + nfull * kKlUnroll * THREADS;
+      const int64_t nsingle = single0 < nvec ? (nvec - single0 - 1) / THREADS + 1 : 0;
+      for (int64_t q2 = nsingle - 1; q2 >= 0; --q2) {
+        const int64_t i = single0 + q2 * THREADS;
+        float a[VN], b[VN];
+        Row<T>::unpack(load_stream(sv + i), a);
+        Row<T>::unpack(load_stream(tv + i), b);
+#pragma unroll
+        for (int k = 0; k < VN; ++k) a[k] = fast_exp2(fmaf(a[k], kLog2e, k0)) * fmaf(a[k] - b[k], gt, k1);
+        store_stream(dv + i, Row<T>::pack(a));
+      }
+      for (int64_t bi = nfull - 1; bi >= 0; --bi) {
+        const int64_t i = int64_t(tid) + bi * kKlUnroll * THREADS;
         u32x4 rs[kKlUnroll], rt[kKlUnroll];
 #pragma unroll
-        for (int u = 0; u < kKlUnroll; ++u) {
+        for (int u = kKlUnroll - 1; u >= 0; --u) {
           rs[u] = load_stream(sv + i + int64_t(u) * THREADS);
           rt[u] = load_stream(tv + i + int64_t(u) * THREADS);
         }
 #pragma unroll
-        for (int u = 0; u < kKlUnroll; ++u) {
+        for (int u = kKlUnroll - 1; u >= 0; --u) {
           float a[VN], b[VN];
           Row<T>::unpack(rs[u], a);
           Row<T>::unpack(rt[u], b);
@@ -284,14 +300,6 @@ __global__ __launch_bounds__(THREADS) void reverse_kl_step_kernel(
           for (int k = 0; k < VN; ++k) a[k] = fast_exp2(fmaf(a[k], kLog2e, k0)) * fmaf(a[k] - b[k], gt, k1);
           store_stream(dv + i + int64_t(u) * THREADS, Row<T>::pack(a));
         }
-      }
-      for (; i < nvec; i += THREADS) {
-        float a[VN], b[VN];
-        Row<T>::unpack(load_stream(sv + i), a);
-        Row<T>::unpack(load_stream(tv + i), b);
-#pragma unroll
-        for (int k = 0; k < VN; ++k) a[k] = fast_exp2(fmaf(a[k], kLog2e, k0)) * fmaf(a[k] - b[k], gt, k1);
-        store_stream(dv + i, Row<T>::pack(a));
       }
     }
   }
