@@ -7,7 +7,9 @@ library runs both in one fused launch).  Workload = the Qwen3-8B-shaped
 actor step: 16 sequences x 4096 tokens = 65536 rows x 151936 vocabulary, logits ~ N(0, 3) with 5 % spiked rows,
 first 20 % of every sequence masked out.
 
-Prints ONE JSON line (metric, value, roofline of the dominant kernel, CPU baseline of the same arithmetic).
+Prints ONE JSON line (metric, value, roofline of the dominant kernel, CPU baseline of the same arithmetic).  The plain
+invocation then also runs the other configurations below (up to 10 timed steps each, about a minute in all) and
+reports them inside that line as ``other_workloads``; ``--no-secondary`` or ``--cpu-rows 0`` skips them.
 
 ``--workload`` selects the other configurations of the same path, each printed in the same format:
 ``cfg1`` (GRPO plumbing case: 512 responses x 256 tokens, fp32 logits [131072, 32000], rewards -> advantages -> loss),
@@ -258,8 +260,12 @@ def timed_steps(step, warmup: int, steps: int):
     return wall, kernel_ms, launches, out
 
 
+COLLECTED = None  # a list: emit() appends its line there instead of printing it
+
+
 def emit(a, n_tokens, wall, workload, config, roofline, cpu):
-    print(json.dumps({
+    out = COLLECTED.append if COLLECTED is not None else (lambda line: print(json.dumps(line)))
+    out(dict({
         "metric": METRIC, "value": n_tokens / (wall / a.steps), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": wall * 1e3 / a.steps, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": config.pop("logits_dtype", "bf16"), "data": "synthetic",
@@ -787,6 +793,9 @@ def main() -> int:
                     help="actor_fwd_topk: select with torch.topk instead of the library's kernel (comparison)")
     ap.add_argument("--two-launch", action="store_true",
                     help="use the separate forward / backward launches (the path GSPO takes) instead of the fused step")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="plain invocation only: skip the other configurations that otherwise run after the headline "
+                         "workload and ride along in its line as other_workloads")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB device copy, the known-size reference for FETCH_SIZE/WRITE_SIZE")
     a = ap.parse_args()
@@ -801,6 +810,13 @@ def main() -> int:
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if a.workload == "actor_step" and a.cpu_rows > 0 and not a.no_secondary:
+        return run_default_with_secondary(a, dev)
+    run_workload(a, dev)
+    return 0
+
+
+def run_workload(a, dev) -> None:
     if a.workload == "actor_step":
         run_actor_step(a, dev)
     elif a.workload == "cfg1":
@@ -817,6 +833,44 @@ def main() -> int:
         run_actor_fwd_topk(a, dev)
     else:
         run_varlen(a, dev, a.workload.split("_")[1])
+
+
+SECONDARY = ("lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "cfg1", "actor_fwd_topk")
+
+
+def run_default_with_secondary(a, dev) -> int:
+    """The plain invocation (no ``--workload``, CPU baseline on): the headline workload exactly as ``--workload
+    actor_step`` measures it, and after it the other configurations of the path with at most 10 timed steps each, so
+    that one run of this file on one box covers them all.  Their figures ride along in the headline line as
+    ``other_workloads`` (``ms_per_step``, ``tokens_per_s`` and the roofline block of each workload's own line); they
+    take about a minute and change nothing in the headline measurement, which is finished before they start."""
+    import copy
+    import gc
+
+    global COLLECTED
+    COLLECTED = []
+    run_actor_step(a, dev)
+    line = COLLECTED.pop()
+    others = {}
+    for name in SECONDARY:
+        gc.collect()
+        torch.cuda.empty_cache()
+        b = copy.copy(a)
+        b.workload, b.steps, b.warmup, b.cpu_rows, b.rows = name, min(a.steps, 10), min(a.warmup, 3), 0, 0
+        try:
+            run_workload(b, dev)
+            got = COLLECTED.pop()
+            others[name] = {"ms_per_step": got["ms_per_step"], "tokens_per_s": got["value"], "steps": got["steps"],
+                            "dtype": got["dtype"], "workload": got["config"]["workload"],
+                            "roofline": {k: v for k, v in got["roofline"].items()
+                                         if k in ("bound", "kernel", "achieved", "peak", "unit", "frac", "traffic",
+                                                  "avg_launch_ms", "kernel_ms")}}
+        except Exception as e:  # a secondary workload must not cost the headline line
+            others[name] = {"error": f"{type(e).__name__}: {e}"}
+            COLLECTED.clear()
+    COLLECTED = None
+    line["other_workloads"] = others
+    print(json.dumps(line))
     return 0
 
 
