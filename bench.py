@@ -842,8 +842,9 @@ def run_default_with_secondary(a, dev) -> int:
     """The plain invocation (no ``--workload``, CPU baseline on): the headline workload exactly as ``--workload
     actor_step`` measures it, and after it the other configurations of the path with at most 10 timed steps each, so
     that one run of this file on one box covers them all.  Their figures ride along in the headline line as
-    ``other_workloads`` (``ms_per_step``, ``tokens_per_s`` and the roofline block of each workload's own line); they
-    take about a minute and change nothing in the headline measurement, which is finished before they start."""
+    ``other_workloads`` (a few figures of each workload's own line, kept short: ``ms_per_step``, ``tokens_per_s``, the
+    dominant kernel with its launch time and roofline fraction); they take some ten seconds and change nothing in the
+    headline measurement, which is finished before they start."""
     import copy
     import gc
 
@@ -860,11 +861,11 @@ def run_default_with_secondary(a, dev) -> int:
         try:
             run_workload(b, dev)
             got = COLLECTED.pop()
-            others[name] = {"ms_per_step": got["ms_per_step"], "tokens_per_s": got["value"], "steps": got["steps"],
-                            "dtype": got["dtype"], "workload": got["config"]["workload"],
-                            "roofline": {k: v for k, v in got["roofline"].items()
-                                         if k in ("bound", "kernel", "achieved", "peak", "unit", "frac", "traffic",
-                                                  "avg_launch_ms", "kernel_ms")}}
+            r = got["roofline"]
+            others[name] = {"ms_per_step": round(got["ms_per_step"], 4), "tokens_per_s": round(got["value"]),
+                            "steps": got["steps"], "kernel": r["kernel"], "bound": r["bound"],
+                            "avg_launch_ms": round(r["avg_launch_ms"], 4), "achieved": round(r["achieved"], 1),
+                            "unit": r["unit"], "frac": round(r["frac"], 4)}
         except Exception as e:  # a secondary workload must not cost the headline line
             others[name] = {"error": f"{type(e).__name__}: {e}"}
             COLLECTED.clear()
