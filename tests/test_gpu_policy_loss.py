@@ -817,6 +817,93 @@ def test_full_size_packed_varlen_gspo_and_cispo_properties():
     assert changed[inside & (flat_mask != 0)].float().mean().item() > 0.99
 
 
+def test_full_size_grpo_plumbing_case_rewards_to_dlogits():
+    """The GRPO plumbing configuration at its stated size: 64 prompts x group 8 = 512 responses x 256 tokens, fp32
+    logits [131072, 32000] ~ N(0, 2), Bernoulli(0.4) rewards, a trailing pad of 0..63 masked tokens per response,
+    group-normalised advantages (mean / std, eps 1e-6), PPO-clip 0.2, old = lp + N(0, 0.05), token-mean.  Rewards ->
+    advantages against the oracle for all 512 responses; log-probs, loss share and dlogits of 12 whole responses
+    (3072 rows, picked across the batch) against the oracle run on those rows; for every row: masked rows exactly zero,
+    gradient rows summing to zero."""
+    from types import SimpleNamespace
+
+    import relax_amd
+    from oracle import advantages as A
+    from relax_amd import utils as U
+
+    dev = require_gpu()
+    prompts, group, resp_len, v = 64, 8, 256, 32000
+    seqs, n = prompts * group, prompts * group * resp_len
+    announce("GRPO plumbing case, full size", n, v)
+    cpu = torch.Generator().manual_seed(0)
+    g = torch.Generator(device=dev).manual_seed(0)
+    logits = torch.empty((1, n, v), dtype=torch.float32, device=dev)
+    for s0 in range(0, n, 4096):
+        logits[0, s0:s0 + 4096] = torch.randn((4096, v), device=dev, generator=g) * 2.0
+    rewards = torch.bernoulli(torch.full((seqs,), 0.4), generator=cpu).tolist()
+    pads = torch.randint(0, 64, (seqs,), generator=cpu).tolist()
+    masks = []
+    for pad in pads:
+        m = torch.ones(resp_len)
+        if pad:
+            m[resp_len - pad:] = 0.0
+        masks.append(m)
+    kw = dict(advantage_estimator="grpo", eps_clip=0.2, eps_clip_high=0.2, rewards_normalization=True,
+              grpo_std_normalization=True, n_samples_per_prompt=group, global_batch_size=seqs)
+    args = P.make_args(**kw)
+    samples = [SimpleNamespace(group_index=i // group, get_reward_value=(lambda _a, r=r: r))
+               for i, r in enumerate(rewards)]
+    # rewards -> group-normalised rewards -> per-token advantages
+    raw, normed = U.post_process_rewards(args, samples, device=dev)
+    want_normed = A.group_normalise(rewards, [i // group for i in range(seqs)], group, "grpo", True)
+    assert raw == rewards
+    torch.testing.assert_close(torch.tensor(normed), want_normed, rtol=1e-6, atol=1e-7)
+    toks = [torch.randint(0, v, (resp_len,), device=dev, generator=g) for _ in range(seqs)]
+    dmasks = [m.to(dev) for m in masks]
+    with torch.no_grad():
+        _, out = relax_amd.get_log_probs_and_entropy(logits, args=args, unconcat_tokens=toks,
+                                                     total_lengths=[resp_len] * seqs,
+                                                     response_lengths=[resp_len] * seqs, with_entropy=False)
+    old = [lp + 0.05 * torch.randn(lp.shape, device=dev, generator=g) for lp in out["log_probs"]]
+    data = dict(log_probs=old, rewards=normed, loss_masks=dmasks)
+    relax_amd.compute_advantages_and_returns(args, data)
+    adv = data["advantages"]
+    for i in (0, 7, 8, 300, 511):
+        assert torch.equal(adv[i].cpu(), torch.full((resp_len,), float(want_normed[i])))
+    total_unmasked = float(sum(resp_len - pad for pad in pads))
+    batch = dict(unconcat_tokens=toks, total_lengths=[resp_len] * seqs, response_lengths=[resp_len] * seqs,
+                 loss_masks=dmasks, advantages=adv, log_probs=old,
+                 relax_amd_sample_denominators=torch.full((seqs,), total_unmasked, device=dev))
+    logits.requires_grad_()
+    loss, met = relax_amd.policy_loss_function(args, batch, logits, None)
+    loss.backward()
+    assert torch.isfinite(loss) and all(torch.isfinite(x) for x in met.values())
+    d = logits.grad[0]
+    flat_mask = torch.cat(dmasks)
+    for s0 in range(0, n, 16384):
+        rows = d[s0:s0 + 16384]
+        assert rows.sum(-1).abs().max().item() < 1e-6
+        assert (rows[flat_mask[s0:s0 + 16384] == 0] == 0).all()
+    # 12 whole responses against the oracle: their rows, their share of the token-mean loss, their gradient rows
+    picked = [0, 1, 63, 64, 100, 255, 256, 301, 400, 448, 510, 511]
+    rows = torch.cat([torch.arange(i * resp_len, (i + 1) * resp_len) for i in picked])
+    sub_logits = logits.detach()[0, rows.to(dev)].cpu().unsqueeze(0).requires_grad_()
+    sub = dict(unconcat_tokens=[toks[i].cpu() for i in picked], total_lengths=[resp_len] * len(picked),
+               response_lengths=[resp_len] * len(picked), loss_masks=[masks[i] for i in picked],
+               advantages=[adv[i].cpu() for i in picked], log_probs=[old[i].cpu() for i in picked])
+    reducer = R.make_reducer([resp_len] * len(picked), sub["loss_masks"],
+                             sample_denoms=[total_unmasked] * len(picked))
+    want, want_met = P.policy_loss_function(args, sub, sub_logits, reducer)
+    want.backward()
+    torch.testing.assert_close(d[rows.to(dev)].cpu(), sub_logits.grad[0], atol=3e-9, rtol=2e-4)
+    # the same 12 responses' share of the loss from the product: a second, small call on just those rows
+    lg2 = logits.detach()[0, rows.to(dev)].unsqueeze(0).clone().requires_grad_()
+    dsub = {k: ([x.to(dev) for x in val] if isinstance(val, list) and torch.is_tensor(val[0]) else val)
+            for k, val in sub.items()}
+    dsub["relax_amd_sample_denominators"] = torch.full((len(picked),), total_unmasked, device=dev)
+    got, _ = relax_amd.policy_loss_function(args, dsub, lg2, None)
+    assert abs(got.item() - want.item()) < 3e-5 * max(1.0, abs(want.item()))
+
+
 def _cfg4_lengths():
     """The benchmark's packed lengths: 8 draws from U[2048, 32768], the longest halved until the total fits 131072."""
     cpu = torch.Generator().manual_seed(0)
