@@ -3,11 +3,14 @@
 //
 // A 1024-thread workgroup holds a whole row in its vector registers (V = 151936 bf16 is 18992 16-byte vectors = 19 per
 // thread = 76 registers), so HBM sees exactly one read and one write per row and the second walk over the row costs no
-// cache or fabric traffic at all.  One such workgroup fits a CU; to keep loads, arithmetic and stores of different rows
-// overlapped the workgroups are persistent (one per CU, rows b, b + grid, ...) and roll the next row in behind the
-// stores of the current one: as soon as a vector's gradient has been stored, its registers receive the same vector of
-// the workgroup's next live row, and a few vectors behind the loads the next row's softmax scan follows.  No workgroup
-// waits for another; the loop bound is the only exit condition.
+// cache or fabric traffic at all.  One such workgroup fits a CU; the workgroups are persistent (one per CU, rows b,
+// b + grid, ...) and take a row in three steps: the resident row becomes its gradient in place; the gradient leaves in
+// one burst of stores and, into the registers those free, the workgroup's next live row arrives in one burst of loads
+// (304 KB out, 304 KB in, each contiguous); the new row's softmax scan follows its loads in their order.  Memory rewards
+// the long bursts: with a store and a load alternating vector by vector (and the scan trailing four vectors behind) the
+// launch took 6.95 - 7.05 ms on the 65536 x 151936 workload, in blocks of 4 / 8 / 12 vectors 6.77 / 6.63 / 6.57 ms, a
+// whole row at a time 6.49 ms, although nothing of one workgroup's arithmetic overlaps its own memory traffic any more
+// (other CUs' bursts fill the gaps).  No workgroup waits for another; the loop bound is the only exit condition.
 //
 // The number of vectors per thread is a template parameter (full vector positions NVF, plus one partially filled
 // position when PARTIAL), so the store / load loop is straight-line code without per-lane bounds checks.  That matters
@@ -36,7 +39,6 @@
 namespace relax_amd {
 
 constexpr int kResThreads = 1024;
-constexpr int kResLag = 4;  // vector positions between a load and the scan step that uses it
 
 // scan_absorb() over the values of kScanUnroll raw vectors, without holding them all unpacked
 template <typename T>
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(kResThreads, 4) void actor_step_resident_kernel(
     const int64_t* __restrict__ targets, float c, float inv_t, relax_amd_policy_loss_args a, float grad_scale,
     float* __restrict__ log_prob, float* __restrict__ entropy, float* __restrict__ lse_out,
     float* __restrict__ spx_out, T* __restrict__ dlogits, int64_t d_stride) {
-  constexpr int THREADS = kResThreads, LAG = kResLag, kU = kScanUnroll;
+  constexpr int THREADS = kResThreads, kU = kScanUnroll;
   constexpr int VN = Row<T>::kPerVec;
   constexpr int NV = NVF + (PARTIAL ? 1 : 0);  // vector positions per thread
   constexpr int kGroups = (NV + kU - 1) / kU;
@@ -233,14 +235,11 @@ __global__ __launch_bounds__(kResThreads, 4) void actor_step_resident_kernel(
     const int64_t tg = bc_target;
     const bool emit_zero = bc[4] != 0.f;  // both gradient coefficients vanish: a zero row, whatever the logits hold
 
-    // The gradient of this row goes out vector by vector; each vector's registers then receive the same vector of
-    // the next live row, and LAG positions behind the loads the next row's scan follows.
+    // The row becomes its gradient in place, vector by vector ...
     u32x4* dv = reinterpret_cast<u32x4*>(dlogits + row * d_stride);
     const u32x4* nxv = reinterpret_cast<const u32x4*>(logits + (has_next ? next : row) * row_stride);
     const int tvec = (tg >= 0 && tg < vocab) ? int(tg / VN) : -1;
     const int tsub = int(tg % VN);
-    st = SoftmaxAcc{kNegHuge, 0.f, 0.f};
-    bool grouped = true;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       int lane_id = tid;
@@ -255,27 +254,36 @@ __global__ __launch_bounds__(kResThreads, 4) void actor_step_resident_kernel(
         // row out to scratch (four waves per SIMD cover the latency of the exponentials)
         if (k == VN / 2 - 1) __builtin_amdgcn_sched_barrier(0);
       }
-      if (idx == tvec) {  // one lane of the workgroup per row; no memory operation inside, so waits stay countable
+      if (idx == tvec) {  // one lane of the workgroup per row
 #pragma unroll
         for (int k = 0; k < VN; ++k)
           if (k == tsub) v[k] += hot;
       }
-      u32x4 out = Row<T>::pack(v);
-      if (emit_zero) out = u32x4{0u, 0u, 0u, 0u};
-      if (has(j)) {
-        store_stream(dv + idx, out);
-        // without a next row the row itself is read again: a branch here would cost the precise wait counts, and
-        // the last row of a workgroup is one in hundreds
-        reg[j] = load_stream(nxv + idx);
-      }
+      reg[j] = emit_zero ? u32x4{0u, 0u, 0u, 0u} : Row<T>::pack(v);
       __builtin_amdgcn_sched_barrier(0);  // one vector at a time: hoisting the next one's unpacking spills
-      if (j - LAG - (kU - 1) >= 0 && (j - LAG - (kU - 1)) % kU == 0)
-        absorb_group((j - LAG - (kU - 1)) / kU, st, grouped);
     }
-    if (!has_next) return;
+    // ... leaves in one burst of stores, and the next live row arrives in one burst of loads into the same registers
+    // (without a next row the row itself is read again: a branch here would cost the precise wait counts, and the
+    // last row of a workgroup is one in hundreds)
 #pragma unroll
-    for (int g = 0; g < kGroups; ++g)
-      if (kU * g + kU - 1 + LAG > NV - 1) absorb_group(g, st, grouped);
+    for (int j = 0; j < NV; ++j) {
+      int lane_id = tid;
+      asm volatile("" : "+v"(lane_id));
+      if (has(j)) store_stream(dv + lane_id + j * THREADS, reg[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      int lane_id = tid;
+      asm volatile("" : "+v"(lane_id));
+      if (has(j)) reg[j] = load_stream(nxv + lane_id + j * THREADS);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (!has_next) return;
+    // the next row's scan, group by group as its vectors arrive (loads return in the order they were requested)
+    st = SoftmaxAcc{kNegHuge, 0.f, 0.f};
+    bool grouped = true;
+#pragma unroll
+    for (int g = 0; g < kGroups; ++g) absorb_group(g, st, grouped);
     row = next;
     tok = next_tok;
   }
