@@ -80,15 +80,18 @@ def hbm_roofline(kernel: str, launch_ms: float, necessary_bytes: float, rows: in
     return out
 
 
-def fused_step_kernel_name(vocab: int) -> str:
-    """Which kernel relax_amd_actor_step_fused runs for bf16 rows of ``vocab`` entries (the library's own rule)."""
-    nvec = vocab // 8
-    shape = (nvec // 1024, nvec % 1024 != 0)
-    if vocab % 8 == 0 and shape in ((18, True), (15, True), (16, False), (12, True)) \
-            and os.environ.get("RELAX_AMD_FUSED_STEP_KERNEL") != "cached":
-        return f"actor_step_resident_kernel<bf16_t, {shape[0]}, {str(shape[1]).lower()}>"
+def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
+    """Which kernel relax_amd_actor_step_fused runs for bf16 / fp32 rows of ``vocab`` entries (the library's own rule:
+    the register-resident kernel in workgroups as wide as the forward-only scan's, where the row shape is built)."""
+    per_vec, width, shapes = {"bf16_t": (8, 1024, ((18, True), (15, True), (16, False), (12, True))),
+                              "float": (4, 512, ((15, True),))}[dtype]
+    nvec = vocab // per_vec
     threads = 1024 if nvec >= 8192 else 512 if nvec >= 2048 else 256
-    return f"actor_step_fused_kernel<bf16_t, true, {threads}>"
+    shape = (nvec // width, nvec % width != 0)
+    if vocab % per_vec == 0 and threads == width and shape in shapes \
+            and os.environ.get("RELAX_AMD_FUSED_STEP_KERNEL") != "cached":
+        return f"actor_step_resident_kernel<{dtype}, {shape[0]}, {str(shape[1]).lower()}>"
+    return f"actor_step_fused_kernel<{dtype}, true, {threads}>"
 
 
 def kl_step_kernel_name(vocab: int) -> str:
@@ -679,7 +682,7 @@ def run_cfg1(a, dev) -> None:
          f"logits, group-normalised advantages, PPO-clip 0.2, token-mean, fwd + bwd to dlogits",
          {"rows": n, "live_rows": live, "vocab": v, "loss": float(loss.item()), "logits_dtype": "f32",
           "advantages_ms": adv_ms},
-         hbm_roofline("actor_step_fused_kernel<float, true, 512>", dom, row_bytes * (live + n), n, v, kernel_ms,
+         hbm_roofline(fused_step_kernel_name(v, "float"), dom, row_bytes * (live + n), n, v, kernel_ms,
                       wall * 1e3 / a.steps, survey_bytes=3.0 * row_bytes * n),
          out_cpu)
 

@@ -38,8 +38,6 @@
 
 namespace relax_amd {
 
-constexpr int kResThreads = 1024;
-
 // scan_absorb() over the values of kScanUnroll raw vectors, without holding them all unpacked
 template <typename T>
 __device__ __forceinline__ void absorb_raw_group(const u32x4* raw, float c, SoftmaxAcc& st) {
@@ -85,14 +83,21 @@ struct ResidentTokenData {
   int64_t tg;
 };
 
+// Workgroup width by element type: 16-bit rows in 1024-thread workgroups (one per CU), 32-bit rows in 512-thread
+// workgroups (two per CU; only short rows fit: a thread can give the row about 64 of its 128 registers).
+template <typename T>
+constexpr int resident_threads() {
+  return sizeof(T) == 2 ? 1024 : 512;
+}
+
 template <typename T, int NVF, bool PARTIAL>
-__global__ __launch_bounds__(kResThreads, 4) void actor_step_resident_kernel(
+__global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_kernel(
     const T* __restrict__ logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
     const int32_t* __restrict__ token_of_row, const int32_t* __restrict__ sample_ids,
     const int64_t* __restrict__ targets, float c, float inv_t, relax_amd_policy_loss_args a, float grad_scale,
     float* __restrict__ log_prob, float* __restrict__ entropy, float* __restrict__ lse_out,
     float* __restrict__ spx_out, T* __restrict__ dlogits, int64_t d_stride) {
-  constexpr int THREADS = kResThreads, kU = kScanUnroll;
+  constexpr int THREADS = resident_threads<T>(), kU = kScanUnroll;
   constexpr int VN = Row<T>::kPerVec;
   constexpr int NV = NVF + (PARTIAL ? 1 : 0);  // vector positions per thread
   constexpr int kGroups = (NV + kU - 1) / kU;
@@ -289,35 +294,6 @@ __global__ __launch_bounds__(kResThreads, 4) void actor_step_resident_kernel(
   }
 }
 
-template <typename T>
-struct ResidentSupported {
-  static constexpr bool value = false;
-};
-template <>
-struct ResidentSupported<bf16_t> {
-  static constexpr bool value = true;
-};
-template <>
-struct ResidentSupported<f16_t> {
-  static constexpr bool value = true;
-};
-
-template <typename T>
-int launch_actor_step_resident(const T* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
-                               const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,
-                               float inv_t, const relax_amd_policy_loss_args& a, float grad_scale, float* log_prob,
-                               float* entropy, float* lse, float* spx, T* dlogits, int64_t d_stride,
-                               int compute_units, hipStream_t stream) {
-  if constexpr (!ResidentSupported<T>::value) {
-    return RELAX_AMD_EUNSUPPORTED;
-  } else {
-    constexpr int VN = Row<T>::kPerVec;
-    if (vocab % VN != 0 || scan_threads(vocab, VN) != kResThreads) return RELAX_AMD_EUNSUPPORTED;
-    const int64_t nvec = vocab / VN;
-    const int full = int(nvec / kResThreads);
-    const bool partial = nvec % kResThreads != 0;
-    const int64_t blocks = n_rows < compute_units ? n_rows : compute_units;
-    const dim3 grid(static_cast<unsigned>(blocks)), block(kResThreads);
 #define RELAX_AMD_RESIDENT(NVF, PARTIAL)                                                                             \
   if (full == NVF && partial == PARTIAL) {                                                                            \
     hipLaunchKernelGGL((actor_step_resident_kernel<T, NVF, PARTIAL>), grid, block, 0, stream, logits, row_stride,    \
@@ -325,16 +301,35 @@ int launch_actor_step_resident(const T* logits, int64_t row_stride, int64_t voca
                        log_prob, entropy, lse, spx, dlogits, d_stride);                                              \
     return check_launch("actor_step_resident");                                                                      \
   }
+
+template <typename T>
+int launch_actor_step_resident(const T* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
+                               const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,
+                               float inv_t, const relax_amd_policy_loss_args& a, float grad_scale, float* log_prob,
+                               float* entropy, float* lse, float* spx, T* dlogits, int64_t d_stride,
+                               int compute_units, hipStream_t stream) {
+  constexpr int VN = Row<T>::kPerVec, THREADS = resident_threads<T>();
+  // the workgroup must be as wide as the forward-only kernel's for this row length: both scan in the same order
+  if (vocab % VN != 0 || scan_threads(vocab, VN) != THREADS) return RELAX_AMD_EUNSUPPORTED;
+  const int64_t nvec = vocab / VN;
+  const int full = int(nvec / THREADS);
+  const bool partial = nvec % THREADS != 0;
+  const int64_t slots = int64_t(compute_units) * (1024 / THREADS);  // persistent workgroups: as many as fit the chip
+  const dim3 grid(static_cast<unsigned>(n_rows < slots ? n_rows : slots)), block(THREADS);
+  if constexpr (sizeof(T) == 2) {
     // vocabularies of 151936 / 152064 (18992 / 19008 vectors), 128256 / 129280 (16032 / 16160), 131072 (16384),
     // 100352 / 102400 (12544 / 12800) entries
     RELAX_AMD_RESIDENT(18, true)
     RELAX_AMD_RESIDENT(15, true)
     RELAX_AMD_RESIDENT(16, false)
     RELAX_AMD_RESIDENT(12, true)
-#undef RELAX_AMD_RESIDENT
-    return RELAX_AMD_EUNSUPPORTED;
+  } else {
+    // fp32 rows of 32000 entries (8000 vectors: 15 per thread and 320 lanes with a sixteenth)
+    RELAX_AMD_RESIDENT(15, true)
   }
+  return RELAX_AMD_EUNSUPPORTED;
 }
+#undef RELAX_AMD_RESIDENT
 
 template int launch_actor_step_resident<float>(const float*, int64_t, int64_t, int64_t, const int32_t*, const int32_t*,
                                                const int64_t*, float, const relax_amd_policy_loss_args&, float, float*,

@@ -1410,12 +1410,12 @@ def test_custom_loss_function_path_dispatch():
 
 @pytest.mark.parametrize("v,dtype,n_samples", [(100352, torch.bfloat16, 18), (128256, torch.float16, 18),
                                                 (131072, torch.bfloat16, 18), (151936, torch.bfloat16, 18),
-                                                (65536, torch.bfloat16, 18)])
+                                                (65536, torch.bfloat16, 18), (32000, torch.float32, 40)])
 def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples):
     """More logits rows than persistent workgroups, so every workgroup of the register-resident kernel rolls several
     rows through its registers (prompt rows, fully masked samples and masked tokens in between), for every row shape
-    the kernel is built for (12 / 15 / 18 full vectors per thread plus a partial one, 16 exactly) and one it is not
-    (65536: two-walk kernel): same loss bits as the two-launch path, gradients equal to it and to the oracle."""
+    the kernel is built for (12 / 15 / 18 full vectors per thread plus a partial one, 16 exactly; fp32 rows of 32000
+    entries in 512-thread workgroups, two per CU) and one it is not (65536: two-walk kernel): same loss bits as the two-launch path, gradients equal to it and to the oracle."""
     import relax_amd
 
     dev = require_gpu()
@@ -1425,7 +1425,7 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
     resp = [int(torch.randint(1, t, (1,), generator=g)) for t in tot]
     logits, batch = _make_batch(29, tot, resp, v, dtype)
     batch["loss_masks"][3] = torch.zeros_like(batch["loss_masks"][3])
-    assert sum(tot) > 600
+    assert sum(tot) > (600 if dtype != torch.float32 else 1200)
     db = _to_dev(batch, dev)
     kw = dict(eps_clip_high=0.28, use_kl_loss=True, kl_loss_coef=1e-3, kl_loss_type="k3", entropy_coef=0.01)
     outs = {}
@@ -1435,7 +1435,7 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
         loss.backward()
         outs[mode] = (loss.detach(), met, lg.grad)
     assert torch.equal(outs["auto"][0], outs["off"][0])
-    ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7, torch.float32: 1e-5}[dtype]
     torch.testing.assert_close(outs["auto"][2].float(), outs["off"][2].float(), atol=1e-6, rtol=ulp)
     lo = logits.float().clone().requires_grad_()
     want, _ = P.policy_loss_function(P.make_args(**kw), dict(batch), lo, R.make_reducer(resp, batch["loss_masks"]))
@@ -1445,21 +1445,23 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
     torch.testing.assert_close(outs["auto"][2].float().cpu(), lo.grad, atol=tol, rtol=max(ulp, 1e-5))
 
 
+@pytest.mark.parametrize("v,dtype,n_rows", [(100352, torch.bfloat16, 700), (32000, torch.float32, 1500)])
 @pytest.mark.parametrize("pattern", ["all_dead", "one_live_last", "few_live", "random", "all_live_no_map",
                                      "zero_advantage"])
-def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, monkeypatch):
+def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dtype, n_rows, monkeypatch):
     """The two kernels behind relax_amd_actor_step_fused, switched with RELAX_AMD_FUSED_STEP_KERNEL, on row / token
     layouts that stress the persistent loop of the register-resident one: no live row at all, a single live row at
     the very end, fewer live rows than workgroups, random prompt rows and masked tokens over several rows per
     workgroup, no row map (every row scores its own token), and tokens whose gradient coefficients vanish (zero
-    rows without a look at the logits).  Every output must be bit-identical."""
+    rows without a look at the logits); on 16-bit rows of 12 full vectors per thread plus a partial one (one
+    1024-thread workgroup per CU) and on fp32 rows of 32000 entries (two 512-thread workgroups per CU).  Every output
+    must be bit-identical."""
     from relax_amd import ops
 
     dev = require_gpu()
-    announce("resident vs two-walk", pattern)
-    v, n_rows = 100352, 700  # 12 full vectors per thread + a partial one
+    announce("resident vs two-walk", pattern, v, dtype)
     g = torch.Generator().manual_seed(len(pattern))
-    logits = (torch.randn(n_rows, v, generator=g) * 2).bfloat16().to(dev)
+    logits = (torch.randn(n_rows, v, generator=g) * 2).to(dtype).to(dev)
     if pattern == "all_live_no_map":
         token_of_row, n_tok = None, n_rows
     else:
@@ -1496,7 +1498,8 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, monkey
         monkeypatch.setenv("RELAX_AMD_FUSED_STEP_KERNEL", kind)
         out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, token_of_row, sample_ids, n_tok, 1.0, 1.0, **kw)
         torch.cuda.synchronize()
-        results[kind] = dict(lp=lp, ent=ent, lse=lse, spx=spx, d=d.view(torch.int16), coef=out["coef_log_prob"],
+        results[kind] = dict(lp=lp, ent=ent, lse=lse, spx=spx, coef=out["coef_log_prob"],
+                             d=d.view(torch.int16 if dtype != torch.float32 else torch.int32),
                              coef_ent=out["coef_entropy"], metrics=out["metrics"])
     for key, want in results["cached"].items():
         got = results["resident"][key]
