@@ -190,7 +190,31 @@ typedef struct relax_amd_policy_loss_args {
   const float* distill_teacher_log_prob;
   int32_t distill_kl_kind;
   float distill_min_clamp, distill_token_clip, distill_is_clip;
+  /* optional, relax_amd_actor_step_fused only (relax_amd_policy_loss leaves the signal out: with topk_ids set it
+   * treats extra_coef_log_prob as absent and touches none of the topk_* fields): the top-K distillation signal of
+   * compute_policy_opd_loss (opd_utils.py:1368-1455 with compute_log_probs_on_topk_token_ids, :1022-1094, and
+   * compute_opd_kl_topk, :1190-1228) evaluated next to each row's log-sum-exp, so that its gradient leaves in the
+   * step's one dlogits launch.  With topk_ids set, extra_coef_log_prob[t] is the weight of token t's signal in the
+   * loss; the kernel gathers the row's logits at topk_ids[t, :], forms the per-token KL, clips it from above at
+   * distill_token_clip, multiplies by min(exp(log_prob - old_log_prob), distill_is_clip) taken as a constant (NaN
+   * switches either off), writes the un-clipped signal to topk_kl[t] and d loss / d log p[id_k] to topk_grad[t, k],
+   * and adds the sum of the latter to the multiple of the row's softmax it subtracts.  The caller then adds
+   * topk_grad * inv_temperature * grad_scale at the K ids of every row (relax_amd_sparse_row_add).  Rows the step does
+   * not read (both masks zero) leave their topk_kl / topk_grad entries untouched: zero them beforehand. */
+  const int64_t* topk_ids;              /* [n_tokens, topk_k]; < 0: sentinel (log-prob -inf, no gradient) */
+  const float* topk_teacher_log_prob;   /* [n_tokens, topk_k] */
+  const int32_t* topk_width;            /* optional [n_tokens]: entries of token t that exist (NULL = topk_k) */
+  const int32_t* topk_valid;            /* optional [n_tokens]: union mask, entries k >= topk_valid[t] are masked;
+                                           < 0 (or NULL) = no mask for that token */
+  int32_t topk_k;                       /* 1 .. RELAX_AMD_FUSED_TOPK_MAX */
+  int32_t topk_kl_mode, topk_norm_mode; /* RELAX_AMD_OPD_JSD / _LOW_VAR, RELAX_AMD_OPD_NORM_* */
+  int32_t topk_has_clamp;
+  float topk_jsd_alpha, topk_min_clamp;
+  float* topk_kl;                       /* out [n_tokens] */
+  float* topk_grad;                     /* out [n_tokens, topk_k] */
 } relax_amd_policy_loss_args;
+
+#define RELAX_AMD_FUSED_TOPK_MAX 256
 
 int relax_amd_policy_loss(const relax_amd_policy_loss_args* args, void* stream);
 

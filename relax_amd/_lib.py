@@ -52,7 +52,13 @@ class PolicyLossArgs(C.Structure):
         ("extra_coef_log_prob", _vp),
         ("distill_teacher_log_prob", _vp), ("distill_kl_kind", _i32),
         ("distill_min_clamp", _f32), ("distill_token_clip", _f32), ("distill_is_clip", _f32),
+        ("topk_ids", _vp), ("topk_teacher_log_prob", _vp), ("topk_width", _vp), ("topk_valid", _vp),
+        ("topk_k", _i32), ("topk_kl_mode", _i32), ("topk_norm_mode", _i32), ("topk_has_clamp", _i32),
+        ("topk_jsd_alpha", _f32), ("topk_min_clamp", _f32), ("topk_kl", _vp), ("topk_grad", _vp),
     ]
+
+
+FUSED_TOPK_MAX = 256
 
 
 SIGNATURES = {

@@ -22,6 +22,7 @@
 // (relax/backends/megatron/loss.py:961-1100).
 #include "device_utils.h"
 #include "loss_math.h"
+#include "opd_topk_math.h"
 #include "relax_amd.h"
 #include "row_scan.h"
 
@@ -55,6 +56,7 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
   __shared__ float wave_state[THREADS / kWave][3];
   __shared__ float bc[5];
   __shared__ int64_t bc_target;
+  __shared__ float topk_stage[2 * RELAX_AMD_FUSED_TOPK_MAX];
   const int tid = threadIdx.x;
   const int64_t row = blockIdx.x;
   T* d = dlogits + row * d_stride;
@@ -93,24 +95,37 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
   // pass 1: cached loads, the row stays in L2 / the memory-side cache for pass 2
   SoftmaxAcc st = scan_row<T, VEC, false, THREADS>(x, vocab, c);
   scan_block_merge<THREADS>(st, wave_state);
-  if (tid == 0) {
-    float lse, spx, ent, lp;
-    scan_finish(st, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
-    log_prob[tok] = lp;
-    entropy[tok] = ent;
-    lse_out[tok] = lse;
-    spx_out[tok] = spx;
-    const TokenResult tr = token_terms(a, in, lp, ent, false, 0.f, den, pg_den);
-    a.coef_log_prob[tok] = tr.coef_lp;
-    if (a.coef_entropy) a.coef_entropy[tok] = tr.coef_ent;
-    const float glp = tr.coef_lp * grad_scale, gh = tr.coef_ent * grad_scale;
-    const float b = gh * inv_t;
-    bc[0] = -lse * kLog2e;           // k0: p = exp2(x*c + k0)
-    bc[1] = -glp * inv_t + b * spx;  // a0
-    bc[2] = -b * inv_t;              // a1: d = p * (a0 + a1*x)
-    bc[3] = glp * inv_t;             // added at the target
-    bc[4] = (glp == 0.f && gh == 0.f) ? 1.f : 0.f;
-    bc_target = tg;
+  if (tid < kWave) {  // the first wave; thread 0 holds the merged state and the token's scalars
+    float lse = 0.f, spx = 0.f, ent = 0.f, lp = 0.f;
+    if (tid == 0) {
+      scan_finish(st, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
+      log_prob[tok] = lp;
+      entropy[tok] = ent;
+      lse_out[tok] = lse;
+      spx_out[tok] = spx;
+    }
+    // the top-K distillation signal, when configured: K gathered logits of this row against the log-sum-exp just found
+    float g_topk = 0.f;
+    if (a.topk_ids) {
+      const float lp0 = __shfl(lp, 0, kWave);
+      g_topk = topk_distill_row<T>(a, x, vocab, tok, __shfl(lse, 0, kWave), inv_t, lp0,
+                                   __shfl(in.has_old ? in.old_lp : lp, 0, kWave), __shfl(in.extra_lp, 0, kWave), tid,
+                                   topk_stage);
+    }
+    if (tid == 0) {
+      const TokenResult tr = token_terms(a, in, lp, ent, false, 0.f, den, pg_den);
+      a.coef_log_prob[tok] = tr.coef_lp;
+      if (a.coef_entropy) a.coef_entropy[tok] = tr.coef_ent;
+      const float glp = tr.coef_lp * grad_scale, gh = tr.coef_ent * grad_scale;
+      const float gsm = glp + g_topk * grad_scale;  // what the row's softmax is subtracted with
+      const float b = gh * inv_t;
+      bc[0] = -lse * kLog2e;           // k0: p = exp2(x*c + k0)
+      bc[1] = -gsm * inv_t + b * spx;  // a0
+      bc[2] = -b * inv_t;              // a1: d = p * (a0 + a1*x)
+      bc[3] = glp * inv_t;             // added at the target
+      bc[4] = (gsm == 0.f && glp == 0.f && gh == 0.f) ? 1.f : 0.f;
+      bc_target = tg;
+    }
   }
   __syncthreads();
   const float k0 = bc[0], a0 = bc[1], a1 = bc[2], hot = bc[3];
@@ -250,7 +265,9 @@ extern "C" int relax_amd_actor_step_fused(const void* logits, int dtype, int64_t
     set_error("actor_step_fused: NULL argument");
     return RELAX_AMD_EINVAL;
   }
-  if (const char* why = distill_args_error(*loss)) {
+  const char* why = distill_args_error(*loss);
+  if (!why) why = topk_distill_args_error(*loss);
+  if (why) {
     set_error("actor_step_fused: %s", why);
     return RELAX_AMD_EINVAL;
   }

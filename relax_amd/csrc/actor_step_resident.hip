@@ -34,6 +34,7 @@
 
 #include "device_utils.h"
 #include "loss_math.h"
+#include "opd_topk_math.h"
 #include "row_scan.h"
 
 namespace relax_amd {
@@ -90,7 +91,7 @@ constexpr int resident_threads() {
   return sizeof(T) == 2 ? 1024 : 512;
 }
 
-template <typename T, int NVF, bool PARTIAL>
+template <typename T, int NVF, bool PARTIAL, bool TOPK = false>
 __global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_kernel(
     const T* __restrict__ logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
     const int32_t* __restrict__ token_of_row, const int32_t* __restrict__ sample_ids,
@@ -104,6 +105,7 @@ __global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_
   __shared__ float wave_state[THREADS / kWave][3];
   __shared__ float bc[5];
   __shared__ int64_t bc_target;
+  __shared__ float topk_stage[TOPK ? 2 * RELAX_AMD_FUSED_TOPK_MAX : 1];
   const int tid = threadIdx.x;
   const bool wave0 = __builtin_amdgcn_readfirstlane(tid) < kWave;  // scalar: other waves branch around thread 0's work
   const int rem = int(vocab / VN) - NVF * THREADS;  // lanes that hold a vector at the partial position (host-checked)
@@ -208,13 +210,24 @@ __global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_
     const ResidentTokenData td = fetch_token(row, tok);
     scan_block_merge<THREADS>(st, wave_state);
     if (wave0) {
+      float lse = 0.f, spx = 0.f, ent = 0.f, lp = 0.f;
       if (tid == 0) {
-        float lse, spx, ent, lp;
         scan_finish(st, td.x_target, td.tg >= 0 && td.tg < vocab, inv_t, lse, spx, ent, lp);
         log_prob[tok] = lp;
         entropy[tok] = ent;
         lse_out[tok] = lse;
         spx_out[tok] = spx;
+      }
+      // the top-K distillation signal: K gathered logits of this row against the log-sum-exp just found
+      float g_topk = 0.f;
+      if constexpr (TOPK) {
+        int lane = tid;
+        asm volatile("" : "+v"(lane));
+        g_topk = topk_distill_row<T>(a, logits + row * row_stride, vocab, tok, __shfl(lse, 0, kWave), inv_t,
+                                     __shfl(lp, 0, kWave), __shfl(td.in.has_old ? td.in.old_lp : lp, 0, kWave),
+                                     __shfl(td.in.extra_lp, 0, kWave), lane, topk_stage);
+      }
+      if (tid == 0) {
         relax_amd_policy_loss_args al = a;
         // opaque copies: derived constants (1 + eps, ...) would otherwise be hoisted out of the row loop into vector
         // registers that every wave has to keep for thread 0's sake
@@ -224,12 +237,13 @@ __global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_
         a.coef_log_prob[tok] = tr.coef_lp;
         if (a.coef_entropy) a.coef_entropy[tok] = tr.coef_ent;
         const float glp = tr.coef_lp * grad_scale, gh = tr.coef_ent * grad_scale;
+        const float gsm = TOPK ? glp + g_topk * grad_scale : glp;  // what the row's softmax is subtracted with
         const float b = gh * inv_t;
         bc[0] = -lse * kLog2e;           // k0: p = exp2(x*c + k0)
-        bc[1] = -glp * inv_t + b * spx;  // a0
+        bc[1] = -gsm * inv_t + b * spx;  // a0
         bc[2] = -b * inv_t;              // a1: d = p * (a0 + a1*x)
         bc[3] = glp * inv_t;             // added at the target
-        bc[4] = (glp == 0.f && gh == 0.f) ? 1.f : 0.f;
+        bc[4] = (gsm == 0.f && glp == 0.f && gh == 0.f) ? 1.f : 0.f;
         bc_target = td.tg;
       }
     }
@@ -296,9 +310,14 @@ __global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_
 
 #define RELAX_AMD_RESIDENT(NVF, PARTIAL)                                                                             \
   if (full == NVF && partial == PARTIAL) {                                                                            \
-    hipLaunchKernelGGL((actor_step_resident_kernel<T, NVF, PARTIAL>), grid, block, 0, stream, logits, row_stride,    \
-                       vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a, grad_scale,       \
-                       log_prob, entropy, lse, spx, dlogits, d_stride);                                              \
+    if (a.topk_ids)                                                                                                   \
+      hipLaunchKernelGGL((actor_step_resident_kernel<T, NVF, PARTIAL, true>), grid, block, 0, stream, logits,        \
+                         row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
+                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride);                                \
+    else                                                                                                              \
+      hipLaunchKernelGGL((actor_step_resident_kernel<T, NVF, PARTIAL, false>), grid, block, 0, stream, logits,       \
+                         row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
+                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride);                                \
     return check_launch("actor_step_resident");                                                                      \
   }
 

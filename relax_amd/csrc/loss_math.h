@@ -191,6 +191,7 @@ __device__ __forceinline__ TokenResult token_terms(const relax_amd_policy_loss_a
     o.coef_lp += a.kl_coef * (m / den) * dkl;
   }
   float extra = in.extra_lp;
+  if (a.topk_ids) extra = 0.f;  // the weight of the top-K distillation signal, which the fused step evaluates itself
   if (a.distill_teacher_log_prob) {
     // extra_lp is the weight of this token's distillation signal in the loss; the signal's own derivative follows
     // the chain clamp_min -> estimator -> clamp(max = token clip) -> x min(ratio, clip) with the ratio detached

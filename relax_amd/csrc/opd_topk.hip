@@ -8,6 +8,7 @@
 // already produced (K scalar loads per row) or scans the row itself; the backward is one streaming pass
 // d[v] = -p[v] * sum_k g_k  followed by K read-modify-writes at the gathered positions.
 #include "device_utils.h"
+#include "opd_topk_math.h"
 #include "relax_amd.h"
 #include "row_scan.h"
 
@@ -118,48 +119,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_logprob_bwd_kernel(
 
 // ---- per-token KL on [R, K] ------------------------------------------------------------------------------------
 
-struct OpdParams {
-  int mode;       // RELAX_AMD_OPD_JSD family (alpha = 0: reverse KL, 1: forward KL) or RELAX_AMD_OPD_LOW_VAR
-  int norm;       // RELAX_AMD_OPD_NORM_*
-  float alpha;
-  int has_clamp;
-  float clamp;
-};
-
-// log-sum-exp over the lanes' strided values (−inf entries contribute nothing; all −inf gives −inf)
-__device__ __forceinline__ float row_logsumexp(const float* v, int n, int lane) {
-  float m = -INFINITY;
-  for (int k = lane; k < n; k += kWave) m = fmaxf(m, v[k]);
-  m = wave_max(m);
-  if (m == -INFINITY) return -INFINITY;
-  float s = 0.f;
-  for (int k = lane; k < n; k += kWave) s += expf(v[k] - m);
-  s = wave_sum(s);
-  return m + logf(s);
-}
-
-// term of one (s', t') entry and its derivative w.r.t. s'
-__device__ __forceinline__ void opd_entry(float s, float t, float alpha, float log_1ma, float log_a, float& term,
-                                          float& dterm) {
-  if (alpha == 0.f) {
-    const float p = expf(s);
-    term = p * (s - t);
-    dterm = p * (s - t + 1.f);
-  } else if (alpha == 1.f) {
-    const float q = expf(t);
-    term = q * (t - s);
-    dterm = -q;
-  } else {
-    const float u = s + log_1ma, w = t + log_a;
-    const float hi = fmaxf(u, w);
-    const float m = (hi == -INFINITY) ? -INFINITY : hi + logf(expf(u - hi) + expf(w - hi));
-    const float p = expf(s), q = expf(t);
-    term = (1.f - alpha) * (p * (s - m)) + alpha * (q * (t - m));
-    dterm = (1.f - alpha) * p * (s - m);
-  }
-}
-
-// One wave per row; `sv`/`tv` are the row's clamped + masked log-probs staged in LDS (k is a run-time size).
+// One wave per row; the row's clamped + masked log-probs are staged in LDS (k is a run-time size).
 template <bool BWD>
 __global__ __launch_bounds__(256) void opd_kl_topk_kernel(const float* __restrict__ s_lp,
     const float* __restrict__ t_lp,
@@ -171,84 +131,15 @@ __global__ __launch_bounds__(256) void opd_kl_topk_kernel(const float* __restric
   const int64_t r = blockIdx.x * 4LL + w;
   if (r >= n_rows) return;
   float* sv = stage + (w * 2) * k_ids;
-  float* tv = sv + k_ids;
   const float* s = s_lp + r * k_ids;
   const float* t = t_lp + r * k_ids;
   const uint8_t* mk = mask ? mask + r * k_ids : nullptr;
-  for (int k = lane; k < k_ids; k += kWave) {
-    float a = s[k], b = t[k];
-    if (p.has_clamp) {
-      a = fmaxf(a, p.clamp);  // NaN stays out of scope: log-probs are never NaN on entry
-      b = fmaxf(b, p.clamp);
-    }
-    if (mk && !mk[k]) a = b = -INFINITY;
-    sv[k] = a;
-    tv[k] = b;
-  }
-  // every lane re-reads only the entries it staged itself (k = lane, lane + 64, ...), so no barrier is needed
   const float gr = BWD ? g[r] : 0.f;
-  if (p.mode == RELAX_AMD_OPD_LOW_VAR) {
-    float acc = 0.f;
-    for (int k = lane; k < k_ids; k += kWave) {
-      const bool valid = !mk || mk[k];
-      const float d = sv[k] - tv[k];
-      const float e = expf(-d);
-      if (valid) acc += e - 1.f + d;
-      if (BWD) {
-        const bool pass = !p.has_clamp || s[k] >= p.clamp;
-        d_s[r * k_ids + k] = (valid && pass) ? gr * (1.f - e) : 0.f;
-      }
-    }
-    acc = wave_sum(acc);
-    if (!BWD && lane == 0) out[r] = acc;
-    return;
-  }
-  const float ls = row_logsumexp(sv, k_ids, lane), lt = row_logsumexp(tv, k_ids, lane);
-  float shift_s = 0.f, shift_t = 0.f, tail_s = 0.f, tail_t = 0.f;
-  bool with_tail = false, tail_grad = false;
-  if (p.norm == RELAX_AMD_OPD_NORM_NORM) {
-    shift_s = ls;
-    shift_t = lt;
-  } else if (p.norm == RELAX_AMD_OPD_NORM_TAIL) {
-    // tail bin log(1 - sum p) with the log-sum-exp clamped to <= -1e-7; the union path's mask cuts it off again
-    tail_s = logf(-expm1f(fminf(ls, -1e-7f)));
-    tail_t = logf(-expm1f(fminf(lt, -1e-7f)));
-    with_tail = mk == nullptr;
-    tail_grad = ls <= -1e-7f;
-  }
-  const float log_1ma = logf(1.f - p.alpha), log_a = logf(p.alpha);
-  float acc = 0.f, dsum = 0.f;
-  for (int k = lane; k < k_ids; k += kWave) {
-    if (mk && !mk[k]) continue;
-    float term, dterm;
-    opd_entry(sv[k] - shift_s, tv[k] - shift_t, p.alpha, log_1ma, log_a, term, dterm);
-    acc += term;
-    dsum += dterm;
-  }
-  acc = wave_sum(acc);
-  float d_tail = 0.f;
-  if (with_tail) {
-    float term;
-    opd_entry(tail_s, tail_t, p.alpha, log_1ma, log_a, term, d_tail);
-    acc += term;
-  }
-  if (!BWD) {
-    if (lane == 0) out[r] = acc;
-    return;
-  }
-  dsum = wave_sum(dsum);
-  for (int k = lane; k < k_ids; k += kWave) {
-    float dk = 0.f;
-    if (!mk || mk[k]) {
-      float term, dterm;
-      opd_entry(sv[k] - shift_s, tv[k] - shift_t, p.alpha, log_1ma, log_a, term, dterm);
-      dk = dterm;
-      if (p.norm == RELAX_AMD_OPD_NORM_NORM) dk -= expf(sv[k] - ls) * dsum;
-      if (with_tail && tail_grad) dk -= d_tail * expf(sv[k] - tail_s);
-      if (p.has_clamp && !(s[k] >= p.clamp)) dk = 0.f;
-    }
-    d_s[r * k_ids + k] = gr * dk;
-  }
+  const float acc = opd_kl_row<BWD>(
+      k_ids, mk != nullptr, p, lane, sv, sv + k_ids, [&](int k) { return s[k]; }, [&](int k) { return t[k]; },
+      [&](int k) { return mk[k] != 0; },
+      [&](int k, float dk, bool nonzero) { d_s[r * k_ids + k] = nonzero ? gr * dk : 0.f; });
+  if (!BWD && lane == 0) out[r] = acc;
 }
 
 // dlogits[row(t), id] += value * scale for the K (id, value) pairs of token t plus one pair at its target id: the

@@ -344,7 +344,7 @@ def _sft_single_pass(args: Namespace, batch: dict, logits: torch.Tensor):
         use_tis=False, mismatch_metrics=False, abs_diff_from_old=2, eps_clip=0.2, eps_clip_high=0.2, entropy_coef=0.0,
         kl_coef=0.0, tis_lo=0.0, tis_hi=2.0, opsm_delta=1e-4, tau_pos=1.0, tau_neg=1.05)
     inv_t = 1.0 / float(getattr(args, "rollout_temperature", 1.0))
-    loss, _metrics, _lp, _ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw, expected_grad_scale(batch))
+    loss, _metrics, _lp, _ent, _ = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw, expected_grad_scale(batch))
     return loss
 
 
@@ -523,13 +523,22 @@ class _SinglePassPolicyLoss(torch.autograd.Function):
             flat, lay.targets, lay.token_of_row, lay.sample_ids, lay.n_tokens, inv_t, float(assumed_scale),
             cu_resp=lay.cu_resp, **kw)
         metrics = out["metrics"]
+        topk = kw.get("topk_distill")
+        if topk is not None:
+            # the top-K distillation term: its multiple of each row's softmax left with the launch, the K one-hot
+            # parts are added here (d log p[id] / d logits = (onehot(id) - p) / T)
+            ops.sparse_row_add(dlogits, lay.row_ids, topk["ids"], out["topk_grad"],
+                               scale=float(inv_t) * float(assumed_scale))
+            topk_kl = out["topk_kl"]
+        else:
+            topk_kl = lp.new_zeros(0)
         ctx.dlogits = dlogits
         ctx.assumed_scale = float(assumed_scale)
-        ctx.mark_non_differentiable(metrics, lp, ent)
-        return metrics[_SLOT["loss"]].clone(), metrics, lp, ent
+        ctx.mark_non_differentiable(metrics, lp, ent, topk_kl)
+        return metrics[_SLOT["loss"]].clone(), metrics, lp, ent, topk_kl
 
     @staticmethod
-    def backward(ctx, g_loss, _gm, _glp, _gent):
+    def backward(ctx, g_loss, _gm, _glp, _gent, _gkl):
         d = ctx.dlogits
         if d is None:
             raise RuntimeError("the single-pass policy loss holds its gradient once: backward cannot run twice")
@@ -569,6 +578,60 @@ def _sampled_opd_kernel_args(args, batch, loss_mask, dev):
         out["distill"] = dict(teacher=teacher, kl_kind="k1" if kl_type == "reverse_kl" else "k3", min_clamp=clamp,
                               token_clip=tau, is_clip=is_clip)
     return out, teacher
+
+
+def _topk_opd_kernel_args(args, batch, lay, packed_ids, widths, loss_mask, dev):
+    """Kernel arguments that put the top-K distillation term (relax/utils/opd/opd_utils.py:1368-1455 with the
+    ``student_topk`` / ``teacher_topk`` / ``union`` selections) into the single launch, or None when the batch or the
+    options do not fit it (then the two-launch path takes the step and reports what is wrong with them).
+    ``packed_ids`` / ``widths`` as ``_pack_topk_ids`` returns them; ``extra_coef_log_prob`` holds each token's weight
+    ``opd_loss_coef * mask / clamp_min(sum mask, 1)``."""
+    from ._lib import FUSED_TOPK_MAX
+    from .opd_utils import opd_topk_kernel_modes
+
+    teacher = batch.get("opd_topk_teacher_log_probs")
+    if packed_ids is None or not teacher or packed_ids.size(1) > FUSED_TOPK_MAX or len(teacher) != len(widths) \
+            or min(widths) == 0:
+        return None
+    try:
+        mode, alpha, norm = opd_topk_kernel_modes(args.opd_kl_type, float(args.opd_jsd_alpha),
+                                                  getattr(args, "opd_norm_mode", "tail"))
+    except ValueError:
+        return None
+    clamp, tau, is_clip = (getattr(args, k, None) for k in ("opd_log_prob_min_clamp", "opd_per_token_clip",
+                                                            "opd_is_clip"))
+    if (tau is not None or is_clip is not None) and bool((loss_mask == 0).any()):
+        return None  # the clip-fraction metrics average over masked tokens too, whose rows the single launch skips
+    n, k = packed_ids.shape
+    resp = lay.response_lengths
+    if any(t is None or tuple(t.shape) != (r, w) for t, r, w in zip(teacher, resp, widths)):
+        return None
+    ksz = batch.get("opd_topk_ksz") if args.opd_token_selection == "union" else None
+    uniform = all(w == k for w in widths)
+    if uniform:
+        t_packed = torch.cat([t.to(device=dev, dtype=torch.float32) for t in teacher], dim=0)
+        width = None
+    else:
+        t_packed = torch.zeros((n, k), dtype=torch.float32, device=dev)
+        pos = 0
+        for t, r, w in zip(teacher, resp, widths):
+            t_packed[pos:pos + r, :w] = t.to(device=dev, dtype=torch.float32)
+            pos += r
+        width = torch.repeat_interleave(torch.tensor(widths, dtype=torch.int32, device=dev),
+                                        torch.tensor(resp, dtype=torch.int64, device=dev))
+    valid = None
+    if ksz is not None and any(i < len(ksz) and ksz[i] is not None for i in range(len(resp))):
+        valid = torch.full((n,), -1, dtype=torch.int32, device=dev)
+        pos = 0
+        for i, r in enumerate(resp):
+            if i < len(ksz) and ksz[i] is not None:
+                valid[pos:pos + r] = ksz[i].to(device=dev, dtype=torch.int32).reshape(-1)
+            pos += r
+    return {
+        "extra_coef_log_prob": loss_mask * (float(args.opd_loss_coef) / torch.clamp_min(loss_mask.sum(), 1)),
+        "topk_distill": dict(ids=packed_ids, teacher=t_packed.detach(), width=width, valid=valid, kl_mode=mode,
+                             norm_mode=norm, alpha=alpha, min_clamp=clamp, token_clip=tau, is_clip=is_clip),
+    }
 
 
 def _single_pass_ok(args, flat, kw, needs_bwd) -> bool:
@@ -891,19 +954,30 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         kw["lp_requires_grad"] = True
         if opd_gather is not None:
             kw["gather_topk_ids"], topk_widths = _pack_topk_ids(flat, lay, opd_gather)
-    opd_in_kernel = None
+    opd_in_kernel = topk_in_kernel = None
     if opd_on_lp and opd_gather is None and _single_pass_ok(args, flat, kw, needs_bwd):
         opd_in_kernel = _sampled_opd_kernel_args(args, batch, kw["loss_mask"], dev)
-    if opd_in_kernel is not None:
+    elif opd_on_lp and _single_pass_ok(args, flat, kw, needs_bwd):
+        topk_in_kernel = _topk_opd_kernel_args(args, batch, lay, kw.get("gather_topk_ids"), topk_widths,
+                                               kw["loss_mask"], dev)
+    topk_kl = None
+    if topk_in_kernel is not None:
+        # the top-K term as well: the kernel gathers the K logits of each row next to its log-sum-exp, evaluates the
+        # per-token KL and its derivative, and folds the gradient into the one dlogits launch (plus K sparse additions)
+        kw1 = {k: v for k, v in kw.items() if k not in ("lp_requires_grad", "gather_topk_ids")}
+        loss, mvec, lp, ent, topk_kl = _SinglePassPolicyLoss.apply(flat, lay, inv_t, dict(kw1, **topk_in_kernel),
+                                                                   expected_grad_scale(batch))
+        topk_lp = None
+    elif opd_in_kernel is not None:
         # the sampled-token term's gradient w.r.t. each log-prob is a per-token weight times the signal's derivative,
         # which the kernel evaluates next to the policy loss's: one launch; the term's value and metrics follow from
         # the launch's log-probs on [N] vectors
         kw.pop("lp_requires_grad", None)
-        loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, dict(kw, **opd_in_kernel[0]),
-                                                          expected_grad_scale(batch))
+        loss, mvec, lp, ent, _ = _SinglePassPolicyLoss.apply(flat, lay, inv_t, dict(kw, **opd_in_kernel[0]),
+                                                             expected_grad_scale(batch))
         topk_lp = None
     elif not opd_on_lp and _single_pass_ok(args, flat, kw, needs_bwd):
-        loss, mvec, lp, ent = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw, expected_grad_scale(batch))
+        loss, mvec, lp, ent, _ = _SinglePassPolicyLoss.apply(flat, lay, inv_t, kw, expected_grad_scale(batch))
         topk_lp = None
     else:
         loss, mvec, lp, ent, topk_lp = _FusedPolicyLoss.apply(flat, lay, inv_t, kw)
@@ -913,7 +987,14 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
 
     opd_reported = {}
     loss_metric = m("loss")
-    if opd_in_kernel is not None:
+    if topk_kl is not None:
+        from .opd_utils import finish_policy_opd_loss
+
+        with torch.no_grad():
+            opd_value, opd_reported = finish_policy_opd_loss(args, batch, topk_kl, lp, old if old is not None else lp)
+        loss = loss + opd_value
+        loss_metric = loss.detach().clone()
+    elif opd_in_kernel is not None:
         with torch.no_grad():
             if "distill" in opd_in_kernel[0]:
                 opd_value, opd_reported = compute_policy_opd_loss(

@@ -113,12 +113,9 @@ class _OpdKlTopk(torch.autograd.Function):
         return d, None, None, None, None, None, None
 
 
-def compute_opd_kl_topk(student_topk_lp: torch.Tensor, teacher_topk_lp: torch.Tensor, kl_type: str = "reverse_kl",
-                        jsd_alpha: float = 0.5, norm_mode: str = "tail", log_prob_min_clamp: float | None = None,
-                        mask: torch.Tensor | None = None) -> torch.Tensor:
-    """Per-token KL ``[R]`` (fp32) from ``[R, K]`` top-K log-probs, opd_utils.py:1190-1228: reverse / forward KL are
-    the ``jsd_alpha`` = 0 / 1 ends of the JSD family, ``low_var_kl`` is summed element-wise over K.  ``mask`` (bool
-    ``[R, K]``, True = valid) is the union path's padding mask.  Differentiable w.r.t. the student log-probs."""
+def opd_topk_kernel_modes(kl_type: str, jsd_alpha: float, norm_mode: str):
+    """``(kl mode, jsd alpha, norm mode)`` codes of the top-K KL kernels for the reference's option strings
+    (opd_utils.py:1190-1228); raises as ``compute_opd_kl_topk`` does on unknown ones."""
     if kl_type not in OPD_KL_TYPES:
         raise ValueError(f"Unknown opd_kl_type: {kl_type}. Choose one of {OPD_KL_TYPES}.")
     if kl_type == "low_var_kl":
@@ -130,6 +127,16 @@ def compute_opd_kl_topk(student_topk_lp: torch.Tensor, teacher_topk_lp: torch.Te
             raise ValueError(f"jsd_alpha must be in [0, 1], got {jsd_alpha}")
     if norm_mode not in _NORM_MODES:
         raise ValueError(f"Unknown opd_norm_mode: {norm_mode}. Choose one of {tuple(_NORM_MODES)}.")
+    return mode, alpha, _NORM_MODES[norm_mode]
+
+
+def compute_opd_kl_topk(student_topk_lp: torch.Tensor, teacher_topk_lp: torch.Tensor, kl_type: str = "reverse_kl",
+                        jsd_alpha: float = 0.5, norm_mode: str = "tail", log_prob_min_clamp: float | None = None,
+                        mask: torch.Tensor | None = None) -> torch.Tensor:
+    """Per-token KL ``[R]`` (fp32) from ``[R, K]`` top-K log-probs, opd_utils.py:1190-1228: reverse / forward KL are
+    the ``jsd_alpha`` = 0 / 1 ends of the JSD family, ``low_var_kl`` is summed element-wise over K.  ``mask`` (bool
+    ``[R, K]``, True = valid) is the union path's padding mask.  Differentiable w.r.t. the student log-probs."""
+    mode, alpha, norm = opd_topk_kernel_modes(kl_type, jsd_alpha, norm_mode)
     if student_topk_lp.dim() != 2 or student_topk_lp.shape != teacher_topk_lp.shape:
         raise ValueError(f"expected matching [R, K] inputs, got {tuple(student_topk_lp.shape)} and "
                          f"{tuple(teacher_topk_lp.shape)}")
@@ -143,7 +150,7 @@ def compute_opd_kl_topk(student_topk_lp: torch.Tensor, teacher_topk_lp: torch.Te
         mask = mask.to(device=dev, dtype=torch.uint8).contiguous()
     if s.size(0) == 0:
         return s.sum(dim=-1)
-    return _OpdKlTopk.apply(s, t, mask, mode, _NORM_MODES[norm_mode], alpha, log_prob_min_clamp)
+    return _OpdKlTopk.apply(s, t, mask, mode, norm, alpha, log_prob_min_clamp)
 
 
 def compute_opd_kl(student_log_probs, teacher_log_probs, kl_type: str = "reverse_kl", jsd_alpha: float = 0.5,
@@ -286,6 +293,12 @@ def compute_policy_opd_loss(*, args, batch, log_probs, old_log_probs, log_probs_
             return None, {}
         teacher = torch.cat(batch["teacher_log_probs"], dim=0).to(device=dev, dtype=log_probs.dtype).detach()
         per_token = compute_opd_kl(log_probs, teacher, kl_type, alpha, norm, clamp).to(log_probs.dtype)
+    return finish_policy_opd_loss(args, batch, per_token, log_probs, old_log_probs)
+
+
+def finish_policy_opd_loss(args, batch, per_token, log_probs, old_log_probs):
+    """The tail of ``compute_policy_opd_loss`` on the per-token signal ``[N]``: per-token clip, importance-ratio clip
+    (ratio detached), ``opd_loss_coef`` times the masked token mean, and the two clip-fraction metrics."""
     reported = {}
     tau = getattr(args, "opd_per_token_clip", None)
     if tau is not None:
@@ -299,7 +312,7 @@ def compute_policy_opd_loss(*, args, batch, log_probs, old_log_probs, log_probs_
         per_token = per_token * torch.clamp(ratio, max=float(clip)).to(per_token.dtype)
         with torch.no_grad():
             reported["opd_is_clip_frac"] = (ratio > float(clip)).float().mean().clone().detach()
-    return coef * reduce_opd_loss(batch, per_token), reported
+    return float(args.opd_loss_coef) * reduce_opd_loss(batch, per_token), reported
 
 
 def apply_opd_to_advantages(args, rollout_data, advantages: list) -> None:

@@ -254,12 +254,15 @@ def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_pr
                  use_tis=False, mismatch_metrics=False, abs_diff_from_old=1, eps_clip=0.2, eps_clip_high=0.2,
                  eps_clip_c=None, entropy_coef=0.0, kl_coef=0.0, tis_lo=0.0, tis_hi=2.0, opsm_delta=1e-4,
                  tau_pos=1.0, tau_neg=1.05, per_token_outputs=False, want_coef_entropy=False,
-                 extra_coef_log_prob=None, distill=None):
+                 extra_coef_log_prob=None, distill=None, topk_distill=None):
     """Fills a ``relax_amd_policy_loss_args`` block; returns (struct, outputs dict holding every live tensor).
     ``extra_coef_log_prob`` [n]: added to d loss / d log_prob of every unmasked token (the gradient of a caller's loss
     term that is linear in the log-probs).  ``distill`` = dict(teacher [n], kl_kind "k1" | "k3", min_clamp, token_clip,
     is_clip; None = off): ``extra_coef_log_prob`` then holds the weights of the sampled-token distillation signal and
-    the kernel applies the signal's own derivative."""
+    the kernel applies the signal's own derivative.  ``topk_distill`` = dict(ids int64 [n, K], teacher [n, K], width /
+    valid int32 [n] | None, kl_mode, norm_mode, alpha, min_clamp, token_clip, is_clip; None = off; the fused step
+    only): ``extra_coef_log_prob`` holds the weights of the top-K distillation signal, the step evaluates it next to
+    each row's log-sum-exp and leaves ``topk_kl`` [n] and ``topk_grad`` [n, K] in the outputs."""
     dev = _need_gpu(advantages, loss_mask, cu_resp)
     b = int(cu_resp.numel()) - 1
     if loss_kind not in _lib.LOSS_KINDS:
@@ -319,7 +322,39 @@ def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_pr
         nan = float("nan")
         a.distill_min_clamp, a.distill_token_clip, a.distill_is_clip = (
             nan if distill.get(k) is None else float(distill[k]) for k in ("min_clamp", "token_clip", "is_clip"))
-    out["_keepalive"] = (keep, partials, cu_resp, extra, teacher)
+    held = None
+    if topk_distill is not None:
+        td = topk_distill
+        ids, t_lp = td["ids"], _f32(td["teacher"])
+        k = int(ids.size(1)) if ids.dim() == 2 else 0
+        if extra is None or distill is not None or ids.dtype != torch.int64 or tuple(ids.shape) != (n, k) \
+                or tuple(t_lp.shape) != (n, k) or not (1 <= k <= _lib.FUSED_TOPK_MAX):
+            raise ValueError("topk_distill needs extra_coef_log_prob, no sampled-token distill block, int64 ids "
+                             f"[n, K] and teacher log-probs of the same shape, 1 <= K <= {_lib.FUSED_TOPK_MAX}")
+        ids, t_lp = ids.contiguous(), t_lp.contiguous()
+        per_tok = []
+        for key in ("width", "valid"):
+            v = td.get(key)
+            if v is not None:
+                if v.dtype != torch.int32 or v.numel() != n:
+                    raise ValueError(f"topk_distill[{key!r}] must be int32 [n]")
+                v = v.contiguous()
+            per_tok.append(v)
+        out["topk_kl"] = torch.zeros(n, **kw)
+        out["topk_grad"] = torch.zeros((n, k), **kw)
+        a.topk_ids, a.topk_teacher_log_prob = ids.data_ptr(), t_lp.data_ptr()
+        a.topk_width, a.topk_valid = (None if v is None else v.data_ptr() for v in per_tok)
+        a.topk_k, a.topk_kl_mode, a.topk_norm_mode = k, int(td["kl_mode"]), int(td["norm_mode"])
+        a.topk_jsd_alpha = float(td["alpha"])
+        clamp = td.get("min_clamp")
+        a.topk_has_clamp, a.topk_min_clamp = (0, 0.0) if clamp is None else (1, float(clamp))
+        nan = float("nan")
+        a.distill_min_clamp = nan
+        a.distill_token_clip, a.distill_is_clip = (
+            nan if td.get(key) is None else float(td[key]) for key in ("token_clip", "is_clip"))
+        a.topk_kl, a.topk_grad = out["topk_kl"].data_ptr(), out["topk_grad"].data_ptr()
+        held = (ids, t_lp, per_tok)
+    out["_keepalive"] = (keep, partials, cu_resp, extra, teacher, held)
     return a, out
 
 

@@ -31,17 +31,23 @@ def test_struct_layout_matches_c_header(tmp_path):
         " offsetof(relax_amd_policy_loss_args, metrics), RELAX_AMD_NUM_METRICS,"
         " offsetof(relax_amd_policy_loss_args, extra_coef_log_prob),"
         " offsetof(relax_amd_policy_loss_args, distill_kl_kind),"
-        " offsetof(relax_amd_policy_loss_args, distill_is_clip));return 0;}\n"
+        " offsetof(relax_amd_policy_loss_args, distill_is_clip));"
+        "printf(\"%zu %zu %zu %zu %d\\n\", offsetof(relax_amd_policy_loss_args, topk_ids),"
+        " offsetof(relax_amd_policy_loss_args, topk_k), offsetof(relax_amd_policy_loss_args, topk_min_clamp),"
+        " offsetof(relax_amd_policy_loss_args, topk_grad), RELAX_AMD_FUSED_TOPK_MAX);return 0;}\n"
     )
     exe = tmp_path / "layout"
     subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
-    size, off_n, off_eps, off_metrics, nmet, off_extra, off_kind, off_is = map(
-        int, subprocess.check_output([str(exe)]).split())
+    (size, off_n, off_eps, off_metrics, nmet, off_extra, off_kind, off_is, off_tk_ids, off_tk_k, off_tk_clamp,
+     off_tk_grad, tk_max) = map(int, subprocess.check_output([str(exe)]).split())
     S = _lib.PolicyLossArgs
     assert C.sizeof(S) == size
     assert S.n_samples.offset == off_n and S.eps_clip.offset == off_eps and S.metrics.offset == off_metrics
     assert S.extra_coef_log_prob.offset == off_extra and S.distill_kl_kind.offset == off_kind
     assert S.distill_is_clip.offset == off_is
+    assert S.topk_ids.offset == off_tk_ids and S.topk_k.offset == off_tk_k
+    assert S.topk_min_clamp.offset == off_tk_clamp and S.topk_grad.offset == off_tk_grad
+    assert tk_max == _lib.FUSED_TOPK_MAX
     assert nmet == _lib.NUM_METRICS
 
 
@@ -61,6 +67,23 @@ def test_argument_validation_reports_errors_without_touching_the_gpu():
     assert L.relax_amd_policy_loss(C.byref(a), None) == -1 and b"extra_coef_log_prob" in L.relax_amd_last_error()
     a.extra_coef_log_prob, a.distill_kl_kind = 16, _lib.KL_KINDS["k2"]
     assert L.relax_amd_policy_loss(C.byref(a), None) == -1 and b"distill_kl_kind" in L.relax_amd_last_error()
+    # ... and so is the top-K distillation block of the fused step
+    f = _lib.PolicyLossArgs()
+    f.advantages = f.loss_mask = f.coef_log_prob = f.topk_ids = 16
+    p16 = C.c_void_p(16)
+
+    def fused():
+        return L.relax_amd_actor_step_fused(p16, 2, 4, 64, 64, None, None, p16, 1.0, C.byref(f), 1.0, p16, p16, p16,
+                                            p16, p16, 64, None)
+
+    assert fused() == -1 and b"extra_coef_log_prob" in L.relax_amd_last_error()
+    f.extra_coef_log_prob = 16
+    assert fused() == -1 and b"topk_teacher_log_prob" in L.relax_amd_last_error()
+    f.topk_teacher_log_prob = f.topk_kl = f.topk_grad = 16
+    f.topk_k = _lib.FUSED_TOPK_MAX + 1
+    assert fused() == -1 and b"topk_k" in L.relax_amd_last_error()
+    f.topk_k, f.topk_norm_mode = 8, 7
+    assert fused() == -1 and b"topk_norm_mode" in L.relax_amd_last_error()
     rc = L.relax_amd_group_rewards(None, 0, None, 4, 7, None, None, None)
     assert rc == -1 and b"mode" in L.relax_amd_last_error()
     rc = L.relax_amd_masked_whiten(None, None, 0, 1, 1e-8, None, None, None, None)

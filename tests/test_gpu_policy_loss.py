@@ -1083,7 +1083,9 @@ def test_get_log_probs_and_entropy_topk_outputs_vs_oracle():
 
 
 @pytest.mark.parametrize("case", ["sampled_plain", "sampled_clips", "sampled_clamped", "sampled_clips_all_tokens",
-                                  "sampled_clamped_all_tokens", "student_topk_forward", "union_jsd"])
+                                  "sampled_clamped_all_tokens", "student_topk_forward", "union_jsd",
+                                  "teacher_topk_reverse_tail", "topk_low_var_clips_all_tokens",
+                                  "topk_norm_clamped_clips_all_tokens", "topk_ragged_widths", "topk_clips_masked"])
 @pytest.mark.parametrize("single_pass", ["auto", "off"])
 def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
     """``opd_loss_coef != 0``: the distillation term (sampled-token or top-K, union mask, per-token and
@@ -1119,6 +1121,21 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
                                                for r in resp]
         if case == "student_topk_forward":
             kw.update(opd_token_selection="student_topk", opd_kl_type="forward_kl", opd_norm_mode="tail")
+        elif case == "teacher_topk_reverse_tail":
+            kw.update(opd_token_selection="teacher_topk", opd_kl_type="reverse_kl", opd_norm_mode="tail")
+        elif case == "topk_low_var_clips":  # every token unmasked: the clips are applied inside the single launch
+            kw.update(opd_token_selection="teacher_topk", opd_kl_type="low_var_kl", opd_per_token_clip=8.0,
+                      opd_is_clip=1.01, opd_log_prob_min_clamp=-9.0)
+        elif case == "topk_norm_clamped_clips":
+            kw.update(opd_token_selection="student_topk", opd_kl_type="jsd", opd_jsd_alpha=0.3, opd_norm_mode="norm",
+                      opd_log_prob_min_clamp=-7.0, opd_per_token_clip=0.5, opd_is_clip=0.99)
+        elif case == "topk_clips_masked":  # clips with masked tokens: their metrics need every row, two launches run
+            kw.update(opd_token_selection="teacher_topk", opd_kl_type="reverse_kl", opd_per_token_clip=0.5)
+        elif case == "topk_ragged_widths":  # samples with different K: packed to the widest, trimmed per token
+            kw.update(opd_token_selection="teacher_topk", opd_kl_type="jsd", opd_jsd_alpha=0.6, opd_norm_mode="tail")
+            for i, w in enumerate([6, 3, 5, 1]):
+                batch["opd_topk_token_ids"][i] = batch["opd_topk_token_ids"][i][:, :w].contiguous()
+                batch["opd_topk_teacher_log_probs"][i] = batch["opd_topk_teacher_log_probs"][i][:, :w].contiguous()
         else:
             kw.update(opd_token_selection="union", opd_kl_type="jsd", opd_jsd_alpha=0.4, opd_norm_mode="trunc",
                       opd_log_prob_min_clamp=-12.0)
@@ -1137,9 +1154,67 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
     torch.testing.assert_close(lg.grad.cpu(), lo.grad, atol=3e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("v,dtype,k,variant", [(100352, torch.bfloat16, 64, "reverse_tail"),
+                                               (100352, torch.bfloat16, 200, "union_jsd_clips"),
+                                               (151936, torch.bfloat16, 64, "forward_norm"),
+                                               (32000, torch.float32, 96, "low_var")])
+def test_topk_opd_term_in_the_register_resident_step(v, dtype, k, variant):
+    """The top-K distillation term inside the single launch on the row shapes of the register-resident kernel (several
+    rows per persistent workgroup, K below and above one wave's width, the union mask, clips): loss, metrics and
+    dlogits against the two-launch path and against the oracle."""
+    import relax_amd
+
+    dev = require_gpu()
+    announce("top-K OPD in the resident step", v, dtype, k, variant)
+    g = torch.Generator().manual_seed(v + k)
+    n_samples = 12 if dtype != torch.float32 else 30
+    tot = [int(x) for x in torch.randint(20, 60, (n_samples,), generator=g)]
+    resp = [int(torch.randint(1, t, (1,), generator=g)) for t in tot]
+    logits, batch = _make_batch(37, tot, resp, v, dtype)
+    kw = dict(opd_loss_coef=0.6, eps_clip_high=0.28, use_kl_loss=True, kl_loss_coef=1e-3, kl_loss_type="k3",
+              entropy_coef=0.01)
+    batch["opd_topk_token_ids"] = [torch.stack([torch.randperm(v, generator=g)[:k] for _ in range(r)]) for r in resp]
+    batch["opd_topk_teacher_log_probs"] = [torch.log_softmax(2 * torch.randn(r, 4 * k, generator=g), -1)[:, :k]
+                                           .contiguous() for r in resp]
+    if variant == "reverse_tail":
+        kw.update(opd_token_selection="teacher_topk", opd_kl_type="reverse_kl", opd_norm_mode="tail")
+        batch["loss_masks"][2] = torch.zeros_like(batch["loss_masks"][2])
+    elif variant == "union_jsd_clips":
+        kw.update(opd_token_selection="union", opd_kl_type="jsd", opd_jsd_alpha=0.4, opd_norm_mode="trunc",
+                  opd_log_prob_min_clamp=-14.0, opd_per_token_clip=0.05, opd_is_clip=1.01)
+        batch["opd_topk_ksz"] = [torch.randint(1, k + 1, (r,), generator=g) for r in resp]
+        batch["loss_masks"] = [torch.ones_like(m) for m in batch["loss_masks"]]
+    elif variant == "forward_norm":
+        kw.update(opd_token_selection="student_topk", opd_kl_type="forward_kl", opd_norm_mode="norm")
+    else:
+        kw.update(opd_token_selection="teacher_topk", opd_kl_type="low_var_kl", opd_log_prob_min_clamp=-11.0)
+    db = _to_dev(batch, dev)
+    outs = {}
+    for mode in ("auto", "off"):
+        lg = logits.to(dev).requires_grad_()
+        loss, met = relax_amd.policy_loss_function(P.make_args(relax_amd_single_pass=mode, **kw), db, lg, None)
+        loss.backward()
+        outs[mode] = (loss.detach(), met, lg.grad)
+    ulp = {torch.bfloat16: 2.0 ** -7, torch.float32: 1e-5}[dtype]
+    assert abs(outs["auto"][0].item() - outs["off"][0].item()) < 1e-5 * max(1.0, abs(outs["off"][0].item()))
+    assert set(outs["auto"][1]) == set(outs["off"][1])
+    for key, w in outs["off"][1].items():
+        assert abs(outs["auto"][1][key].item() - w.item()) < 1e-5 * max(1.0, abs(w.item())), key
+    torch.testing.assert_close(outs["auto"][2].float(), outs["off"][2].float(), atol=2e-6, rtol=2 * ulp)
+    lo = logits.float().clone().requires_grad_()
+    want, want_m = P.policy_loss_function(P.make_args(**kw), dict(batch), lo, R.make_reducer(resp, batch["loss_masks"]))
+    want.backward()
+    tol = 2e-3 if dtype != torch.float32 else 5e-5
+    assert abs(outs["auto"][0].item() - want.item()) < tol * max(1.0, abs(want.item()))
+    for key, w in want_m.items():
+        assert abs(outs["auto"][1][key].item() - float(w)) < tol * max(1.0, abs(float(w))), key
+    torch.testing.assert_close(outs["auto"][2].float().cpu(), lo.grad, atol=tol, rtol=max(2 * ulp, 1e-5))
+
+
 def test_linear_opd_term_rides_the_single_launch(monkeypatch):
     """Sampled-token distillation signals (plain reverse_kl: linear in the log-probs; low_var_kl or clipped: derivative
-    evaluated by the kernel): one fused launch, no separate log-prob or dlogits launch."""
+    evaluated by the kernel) and the top-K signals (evaluated by the kernel next to each row's log-sum-exp): one fused
+    launch, no separate log-prob or dlogits launch."""
     import relax_amd
     from relax_amd import ops
 
@@ -1166,6 +1241,20 @@ def test_linear_opd_term_rides_the_single_launch(monkeypatch):
         loss, _ = relax_amd.policy_loss_function(args, _to_dev(case_batch, dev), lg, None)
         loss.backward()
         assert calls == want, (kl_type, clip, calls)
+    k = 5
+    batch["opd_topk_token_ids"] = [torch.randint(0, v, (r, k), generator=g) for r in resp]
+    batch["opd_topk_teacher_log_probs"] = [torch.log_softmax(torch.randn(r, v, generator=g), -1)[:, :k].contiguous()
+                                           for r in resp]
+    for kl_type, clip, masks, want in (("reverse_kl", None, None, ["actor_step_fused"]),
+                                       ("jsd", 0.5, ones, ["actor_step_fused"]), ("jsd", 0.5, None, two)):
+        calls.clear()
+        case_batch = batch if masks is None else dict(batch, loss_masks=masks)
+        args = P.make_args(opd_loss_coef=0.7, opd_token_selection="teacher_topk", opd_kl_type=kl_type,
+                           opd_jsd_alpha=0.5, opd_norm_mode="tail", opd_per_token_clip=clip)
+        lg = logits.to(dev).requires_grad_()
+        loss, _ = relax_amd.policy_loss_function(args, _to_dev(case_batch, dev), lg, None)
+        loss.backward()
+        assert calls == want, ("top-K", kl_type, clip, calls)
 
 
 def test_outputs_leave_as_one_packed_copy_in_the_reference_wire_format():
