@@ -56,7 +56,7 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
   __shared__ float wave_state[THREADS / kWave][3];
   __shared__ float bc[5];
   __shared__ int64_t bc_target;
-  __shared__ float topk_stage[2 * RELAX_AMD_FUSED_TOPK_MAX];
+  __shared__ float topk_stage[kTopkStageFloats];
   const int tid = threadIdx.x;
   const int64_t row = blockIdx.x;
   T* d = dlogits + row * d_stride;
@@ -92,6 +92,9 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
     den = a.sample_denom ? a.sample_denom[sid] : 1.0f;
     pg_den = a.pg_sample_denom ? a.pg_sample_denom[sid] : den;
   }
+  // the first wave's gathers for the top-K distillation signal, when configured, likewise
+  TopkGather gathered{};
+  if (a.topk_ids && tid < kWave) gathered = topk_gather<T>(a, x, vocab, tok, tid);
   // pass 1: cached loads, the row stays in L2 / the memory-side cache for pass 2
   SoftmaxAcc st = scan_row<T, VEC, false, THREADS>(x, vocab, c);
   scan_block_merge<THREADS>(st, wave_state);
@@ -108,9 +111,9 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
     float g_topk = 0.f;
     if (a.topk_ids) {
       const float lp0 = __shfl(lp, 0, kWave);
-      g_topk = topk_distill_row<T>(a, x, vocab, tok, __shfl(lse, 0, kWave), inv_t, lp0,
-                                   __shfl(in.has_old ? in.old_lp : lp, 0, kWave), __shfl(in.extra_lp, 0, kWave), tid,
-                                   topk_stage);
+      g_topk = topk_distill_row(a, gathered, tok, __shfl(lse, 0, kWave), inv_t, lp0,
+                                __shfl(in.has_old ? in.old_lp : lp, 0, kWave), __shfl(in.extra_lp, 0, kWave), tid,
+                                topk_stage);
     }
     if (tid == 0) {
       const TokenResult tr = token_terms(a, in, lp, ent, false, 0.f, den, pg_den);

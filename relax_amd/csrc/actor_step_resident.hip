@@ -105,7 +105,7 @@ __global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_
   __shared__ float wave_state[THREADS / kWave][3];
   __shared__ float bc[5];
   __shared__ int64_t bc_target;
-  __shared__ float topk_stage[TOPK ? 2 * RELAX_AMD_FUSED_TOPK_MAX : 1];
+  __shared__ float topk_stage[TOPK ? kTopkStageFloats : 1];
   const int tid = threadIdx.x;
   const bool wave0 = __builtin_amdgcn_readfirstlane(tid) < kWave;  // scalar: other waves branch around thread 0's work
   const int rem = int(vocab / VN) - NVF * THREADS;  // lanes that hold a vector at the partial position (host-checked)
@@ -208,6 +208,16 @@ __global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_
     // here, behind the merge of the waves' partial states, costs less than carrying them through the scan in
     // registers that every wave would have to set aside.
     const ResidentTokenData td = fetch_token(row, tok);
+    // likewise the first wave's gathers for the top-K distillation signal: two dependent requests (ids, then the
+    // row's logits there) that need nothing of the scan's result
+    TopkGather gathered{};
+    if constexpr (TOPK) {
+      if (wave0) {
+        int lane = tid;
+        asm volatile("" : "+v"(lane));
+        gathered = topk_gather<T>(a, logits + row * row_stride, vocab, tok, lane);
+      }
+    }
     scan_block_merge<THREADS>(st, wave_state);
     if (wave0) {
       float lse = 0.f, spx = 0.f, ent = 0.f, lp = 0.f;
@@ -223,9 +233,9 @@ __global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_
       if constexpr (TOPK) {
         int lane = tid;
         asm volatile("" : "+v"(lane));
-        g_topk = topk_distill_row<T>(a, logits + row * row_stride, vocab, tok, __shfl(lse, 0, kWave), inv_t,
-                                     __shfl(lp, 0, kWave), __shfl(td.in.has_old ? td.in.old_lp : lp, 0, kWave),
-                                     __shfl(td.in.extra_lp, 0, kWave), lane, topk_stage);
+        g_topk = topk_distill_row(a, gathered, tok, __shfl(lse, 0, kWave), inv_t, __shfl(lp, 0, kWave),
+                                  __shfl(td.in.has_old ? td.in.old_lp : lp, 0, kWave),
+                                  __shfl(td.in.extra_lp, 0, kWave), lane, topk_stage);
       }
       if (tid == 0) {
         relax_amd_policy_loss_args al = a;

@@ -150,48 +150,88 @@ inline const char* topk_distill_args_error(const relax_amd_policy_loss_args& a) 
   return nullptr;
 }
 
-// The top-K distillation signal of one token inside the fused actor step, by the workgroup's first wave once the row's
-// log-sum-exp is known: log-probs at the token's K ids (as topk_logprob_fwd_kernel forms them), the per-token KL,
-// clips and weight, topk_kl / topk_grad written.  `x` = the token's logits row, `weight` = the signal's weight in the
-// loss, `old` = the token's old log-prob (the current one when there is none).  Returns, in every lane, the sum of
-// d loss / d log p[id_k] over the non-sentinel ids: what the row's softmax is multiplied by, next to the policy
-// terms' own coefficient.  `stage` = 2 * RELAX_AMD_FUSED_TOPK_MAX floats of LDS.
+// What a lane of the first wave requests ahead of time for the top-K distillation signal of a token: the row's logits
+// at its ids (entries lane, lane + 64, ...) and the teacher's log-probs there.  Nothing here depends on the row's
+// log-sum-exp, so the two dependent gathers (ids, then logits) are requested before the workgroup merges its scan
+// (the merge's barrier waits for them: they overlap the other waves' way to that barrier, not the merge itself).
+constexpr int kTopkPerLane = RELAX_AMD_FUSED_TOPK_MAX / kWave;
+struct TopkGather {
+  float x[kTopkPerLane];  // the gathered logit; -inf for a sentinel id, 0 for an id outside the vocabulary
+  float t[kTopkPerLane];
+  bool real[kTopkPerLane];  // the id is not a sentinel (its log-prob carries the row's log-sum-exp)
+};
+
 template <typename T>
-__device__ __forceinline__ float topk_distill_row(const relax_amd_policy_loss_args& a, const T* x, int64_t vocab,
-                                                  int64_t tok, float lse, float inv_t, float lp, float old,
-                                                  float weight, int lane, float* stage) {
+__device__ __forceinline__ TopkGather topk_gather(const relax_amd_policy_loss_args& a, const T* x, int64_t vocab,
+                                                  int64_t tok, int lane) {
+  TopkGather g;
   const int kmax = a.topk_k;
   const int64_t* ids = a.topk_ids + tok * kmax;
   const float* teacher = a.topk_teacher_log_prob + tok * kmax;
+#pragma unroll
+  for (int i = 0; i < kTopkPerLane; ++i) {
+    const int k = lane + i * kWave;
+    g.x[i] = g.t[i] = 0.f;
+    g.real[i] = false;
+    if (k < kmax) {
+      const int64_t id = ids[k];
+      g.t[i] = teacher[k];
+      g.real[i] = id >= 0;
+      // a sentinel yields log-prob -inf; outside the vocabulary slice the reference gathers a zero logit
+      g.x[i] = id < 0 ? -INFINITY : (id >= vocab ? 0.f : Row<T>::load1(x + id));
+    }
+  }
+  return g;
+}
+
+// The top-K distillation signal of one token inside the fused actor step, by the workgroup's first wave once the row's
+// log-sum-exp is known: log-probs at the token's K ids (as topk_logprob_fwd_kernel forms them), the per-token KL,
+// clips and weight, topk_kl / topk_grad written.  `g` = this lane's topk_gather(), `weight` = the signal's weight in
+// the loss, `old` = the token's old log-prob (the current one when there is none).  Returns, in every lane, the sum of
+// d loss / d log p[id_k] over the non-sentinel ids: what the row's softmax is multiplied by, next to the policy
+// terms' own coefficient.  `stage` = kTopkStageFloats floats of LDS.
+constexpr int kTopkStageFloats = 4 * RELAX_AMD_FUSED_TOPK_MAX;
+
+__device__ __forceinline__ float topk_distill_row(const relax_amd_policy_loss_args& a, const TopkGather& g,
+                                                  int64_t tok, float lse, float inv_t, float lp, float old,
+                                                  float weight, int lane, float* stage) {
+  const int kmax = a.topk_k;
   int width = a.topk_width ? a.topk_width[tok] : kmax;
   width = width < 0 ? 0 : (width > kmax ? kmax : width);
   const int nvalid = a.topk_valid ? a.topk_valid[tok] : -1;
   const OpdParams p{a.topk_kl_mode, a.topk_norm_mode, a.topk_jsd_alpha, a.topk_has_clamp, a.topk_min_clamp};
   float* sv = stage;
   float* tv = stage + RELAX_AMD_FUSED_TOPK_MAX;
-  auto student = [&](int k) -> float {
-    const int64_t id = ids[k];
-    if (id < 0) return -INFINITY;  // sentinel
-    if (id >= vocab) return -lse;  // outside the vocabulary slice: the reference gathers a zero logit
-    return fmaf(Row<T>::load1(x + id), inv_t, -lse);
-  };
+  float* raw_s = stage + 2 * RELAX_AMD_FUSED_TOPK_MAX;  // the student log-probs before clamp and mask
+  float* raw_t = stage + 3 * RELAX_AMD_FUSED_TOPK_MAX;
+#pragma unroll
+  for (int i = 0; i < kTopkPerLane; ++i) {
+    const int k = lane + i * kWave;
+    if (k < kmax) {
+      raw_s[k] = fmaf(g.x[i], inv_t, -lse);
+      raw_t[k] = g.t[i];
+    }
+  }
   // the derivatives land in sv[] (store_d is the last use of an entry's staged values)
   const float kl = opd_kl_row<true>(
-      width, nvalid >= 0, p, lane, sv, tv, student, [&](int k) { return teacher[k]; },
+      width, nvalid >= 0, p, lane, sv, tv, [&](int k) { return raw_s[k]; }, [&](int k) { return raw_t[k]; },
       [&](int k) { return k < nvalid; }, [&](int k, float dk, bool nonzero) { sv[k] = nonzero ? dk : 0.f; });
   float pass = 1.f;
   if (a.distill_token_clip == a.distill_token_clip && kl > a.distill_token_clip) pass = 0.f;
   if (a.distill_is_clip == a.distill_is_clip) pass *= fminf(expf(lp - old), a.distill_is_clip);
   const float f = weight * pass;
   float total = 0.f;
-  for (int k = lane; k < kmax; k += kWave) {
-    float g = 0.f;
-    if (k < width) {
-      g = f * sv[k];
-      if (!(sv[k] != 0.f)) g = 0.f;  // entries without gradient stay exact zeros whatever the weight holds
-      if (ids[k] >= 0 && g != 0.f) total += g;
+#pragma unroll
+  for (int i = 0; i < kTopkPerLane; ++i) {
+    const int k = lane + i * kWave;
+    if (k < kmax) {
+      float d = 0.f;
+      if (k < width && sv[k] != 0.f) {  // entries without gradient stay exact zeros whatever the weight holds
+        d = f * sv[k];
+        if (g.real[i] && d != 0.f) total += d;
+      }
+      a.topk_grad[tok * kmax + k] = d;
     }
-    a.topk_grad[tok * kmax + k] = g;
   }
   if (lane == 0) a.topk_kl[tok] = kl;
   return wave_sum(total);
