@@ -294,6 +294,19 @@ def run_actor_step(a, dev) -> None:
     n_tokens = a.seqs * a.seq_len
     if a.two_launch:
         args.relax_amd_single_pass = "off"
+    opd = ""
+    if a.opd_topk > 0:
+        # on-policy distillation as production runs it: the teacher's top-K ids and log-probs of every response token,
+        # reverse KL with the tail bin, added to the policy loss (opd_loss_coef)
+        k = a.opd_topk
+        args.opd_loss_coef, args.opd_kl_type, args.opd_token_selection = 0.5, "reverse_kl", "teacher_topk"
+        args.opd_jsd_alpha, args.opd_norm_mode, args.opd_log_prob_min_clamp = 0.5, "tail", None
+        args.opd_per_token_clip = args.opd_is_clip = None
+        resp = batch["response_lengths"]
+        batch["opd_topk_token_ids"] = [torch.randint(0, a.vocab, (r, k), device=dev, generator=g) for r in resp]
+        batch["opd_topk_teacher_log_probs"] = [
+            torch.log_softmax(torch.randn(r, k + 1, device=dev, generator=g), -1)[:, :k].contiguous() for r in resp]
+        opd = f" + top-{k} distillation term (teacher_topk, reverse KL, tail bin)"
     # the step as the training loop runs it: loss_function applies Megatron's gradient-accumulation scaling
     # (num_microbatches / global_batch_size * dp = 1 / 16 here), so the loss's upstream gradient is not 1
     num_microbatches = 1
@@ -319,12 +332,14 @@ def run_actor_step(a, dev) -> None:
     necessary = row_bytes * (live + n_tokens)
     if "actor_step_fused" in kernel_ms:
         dom, dom_name = kernel_ms["actor_step_fused"], fused_step_kernel_name(a.vocab)
+        if a.opd_topk > 0:
+            dom_name = dom_name[:-1] + ", true>"  # the instantiation that evaluates the top-K term
     else:  # two launches: the backward (read live rows, write all rows) dominates; the forward read is its own launch
         dom, dom_name = kernel_ms["logprob_entropy_bwd"], "logprob_entropy_bwd_kernel<bf16_t, true>"
     emit(a, n_tokens, wall,
          f"Qwen3-8B-shaped actor step: {a.seqs} seqs x {a.seq_len} tokens = {n_tokens} rows x V={a.vocab} bf16 "
-         f"logits, PPO-clip 0.2/0.28 + k3 KL 1e-3, loss_function (scale 1/{args.global_batch_size}) fwd + bwd to "
-         f"dlogits",
+         f"logits, PPO-clip 0.2/0.28 + k3 KL 1e-3{opd}, loss_function (scale 1/{args.global_batch_size}) fwd + bwd "
+         f"to dlogits",
          {"rows": n_tokens, "live_rows": live, "vocab": a.vocab, "loss": float(loss.item())},
          hbm_roofline(dom_name, dom, necessary, n_tokens, a.vocab, kernel_ms, ms_per_step,
                       survey_bytes=3.0 * row_bytes * n_tokens if "actor_step_fused" in kernel_ms else None),
@@ -767,7 +782,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="actor_step",
-                    choices=["actor_step", "cfg1", "lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "actor_fwd_topk",
+                    choices=["actor_step", "actor_step_opd_topk", "cfg1", "lmhead", "reverse_kl", "varlen_gspo",
+                             "varlen_cispo", "actor_fwd_topk",
                              "mfma_ceiling", "hbm_ceiling"])
     ap.add_argument("--seqs", type=int, default=SEQS)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
@@ -796,6 +812,8 @@ def main() -> int:
                     help="actor_fwd_topk: select with torch.topk instead of the library's kernel (comparison)")
     ap.add_argument("--two-launch", action="store_true",
                     help="use the separate forward / backward launches (the path GSPO takes) instead of the fused step")
+    ap.add_argument("--opd-topk", type=int, default=0,
+                    help="actor_step: add the top-K on-policy distillation term with this K (0 = none)")
     ap.add_argument("--no-secondary", action="store_true",
                     help="plain invocation only: skip the other configurations that otherwise run after the headline "
                          "workload and ride along in its line as other_workloads")
@@ -813,14 +831,18 @@ def main() -> int:
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if a.workload == "actor_step" and a.cpu_rows > 0 and not a.no_secondary:
+    if a.workload == "actor_step_opd_topk" and a.opd_topk == 0:
+        a.opd_topk = 64
+    if a.opd_topk > 0:
+        a.cpu_rows = 0  # the CPU baseline is timed on the headline workload only
+    if a.workload == "actor_step" and a.opd_topk == 0 and a.cpu_rows > 0 and not a.no_secondary:
         return run_default_with_secondary(a, dev)
     run_workload(a, dev)
     return 0
 
 
 def run_workload(a, dev) -> None:
-    if a.workload == "actor_step":
+    if a.workload in ("actor_step", "actor_step_opd_topk"):
         run_actor_step(a, dev)
     elif a.workload == "cfg1":
         run_cfg1(a, dev)
@@ -838,7 +860,7 @@ def run_workload(a, dev) -> None:
         run_varlen(a, dev, a.workload.split("_")[1])
 
 
-SECONDARY = ("lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "cfg1", "actor_fwd_topk")
+SECONDARY = ("lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "cfg1", "actor_fwd_topk", "actor_step_opd_topk")
 
 
 def run_default_with_secondary(a, dev) -> int:
@@ -861,6 +883,7 @@ def run_default_with_secondary(a, dev) -> int:
         torch.cuda.empty_cache()
         b = copy.copy(a)
         b.workload, b.steps, b.warmup, b.cpu_rows, b.rows = name, min(a.steps, 10), min(a.warmup, 3), 0, 0
+        b.opd_topk = 64 if name == "actor_step_opd_topk" else 0
         try:
             run_workload(b, dev)
             got = COLLECTED.pop()
