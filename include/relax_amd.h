@@ -212,6 +212,11 @@ typedef struct relax_amd_policy_loss_args {
   float topk_jsd_alpha, topk_min_clamp;
   float* topk_kl;                       /* out [n_tokens] */
   float* topk_grad;                     /* out [n_tokens, topk_k] */
+  /* relax_amd_actor_step_fused only: 0 = rows of tokens whose masks are both zero are not read (their log_prob,
+   * entropy and distillation outputs are 0, their dlogits rows zeros); 1 = they are scanned like any other row, so
+   * that log_prob / entropy / topk_kl hold their true values (what metrics that average over masked tokens too
+   * need: opd_per_token_clip_frac, opd_is_clip_frac); their dlogits rows are zeros either way. */
+  int32_t read_masked_rows;
 } relax_amd_policy_loss_args;
 
 #define RELAX_AMD_FUSED_TOPK_MAX 256

@@ -55,6 +55,7 @@ class PolicyLossArgs(C.Structure):
         ("topk_ids", _vp), ("topk_teacher_log_prob", _vp), ("topk_width", _vp), ("topk_valid", _vp),
         ("topk_k", _i32), ("topk_kl_mode", _i32), ("topk_norm_mode", _i32), ("topk_has_clamp", _i32),
         ("topk_jsd_alpha", _f32), ("topk_min_clamp", _f32), ("topk_kl", _vp), ("topk_grad", _vp),
+        ("read_masked_rows", _i32),
     ]
 
 

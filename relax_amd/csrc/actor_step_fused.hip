@@ -65,7 +65,7 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
   if (live) {
     const float m = a.loss_mask[tok];
     const float mp = a.pg_loss_mask ? a.pg_loss_mask[tok] : m;
-    live = !(m == 0.f && mp == 0.f);
+    live = !(m == 0.f && mp == 0.f) || a.read_masked_rows != 0;
   }
   if (!live) {
     fused_zero_row<T, VEC, THREADS>(d, vocab);

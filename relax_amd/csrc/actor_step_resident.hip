@@ -121,7 +121,7 @@ __global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_
     if (tok < 0) return -1;
     const float m = a.loss_mask[tok];
     const float mp = a.pg_loss_mask ? a.pg_loss_mask[tok] : m;
-    return (m == 0.f && mp == 0.f) ? -1 : tok;
+    return (m == 0.f && mp == 0.f && !a.read_masked_rows) ? -1 : tok;
   };
   auto fetch_token = [&](int64_t row, int64_t tok) {
     ResidentTokenData td{};

@@ -569,11 +569,11 @@ def _sampled_opd_kernel_args(args, batch, loss_mask, dev):
         return None
     clamp, tau, is_clip = (getattr(args, k, None) for k in ("opd_log_prob_min_clamp", "opd_per_token_clip",
                                                             "opd_is_clip"))
-    if (tau is not None or is_clip is not None) and bool((loss_mask == 0).any()):
-        # the clip-fraction metrics are plain means over every response token, masked ones included, and the single
-        # launch does not read the rows of masked tokens: their log-probs come from the two-launch path
-        return None
     out = {"extra_coef_log_prob": loss_mask * (float(args.opd_loss_coef) / torch.clamp_min(loss_mask.sum(), 1))}
+    if tau is not None or is_clip is not None:
+        # the clip-fraction metrics are plain means over every response token, masked ones included: the launch then
+        # scans the rows of masked tokens as well (it skips them otherwise)
+        out["read_masked_rows"] = True
     if kl_type != "reverse_kl" or any(v is not None for v in (clamp, tau, is_clip)):
         out["distill"] = dict(teacher=teacher, kl_kind="k1" if kl_type == "reverse_kl" else "k3", min_clamp=clamp,
                               token_clip=tau, is_clip=is_clip)
@@ -600,8 +600,6 @@ def _topk_opd_kernel_args(args, batch, lay, packed_ids, widths, loss_mask, dev):
         return None
     clamp, tau, is_clip = (getattr(args, k, None) for k in ("opd_log_prob_min_clamp", "opd_per_token_clip",
                                                             "opd_is_clip"))
-    if (tau is not None or is_clip is not None) and bool((loss_mask == 0).any()):
-        return None  # the clip-fraction metrics average over masked tokens too, whose rows the single launch skips
     n, k = packed_ids.shape
     resp = lay.response_lengths
     if any(t is None or tuple(t.shape) != (r, w) for t, r, w in zip(teacher, resp, widths)):
@@ -631,6 +629,8 @@ def _topk_opd_kernel_args(args, batch, lay, packed_ids, widths, loss_mask, dev):
         "extra_coef_log_prob": loss_mask * (float(args.opd_loss_coef) / torch.clamp_min(loss_mask.sum(), 1)),
         "topk_distill": dict(ids=packed_ids, teacher=t_packed.detach(), width=width, valid=valid, kl_mode=mode,
                              norm_mode=norm, alpha=alpha, min_clamp=clamp, token_clip=tau, is_clip=is_clip),
+        # the clip-fraction metrics average over masked tokens too: their rows are then scanned as well
+        "read_masked_rows": tau is not None or is_clip is not None,
     }
 
 

@@ -254,7 +254,7 @@ def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_pr
                  use_tis=False, mismatch_metrics=False, abs_diff_from_old=1, eps_clip=0.2, eps_clip_high=0.2,
                  eps_clip_c=None, entropy_coef=0.0, kl_coef=0.0, tis_lo=0.0, tis_hi=2.0, opsm_delta=1e-4,
                  tau_pos=1.0, tau_neg=1.05, per_token_outputs=False, want_coef_entropy=False,
-                 extra_coef_log_prob=None, distill=None, topk_distill=None):
+                 extra_coef_log_prob=None, distill=None, topk_distill=None, read_masked_rows=False):
     """Fills a ``relax_amd_policy_loss_args`` block; returns (struct, outputs dict holding every live tensor).
     ``extra_coef_log_prob`` [n]: added to d loss / d log_prob of every unmasked token (the gradient of a caller's loss
     term that is linear in the log-probs).  ``distill`` = dict(teacher [n], kl_kind "k1" | "k3", min_clamp, token_clip,
@@ -262,7 +262,9 @@ def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_pr
     the kernel applies the signal's own derivative.  ``topk_distill`` = dict(ids int64 [n, K], teacher [n, K], width /
     valid int32 [n] | None, kl_mode, norm_mode, alpha, min_clamp, token_clip, is_clip; None = off; the fused step
     only): ``extra_coef_log_prob`` holds the weights of the top-K distillation signal, the step evaluates it next to
-    each row's log-sum-exp and leaves ``topk_kl`` [n] and ``topk_grad`` [n, K] in the outputs."""
+    each row's log-sum-exp and leaves ``topk_kl`` [n] and ``topk_grad`` [n, K] in the outputs.  ``read_masked_rows``
+    (the fused step only): rows of fully masked tokens are scanned too, so their log-probs, entropies and distillation
+    signals are real instead of 0."""
     dev = _need_gpu(advantages, loss_mask, cu_resp)
     b = int(cu_resp.numel()) - 1
     if loss_kind not in _lib.LOSS_KINDS:
@@ -322,6 +324,7 @@ def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_pr
         nan = float("nan")
         a.distill_min_clamp, a.distill_token_clip, a.distill_is_clip = (
             nan if distill.get(k) is None else float(distill[k]) for k in ("min_clamp", "token_clip", "is_clip"))
+    a.read_masked_rows = int(bool(read_masked_rows))
     held = None
     if topk_distill is not None:
         td = topk_distill

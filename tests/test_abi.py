@@ -34,12 +34,13 @@ def test_struct_layout_matches_c_header(tmp_path):
         " offsetof(relax_amd_policy_loss_args, distill_is_clip));"
         "printf(\"%zu %zu %zu %zu %d\\n\", offsetof(relax_amd_policy_loss_args, topk_ids),"
         " offsetof(relax_amd_policy_loss_args, topk_k), offsetof(relax_amd_policy_loss_args, topk_min_clamp),"
-        " offsetof(relax_amd_policy_loss_args, topk_grad), RELAX_AMD_FUSED_TOPK_MAX);return 0;}\n"
+        " offsetof(relax_amd_policy_loss_args, topk_grad), RELAX_AMD_FUSED_TOPK_MAX);"
+        "printf(\"%zu\\n\", offsetof(relax_amd_policy_loss_args, read_masked_rows));return 0;}\n"
     )
     exe = tmp_path / "layout"
     subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
     (size, off_n, off_eps, off_metrics, nmet, off_extra, off_kind, off_is, off_tk_ids, off_tk_k, off_tk_clamp,
-     off_tk_grad, tk_max) = map(int, subprocess.check_output([str(exe)]).split())
+     off_tk_grad, tk_max, off_masked) = map(int, subprocess.check_output([str(exe)]).split())
     S = _lib.PolicyLossArgs
     assert C.sizeof(S) == size
     assert S.n_samples.offset == off_n and S.eps_clip.offset == off_eps and S.metrics.offset == off_metrics
@@ -47,7 +48,7 @@ def test_struct_layout_matches_c_header(tmp_path):
     assert S.distill_is_clip.offset == off_is
     assert S.topk_ids.offset == off_tk_ids and S.topk_k.offset == off_tk_k
     assert S.topk_min_clamp.offset == off_tk_clamp and S.topk_grad.offset == off_tk_grad
-    assert tk_max == _lib.FUSED_TOPK_MAX
+    assert tk_max == _lib.FUSED_TOPK_MAX and S.read_masked_rows.offset == off_masked
     assert nmet == _lib.NUM_METRICS
 
 

@@ -1100,8 +1100,8 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
     kw = dict(relax_amd_single_pass=single_pass, opd_loss_coef=0.7, use_kl_loss=True, kl_loss_coef=0.01,
               kl_loss_type="k3")
     if case.endswith("_all_tokens"):
-        # no masked token: the clipped signals' derivative is evaluated inside the single launch (with masked tokens
-        # their clip-fraction metrics need log-probs the single launch does not produce, and two launches run)
+        # no masked token at all (with masked tokens the single launch scans their rows as well: the clip-fraction
+        # metrics average over them)
         batch["loss_masks"] = [torch.ones_like(m) for m in batch["loss_masks"]]
         case = case[:-len("_all_tokens")]
     if case == "sampled_plain":  # linear in the log-probs: its gradient leaves with the single launch
@@ -1129,7 +1129,7 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
         elif case == "topk_norm_clamped_clips":
             kw.update(opd_token_selection="student_topk", opd_kl_type="jsd", opd_jsd_alpha=0.3, opd_norm_mode="norm",
                       opd_log_prob_min_clamp=-7.0, opd_per_token_clip=0.5, opd_is_clip=0.99)
-        elif case == "topk_clips_masked":  # clips with masked tokens: their metrics need every row, two launches run
+        elif case == "topk_clips_masked":  # clips with masked tokens: the launch scans the masked rows as well
             kw.update(opd_token_selection="teacher_topk", opd_kl_type="reverse_kl", opd_per_token_clip=0.5)
         elif case == "topk_ragged_widths":  # samples with different K: packed to the widest, trimmed per token
             kw.update(opd_token_selection="teacher_topk", opd_kl_type="jsd", opd_jsd_alpha=0.6, opd_norm_mode="tail")
@@ -1183,7 +1183,7 @@ def test_topk_opd_term_in_the_register_resident_step(v, dtype, k, variant):
         kw.update(opd_token_selection="union", opd_kl_type="jsd", opd_jsd_alpha=0.4, opd_norm_mode="trunc",
                   opd_log_prob_min_clamp=-14.0, opd_per_token_clip=0.05, opd_is_clip=1.01)
         batch["opd_topk_ksz"] = [torch.randint(1, k + 1, (r,), generator=g) for r in resp]
-        batch["loss_masks"] = [torch.ones_like(m) for m in batch["loss_masks"]]
+        batch["loss_masks"][1] = torch.zeros_like(batch["loss_masks"][1])  # masked rows are scanned: clip metrics
     elif variant == "forward_norm":
         kw.update(opd_token_selection="student_topk", opd_kl_type="forward_kl", opd_norm_mode="norm")
     else:
@@ -1214,7 +1214,8 @@ def test_topk_opd_term_in_the_register_resident_step(v, dtype, k, variant):
 def test_linear_opd_term_rides_the_single_launch(monkeypatch):
     """Sampled-token distillation signals (plain reverse_kl: linear in the log-probs; low_var_kl or clipped: derivative
     evaluated by the kernel) and the top-K signals (evaluated by the kernel next to each row's log-sum-exp): one fused
-    launch, no separate log-prob or dlogits launch."""
+    launch, no separate log-prob or dlogits launch; with clips on a batch that has masked tokens the launch scans the
+    masked rows too (their clip-fraction metrics need those log-probs) and is still the only one."""
     import relax_amd
     from relax_amd import ops
 
@@ -1228,11 +1229,10 @@ def test_linear_opd_term_rides_the_single_launch(monkeypatch):
     for name in ("actor_step_fused", "logprob_entropy_fwd", "logprob_entropy_bwd"):
         real = getattr(ops, name)
         monkeypatch.setattr(ops, name, lambda *a, _n=name, _r=real, **k: (calls.append(_n), _r(*a, **k))[1])
-    two = ["logprob_entropy_fwd", "logprob_entropy_bwd"]
     ones = [torch.ones_like(m) for m in batch["loss_masks"]]
     for kl_type, clip, masks, want in (
             ("reverse_kl", None, None, ["actor_step_fused"]), ("low_var_kl", None, None, ["actor_step_fused"]),
-            ("reverse_kl", 0.02, ones, ["actor_step_fused"]), ("reverse_kl", 0.02, None, two)):
+            ("reverse_kl", 0.02, ones, ["actor_step_fused"]), ("reverse_kl", 0.02, None, ["actor_step_fused"])):
         calls.clear()
         case_batch = batch if masks is None else dict(batch, loss_masks=masks)
         args = P.make_args(opd_loss_coef=0.7, opd_token_selection="sampled", opd_kl_type=kl_type,
@@ -1246,7 +1246,8 @@ def test_linear_opd_term_rides_the_single_launch(monkeypatch):
     batch["opd_topk_teacher_log_probs"] = [torch.log_softmax(torch.randn(r, v, generator=g), -1)[:, :k].contiguous()
                                            for r in resp]
     for kl_type, clip, masks, want in (("reverse_kl", None, None, ["actor_step_fused"]),
-                                       ("jsd", 0.5, ones, ["actor_step_fused"]), ("jsd", 0.5, None, two)):
+                                       ("jsd", 0.5, ones, ["actor_step_fused"]),
+                                       ("jsd", 0.5, None, ["actor_step_fused"])):
         calls.clear()
         case_batch = batch if masks is None else dict(batch, loss_masks=masks)
         args = P.make_args(opd_loss_coef=0.7, opd_token_selection="teacher_topk", opd_kl_type=kl_type,
