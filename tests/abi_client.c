@@ -5,7 +5,9 @@
  * of two rows, and compares with the closed forms evaluated here in double precision; then the one-read log-prob +
  * top-K entry point on the same rows (k = 2) and the group-normalised rewards of the reference's GRPO literal
  * (tests/utils/training/test_rloo_advantages.py:160-172: rewards [0,1,0,1] in one group -> (r - 0.5) / (std + 1e-6)
- * with the sample standard deviation) and its leave-one-out brute force.  Exit status 0 = all good. */
+ * with the sample standard deviation) and its leave-one-out brute force; then the fused actor step with the top-K
+ * distillation term (relax_amd_actor_step_fused + relax_amd_sparse_row_add + relax_amd_policy_loss) against its closed
+ * form.  Exit status 0 = all good. */
 #include <hip/hip_runtime_api.h>
 #include <math.h>
 #include <stdint.h>
@@ -168,6 +170,87 @@ int main(void) {
       for (int j = 0; j < G; ++j)
         if (j != i) others += rewards[j];
       ok &= close_enough("rloo reward", i, out[i], rewards[i] - others / (G - 1), 1e-6);
+    }
+  }
+  /* the fused actor step with the top-K distillation term, from C: PPO at ratio 1 (no old log-probs), token-mean over
+   * one sample of three tokens, plus 0.5 * mean_t KL_t with KL_t = sum_k p_k (log p_k - teacher_k) over two given ids
+   * per row (reverse KL, entries used as they are); then the K one-hot parts; against the closed forms:
+   *   dlogits[t, v] = -(A_t / 3) (1[v = token_t] - p_v) + sum_k w d_k (1[v = id_k] - p_v),  d_k = p_k (log p_k - teacher_k + 1) */
+  {
+    enum { K = 2 };
+    const float adv[N] = {1.0f, -2.0f, 0.5f}, ones[N] = {1, 1, 1}, denom[1] = {3.0f};
+    const int64_t cu[2] = {0, N}, ids[N][K] = {{3, 1}, {0, 2}, {1, 3}};
+    const int32_t sample_ids[N] = {0, 0, 0};
+    const float teacher_lp[N][K] = {{-0.5f, -2.0f}, {-0.3f, -3.0f}, {-1.0f, -1.5f}};
+    const float w = 0.5f / 3.0f, weight[N] = {w, w, w};
+    void *d_adv = to_device(adv, sizeof adv), *d_mask = to_device(ones, sizeof ones), *d_den = to_device(denom, sizeof denom);
+    void *d_cu = to_device(cu, sizeof cu), *d_ids = to_device(ids, sizeof ids), *d_sid = to_device(sample_ids, sizeof sample_ids);
+    void *d_tlp = to_device(teacher_lp, sizeof teacher_lp), *d_w = to_device(weight, sizeof weight);
+    float *d_coef = to_device(NULL, N * sizeof(float)), *d_part = to_device(NULL, RELAX_AMD_NUM_METRICS * sizeof(float));
+    float *d_met = to_device(NULL, RELAX_AMD_NUM_METRICS * sizeof(float)), *d_tkl = to_device(NULL, N * sizeof(float));
+    float* d_tgrad = to_device(NULL, N * K * sizeof(float));
+    float *d_lp3 = to_device(NULL, N * sizeof(float)), *d_ent3 = to_device(NULL, N * sizeof(float));
+    if (!d_adv || !d_mask || !d_den || !d_cu || !d_ids || !d_sid || !d_tlp || !d_w || !d_coef || !d_part || !d_met ||
+        !d_tkl || !d_tgrad || !d_lp3 || !d_ent3)
+      return 2;
+    relax_amd_policy_loss_args a = {0};
+    a.advantages = d_adv;
+    a.loss_mask = d_mask;
+    a.cu_resp = d_cu;
+    a.sample_denom = d_den;
+    a.n_samples = 1;
+    a.n_tokens = N;
+    a.loss_kind = RELAX_AMD_LOSS_PPO;
+    a.kl_kind = RELAX_AMD_KL_NONE;
+    a.eps_clip = a.eps_clip_high = 0.2f;
+    a.eps_clip_c = -1.0f;
+    a.tis_hi = 2.0f;
+    a.coef_log_prob = d_coef;
+    a.sample_partials = d_part;
+    a.metrics = d_met;
+    a.extra_coef_log_prob = d_w;
+    a.distill_min_clamp = a.distill_token_clip = a.distill_is_clip = NAN;
+    a.topk_ids = d_ids;
+    a.topk_teacher_log_prob = d_tlp;
+    a.topk_k = K;
+    a.topk_kl_mode = RELAX_AMD_OPD_JSD;
+    a.topk_norm_mode = RELAX_AMD_OPD_NORM_TRUNC;
+    a.topk_jsd_alpha = 0.0f;
+    a.topk_kl = d_tkl;
+    a.topk_grad = d_tgrad;
+    CHECK_LIB(relax_amd_actor_step_fused(d_logits, RELAX_AMD_F32, N, V, V, NULL, (const int32_t*)d_sid,
+                                         (const int64_t*)d_tokens, 1.0f, &a, 1.0f, d_lp3, d_ent3, d_lse, d_spx, d_grad, V,
+                                         stream));
+    CHECK_LIB(relax_amd_sparse_row_add(d_grad, RELAX_AMD_F32, N, V, V, NULL, (const int64_t*)d_ids, d_tgrad, K, NULL, NULL,
+                                       1.0f, stream));
+    a.log_prob = d_lp3; /* the loss value and metrics of the policy terms, from the step's log-probs */
+    a.entropy = d_ent3;
+    CHECK_LIB(relax_amd_policy_loss(&a, stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    float lp3[N], tkl[N], met[RELAX_AMD_NUM_METRICS];
+    CHECK_HIP(hipMemcpy(lp3, d_lp3, sizeof lp3, hipMemcpyDeviceToHost));
+    CHECK_HIP(hipMemcpy(tkl, d_tkl, sizeof tkl, hipMemcpyDeviceToHost));
+    CHECK_HIP(hipMemcpy(met, d_met, sizeof met, hipMemcpyDeviceToHost));
+    CHECK_HIP(hipMemcpy(grad, d_grad, sizeof grad, hipMemcpyDeviceToHost));
+    ok &= close_enough("fused pg loss", 0, met[RELAX_AMD_M_PG_LOSS], -(1.0 - 2.0 + 0.5) / 3.0, 2e-6);
+    for (int i = 0; i < N; ++i) {
+      double z = 0;
+      for (int v = 0; v < V; ++v) z += exp((double)logits[i][v]);
+      const double lse = log(z);
+      ok &= close_enough("fused log_prob", i, lp3[i], lp[i], 0.0);
+      double want_kl = 0, dk[K];
+      for (int k = 0; k < K; ++k) {
+        const double s = logits[i][ids[i][k]] - lse;
+        want_kl += exp(s) * (s - teacher_lp[i][k]);
+        dk[k] = exp(s) * (s - teacher_lp[i][k] + 1.0);
+      }
+      ok &= close_enough("fused top-K KL", i, tkl[i], want_kl, 2e-6);
+      for (int v = 0; v < V; ++v) {
+        const double p = exp(logits[i][v] - lse);
+        double want = -(adv[i] / 3.0) * ((v == tokens[i]) - p);
+        for (int k = 0; k < K; ++k) want += w * dk[k] * ((v == ids[i][k]) - p);
+        ok &= close_enough("fused dlogits", i * V + v, grad[i][v], want, 2e-6);
+      }
     }
   }
   /* error path: the library reports instead of launching */
