@@ -145,7 +145,8 @@ __global__ __launch_bounds__(256) void opd_kl_topk_kernel(const float* __restric
 // dlogits[row(t), id] += value * scale for the K (id, value) pairs of token t plus one pair at its target id: the
 // sparse part of a gradient whose dense part (a multiple of the row's softmax) another kernel has already written.
 // One thread walks all pairs of a token one after the other, so two pairs on the same element (a gathered id that
-// equals the target) cannot race; ids outside [0, vocab) are skipped.
+// equals the target) cannot race; ids outside [0, vocab) are skipped.  (The form for very long lists; the usual ones
+// take sparse_row_add_wave_kernel below.)
 template <typename T>
 __global__ __launch_bounds__(256) void sparse_row_add_kernel(T* __restrict__ dlogits, int64_t stride, int64_t vocab,
                                                              const int32_t* __restrict__ row_ids,
@@ -169,6 +170,53 @@ __global__ __launch_bounds__(256) void sparse_row_add_kernel(T* __restrict__ dlo
   }
 }
 
+// The same for up to kSparseWaveMax pairs per token, one wave per token: lane l takes pairs l, l + 64, ... (the target
+// pair counts as the last one).  Pairs on the same element are all applied by the lane of the first of them, so no two
+// lanes touch one element; elements are read and written at their own width, so neighbours in one 32-bit word do not
+// collide.
+constexpr int kSparseWaveMax = 1024;
+
+template <typename T>
+__global__ __launch_bounds__(256) void sparse_row_add_wave_kernel(T* __restrict__ dlogits, int64_t stride,
+                                                                  int64_t vocab, const int32_t* __restrict__ row_ids,
+                                                                  const int64_t* __restrict__ ids,
+                                                                  const float* __restrict__ values, int k,
+                                                                  const int64_t* __restrict__ targets,
+                                                                  const float* __restrict__ target_values, float scale,
+                                                                  int64_t n_tokens) {
+  extern __shared__ int64_t sparse_stage[];  // [4 waves][k + 1] ids, then [4 waves][k + 1] values
+  const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+  const int64_t tok = blockIdx.x * 4LL + w;
+  if (tok >= n_tokens) return;
+  const int n = k + (targets ? 1 : 0);
+  int64_t* sid = sparse_stage + w * (k + 1);
+  float* sval = reinterpret_cast<float*>(sparse_stage + 4 * (k + 1)) + w * (k + 1);
+  for (int j = lane; j < n; j += kWave) {
+    const int64_t id = j < k ? ids[tok * k + j] : targets[tok];
+    const float v = j < k ? values[tok * k + j] : target_values[tok];
+    const bool live = id >= 0 && id < vocab && v != 0.f;
+    sid[j] = live ? id : -1;
+    sval[j] = v;
+  }
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  T* d = dlogits + (row_ids ? int64_t(row_ids[tok]) : tok) * stride;
+  for (int j = lane; j < n; j += kWave) {
+    const int64_t id = sid[j];
+    if (id < 0) continue;
+    bool first = true;
+    for (int o = 0; o < j; ++o) first = first && sid[o] != id;
+    if (!first) continue;
+    // this pair and, one after the other, the later ones on the same element: each addition rounded to the element
+    // type, as a walk over the list in its order would do
+    T* slot = d + id;
+    Row<T>::store1(slot, Row<T>::load1(const_cast<const T*>(slot)) + sval[j] * scale);
+    for (int o = j + 1; o < n; ++o)
+      if (sid[o] == id) Row<T>::store1(slot, Row<T>::load1(const_cast<const T*>(slot)) + sval[o] * scale);
+  }
+}
+
 }  // namespace relax_amd
 
 using namespace relax_amd;
@@ -185,6 +233,21 @@ extern "C" int relax_amd_sparse_row_add(void* dlogits, int dtype, int64_t n_toke
     return RELAX_AMD_EINVAL;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (k < kSparseWaveMax) {  // one wave per token
+    const dim3 wgrid(static_cast<unsigned>((n_tokens + 3) / 4)), wblock(256);
+    const size_t lds = size_t(4) * size_t(k + 1) * (sizeof(int64_t) + sizeof(float));
+#define RELAX_AMD_SPARSE_WAVE(T)                                                                                   \
+  hipLaunchKernelGGL(sparse_row_add_wave_kernel<T>, wgrid, wblock, lds, s, static_cast<T*>(dlogits), row_stride,    \
+                     vocab, row_ids, ids, values, int(k), targets, target_values, scale, n_tokens)
+    switch (dtype) {
+      case RELAX_AMD_F32: RELAX_AMD_SPARSE_WAVE(float); break;
+      case RELAX_AMD_BF16: RELAX_AMD_SPARSE_WAVE(bf16_t); break;
+      case RELAX_AMD_F16: RELAX_AMD_SPARSE_WAVE(f16_t); break;
+      default: set_error("sparse_row_add: unknown dtype code %d", dtype); return RELAX_AMD_EINVAL;
+    }
+#undef RELAX_AMD_SPARSE_WAVE
+    return check_launch("sparse_row_add");
+  }
   const dim3 grid(static_cast<unsigned>((n_tokens + 255) / 256)), block(256);
   switch (dtype) {
     case RELAX_AMD_F32:
