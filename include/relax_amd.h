@@ -422,10 +422,14 @@ int relax_amd_logprob_entropy_topk_fwd(const void* logits, int dtype, int64_t n_
  *   sample_ids  [n_tokens] int32 sample of each token (needed with per-sample denominators)
  *   grad_scale  host scalar folded into dlogits (the upstream gradient the caller expects, normally 1)
  *   log_prob, entropy, lse, spx  [n_tokens] out; tokens whose masks are both zero get zeros (their row is not read)
+ *               unless loss->read_masked_rows is set
  *   dlogits     [n_rows, vocab] out, every row written (zero rows where token_of_row < 0 or the coefficients vanish)
+ * With loss->topk_ids set the step also evaluates the top-K distillation signal of every row it reads (see the
+ * argument block); the caller adds the K one-hot parts of its gradient with relax_amd_sparse_row_add afterwards.
  * Two kernels sit behind this entry point and are chosen by row length and element type: a register-resident one
- * (one read and one write of HBM per row; 16-bit rows of 100352 .. 152064 entries in the built shapes) and a two-walk
- * one for everything else; RELAX_AMD_FUSED_STEP_KERNEL=cached in the environment forces the latter.  Same results.
+ * (one read and one write of HBM per row; 16-bit rows of 100352 .. 152064 entries and fp32 rows of 32000 entries in
+ * the built shapes) and a two-walk one for everything else; RELAX_AMD_FUSED_STEP_KERNEL=cached in the environment
+ * forces the latter.  Same results.
  */
 int relax_amd_actor_step_fused(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                                const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,

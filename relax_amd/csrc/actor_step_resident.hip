@@ -1,9 +1,11 @@
 // Register-resident fused actor step: the same computation as actor_step_fused_kernel (log-prob + entropy forward,
-// per-token policy-loss coefficients, dlogits backward, one launch) for long 16-bit rows of the common vocabulary sizes.
+// per-token policy-loss coefficients, dlogits backward, one launch) for long 16-bit rows of the common vocabulary sizes
+// and for fp32 rows of 32000 entries.
 //
 // A 1024-thread workgroup holds a whole row in its vector registers (V = 151936 bf16 is 18992 16-byte vectors = 19 per
 // thread = 76 registers), so HBM sees exactly one read and one write per row and the second walk over the row costs no
-// cache or fabric traffic at all.  One such workgroup fits a CU; the workgroups are persistent (one per CU, rows b,
+// cache or fabric traffic at all.  One such workgroup fits a CU (fp32 rows: 512-thread workgroups with 16 vectors per
+// thread, two per CU); the workgroups are persistent (one per CU, rows b,
 // b + grid, ...) and take a row in three steps: the resident row becomes its gradient in place; the gradient leaves in
 // one burst of stores and, into the registers those free, the workgroup's next live row arrives in one burst of loads
 // (304 KB out, 304 KB in, each contiguous); the new row's softmax scan follows its loads in their order.  Memory rewards
