@@ -1211,6 +1211,42 @@ def test_topk_opd_term_in_the_register_resident_step(v, dtype, k, variant):
     torch.testing.assert_close(outs["auto"][2].float().cpu(), lo.grad, atol=tol, rtol=max(2 * ulp, 1e-5))
 
 
+@pytest.mark.parametrize("k", [1, 63, 65, 256, 300])
+def test_topk_opd_term_widths_of_the_single_launch(k, monkeypatch):
+    """K = 1, around one wave's width, the largest K the single launch takes and one beyond it (two launches), with
+    repeated ids in a row: loss, metrics and dlogits against the oracle, and which launches ran."""
+    import relax_amd
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("top-K OPD widths", k)
+    tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 3000
+    logits, batch = _make_batch(41, tot, resp, v)
+    g = torch.Generator().manual_seed(k)
+    batch["opd_topk_token_ids"] = [torch.randint(0, v, (r, k), generator=g) for r in resp]
+    batch["opd_topk_token_ids"][2][1, 0] = batch["opd_topk_token_ids"][2][1, k - 1]  # a repeated id (k > 1)
+    batch["opd_topk_teacher_log_probs"] = [torch.log_softmax(torch.randn(r, 2 * k + 3, generator=g), -1)[:, :k]
+                                           .contiguous() for r in resp]
+    args = P.make_args(opd_loss_coef=0.7, opd_token_selection="teacher_topk", opd_kl_type="jsd", opd_jsd_alpha=0.5,
+                       opd_norm_mode="trunc", use_kl_loss=True, kl_loss_coef=0.01, kl_loss_type="k3")
+    calls = []
+    for name in ("actor_step_fused", "logprob_entropy_fwd", "logprob_entropy_bwd"):
+        real = getattr(ops, name)
+        monkeypatch.setattr(ops, name, lambda *a, _n=name, _r=real, **kw: (calls.append(_n), _r(*a, **kw))[1])
+    lo = logits.clone().requires_grad_()
+    want_loss, want_m = P.policy_loss_function(args, dict(batch), lo, R.make_reducer(resp, batch["loss_masks"]))
+    want_loss.backward()
+    lg = logits.to(dev).requires_grad_()
+    loss, met = relax_amd.policy_loss_function(args, _to_dev(batch, dev), lg, None)
+    loss.backward()
+    assert calls == (["actor_step_fused"] if k <= 256 else ["logprob_entropy_fwd", "logprob_entropy_bwd"]), calls
+    assert abs(loss.item() - want_loss.item()) < 3e-5 * max(1.0, abs(want_loss.item()))
+    assert set(met) == set(want_m)
+    for key, w in want_m.items():
+        assert abs(met[key].item() - float(w)) < 3e-5 * max(1.0, abs(float(w))), key
+    torch.testing.assert_close(lg.grad.cpu(), lo.grad, atol=3e-5, rtol=1e-5)
+
+
 def test_linear_opd_term_rides_the_single_launch(monkeypatch):
     """Sampled-token distillation signals (plain reverse_kl: linear in the log-probs; low_var_kl or clipped: derivative
     evaluated by the kernel) and the top-K signals (evaluated by the kernel next to each row's log-sum-exp): one fused
