@@ -320,24 +320,28 @@ extern "C" int relax_amd_actor_step_fused(const void* logits, int dtype, int64_t
 // assumed at forward time without a host read-back.
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void rescale_rows_kernel(T* __restrict__ data, int64_t stride, int64_t vocab,
-                                                           const float* __restrict__ factor) {
+                                                           int64_t n_rows, const float* __restrict__ factor) {
   const float f = *factor;
   if (fabsf(f - 1.0f) <= 0x1p-20f) return;
-  T* r = data + int64_t(blockIdx.x) * stride;
-  if constexpr (VEC) {
-    constexpr int kPer = Row<T>::kPerVec;
-    u32x4* rv = reinterpret_cast<u32x4*>(r);
-    const int64_t nvec = vocab / kPer;
-    for (int64_t i = threadIdx.x; i < nvec; i += 256) {
-      float x[kPer];
-      Row<T>::unpack(rv[i], x);
-#pragma unroll
-      for (int k = 0; k < kPer; ++k) x[k] *= f;
-      rv[i] = Row<T>::pack(x);
+  // a bounded grid walks the rows: in the usual case (factor 1) the launch is a few thousand workgroups that return
+  // at once instead of one per row
+  for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+    T* r = data + row * stride;
+    if constexpr (VEC) {
+      constexpr int kPer = Row<T>::kPerVec;
+      u32x4* rv = reinterpret_cast<u32x4*>(r);
+      const int64_t nvec = vocab / kPer;
+      for (int64_t i = threadIdx.x; i < nvec; i += 256) {
+        float x[kPer];
+        Row<T>::unpack(rv[i], x);
+  #pragma unroll
+        for (int k = 0; k < kPer; ++k) x[k] *= f;
+        rv[i] = Row<T>::pack(x);
+      }
+      for (int64_t e = nvec * kPer + threadIdx.x; e < vocab; e += 256) Row<T>::store1(r + e, Row<T>::load1(r + e) * f);
+    } else {
+      for (int64_t e = threadIdx.x; e < vocab; e += 256) Row<T>::store1(r + e, Row<T>::load1(r + e) * f);
     }
-    for (int64_t e = nvec * kPer + threadIdx.x; e < vocab; e += 256) Row<T>::store1(r + e, Row<T>::load1(r + e) * f);
-  } else {
-    for (int64_t e = threadIdx.x; e < vocab; e += 256) Row<T>::store1(r + e, Row<T>::load1(r + e) * f);
   }
 }
 
@@ -345,11 +349,13 @@ template <typename T>
 static void launch_rescale(void* data, int64_t n_rows, int64_t vocab, int64_t stride, const float* factor,
                            hipStream_t s) {
   const bool vec = aligned16(data) && (stride * int64_t(sizeof(T))) % 16 == 0;
-  const dim3 grid(static_cast<unsigned>(n_rows)), block(256);
+  const dim3 grid(static_cast<unsigned>(n_rows < 4096 ? n_rows : 4096)), block(256);
   if (vec)
-    hipLaunchKernelGGL((rescale_rows_kernel<T, true>), grid, block, 0, s, static_cast<T*>(data), stride, vocab, factor);
+    hipLaunchKernelGGL((rescale_rows_kernel<T, true>), grid, block, 0, s, static_cast<T*>(data), stride, vocab, n_rows,
+                       factor);
   else
-    hipLaunchKernelGGL((rescale_rows_kernel<T, false>), grid, block, 0, s, static_cast<T*>(data), stride, vocab, factor);
+    hipLaunchKernelGGL((rescale_rows_kernel<T, false>), grid, block, 0, s, static_cast<T*>(data), stride, vocab, n_rows,
+                       factor);
 }
 
 extern "C" int relax_amd_scale_rows_inplace(void* data, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
