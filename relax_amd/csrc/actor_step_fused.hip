@@ -201,12 +201,14 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
   }
 }
 
-// RELAX_AMD_FUSED_STEP_KERNEL = "cached" forces the two-walk kernel (second walk out of cache); unset or anything
-// else lets the row lengths the register-resident kernel is built for take that one.  Read at every launch; meant for
-// measurements.
-static bool fused_step_force_cached() {
+// RELAX_AMD_FUSED_STEP_KERNEL = "cached" forces the two-walk kernel (second walk out of cache); "resident" insists on
+// the register-resident one and makes the call fail for rows it is not built for (so that a comparison of the two
+// cannot pass on one kernel compared with itself); unset or anything else lets the row lengths the register-resident
+// kernel is built for take that one and all others the two-walk kernel.  Read at every launch; meant for measurements
+// and tests.
+static bool fused_step_kernel_is(const char* name) {
   const char* e = getenv("RELAX_AMD_FUSED_STEP_KERNEL");
-  return e && strcmp(e, "cached") == 0;
+  return e && strcmp(e, name) == 0;
 }
 
 static int device_compute_units() {
@@ -227,10 +229,15 @@ static int dispatch_fused(const void* logits, int64_t n_rows, int64_t vocab, int
   const T* x = static_cast<const T*>(logits);
   T* d = static_cast<T*>(dlogits);
   dim3 grid(static_cast<unsigned>(n_rows));
-  if (vec && !fused_step_force_cached()) {
+  if (vec && !fused_step_kernel_is("cached")) {
     const int rc = launch_actor_step_resident<T>(x, stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t, a,
                                                  grad_scale, lp, ent, lse, spx, d, d_stride, device_compute_units(), s);
     if (rc != RELAX_AMD_EUNSUPPORTED) return rc;  // launched (or failed to): otherwise the row length is not built
+  }
+  if (fused_step_kernel_is("resident")) {
+    set_error("actor_step_fused: RELAX_AMD_FUSED_STEP_KERNEL=resident, but no register-resident kernel is built for "
+              "rows of %lld elements of this type and alignment", (long long)vocab);
+    return RELAX_AMD_EUNSUPPORTED;
   }
 #define RELAX_AMD_FUSED(V, TH)                                                                                     \
   hipLaunchKernelGGL((actor_step_fused_kernel<T, V, TH>), grid, dim3(TH), 0, s, x, stride, vocab, token_of_row,       \

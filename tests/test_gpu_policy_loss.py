@@ -1634,6 +1634,46 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
         assert not results["resident"]["d"].any()
 
 
+@pytest.mark.parametrize("v,dtype", [(8 * (18 * 1024 + 1), torch.bfloat16), (8 * (19 * 1024 - 1), torch.bfloat16),
+                                     (8 * (12 * 1024 + 1), torch.float16), (8 * (16 * 1024 - 1), torch.bfloat16),
+                                     (4 * (15 * 512 + 1), torch.float32), (4 * (16 * 512 - 1), torch.float32)])
+def test_register_resident_kernel_at_the_edges_of_its_row_shapes(v, dtype, monkeypatch):
+    """Row lengths at both ends of a built shape: one lane, or all lanes but one, hold a vector at the partially filled
+    position.  Every output bit-identical to the two-walk kernel's."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("resident kernel, shape edges", v, dtype)
+    n_rows = 600 if dtype != torch.float32 else 1200
+    g = torch.Generator().manual_seed(v)
+    logits = (torch.randn(n_rows, v, generator=g) * 2).to(dtype).to(dev)
+    scores = torch.rand(n_rows, generator=g) > 0.2
+    idx = torch.cumsum(scores.int(), 0) - 1
+    token_of_row = torch.where(scores, idx, torch.full_like(idx, -1)).int().to(dev)
+    n_tok = int(scores.sum())
+    mask = (torch.rand(n_tok, generator=g) > 0.2).float()
+    base = -2.0 + 0.3 * torch.randn(n_tok, generator=g)
+    targets = torch.randint(0, v, (n_tok,), generator=g)
+    targets[:4] = torch.tensor([0, v - 1, v - 2, v // 2])  # the row's first and last elements among the targets
+    kw = dict(advantages=torch.randn(n_tok, generator=g).to(dev), loss_mask=mask.to(dev),
+              cu_resp=torch.tensor([0, n_tok], dtype=torch.int64, device=dev), old_log_prob=base.to(dev),
+              ref_log_prob=(base + 0.1 * torch.randn(n_tok, generator=g)).to(dev), kl_kind="k3", kl_coef=1e-3,
+              entropy_coef=0.01, sample_denom=torch.tensor([max(1.0, mask.sum().item())], device=dev),
+              loss_kind="ppo", eps_clip=0.2, eps_clip_high=0.28)
+    sample_ids = torch.zeros(n_tok, dtype=torch.int32, device=dev)
+    results = {}
+    for kind in ("cached", "resident"):
+        monkeypatch.setenv("RELAX_AMD_FUSED_STEP_KERNEL", kind)
+        out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets.to(dev), token_of_row, sample_ids, n_tok, 1.0,
+                                                         1.0, **kw)
+        torch.cuda.synchronize()
+        results[kind] = dict(lp=lp, ent=ent, lse=lse, spx=spx, coef=out["coef_log_prob"],
+                             d=d.view(torch.int16 if dtype != torch.float32 else torch.int32))
+    for key, want in results["cached"].items():
+        assert torch.equal(results["resident"][key], want), key
+    assert results["resident"]["d"].any()
+
+
 def test_forward_only_topk_gather_on_logits_that_require_grad():
     """The ActorFwd pass runs under ``torch.no_grad()`` on logits that may still carry ``requires_grad``: the top-K
     gather then reuses the log-prob launch's log-sum-exps and returns the same values as the differentiable path."""
