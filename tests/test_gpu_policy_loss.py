@@ -1247,6 +1247,61 @@ def test_topk_opd_term_widths_of_the_single_launch(k, monkeypatch):
     torch.testing.assert_close(lg.grad.cpu(), lo.grad, atol=3e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_topk_opd_term_random_option_sweep_vs_oracle(seed):
+    """Random draws over the top-K term's options (KL family and jsd_alpha, norm mode, lower clamp, per-token and
+    importance-ratio clips, selection with and without the union mask, ragged per-sample K, masked tokens and a fully
+    masked sample, temperature, per-token-loss reduction) through the single launch: loss, metrics and dlogits against
+    the oracle."""
+    import relax_amd
+
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(1000 + seed)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=g))]
+
+    tot, resp = [9, 6, 12, 7, 5], [4, 3, 7, 5, 2]
+    v = pick([264, 1000, 3001])
+    k = pick([1, 3, 8, 70])
+    logits, batch = _make_batch(50 + seed, tot, resp, v)
+    kl_type = pick(["reverse_kl", "forward_kl", "jsd", "low_var_kl"])
+    selection = pick(["teacher_topk", "student_topk", "union"])
+    kw = dict(opd_loss_coef=pick([0.3, 1.0]), opd_token_selection=selection, opd_kl_type=kl_type,
+              opd_jsd_alpha=pick([0.2, 0.5, 0.9]), opd_norm_mode=pick(["tail", "norm", "trunc"]),
+              opd_log_prob_min_clamp=pick([None, -6.0, -12.0]), opd_per_token_clip=pick([None, 0.05, 2.0]),
+              opd_is_clip=pick([None, 0.99, 1.05]), rollout_temperature=pick([1.0, 0.7]),
+              calculate_per_token_loss=pick([False, True]), use_kl_loss=True, kl_loss_coef=0.01, kl_loss_type="k3",
+              entropy_coef=pick([0.0, 0.01]))
+    if selection == "union" and kw["opd_norm_mode"] == "norm":
+        kw["opd_norm_mode"] = "tail"  # the reference's autograd returns NaN for masked entries under "norm"
+    announce("top-K OPD option sweep", seed, v, k, kl_type, selection, kw["opd_norm_mode"])
+    widths = [k] * len(resp)
+    if pick([False, True]) and k > 1:
+        widths = [int(torch.randint(1, k + 1, (1,), generator=g)) for _ in resp]
+    batch["opd_topk_token_ids"] = [torch.stack([torch.randperm(v, generator=g)[:w] for _ in range(r)])
+                                   for r, w in zip(resp, widths)]
+    batch["opd_topk_teacher_log_probs"] = [torch.log_softmax(2 * torch.randn(r, 3 * w + 2, generator=g), -1)[:, :w]
+                                           .contiguous() for r, w in zip(resp, widths)]
+    if selection == "union":
+        batch["opd_topk_ksz"] = [torch.randint(1, w + 1, (r,), generator=g) for r, w in zip(resp, widths)]
+    if pick([False, True]):
+        batch["loss_masks"][1] = torch.zeros_like(batch["loss_masks"][1])
+    args = P.make_args(**kw)
+    lo = logits.clone().requires_grad_()
+    want_loss, want_m = P.policy_loss_function(args, dict(batch), lo, R.make_reducer(resp, batch["loss_masks"],
+                                                                                     kw["calculate_per_token_loss"]))
+    want_loss.backward()
+    lg = logits.to(dev).requires_grad_()
+    loss, met = relax_amd.policy_loss_function(args, _to_dev(batch, dev), lg, None)
+    loss.backward()
+    assert abs(loss.item() - want_loss.item()) < 5e-5 * max(1.0, abs(want_loss.item())), (loss.item(), want_loss.item())
+    assert set(met) == set(want_m), (sorted(met), sorted(want_m))
+    for key, w in want_m.items():
+        assert abs(met[key].item() - float(w)) < 5e-5 * max(1.0, abs(float(w))), (key, met[key].item(), float(w))
+    torch.testing.assert_close(lg.grad.cpu(), lo.grad, atol=5e-5, rtol=2e-5)
+
+
 def test_linear_opd_term_rides_the_single_launch(monkeypatch):
     """Sampled-token distillation signals (plain reverse_kl: linear in the log-probs; low_var_kl or clipped: derivative
     evaluated by the kernel) and the top-K signals (evaluated by the kernel next to each row's log-sum-exp): one fused
