@@ -5,11 +5,17 @@
 // A 1024-thread workgroup keeps the STUDENT row in its vector registers (19 16-byte vectors per thread at
 // V = 151936) and streams the teacher row past it twice: once for the two online softmaxes, once for the gradient
 // d = p_s * g * ((x_s - x_t) + lse_t - lse_s - KL).  HBM sees the student row once instead of twice (the two-walk
-// kernel re-fetches ~85 % of both rows through the fabric).  Workgroups are persistent, one per CU, rows b, b + grid,
-// ...; a row's gradient replaces the student row in the registers, leaves in one burst of stores, and the workgroup's
-// next student row arrives in one burst of loads (with a store and a load alternating vector by vector behind the
-// gradient arithmetic the launch took 2.97 ms on 16384 x 151936 rows instead of 2.84 ms: memory rewards the long
-// bursts).  No workgroup waits for another; the loop bound is the only exit condition.
+// kernel re-fetches ~85 % of both rows through the fabric).  The teacher row passes through eight slots of LDS (one
+// 16-byte vector per thread each, 128 KB), filled by loads that go from global memory straight to LDS: up to eight
+// vectors per thread are in flight ahead of their use without a register being held for them, and since the scan ends
+// with the row's last eight vectors in the slots, the gradient pass walks the row backwards and reads only the other
+// NV - 8 again.  Workgroups are persistent, one per CU, rows b, b + grid, ...; a row's gradient replaces the student
+// row in the registers, leaves in one burst of stores, and the workgroup's next student row arrives in one burst of
+// loads, which the next scan lets land completely before it starts.  On 16384 x 151936 rows: 2.97 ms with a register
+// ring of four teacher vectors and the gradient stored / the next row loaded vector by vector behind the arithmetic,
+// 2.84 ms with the two bursts, 2.75 ms with the LDS slots (and 2.78 ms when the scan starts on the first vectors of
+// the arriving burst instead of waiting for all of it: memory rewards requests of one kind in long runs).  No
+// workgroup waits for another; the loop bound is the only exit condition.
 //
 // As in the register-resident actor step, the row shape (NVF full vector positions per thread, plus a partially
 // filled one when PARTIAL) is a template parameter so that every loop is straight-line code and the compiler can count
@@ -31,10 +37,9 @@
 namespace relax_amd {
 
 constexpr int kKlResThreads = 1024;
-// Teacher vectors in flight ahead of their use.  The slots freed by a pass's last positions take the next pass's first
-// vectors in rotated order, starting with vector NV % depth; the depth is chosen so that vector 0, needed first, is not
-// the one requested last (which would make the next pass wait for everything in flight).
-constexpr int kl_ring_depth(int nv) { return nv % 4 == 1 ? 5 : 4; }
+// Teacher vectors in flight ahead of their use, or kept for the second pass: slots of one 16-byte vector per thread in
+// LDS (128 KB of the CU's 160), filled by loads that go from global memory straight to LDS and cost no registers.
+constexpr int kKlSlots = 8;
 
 // absorb_pair() over the values of kKlUnroll raw vector pairs, without holding them all unpacked
 // marks a raw vector as changed without touching it: what is unpacked from it afterwards is a new value to the
@@ -49,15 +54,42 @@ __device__ __forceinline__ P* row_vec(P* row_base, uint32_t index) {
   return reinterpret_cast<P*>(reinterpret_cast<Byte*>(row_base) + index * uint32_t(sizeof(u32x4)));
 }
 
+// This thread's 16 bytes of an LDS slot once the request that fills them has arrived: vector-memory operations complete
+// in the order they were issued, so "at most VM still in flight" says it has, VM being the number of operations this
+// wave is known to have issued after it.  The wait and the read are one opaque statement because the compiler's own
+// bookkeeping of loads that land in LDS only knows "all of them": it would wait for every request in flight, the ones
+// issued a moment ago included, in front of every read.
+template <int VM>
+__device__ __forceinline__ u32x4 lds_read_when_at_most(uint32_t lds_byte_address) {
+  u32x4 r;
+  asm volatile("s_waitcnt vmcnt(%2)\n\tds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+               : "=v"(r)
+               : "v"(lds_byte_address), "n"(VM)
+               : "memory");
+  return r;
+}
+// the largest wait count <= in_flight_after that has an instantiation (in_flight_after folds to a constant where the
+// loops around the call are unrolled)
+template <int N>
+struct SlotRead {
+  static __device__ __forceinline__ u32x4 go(uint32_t a, int in_flight_after) {
+    return in_flight_after >= N ? lds_read_when_at_most<N>(a) : SlotRead<N - 1>::go(a, in_flight_after);
+  }
+};
+template <>
+struct SlotRead<0> {
+  static __device__ __forceinline__ u32x4 go(uint32_t a, int) { return lds_read_when_at_most<0>(a); }
+};
+
 template <typename T>
-__device__ __forceinline__ void absorb_raw_pairs(u32x4* s_raw, u32x4** t_raw, KlState& q) {
+__device__ __forceinline__ void absorb_raw_pairs(u32x4* s_raw, u32x4* t_raw, KlState& q) {
   constexpr int VN = Row<T>::kPerVec;
   float smax = 0.f, tmax = 0.f;
 #pragma unroll
   for (int u = 0; u < kKlUnroll; ++u) {
     float a[VN], b[VN];
     Row<T>::unpack(s_raw[u], a);
-    Row<T>::unpack(*t_raw[u], b);
+    Row<T>::unpack(t_raw[u], b);
 #pragma unroll
     for (int k = 0; k < VN; ++k) {
       smax = (u == 0 && k == 0) ? a[0] : fmaxf(smax, a[k]);
@@ -80,10 +112,10 @@ __device__ __forceinline__ void absorb_raw_pairs(u32x4* s_raw, u32x4** t_raw, Kl
     // unpack again: the values of the first walk kept alive (what common-subexpression elimination would do) do not
     // fit the register file next to the resident row
     launder(s_raw[u]);
-    launder(*t_raw[u]);
+    launder(t_raw[u]);
     // one 32-bit word of the vectors at a time, in element order
     const uint32_t sw[4] = {s_raw[u].x, s_raw[u].y, s_raw[u].z, s_raw[u].w};
-    const uint32_t tw[4] = {t_raw[u]->x, t_raw[u]->y, t_raw[u]->z, t_raw[u]->w};
+    const uint32_t tw[4] = {t_raw[u].x, t_raw[u].y, t_raw[u].z, t_raw[u].w};
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
       float a[VN], b[VN];
@@ -107,32 +139,67 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
     const T* __restrict__ student, const T* __restrict__ teacher, int64_t stride, int64_t vocab, int64_t n_rows,
     const float* __restrict__ g, float grad_scale, float* __restrict__ kl, float* __restrict__ lse_s,
     float* __restrict__ lse_t, T* __restrict__ dstudent) {
-  constexpr int THREADS = kKlResThreads, kU = kKlUnroll;
+  constexpr int THREADS = kKlResThreads, kU = kKlUnroll, S = kKlSlots;
   constexpr int VN = Row<T>::kPerVec;
   constexpr int NV = NVF + (PARTIAL ? 1 : 0);  // vector positions per thread
-  constexpr int D = kl_ring_depth(NV);
   constexpr int kGroups = (NV + kU - 1) / kU;
-  static_assert(kU == 2 && D >= kU && D <= NVF, "the teacher ring is refilled pair by pair");
+  static_assert(kU == 2 && NV > S && S % kU == 0, "the teacher slots are refilled pair by pair");
   __shared__ float lds[THREADS / kWave][5];
   __shared__ float bc[2];
+  // one object per slot: reads of one slot can then be told apart from the loads in flight into the others
+  __shared__ u32x4 slot0[THREADS], slot1[THREADS], slot2[THREADS], slot3[THREADS], slot4[THREADS], slot5[THREADS],
+      slot6[THREADS], slot7[THREADS];
   const int tid = threadIdx.x;
   const int rem = int(vocab / VN) - NVF * THREADS;  // lanes that hold a vector at the partial position (host-checked)
   u32x4 srow[NV];  // the student row
-  u32x4 ring[D];   // teacher vectors in flight
 
   // does this lane hold a vector at position j?  A compile-time answer except at the partial position.
   auto has = [&](int j) -> bool { return j < NVF || (PARTIAL && j == NVF && tid < rem); };
+  auto slot = [&](int k) -> u32x4* {
+    switch (k) {
+      case 0: return slot0;
+      case 1: return slot1;
+      case 2: return slot2;
+      case 3: return slot3;
+      case 4: return slot4;
+      case 5: return slot5;
+      case 6: return slot6;
+      default: return slot7;
+    }
+  };
+  // teacher vector j of the row at `base` -> slot j % S, this thread's 16 bytes of it; global memory to LDS without a
+  // register in between.  A lane without a vector at the partial position requests its first vector again (never
+  // used): the request is issued by every wave, which keeps the count of requests in flight the same for all.
+  auto request = [&](const u32x4* base, int j, uint32_t scale) {
+    int lane_id = tid;
+    asm volatile("" : "+v"(lane_id));  // recomputed per request: loop-invariant index registers would not fit
+    const uint32_t index = uint32_t(has(j) ? lane_id + j * THREADS : lane_id) * scale;
+    const int wave = __builtin_amdgcn_readfirstlane(lane_id / kWave);
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(row_vec(base, index)),
+                                     (__attribute__((address_space(3))) void*)(slot(j % S) + wave * kWave), 16, 0, 0);
+  };
+
+  // the slot of teacher vector j, valid once at most `in_flight_after` of this wave's later vector-memory operations
+  // are outstanding
+  auto teacher_vec = [&](int j, int in_flight_after) -> u32x4 {
+    int lane_id = tid;
+    asm volatile("" : "+v"(lane_id));
+    const uint32_t a = uint32_t(uintptr_t((__attribute__((address_space(3))) u32x4*)(slot(j % S) + lane_id)));
+    // the counts that occur: NV or more ahead of the scan's own requests, fewer than S behind them
+    return in_flight_after >= NV ? lds_read_when_at_most<NV>(a) : SlotRead<S - 1>::go(a, in_flight_after);
+  };
 
   int64_t row = blockIdx.x;
   if (row >= n_rows) return;
   {
-    const u32x4* sv = reinterpret_cast<const u32x4*>(student + row * stride);
-#pragma unroll
-    for (int j = 0; j < NV; ++j)
-      if (has(j)) srow[j] = load_stream(row_vec(sv, tid + j * THREADS));
+    // the first S teacher vectors, last first (as every later row finds them requested by its predecessor), then the
+    // student row
     const u32x4* tv0 = reinterpret_cast<const u32x4*>(teacher + row * stride);
 #pragma unroll
-    for (int j = 0; j < D; ++j) ring[j] = *row_vec(tv0, tid + j * THREADS);
+    for (int j = S - 1; j >= 0; --j) request(tv0, j, 1u);
+    const u32x4* sv = reinterpret_cast<const u32x4*>(student + row * stride);
+#pragma unroll
+    for (int j = 0; j < NV; ++j) srow[j] = load_stream(row_vec(sv, has(j) ? tid + j * THREADS : tid));
   }
 
   while (true) {
@@ -141,24 +208,32 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
     const float gt = g[row] * grad_scale;
     const u32x4* tv = reinterpret_cast<const u32x4*>(teacher + row * stride);
 
-    // a token without gradient (g == 0) gets a zero row; the second pass's teacher loads then all go to the row's
+    // a token without gradient (g == 0) gets a zero row; the second pass's teacher requests then all go to the row's
     // first vector, which costs nothing, so that the instruction stream -- and with it the wait counts -- stays the same
     const bool emit_zero = gt == 0.f;
-    const int tscale = emit_zero ? 0 : 1;
+    const uint32_t tscale = emit_zero ? 0u : 1u;
 
-    // ---- scan: both online softmaxes and sum e_s * (x_s - x_t).  The teacher row streams through the ring (ordinary
-    // loads: it is read again in a moment); its first D vectors are already on their way (requested during the previous
-    // row's gradient pass), and the slots freed by the last D positions take the first vectors of the second pass, which
-    // land during the merge.
+    // ---- scan: both online softmaxes and sum e_s * (x_s - x_t).  The teacher row streams through the S slots: its
+    // first S vectors are already on their way (requested during the previous row's gradient pass), a slot just read
+    // takes the vector S positions further on, and the pass ends with the row's last S vectors in LDS.
     KlState q{kNegHuge, 0.f, 0.f, kNegHuge, 0.f};
     bool grouped = true;
+    // The whole student row first (vmcnt = 0, the other counters left alone): a scan that starts on the first vectors
+    // of the arriving burst mixes its own teacher requests into it and measured slower (2.78 against 2.75 ms).
+    __builtin_amdgcn_s_waitcnt(0x0F70);
 #pragma unroll
     for (int gi = 0; gi < kGroups; ++gi) {
       const int j0 = kU * gi, j1 = kU * gi + 1;
       int lane_id = tid;
-      asm volatile("" : "+v"(lane_id));  // recomputed per group: loop-invariant index registers would not fit
+      asm volatile("" : "+v"(lane_id));
+      // Requests of this wave issued after the one that filled the slot of vector j, at the least: for the first S
+      // vectors (requested during the previous row's gradient pass, or ahead of the first row) the NV loads of the
+      // student row and this scan's own requests so far; for the others the scan's requests that followed theirs.
+      constexpr int kScanRequests = NV - S;
+      const int issued = kU * gi < kScanRequests ? kU * gi : kScanRequests;  // by the groups before this one
+      auto after = [&](int j) -> int { return j < S ? NV + issued : issued - (j - S) - 1; };
       if (grouped && j1 < NV && has(j1)) {
-        u32x4* tpair[kU] = {&ring[j0 % D], &ring[j1 % D]};
+        u32x4 tpair[kU] = {teacher_vec(j0, after(j1)), teacher_vec(j1, after(j1))};
         absorb_raw_pairs<T>(&srow[j0 < NV - 1 ? j0 : 0], tpair, q);
       } else {
         grouped = false;
@@ -168,21 +243,13 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
             float a[VN], b[VN];
             launder(srow[j0 + u < NV ? j0 + u : NV - 1]);
             Row<T>::unpack(srow[j0 + u < NV ? j0 + u : NV - 1], a);
-            Row<T>::unpack(ring[(j0 + u) % D], b);
+            Row<T>::unpack(teacher_vec(j0 + u, after(j0 + u)), b);
             absorb_pair(a, b, q);
           }
       }
-      // the ring slots just consumed take the vectors D positions further on, or the second pass's first ones
 #pragma unroll
-      for (int u = 0; u < kU; ++u) {
-        const int j = j0 + u;
-        if (j >= NV) continue;
-        if (j + D < NV) {
-          if (has(j + D)) ring[j % D] = *row_vec(tv, lane_id + (j + D) * THREADS);
-        } else {
-          ring[j % D] = load_stream(row_vec(tv, (lane_id + (j % D) * THREADS) * tscale));
-        }
-      }
+      for (int u = 0; u < kU; ++u)
+        if (j0 + u + S < NV) request(tv, j0 + u + S, 1u);
       asm volatile("" : "+v"(q.ss), "+v"(q.us), "+v"(q.st));  // keeps each group's work where it is written
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -221,21 +288,22 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
     __syncthreads();
     const float k0 = bc[0], k1 = bc[1];
 
-    // ---- gradient: d = p_s * g * ((x_s - x_t) + lse_t - lse_s - KL), the teacher row a second time (last use:
-    // non-temporal), written over the student row in place; the ring slots freed by the last D positions take the first
-    // teacher vectors of the next row.
-    u32x4* dv = reinterpret_cast<u32x4*>(dstudent + row * stride);
-    const u32x4* nsv = reinterpret_cast<const u32x4*>(student + (has_next ? next : row) * stride);
+    // ---- gradient: d = p_s * g * ((x_s - x_t) + lse_t - lse_s - KL), written over the student row in place, from the
+    // row's end to its beginning: the last S teacher vectors are still in LDS, each slot read takes the vector S
+    // positions further down (the teacher's second read: only NV - S of its NV vectors), and the slots of the first
+    // S positions take the first teacher vectors of the next row.
     const u32x4* ntv = reinterpret_cast<const u32x4*>(teacher + (has_next ? next : row) * stride);
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
+    for (int j = NV - 1; j >= 0; --j) {
       int lane_id = tid;
-      asm volatile("" : "+v"(lane_id));  // recomputed per vector: loop-invariant index registers would not fit
-      const int idx = lane_id + j * THREADS;
+      asm volatile("" : "+v"(lane_id));
       launder(srow[j]);
+      // the last S vectors have been in LDS since the scan; the others were requested S steps ago, S - 1 requests
+      // (one per step) followed theirs
+      const u32x4 tvec = teacher_vec(j, NV - 1 - j < S - 1 ? NV - 1 - j : S - 1);
       // one 32-bit word of the vector at a time: a whole vector of both rows unpacked does not fit
       const uint32_t sw[4] = {srow[j].x, srow[j].y, srow[j].z, srow[j].w};
-      const uint32_t tw[4] = {ring[j % D].x, ring[j % D].y, ring[j % D].z, ring[j % D].w};
+      const uint32_t tw[4] = {tvec.x, tvec.y, tvec.z, tvec.w};
       uint32_t ow[4] = {0u, 0u, 0u, 0u};
       if (!emit_zero) {  // the same answer in every lane of the workgroup: a jump, not a mask
 #pragma unroll
@@ -250,14 +318,15 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
         }
       }
       srow[j] = u32x4{ow[0], ow[1], ow[2], ow[3]};
-      if (j + D < NV) {
-        if (has(j + D)) ring[j % D] = load_stream(row_vec(tv, (idx + D * THREADS) * tscale));
-      } else {
-        ring[j % D] = *row_vec(ntv, lane_id + (j % D) * THREADS);  // the row itself again when there is no next one
-      }
+      if (j >= S)
+        request(tv, j - S, tscale);
+      else
+        request(ntv, j, 1u);  // the row itself again when there is no next one
       __builtin_amdgcn_sched_barrier(0);  // one vector at a time: hoisting the next one's unpacking spills
     }
     // ---- the gradient out in one burst, the next student row in in one burst
+    u32x4* dv = reinterpret_cast<u32x4*>(dstudent + row * stride);
+    const u32x4* nsv = reinterpret_cast<const u32x4*>(student + (has_next ? next : row) * stride);
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       int lane_id = tid;
