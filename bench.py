@@ -60,10 +60,10 @@ def measured_traffic(kernel: str, rows: int, vocab: int):
 
 
 def hbm_roofline(kernel: str, launch_ms: float, necessary_bytes: float, rows: int, vocab: int, kernel_ms: dict,
-                 ms_per_step: float, survey_bytes: float | None = None) -> dict:
+                 ms_per_step: float, two_pass_bytes: float | None = None) -> dict:
     """Roofline block of a bandwidth-bound launch.  ``achieved`` = the bytes the launch has to move (every input row
     it needs read once, every output row written once) / its HIP-event time; ``frac`` = achieved / 8 TB/s, a true
-    fraction.  ``survey_bytes`` (the forward-read + backward-read + write count of a two-pass implementation) is kept
+    fraction.  ``two_pass_bytes`` (the forward-read + backward-read + write count of a two-pass implementation) is kept
     beside it as ``two_pass_*``: a kernel that keeps the row on chip moves fewer bytes than that, so the figure can
     exceed the memory system's peak and is not a roofline fraction."""
     achieved = necessary_bytes / (launch_ms * 1e-3) / 1e9
@@ -74,9 +74,9 @@ def hbm_roofline(kernel: str, launch_ms: float, necessary_bytes: float, rows: in
            "traffic": traffic, "traffic_source": source, "algorithmic_bytes_per_launch": necessary_bytes,
            "avg_launch_ms": launch_ms, "kernel_ms": kernel_ms,
            "step_GBs": necessary_bytes / (ms_per_step * 1e-3) / 1e9}
-    if survey_bytes is not None:
-        out["two_pass_bytes_per_launch"] = survey_bytes
-        out["two_pass_GBs"] = survey_bytes / (launch_ms * 1e-3) / 1e9
+    if two_pass_bytes is not None:
+        out["two_pass_bytes_per_launch"] = two_pass_bytes
+        out["two_pass_GBs"] = two_pass_bytes / (launch_ms * 1e-3) / 1e9
     return out
 
 
@@ -342,7 +342,7 @@ def run_actor_step(a, dev) -> None:
          f"to dlogits",
          {"rows": n_tokens, "live_rows": live, "vocab": a.vocab, "loss": float(loss.item())},
          hbm_roofline(dom_name, dom, necessary, n_tokens, a.vocab, kernel_ms, ms_per_step,
-                      survey_bytes=3.0 * row_bytes * n_tokens if "actor_step_fused" in kernel_ms else None),
+                      two_pass_bytes=3.0 * row_bytes * n_tokens if "actor_step_fused" in kernel_ms else None),
          cpu_baseline(args, a.cpu_rows, a.vocab) if a.cpu_rows > 0 else None)
 
 
@@ -610,15 +610,15 @@ def run_reverse_kl(a, dev) -> None:
     if "reverse_kl_step_fused" in kernel_ms:
         # every token reports its KL, so both rows of every token are read once; one gradient row written per token
         dom, dom_name, necessary = kernel_ms["reverse_kl_step_fused"], kl_step_kernel_name(v), 3.0 * row_bytes * n
-        survey = 5.0 * row_bytes * n  # forward read of both rows, backward re-read of both, gradient write
+        two_pass = 5.0 * row_bytes * n  # forward read of both rows, backward re-read of both, gradient write
     else:
         dom, dom_name, necessary = kernel_ms["reverse_kl_bwd"], "reverse_kl_bwd_kernel<bf16_t, true>", 3.0 * row_bytes * n
-        survey = None
+        two_pass = None
     emit(a, n, wall,
          f"on-policy distillation: student/teacher bf16 logits [{n}, {v}], full-vocab reverse KL, token-mean, fwd + "
          f"student dlogits bwd",
          {"rows": n, "vocab": v, "loss": float(loss.item())},
-         hbm_roofline(dom_name, dom, necessary, n, v, kernel_ms, wall * 1e3 / a.steps, survey_bytes=survey),
+         hbm_roofline(dom_name, dom, necessary, n, v, kernel_ms, wall * 1e3 / a.steps, two_pass_bytes=two_pass),
          None)
 
 
@@ -698,7 +698,7 @@ def run_cfg1(a, dev) -> None:
          {"rows": n, "live_rows": live, "vocab": v, "loss": float(loss.item()), "logits_dtype": "f32",
           "advantages_ms": adv_ms},
          hbm_roofline(fused_step_kernel_name(v, "float"), dom, row_bytes * (live + n), n, v, kernel_ms,
-                      wall * 1e3 / a.steps, survey_bytes=3.0 * row_bytes * n),
+                      wall * 1e3 / a.steps, two_pass_bytes=3.0 * row_bytes * n),
          out_cpu)
 
 
@@ -772,7 +772,7 @@ def run_varlen(a, dev, loss_kind: str) -> None:
           "lengths": lengths},
          hbm_roofline(fused_step_kernel_name(v) if fused else name + "_kernel<bf16_t, true>", dom,
                       row_bytes * (read_rows + n), n, v, kernel_ms, wall * 1e3 / a.steps,
-                      survey_bytes=3.0 * row_bytes * n if fused else None),
+                      two_pass_bytes=3.0 * row_bytes * n if fused else None),
          None)
 
 
