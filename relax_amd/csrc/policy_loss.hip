@@ -89,14 +89,30 @@ __global__ __launch_bounds__(kLossThreads) void policy_loss_sample_kernel(relax_
   }
 }
 
-__global__ __launch_bounds__(kWave) void policy_loss_finish_kernel(const float* __restrict__ partials,
-                                                                   int64_t n_samples, float entropy_coef,
-                                                                   float kl_coef, int has_kl,
-                                                                   float* __restrict__ metrics) {
+// Sums the per-sample partial metrics in sample order (one lane per metric, each a plain sequence of fp32 additions,
+// so the result does not depend on how many samples a launch stages at a time).  The partials are staged through LDS
+// by the whole workgroup, 512 samples at a time: a lane adding straight from global memory waits out one memory
+// latency per sample (74 us for 512 samples).
+constexpr int kFinishThreads = 256;
+constexpr int kFinishStage = 512;  // samples per staging round (32 KB)
+
+__global__ __launch_bounds__(kFinishThreads) void policy_loss_finish_kernel(const float* __restrict__ partials,
+                                                                           int64_t n_samples, float entropy_coef,
+                                                                           float kl_coef, int has_kl,
+                                                                           float* __restrict__ metrics) {
+  __shared__ float stage[kFinishStage * RELAX_AMD_NUM_METRICS];
   const int k = threadIdx.x;
   float total = 0.f;
-  if (k < RELAX_AMD_NUM_METRICS)
-    for (int64_t i = 0; i < n_samples; ++i) total += partials[i * RELAX_AMD_NUM_METRICS + k];
+  for (int64_t base = 0; base < n_samples; base += kFinishStage) {
+    const int count = int(n_samples - base < kFinishStage ? n_samples - base : kFinishStage);
+    for (int e = k; e < count * RELAX_AMD_NUM_METRICS; e += kFinishThreads)
+      stage[e] = partials[base * RELAX_AMD_NUM_METRICS + e];
+    __syncthreads();
+    if (k < RELAX_AMD_NUM_METRICS)
+      for (int i = 0; i < count; ++i) total += stage[i * RELAX_AMD_NUM_METRICS + k];
+    __syncthreads();
+  }
+  if (k >= kWave) return;
   const float pg = __shfl(total, RELAX_AMD_M_PG_LOSS, kWave);
   const float ent = __shfl(total, RELAX_AMD_M_ENTROPY, kWave);
   const float kl = __shfl(total, RELAX_AMD_M_KL_LOSS, kWave);
@@ -213,7 +229,7 @@ extern "C" int relax_amd_policy_loss(const relax_amd_policy_loss_args* a, void* 
     int rc = check_launch("policy_loss_sample");
     if (rc) return rc;
   }
-  hipLaunchKernelGGL(policy_loss_finish_kernel, dim3(1), dim3(kWave), 0, s, a->sample_partials, a->n_samples,
+  hipLaunchKernelGGL(policy_loss_finish_kernel, dim3(1), dim3(kFinishThreads), 0, s, a->sample_partials, a->n_samples,
                      a->entropy_coef, a->kl_coef, int(a->kl_kind != RELAX_AMD_KL_NONE), a->metrics);
   return check_launch("policy_loss_finish");
 }
