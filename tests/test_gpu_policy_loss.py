@@ -817,6 +817,78 @@ def test_full_size_packed_varlen_gspo_and_cispo_properties():
     assert changed[inside & (flat_mask != 0)].float().mean().item() > 0.99
 
 
+def test_full_size_actor_step_with_topk_distillation_term():
+    """The headline shape (16 sequences x 4096 tokens, V = 151936, bf16, first 20 % of every sequence masked) with the
+    top-64 distillation term in the single launch: the same loss and metrics as the two-launch path; one whole
+    sequence's rows (4096) against the oracle's gradient for that sequence's share of the loss; for every row: masked
+    rows exactly zero, gradient rows summing to zero up to the rounding of 151936 bf16 terms."""
+    import relax_amd
+
+    dev = require_gpu()
+    seqs, seq_len, v, k = 16, 4096, 151936, 64
+    n = seqs * seq_len
+    announce("actor step + top-K distillation, full size", n, v, k)
+    g = torch.Generator(device=dev).manual_seed(3)
+    logits = torch.empty((1, n, v), dtype=torch.bfloat16, device=dev)
+    for s0 in range(0, n, 2048):
+        logits[0, s0:s0 + 2048] = (torch.randn((2048, v), device=dev, generator=g) * 3.0).bfloat16()
+    toks = [torch.randint(0, v, (seq_len,), device=dev, generator=g) for _ in range(seqs)]
+    mask = torch.ones(seq_len, device=dev)
+    mask[: seq_len // 5] = 0.0
+    kw = dict(eps_clip_high=0.28, use_kl_loss=True, kl_loss_coef=1e-3, kl_loss_type="k3", opd_loss_coef=0.5,
+              opd_token_selection="teacher_topk", opd_kl_type="reverse_kl", opd_norm_mode="tail")
+    args = P.make_args(**kw)
+    with torch.no_grad():
+        _, out = relax_amd.get_log_probs_and_entropy(logits, args=args, unconcat_tokens=toks,
+                                                     total_lengths=[seq_len] * seqs,
+                                                     response_lengths=[seq_len] * seqs, with_entropy=False)
+    old = [lp + 0.05 * torch.randn(lp.shape, device=dev, generator=g) for lp in out["log_probs"]]
+    ref = [lp + 0.05 * torch.randn(lp.shape, device=dev, generator=g) for lp in out["log_probs"]]
+    total_unmasked = float(mask.sum().item()) * seqs
+    batch = dict(
+        unconcat_tokens=toks, total_lengths=[seq_len] * seqs, response_lengths=[seq_len] * seqs,
+        loss_masks=[mask] * seqs, advantages=[torch.randn(seq_len, device=dev, generator=g) for _ in range(seqs)],
+        log_probs=old, ref_log_probs=ref,
+        relax_amd_sample_denominators=torch.full((seqs,), total_unmasked, device=dev),
+        opd_topk_token_ids=[torch.randint(0, v, (seq_len, k), device=dev, generator=g) for _ in range(seqs)],
+        opd_topk_teacher_log_probs=[torch.log_softmax(torch.randn(seq_len, k + 1, device=dev, generator=g), -1)[:, :k]
+                                    .contiguous() for _ in range(seqs)])
+    results = {}
+    for mode in ("auto", "off"):
+        lg = logits.detach().requires_grad_()
+        loss, met = relax_amd.policy_loss_function(P.make_args(relax_amd_single_pass=mode, **kw), batch, lg, None)
+        loss.backward()
+        results[mode] = (loss.detach(), met, lg.grad)
+        lg.grad = None
+        if mode == "auto":
+            d = results["auto"][2][0]
+            flat_mask = mask.repeat(seqs)
+            for s0 in range(0, n, 8192):
+                rows = d[s0:s0 + 8192]
+                assert rows.float().sum(-1).abs().max().item() < 5e-2
+                assert (rows[flat_mask[s0:s0 + 8192] == 0] == 0).all()
+            picked = 5
+            sub_rows = d[picked * seq_len:(picked + 1) * seq_len].float().cpu()
+            results["auto"] = (results["auto"][0], met, None)
+            del d, lg, loss
+            torch.cuda.empty_cache()
+    assert abs(results["auto"][0].item() - results["off"][0].item()) < 1e-5 * max(1.0, abs(results["off"][0].item()))
+    for key, w in results["off"][1].items():
+        assert abs(results["auto"][1][key].item() - w.item()) < 1e-5 * max(1.0, abs(w.item())), key
+    d_off = results["off"][2][0][picked * seq_len:(picked + 1) * seq_len].float().cpu()
+    torch.testing.assert_close(sub_rows, d_off, atol=2e-9, rtol=2.0 ** -6)
+    # the picked sequence against the oracle: its rows, its share of the token-mean loss
+    sub_logits = logits[0, picked * seq_len:(picked + 1) * seq_len].float().cpu().unsqueeze(0).requires_grad_()
+    sub = {key: [val[picked].cpu()] for key, val in batch.items()
+           if isinstance(val, list) and torch.is_tensor(val[0])}
+    sub.update(total_lengths=[seq_len], response_lengths=[seq_len])
+    # the term's token mean runs over the whole batch's unmasked tokens: the sequence's share has weight 1 / seqs
+    want, _ = P.policy_loss_function(P.make_args(**dict(kw, opd_loss_coef=kw["opd_loss_coef"] / seqs)), sub, sub_logits,
+                                     R.make_reducer([seq_len], sub["loss_masks"], sample_denoms=[total_unmasked]))
+    want.backward()
+    torch.testing.assert_close(sub_rows, sub_logits.grad[0], atol=3e-9, rtol=2.0 ** -6)
+
+
 def test_full_size_grpo_plumbing_case_rewards_to_dlogits():
     """The GRPO plumbing configuration at its stated size: 64 prompts x group 8 = 512 responses x 256 tokens, fp32
     logits [131072, 32000] ~ N(0, 2), Bernoulli(0.4) rewards, a trailing pad of 0..63 masked tokens per response,
