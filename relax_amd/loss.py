@@ -390,6 +390,8 @@ def _pack_topk_ids(flat, lay, gather_topk_token_ids):
     k_max = max(widths) if widths else 0
     if k_max == 0 or lay.n_tokens == 0:
         return None, widths
+    if all(w == k_max for w in widths):  # the usual case, every sample with the same K: one concatenation
+        return (per_sample[0] if len(per_sample) == 1 else torch.cat(per_sample, dim=0)).contiguous(), widths
     packed = torch.full((lay.n_tokens, k_max), -1, dtype=torch.long, device=dev)
     pos = 0
     for ids, r, w in zip(per_sample, lay.response_lengths, widths):
