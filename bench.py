@@ -94,6 +94,15 @@ def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
     return f"actor_step_fused_kernel<{dtype}, true, {threads}>"
 
 
+def bwd_kernel_name(vocab: int) -> str:
+    """Which kernel relax_amd_logprob_entropy_bwd runs for bf16 rows of ``vocab`` entries (the library's rule: the
+    persistent burst form for the row shapes of the register-resident step)."""
+    name = fused_step_kernel_name(vocab)
+    if name.startswith("actor_step_resident_kernel"):
+        return name.replace("actor_step_resident_kernel", "logprob_entropy_bwd_resident_kernel")
+    return "logprob_entropy_bwd_kernel<bf16_t, true>"
+
+
 def kl_step_kernel_name(vocab: int) -> str:
     """Which kernel relax_amd_reverse_kl_step_fused runs for bf16 rows of ``vocab`` entries (the library's rule)."""
     nvec = vocab // 8
@@ -335,7 +344,7 @@ def run_actor_step(a, dev) -> None:
         if a.opd_topk > 0:
             dom_name = dom_name[:-1] + ", true>"  # the instantiation that evaluates the top-K term
     else:  # two launches: the backward (read live rows, write all rows) dominates; the forward read is its own launch
-        dom, dom_name = kernel_ms["logprob_entropy_bwd"], "logprob_entropy_bwd_kernel<bf16_t, true>"
+        dom, dom_name = kernel_ms["logprob_entropy_bwd"], bwd_kernel_name(a.vocab)
     emit(a, n_tokens, wall,
          f"Qwen3-8B-shaped actor step: {a.seqs} seqs x {a.seq_len} tokens = {n_tokens} rows x V={a.vocab} bf16 "
          f"logits, PPO-clip 0.2/0.28 + k3 KL 1e-3{opd}, loss_function (scale 1/{args.global_batch_size}) fwd + bwd "
@@ -770,7 +779,7 @@ def run_varlen(a, dev, loss_kind: str) -> None:
          f"advantages, {loss_kind.upper()} loss, sequence-mean-token-sum, fwd + bwd to dlogits",
          {"rows": n, "live_rows": live, "rows_read_by_the_launch": read_rows, "vocab": v, "loss": float(loss.item()),
           "lengths": lengths},
-         hbm_roofline(fused_step_kernel_name(v) if fused else name + "_kernel<bf16_t, true>", dom,
+         hbm_roofline(fused_step_kernel_name(v) if fused else bwd_kernel_name(v), dom,
                       row_bytes * (read_rows + n), n, v, kernel_ms, wall * 1e3 / a.steps,
                       two_pass_bytes=3.0 * row_bytes * n if fused else None),
          None)

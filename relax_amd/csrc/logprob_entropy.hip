@@ -9,7 +9,11 @@
 //
 // Arithmetic follows relax/utils/training/ppo_utils.py:481-629 (reference paths are relative to its checkout):
 //   lp = x[tok] - lse,  H = lse - sum_v p*x,  dx = g_lp*(onehot - p) + g_H*p*(sum_v p*x - x),  x = logits / T.
+#include <cstdlib>
+#include <cstring>
+
 #include "device_utils.h"
+#include "logprob_bwd_resident.h"
 #include "relax_amd.h"
 #include "row_scan.h"
 
@@ -176,6 +180,24 @@ static int launch_bwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t
   dim3 grid(static_cast<unsigned>(n_rows)), block(kRowThreads);
   const T* x = static_cast<const T*>(logits);
   T* d = static_cast<T*>(dlogits);
+  // Long rows of the built shapes take the persistent burst form (same bits, faster).  RELAX_AMD_FUSED_STEP_KERNEL =
+  // "cached" keeps every row length on the row-per-workgroup kernel, "resident" fails where the burst form is not
+  // built (for tests that compare the two); read at every launch.
+  const char* forced = getenv("RELAX_AMD_FUSED_STEP_KERNEL");
+  if (vec && !(forced && strcmp(forced, "cached") == 0)) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    const int rc = launch_logprob_bwd_resident<T>(x, stride, vocab, n_rows, token_of_row, targets, lse, spx, g_lp,
+                                                  g_ent, grad_scale, grad_scale_dev, inv_t, d, d_stride, cus, s);
+    if (rc != RELAX_AMD_EUNSUPPORTED) return rc;  // launched (or failed to): otherwise the row length is not built
+  }
+  if (forced && strcmp(forced, "resident") == 0) {
+    set_error("logprob_entropy_bwd: RELAX_AMD_FUSED_STEP_KERNEL=resident, but no burst-form kernel is built for rows "
+              "of %lld elements of this type and alignment", (long long)vocab);
+    return RELAX_AMD_EUNSUPPORTED;
+  }
   if (vec)
     hipLaunchKernelGGL((logprob_entropy_bwd_kernel<T, true>), grid, block, 0, s, x, stride, vocab, token_of_row,
                        targets, lse, spx, g_lp, g_ent, grad_scale, grad_scale_dev, c, inv_t, d, d_stride);

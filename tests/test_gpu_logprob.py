@@ -237,6 +237,53 @@ def test_full_size_properties_headline_shape():
     torch.testing.assert_close(ent[idx].cpu(), rent, atol=2e-3, rtol=0)
 
 
+@pytest.mark.parametrize("v,dtype,n", [(151936, torch.bfloat16, 700), (8 * (18 * 1024 + 1), torch.bfloat16, 300),
+                                       (128256, torch.float16, 600), (131072, torch.bfloat16, 40),
+                                       (100352, torch.bfloat16, 1100), (8 * (16 * 1024 - 1), torch.float16, 300),
+                                       (32000, torch.float32, 1500), (4 * (16 * 512 - 1), torch.float32, 700)])
+def test_backward_burst_form_equals_row_per_workgroup_kernel_bitwise(v, dtype, n, monkeypatch):
+    """The two kernels behind relax_amd_logprob_entropy_bwd, switched with RELAX_AMD_FUSED_STEP_KERNEL, on every row
+    shape the persistent burst form is built for (and the ends of two of them), with rows that score no token, tokens
+    without gradient (zero rows, in runs and scattered), a device-side gradient scale and targets on a row's first and
+    last element: bit-identical gradients."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("backward: burst form vs row-per-workgroup", v, dtype, n)
+    g = torch.Generator().manual_seed(v + n)
+    x = (torch.randn(n, v, generator=g) * 2).to(dtype).to(dev)
+    scores = torch.rand(n, generator=g) > 0.2
+    idx = torch.cumsum(scores.int(), 0) - 1
+    token_of_row = torch.where(scores, idx, torch.full_like(idx, -1)).int().to(dev)
+    row_ids = torch.nonzero(scores).flatten().int().to(dev)
+    n_tok = int(scores.sum())
+    tok = torch.randint(0, v, (n_tok,), generator=g)
+    tok[:3] = torch.tensor([0, v - 1, v - 2])
+    tok = tok.to(dev)
+    lp, ent, lse, spx = ops.logprob_entropy_fwd(x, tok, row_ids, 0.8, True)
+    glp = torch.randn(n_tok, generator=g)
+    gen = torch.randn(n_tok, generator=g) * 0.1
+    dead = torch.rand(n_tok, generator=g) < 0.25
+    dead[n_tok // 2:n_tok // 2 + 12] = True
+    glp[dead] = 0.0
+    gen[dead] = 0.0
+    scale = torch.tensor([0.37], device=dev)
+    outs = {}
+    for kind in ("cached", "resident"):
+        monkeypatch.setenv("RELAX_AMD_FUSED_STEP_KERNEL", kind)
+        for with_ent in (True, False):
+            d = ops.logprob_entropy_bwd(x, tok, lse, spx, glp.to(dev), gen.to(dev) if with_ent else None,
+                                        token_of_row=token_of_row, grad_scale_dev=scale, inv_temperature=0.8)
+            torch.cuda.synchronize()
+            outs[kind, with_ent] = d.view(torch.int16 if dtype != torch.float32 else torch.int32)
+    for with_ent in (True, False):
+        assert torch.equal(outs["resident", with_ent], outs["cached", with_ent]), with_ent
+        assert outs["resident", with_ent].any()
+    zero_rows = torch.ones(n, dtype=torch.bool)
+    zero_rows[row_ids.cpu().long()[~dead]] = False
+    assert not outs["resident", True][zero_rows.to(dev)].any()
+
+
 # ------------------------------------------------------------------------------------------------- top-K selection
 
 
