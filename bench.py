@@ -83,7 +83,7 @@ def hbm_roofline(kernel: str, launch_ms: float, necessary_bytes: float, rows: in
 def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
     """Which kernel relax_amd_actor_step_fused runs for bf16 / fp32 rows of ``vocab`` entries (the library's own rule:
     the register-resident kernel in workgroups as wide as the forward-only scan's, where the row shape is built)."""
-    per_vec, width, shapes = {"bf16_t": (8, 1024, ((18, True), (15, True), (16, False), (12, True))),
+    per_vec, width, shapes = {"bf16_t": (8, 1024, ((20, False), (19, True), (18, True), (15, True), (16, False), (12, True))),
                               "float": (4, 512, ((15, True),))}[dtype]
     nvec = vocab // per_vec
     threads = 1024 if nvec >= 8192 else 512 if nvec >= 2048 else 256
@@ -107,7 +107,7 @@ def kl_step_kernel_name(vocab: int) -> str:
     """Which kernel relax_amd_reverse_kl_step_fused runs for bf16 rows of ``vocab`` entries (the library's rule)."""
     nvec = vocab // 8
     shape = (nvec // 1024, nvec % 1024 != 0)
-    if vocab % 8 == 0 and shape in ((18, True), (15, True), (16, False), (12, True)) \
+    if vocab % 8 == 0 and shape in ((20, False), (19, True), (18, True), (15, True), (16, False), (12, True)) \
             and os.environ.get("RELAX_AMD_FUSED_STEP_KERNEL") != "cached":
         return f"reverse_kl_resident_kernel<bf16_t, {shape[0]}, {str(shape[1]).lower()}>"
     return f"reverse_kl_step_kernel<bf16_t, true, {1024 if nvec >= 2048 else 256}>"

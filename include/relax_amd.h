@@ -301,8 +301,8 @@ int relax_amd_reverse_kl_bwd(const void* student, const void* teacher, int dtype
  * g[t] = mask[t] / clamp_min(sum mask, 1).  Same outputs as relax_amd_reverse_kl_fwd followed by
  * relax_amd_reverse_kl_bwd (dstudent row stride = row_stride); each workgroup re-reads its two rows out of cache, so
  * HBM moves 3*V*s bytes per token instead of 5*V*s.  Two kernels sit behind it, with bit-identical results: 16-bit
- * rows of the built vocabulary shapes (12 / 15 / 18 full 16-byte vectors per thread of a 1024-thread workgroup plus
- * a partial one, or 16 exactly) keep the student row in registers and stream the teacher row past it twice; other
+ * rows of the built vocabulary shapes (12 / 15 / 18 / 19 full 16-byte vectors per thread of a 1024-thread workgroup
+ * plus a partial one, or 16 / 20 exactly) keep the student row in registers and stream the teacher row past it twice; other
  * rows, and every row when RELAX_AMD_FUSED_STEP_KERNEL=cached is in the environment, walk both rows twice.
  */
 int relax_amd_reverse_kl_step_fused(const void* student, const void* teacher, int dtype, int64_t n_tokens,
@@ -427,7 +427,7 @@ int relax_amd_logprob_entropy_topk_fwd(const void* logits, int dtype, int64_t n_
  * With loss->topk_ids set the step also evaluates the top-K distillation signal of every row it reads (see the
  * argument block); the caller adds the K one-hot parts of its gradient with relax_amd_sparse_row_add afterwards.
  * Two kernels sit behind this entry point and are chosen by row length and element type: a register-resident one
- * (one read and one write of HBM per row; 16-bit rows of 100352 .. 152064 entries and fp32 rows of 32000 entries in
+ * (one read and one write of HBM per row; 16-bit rows of 100352 .. 163840 entries and fp32 rows of 32000 entries in
  * the built shapes) and a two-walk one for everything else; RELAX_AMD_FUSED_STEP_KERNEL=cached in the environment
  * forces the latter.  Same results.
  */

@@ -348,8 +348,11 @@ int launch_actor_step_resident(const T* logits, int64_t row_stride, int64_t voca
   const int64_t slots = int64_t(compute_units) * (1024 / THREADS);  // persistent workgroups: as many as fit the chip
   const dim3 grid(static_cast<unsigned>(n_rows < slots ? n_rows : slots)), block(THREADS);
   if constexpr (sizeof(T) == 2) {
-    // vocabularies of 151936 / 152064 (18992 / 19008 vectors), 128256 / 129280 (16032 / 16160), 131072 (16384),
+    // vocabularies of 163840 (20480 vectors) and up to it, 151936 / 152064 (18992 / 19008), 128256 / 129280
+    // (16032 / 16160), 131072 (16384),
     // 100352 / 102400 (12544 / 12800) entries
+    RELAX_AMD_RESIDENT(20, false)
+    RELAX_AMD_RESIDENT(19, true)
     RELAX_AMD_RESIDENT(18, true)
     RELAX_AMD_RESIDENT(15, true)
     RELAX_AMD_RESIDENT(16, false)

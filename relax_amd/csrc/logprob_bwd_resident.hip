@@ -170,7 +170,9 @@ int launch_logprob_bwd_resident(const T* logits, int64_t row_stride, int64_t voc
   const int64_t slots = int64_t(compute_units) * (1024 / THREADS);  // persistent workgroups: as many as fit the chip
   const dim3 grid(static_cast<unsigned>(n_rows < slots ? n_rows : slots)), block(THREADS);
   if constexpr (sizeof(T) == 2) {
-    // vocabularies of 151936 / 152064, 128256 / 129280, 131072, 100352 / 102400 entries
+    // vocabularies of 163840 and up to it, 151936 / 152064, 128256 / 129280, 131072, 100352 / 102400 entries
+    RELAX_AMD_BWD_RESIDENT(20, false)
+    RELAX_AMD_BWD_RESIDENT(19, true)
     RELAX_AMD_BWD_RESIDENT(18, true)
     RELAX_AMD_BWD_RESIDENT(15, true)
     RELAX_AMD_BWD_RESIDENT(16, false)

@@ -380,8 +380,11 @@ int launch_reverse_kl_resident(const T* student, const T* teacher, int64_t strid
                        stride, vocab, n_rows, g, grad_scale, kl, lse_s, lse_t, dstudent);                            \
     return check_launch("reverse_kl_resident");                                                                      \
   }
-    // vocabularies of 151936 / 152064 (18992 / 19008 vectors), 128256 / 129280 (16032 / 16160), 131072 (16384),
+    // vocabularies of 163840 (20480 vectors) and up to it, 151936 / 152064 (18992 / 19008), 128256 / 129280
+    // (16032 / 16160), 131072 (16384),
     // 100352 / 102400 (12544 / 12800) entries
+    RELAX_AMD_KL_RESIDENT(20, false)
+    RELAX_AMD_KL_RESIDENT(19, true)
     RELAX_AMD_KL_RESIDENT(18, true)
     RELAX_AMD_KL_RESIDENT(15, true)
     RELAX_AMD_KL_RESIDENT(16, false)

@@ -230,7 +230,8 @@ def test_fused_opd_loss_matches_oracle_and_two_launch_path(n, v, dtype, tol):
 
 @pytest.mark.parametrize("v,dtype,n", [(151936, torch.bfloat16, 700), (152064, torch.float16, 300),
                                        (128256, torch.bfloat16, 520), (131072, torch.float16, 515),
-                                       (100352, torch.bfloat16, 1030), (102400, torch.bfloat16, 40)])
+                                       (100352, torch.bfloat16, 1030), (102400, torch.bfloat16, 40),
+                                       (163840, torch.bfloat16, 300), (8 * (19 * 1024 + 3), torch.float16, 530)])
 def test_register_resident_reverse_kl_step_equals_two_walk_kernel_bitwise(v, dtype, n, monkeypatch):
     """The two kernels behind relax_amd_reverse_kl_step_fused, switched with RELAX_AMD_FUSED_STEP_KERNEL, for every
     row shape the register-resident one is built for (partial and full last vector positions), with more rows than

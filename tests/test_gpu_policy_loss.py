@@ -1663,11 +1663,12 @@ def test_custom_loss_function_path_dispatch():
 
 @pytest.mark.parametrize("v,dtype,n_samples", [(100352, torch.bfloat16, 18), (128256, torch.float16, 18),
                                                 (131072, torch.bfloat16, 18), (151936, torch.bfloat16, 18),
+                                                (163840, torch.bfloat16, 18), (160000, torch.float16, 18),
                                                 (65536, torch.bfloat16, 18), (32000, torch.float32, 40)])
 def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples):
     """More logits rows than persistent workgroups, so every workgroup of the register-resident kernel rolls several
     rows through its registers (prompt rows, fully masked samples and masked tokens in between), for every row shape
-    the kernel is built for (12 / 15 / 18 full vectors per thread plus a partial one, 16 exactly; fp32 rows of 32000
+    the kernel is built for (12 / 15 / 18 / 19 full vectors per thread plus a partial one, 16 or 20 exactly; fp32 rows of 32000
     entries in 512-thread workgroups, two per CU) and one it is not (65536: two-walk kernel): same loss bits as the two-launch path, gradients equal to it and to the oracle."""
     import relax_amd
 
@@ -1762,6 +1763,7 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
 
 
 @pytest.mark.parametrize("v,dtype", [(8 * (18 * 1024 + 1), torch.bfloat16), (8 * (19 * 1024 - 1), torch.bfloat16),
+                                     (8 * (19 * 1024 + 1), torch.bfloat16), (8 * 20 * 1024, torch.float16),
                                      (8 * (12 * 1024 + 1), torch.float16), (8 * (16 * 1024 - 1), torch.bfloat16),
                                      (4 * (15 * 512 + 1), torch.float32), (4 * (16 * 512 - 1), torch.float32)])
 def test_register_resident_kernel_at_the_edges_of_its_row_shapes(v, dtype, monkeypatch):
