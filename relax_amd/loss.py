@@ -882,7 +882,10 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         assert "rollout_log_probs" in batch, "rollout_log_probs must be provided for TIS"
     rollout = _cat_f32(batch.get("rollout_log_probs"), dev)
     # train-engine log-probs: batch["log_probs"], or this step's own forward (kernel default) in true on-policy mode
-    train = None if (true_on_policy or not batch.get("log_probs")) else _cat_f32(batch["log_probs"], dev)
+    if true_on_policy or not batch.get("log_probs"):
+        train = None
+    else:  # the same packed vector as `old` unless that one holds the rollout engine's log-probs
+        train = old if (old is not None and not use_rollout) else _cat_f32(batch["log_probs"], dev)
     # which log-probs the |train - rollout| metrics compare (loss.py:1125-1130): 1 = old, 0 = train, 2 = current
     if not use_rollout:
         abs_from = 2 if true_on_policy else 1
