@@ -661,6 +661,25 @@ def _cat_f32(parts, device):
     return torch.cat([p.to(device=device).reshape(-1) for p in parts]).to(torch.float32)
 
 
+def _cat_fields_f32(device, n_tokens: int, **fields):
+    """Several per-sample lists -> packed fp32 vectors, ``{name: [N] tensor | None}``.  When every list holds 1-D fp32
+    tensors on ``device`` that add up to ``n_tokens`` elements, all of them are packed by ONE concatenation and the
+    results are views of its output (a batch arrives as a handful of such lists, and each concatenation is a launch of
+    its own that costs more than it moves); anything else falls back to one ``_cat_f32`` per field."""
+    live = {k: v for k, v in fields.items() if v is not None}
+    simple = len(live) > 1 and all(
+        isinstance(v, (list, tuple)) and len(v) > 0 and all(
+            torch.is_tensor(t) and t.dim() == 1 and t.dtype == torch.float32 and t.device == device for t in v)
+        and sum(int(t.numel()) for t in v) == n_tokens for v in live.values())
+    if not simple:
+        return {k: _cat_f32(v, device) for k, v in fields.items()}
+    packed = torch.cat([t for v in live.values() for t in v])
+    out = {k: None for k in fields}
+    for i, k in enumerate(live):
+        out[k] = packed[i * n_tokens:(i + 1) * n_tokens]
+    return out
+
+
 def load_function(path: str):
     """``"pkg.module.fn"`` -> the function object (relax/utils/misc.py:30-38)."""
     import importlib
@@ -876,11 +895,18 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
 
     true_on_policy = getattr(args, "true_on_policy_mode", False)
     use_rollout = getattr(args, "use_rollout_logprobs", False)
-    old = None if true_on_policy else _cat_f32(batch["rollout_log_probs"] if use_rollout else batch["log_probs"], dev)
+    use_kl = bool(getattr(args, "use_kl_loss", False))
     mismatch = bool(getattr(args, "get_mismatch_metrics", False) or getattr(args, "use_tis", False))
     if mismatch:
         assert "rollout_log_probs" in batch, "rollout_log_probs must be provided for TIS"
-    rollout = _cat_f32(batch.get("rollout_log_probs"), dev)
+    # the batch's per-sample lists, packed (one concatenation for all of them where their form allows)
+    cat = _cat_fields_f32(
+        dev, lay.n_tokens,
+        old=None if true_on_policy else (batch["rollout_log_probs"] if use_rollout else batch["log_probs"]),
+        rollout=batch.get("rollout_log_probs") if not (use_rollout and not true_on_policy) else None,
+        ref=batch["ref_log_probs"] if use_kl else None, advantages=batch["advantages"], masks=batch["loss_masks"])
+    old = cat["old"]
+    rollout = cat["rollout"] if not (use_rollout and not true_on_policy) else old
     # train-engine log-probs: batch["log_probs"], or this step's own forward (kernel default) in true on-policy mode
     if true_on_policy or not batch.get("log_probs"):
         train = None
@@ -891,19 +917,18 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         abs_from = 2 if true_on_policy else 1
     else:
         abs_from = 0 if train is not None else 2
-    masks = _cat_f32(batch["loss_masks"], dev)
+    masks = cat["masks"]
     per_token = bool(getattr(args, "calculate_per_token_loss", False))
     denom = batch.get("relax_amd_sample_denominators")
     if denom is None and not per_token:
         denom = sample_denominators(batch["loss_masks"], lay, batch.get("sample_index_mask_sums"))
     pg_denom = hook_pg_denom if hook_pg_denom is not None else batch.get("relax_amd_pg_sample_denominators")
-    use_kl = bool(getattr(args, "use_kl_loss", False))
     kw = dict(
         old_log_prob=old,
-        ref_log_prob=_cat_f32(batch["ref_log_probs"], dev) if use_kl else None,
+        ref_log_prob=cat["ref"],
         train_log_prob=train,
         rollout_log_prob=rollout,
-        advantages=_cat_f32(batch["advantages"], dev),
+        advantages=cat["advantages"],
         loss_mask=masks,
         sample_denom=None if denom is None else denom.to(device=dev, dtype=torch.float32),
         pg_sample_denom=None if pg_denom is None else pg_denom.to(device=dev, dtype=torch.float32),
