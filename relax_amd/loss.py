@@ -1220,7 +1220,15 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
     if is_dummy:
         loss = 0.0 * loss
     elif not per_token:
-        loss = loss * explicit if explicit is not None else loss * num_microbatches / gbs * dp_world_size
+        if explicit is not None:
+            loss = loss * explicit
+        elif all(isinstance(x, (int, float)) for x in (num_microbatches, gbs, dp_world_size)):
+            # loss.py:1567 multiplies and divides step by step; with plain numbers the factor is formed on the host and
+            # applied once (one launch forward, one backward, instead of three each; the value may differ from the
+            # step-by-step one in the last bit)
+            loss = loss * (num_microbatches / gbs * dp_world_size)
+        else:
+            loss = loss * num_microbatches / gbs * dp_world_size
     effective = torch.zeros_like(num_tokens) if is_dummy else num_tokens
     denominator = effective if per_token else torch.zeros_like(num_tokens)
     values = torch.stack([denominator.to(torch.float32)] + [v.to(torch.float32) for v in log.values()])
