@@ -1172,7 +1172,12 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
     loss_type = getattr(args, "loss_type", "policy_loss")
     if loss_type not in ("policy_loss", "value_loss", "sft", "custom_loss"):
         raise ValueError(f"Unknown loss type: {loss_type}")
-    num_tokens = get_cp_local_num_tokens(batch["total_lengths"], batch["response_lengths"], batch["loss_masks"])
+    per_token = bool(getattr(args, "calculate_per_token_loss", False))
+    # the micro-batch's token count (loss.py:1504) is what per-token mode returns as its normalizer; in sample-mean
+    # mode nothing reads it, and its five small launches are left out
+    num_tokens = None
+    if per_token:
+        num_tokens = get_cp_local_num_tokens(batch["total_lengths"], batch["response_lengths"], batch["loss_masks"])
     reducer = None
     if getattr(args, "mtp_only_training", False):
         func = mtp_only_loss_function
@@ -1207,7 +1212,6 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
                                use_reentrant=getattr(args, "recompute_loss_function_use_reentrant", True))
     else:
         loss, log = func(args, batch, logits, reducer)
-    per_token = bool(getattr(args, "calculate_per_token_loss", False))
     if per_token and getattr(args, "advantage_estimator", None) == "m2po":
         # the M2PO scalars are global, not per-token sums: pre-multiplied so that the logger's division by the token
         # count gives them back (loss.py:1547-1552)
@@ -1229,9 +1233,13 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
             loss = loss * (num_microbatches / gbs * dp_world_size)
         else:
             loss = loss * num_microbatches / gbs * dp_world_size
-    effective = torch.zeros_like(num_tokens) if is_dummy else num_tokens
-    denominator = effective if per_token else torch.zeros_like(num_tokens)
-    values = torch.stack([denominator.to(torch.float32)] + [v.to(torch.float32) for v in log.values()])
+    zero_count = torch.zeros((), dtype=torch.float32, device=logits.device)
+    if per_token:
+        effective = torch.zeros_like(num_tokens) if is_dummy else num_tokens
+        denominator = effective.to(torch.float32)
+    else:
+        denominator = zero_count
+    values = torch.stack([denominator] + [v.to(torch.float32) for v in log.values()])
     if is_dummy:
         values = torch.zeros_like(values)
     normalizer = effective if per_token else torch.ones((), dtype=torch.int64, device=logits.device)  # no host copy
