@@ -537,10 +537,13 @@ class _SinglePassPolicyLoss(torch.autograd.Function):
         ctx.dlogits = dlogits
         ctx.assumed_scale = float(assumed_scale)
         ctx.mark_non_differentiable(metrics, lp, ent, topk_kl)
+        ctx.set_materialize_grads(False)  # no zero tensors for the outputs nothing differentiates (three fills a step)
         return metrics[_SLOT["loss"]].clone(), metrics, lp, ent, topk_kl
 
     @staticmethod
     def backward(ctx, g_loss, _gm, _glp, _gent, _gkl):
+        if g_loss is None:  # the loss itself took no part in what was differentiated
+            return None, None, None, None, None
         d = ctx.dlogits
         if d is None:
             raise RuntimeError("the single-pass policy loss holds its gradient once: backward cannot run twice")
