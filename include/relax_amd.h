@@ -373,7 +373,8 @@ int relax_amd_opd_kl_topk_bwd(const float* student_lp, const float* teacher_lp, 
  * target_values[t] * scale: the sparse part of the gradient of gathered log-probs (the scatter of
  * compute_log_probs_on_topk_token_ids' backward, relax/utils/opd/opd_utils.py:1022-1094) when its dense part, a
  * multiple of the row's softmax, has been folded into the dlogits launch of the log-prob backward.  Ids outside
- * [0, vocab) and zero values are skipped; targets / target_values may be NULL; row_ids NULL = row t.
+ * [0, vocab), zero values and tokens with a negative row id are skipped; targets / target_values may be NULL;
+ * row_ids NULL = row t.
  */
 int relax_amd_sparse_row_add(void* dlogits, int dtype, int64_t n_tokens, int64_t vocab, int64_t row_stride,
                              const int32_t* row_ids, const int64_t* ids, const float* values, int64_t k,

@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256) void opd_kl_topk_kernel(const float* __restric
 // dlogits[row(t), id] += value * scale for the K (id, value) pairs of token t plus one pair at its target id: the
 // sparse part of a gradient whose dense part (a multiple of the row's softmax) another kernel has already written.
 // One thread walks all pairs of a token one after the other, so two pairs on the same element (a gathered id that
-// equals the target) cannot race; ids outside [0, vocab) are skipped.  (The form for very long lists; the usual ones
+// equals the target) cannot race; ids outside [0, vocab) and tokens whose row id is negative are skipped.  (The form for very long lists; the usual ones
 // take sparse_row_add_wave_kernel below.)
 template <typename T>
 __global__ __launch_bounds__(256) void sparse_row_add_kernel(T* __restrict__ dlogits, int64_t stride, int64_t vocab,
@@ -157,7 +157,9 @@ __global__ __launch_bounds__(256) void sparse_row_add_kernel(T* __restrict__ dlo
                                                              int64_t n_tokens) {
   const int64_t tok = blockIdx.x * 256LL + threadIdx.x;
   if (tok >= n_tokens) return;
-  T* d = dlogits + (row_ids ? int64_t(row_ids[tok]) : tok) * stride;
+  const int64_t row = row_ids ? int64_t(row_ids[tok]) : tok;
+  if (row < 0) return;  // a token without a row
+  T* d = dlogits + row * stride;
   for (int j = 0; j < k; ++j) {
     const int64_t id = ids[tok * k + j];
     const float v = values[tok * k + j];
@@ -188,6 +190,8 @@ __global__ __launch_bounds__(256) void sparse_row_add_wave_kernel(T* __restrict_
   const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
   const int64_t tok = blockIdx.x * 4LL + w;
   if (tok >= n_tokens) return;
+  const int64_t row = row_ids ? int64_t(row_ids[tok]) : tok;
+  if (row < 0) return;  // a token without a row (uniform over the wave)
   const int n = k + (targets ? 1 : 0);
   int64_t* sid = sparse_stage + w * (k + 1);
   float* sval = reinterpret_cast<float*>(sparse_stage + 4 * (k + 1)) + w * (k + 1);
@@ -201,7 +205,7 @@ __global__ __launch_bounds__(256) void sparse_row_add_wave_kernel(T* __restrict_
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  T* d = dlogits + (row_ids ? int64_t(row_ids[tok]) : tok) * stride;
+  T* d = dlogits + row * stride;
   for (int j = lane; j < n; j += kWave) {
     const int64_t id = sid[j];
     if (id < 0) continue;
@@ -226,7 +230,8 @@ extern "C" int relax_amd_sparse_row_add(void* dlogits, int dtype, int64_t n_toke
                                         const int64_t* targets, const float* target_values, float scale,
                                         void* stream) {
   if (n_tokens == 0) return RELAX_AMD_OK;
-  if (n_tokens < 0 || vocab <= 0 || row_stride < vocab || k < 0 || k > (1 << 20) || !dlogits ||
+  if (n_tokens < 0 || n_tokens > 2147483647LL || vocab <= 0 || row_stride < vocab || k < 0 || k > (1 << 20) ||
+      !dlogits ||
       (k > 0 && (!ids || !values)) || (targets && !target_values)) {
     set_error("sparse_row_add: NULL argument or bad shape n=%lld vocab=%lld row_stride=%lld k=%lld",
               (long long)n_tokens, (long long)vocab, (long long)row_stride, (long long)k);
