@@ -94,7 +94,11 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
   }
   // the first wave's gathers for the top-K distillation signal, when configured, likewise
   TopkGather gathered{};
-  if (a.topk_ids && tid < kWave) gathered = topk_gather<T>(a, x, vocab, tok, tid);
+  TopkRowShape topk_shape{};
+  if (a.topk_ids && tid < kWave) {
+    gathered = topk_gather<T>(a, x, vocab, tok, tid);
+    topk_shape = topk_row_shape(a, tok);
+  }
   // pass 1: cached loads, the row stays in L2 / the memory-side cache for pass 2
   SoftmaxAcc st = scan_row<T, VEC, false, THREADS>(x, vocab, c);
   scan_block_merge<THREADS>(st, wave_state);
@@ -110,9 +114,9 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
     // the top-K distillation signal, when configured: K gathered logits of this row against the log-sum-exp just found
     float g_topk = 0.f;
     if (a.topk_ids) {
-      const float lp0 = __shfl(lp, 0, kWave);
-      g_topk = topk_distill_row(a, gathered, tok, __shfl(lse, 0, kWave), inv_t, lp0,
-                                __shfl(in.has_old ? in.old_lp : lp, 0, kWave), __shfl(in.extra_lp, 0, kWave), tid,
+      const float lp0 = lane_value(lp);
+      g_topk = topk_distill_row(a, gathered, topk_shape, tok, lane_value(lse), inv_t, lp0,
+                                lane_value(in.has_old ? in.old_lp : lp), lane_value(in.extra_lp), tid,
                                 topk_stage);
     }
     if (tid == 0) {

@@ -210,14 +210,14 @@ __global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_
     // here, behind the merge of the waves' partial states, costs less than carrying them through the scan in
     // registers that every wave would have to set aside.
     const ResidentTokenData td = fetch_token(row, tok);
-    // likewise the first wave's gathers for the top-K distillation signal: two dependent requests (ids, then the
-    // row's logits there) that need nothing of the scan's result
     TopkGather gathered{};
+    TopkRowShape topk_shape{};
     if constexpr (TOPK) {
       if (wave0) {
         int lane = tid;
         asm volatile("" : "+v"(lane));
         gathered = topk_gather<T>(a, logits + row * row_stride, vocab, tok, lane);
+        topk_shape = topk_row_shape(a, tok);
       }
     }
     scan_block_merge<THREADS>(st, wave_state);
@@ -235,9 +235,9 @@ __global__ __launch_bounds__(resident_threads<T>(), 4) void actor_step_resident_
       if constexpr (TOPK) {
         int lane = tid;
         asm volatile("" : "+v"(lane));
-        g_topk = topk_distill_row(a, gathered, tok, __shfl(lse, 0, kWave), inv_t, __shfl(lp, 0, kWave),
-                                  __shfl(td.in.has_old ? td.in.old_lp : lp, 0, kWave),
-                                  __shfl(td.in.extra_lp, 0, kWave), lane, topk_stage);
+        g_topk = topk_distill_row(a, gathered, topk_shape, tok, lane_value(lse), inv_t, lane_value(lp),
+                                  lane_value(td.in.has_old ? td.in.old_lp : lp), lane_value(td.in.extra_lp), lane,
+                                  topk_stage);
       }
       if (tid == 0) {
         relax_amd_policy_loss_args al = a;

@@ -131,19 +131,81 @@ struct Row<f16_t> {
 __device__ __forceinline__ u32x4 load_stream(const u32x4* p) { return __builtin_nontemporal_load(p); }
 __device__ __forceinline__ void store_stream(u32x4* p, const u32x4& v) { __builtin_nontemporal_store(v, p); }
 
+// Value that lane (this lane ^ O) of the wave holds, O a power of two below 64: the exchange of __shfl_xor() done by
+// cross-lane moves inside the vector ALU (quad permutes, row rotates / mirrors, the 16- and 32-lane swaps) instead
+// of a trip through the LDS crossbar, which a wave with nothing else to do waits some hundred cycles for, six times
+// per reduction.  Every lane of the wave must be active.
+typedef unsigned lane_pair_t __attribute__((ext_vector_type(2)));
+template <int O>
+__device__ __forceinline__ uint32_t lane_xor(uint32_t b) {
+  static_assert(O == 32 || O == 16 || O == 8 || O == 4 || O == 2 || O == 1, "one bit of the lane index");
+  if constexpr (O == 32) {
+    // both halves of the wave in both results: r[0] = (low, low), r[1] = (high, high)
+    const lane_pair_t r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+    return (threadIdx.x & 32) ? r[0] : r[1];
+  } else if constexpr (O == 16) {
+    // rows of 16 lanes: r[0] = (row 0, row 0, row 2, row 2), r[1] = (row 1, row 1, row 3, row 3)
+    const lane_pair_t r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    return (threadIdx.x & 16) ? r[0] : r[1];
+  } else if constexpr (O == 8) {
+    return uint32_t(__builtin_amdgcn_update_dpp(0, int(b), 0x128, 0xF, 0xF, true));  // row_ror:8
+  } else if constexpr (O == 4) {
+    const int h = __builtin_amdgcn_update_dpp(0, int(b), 0x141, 0xF, 0xF, true);  // row_half_mirror: i -> 7 - i
+    return uint32_t(__builtin_amdgcn_update_dpp(0, h, 0x1B, 0xF, 0xF, true));      // quad_perm [3, 2, 1, 0]
+  } else if constexpr (O == 2) {
+    return uint32_t(__builtin_amdgcn_update_dpp(0, int(b), 0x4E, 0xF, 0xF, true));  // quad_perm [2, 3, 0, 1]
+  } else {
+    return uint32_t(__builtin_amdgcn_update_dpp(0, int(b), 0xB1, 0xF, 0xF, true));  // quad_perm [1, 0, 3, 2]
+  }
+}
+template <int O>
+__device__ __forceinline__ float lane_xor(float v) {
+  return __uint_as_float(lane_xor<O>(__float_as_uint(v)));
+}
+template <int O>
+__device__ __forceinline__ uint64_t lane_xor(uint64_t v) {
+  return uint64_t(lane_xor<O>(uint32_t(v))) | (uint64_t(lane_xor<O>(uint32_t(v >> 32))) << 32);
+}
+template <int O>
+__device__ __forceinline__ double lane_xor(double v) {
+  return __longlong_as_double((long long)lane_xor<O>(uint64_t(__double_as_longlong(v))));
+}
+template <int O>
+__device__ __forceinline__ long long lane_xor(long long v) {
+  return (long long)lane_xor<O>(uint64_t(v));
+}
+
+// The wave64 xor butterfly: step(lane distance as an integral constant) for 32, 16, 8, 4, 2, 1 in this order.
+template <int O>
+struct LaneDistance {
+  static constexpr int value = O;
+};
+template <typename Step>
+__device__ __forceinline__ void wave_butterfly(Step&& step) {
+  step(LaneDistance<32>{});
+  step(LaneDistance<16>{});
+  step(LaneDistance<8>{});
+  step(LaneDistance<4>{});
+  step(LaneDistance<2>{});
+  step(LaneDistance<1>{});
+}
+
+// lane `LANE`'s value in every lane
+template <int LANE = 0>
+__device__ __forceinline__ float lane_value(float v) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), LANE));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  wave_butterfly([&](auto o) { v += lane_xor<decltype(o)::value>(v); });
   return v;
 }
 __device__ __forceinline__ double wave_sum(double v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  wave_butterfly([&](auto o) { v += lane_xor<decltype(o)::value>(v); });
   return v;
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  wave_butterfly([&](auto o) { v = fmaxf(v, lane_xor<decltype(o)::value>(v)); });
   return v;
 }
 

@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kLmThreads, 1) void lmhead_fwd_kernel(const uint16_
   __syncthreads();
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const float m2 = __shfl_xor(m[j], 32, kWave), s2 = __shfl_xor(s[j], 32, kWave), t2 = __shfl_xor(t[j], 32, kWave);
+    const float m2 = lane_xor<32>(m[j]), s2 = lane_xor<32>(s[j]), t2 = lane_xor<32>(t[j]);
     const float mn = fmaxf(m[j], m2);
     const float fa = fast_exp2(m[j] - mn), fb = fast_exp2(m2 - mn);
     s[j] = s[j] * fa + s2 * fb;

@@ -184,21 +184,29 @@ __device__ __forceinline__ TopkGather topk_gather(const relax_amd_policy_loss_ar
   return g;
 }
 
+// Token `tok`'s entry count and union-mask length for the signal (the whole list / no mask without the arrays): two
+// more scalars that can be on their way before the row's log-sum-exp is known.
+struct TopkRowShape {
+  int width, nvalid;
+};
+__device__ __forceinline__ TopkRowShape topk_row_shape(const relax_amd_policy_loss_args& a, int64_t tok) {
+  return {a.topk_width ? a.topk_width[tok] : a.topk_k, a.topk_valid ? a.topk_valid[tok] : -1};
+}
+
 // The top-K distillation signal of one token inside the fused actor step, by the workgroup's first wave once the row's
 // log-sum-exp is known: log-probs at the token's K ids (as topk_logprob_fwd_kernel forms them), the per-token KL,
-// clips and weight, topk_kl / topk_grad written.  `g` = this lane's topk_gather(), `weight` = the signal's weight in
-// the loss, `old` = the token's old log-prob (the current one when there is none).  Returns, in every lane, the sum of
-// d loss / d log p[id_k] over the non-sentinel ids: what the row's softmax is multiplied by, next to the policy
-// terms' own coefficient.  `stage` = kTopkStageFloats floats of LDS.
+// clips and weight, topk_kl / topk_grad written.  `g` = this lane's topk_gather(), `shape` = topk_row_shape() of the
+// token, `weight` = the signal's weight in the loss, `old` = the token's old log-prob (the current one when there is
+// none).  Returns, in every lane, the sum of d loss / d log p[id_k] over the non-sentinel ids: what the row's softmax
+// is multiplied by, next to the policy terms' own coefficient.  `stage` = kTopkStageFloats floats of LDS.
 constexpr int kTopkStageFloats = 4 * RELAX_AMD_FUSED_TOPK_MAX;
 
 __device__ __forceinline__ float topk_distill_row(const relax_amd_policy_loss_args& a, const TopkGather& g,
-                                                  int64_t tok, float lse, float inv_t, float lp, float old,
-                                                  float weight, int lane, float* stage) {
+                                                  const TopkRowShape& shape, int64_t tok, float lse, float inv_t,
+                                                  float lp, float old, float weight, int lane, float* stage) {
   const int kmax = a.topk_k;
-  int width = a.topk_width ? a.topk_width[tok] : kmax;
-  width = width < 0 ? 0 : (width > kmax ? kmax : width);
-  const int nvalid = a.topk_valid ? a.topk_valid[tok] : -1;
+  const int width = shape.width < 0 ? 0 : (shape.width > kmax ? kmax : shape.width);
+  const int nvalid = shape.nvalid;
   const OpdParams p{a.topk_kl_mode, a.topk_norm_mode, a.topk_jsd_alpha, a.topk_has_clamp, a.topk_min_clamp};
   float* sv = stage;
   float* tv = stage + RELAX_AMD_FUSED_TOPK_MAX;

@@ -113,9 +113,9 @@ __global__ __launch_bounds__(kFinishThreads) void policy_loss_finish_kernel(cons
     __syncthreads();
   }
   if (k >= kWave) return;
-  const float pg = __shfl(total, RELAX_AMD_M_PG_LOSS, kWave);
-  const float ent = __shfl(total, RELAX_AMD_M_ENTROPY, kWave);
-  const float kl = __shfl(total, RELAX_AMD_M_KL_LOSS, kWave);
+  const float pg = lane_value<RELAX_AMD_M_PG_LOSS>(total);
+  const float ent = lane_value<RELAX_AMD_M_ENTROPY>(total);
+  const float kl = lane_value<RELAX_AMD_M_KL_LOSS>(total);
   if (k == RELAX_AMD_M_LOSS) {
     total = pg - entropy_coef * ent;
     if (has_kl) total = total + kl_coef * kl;

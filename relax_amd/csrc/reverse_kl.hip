@@ -70,12 +70,11 @@ __global__ __launch_bounds__(kKlThreads) void reverse_kl_fwd_kernel(const T* __r
       absorb_pair(a, b, q);
     }
   }
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) {
-    KlState other{__shfl_xor(q.ms, o, kWave), __shfl_xor(q.ss, o, kWave), __shfl_xor(q.us, o, kWave),
-                  __shfl_xor(q.mt, o, kWave), __shfl_xor(q.st, o, kWave)};
+  wave_butterfly([&](auto o) {
+    constexpr int O = decltype(o)::value;
+    KlState other{lane_xor<O>(q.ms), lane_xor<O>(q.ss), lane_xor<O>(q.us), lane_xor<O>(q.mt), lane_xor<O>(q.st)};
     merge_kl(q, other);
-  }
+  });
   const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
   if (lane == 0) {
     lds[w][0] = q.ms;
@@ -227,12 +226,11 @@ __global__ __launch_bounds__(THREADS) void reverse_kl_step_kernel(
     float a[1] = {Row<T>::load1(xs + e)}, b[1] = {Row<T>::load1(xt + e)};
     absorb_pair(a, b, q);
   }
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) {
-    KlState other{__shfl_xor(q.ms, o, kWave), __shfl_xor(q.ss, o, kWave), __shfl_xor(q.us, o, kWave),
-                  __shfl_xor(q.mt, o, kWave), __shfl_xor(q.st, o, kWave)};
+  wave_butterfly([&](auto o) {
+    constexpr int O = decltype(o)::value;
+    KlState other{lane_xor<O>(q.ms), lane_xor<O>(q.ss), lane_xor<O>(q.us), lane_xor<O>(q.mt), lane_xor<O>(q.st)};
     merge_kl(q, other);
-  }
+  });
   const int lane = tid & (kWave - 1), w = tid / kWave;
   if (lane == 0) {
     lds[w][0] = q.ms;

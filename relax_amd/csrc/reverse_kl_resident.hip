@@ -254,12 +254,11 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
       __builtin_amdgcn_sched_barrier(0);
     }
     // merge: wave64 butterfly, then the waves in index order through LDS (as in the two-walk kernel)
-#pragma unroll
-    for (int o = kWave / 2; o > 0; o >>= 1) {
-      KlState other{__shfl_xor(q.ms, o, kWave), __shfl_xor(q.ss, o, kWave), __shfl_xor(q.us, o, kWave),
-                    __shfl_xor(q.mt, o, kWave), __shfl_xor(q.st, o, kWave)};
+    wave_butterfly([&](auto o) {
+      constexpr int O = decltype(o)::value;
+      KlState other{lane_xor<O>(q.ms), lane_xor<O>(q.ss), lane_xor<O>(q.us), lane_xor<O>(q.mt), lane_xor<O>(q.st)};
       merge_kl(q, other);
-    }
+    });
     int merge_id = tid;
     asm volatile("" : "+v"(merge_id));  // the LDS slot is recomputed per row rather than kept (and spilled)
     const int lane = merge_id & (kWave - 1), w = merge_id / kWave;

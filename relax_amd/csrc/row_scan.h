@@ -99,9 +99,10 @@ __device__ __forceinline__ SoftmaxAcc scan_row(const T* __restrict__ x, int64_t 
 // Wave64 xor-butterfly, then waves in index order through LDS; the merged state is valid in thread 0 only.
 template <int THREADS>
 __device__ __forceinline__ void scan_block_merge(SoftmaxAcc& st, float (*wave_state)[3]) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1)
-    scan_merge(st, __shfl_xor(st.m, o, kWave), __shfl_xor(st.s, o, kWave), __shfl_xor(st.t, o, kWave));
+  wave_butterfly([&](auto o) {
+    constexpr int O = decltype(o)::value;
+    scan_merge(st, lane_xor<O>(st.m), lane_xor<O>(st.s), lane_xor<O>(st.t));
+  });
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   if (lane == 0) {
     wave_state[wave][0] = st.m;

@@ -43,11 +43,10 @@ __global__ __launch_bounds__(kWave) void reinforce_pp_returns_kernel(const F* __
   long long last = -1;
   for (int64_t j = lane; j < len; j += kWave)
     if (mask[beg + j] != F(0)) last = j;
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) {
-    const long long other = __shfl_xor(last, o, kWave);
+  wave_butterfly([&](auto o) {
+    const long long other = lane_xor<decltype(o)::value>(last);
     last = other > last ? other : last;
-  }
+  });
   if (last < 0) {
     for (int64_t j = lane; j < len; j += kWave) out[beg + j] = F(0);
     return;

@@ -284,9 +284,12 @@ __global__ __launch_bounds__(kTkThreads, 8) void topk_rows_fast_kernel(const T* 
         uint32_t top = nan ? 0xFFFFFFFFu : tk_key(vmax);
         top = i < nvec ? top : 0u;
         best = top > best ? top : best;
-#pragma unroll
-        for (int o = 1; o < 8; o <<= 1) {
-          const uint32_t other = __shfl_xor(top, o, kWave);
+        {
+          uint32_t other = lane_xor<1>(top);
+          top = other > top ? other : top;
+          other = lane_xor<2>(top);
+          top = other > top ? other : top;
+          other = lane_xor<4>(top);
           top = other > top ? other : top;
         }
         if ((tid & 7) == 0 && i < nvec) group_best[i >> 3] = top;
