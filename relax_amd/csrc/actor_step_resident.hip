@@ -4,9 +4,8 @@
 //
 // A 1024-thread workgroup holds a whole row in its vector registers (V = 151936 bf16 is 18992 16-byte vectors = 19 per
 // thread = 76 registers), so HBM sees exactly one read and one write per row and the second walk over the row costs no
-// cache or fabric traffic at all.  One such workgroup fits a CU (fp32 rows: 512-thread workgroups with 16 vectors per
-// thread, two per CU); the workgroups are persistent (one per CU, rows b,
-// b + grid, ...) and take a row in three steps: the resident row becomes its gradient in place; the gradient leaves in
+// cache or fabric traffic at all.  One such workgroup fits a CU (fp32 rows of 32000 entries: 8 vectors per thread); the
+// workgroups are persistent (one per CU, rows b, b + grid, ...) and take a row in three steps: the resident row becomes its gradient in place; the gradient leaves in
 // one burst of stores and, into the registers those free, the workgroup's next live row arrives in one burst of loads
 // (304 KB out, 304 KB in, each contiguous); the new row's softmax scan follows its loads in their order.  Memory rewards
 // the long bursts: with a store and a load alternating vector by vector (and the scan trailing four vectors behind) the
@@ -86,11 +85,12 @@ struct ResidentTokenData {
   int64_t tg;
 };
 
-// Workgroup width by element type: 16-bit rows in 1024-thread workgroups (one per CU), 32-bit rows in 512-thread
-// workgroups (two per CU; only short rows fit: a thread can give the row about 64 of its 128 registers).
+// Workgroup width: one 1024-thread workgroup per CU for every element type.  (fp32 rows of 32000 entries used to run
+// in two 512-thread workgroups per CU with 16 vectors per thread; a plain stream of such rows in that arrangement
+// moves 5.39 TB/s, in this one 5.62: a CU's stores and loads leave in longer runs of one kind.)
 template <typename T>
 constexpr int resident_threads() {
-  return sizeof(T) == 2 ? 1024 : 512;
+  return 1024;
 }
 
 template <typename T, int NVF, bool PARTIAL, bool TOPK = false>
@@ -358,8 +358,8 @@ int launch_actor_step_resident(const T* logits, int64_t row_stride, int64_t voca
     RELAX_AMD_RESIDENT(16, false)
     RELAX_AMD_RESIDENT(12, true)
   } else {
-    // fp32 rows of 32000 entries (8000 vectors: 15 per thread and 320 lanes with a sixteenth)
-    RELAX_AMD_RESIDENT(15, true)
+    // fp32 rows of 32000 entries (8000 vectors: 7 per thread and 832 lanes with an eighth)
+    RELAX_AMD_RESIDENT(7, true)
   }
   return RELAX_AMD_EUNSUPPORTED;
 }

@@ -1,5 +1,5 @@
 // dlogits backward of the log-prob / entropy pair in the burst form of the register-resident actor step: persistent
-// workgroups (one per CU for 16-bit rows, two for fp32 rows of 32000 entries), each taking a whole row into its
+// workgroups (one of 1024 threads per CU), each taking a whole row into its
 // registers in one burst of loads, turning it into its gradient in place and writing it out in one burst of stores.
 // Same arithmetic, element by element, as logprob_entropy_bwd_kernel (logprob_entropy.hip):
 //   d = inv_t * p * (-g_lp + g_H * (spx - x * inv_t))  (+ inv_t * g_lp at the target),  p = exp(x * inv_t - lse),
@@ -19,10 +19,10 @@
 
 namespace relax_amd {
 
-// Workgroup width by element type, as in the register-resident actor step.
+// Workgroup width, as in the register-resident actor step.
 template <typename T>
 constexpr int bwd_resident_threads() {
-  return sizeof(T) == 2 ? 1024 : 512;
+  return 1024;
 }
 
 template <typename T, int NVF, bool PARTIAL>
@@ -179,7 +179,7 @@ int launch_logprob_bwd_resident(const T* logits, int64_t row_stride, int64_t voc
     RELAX_AMD_BWD_RESIDENT(12, true)
   } else {
     // fp32 rows of 32000 entries
-    RELAX_AMD_BWD_RESIDENT(15, true)
+    RELAX_AMD_BWD_RESIDENT(7, true)
   }
   return RELAX_AMD_EUNSUPPORTED;
 }

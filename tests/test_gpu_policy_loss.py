@@ -1669,7 +1669,7 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
     """More logits rows than persistent workgroups, so every workgroup of the register-resident kernel rolls several
     rows through its registers (prompt rows, fully masked samples and masked tokens in between), for every row shape
     the kernel is built for (12 / 15 / 18 / 19 full vectors per thread plus a partial one, 16 or 20 exactly; fp32 rows of 32000
-    entries in 512-thread workgroups, two per CU) and one it is not (65536: two-walk kernel): same loss bits as the two-launch path, gradients equal to it and to the oracle."""
+    entries: 7 plus a partial one) and one it is not (65536: two-walk kernel): same loss bits as the two-launch path, gradients equal to it and to the oracle."""
     import relax_amd
 
     dev = require_gpu()
@@ -1708,7 +1708,7 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
     the very end, fewer live rows than workgroups, random prompt rows and masked tokens over several rows per
     workgroup, no row map (every row scores its own token), and tokens whose gradient coefficients vanish (zero
     rows without a look at the logits); on 16-bit rows of 12 full vectors per thread plus a partial one (one
-    1024-thread workgroup per CU) and on fp32 rows of 32000 entries (two 512-thread workgroups per CU).  Every output
+    1024-thread workgroup per CU) and on fp32 rows of 32000 entries.  Every output
     must be bit-identical."""
     from relax_amd import ops
 
@@ -1765,7 +1765,7 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
 @pytest.mark.parametrize("v,dtype", [(8 * (18 * 1024 + 1), torch.bfloat16), (8 * (19 * 1024 - 1), torch.bfloat16),
                                      (8 * (19 * 1024 + 1), torch.bfloat16), (8 * 20 * 1024, torch.float16),
                                      (8 * (12 * 1024 + 1), torch.float16), (8 * (16 * 1024 - 1), torch.bfloat16),
-                                     (4 * (15 * 512 + 1), torch.float32), (4 * (16 * 512 - 1), torch.float32)])
+                                     (4 * (7 * 1024 + 1), torch.float32), (4 * (8 * 1024 - 1), torch.float32)])
 def test_register_resident_kernel_at_the_edges_of_its_row_shapes(v, dtype, monkeypatch):
     """Row lengths at both ends of a built shape: one lane, or all lanes but one, hold a vector at the partially filled
     position.  Every output bit-identical to the two-walk kernel's."""
