@@ -334,7 +334,9 @@ def test_topk_rows_equals_torch_topk(n, v, k, dtype):
 @pytest.mark.parametrize("n,v,k,dtype,temperature", [
     (96, 151936, 64, torch.bfloat16, 1.0),    # the production row: one read serves both
     (40, 151936, 8, torch.float32, 0.7),      # fp32 rows of the same vocabulary
-    (50, 65536, 512, torch.float16, 1.0),     # the shortest row the fused kernel takes, the largest k
+    (50, 65536, 512, torch.float16, 1.0),     # a short row for the fused kernel, the largest k
+    (44, 8 * 7168, 64, torch.bfloat16, 1.0),  # the shortest row the fused kernel takes (1024-thread workgroups from here on)
+    (36, 32000, 32, torch.float32, 1.0),      # fp32 rows of the small benchmark vocabulary: 8000 vectors, likewise
     (50, 32003, 100, torch.float16, 1.0),     # rows that are not 16-byte aligned: the two passes run one after the other
     (30, 4104, 16, torch.bfloat16, 1.3),      # a short row: likewise
 ])
