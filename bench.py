@@ -450,6 +450,9 @@ def load_ceilings():
     lib.ceiling_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
     lib.ceiling_row_copy.restype = C.c_int
     lib.ceiling_row_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_void_p]
+    lib.ceiling_burst_copy.restype = C.c_int
+    lib.ceiling_burst_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int,
+                                       C.c_void_p, C.c_void_p]
 
     def check(rc):
         if rc != 0:
@@ -505,8 +508,11 @@ def run_mfma_ceiling(a, dev) -> None:
 
 def run_hbm_ceiling(a, dev) -> None:
     """Diagnostic, not a workload of the path: plain read / write / copy streams over a buffer of the actor step's
-    logits size (65536 x 151936 bf16 = 19.9 GB), 16-byte accesses.  What these sustain is the practical ceiling for the
-    bandwidth-bound kernels on this box.  A "step" is one read, one write and one copy launch."""
+    logits size (65536 x 151936 bf16 = 19.9 GB), 16-byte accesses, and the same copy in the burst form of the
+    register-resident kernels (persistent workgroups, a row in by one run of loads, out by one run of stores) on the
+    rows of the two actor-step shapes, in the workgroup arrangements that were compared for them and with the grid's
+    workgroups kept in step.  What these sustain is the practical ceiling for the bandwidth-bound kernels on this box.
+    A "step" is one launch of each."""
     import ctypes as C
     from relax_amd import ops
 
@@ -515,8 +521,14 @@ def run_hbm_ceiling(a, dev) -> None:
     src = torch.ones(nbytes // 2, dtype=torch.bfloat16, device=dev)
     dst = torch.empty_like(src)
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    phases = torch.zeros(4, dtype=torch.int32, device=dev)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     p = lambda t: C.c_void_p(t.data_ptr())
+    bf16_rows, f32_rows = (65536, 151936 * 2), (131072, 32000 * 4)  # (rows, bytes per row) of cfg2 and cfg1
+    # name -> (rows, threads per workgroup, workgroups per CU, kept in step)
+    bursts = {"burst_copy_bf16_rows": (bf16_rows, 1024, 1, 0), "burst_copy_bf16_rows_in_step": (bf16_rows, 1024, 1, 1),
+              "burst_copy_f32_rows_1024x1": (f32_rows, 1024, 1, 0), "burst_copy_f32_rows_512x2": (f32_rows, 512, 2, 0),
+              "burst_copy_f32_rows_1024x2": (f32_rows, 1024, 2, 0), "burst_copy_f32_rows_in_step": (f32_rows, 1024, 1, 1)}
 
     def step():
         for mode, name in ((0, "diag_stream_read"), (1, "diag_stream_write"), (2, "diag_stream_copy")):
@@ -524,6 +536,12 @@ def run_hbm_ceiling(a, dev) -> None:
                 check(lib.ceiling_stream(mode, p(src), p(dst), nbytes, p(sink), stream))
         with ops._timed("diag_row_copy"):  # the same copy, one persistent workgroup per CU walking whole rows
             check(lib.ceiling_row_copy(p(src), p(dst), 65536, 151936 * 2, 256, stream))
+        for name, ((rows, row_bytes), threads, per_cu, in_step) in bursts.items():
+            if in_step:
+                phases.zero_()
+            with ops._timed(name):
+                check(lib.ceiling_burst_copy(p(src), p(dst), rows, row_bytes, threads, per_cu, in_step, p(phases),
+                                             stream))
         with ops._timed("memset"):
             dst.view(torch.int32).zero_()
         return dst
@@ -534,12 +552,17 @@ def run_hbm_ceiling(a, dev) -> None:
              "copy_GBs": 2 * nbytes / kernel_ms["diag_stream_copy"] / 1e6,
              "row_copy_GBs": 2 * nbytes / kernel_ms["diag_row_copy"] / 1e6,
              "torch_zero_fill_GBs": nbytes / kernel_ms["memset"] / 1e6}
+    for name, ((rows, row_bytes), *_rest) in bursts.items():
+        rates[name + "_GBs"] = 2 * rows * row_bytes / kernel_ms[name] / 1e6
+    rates["in_step_waits_given_up"] = int(phases[2].item())  # of the last launch kept in step; 0 = it ran as meant
     print(json.dumps({
         "metric": "GB/s of plain HBM streams [diagnostic ceiling, not the headline metric]", "value": rates["read_GBs"],
         "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": wall * 1e3 / a.steps,
         "higher_is_better": True, "dtype": "u8", "data": "synthetic",
         "config": {"workload": "hbm_ceiling: read, write, copy, row-wise copy (65536 rows of 303872 bytes, 256 persistent "
-                               "workgroups) and zero fill of 19.9 GB with 16-byte accesses", **rates},
+                               "workgroups) and zero fill of 19.9 GB with 16-byte accesses; burst-form copies of the "
+                               "65536 x 303872-byte and 131072 x 128000-byte rows (threads x workgroups per CU; "
+                               "in_step = the grid's workgroups aligned turn by turn)", **rates},
         "roofline": {"bound": "hbm", "kernel": "diag_stream_kernel<0> (read)", "achieved": rates["read_GBs"],
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": rates["read_GBs"] / HBM_PEAK_GBS, "traffic": None,
                      "kernel_ms": kernel_ms},

@@ -131,6 +131,65 @@ __global__ __launch_bounds__(1024) void diag_row_copy_kernel(const u32x4* __rest
   }
 }
 
+// The copy in the burst form of the register-resident kernels: persistent workgroups, a whole row into the registers
+// by one run of loads, out again by one run of stores, the next row's loads issued right behind them.  Nothing else:
+// what this sustains is the ceiling of those kernels' memory pattern.  THREADS x NV vectors hold a row (rows shorter
+// than that leave the last positions partly empty), OCC workgroups share a CU.  With ALIGN the workgroups of the
+// whole grid keep in step: each announces that its loads are issued and waits, for a bounded number of polls, until
+// all have done so before its stores go out (phases[0] counts the announcements, phases[1] is set when a wait ran
+// out, after which nobody waits any more, phases[2] counts such waits).
+template <int THREADS, int NV, int OCC, bool ALIGN>
+__global__ __launch_bounds__(THREADS, OCC) void diag_burst_copy_kernel(const u32x4* __restrict__ in,
+                                                                       u32x4* __restrict__ out, int64_t rows,
+                                                                       int64_t row_vecs, unsigned* phases) {
+  const int tid = threadIdx.x;
+  u32x4 reg[NV];
+  int64_t row = blockIdx.x;
+  if (row >= rows) return;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int64_t v = tid + j * THREADS;
+    reg[j] = __builtin_nontemporal_load(in + row * row_vecs + (v < row_vecs ? v : 0));
+  }
+  unsigned turn = 0;
+  if (ALIGN && tid == 0) __hip_atomic_fetch_add(&phases[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  while (true) {
+    __syncthreads();  // as the row kernels: the row is complete in the registers behind their barrier
+    if (ALIGN) {
+      if (tid == 0 && !__hip_atomic_load(&phases[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+        const unsigned target = (turn + 1) * gridDim.x;
+        int polls = 0;
+        while (__hip_atomic_load(&phases[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+          if (++polls > 3000) {  // a few milliseconds: workgroups that are not co-resident, or an uneven row count
+            __hip_atomic_store(&phases[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_fetch_add(&phases[2], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+          __builtin_amdgcn_s_sleep(4);
+        }
+      }
+      __syncthreads();
+    }
+    const int64_t next = row + gridDim.x;
+    const bool has_next = next < rows;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int64_t v = tid + j * THREADS;
+      if (v < row_vecs) __builtin_nontemporal_store(reg[j], out + row * row_vecs + v);
+    }
+    const int64_t src = has_next ? next : row;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int64_t v = tid + j * THREADS;
+      reg[j] = __builtin_nontemporal_load(in + src * row_vecs + (v < row_vecs ? v : 0));
+    }
+    ++turn;
+    if (ALIGN && tid == 0) __hip_atomic_fetch_add(&phases[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!has_next) return;
+    row = next;
+  }
+}
+
 }  // namespace relax_amd
 
 using namespace relax_amd;
@@ -181,4 +240,43 @@ extern "C" int ceiling_mfma_loop(const void* src, float* out, int blocks, int it
     hipLaunchKernelGGL(diag_mfma_loop16_kernel, dim3(unsigned(blocks)), dim3(512), 0, s,
                        static_cast<const diag_bf16x8*>(src), out, iters);
   return int(hipGetLastError());
+}
+
+// Burst-form copy of `rows` rows of `row_bytes` bytes.  threads = 1024 or 512 per workgroup, per_cu = 1 or 2
+// persistent workgroups per CU; rows of up to 8 (1024 threads) / 16 (512 threads) vectors per thread take the short
+// shape, longer ones (1024 threads only) 19 vectors per thread.  align != 0: the phase-aligned form, `phases` = three
+// zeroed 32-bit words of device memory (see the kernel).
+extern "C" int ceiling_burst_copy(const void* src, void* dst, int64_t rows, int64_t row_bytes, int threads, int per_cu,
+                                  int align, unsigned* phases, void* stream) {
+  if (!src || !dst || rows < 0 || row_bytes <= 0 || row_bytes % 16 != 0 || !aligned16(src) || !aligned16(dst) ||
+      (threads != 1024 && threads != 512) || (per_cu != 1 && per_cu != 2) || (align && !phases))
+    return -1;
+  if (rows == 0) return 0;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    return -1;
+  const int64_t row_vecs = row_bytes / 16;
+  const int64_t slots = int64_t(cus) * per_cu;
+  const dim3 grid(unsigned(rows < slots ? rows : slots));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const u32x4* in = static_cast<const u32x4*>(src);
+  u32x4* out = static_cast<u32x4*>(dst);
+#define RELAX_AMD_BURST(THREADS, NV, OCC)                                                                          \
+  if (threads == THREADS && per_cu == OCC && row_vecs <= int64_t(THREADS) * NV) {                                   \
+    if (align)                                                                                                      \
+      hipLaunchKernelGGL((diag_burst_copy_kernel<THREADS, NV, OCC, true>), grid, dim3(THREADS), 0, s, in, out, rows, \
+                         row_vecs, phases);                                                                         \
+    else                                                                                                            \
+      hipLaunchKernelGGL((diag_burst_copy_kernel<THREADS, NV, OCC, false>), grid, dim3(THREADS), 0, s, in, out,      \
+                         rows, row_vecs, phases);                                                                   \
+    return int(hipGetLastError());                                                                                  \
+  }
+  RELAX_AMD_BURST(1024, 8, 1)
+  RELAX_AMD_BURST(1024, 8, 2)
+  RELAX_AMD_BURST(512, 16, 2)
+  RELAX_AMD_BURST(512, 16, 1)
+  RELAX_AMD_BURST(1024, 19, 1)
+#undef RELAX_AMD_BURST
+  return -1;
 }
