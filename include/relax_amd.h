@@ -428,8 +428,8 @@ int relax_amd_logprob_entropy_topk_fwd(const void* logits, int dtype, int64_t n_
  * With loss->topk_ids set the step also evaluates the top-K distillation signal of every row it reads (see the
  * argument block); the caller adds the K one-hot parts of its gradient with relax_amd_sparse_row_add afterwards.
  * Two kernels sit behind this entry point and are chosen by row length and element type: a register-resident one
- * (one read and one write of HBM per row; 16-bit rows of 100352 .. 163840 entries and fp32 rows of 32000 entries in
- * the built shapes) and a two-walk one for everything else; RELAX_AMD_FUSED_STEP_KERNEL=cached in the environment
+ * (one read and one write of HBM per row; 16-bit rows of 57352 .. 65536 and 100352 .. 163840 entries, fp32 rows of
+ * 28676 .. 32768, 49156 .. 53248 and 61444 .. 65536 entries, in the built shapes) and a two-walk one for everything else; RELAX_AMD_FUSED_STEP_KERNEL=cached in the environment
  * forces the latter.  Same results.
  */
 int relax_amd_actor_step_fused(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,

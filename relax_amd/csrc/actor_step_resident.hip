@@ -1,6 +1,6 @@
 // Register-resident fused actor step: the same computation as actor_step_fused_kernel (log-prob + entropy forward,
 // per-token policy-loss coefficients, dlogits backward, one launch) for long 16-bit rows of the common vocabulary sizes
-// and for fp32 rows of 32000 entries.
+// and for fp32 rows of 32000 entries (and a few neighbouring sizes of either kind, see the launcher).
 //
 // A 1024-thread workgroup holds a whole row in its vector registers (V = 151936 bf16 is 18992 16-byte vectors = 19 per
 // thread = 76 registers), so HBM sees exactly one read and one write per row and the second walk over the row costs no
@@ -357,9 +357,17 @@ int launch_actor_step_resident(const T* logits, int64_t row_stride, int64_t voca
     RELAX_AMD_RESIDENT(15, true)
     RELAX_AMD_RESIDENT(16, false)
     RELAX_AMD_RESIDENT(12, true)
-  } else {
-    // fp32 rows of 32000 entries (8000 vectors: 7 per thread and 832 lanes with an eighth)
+    // and the short end of the 1024-thread rows: 65536 entries (8192 vectors) and 57352 .. 65528 (64000: 8000)
+    RELAX_AMD_RESIDENT(8, false)
     RELAX_AMD_RESIDENT(7, true)
+  } else {
+    // fp32 rows of 32000 entries (8000 vectors: 7 per thread and 832 lanes with an eighth), of 32768, of
+    // 49156 .. 53248 (50304: 12576 vectors), of 61444 .. 65532 (64000) and of 65536
+    RELAX_AMD_RESIDENT(7, true)
+    RELAX_AMD_RESIDENT(8, false)
+    RELAX_AMD_RESIDENT(12, true)
+    RELAX_AMD_RESIDENT(15, true)
+    RELAX_AMD_RESIDENT(16, false)
   }
   return RELAX_AMD_EUNSUPPORTED;
 }

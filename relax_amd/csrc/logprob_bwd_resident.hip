@@ -177,9 +177,16 @@ int launch_logprob_bwd_resident(const T* logits, int64_t row_stride, int64_t voc
     RELAX_AMD_BWD_RESIDENT(15, true)
     RELAX_AMD_BWD_RESIDENT(16, false)
     RELAX_AMD_BWD_RESIDENT(12, true)
-  } else {
-    // fp32 rows of 32000 entries
+    // 65536 and 57352 .. 65528 (64000)
+    RELAX_AMD_BWD_RESIDENT(8, false)
     RELAX_AMD_BWD_RESIDENT(7, true)
+  } else {
+    // fp32 rows of 32000 entries, of 32768, of 49156 .. 53248, of 61444 .. 65532 and of 65536
+    RELAX_AMD_BWD_RESIDENT(7, true)
+    RELAX_AMD_BWD_RESIDENT(8, false)
+    RELAX_AMD_BWD_RESIDENT(12, true)
+    RELAX_AMD_BWD_RESIDENT(15, true)
+    RELAX_AMD_BWD_RESIDENT(16, false)
   }
   return RELAX_AMD_EUNSUPPORTED;
 }

@@ -241,7 +241,9 @@ def test_full_size_properties_headline_shape():
                                        (128256, torch.float16, 600), (131072, torch.bfloat16, 40),
                                        (100352, torch.bfloat16, 1100), (8 * (16 * 1024 - 1), torch.float16, 300),
                                        (163840, torch.bfloat16, 300), (8 * (19 * 1024 + 1), torch.float16, 520),
-                                       (32000, torch.float32, 1500), (4 * (8 * 1024 - 1), torch.float32, 700)])
+                                       (32000, torch.float32, 1500), (4 * (8 * 1024 - 1), torch.float32, 700),
+                                       (64000, torch.bfloat16, 900), (65536, torch.float16, 600),
+                                       (50304, torch.float32, 700), (65536, torch.float32, 500)])
 def test_backward_burst_form_equals_row_per_workgroup_kernel_bitwise(v, dtype, n, monkeypatch):
     """The two kernels behind relax_amd_logprob_entropy_bwd, switched with RELAX_AMD_FUSED_STEP_KERNEL, on every row
     shape the persistent burst form is built for (and the ends of two of them), with rows that score no token, tokens

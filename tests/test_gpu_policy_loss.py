@@ -1664,12 +1664,15 @@ def test_custom_loss_function_path_dispatch():
 @pytest.mark.parametrize("v,dtype,n_samples", [(100352, torch.bfloat16, 18), (128256, torch.float16, 18),
                                                 (131072, torch.bfloat16, 18), (151936, torch.bfloat16, 18),
                                                 (163840, torch.bfloat16, 18), (160000, torch.float16, 18),
-                                                (65536, torch.bfloat16, 18), (32000, torch.float32, 40)])
+                                                (65536, torch.bfloat16, 18), (64000, torch.float16, 20),
+                                                (90112, torch.bfloat16, 20), (32000, torch.float32, 40),
+                                                (32768, torch.float32, 40), (50304, torch.float32, 30),
+                                                (64000, torch.float32, 24), (65536, torch.float32, 24)])
 def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples):
     """More logits rows than persistent workgroups, so every workgroup of the register-resident kernel rolls several
     rows through its registers (prompt rows, fully masked samples and masked tokens in between), for every row shape
-    the kernel is built for (12 / 15 / 18 / 19 full vectors per thread plus a partial one, 16 or 20 exactly; fp32 rows of 32000
-    entries: 7 plus a partial one) and one it is not (65536: two-walk kernel): same loss bits as the two-launch path, gradients equal to it and to the oracle."""
+    the kernel is built for (7 / 12 / 15 / 18 / 19 full vectors per thread plus a partial one, 8 / 16 / 20 exactly; fp32 rows
+    of 7 / 12 / 15 plus a partial one, 8 / 16 exactly) and one it is not (90112, 11 exactly: two-walk kernel): same loss bits as the two-launch path, gradients equal to it and to the oracle."""
     import relax_amd
 
     dev = require_gpu()
@@ -1679,7 +1682,7 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
     resp = [int(torch.randint(1, t, (1,), generator=g)) for t in tot]
     logits, batch = _make_batch(29, tot, resp, v, dtype)
     batch["loss_masks"][3] = torch.zeros_like(batch["loss_masks"][3])
-    assert sum(tot) > (600 if dtype != torch.float32 else 1200)
+    assert sum(tot) > 600  # more than two rows for each of the 256 persistent workgroups
     db = _to_dev(batch, dev)
     kw = dict(eps_clip_high=0.28, use_kl_loss=True, kl_loss_coef=1e-3, kl_loss_type="k3", entropy_coef=0.01)
     outs = {}
@@ -1765,7 +1768,9 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
 @pytest.mark.parametrize("v,dtype", [(8 * (18 * 1024 + 1), torch.bfloat16), (8 * (19 * 1024 - 1), torch.bfloat16),
                                      (8 * (19 * 1024 + 1), torch.bfloat16), (8 * 20 * 1024, torch.float16),
                                      (8 * (12 * 1024 + 1), torch.float16), (8 * (16 * 1024 - 1), torch.bfloat16),
-                                     (4 * (7 * 1024 + 1), torch.float32), (4 * (8 * 1024 - 1), torch.float32)])
+                                     (4 * (7 * 1024 + 1), torch.float32), (4 * (8 * 1024 - 1), torch.float32),
+                                     (8 * (7 * 1024 + 1), torch.bfloat16), (8 * 8 * 1024, torch.float16),
+                                     (4 * (12 * 1024 + 1), torch.float32), (4 * (16 * 1024 - 1), torch.float32)])
 def test_register_resident_kernel_at_the_edges_of_its_row_shapes(v, dtype, monkeypatch):
     """Row lengths at both ends of a built shape: one lane, or all lanes but one, hold a vector at the partially filled
     position.  Every output bit-identical to the two-walk kernel's."""
