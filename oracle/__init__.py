@@ -45,11 +45,20 @@ live in ``tests/test_oracle_*.py``):
   of tests/backends/megatron/test_ppo_gae_parity.py:41-60.  ``advantages.masked_normalize``: numpy
   population moments.  ``opd.opd_kl`` union mask / ``log_probs_on_topk_ids``: closed forms (row-prefix
   equivalence, textbook JSD, ``log_softmax`` gather).
-* ``losses.m2po*`` (second-moment trust region): no reference test or fixture; ``m2po_solve_tau`` is pinned by
-  enumeration (every data value tried as the cap: the chosen one is the largest whose capped sum stays below the
-  budget, and the reported moment is that capped sum / n), the harmful-token set, the within-budget, no-harmful-token
-  and all-equal cases by closed forms, the loss by ``policy_clip`` with the solved margins.  The reference's quirk that
-  a stop at the first element reports the uncapped moment is kept (read from ppo_utils.py:417-418).
+* ``opd.reduce_token_mean``: the literal of tests/backends/megatron/test_opd_loss_aggregation.py:36-49 (12 / 3), a
+  case where the token mean differs from a mean of sample means, the clamp on the whole count, the gradient
+  mask / count.  ``opd.policy_opd_loss`` (opd_utils.py:1368-1455): per-token Python loops for the sampled-token and
+  the three top-K selections (row loops over the K entries for reverse / forward KL and JSD in the ``tail`` / ``norm``
+  / ``trunc`` modes, the union path's per-row lengths); the clip order (per-token clip, then the truncated importance
+  ratio as a constant), both clip fractions as means over every token (masked ones included), the ``None`` returns,
+  the detached teacher.  ``opd.apply_to_advantages`` (opd_utils.py:1275-1351): the same row loops; the clip acts on
+  the top-K branch only, the term is detached, list entries are replaced.  All in ``tests/test_oracle_opd.py``.
+* ``policy.sft_loss_function`` (loss.py:1247-1293): ``F.cross_entropy`` on the shifted targets (row t scores token
+  t + 1, pad id 0 for the last row) with the masked reduction written as a loop, both reducer modes.
+  ``policy.loss_function`` tail (loss.py:1515-1620): a three-token case with every log-prob = log 1/2 worked by hand
+  for the micro-batch scale, ``dynamic_global_batch_size``, ``__loss_scale__``, the per-token mode and dummy
+  micro-batches in both modes (zero loss still attached to the graph, zeroed ``values``, normaliser 0 / 1); the
+  ``loss_type`` dispatch and an explicit callable.
 * ``policy.value_loss_function`` / ``policy.get_values``: a three-token case worked by hand (clipped and unclipped
   branches of the maximum, the clip fraction, the response-row slicing).
 * ``losses.opsm_mask`` (ppo_utils.py:142-180): scalar per-sequence / per-token Python loops on a hand-worked case

@@ -120,63 +120,3 @@ def icepop(pg_loss, train_lp, rollout_lp, clip_low: float, clip_high: float):
         "mismatch_k3_kl": (tis - log_ratio - 1).detach(),
     }
     return pg_loss * w, metrics
-
-
-# ---- M2PO: second-moment trust region (ppo_utils.py:404-460)
-
-
-def m2po_delta_sq(ppo_kl, adv):
-    """Squared log-ratio of the tokens a clip would act on (ppo_utils.py:426-430): positive advantage with a ratio
-    above one, negative advantage with a ratio below one (margins of 1e-12)."""
-    ratio = (-ppo_kl).exp()
-    harmful = ((adv > 1e-12) & (ratio > 1.0 + 1e-12)) | ((adv < -1e-12) & (ratio < 1.0 - 1e-12))
-    return ppo_kl[harmful].pow(2)
-
-
-def m2po_solve_tau(sorted_delta2, target_sum: float):
-    """(tau, second moment after capping) for ascending ``sorted_delta2`` (ppo_utils.py:404-423): the cap is the
-    largest data value whose capped sum stays below ``target_sum``; the scan runs in Python floats over the fp32
-    values and their fp32 running sum, like the reference's."""
-    n = sorted_delta2.numel()
-    total = float(sorted_delta2.sum().item())
-    if target_sum >= total - 1e-12:
-        return 100000.0, total / n
-    if target_sum <= 1e-12:
-        return 0.0, 0.0
-    values = [float(x) for x in sorted_delta2.tolist()]
-    running = [float(x) for x in torch.cumsum(sorted_delta2, dim=0).tolist()]
-    for k in range(n):
-        above = n - k - 1
-        if (values[k] - 1e-12) * above + running[k] >= target_sum - 1e-12:
-            if k == 0:
-                return 0.0, running[-1] / n
-            after = (values[k - 1] * (above + 1) + running[k - 1]) / n
-            return max(values[k - 1] - 1e-12, 0.0) ** 0.5, after
-    return 100000.0, total / n
-
-
-def m2po_clip_bounds(ppo_kl, adv, kl2_budget: float):
-    """(ratio lower bound, ratio upper bound, M2 before, M2 after) -- kpo_clip_harmful_tokens, ppo_utils.py:433-445."""
-    import math
-
-    d2 = m2po_delta_sq(ppo_kl, adv)
-    n = d2.numel()
-    if n == 0:
-        return 0.0, 100000.0, 0.0, 0.0
-    m2_now = float(d2.sum().detach().item() / n)
-    if m2_now <= kl2_budget + 1e-12:
-        return 0.0, 100000.0, m2_now, m2_now
-    tau, m2_after = m2po_solve_tau(torch.sort(d2)[0], kl2_budget * float(n))
-    return math.exp(-tau), math.exp(tau), m2_now, m2_after
-
-
-def m2po(ppo_kl, adv, kl2_budget: float, miniclip_low: float = 0.3, miniclip_high: float = 0.5):
-    """compute_m2po_loss, ppo_utils.py:448-463: PPO-clip with margins max(adaptive, floor).  Returns
-    (pg_losses, clipfrac, M2 before, M2 after, eps_low, eps_high)."""
-    lo, hi, m2_now, m2_after = m2po_clip_bounds(ppo_kl, adv, kl2_budget)
-    eps_low = max(1.0 - lo, miniclip_low)
-    eps_high = max(hi - 1.0, miniclip_high)
-    ratio = (-ppo_kl).exp()
-    l1 = -adv * ratio
-    l2 = -adv * ratio.clamp(1.0 - eps_low, 1.0 + eps_high)
-    return torch.maximum(l1, l2), (l2 > l1).float(), m2_now, m2_after, eps_low, eps_high

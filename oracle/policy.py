@@ -32,9 +32,6 @@ DEFAULT_ARGS = dict(
     tis_clip_low=0.0,
     sapo_tau_pos=1.0,
     sapo_tau_neg=1.05,
-    m2po_kl2_budget=0.01,
-    m2po_miniclip_low=0.3,
-    m2po_miniclip_high=0.5,
     rollout_temperature=1.0,
     log_probs_chunk_size=-1,
     calculate_per_token_loss=False,
@@ -188,9 +185,6 @@ def policy_loss_function(args, batch, logits, reducer, pg_reducer=None, tis_fn=N
         pg, clipfrac = losses.sapo(ppo_kl, adv, args.sapo_tau_pos, args.sapo_tau_neg)
     elif est == "cispo":
         pg, clipfrac = losses.cispo(lp, ppo_kl, adv, args.eps_clip, args.eps_clip_high)
-    elif est == "m2po":  # :990-993
-        pg, clipfrac, m2_now, m2_after, m2_eps_low, m2_eps_high = losses.m2po(
-            ppo_kl, adv, args.m2po_kl2_budget, args.m2po_miniclip_low, args.m2po_miniclip_high)
     elif est == "rloo":
         pg, clipfrac = losses.rloo_loss(lp, adv)
     else:
@@ -263,10 +257,6 @@ def policy_loss_function(args, batch, logits, reducer, pg_reducer=None, tis_fn=N
             metrics[k] = metric_reducer(v)
     if args.use_opsm:
         metrics["opsm_clipfrac"] = opsm_frac
-    if est == "m2po":  # :1179-1183
-        for key, value in (("ppo_kl_m2_before", m2_now), ("ppo_kl_m2_after", m2_after),
-                           ("m2po_eps_low", m2_eps_low), ("m2po_eps_high", m2_eps_high)):
-            metrics[key] = torch.tensor(value, device=ppo_kl.device).detach()
     return loss, metrics
 
 

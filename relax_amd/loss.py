@@ -30,7 +30,7 @@ from .cp_utils import (PerSampleDivisorReducer, get_cp_local_num_tokens, get_sum
 from .ppo_utils import get_grpo_returns
 
 _SLOT = {k: i for i, k in enumerate(METRIC_SLOTS)}
-GRPO_FAMILY = ("grpo", "gspo", "sapo", "cispo", "m2po", "rloo")
+GRPO_FAMILY = ("grpo", "gspo", "sapo", "cispo", "rloo")
 
 
 def _check_logits(logits: torch.Tensor, args, max_seq_lens=None) -> torch.Tensor:
@@ -435,19 +435,6 @@ class _FusedPolicyLoss(torch.autograd.Function):
         lp_visible = bool(kw.get("lp_requires_grad", False))
         gather_ids = kw.get("gather_topk_ids")
         kw = {k: v for k, v in kw.items() if k not in ("lp_requires_grad", "gather_topk_ids")}
-        m2po = kw.get("m2po")
-        if m2po is not None:
-            # M2PO (loss.py:990-993): the clip margins are solved from this micro-batch's log-ratios, which exist only
-            # now; the PPO-clip kernel then runs with them
-            from .ppo_utils import m2po_clip_margins
-
-            old = kw["old_log_prob"]
-            ppo_kl = old - lp if old is not None else torch.zeros_like(lp)
-            eps_low, eps_high, m2_now, m2_after = m2po_clip_margins(
-                ppo_kl, kw["advantages"], m2po["kl2_budget"], m2po["miniclip_low"], m2po["miniclip_high"])
-            m2po["scalars"] = (m2_now, m2_after, eps_low, eps_high)
-            kw = {k: v for k, v in kw.items() if k != "m2po"}
-            kw["eps_clip"], kw["eps_clip_high"] = eps_low, eps_high
         out = ops.policy_loss(log_prob=lp, entropy=ent, cu_resp=lay.cu_resp, **kw)
         metrics = out["metrics"]
         entropy_grad = kw.get("entropy_coef", 0.0) != 0
@@ -645,8 +632,6 @@ def _single_pass_ok(args, flat, kw, needs_bwd) -> bool:
         return False
     if kw["loss_kind"] == "gspo" or kw["use_opsm"]:
         return False  # sequence-coupled gradients need the per-sequence reduction between forward and backward
-    if kw.get("m2po") is not None:
-        return False  # the clip margins depend on every token's log-prob: they are solved between the two launches
     return True
 
 
@@ -780,9 +765,6 @@ def _composed_policy_loss_function(args: Namespace, batch: dict, logits: torch.T
         pg_loss, pg_clipfrac = PU.compute_cispo_loss(lp, ppo_kl, adv, args.eps_clip, args.eps_clip_high)
     elif est == "rloo":
         pg_loss, pg_clipfrac = PU.compute_rloo_loss(lp, adv)
-    elif est == "m2po":
-        pg_loss, pg_clipfrac, *m2po_scalars = PU.compute_m2po_loss(
-            ppo_kl, adv, args.m2po_kl2_budget, args.m2po_miniclip_low, args.m2po_miniclip_high)
     elif est in ("grpo", "gspo", "ppo") or pp:
         pg_loss, pg_clipfrac = PU.compute_policy_loss(ppo_kl, adv, args.eps_clip, args.eps_clip_high)
     else:
@@ -852,17 +834,7 @@ def _composed_policy_loss_function(args: Namespace, batch: dict, logits: torch.T
             reported[k] = metric_reduce(v)  # over the tokens valid before any rejection (loss.py:1007-1014)
     if getattr(args, "use_opsm", False):
         reported["opsm_clipfrac"] = opsm_clipfrac
-    if est == "m2po":
-        reported.update(_m2po_reported(m2po_scalars, dev))
     return loss, reported
-
-
-_M2PO_KEYS = ("ppo_kl_m2_before", "ppo_kl_m2_after", "m2po_eps_low", "m2po_eps_high")
-
-
-def _m2po_reported(scalars, device) -> dict:
-    """(M2 before, M2 after, eps_low, eps_high) -> the reference's four metric entries (loss.py:1179-1183)."""
-    return {key: torch.tensor(value, device=device).detach() for key, value in zip(_M2PO_KEYS, scalars, strict=True)}
 
 
 def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum_of_sample_mean=None):
@@ -936,9 +908,8 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         sample_denom=None if denom is None else denom.to(device=dev, dtype=torch.float32),
         pg_sample_denom=None if pg_denom is None else pg_denom.to(device=dev, dtype=torch.float32),
         # REINFORCE++ trains with the PPO-clip surrogate; its mask-safe reduction is what the kernel does anyway
-        # M2PO is the PPO-clip surrogate with margins solved per micro-batch (set in _FusedPolicyLoss.forward)
         loss_kind={"grpo": "ppo", "ppo": "ppo", "reinforce_plus_plus": "ppo",
-                   "reinforce_plus_plus_baseline": "ppo", "m2po": "ppo"}.get(est, est),
+                   "reinforce_plus_plus_baseline": "ppo"}.get(est, est),
         kl_kind=args.kl_loss_type if use_kl else None,
         unbiased_kl=bool(getattr(args, "use_unbiased_kl", False)) and use_kl,
         use_opsm=bool(getattr(args, "use_opsm", False)),
@@ -957,9 +928,6 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     )
     if kw["loss_kind"] not in ("ppo", "gspo", "cispo", "rloo", "sapo"):
         raise NotImplementedError(f"advantage_estimator {est} is not supported. ")
-    if est == "m2po":
-        kw["m2po"] = dict(kl2_budget=float(args.m2po_kl2_budget), miniclip_low=float(args.m2po_miniclip_low),
-                          miniclip_high=float(args.m2po_miniclip_high))
     inv_t = 1.0 / float(getattr(args, "rollout_temperature", 1.0))
     if lay.n_tokens == 0:
         loss = 0 * logits.sum()
@@ -967,9 +935,6 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
         metrics = {k: zero.clone() for k in ("loss", "pg_loss", "entropy_loss", "pg_clipfrac", "ppo_kl")}
         if use_kl:
             metrics["kl_loss"] = zero.clone()
-        if est == "m2po":  # no token is harmful: no adaptive clip, the margins are the wide defaults
-            metrics.update(_m2po_reported((0.0, 0.0, max(1.0, kw["m2po"]["miniclip_low"]),
-                                           max(99999.0, kw["m2po"]["miniclip_high"])), dev))
         return loss, metrics
     opd_on = float(getattr(args, "opd_loss_coef", 0.0) or 0.0) != 0.0
     opd_gather = None
@@ -1077,8 +1042,6 @@ def policy_loss_function(args: Namespace, batch: dict, logits: torch.Tensor, sum
     reported.update(opd_reported)
     if kw["use_opsm"]:
         reported["opsm_clipfrac"] = m("opsm_clipfrac")
-    if est == "m2po":
-        reported.update(_m2po_reported(kw["m2po"]["scalars"], dev))
     return loss, reported
 
 
@@ -1215,12 +1178,6 @@ def loss_function(args: Namespace, batch: dict, num_microbatches: int, logits: t
                                use_reentrant=getattr(args, "recompute_loss_function_use_reentrant", True))
     else:
         loss, log = func(args, batch, logits, reducer)
-    if per_token and getattr(args, "advantage_estimator", None) == "m2po":
-        # the M2PO scalars are global, not per-token sums: pre-multiplied so that the logger's division by the token
-        # count gives them back (loss.py:1547-1552)
-        for key in _M2PO_KEYS:
-            if key in log:
-                log[key] = log[key] * num_tokens
     is_dummy = batch.get("__is_dummy__", False)
     explicit = batch.get("__loss_scale__", None)
     gbs = batch.get("dynamic_global_batch_size", getattr(args, "global_batch_size", 1))

@@ -132,77 +132,6 @@ def compute_sapo_loss(ppo_kl, advantages, tau_pos, tau_neg):
     return _TokenLoss.apply("sapo", None, ppo_kl, advantages, 0.2, 0.2, None, tau_pos, tau_neg)
 
 
-# M2PO: second-moment trust region (relax/utils/training/ppo_utils.py:404-463).  The clip margins are two scalars
-# solved from this micro-batch's log-ratios; the loss itself is the PPO-clip kernel run with those margins.
-
-
-def _get_trust_region_delta_sq(ppo_kl: torch.Tensor, advantages: torch.Tensor) -> torch.Tensor:
-    """Squared log-ratio of the tokens a clip would act on (ppo_utils.py:426-430)."""
-    ratio = (-ppo_kl).exp()
-    pos_harmful = (advantages > 1e-12) & (ratio > 1.0 + 1e-12)
-    neg_harmful = (advantages < -1e-12) & (ratio < 1.0 - 1e-12)
-    return ppo_kl[pos_harmful | neg_harmful].pow(2)
-
-
-def _solve_tau_from_sorted_delta2(sorted_delta2: torch.Tensor, target_sum: float) -> tuple[float, float]:
-    """ppo_utils.py:404-423 without its per-element host loop: the reference walks the sorted values in Python floats
-    until ``(d2[k] - 1e-12) * (n - k - 1) + cumsum[k] >= target - 1e-12``; the same test is evaluated for every k at
-    once in float64 on the device (the arithmetic of Python floats), and the first hit and its neighbours come back
-    in one transfer."""
-    n = sorted_delta2.numel()
-    running = torch.cumsum(sorted_delta2, dim=0)
-    total = float(sorted_delta2.sum().item())
-    if target_sum >= total - 1e-12:
-        return 100000.0, total / n
-    if target_sum <= 1e-12:
-        return 0.0, 0.0
-    values64, running64 = sorted_delta2.double(), running.double()
-    above = torch.arange(n - 1, -1, -1, device=sorted_delta2.device, dtype=torch.float64)
-    hit = (values64 - 1e-12) * above + running64 >= target_sum - 1e-12
-    first = torch.argmax(hit.to(torch.int8))  # first True; 0 when there is none (told apart by ``any`` below)
-    before = torch.clamp(first - 1, min=0)
-    any_hit, k, value_before, running_before, running_last = torch.stack(
-        [hit.any().double(), first.double(), values64[before], running64[before], running64[-1]]).tolist()
-    if not any_hit:
-        return 100000.0, total / n
-    k = int(k)
-    if k == 0:
-        return 0.0, running_last / n
-    m2_after = (value_before * (n - k) + running_before) / n
-    return max(value_before - 1e-12, 0.0) ** 0.5, m2_after
-
-
-def kpo_clip_harmful_tokens(ppo_kl: torch.Tensor, advantages: torch.Tensor,
-                            kl2_budget: float) -> tuple[float, float, float, float]:
-    """(ratio lower bound, ratio upper bound, M2 before, M2 after capping), ppo_utils.py:433-445."""
-    import math
-
-    tr_delta_sq = _get_trust_region_delta_sq(ppo_kl.detach(), advantages)
-    n = tr_delta_sq.numel()
-    if n == 0:
-        return 0.0, 100000.0, 0.0, 0.0
-    m2_now = float(tr_delta_sq.sum().item() / n)
-    if m2_now <= kl2_budget + 1e-12:
-        return 0.0, 100000.0, m2_now, m2_now
-    sorted_delta2, _ = torch.sort(tr_delta_sq)
-    tau, m2_after = _solve_tau_from_sorted_delta2(sorted_delta2, kl2_budget * float(n))
-    return math.exp(-tau), math.exp(tau), m2_now, m2_after
-
-
-def m2po_clip_margins(ppo_kl, advantages, kl2_budget: float, miniclip_low: float = 0.3, miniclip_high: float = 0.5):
-    """(eps_low, eps_high, M2 before, M2 after): the adaptive margins, never tighter than the floors
-    (ppo_utils.py:455-457)."""
-    clip_low, clip_high, m2_now, m2_after = kpo_clip_harmful_tokens(ppo_kl, advantages, kl2_budget)
-    return max(1.0 - clip_low, miniclip_low), max(clip_high - 1.0, miniclip_high), m2_now, m2_after
-
-
-def compute_m2po_loss(ppo_kl, advantages, kl2_budget: float, miniclip_low: float = 0.3, miniclip_high: float = 0.5):
-    """ppo_utils.py:448-463: ``(pg_loss, clipfrac, M2_now, M2_after, eps_low, eps_high)``."""
-    eps_low, eps_high, m2_now, m2_after = m2po_clip_margins(ppo_kl, advantages, kl2_budget, miniclip_low, miniclip_high)
-    pg_loss, clipfrac = _TokenLoss.apply("ppo", None, ppo_kl, advantages, eps_low, eps_high, None, 1.0, 1.05)
-    return pg_loss, clipfrac, m2_now, m2_after, eps_low, eps_high
-
-
 class _ApproxKL(torch.autograd.Function):
     @staticmethod
     def forward(ctx, lp, base, kind):

@@ -65,14 +65,6 @@ CASES = {
     "true_on_policy": dict(true_on_policy_mode=True),
     "use_rollout_logprobs": dict(use_rollout_logprobs=True),
     "temperature": dict(rollout_temperature=0.7, entropy_coef=0.01),
-    # M2PO: the batch's squared log-ratios average 38.7 (random logits against old log-probs near -2), so a budget of
-    # 20 makes the solve pick an interior cap; the default budget stops at the first element (floors decide); a huge
-    # one leaves the ratios unclipped
-    "m2po_interior": dict(advantage_estimator="m2po", m2po_kl2_budget=20.0, m2po_miniclip_low=0.01,
-                          m2po_miniclip_high=0.01, use_kl_loss=True, kl_loss_coef=1e-3, kl_loss_type="k3"),
-    "m2po_floors": dict(advantage_estimator="m2po"),
-    "m2po_within_budget": dict(advantage_estimator="m2po", m2po_kl2_budget=1e6, use_tis=True),
-    "m2po_per_token": dict(advantage_estimator="m2po", m2po_kl2_budget=20.0, calculate_per_token_loss=True),
     "reinforce_pp": dict(advantage_estimator="reinforce_plus_plus"),
     "reinforce_pp_baseline_k2": dict(advantage_estimator="reinforce_plus_plus_baseline", use_kl_loss=True,
                                      kl_loss_coef=0.1, kl_loss_type="k2"),
@@ -539,70 +531,6 @@ def test_standalone_token_losses_vs_oracle():
     torch.testing.assert_close(lpd.grad.cpu(), lp.grad, atol=2e-5, rtol=1e-5)
 
 
-@pytest.mark.parametrize("n,scale,budget", [(777, 0.3, 0.02), (5000, 0.5, 0.05), (40, 0.2, 1e-4), (3, 0.4, 0.05),
-                                            (2048, 0.1, 0.5)])
-def test_m2po_margins_and_loss_vs_oracle(n, scale, budget):
-    """The trust-region solve on the device (one sort, one running sum, the reference's stopping test for every
-    element at once in float64) against the oracle's element-by-element scan: same stopping element, hence the same
-    margins; then the per-token loss, clip indicator and gradient of compute_m2po_loss."""
-    from oracle import losses as L
-    from relax_amd import ppo_utils as K
-
-    dev = require_gpu()
-    announce("m2po margins", n, scale, budget)
-    g = torch.Generator().manual_seed(n)
-    kl = torch.randn(n, generator=g) * scale
-    adv = torch.randn(n, generator=g)
-    adv[::7] = 0
-    want_bounds = L.m2po_clip_bounds(kl, adv, budget)
-    got_bounds = K.kpo_clip_harmful_tokens(kl.to(dev), adv.to(dev), budget)
-    for w, got in zip(want_bounds, got_bounds):
-        assert abs(got - w) <= 1e-6 * max(1.0, abs(w)), (want_bounds, got_bounds)
-    d2 = torch.sort(L.m2po_delta_sq(kl, adv))[0]
-    if d2.numel():
-        # (a target within rounding of the total is decided by the summation order of the fp32 total: not probed)
-        for frac in (0.0, 1e-13, 0.3, 0.99, 1.5):
-            target = float(d2.sum()) * frac
-            want = L.m2po_solve_tau(d2, target)
-            got = K._solve_tau_from_sorted_delta2(d2.to(dev), target)
-            assert abs(got[0] - want[0]) <= 1e-7 and abs(got[1] - want[1]) <= 1e-6 * max(1.0, want[1]), (frac, want, got)
-    w = torch.randn(n, generator=g)
-    klc = kl.clone().requires_grad_()
-    kld = kl.to(dev).requires_grad_()
-    want = L.m2po(klc, adv, budget, 0.05, 0.08)
-    got = K.compute_m2po_loss(kld, adv.to(dev), budget, 0.05, 0.08)
-    (want[0] * w).sum().backward()
-    (got[0] * w.to(dev)).sum().backward()
-    torch.testing.assert_close(got[0].detach().cpu(), want[0].detach(), atol=2e-5, rtol=1e-5)
-    assert torch.equal(got[1].cpu(), want[1])
-    torch.testing.assert_close(kld.grad.cpu(), klc.grad, atol=2e-5, rtol=1e-5)
-    for a, b in zip(got[2:], want[2:]):
-        assert isinstance(a, float) and abs(a - b) <= 1e-6 * max(1.0, abs(b))
-
-
-def test_m2po_scalars_survive_the_per_token_logging_division():
-    """loss_function with calculate_per_token_loss: the four M2PO scalars are pre-multiplied by the token count so that
-    the logger's division gives them back (loss.py:1547-1552); the other entries are unchanged."""
-    import relax_amd
-    from relax_amd.loss import loss_function
-
-    dev = require_gpu()
-    announce("m2po per-token logging")
-    tot, resp, v = [9, 6, 12, 7], [4, 3, 7, 5], 264
-    logits, batch = _make_batch(31, tot, resp, v)
-    args = P.make_args(advantage_estimator="m2po", m2po_kl2_budget=30.0, calculate_per_token_loss=True)
-    bd = _to_dev(batch, dev)
-    _, met = relax_amd.policy_loss_function(args, bd, logits.to(dev), None)
-    _, normalizer, log = loss_function(args, bd, 1, logits.to(dev))
-    n_tok = sum(max(float(m.sum()), 1.0) for m in batch["loss_masks"])  # each sample counts at least one token
-    assert float(normalizer) == n_tok
-    values = dict(zip(log["keys"], log["values"][1:].tolist()))
-    for key in ("ppo_kl_m2_before", "ppo_kl_m2_after", "m2po_eps_low", "m2po_eps_high"):
-        assert abs(values[key] / n_tok - met[key].item()) <= 1e-5 * max(1.0, abs(met[key].item())), key
-    assert abs(values["pg_loss"] - met["pg_loss"].item()) <= 1e-5 * max(1.0, abs(met["pg_loss"].item()))
-    assert met["ppo_kl_m2_after"].item() <= 30.0 < met["ppo_kl_m2_before"].item()  # an interior cap was solved
-
-
 @pytest.mark.parametrize("per_token", [False, True])
 def test_value_loss_function_vs_oracle_and_closed_forms(per_token):
     """The critic's loss (``--loss-type value_loss``): value-head output [1, T, 1] sliced to the response rows, clipped
@@ -665,7 +593,7 @@ def test_value_loss_function_vs_oracle_and_closed_forms(per_token):
     assert met4["value_clipfrac"].item() == 0
 
 
-@pytest.mark.parametrize("case", ["ppo_k3_entropy", "gspo", "m2po_interior"])
+@pytest.mark.parametrize("case", ["ppo_k3_entropy", "gspo", "cispo"])
 def test_padded_bshd_layout_equals_packed_layout(case):
     """``qkv_format="bshd"``: logits [B, S, V] padded to S = max_seq_len rows per sample (loss.py:94-117).  The same
     samples laid out packed and padded give the same loss and metrics bit for bit, the same gradient on every real

@@ -212,68 +212,6 @@ def test_sapo_gate_value_at_ratio_one():
     assert abs(loss[0].item() + 2.0) < 1e-6 and abs(loss[1].item() - 2.0 / 1.05) < 1e-6 and cf.sum() == 0
 
 
-# ---- M2PO: the trust-region solve pinned by what the mathematics fixes
-
-
-def _capped_sum(d2, cap):
-    return float(torch.minimum(d2.double(), torch.tensor(cap, dtype=torch.float64)).sum())
-
-
-@pytest.mark.parametrize("seed", range(12))
-def test_m2po_tau_is_the_largest_data_cap_below_budget_bruteforce(seed):
-    """Water-filling by enumeration: among the data values, tau^2 is the largest one whose capped sum
-    sum_t min(d_t^2, cap) stays below n * budget (zero when even the smallest is too much), and the reported second
-    moment after capping is that capped sum / n.  Budgets are drawn away from the 1e-12 tie margins."""
-    from oracle import losses as L
-
-    g = torch.Generator().manual_seed(seed)
-    n = int(torch.randint(2, 40, (1,), generator=g))
-    d2 = torch.sort((torch.randn(n, generator=g) * 0.7).pow(2))[0]
-    total = float(d2.sum())
-    target = total * float(torch.rand(1, generator=g).clamp(0.05, 0.95))
-    tau, after = L.m2po_solve_tau(d2, target)
-    caps = [float(x) for x in d2.tolist()]
-    feasible = [c for c in caps if _capped_sum(d2, c) < target - 1e-9]
-    want_cap = max(feasible) if feasible else None
-    if want_cap is None:
-        assert tau == 0.0 and abs(after - total / n) < 1e-6  # the reference reports the uncapped moment here
-    else:
-        assert abs(tau ** 2 - want_cap) < 1e-9
-        assert abs(after - _capped_sum(d2, want_cap) / n) < 1e-6
-        assert after <= target / n + 1e-9
-        bigger = [c for c in caps if c > want_cap]
-        assert not bigger or _capped_sum(d2, min(bigger)) >= target - 1e-9  # the next cap would overshoot
-
-
-def test_m2po_special_cases():
-    """Closed forms: no harmful token -> no clip; below the budget -> no clip and M2 unchanged; all deviations equal
-    and over budget -> the scan stops at its first element (tau 0: every ratio clipped to 1, floors decide the
-    margins); the harmful set is sign(advantage) * (ratio - 1) > 0; the loss is PPO-clip with the solved margins."""
-    import math
-
-    from oracle import losses as L
-
-    kl = torch.tensor([-0.5, 0.5, -0.2, 0.3, 0.0, -0.4])
-    adv = torch.tensor([1.0, 1.0, -1.0, -1.0, 2.0, 0.0])
-    # ratio = exp(-kl) > 1 <=> kl < 0: harmful are (A>0, kl<0) = token 0 and (A<0, kl>0) = token 3
-    torch.testing.assert_close(L.m2po_delta_sq(kl, adv), torch.tensor([0.25, 0.09]))
-    assert L.m2po_clip_bounds(torch.zeros(4), torch.ones(4), 0.01) == (0.0, 100000.0, 0.0, 0.0)
-    lo, hi, now, after = L.m2po_clip_bounds(kl, adv, 0.2)  # M2 = 0.17 <= 0.2
-    assert (lo, hi) == (0.0, 100000.0) and abs(now - 0.17) < 1e-7 and after == now
-    lo, hi, now, after = L.m2po_clip_bounds(kl, adv, 0.1)  # target 0.2: cap 0.09 gives 0.18 < 0.2, cap 0.25 gives 0.34
-    assert abs(lo - math.exp(-0.3)) < 1e-6 and abs(hi - math.exp(0.3)) < 1e-6 and abs(after - 0.09) < 1e-7
-    same = torch.full((5,), -0.3)
-    lo, hi, now, after = L.m2po_clip_bounds(same, torch.ones(5), 0.01)
-    assert (lo, hi) == (1.0, 1.0) and abs(now - 0.09) < 1e-7
-    pg, frac, _now, _after, eps_low, eps_high = L.m2po(kl, adv, 0.1, miniclip_low=0.05, miniclip_high=0.05)
-    assert abs(eps_low - (1 - math.exp(-0.3))) < 1e-6 and abs(eps_high - (math.exp(0.3) - 1)) < 1e-6
-    want, want_frac = L.policy_clip(kl, adv, eps_low, eps_high)
-    torch.testing.assert_close(pg, want)
-    assert torch.equal(frac, want_frac)
-    _pg, _frac, _n, _a, eps_low, eps_high = L.m2po(kl, adv, 0.1)  # default floors 0.3 / 0.5 win over 0.26 / 0.35
-    assert (eps_low, eps_high) == (0.3, 0.5)
-
-
 def test_value_loss_hand_computed():
     """Clipped value loss, worked by hand for clip 0.5 and old values 0: (v, R) = (1, 0) -> clipped to 0.5, max(0.25, 1)
     = 1, counted as clipped; (0.2, 0) -> 0.04, not clipped; (1, 2) -> max((0.5 - 2)^2, (1 - 2)^2) = 2.25, clipped.
