@@ -36,6 +36,19 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 PEAK_SCLK_MHZ = 2400.0  # the shader clock the published matrix-core peak is quoted at
 METRIC = "tokens/s fused logprob+entropy+loss fwd+bwd @V=151936 bf16; % HBM/MFMA peak"
 PROFILES_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles")
+KERNEL_CHOICE = "auto"  # --kernel-choice, as handed to relax_amd_set_kernel_choice
+
+
+def known_size_copy(dev) -> None:
+    """One untimed plain device copy of 1 GiB (reads 1 GiB, writes 1 GiB) before the timed region: under
+    ``rocprofv3 --pmc FETCH_SIZE`` / ``WRITE_SIZE`` its dispatch is the known-size reference that the counters of the
+    step's kernels are scaled by."""
+    src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).fill_(1.0)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
 
 
 def measured_traffic(kernel: str, rows: int, vocab: int):
@@ -90,7 +103,7 @@ def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
     threads = 1024 if nvec >= 7168 else 512 if nvec >= 2048 else 256
     shape = (nvec // width, nvec % width != 0)
     if vocab % per_vec == 0 and threads == width and shape in shapes \
-            and os.environ.get("RELAX_AMD_FUSED_STEP_KERNEL") != "cached":
+            and KERNEL_CHOICE != "two_walk":
         return f"actor_step_resident_kernel<{dtype}, {shape[0]}, {str(shape[1]).lower()}>"
     return f"actor_step_fused_kernel<{dtype}, true, {threads}>"
 
@@ -109,7 +122,7 @@ def kl_step_kernel_name(vocab: int) -> str:
     nvec = vocab // 8
     shape = (nvec // 1024, nvec % 1024 != 0)
     if vocab % 8 == 0 and shape in ((20, False), (19, True), (18, True), (15, True), (16, False), (12, True)) \
-            and os.environ.get("RELAX_AMD_FUSED_STEP_KERNEL") != "cached":
+            and KERNEL_CHOICE != "two_walk":
         return f"reverse_kl_resident_kernel<bf16_t, {shape[0]}, {str(shape[1]).lower()}>"
     return f"reverse_kl_step_kernel<bf16_t, true, {1024 if nvec >= 2048 else 256}>"
 
@@ -327,13 +340,7 @@ def run_actor_step(a, dev) -> None:
         loss.backward()
         return loss
 
-    if a.calibrate_copy:
-        src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).fill_(1.0)
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
-        torch.cuda.synchronize()
-        del src, dst
+    known_size_copy(dev)
     wall, kernel_ms, _, loss = timed_steps(step, a.warmup, a.steps)
     ms_per_step = wall * 1e3 / a.steps
     row_bytes = float(a.vocab * logits.element_size())
@@ -368,26 +375,13 @@ def run_lmhead(a, dev) -> None:
     tokens = torch.randint(0, v, (n,), device=dev, generator=g)
     adv = torch.randn(n, device=dev, generator=g) / n
 
-    if a.lmhead_operands == "zeros":  # diagnostic: same kernels and addresses, no switching activity in the operands
-        with torch.no_grad():
-            hidden.zero_()
-            weight.zero_()
-
-    vendor_out = torch.empty((min(n, 8192), v), dtype=torch.bfloat16, device=dev) if a.vendor_gemm else None
-
     def surrogate(begin, end, lp, _ent):  # PPO's surrogate at ratio 1 (old log-probs = current ones): -A * lp
         return -(adv[begin:end] * lp).sum()
 
     def step():
         hidden.grad = None
         weight.grad = None
-        if a.vendor_gemm:  # diagnostic: the library's plain GEMM of the same shape, logits written, 8192 rows at a time
-            from relax_amd import ops
-            with torch.no_grad(), ops._timed("lmhead_logprob_fwd"):
-                for s0 in range(0, n, 8192):
-                    torch.matmul(hidden[s0:s0 + 8192], weight.t(), out=vendor_out[: min(n, s0 + 8192) - s0])
-            return vendor_out[0, 0].float()
-        if a.forward_only:  # diagnostic: the clock / power samples then belong to the forward kernel alone
+        if a.forward_only:  # the clock / power samples then belong to the forward kernel alone
             with torch.no_grad():
                 lp, ent = lm_head_log_probs_and_entropy(hidden, weight, tokens, 1.0, True, False)
             return -(adv * lp).sum()
@@ -417,14 +411,11 @@ def run_lmhead(a, dev) -> None:
          + ("(bf16 logits kept for the backward pass)" if a.keep_logits else
             "(no logits in HBM; backward projects a second time)" if a.two_projections else
             f"(logits of {min(n, a.lmhead_slab)} rows at a time become their gradient in place)")
-         + (" only [diagnostic]" if a.forward_only else " + bwd to dhidden/dweight from a scalar loss")
-         + (" [diagnostic: all-zero operands]" if a.lmhead_operands == "zeros" else "")
-         + (" [diagnostic: NOT the fused kernel -- hipBLASLt GEMM of the forward shape, logits written]"
-            if a.vendor_gemm else ""),
+         + (" only" if a.forward_only else " + bwd to dhidden/dweight from a scalar loss"),
          {"rows": n, "hidden": h, "vocab": v, "keep_logits": bool(a.keep_logits),
           "two_projections": bool(a.two_projections), "slab_rows": int(min(n, a.lmhead_slab)),
           "loss": float(loss.item())},
-         {"bound": "mfma", "kernel": "hipBLASLt GEMM (diagnostic)" if a.vendor_gemm else "lmhead_fwd_kernel",
+         {"bound": "mfma", "kernel": "lmhead_fwd_kernel",
           "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
           "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
           "algorithmic_flops_per_launch": flops, "avg_launch_ms": dom, "kernel_ms": kernel_ms,
@@ -436,145 +427,10 @@ def run_lmhead(a, dev) -> None:
          None)
 
 
-def load_ceilings():
-    """(library, check) of the benchmark's own measurement kernels, relax_amd/libceilings.so (built by
-    relax_amd/build.py next to the product library, which does not contain them)."""
-    import ctypes as C
-
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "relax_amd", "libceilings.so")
-    if not os.path.exists(path):
-        raise RuntimeError(f"{path} is missing: run python relax_amd/build.py")
-    lib = C.CDLL(path)
-    lib.ceiling_mfma_loop.restype = C.c_int
-    lib.ceiling_mfma_loop.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
-    lib.ceiling_stream.restype = C.c_int
-    lib.ceiling_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
-    lib.ceiling_row_copy.restype = C.c_int
-    lib.ceiling_row_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_void_p]
-    lib.ceiling_burst_copy.restype = C.c_int
-    lib.ceiling_burst_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int,
-                                       C.c_void_p, C.c_void_p]
-
-    def check(rc):
-        if rc != 0:
-            raise RuntimeError(f"measurement kernel failed: code {rc}")
-
-    return lib, check
-
-
-def run_mfma_ceiling(a, dev) -> None:
-    """Diagnostic, not a workload of the path: bf16 32x32x16 MFMAs on register-resident N(0, 1) operand fragments, one
-    wave per SIMD on every CU, no memory traffic.  What this sustains under the board's power limit is the practical
-    ceiling for the LM-head kernels on this box.  A "step" is one launch of 256 workgroups x 20000 iterations."""
-    import ctypes as C
-    from relax_amd import ops
-
-    lib, check = load_ceilings()
-    shape = 1 if a.mfma_shape == "16x16x32" else 0
-    blocks, iters = 256, (10000 if shape else 20000)  # the same FLOP per launch for both shapes
-    g = torch.Generator(device=dev).manual_seed(0)
-    src = torch.randn(4096 * 8, device=dev, generator=g).bfloat16()
-    if a.lmhead_operands == "zeros":
-        src.zero_()
-    out = torch.empty(blocks * 512, dtype=torch.float32, device=dev)
-    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-
-    def step():
-        with ops._timed("diag_mfma_loop"):
-            check(lib.ceiling_mfma_loop(C.c_void_p(src.data_ptr()), C.c_void_p(out.data_ptr()), blocks, iters,
-                                               shape, stream))
-        return out
-
-    with ClockSampler() as clock:
-        wall, kernel_ms, launches, _ = timed_steps(step, a.warmup, a.steps)
-    clk = clock.summary()
-    flops = blocks * (8 * iters * 128 * 16384.0 if shape else 4 * iters * 64 * 32768.0)
-    achieved = flops / (kernel_ms["diag_mfma_loop"] * 1e-3) / 1e12
-    print(json.dumps({
-        "metric": "TFLOP/s of register-fed bf16 MFMAs [diagnostic ceiling, not the headline metric]", "value": achieved,
-        "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": wall * 1e3 / a.steps,
-        "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "mfma_ceiling: 256 workgroups x "
-                               + ("8 waves (two per SIMD) x 10000 x 128 MFMA 16x16x32" if shape else
-                                  "4 waves (one per SIMD) x 20000 x 64 MFMA 32x32x16") + " bf16, operands "
-                               + ("all zero" if a.lmhead_operands == "zeros" else "N(0, 1)") + ", no memory traffic"},
-        "roofline": {"bound": "mfma", "kernel": "diag_mfma_loop16_kernel" if shape else "diag_mfma_loop_kernel",
-                     "achieved": achieved,
-                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "avg_launch_ms": kernel_ms["diag_mfma_loop"], "clock": clk,
-                     "frac_at_measured_clock":
-                         (achieved / (MFMA_BF16_PEAK_TFLOPS * clk["sclk_mhz"] / PEAK_SCLK_MHZ)) if clk else None},
-        "cpu_baseline": None}))
-
-
-def run_hbm_ceiling(a, dev) -> None:
-    """Diagnostic, not a workload of the path: plain read / write / copy streams over a buffer of the actor step's
-    logits size (65536 x 151936 bf16 = 19.9 GB), 16-byte accesses, and the same copy in the burst form of the
-    register-resident kernels (persistent workgroups, a row in by one run of loads, out by one run of stores) on the
-    rows of the two actor-step shapes, in the workgroup arrangements that were compared for them and with the grid's
-    workgroups kept in step.  What these sustain is the practical ceiling for the bandwidth-bound kernels on this box.
-    A "step" is one launch of each."""
-    import ctypes as C
-    from relax_amd import ops
-
-    lib, check = load_ceilings()
-    nbytes = 65536 * 151936 * 2
-    src = torch.ones(nbytes // 2, dtype=torch.bfloat16, device=dev)
-    dst = torch.empty_like(src)
-    sink = torch.zeros(4, dtype=torch.int32, device=dev)
-    phases = torch.zeros(4, dtype=torch.int32, device=dev)
-    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    p = lambda t: C.c_void_p(t.data_ptr())
-    bf16_rows, f32_rows = (65536, 151936 * 2), (131072, 32000 * 4)  # (rows, bytes per row) of cfg2 and cfg1
-    # name -> (rows, threads per workgroup, workgroups per CU, kept in step)
-    bursts = {"burst_copy_bf16_rows": (bf16_rows, 1024, 1, 0), "burst_copy_bf16_rows_in_step": (bf16_rows, 1024, 1, 1),
-              "burst_copy_f32_rows_1024x1": (f32_rows, 1024, 1, 0), "burst_copy_f32_rows_512x2": (f32_rows, 512, 2, 0),
-              "burst_copy_f32_rows_1024x2": (f32_rows, 1024, 2, 0), "burst_copy_f32_rows_in_step": (f32_rows, 1024, 1, 1)}
-
-    def step():
-        for mode, name in ((0, "diag_stream_read"), (1, "diag_stream_write"), (2, "diag_stream_copy")):
-            with ops._timed(name):
-                check(lib.ceiling_stream(mode, p(src), p(dst), nbytes, p(sink), stream))
-        with ops._timed("diag_row_copy"):  # the same copy, one persistent workgroup per CU walking whole rows
-            check(lib.ceiling_row_copy(p(src), p(dst), 65536, 151936 * 2, 256, stream))
-        for name, ((rows, row_bytes), threads, per_cu, in_step) in bursts.items():
-            if in_step:
-                phases.zero_()
-            with ops._timed(name):
-                check(lib.ceiling_burst_copy(p(src), p(dst), rows, row_bytes, threads, per_cu, in_step, p(phases),
-                                             stream))
-        with ops._timed("memset"):
-            dst.view(torch.int32).zero_()
-        return dst
-
-    wall, kernel_ms, launches, _ = timed_steps(step, a.warmup, a.steps)
-    rates = {"read_GBs": nbytes / kernel_ms["diag_stream_read"] / 1e6,
-             "write_GBs": nbytes / kernel_ms["diag_stream_write"] / 1e6,
-             "copy_GBs": 2 * nbytes / kernel_ms["diag_stream_copy"] / 1e6,
-             "row_copy_GBs": 2 * nbytes / kernel_ms["diag_row_copy"] / 1e6,
-             "torch_zero_fill_GBs": nbytes / kernel_ms["memset"] / 1e6}
-    for name, ((rows, row_bytes), *_rest) in bursts.items():
-        rates[name + "_GBs"] = 2 * rows * row_bytes / kernel_ms[name] / 1e6
-    rates["in_step_waits_given_up"] = int(phases[2].item())  # of the last launch kept in step; 0 = it ran as meant
-    print(json.dumps({
-        "metric": "GB/s of plain HBM streams [diagnostic ceiling, not the headline metric]", "value": rates["read_GBs"],
-        "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": wall * 1e3 / a.steps,
-        "higher_is_better": True, "dtype": "u8", "data": "synthetic",
-        "config": {"workload": "hbm_ceiling: read, write, copy, row-wise copy (65536 rows of 303872 bytes, 256 persistent "
-                               "workgroups) and zero fill of 19.9 GB with 16-byte accesses; burst-form copies of the "
-                               "65536 x 303872-byte and 131072 x 128000-byte rows (threads x workgroups per CU; "
-                               "in_step = the grid's workgroups aligned turn by turn)", **rates},
-        "roofline": {"bound": "hbm", "kernel": "diag_stream_kernel<0> (read)", "achieved": rates["read_GBs"],
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": rates["read_GBs"] / HBM_PEAK_GBS, "traffic": None,
-                     "kernel_ms": kernel_ms},
-        "cpu_baseline": None}))
-
-
 def run_actor_fwd_topk(a, dev) -> None:
     """The forward-only pass the actor runs when it also collects the student's top-K ids for on-policy distillation
     (compute_log_prob(collect_topk=True)): log-probs + entropy and ``topk_token_ids`` of every response row of the
-    actor-step logits, no gradient.  ``--vendor-topk`` times torch.topk on the same rows instead of the library's
-    selection kernel (the rest of the pass unchanged)."""
+    actor-step logits, no gradient."""
     import relax_amd
     from relax_amd import ops
 
@@ -582,8 +438,6 @@ def run_actor_fwd_topk(a, dev) -> None:
     args.opd_log_prob_top_k = a.topk
     logits, batch, _ = make_workload(dev, a.seqs, a.seq_len, a.vocab)
     n_tokens = a.seqs * a.seq_len
-    if a.vendor_topk:
-        ops.TOPK_ROWS_MAX_K = 0  # get_log_probs_and_entropy then selects with torch.topk, sample by sample
 
     def step():
         with torch.no_grad():
@@ -604,7 +458,7 @@ def run_actor_fwd_topk(a, dev) -> None:
         dom, dom_name = kernel_ms["logprob_entropy_fwd"], "logprob_entropy_fwd_kernel<bf16_t, true, 1024>"
     emit(a, n_tokens, wall,
          f"actor forward-only pass with student top-{a.topk} ids: {a.seqs} seqs x {a.seq_len} tokens x V={a.vocab} bf16 "
-         f"logits, log-prob + entropy + top-K selection" + (" [torch.topk selection]" if a.vendor_topk else ""),
+         f"logits, log-prob + entropy + top-K selection",
          {"rows": n_tokens, "vocab": a.vocab, "k": a.topk},
          hbm_roofline(dom_name, dom, row_bytes, n_tokens, a.vocab, kernel_ms, wall * 1e3 / a.steps), None)
 
@@ -816,8 +670,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="actor_step",
                     choices=["actor_step", "actor_step_opd_topk", "cfg1", "lmhead", "reverse_kl", "varlen_gspo",
-                             "varlen_cispo", "actor_fwd_topk",
-                             "mfma_ceiling", "hbm_ceiling"])
+                             "varlen_cispo", "actor_fwd_topk"])
     ap.add_argument("--seqs", type=int, default=SEQS)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
     ap.add_argument("--vocab", type=int, default=VOCAB)
@@ -832,17 +685,8 @@ def main() -> int:
     ap.add_argument("--lmhead-slab", type=int, default=8192,
                     help="lmhead: rows of logits that exist in HBM at a time in the one-projection step")
     ap.add_argument("--forward-only", action="store_true",
-                    help="lmhead workload, diagnostic: time the forward pass alone (clock samples of that kernel only)")
-    ap.add_argument("--mfma-shape", choices=["32x32x16", "16x16x32"], default="32x32x16",
-                    help="mfma_ceiling workload: instruction shape (16x16x32 runs two waves per SIMD)")
-    ap.add_argument("--vendor-gemm", action="store_true",
-                    help="lmhead workload, diagnostic: time the library's plain GEMM of the forward shape instead of "
-                         "the fused kernel (same operands, logits written to HBM), for comparison")
-    ap.add_argument("--lmhead-operands", choices=["random", "zeros"], default="random",
-                    help="lmhead workload, diagnostic: all-zero operands show the kernel without the board power limit")
+                    help="lmhead workload: time the forward pass alone (clock samples of that kernel only)")
     ap.add_argument("--topk", type=int, default=64, help="k of the actor_fwd_topk workload")
-    ap.add_argument("--vendor-topk", action="store_true",
-                    help="actor_fwd_topk: select with torch.topk instead of the library's kernel (comparison)")
     ap.add_argument("--two-launch", action="store_true",
                     help="use the separate forward / backward launches (the path GSPO takes) instead of the fused step")
     ap.add_argument("--opd-topk", type=int, default=0,
@@ -850,8 +694,9 @@ def main() -> int:
     ap.add_argument("--no-secondary", action="store_true",
                     help="plain invocation only: skip the other configurations that otherwise run after the headline "
                          "workload and ride along in its line as other_workloads")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also launch one plain 1 GiB device copy, the known-size reference for FETCH_SIZE/WRITE_SIZE")
+    ap.add_argument("--kernel-choice", choices=["auto", "two_walk", "resident"], default="auto",
+                    help="relax_amd_set_kernel_choice: which of the two bit-identical kernels the fused entry points "
+                         "launch (two_walk = the row-per-workgroup kernels for every row length)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (token rows shard without any exchange). "
@@ -861,6 +706,11 @@ def main() -> int:
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         return 2
     import relax_amd  # noqa: F401  (fails loudly when the HIP library is missing)
+    from relax_amd import ops
+
+    global KERNEL_CHOICE
+    KERNEL_CHOICE = a.kernel_choice
+    ops.set_kernel_choice(a.kernel_choice)
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -881,10 +731,6 @@ def run_workload(a, dev) -> None:
         run_cfg1(a, dev)
     elif a.workload == "lmhead":
         run_lmhead(a, dev)
-    elif a.workload == "mfma_ceiling":
-        run_mfma_ceiling(a, dev)
-    elif a.workload == "hbm_ceiling":
-        run_hbm_ceiling(a, dev)
     elif a.workload == "reverse_kl":
         run_reverse_kl(a, dev)
     elif a.workload == "actor_fwd_topk":

@@ -27,7 +27,10 @@
 extern "C" {
 #endif
 
-#define RELAX_AMD_ABI_VERSION 1
+/* 2: relax_amd_policy_loss_args starts with its own size and carries the top-K distillation block and
+ *    read_masked_rows; relax_amd_set_kernel_choice replaces the environment switch; relax_amd_transpose_16bit,
+ *    relax_amd_diag_mfma_loop and relax_amd_diag_stream are gone.  A client built against version 1 must be rebuilt. */
+#define RELAX_AMD_ABI_VERSION 2
 
 enum { RELAX_AMD_F32 = 0, RELAX_AMD_BF16 = 1, RELAX_AMD_F16 = 2, RELAX_AMD_F64 = 3 };
 
@@ -68,6 +71,19 @@ enum {
 int relax_amd_version(void);
 /* Message of the last failing call on this thread ("" if none). Host pointer, valid until the next call. */
 const char* relax_amd_last_error(void);
+
+/* which of two bit-identical kernels the fused entry points launch (see relax_amd_set_kernel_choice) */
+enum { RELAX_AMD_KERNEL_AUTO = 0, RELAX_AMD_KERNEL_TWO_WALK = 1, RELAX_AMD_KERNEL_RESIDENT = 2 };
+/*
+ * relax_amd_actor_step_fused, relax_amd_logprob_entropy_bwd and relax_amd_reverse_kl_step_fused each hold a
+ * register-resident kernel for the row lengths it is built for and a two-walk (row-per-workgroup) kernel for every
+ * row length; both give the same bits.  AUTO (the default) takes the resident one where it exists.  TWO_WALK keeps
+ * every row on the two-walk kernel; RESIDENT makes those entry points fail with RELAX_AMD_EUNSUPPORTED where no
+ * resident kernel is built, so that a comparison of the two cannot pass on one kernel compared with itself.
+ * Process-wide, read atomically at each launch; returns the previous choice, or RELAX_AMD_EINVAL.  No counterpart
+ * in the reference: it exists for tests and measurements.
+ */
+int relax_amd_set_kernel_choice(int choice);
 
 /*
  * Target-token log-prob and full-vocab entropy of each row, one streaming
@@ -142,6 +158,10 @@ int relax_amd_gather_targets(const int64_t* tokens, const int64_t* src_begin, co
  * reducers of get_sum_of_sample_mean (relax/backends/megatron/cp_utils.py:144-162).
  */
 typedef struct relax_amd_policy_loss_args {
+  /* sizeof(relax_amd_policy_loss_args) as the caller was compiled; a smaller value than the library's own is
+     refused with RELAX_AMD_EINVAL before any field behind it is read */
+  uint32_t struct_size;
+  uint32_t reserved;             /* 0 */
   /* packed per-token inputs, fp32 [n_tokens]; NULL where marked optional */
   const float* log_prob;
   const float* old_log_prob;     /* NULL: old = current (true on-policy, ratio == 1) */
@@ -303,7 +323,7 @@ int relax_amd_reverse_kl_bwd(const void* student, const void* teacher, int dtype
  * HBM moves 3*V*s bytes per token instead of 5*V*s.  Two kernels sit behind it, with bit-identical results: 16-bit
  * rows of the built vocabulary shapes (12 / 15 / 18 / 19 full 16-byte vectors per thread of a 1024-thread workgroup
  * plus a partial one, or 16 / 20 exactly) keep the student row in registers and stream the teacher row past it twice; other
- * rows, and every row when RELAX_AMD_FUSED_STEP_KERNEL=cached is in the environment, walk both rows twice.
+ * rows, and every row after relax_amd_set_kernel_choice(RELAX_AMD_KERNEL_TWO_WALK), walk both rows twice.
  */
 int relax_amd_reverse_kl_step_fused(const void* student, const void* teacher, int dtype, int64_t n_tokens,
                                     int64_t vocab, int64_t row_stride, const float* g, float grad_scale, float* kl,
@@ -429,7 +449,7 @@ int relax_amd_logprob_entropy_topk_fwd(const void* logits, int dtype, int64_t n_
  * argument block); the caller adds the K one-hot parts of its gradient with relax_amd_sparse_row_add afterwards.
  * Two kernels sit behind this entry point and are chosen by row length and element type: a register-resident one
  * (one read and one write of HBM per row; 16-bit rows of 57352 .. 65536 and 100352 .. 163840 entries, fp32 rows of
- * 28676 .. 32768, 49156 .. 53248 and 61444 .. 65536 entries, in the built shapes) and a two-walk one for everything else; RELAX_AMD_FUSED_STEP_KERNEL=cached in the environment
+ * 28676 .. 32768, 49156 .. 53248 and 61444 .. 65536 entries, in the built shapes) and a two-walk one for everything else; relax_amd_set_kernel_choice(RELAX_AMD_KERNEL_TWO_WALK)
  * forces the latter.  Same results.
  */
 int relax_amd_actor_step_fused(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,

@@ -39,6 +39,7 @@ class PolicyLossArgs(C.Structure):
     """Mirror of ``relax_amd_policy_loss_args``."""
 
     _fields_ = [
+        ("struct_size", C.c_uint32), ("reserved", C.c_uint32),
         ("log_prob", _vp), ("old_log_prob", _vp), ("ref_log_prob", _vp), ("train_log_prob", _vp),
         ("rollout_log_prob", _vp), ("advantages", _vp), ("loss_mask", _vp), ("pg_loss_mask", _vp), ("entropy", _vp),
         ("cu_resp", _vp), ("sample_denom", _vp), ("pg_sample_denom", _vp),
@@ -59,12 +60,21 @@ class PolicyLossArgs(C.Structure):
     ]
 
 
+def new_policy_loss_args() -> PolicyLossArgs:
+    """A zeroed argument block with ``struct_size`` filled in (the library refuses a block without it)."""
+    a = PolicyLossArgs()
+    a.struct_size = C.sizeof(PolicyLossArgs)
+    return a
+
+
 FUSED_TOPK_MAX = 256
+KERNEL_CHOICES = {"auto": 0, "two_walk": 1, "resident": 2}
 
 
 SIGNATURES = {
     "relax_amd_version": (C.c_int, []),
     "relax_amd_last_error": (C.c_char_p, []),
+    "relax_amd_set_kernel_choice": (C.c_int, [C.c_int]),
     "relax_amd_logprob_entropy_fwd": (C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp]),
     "relax_amd_logprob_entropy_bwd": (
         C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _f32, _vp, _i64, _vp]),

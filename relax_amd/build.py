@@ -73,24 +73,7 @@ def build(verbose: bool = True) -> str:
     if verbose:
         print(f"built {LIB_PATH} from {len(srcs)} sources")
     build_abi_client(verbose)
-    build_ceilings(verbose)
     return LIB_PATH
-
-
-CEILINGS_SRC = os.path.join(CSRC, "measure", "ceilings.hip")
-CEILINGS_LIB = os.path.join(HERE, "libceilings.so")
-
-
-def build_ceilings(verbose: bool = True) -> str:
-    """The benchmark's own measurement kernels (plain HBM streams, register-fed MFMA loop): a separate small library
-    that the product library neither contains nor links, loaded by bench.py only."""
-    cmd = [HIPCC, *FLAGS, "-shared", CEILINGS_SRC, "-o", CEILINGS_LIB]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed for {CEILINGS_SRC}:\n{r.stdout}\n{r.stderr}")
-    if verbose:
-        print(f"built {CEILINGS_LIB}")
-    return CEILINGS_LIB
 
 
 ABI_CLIENT_SRC = os.path.join(os.path.dirname(HERE), "tests", "abi_client.c")

@@ -205,16 +205,6 @@ __global__ __launch_bounds__(THREADS) void actor_step_fused_kernel(
   }
 }
 
-// RELAX_AMD_FUSED_STEP_KERNEL = "cached" forces the two-walk kernel (second walk out of cache); "resident" insists on
-// the register-resident one and makes the call fail for rows it is not built for (so that a comparison of the two
-// cannot pass on one kernel compared with itself); unset or anything else lets the row lengths the register-resident
-// kernel is built for take that one and all others the two-walk kernel.  Read at every launch; meant for measurements
-// and tests.
-static bool fused_step_kernel_is(const char* name) {
-  const char* e = getenv("RELAX_AMD_FUSED_STEP_KERNEL");
-  return e && strcmp(e, name) == 0;
-}
-
 static int device_compute_units() {
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess ||
@@ -233,13 +223,16 @@ static int dispatch_fused(const void* logits, int64_t n_rows, int64_t vocab, int
   const T* x = static_cast<const T*>(logits);
   T* d = static_cast<T*>(dlogits);
   dim3 grid(static_cast<unsigned>(n_rows));
-  if (vec && !fused_step_kernel_is("cached")) {
+  // relax_amd_set_kernel_choice: TWO_WALK keeps every row on the two-walk kernel (second walk out of cache); RESIDENT
+  // fails for rows the register-resident kernel is not built for
+  const int choice = kernel_choice();
+  if (vec && choice != RELAX_AMD_KERNEL_TWO_WALK) {
     const int rc = launch_actor_step_resident<T>(x, stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t, a,
                                                  grad_scale, lp, ent, lse, spx, d, d_stride, device_compute_units(), s);
     if (rc != RELAX_AMD_EUNSUPPORTED) return rc;  // launched (or failed to): otherwise the row length is not built
   }
-  if (fused_step_kernel_is("resident")) {
-    set_error("actor_step_fused: RELAX_AMD_FUSED_STEP_KERNEL=resident, but no register-resident kernel is built for "
+  if (choice == RELAX_AMD_KERNEL_RESIDENT) {
+    set_error("actor_step_fused: kernel choice RESIDENT, but no register-resident kernel is built for "
               "rows of %lld elements of this type and alignment", (long long)vocab);
     return RELAX_AMD_EUNSUPPORTED;
   }
@@ -274,6 +267,10 @@ extern "C" int relax_amd_actor_step_fused(const void* logits, int dtype, int64_t
     return RELAX_AMD_EINVAL;
   }
   if (n_rows == 0) return RELAX_AMD_OK;
+  if (loss && policy_loss_args_size_error(loss)) {
+    set_error("actor_step_fused: %s", policy_loss_args_size_error(loss));
+    return RELAX_AMD_EINVAL;
+  }
   if (!logits || !targets || !loss || !log_prob || !entropy || !lse || !spx || !dlogits || !loss->advantages ||
       !loss->loss_mask || !loss->coef_log_prob) {
     set_error("actor_step_fused: NULL argument");

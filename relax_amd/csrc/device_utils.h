@@ -228,6 +228,8 @@ __device__ __forceinline__ F block_sum(F v, F* scratch) {
 // ---- host side ------------------------------------------------------------------------------------------------
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);
+// RELAX_AMD_KERNEL_* as last set through relax_amd_set_kernel_choice (one relaxed atomic load)
+int kernel_choice();
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -180,11 +180,11 @@ static int launch_bwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t
   dim3 grid(static_cast<unsigned>(n_rows)), block(kRowThreads);
   const T* x = static_cast<const T*>(logits);
   T* d = static_cast<T*>(dlogits);
-  // Long rows of the built shapes take the persistent burst form (same bits, faster).  RELAX_AMD_FUSED_STEP_KERNEL =
-  // "cached" keeps every row length on the row-per-workgroup kernel, "resident" fails where the burst form is not
-  // built (for tests that compare the two); read at every launch.
-  const char* forced = getenv("RELAX_AMD_FUSED_STEP_KERNEL");
-  if (vec && !(forced && strcmp(forced, "cached") == 0)) {
+  // Long rows of the built shapes take the persistent burst form (same bits, faster).  relax_amd_set_kernel_choice:
+  // TWO_WALK keeps every row length on the row-per-workgroup kernel, RESIDENT fails where the burst form is not
+  // built (for tests that compare the two).
+  const int choice = kernel_choice();
+  if (vec && choice != RELAX_AMD_KERNEL_TWO_WALK) {
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
@@ -193,8 +193,8 @@ static int launch_bwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t
                                                   g_ent, grad_scale, grad_scale_dev, inv_t, d, d_stride, cus, s);
     if (rc != RELAX_AMD_EUNSUPPORTED) return rc;  // launched (or failed to): otherwise the row length is not built
   }
-  if (forced && strcmp(forced, "resident") == 0) {
-    set_error("logprob_entropy_bwd: RELAX_AMD_FUSED_STEP_KERNEL=resident, but no burst-form kernel is built for rows "
+  if (choice == RELAX_AMD_KERNEL_RESIDENT) {
+    set_error("logprob_entropy_bwd: kernel choice RESIDENT, but no burst-form kernel is built for rows "
               "of %lld elements of this type and alignment", (long long)vocab);
     return RELAX_AMD_EUNSUPPORTED;
   }

@@ -93,6 +93,11 @@ __device__ __forceinline__ void kl_term(int kind, float lp, float ref, float& kl
 }
 
 
+// NULL when the caller's struct_size covers this library's relax_amd_policy_loss_args, else the message to report.
+// Checked before any other field is read: a client built against a shorter layout would otherwise have the bytes
+// behind its struct taken for device pointers.
+const char* policy_loss_args_size_error(const relax_amd_policy_loss_args* a);
+
 // Host-side check of the optional distillation fields; NULL when they are consistent.
 inline const char* distill_args_error(const relax_amd_policy_loss_args& a) {
   if (!a.distill_teacher_log_prob) return nullptr;

@@ -190,6 +190,10 @@ extern "C" int relax_amd_policy_loss(const relax_amd_policy_loss_args* a, void* 
     set_error("policy_loss: args is NULL");
     return RELAX_AMD_EINVAL;
   }
+  if (policy_loss_args_size_error(a)) {
+    set_error("policy_loss: %s", policy_loss_args_size_error(a));
+    return RELAX_AMD_EINVAL;
+  }
   if (a->n_samples < 0 || a->n_tokens < 0 || a->n_samples > 2147483647LL) {
     set_error("policy_loss: bad sizes n_samples=%lld n_tokens=%lld", (long long)a->n_samples, (long long)a->n_tokens);
     return RELAX_AMD_EINVAL;

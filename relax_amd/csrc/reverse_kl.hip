@@ -312,9 +312,10 @@ static int launch_kl_step(const void* s, const void* t, int64_t n, int64_t vocab
                           float scale, float* kl, float* ls, float* lt, void* d, hipStream_t st) {
   const bool vec = aligned16(s) && aligned16(t) && aligned16(d) && (stride * int64_t(sizeof(T))) % 16 == 0;
   dim3 grid(static_cast<unsigned>(n));
-  // "cached": the two-walk kernel for every row length; "resident": fail where the register-resident one is not built
-  const char* forced = getenv("RELAX_AMD_FUSED_STEP_KERNEL");
-  if (vec && !(forced && strcmp(forced, "cached") == 0)) {
+  // relax_amd_set_kernel_choice: TWO_WALK = the two-walk kernel for every row length; RESIDENT = fail where the
+  // register-resident one is not built
+  const int choice = kernel_choice();
+  if (vec && choice != RELAX_AMD_KERNEL_TWO_WALK) {
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
@@ -323,8 +324,8 @@ static int launch_kl_step(const void* s, const void* t, int64_t n, int64_t vocab
                                                  g, scale, kl, ls, lt, static_cast<T*>(d), cus, st);
     if (rc != RELAX_AMD_EUNSUPPORTED) return rc;  // launched (or failed to): otherwise the row length is not built
   }
-  if (forced && strcmp(forced, "resident") == 0) {  // a comparison of the two kernels must not pass on one of them
-    set_error("reverse_kl_step_fused: RELAX_AMD_FUSED_STEP_KERNEL=resident, but no register-resident kernel is built "
+  if (choice == RELAX_AMD_KERNEL_RESIDENT) {  // a comparison of the two kernels must not pass on one of them
+    set_error("reverse_kl_step_fused: kernel choice RESIDENT, but no register-resident kernel is built "
               "for rows of %lld elements of this type and alignment", (long long)vocab);
     return RELAX_AMD_EUNSUPPORTED;
   }

@@ -11,9 +11,20 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._lib import BF16, F16, F32, NUM_METRICS, PolicyLossArgs, check, lib
+from ._lib import BF16, F16, F32, NUM_METRICS, check, lib, new_policy_loss_args
 
 _DTYPE_CODES = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+
+
+def set_kernel_choice(name: str) -> str:
+    """``relax_amd_set_kernel_choice``: "auto" | "two_walk" | "resident" for the entry points that hold two
+    bit-identical kernels; returns the previous choice.  For tests and measurements."""
+    from ._lib import KERNEL_CHOICES
+
+    prev = lib.relax_amd_set_kernel_choice(KERNEL_CHOICES[name])
+    if prev < 0:
+        check(prev)
+    return {v: k for k, v in KERNEL_CHOICES.items()}[prev]
 
 
 def _need_gpu(*tensors) -> torch.device:
@@ -293,7 +304,7 @@ def _policy_args(*, n, advantages, loss_mask, cu_resp, log_prob=None, old_log_pr
             out[k] = torch.empty(n, **kw)
         out["kl_tok"] = torch.empty(n, **kw) if kl_kind is not None else None
     partials = torch.empty(max(b, 1) * NUM_METRICS, **kw)
-    a = PolicyLossArgs()
+    a = new_policy_loss_args()
     (a.log_prob, a.old_log_prob, a.ref_log_prob, a.train_log_prob, a.rollout_log_prob, a.advantages, a.loss_mask,
      a.pg_loss_mask, a.entropy, a.sample_denom, a.pg_sample_denom) = [None if t is None else t.data_ptr() for t in keep]
     a.cu_resp = cu_resp.data_ptr()

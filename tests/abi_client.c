@@ -194,6 +194,7 @@ int main(void) {
         !d_tkl || !d_tgrad || !d_lp3 || !d_ent3)
       return 2;
     relax_amd_policy_loss_args a = {0};
+    a.struct_size = sizeof(a);
     a.advantages = d_adv;
     a.loss_mask = d_mask;
     a.cu_resp = d_cu;

@@ -19,3 +19,12 @@ def pytest_configure(config):
 def literals():
     with open(os.path.join(ROOT, "tests", "golden", "reference_literals.json")) as f:
         return json.load(f)
+
+
+@pytest.fixture(autouse=True)
+def _kernel_choice_back_to_auto():
+    """Tests that pin one of two bit-identical kernels leave the process-wide choice at its default."""
+    yield
+    from relax_amd import _lib
+
+    _lib.lib.relax_amd_set_kernel_choice(_lib.KERNEL_CHOICES["auto"])

@@ -19,7 +19,9 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(_lib.lib, n), f"{n} declared in include/relax_amd.h but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
-    assert _lib.lib.relax_amd_version() == 1
+    assert _lib.lib.relax_amd_version() == 2
+    header = open(_lib.HEADER_PATH).read()
+    assert "#define RELAX_AMD_ABI_VERSION 2" in header
 
 
 def test_struct_layout_matches_c_header(tmp_path):
@@ -62,14 +64,30 @@ def test_argument_validation_reports_errors_without_touching_the_gpu():
     assert rc == -1 and b"dtype" in L.relax_amd_last_error()
     assert L.relax_amd_logprob_entropy_fwd(None, 0, 0, 8, 8, None, None, 1.0, None, None, None, None, None) == 0
     # the distillation fields of the policy-loss block are checked before anything is launched
-    a = _lib.PolicyLossArgs()
+    # a block that does not state its size (a client built against a shorter layout) is refused before any field
+    # behind the old end is read
+    short = _lib.PolicyLossArgs()
+    short.metrics = short.sample_partials = short.cu_resp = 16
+    assert L.relax_amd_policy_loss(C.byref(short), None) == -1 and b"struct_size" in L.relax_amd_last_error()
+    short.struct_size = C.sizeof(_lib.PolicyLossArgs) - 8
+    assert L.relax_amd_policy_loss(C.byref(short), None) == -1 and b"struct_size" in L.relax_amd_last_error()
+    short.advantages = short.loss_mask = short.coef_log_prob = 16
+    rc = L.relax_amd_actor_step_fused(C.c_void_p(16), 2, 4, 64, 64, None, None, C.c_void_p(16), 1.0, C.byref(short),
+                                      1.0, C.c_void_p(16), C.c_void_p(16), C.c_void_p(16), C.c_void_p(16),
+                                      C.c_void_p(16), 64, None)
+    assert rc == -1 and b"struct_size" in L.relax_amd_last_error()
+    # the process-wide kernel choice: returns the previous value, refuses unknown ones
+    assert L.relax_amd_set_kernel_choice(1) == 0 and L.relax_amd_set_kernel_choice(2) == 1
+    assert L.relax_amd_set_kernel_choice(7) == -1 and b"unknown choice" in L.relax_amd_last_error()
+    assert L.relax_amd_set_kernel_choice(0) == 2
+    a = _lib.new_policy_loss_args()
     a.metrics = a.sample_partials = a.cu_resp = 16
     a.distill_teacher_log_prob = 16
     assert L.relax_amd_policy_loss(C.byref(a), None) == -1 and b"extra_coef_log_prob" in L.relax_amd_last_error()
     a.extra_coef_log_prob, a.distill_kl_kind = 16, _lib.KL_KINDS["k2"]
     assert L.relax_amd_policy_loss(C.byref(a), None) == -1 and b"distill_kl_kind" in L.relax_amd_last_error()
     # ... and so is the top-K distillation block of the fused step
-    f = _lib.PolicyLossArgs()
+    f = _lib.new_policy_loss_args()
     f.advantages = f.loss_mask = f.coef_log_prob = f.topk_ids = 16
     p16 = C.c_void_p(16)
 

@@ -232,8 +232,8 @@ def test_fused_opd_loss_matches_oracle_and_two_launch_path(n, v, dtype, tol):
                                        (128256, torch.bfloat16, 520), (131072, torch.float16, 515),
                                        (100352, torch.bfloat16, 1030), (102400, torch.bfloat16, 40),
                                        (163840, torch.bfloat16, 300), (8 * (19 * 1024 + 3), torch.float16, 530)])
-def test_register_resident_reverse_kl_step_equals_two_walk_kernel_bitwise(v, dtype, n, monkeypatch):
-    """The two kernels behind relax_amd_reverse_kl_step_fused, switched with RELAX_AMD_FUSED_STEP_KERNEL, for every
+def test_register_resident_reverse_kl_step_equals_two_walk_kernel_bitwise(v, dtype, n):
+    """The two kernels behind relax_amd_reverse_kl_step_fused, switched with relax_amd_set_kernel_choice, for every
     row shape the register-resident one is built for (partial and full last vector positions), with more rows than
     workgroups (several rows per persistent workgroup, uneven counts), fewer rows than workgroups, and rows without
     gradient (zero rows, KL still reported) scattered and in runs.  KL, both log-sum-exps and the gradient must be
@@ -252,7 +252,7 @@ def test_register_resident_reverse_kl_step_equals_two_walk_kernel_bitwise(v, dty
     g[-1] = 0.0
     results = {}
     for kind in ("cached", "resident"):
-        monkeypatch.setenv("RELAX_AMD_FUSED_STEP_KERNEL", kind)
+        ops.set_kernel_choice("two_walk" if kind == "cached" else "resident")
         kl, ls, lt, d = ops.reverse_kl_step_fused(s, t, g, 0.75)
         torch.cuda.synchronize()
         results[kind] = dict(kl=kl, lse_s=ls, lse_t=lt, d=d.view(torch.int16))

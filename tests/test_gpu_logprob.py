@@ -244,8 +244,8 @@ def test_full_size_properties_headline_shape():
                                        (32000, torch.float32, 1500), (4 * (8 * 1024 - 1), torch.float32, 700),
                                        (64000, torch.bfloat16, 900), (65536, torch.float16, 600),
                                        (50304, torch.float32, 700), (65536, torch.float32, 500)])
-def test_backward_burst_form_equals_row_per_workgroup_kernel_bitwise(v, dtype, n, monkeypatch):
-    """The two kernels behind relax_amd_logprob_entropy_bwd, switched with RELAX_AMD_FUSED_STEP_KERNEL, on every row
+def test_backward_burst_form_equals_row_per_workgroup_kernel_bitwise(v, dtype, n):
+    """The two kernels behind relax_amd_logprob_entropy_bwd, switched with relax_amd_set_kernel_choice, on every row
     shape the persistent burst form is built for (and the ends of two of them), with rows that score no token, tokens
     without gradient (zero rows, in runs and scattered), a device-side gradient scale and targets on a row's first and
     last element: bit-identical gradients."""
@@ -273,7 +273,7 @@ def test_backward_burst_form_equals_row_per_workgroup_kernel_bitwise(v, dtype, n
     scale = torch.tensor([0.37], device=dev)
     outs = {}
     for kind in ("cached", "resident"):
-        monkeypatch.setenv("RELAX_AMD_FUSED_STEP_KERNEL", kind)
+        ops.set_kernel_choice("two_walk" if kind == "cached" else "resident")
         for with_ent in (True, False):
             d = ops.logprob_entropy_bwd(x, tok, lse, spx, glp.to(dev), gen.to(dev) if with_ent else None,
                                         token_of_row=token_of_row, grad_scale_dev=scale, inv_temperature=0.8)

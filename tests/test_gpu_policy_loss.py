@@ -1633,8 +1633,8 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
 @pytest.mark.parametrize("v,dtype,n_rows", [(100352, torch.bfloat16, 700), (32000, torch.float32, 1500)])
 @pytest.mark.parametrize("pattern", ["all_dead", "one_live_last", "few_live", "random", "all_live_no_map",
                                      "zero_advantage"])
-def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dtype, n_rows, monkeypatch):
-    """The two kernels behind relax_amd_actor_step_fused, switched with RELAX_AMD_FUSED_STEP_KERNEL, on row / token
+def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dtype, n_rows):
+    """The two kernels behind relax_amd_actor_step_fused, switched with relax_amd_set_kernel_choice, on row / token
     layouts that stress the persistent loop of the register-resident one: no live row at all, a single live row at
     the very end, fewer live rows than workgroups, random prompt rows and masked tokens over several rows per
     workgroup, no row map (every row scores its own token), and tokens whose gradient coefficients vanish (zero
@@ -1680,7 +1680,7 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
     targets = torch.randint(0, v, (n_tok,), generator=g).to(dev)
     results = {}
     for kind in ("cached", "resident"):
-        monkeypatch.setenv("RELAX_AMD_FUSED_STEP_KERNEL", kind)
+        ops.set_kernel_choice("two_walk" if kind == "cached" else "resident")
         out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, token_of_row, sample_ids, n_tok, 1.0, 1.0, **kw)
         torch.cuda.synchronize()
         results[kind] = dict(lp=lp, ent=ent, lse=lse, spx=spx, coef=out["coef_log_prob"],
@@ -1699,7 +1699,7 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
                                      (4 * (7 * 1024 + 1), torch.float32), (4 * (8 * 1024 - 1), torch.float32),
                                      (8 * (7 * 1024 + 1), torch.bfloat16), (8 * 8 * 1024, torch.float16),
                                      (4 * (12 * 1024 + 1), torch.float32), (4 * (16 * 1024 - 1), torch.float32)])
-def test_register_resident_kernel_at_the_edges_of_its_row_shapes(v, dtype, monkeypatch):
+def test_register_resident_kernel_at_the_edges_of_its_row_shapes(v, dtype):
     """Row lengths at both ends of a built shape: one lane, or all lanes but one, hold a vector at the partially filled
     position.  Every output bit-identical to the two-walk kernel's."""
     from relax_amd import ops
@@ -1725,7 +1725,7 @@ def test_register_resident_kernel_at_the_edges_of_its_row_shapes(v, dtype, monke
     sample_ids = torch.zeros(n_tok, dtype=torch.int32, device=dev)
     results = {}
     for kind in ("cached", "resident"):
-        monkeypatch.setenv("RELAX_AMD_FUSED_STEP_KERNEL", kind)
+        ops.set_kernel_choice("two_walk" if kind == "cached" else "resident")
         out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets.to(dev), token_of_row, sample_ids, n_tok, 1.0,
                                                          1.0, **kw)
         torch.cuda.synchronize()
