@@ -545,7 +545,10 @@ int relax_amd_lmhead_logprob_fwd_keep(const void* hidden, const void* weight, in
  * Backward from kept logits: overwrites logits_t in place with the d_t of relax_amd_lmhead_dlogits_t (same formula,
  * x = the stored bf16 logit), one read and one write of the slab instead of a second projection
  * (_VocabParallelLogProbEntropy.backward, ppo_utils.py:591-629, applied to the stored logits).
- * l_stride must be a multiple of 8 and logits_t 16-byte aligned; columns n_tokens..l_stride-1 are left undefined.
+ * l_stride must be a multiple of 8 and logits_t 16-byte aligned.  Columns n_tokens .. ceil8(n_tokens) - 1 are written
+ * as zeros and later columns are not touched, so a slab whose padding was cleared once can go to
+ * relax_amd_lmhead_dhidden / relax_amd_lmhead_dweight as it is (a slab reused for FEWER tokens than a call before
+ * still holds that call's values in columns ceil8(n_tokens) .. and needs them cleared up to ceil128(n_tokens)).
  */
 int relax_amd_lmhead_dlogits_from_logits_t(void* logits_t, int64_t n_tokens, int64_t vocab, int64_t l_stride,
                                            const int64_t* targets, const float* lse, const float* spx,

@@ -189,7 +189,8 @@ __global__ __launch_bounds__(256) void lmhead_target_from_logits_kernel(const ui
 // Backward from stored logits: overwrites l_t [vocab, stride] (bf16 logits, token contiguous) with the gradient
 // dT[v, n] = inv_T * ( g_lp*(onehot - p) + g_H * p * (spx - x) ),  p = exp(x - lse)  -- the same expression the
 // recomputing kernel evaluates on its accumulators.  A thread owns eight neighbouring tokens (one 16-byte access per
-// vocabulary row) and keeps their per-token coefficients in registers while it walks `rows_per_block` rows.
+// vocabulary row) and keeps their per-token coefficients in registers while it walks `rows_per_block` rows.  Columns
+// n_tokens .. ceil8(n_tokens) - 1 (the rest of the last 16-byte vector) are written as zeros, later ones not at all.
 constexpr int kLmInplaceThreads = 256;
 __global__ __launch_bounds__(kLmInplaceThreads) void lmhead_dlogits_inplace_kernel(
     uint16_t* __restrict__ l_t, int64_t stride, int64_t n_tokens, int64_t vocab, int rows_per_block, float c,
@@ -229,6 +230,7 @@ __global__ __launch_bounds__(kLmInplaceThreads) void lmhead_dlogits_inplace_kern
       for (int k = 0; k < 8; ++k) {
         d[k] = fast_exp2(fmaf(x[k], c, k0[k])) * fmaf(x[k], a1[k], a0[k]);
         if (v + u == tg[k]) d[k] += hot[k];
+        if (tok8 + k >= n_tokens) d[k] = 0.f;  // the vector's tail past the last token: padding, kept at zero
       }
       u32x4 o;
       o.x = pack_bf16(d[0], d[1]);

@@ -192,8 +192,6 @@ class FusedLMHeadLogProb(torch.autograd.Function):
                                    "were overwritten with their gradient by the first one")
             slab = ctx.logits_t
             lmhead_dlogits_from_logits_t(slab[:v], n, targets, lse, spx, g_lp, g_ent, ctx.inv_temperature)
-            if slab.size(1) > n:
-                slab[:, n:].zero_()  # the in-place kernel works on whole 16-byte vectors of tokens
             ctx.logits_t = False
             if need_h:
                 lmhead_dhidden(slab, n, weight, d_hidden)
@@ -271,7 +269,7 @@ class _FusedLMHeadTokenLocalStep(torch.autograd.Function):
         lp_all = torch.empty(n, dtype=torch.float32, device=dev)
         ent_all = torch.empty(n if with_entropy else 0, dtype=torch.float32, device=dev)
         loss = torch.zeros((), dtype=torch.float32, device=dev)
-        slab = alloc_slab(v, slab_tokens, dev) if (need_h or need_w) and n > 0 else None
+        slab = alloc_slab(v, min(n, slab_tokens), dev) if (need_h or need_w) and n > 0 else None
         d_hidden = torch.empty_like(hidden) if need_h else None
         single = n <= slab_tokens
         d_weight = None
@@ -305,8 +303,9 @@ class _FusedLMHeadTokenLocalStep(torch.autograd.Function):
             g_ent = None if g_ent is None else g_ent.to(torch.float32).contiguous()
             lmhead_dlogits_from_logits_t(slab[:v], cnt, targets[s:e], lse, spx if g_ent is not None else None, g_lp,
                                          g_ent, inv_temperature)
-            if slab.size(1) > cnt:
-                slab[:, cnt:].zero_()  # the in-place kernel works on whole 16-byte vectors of tokens
+            if s > 0 and cnt < slab.size(1):
+                # a shorter last slab: columns past its last 16-byte vector still hold the previous slab's gradient
+                slab[:, (cnt + 7) // 8 * 8:_ceil128(cnt)].zero_()
             if need_h:
                 lmhead_dhidden(slab, cnt, weight, d_hidden[s:e])
             if need_w:

@@ -155,6 +155,36 @@ def test_kept_logits_slab_is_the_bf16_projection_and_stride_parity():
     torch.testing.assert_close(d_t.t().float().cpu(), want, atol=1e-5, rtol=2 * BF16_ULP)
 
 
+@pytest.mark.parametrize("n", [333, 257, 8 * 31 + 1])
+def test_in_place_gradient_leaves_the_padding_zero_for_the_backward_gemms(n):
+    """n % 8 != 0: relax_amd_lmhead_dlogits_from_logits_t writes whole 16-byte vectors of tokens; the lanes past the
+    last token must be zeros, so that a slab whose padding was cleared once goes to relax_amd_lmhead_dweight /
+    relax_amd_lmhead_dhidden as it is (their k loop runs over the padded token count) -- no clearing in between."""
+    from relax_amd import lm_head as LM
+
+    dev = require_gpu()
+    announce("lmhead in-place gradient padding", n)
+    h, v = 256, 777
+    hid, w, tok, g = _inputs(n, h, v, seed=n, w_scale=0.2)
+    hd, wd, td = hid.to(dev), w.to(dev), tok.to(dev)
+    slab = LM.alloc_slab(v, n, dev)
+    lp, ent, lse, spx = LM.lmhead_logprob_fwd(hd, wd, td, 1.0, True, logits_t=slab[:v])
+    g_lp = (torch.randn(n, generator=g) / 8).to(dev)
+    g_ent = (torch.randn(n, generator=g) / 8).to(dev)
+    # the last token's coefficients are large: if they leaked into the padding lanes the products below would show it
+    g_lp[-1], g_ent[-1] = 50.0, 50.0
+    d_t = LM.lmhead_dlogits_from_logits_t(slab[:v], n, td, lse, spx, g_lp, g_ent, 1.0)
+    assert (slab[:, n:] == 0).all() and (slab[v:] == 0).all()
+    d = d_t.float()
+    dw = torch.full((v, h), float("nan"), dtype=torch.float32, device=dev)
+    LM.lmhead_dweight(slab, n, hd, v, dw)
+    dh = torch.full((n, h), float("nan"), dtype=torch.float32, device=dev)
+    LM.lmhead_dhidden(slab, n, wd, dh)
+    want_dw, want_dh = d @ hd.float(), d.t() @ wd.float()
+    torch.testing.assert_close(dw, want_dw, atol=2e-5 * max(1.0, want_dw.abs().max().item()), rtol=1e-5)
+    torch.testing.assert_close(dh, want_dh, atol=2e-5 * max(1.0, want_dh.abs().max().item()), rtol=1e-5)
+
+
 @pytest.mark.parametrize("n,h,v", [
     (256, 256, 256),       # one tile, two k-slice pairs
     (300, 128, 1000),      # ragged in every dimension, hidden size of half a tile

@@ -53,6 +53,7 @@ def test_reference_literals(literals, key):
         (40, 4100, torch.bfloat16, 3.0, 2e-3),     # vector path + remainder vectors + scalar tail (4100 % 8 = 4)
         (24, 151936, torch.bfloat16, 3.0, 2e-3),   # headline vocabulary, spiked rows
         (24, 151936, torch.float16, 3.0, 2e-3),
+        (24, 151936, torch.float32, 3.0, 2e-5),    # what stock Megatron hands the custom-loss hook (loss.py:92-97)
         (3, 7, torch.bfloat16, 1.0, 2e-3),
     ],
 )

@@ -235,7 +235,9 @@ def test_reinforce_pp_masked_nonfinite_values_do_not_leak(single_pass):
 
 @pytest.mark.parametrize("v,dtype", [(151936, torch.bfloat16), (32000, torch.float32), (4096, torch.float16),
                                      (40960, torch.bfloat16), (100000, torch.bfloat16), (4100, torch.bfloat16),
-                                     (1003, torch.float32), (20000, torch.float32)])
+                                     (1003, torch.float32), (20000, torch.float32),
+                                     # what stock Megatron hands the custom-loss hook (loss.py:92-97)
+                                     (151936, torch.float32)])
 def test_single_pass_matches_two_launch_path_at_real_vocabularies(v, dtype):
     """Every workgroup width of the fused kernel (256 / 512 / 1024 threads), the scalar-tail and the unaligned
     scalar path, an upstream gradient != 1 and the one-shot backward."""
@@ -815,6 +817,89 @@ def test_full_size_actor_step_with_topk_distillation_term():
                                      R.make_reducer([seq_len], sub["loss_masks"], sample_denoms=[total_unmasked]))
     want.backward()
     torch.testing.assert_close(sub_rows, sub_logits.grad[0], atol=3e-9, rtol=2.0 ** -6)
+
+
+def test_full_size_actor_step_plain_spiked_rows_through_loss_function():
+    """The headline workload as the benchmark times it, all 65536 rows: bf16 logits ~ N(0, 3) with 5 % of the rows
+    carrying one logit raised by 15, first 20 % of every sequence masked, PPO-clip 0.2 / 0.28 + k3 KL 1e-3, no
+    distillation term, through loss_function (gradient-accumulation scale 1 / 16).  Runs the register-resident step
+    without the top-K block.  The same loss and metrics as the two-launch path; one whole sequence (4096 rows, some 200
+    of them spiked) against the oracle's log-probs, entropy and gradient; for every row: masked rows exactly zero,
+    gradient rows summing to zero up to the rounding of 151936 bf16 terms."""
+    import relax_amd
+
+    dev = require_gpu()
+    seqs, seq_len, v = 16, 4096, 151936
+    n = seqs * seq_len
+    announce("actor step, plain, spiked rows, full size", n, v)
+    g = torch.Generator(device=dev).manual_seed(0)
+    logits = torch.empty((1, n, v), dtype=torch.bfloat16, device=dev)
+    spiked = torch.zeros(n, dtype=torch.bool, device=dev)
+    for s0 in range(0, n, 2048):
+        x = torch.randn((2048, v), device=dev, generator=g) * 3.0
+        spike = torch.rand(2048, device=dev, generator=g) < 0.05
+        cols = torch.randint(0, v, (2048,), device=dev, generator=g)
+        x[spike, cols[spike]] += 15.0
+        spiked[s0:s0 + 2048] = spike
+        logits[0, s0:s0 + 2048] = x.bfloat16()
+        del x
+    toks = [torch.randint(0, v, (seq_len,), device=dev, generator=g) for _ in range(seqs)]
+    mask = torch.ones(seq_len, device=dev)
+    mask[: seq_len // 5] = 0.0
+    kw = dict(eps_clip=0.2, eps_clip_high=0.28, use_kl_loss=True, kl_loss_coef=1e-3, kl_loss_type="k3",
+              global_batch_size=seqs)
+    args = P.make_args(**kw)
+    with torch.no_grad():
+        _, out = relax_amd.get_log_probs_and_entropy(logits, args=args, unconcat_tokens=toks,
+                                                     total_lengths=[seq_len] * seqs,
+                                                     response_lengths=[seq_len] * seqs, with_entropy=True)
+    old = [lp + 0.05 * torch.randn(lp.shape, device=dev, generator=g) for lp in out["log_probs"]]
+    ref = [lp + 0.1 * torch.randn(lp.shape, device=dev, generator=g) for lp in out["log_probs"]]
+    total_unmasked = float(mask.sum().item()) * seqs
+    batch = dict(
+        unconcat_tokens=toks, total_lengths=[seq_len] * seqs, response_lengths=[seq_len] * seqs,
+        loss_masks=[mask] * seqs, advantages=[torch.randn(seq_len, device=dev, generator=g) for _ in range(seqs)],
+        log_probs=old, ref_log_probs=ref,
+        relax_amd_sample_denominators=torch.full((seqs,), total_unmasked, device=dev))
+    picked = 11
+    rows = slice(picked * seq_len, (picked + 1) * seq_len)
+    assert 100 < int(spiked[rows].sum().item()) < 400
+    results = {}
+    for mode in ("auto", "off"):
+        lg = logits.detach().requires_grad_()
+        loss, normalizer, log = relax_amd.loss_function(P.make_args(relax_amd_single_pass=mode, **kw), batch, 1, lg)
+        loss.backward()
+        met = dict(zip(log["keys"], log["values"][1:].tolist()))
+        d = lg.grad[0]
+        if mode == "auto":
+            flat_mask = mask.repeat(seqs)
+            for s0 in range(0, n, 8192):
+                blk = d[s0:s0 + 8192]
+                assert blk.float().sum(-1).abs().max().item() < 5e-2 / seqs
+                assert (blk[flat_mask[s0:s0 + 8192] == 0] == 0).all()
+                assert (blk[flat_mask[s0:s0 + 8192] != 0] != 0).any(dim=1).all()
+        results[mode] = (loss.detach().item(), met, d[rows].float().cpu())
+        assert float(normalizer) == 1
+        del d, lg, loss
+        torch.cuda.empty_cache()
+    assert abs(results["auto"][0] - results["off"][0]) < 1e-6 * max(1.0, abs(results["off"][0]))
+    for key, w in results["off"][1].items():
+        assert abs(results["auto"][1][key] - w) < 1e-5 * max(1.0, abs(w)), key
+    torch.testing.assert_close(results["auto"][2], results["off"][2], atol=2e-10, rtol=2.0 ** -6)
+    # the picked sequence against the oracle: log-probs, entropy, its share of the token-mean loss, its rows' gradient
+    sub_logits = logits[0, rows].float().cpu().unsqueeze(0).requires_grad_()
+    sub = {key: [val[picked].cpu()] for key, val in batch.items() if isinstance(val, list) and torch.is_tensor(val[0])}
+    sub.update(total_lengths=[seq_len], response_lengths=[seq_len])
+    _, oo = P.get_log_probs_and_entropy(sub_logits.detach(), args=args, unconcat_tokens=sub["unconcat_tokens"],
+                                        total_lengths=[seq_len], response_lengths=[seq_len], with_entropy=True)
+    torch.testing.assert_close(out["log_probs"][picked].cpu(), oo["log_probs"][0], atol=2e-3, rtol=0)
+    torch.testing.assert_close(out["entropy"][picked].cpu(), oo["entropy"][0], atol=2e-3, rtol=0)
+    want, _ = P.policy_loss_function(args, sub, sub_logits,
+                                     R.make_reducer([seq_len], sub["loss_masks"], sample_denoms=[total_unmasked]))
+    (want / seqs).backward()  # loss_function's scale: num_microbatches / global_batch_size * dp = 1 / 16
+    torch.testing.assert_close(results["auto"][2], sub_logits.grad[0], atol=3e-10, rtol=2.0 ** -6)
+    hot = spiked[rows].cpu() & (mask.cpu() != 0)
+    assert results["auto"][2][hot].abs().sum() > 0
 
 
 def test_full_size_grpo_plumbing_case_rewards_to_dlogits():
