@@ -39,16 +39,26 @@ PROFILES_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profile
 KERNEL_CHOICE = "auto"  # --kernel-choice, as handed to relax_amd_set_kernel_choice
 
 
-def known_size_copy(dev) -> None:
-    """One untimed plain device copy of 1 GiB (reads 1 GiB, writes 1 GiB) before the timed region: under
-    ``rocprofv3 --pmc FETCH_SIZE`` / ``WRITE_SIZE`` its dispatch is the known-size reference that the counters of the
-    step's kernels are scaled by."""
-    src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).fill_(1.0)
-    dst = torch.empty_like(src)
+KNOWN_ROWS, KNOWN_VOCAB = 4099, 131072  # an odd row count no workload uses: the reference dispatches' signature
+KNOWN_KIB = KNOWN_ROWS * KNOWN_VOCAB * 2 / 1024.0
+
+
+def known_size_streams(dev) -> None:
+    """Two untimed launches of known traffic before the timed region, the references that ``rocprofv3 --pmc
+    FETCH_SIZE`` / ``WRITE_SIZE`` readings of the step's kernels are scaled by: the library's forward scan over
+    4099 x 131072 bf16 logits (reads 1.0002 GiB, writes a few KB) and its row-per-workgroup backward with all-zero
+    incoming gradients (such rows are zero-filled without being read: writes 1.0002 GiB, reads a few KB)."""
+    from relax_amd import ops
+
+    x = torch.ones((KNOWN_ROWS, KNOWN_VOCAB), dtype=torch.bfloat16, device=dev)
+    tok = torch.zeros(KNOWN_ROWS, dtype=torch.int64, device=dev)
+    zeros = torch.zeros(KNOWN_ROWS, dtype=torch.float32, device=dev)
+    _, _, lse, spx = ops.logprob_entropy_fwd(x, tok, None, 1.0, True)
+    prev = ops.set_kernel_choice("two_walk")
+    ops.logprob_entropy_bwd(x, tok, lse, spx, zeros, zeros)
+    ops.set_kernel_choice(prev)
     torch.cuda.synchronize()
-    dst.copy_(src)
-    torch.cuda.synchronize()
-    del src, dst
+    del x
 
 
 def measured_traffic(kernel: str, rows: int, vocab: int):
@@ -72,6 +82,94 @@ def measured_traffic(kernel: str, rows: int, vocab: int):
     return None, None
 
 
+LIVE_TRAFFIC = None  # {"fetch_KiB": {kernel: mean per dispatch}, "write_KiB": {...}, scales, command} of this run
+
+
+def _pmc_pass(counter: str, argv: list, outdir: str, limit_s: int):
+    """One ``rocprofv3 --pmc <counter>`` run of this file (a child process; one timed step, no CPU baseline, no other
+    workloads).  Returns ([(kernel name, workgroups, counter value) per dispatch], command line) or (None, why)."""
+    import csv
+    import glob
+    import shutil
+    import subprocess
+
+    prof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    if not os.path.exists(prof):
+        return None, "rocprofv3 not found"
+    cmd = ["timeout", "-s", "KILL", str(limit_s), prof, "--pmc", counter, "-d", outdir, "-o", "p", "--output-format",
+           "csv", "--", sys.executable, os.path.abspath(__file__), *argv]
+    env = dict(os.environ, TMPDIR="/tmp")
+    try:
+        r = subprocess.run(cmd, cwd="/tmp", env=env, capture_output=True, text=True, timeout=limit_s + 30)
+    except (OSError, subprocess.TimeoutExpired) as e:
+        return None, f"{type(e).__name__}: {e}"
+    files = glob.glob(os.path.join(outdir, "**", "*counter_collection.csv"), recursive=True)
+    if r.returncode != 0 or not files:
+        return None, f"rocprofv3 exit {r.returncode}: {(r.stderr or r.stdout)[-300:]}"
+    dispatches = []  # (kernel name, workgroups, counter value)
+    with open(files[0], newline="") as f:
+        for row in csv.DictReader(f):
+            if row.get("Counter_Name") == counter:
+                groups = int(row["Grid_Size"]) // max(1, int(row["Workgroup_Size"]))
+                dispatches.append((row["Kernel_Name"], groups, float(row["Counter_Value"])))
+    return dispatches, " ".join(cmd[3:])
+
+
+def collect_live_traffic(argv: list, limit_s: int = 170):
+    """HBM-side bytes per launch of the step's kernels, measured in THIS run: two child runs of this file under
+    ``rocprofv3 --pmc`` (FETCH_SIZE, then WRITE_SIZE: one counter per run), each scaled by what the same counter reads
+    for the known-size launch the child makes before its timed step (``known_size_streams``).  Must be called before this process touches the GPU.
+    Returns a dict for ``measured_traffic`` or {"error": why} (the committed summaries under profiles/ then stand in,
+    and ``traffic_source`` says so)."""
+    import shutil
+    import tempfile
+
+    out = {}
+    tmp = tempfile.mkdtemp(prefix="relax_amd_pmc_", dir="/tmp")
+    try:
+        for counter, key in (("FETCH_SIZE", "fetch"), ("WRITE_SIZE", "write")):
+            dispatches, info = _pmc_pass(counter, argv, os.path.join(tmp, key), limit_s)
+            if dispatches is None:
+                return {"error": f"{counter}: {info}"}
+            ref_kernel = "logprob_entropy_fwd_kernel" if key == "fetch" else "logprob_entropy_bwd_kernel"
+            known = [v for name, groups, v in dispatches if ref_kernel in name and groups == KNOWN_ROWS]
+            if not known or max(known) <= 0:
+                return {"error": f"{counter}: the known-size {ref_kernel} launch was not among the profiled dispatches"}
+            out[key + "_scale"] = KNOWN_KIB / max(known)
+            per_kernel = {}
+            for name, groups, v in dispatches:
+                if groups != KNOWN_ROWS:
+                    per_kernel.setdefault(name, []).append(v)
+            out[key + "_KiB"] = {k: sum(v) / len(v) for k, v in per_kernel.items()}
+            out[key + "_command"] = info
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    return out
+
+
+def live_traffic_of(kernel: str):
+    """(bytes per launch, source) of ``kernel`` from this run's own counter passes, or (None, None)."""
+    t = LIVE_TRAFFIC
+    if not t or "error" in t:
+        return None, None
+    base = kernel.split("<")[0]
+    want = kernel.replace(" ", "")
+
+    def pick(table):
+        exact = [v for k, v in table.items() if want in k.replace(" ", "")]
+        if exact:
+            return sum(exact) / len(exact)
+        loose = [v for k, v in table.items() if base in k]
+        return sum(loose) / len(loose) if loose else None
+
+    f, w = pick(t["fetch_KiB"]), pick(t["write_KiB"])
+    if f is None or w is None:
+        return None, None
+    kib = f * t["fetch_scale"] + w * t["write_scale"]
+    return kib * 1024.0, (f"this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE child passes, per dispatch {f:.0f} x "
+                          f"{t['fetch_scale']:.3f} + {w:.0f} x {t['write_scale']:.3f} KiB (scales: the same counters over known-size launches of this run)")
+
+
 def hbm_roofline(kernel: str, launch_ms: float, necessary_bytes: float, rows: int, vocab: int, kernel_ms: dict,
                  ms_per_step: float, two_pass_bytes: float | None = None) -> dict:
     """Roofline block of a bandwidth-bound launch.  ``achieved`` = the bytes the launch has to move (every input row
@@ -82,7 +180,11 @@ def hbm_roofline(kernel: str, launch_ms: float, necessary_bytes: float, rows: in
     achieved = necessary_bytes / (launch_ms * 1e-3) / 1e9
     frac = achieved / HBM_PEAK_GBS
     assert frac <= 1.0, f"roofline fraction {frac} > 1: the byte count does not describe the launch"
-    traffic, source = measured_traffic(kernel, rows, vocab)
+    traffic, source = live_traffic_of(kernel)
+    if traffic is None:
+        traffic, source = measured_traffic(kernel, rows, vocab)
+        if traffic is not None and LIVE_TRAFFIC and "error" in LIVE_TRAFFIC:
+            source += f" (committed figure; this run's counter passes failed: {LIVE_TRAFFIC['error']})"
     out = {"bound": "hbm", "kernel": kernel, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": frac,
            "traffic": traffic, "traffic_source": source, "algorithmic_bytes_per_launch": necessary_bytes,
            "avg_launch_ms": launch_ms, "kernel_ms": kernel_ms,
@@ -340,7 +442,6 @@ def run_actor_step(a, dev) -> None:
         loss.backward()
         return loss
 
-    known_size_copy(dev)
     wall, kernel_ms, _, loss = timed_steps(step, a.warmup, a.steps)
     ms_per_step = wall * 1e3 / a.steps
     row_bytes = float(a.vocab * logits.element_size())
@@ -694,6 +795,10 @@ def main() -> int:
     ap.add_argument("--no-secondary", action="store_true",
                     help="plain invocation only: skip the other configurations that otherwise run after the headline "
                          "workload and ride along in its line as other_workloads")
+    ap.add_argument("--traffic", choices=["auto", "live", "off"], default="auto",
+                    help="roofline.traffic: 'live' measures it in this run (two child runs of this file under "
+                         "rocprofv3 --pmc before the timed steps, about a minute); 'off' takes the figure committed "
+                         "under profiles/; 'auto' = live for the plain invocation, off otherwise")
     ap.add_argument("--kernel-choice", choices=["auto", "two_walk", "resident"], default="auto",
                     help="relax_amd_set_kernel_choice: which of the two bit-identical kernels the fused entry points "
                          "launch (two_walk = the row-per-workgroup kernels for every row length)")
@@ -702,6 +807,20 @@ def main() -> int:
         print("bench.py measures one GPU: this build has no multi-GPU path (token rows shard without any exchange). "
               "Run with --gpus 1.", file=sys.stderr)
         return 2
+    plain = a.workload == "actor_step" and a.opd_topk == 0 and a.cpu_rows > 0 and not a.no_secondary
+    if a.traffic == "live" or (a.traffic == "auto" and plain):
+        # before anything in this process touches the GPU: the children are separate programs under the profiler
+        global LIVE_TRAFFIC
+        child = ["--workload", a.workload, "--steps", "1", "--warmup", "1", "--cpu-rows", "0", "--no-secondary",
+                 "--traffic", "off", "--seqs", str(a.seqs), "--seq-len", str(a.seq_len), "--vocab", str(a.vocab),
+                 "--kernel-choice", a.kernel_choice]
+        if a.rows:
+            child += ["--rows", str(a.rows)]
+        if a.two_launch:
+            child.append("--two-launch")
+        if a.opd_topk:
+            child += ["--opd-topk", str(a.opd_topk)]
+        LIVE_TRAFFIC = collect_live_traffic(child)
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         return 2
@@ -714,6 +833,7 @@ def main() -> int:
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    known_size_streams(dev)
     if a.workload == "actor_step_opd_topk" and a.opd_topk == 0:
         a.opd_topk = 64
     if a.opd_topk > 0:
