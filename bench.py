@@ -12,6 +12,7 @@ invocation then also runs the other configurations below (up to 10 timed steps e
 reports them inside that line as ``other_workloads``; ``--no-secondary`` or ``--cpu-rows 0`` skips them.
 
 ``--workload`` selects the other configurations of the same path, each printed in the same format:
+``actor_step_fp32`` (the actor step on fp32 logits [32768, 151936], the dtype stock Megatron hands a custom loss),
 ``cfg1`` (GRPO plumbing case: 512 responses x 256 tokens, fp32 logits [131072, 32000], rewards -> advantages -> loss),
 ``lmhead`` (fused LM-head + log-prob/entropy forward and dhidden/dweight backward, hidden [32768, 4096], MFMA-bound),
 ``reverse_kl`` (on-policy distillation, student/teacher [16384, 151936], forward + student dlogits),
@@ -239,11 +240,13 @@ def make_args():
     )
 
 
-def make_workload(device, seqs: int, seq_len: int, vocab: int, seed: int = 0):
-    """Synthetic inputs of the named configuration, generated on the device in row blocks."""
+def make_workload(device, seqs: int, seq_len: int, vocab: int, seed: int = 0, dtype=torch.bfloat16):
+    """Synthetic inputs of the named configuration, generated on the device in row blocks.  ``dtype=torch.float32``
+    holds the same bf16-rounded values widened to fp32: what a bf16 output layer followed by Megatron's ``.float()``
+    hands the loss hook."""
     g = torch.Generator(device=device).manual_seed(seed)
     n = seqs * seq_len
-    logits = torch.empty((1, n, vocab), dtype=torch.bfloat16, device=device)
+    logits = torch.empty((1, n, vocab), dtype=dtype, device=device)
     flat = logits[0]
     block = 2048
     for s in range(0, n, block):
@@ -252,7 +255,7 @@ def make_workload(device, seqs: int, seq_len: int, vocab: int, seed: int = 0):
         spike = torch.rand(e - s, device=device, generator=g) < 0.05
         cols = torch.randint(0, vocab, (e - s,), device=device, generator=g)
         x[spike, cols[spike]] += 15.0
-        flat[s:e] = x.to(torch.bfloat16)
+        flat[s:e] = x.to(torch.bfloat16).to(dtype)
         del x
     tokens = [torch.randint(0, vocab, (seq_len,), device=device, generator=g) for _ in range(seqs)]
     mask = torch.ones(seq_len, device=device)
@@ -413,7 +416,8 @@ def run_actor_step(a, dev) -> None:
 
     args = make_args()
     args.loss_type = "policy_loss"
-    logits, batch, g = make_workload(dev, a.seqs, a.seq_len, a.vocab)
+    fp32 = a.workload == "actor_step_fp32"
+    logits, batch, g = make_workload(dev, a.seqs, a.seq_len, a.vocab, dtype=torch.float32 if fp32 else torch.bfloat16)
     attach_old_and_ref(batch, logits, args, g)
     logits.requires_grad_()
     n_tokens = a.seqs * a.seq_len
@@ -449,16 +453,18 @@ def run_actor_step(a, dev) -> None:
     # what the step must move: every live row read once, every dlogits row written once (masked rows: zeros)
     necessary = row_bytes * (live + n_tokens)
     if "actor_step_fused" in kernel_ms:
-        dom, dom_name = kernel_ms["actor_step_fused"], fused_step_kernel_name(a.vocab)
+        dom, dom_name = kernel_ms["actor_step_fused"], fused_step_kernel_name(a.vocab, "float" if fp32 else "bf16_t")
         if a.opd_topk > 0:
             dom_name = dom_name[:-1] + ", true>"  # the instantiation that evaluates the top-K term
     else:  # two launches: the backward (read live rows, write all rows) dominates; the forward read is its own launch
         dom, dom_name = kernel_ms["logprob_entropy_bwd"], bwd_kernel_name(a.vocab)
     emit(a, n_tokens, wall,
-         f"Qwen3-8B-shaped actor step: {a.seqs} seqs x {a.seq_len} tokens = {n_tokens} rows x V={a.vocab} bf16 "
+         f"Qwen3-8B-shaped actor step: {a.seqs} seqs x {a.seq_len} tokens = {n_tokens} rows x V={a.vocab} "
+         f"{'fp32 (bf16 values widened, as Megatron hands them to a custom loss)' if fp32 else 'bf16'} "
          f"logits, PPO-clip 0.2/0.28 + k3 KL 1e-3{opd}, loss_function (scale 1/{args.global_batch_size}) fwd + bwd "
          f"to dlogits",
-         {"rows": n_tokens, "live_rows": live, "vocab": a.vocab, "loss": float(loss.item())},
+         {"rows": n_tokens, "live_rows": live, "vocab": a.vocab, "loss": float(loss.item()),
+          **({"logits_dtype": "f32"} if fp32 else {})},
          hbm_roofline(dom_name, dom, necessary, n_tokens, a.vocab, kernel_ms, ms_per_step,
                       two_pass_bytes=3.0 * row_bytes * n_tokens if "actor_step_fused" in kernel_ms else None),
          cpu_baseline(args, a.cpu_rows, a.vocab) if a.cpu_rows > 0 else None)
@@ -770,7 +776,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="actor_step",
-                    choices=["actor_step", "actor_step_opd_topk", "cfg1", "lmhead", "reverse_kl", "varlen_gspo",
+                    choices=["actor_step", "actor_step_opd_topk", "actor_step_fp32", "cfg1", "lmhead", "reverse_kl", "varlen_gspo",
                              "varlen_cispo", "actor_fwd_topk"])
     ap.add_argument("--seqs", type=int, default=SEQS)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
@@ -836,6 +842,8 @@ def main() -> int:
     known_size_streams(dev)
     if a.workload == "actor_step_opd_topk" and a.opd_topk == 0:
         a.opd_topk = 64
+    if a.workload == "actor_step_fp32" and a.seqs == SEQS:
+        a.seqs = SEQS // 2  # 32768 rows: the same 19.9 GB of logits as the bf16 step
     if a.opd_topk > 0:
         a.cpu_rows = 0  # the CPU baseline is timed on the headline workload only
     if a.workload == "actor_step" and a.opd_topk == 0 and a.cpu_rows > 0 and not a.no_secondary:
@@ -845,7 +853,7 @@ def main() -> int:
 
 
 def run_workload(a, dev) -> None:
-    if a.workload in ("actor_step", "actor_step_opd_topk"):
+    if a.workload in ("actor_step", "actor_step_opd_topk", "actor_step_fp32"):
         run_actor_step(a, dev)
     elif a.workload == "cfg1":
         run_cfg1(a, dev)
@@ -859,7 +867,8 @@ def run_workload(a, dev) -> None:
         run_varlen(a, dev, a.workload.split("_")[1])
 
 
-SECONDARY = ("lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "cfg1", "actor_fwd_topk", "actor_step_opd_topk")
+SECONDARY = ("lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "cfg1", "actor_fwd_topk", "actor_step_opd_topk",
+             "actor_step_fp32")
 
 
 def run_default_with_secondary(a, dev) -> int:
@@ -883,6 +892,9 @@ def run_default_with_secondary(a, dev) -> int:
         b = copy.copy(a)
         b.workload, b.steps, b.warmup, b.cpu_rows, b.rows = name, min(a.steps, 10), min(a.warmup, 3), 0, 0
         b.opd_topk = 64 if name == "actor_step_opd_topk" else 0
+        if name == "actor_step_fp32":
+            b.seqs = max(1, a.seqs // 2)  # half the rows: the same 19.9 GB of logits as the bf16 step
+        b.traffic = "off"
         try:
             run_workload(b, dev)
             got = COLLECTED.pop()

@@ -422,7 +422,8 @@ int relax_amd_topk_rows(const void* logits, int dtype, int64_t n_tokens, int64_t
  * log-probs / entropy of the response tokens and torch.topk of the same logits rows).  Arguments as in those two
  * functions; log_prob / entropy / lse / spx are bit-identical to relax_amd_logprob_entropy_fwd's, values / indices
  * follow relax_amd_topk_rows' contract (the selection does not depend on the temperature).  Rows that are not whole
- * 16-byte vectors in groups of eight, or shorter than 8192 vectors, run the two passes one after the other.
+ * 16-byte vectors in groups of eight, or too short for the forward scan's 1024-thread workgroups (fewer than 7168
+ * vectors), run the two passes one after the other.
  */
 int relax_amd_logprob_entropy_topk_fwd(const void* logits, int dtype, int64_t n_tokens, int64_t vocab,
                                        int64_t row_stride, const int32_t* row_ids, const int64_t* targets,

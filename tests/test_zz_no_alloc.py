@@ -41,17 +41,34 @@ def _call(lib, static, hidden, weight, targets, inv_t):
 
 
 def test_static_scratch_forward_matches_workspace_forward_on_two_calls_in_a_row():
-    from relax_amd._lib import lib
+    from relax_amd._lib import check, lib
 
     dev = require_gpu()
     names = ("log_prob", "entropy", "lse", "spx")
     # first a larger input (several row blocks, vocabulary splits), then a smaller one that reuses the same array,
     # then an odd-sized one with a temperature
-    for n, h, v, seed, inv_t in ((1500, 256, 5000, 1, 1.0), (300, 256, 5000, 2, 1.0), (777, 128, 1111, 3, 1.0 / 0.7)):
+    for i, (n, h, v, seed, inv_t) in enumerate(((1500, 256, 5000, 1, 1.0), (300, 256, 5000, 2, 1.0),
+                                                (777, 128, 1111, 3, 1.0 / 0.7))):
         announce("lmhead static scratch", n, h, v)
         hidden, weight, targets = _inputs(n, h, v, seed, dev)
         want = _call(lib, False, hidden, weight, targets, inv_t)
         got = _call(lib, True, hidden, weight, targets, inv_t)
+        if i > 0:
+            # what the entry point exists for: once the first call has resolved the array's address, a call takes no
+            # device memory and gives none back -- neither through the runtime nor through torch's allocator
+            outs = [torch.empty(n, device=dev) for _ in range(4)]
+            stream = torch.cuda.current_stream().cuda_stream
+            torch.cuda.synchronize()
+            free_before, held_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
+            reserved_before = torch.cuda.memory_reserved()
+            for _ in range(3):
+                check(lib.relax_amd_lmhead_logprob_fwd_static(
+                    hidden.data_ptr(), weight.data_ptr(), BF16, n, h, v, hidden.stride(0), weight.stride(0),
+                    targets.data_ptr(), inv_t, *[o.data_ptr() for o in outs], stream))
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info()[0] == free_before
+            assert torch.cuda.memory_allocated() == held_before and torch.cuda.memory_reserved() == reserved_before
+            assert torch.equal(outs[0], got[0])
         for name, a, b in zip(names, got, want):
             assert torch.isfinite(a).all(), name
             assert torch.equal(a, b), (name, n, (a - b).abs().max().item())
