@@ -817,16 +817,24 @@ def main() -> int:
     if a.traffic == "live" or (a.traffic == "auto" and plain):
         # before anything in this process touches the GPU: the children are separate programs under the profiler
         global LIVE_TRAFFIC
-        child = ["--workload", a.workload, "--steps", "1", "--warmup", "1", "--cpu-rows", "0", "--no-secondary",
-                 "--traffic", "off", "--seqs", str(a.seqs), "--seq-len", str(a.seq_len), "--vocab", str(a.vocab),
-                 "--kernel-choice", a.kernel_choice]
-        if a.rows:
-            child += ["--rows", str(a.rows)]
-        if a.two_launch:
-            child.append("--two-launch")
-        if a.opd_topk:
-            child += ["--opd-topk", str(a.opd_topk)]
-        LIVE_TRAFFIC = collect_live_traffic(child)
+
+        def child_args(workload):
+            child = ["--workload", workload, "--steps", "1", "--warmup", "1", "--cpu-rows", "0", "--no-secondary",
+                     "--traffic", "off", "--seqs", str(a.seqs), "--seq-len", str(a.seq_len), "--vocab", str(a.vocab),
+                     "--kernel-choice", a.kernel_choice]
+            if a.rows:
+                child += ["--rows", str(a.rows)]
+            if a.two_launch:
+                child.append("--two-launch")
+            if a.opd_topk and workload == a.workload:
+                child += ["--opd-topk", str(a.opd_topk)]
+            return child
+
+        LIVE_TRAFFIC = collect_live_traffic(child_args(a.workload))
+        if plain:  # the bandwidth-bound configurations that ride along get their own counter passes
+            for name in SECONDARY:
+                if name != "lmhead":
+                    SECONDARY_TRAFFIC[name] = collect_live_traffic(child_args(name))
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         return 2
@@ -867,6 +875,7 @@ def run_workload(a, dev) -> None:
         run_varlen(a, dev, a.workload.split("_")[1])
 
 
+SECONDARY_TRAFFIC = {}  # workload -> collect_live_traffic() result, filled by the plain invocation before it touches the GPU
 SECONDARY = ("lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "cfg1", "actor_fwd_topk", "actor_step_opd_topk",
              "actor_step_fp32")
 
@@ -881,12 +890,13 @@ def run_default_with_secondary(a, dev) -> int:
     import copy
     import gc
 
-    global COLLECTED
+    global COLLECTED, LIVE_TRAFFIC
     COLLECTED = []
     run_actor_step(a, dev)
     line = COLLECTED.pop()
     others = {}
     for name in SECONDARY:
+        LIVE_TRAFFIC = SECONDARY_TRAFFIC.get(name)
         gc.collect()
         torch.cuda.empty_cache()
         b = copy.copy(a)
@@ -903,6 +913,10 @@ def run_default_with_secondary(a, dev) -> int:
                             "steps": got["steps"], "kernel": r["kernel"], "bound": r["bound"],
                             "avg_launch_ms": round(r["avg_launch_ms"], 4), "achieved": round(r["achieved"], 1),
                             "unit": r["unit"], "frac": round(r["frac"], 4)}
+            if r.get("traffic"):
+                others[name]["traffic"] = round(r["traffic"])
+                others[name]["traffic_over_algorithmic"] = round(r["traffic"] / r["algorithmic_bytes_per_launch"], 3)
+                others[name]["traffic_measured_in_this_run"] = r["traffic_source"].startswith("this run")
         except Exception as e:  # a secondary workload must not cost the headline line
             others[name] = {"error": f"{type(e).__name__}: {e}"}
             COLLECTED.clear()
