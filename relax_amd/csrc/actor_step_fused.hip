@@ -230,6 +230,12 @@ static int dispatch_fused(const void* logits, int64_t n_rows, int64_t vocab, int
     const int rc = launch_actor_step_resident<T>(x, stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t, a,
                                                  grad_scale, lp, ent, lse, spx, d, d_stride, device_compute_units(), s);
     if (rc != RELAX_AMD_EUNSUPPORTED) return rc;  // launched (or failed to): otherwise the row length is not built
+    if constexpr (sizeof(T) == 4) {  // long fp32 rows: resident as their upper halves where those are exact
+      const int rcw = launch_actor_step_resident_wide(x, stride, vocab, n_rows, token_of_row, sample_ids, targets,
+                                                      inv_t, a, grad_scale, lp, ent, lse, spx, d, d_stride,
+                                                      device_compute_units(), s);
+      if (rcw != RELAX_AMD_EUNSUPPORTED) return rcw;
+    }
   }
   if (choice == RELAX_AMD_KERNEL_RESIDENT) {
     set_error("actor_step_fused: kernel choice RESIDENT, but no register-resident kernel is built for "

@@ -20,4 +20,12 @@ int launch_actor_step_resident(const T* logits, int64_t row_stride, int64_t voca
                                float* entropy, float* lse, float* spx, T* dlogits, int64_t d_stride,
                                int compute_units, hipStream_t stream);
 
+// The same for fp32 rows of 128256 .. 163840 entries, kept in the registers as their upper halves when those are all
+// there is to them (actor_step_resident_wide.hip).
+int launch_actor_step_resident_wide(const float* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
+                                    const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,
+                                    float inv_t, const relax_amd_policy_loss_args& a, float grad_scale,
+                                    float* log_prob, float* entropy, float* lse, float* spx, float* dlogits,
+                                    int64_t d_stride, int compute_units, hipStream_t stream);
+
 }  // namespace relax_amd

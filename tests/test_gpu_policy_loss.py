@@ -1715,10 +1715,15 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
     torch.testing.assert_close(outs["auto"][2].float().cpu(), lo.grad, atol=tol, rtol=max(ulp, 1e-5))
 
 
-@pytest.mark.parametrize("v,dtype,n_rows", [(100352, torch.bfloat16, 700), (32000, torch.float32, 1500)])
+@pytest.mark.parametrize("v,dtype,n_rows,values", [
+    (100352, torch.bfloat16, 700, "plain"), (32000, torch.float32, 1500, "plain"),
+    # long fp32 rows, kept in the registers as their upper halves: bf16 values widened to fp32 (what a bf16 output
+    # layer followed by .float() delivers: one read of the row), fp32 values with low bits (the row is read again), and
+    # rows of both kinds next to each other, one of them with a single low bit in its last element
+    (151936, torch.float32, 600, "widened"), (151936, torch.float32, 600, "plain"), (151936, torch.float32, 600, "mixed")])
 @pytest.mark.parametrize("pattern", ["all_dead", "one_live_last", "few_live", "random", "all_live_no_map",
                                      "zero_advantage"])
-def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dtype, n_rows):
+def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dtype, n_rows, values):
     """The two kernels behind relax_amd_actor_step_fused, switched with relax_amd_set_kernel_choice, on row / token
     layouts that stress the persistent loop of the register-resident one: no live row at all, a single live row at
     the very end, fewer live rows than workgroups, random prompt rows and masked tokens over several rows per
@@ -1731,7 +1736,14 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
     dev = require_gpu()
     announce("resident vs two-walk", pattern, v, dtype)
     g = torch.Generator().manual_seed(len(pattern))
-    logits = (torch.randn(n_rows, v, generator=g) * 2).to(dtype).to(dev)
+    logits = (torch.randn(n_rows, v, generator=g) * 2).to(dtype)
+    if values in ("widened", "mixed"):
+        logits = logits.bfloat16().to(dtype)
+    if values == "mixed":
+        other = torch.randn(n_rows // 3, v, generator=g) * 2
+        logits[1::3][: other.size(0)] = other  # every third row keeps its low bits
+        logits[2::3, -1] += 2.0 ** -14         # and the next one differs from a widened row in one bit of one element
+    logits = logits.to(dev)
     if pattern == "all_live_no_map":
         token_of_row, n_tok = None, n_rows
     else:
@@ -1776,6 +1788,65 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
         assert torch.equal(got, want), (pattern, key, (got.float() - want.float()).abs().max())
     if pattern == "all_dead":
         assert not results["resident"]["d"].any()
+
+
+@pytest.mark.parametrize("v", [128256, 129280, 131072, 152064, 163840, 4 * (31 * 1024 + 1), 4 * (38 * 1024 - 1)])
+def test_long_fp32_rows_resident_as_upper_halves_equal_two_walk_kernel_and_oracle(v):
+    """The other row shapes of the kernel that keeps long fp32 rows as their upper halves (31 / 37 full vector
+    positions per thread plus a partial one, 32 and 40 exactly; one lane or all lanes but one at the partial
+    position): widened-bf16 rows and rows with low bits interleaved, every output bit-identical to the two-walk
+    kernel's; log-probs, entropy and the gradient of the widened rows against the oracle."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("long fp32 rows, upper halves", v)
+    n_rows = 330
+    g = torch.Generator().manual_seed(v)
+    logits = (torch.randn(n_rows, v, generator=g) * 2).bfloat16().float()
+    logits[1::2] += torch.randn(n_rows // 2, v, generator=g) * 1e-3  # odd rows: real fp32 values
+    logits = logits.to(dev)
+    scores = torch.rand(n_rows, generator=g) > 0.2
+    idx = torch.cumsum(scores.int(), 0) - 1
+    token_of_row = torch.where(scores, idx, torch.full_like(idx, -1)).int().to(dev)
+    n_tok = int(scores.sum())
+    mask = (torch.rand(n_tok, generator=g) > 0.2).float()
+    adv = torch.randn(n_tok, generator=g)
+    base = -12.0 + 0.3 * torch.randn(n_tok, generator=g)
+    targets = torch.randint(0, v, (n_tok,), generator=g)
+    targets[:4] = torch.tensor([0, v - 1, v - 2, 4096 * ((v - 1) // 4096)])  # first / last elements, last position
+    cu = torch.tensor([0, n_tok], dtype=torch.int64, device=dev)
+    kw = dict(advantages=adv.to(dev), loss_mask=mask.to(dev), cu_resp=cu, old_log_prob=base.to(dev),
+              ref_log_prob=(base + 0.1 * torch.randn(n_tok, generator=g)).to(dev), kl_kind="k3", kl_coef=1e-3,
+              entropy_coef=0.01, sample_denom=torch.tensor([max(1.0, mask.sum().item())], device=dev),
+              loss_kind="ppo", eps_clip=0.2, eps_clip_high=0.28)
+    sample_ids = torch.zeros(n_tok, dtype=torch.int32, device=dev)
+    results = {}
+    for kind in ("two_walk", "resident"):
+        ops.set_kernel_choice(kind)
+        out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets.to(dev), token_of_row, sample_ids, n_tok, 1.0,
+                                                         1.0, **kw)
+        torch.cuda.synchronize()
+        results[kind] = dict(lp=lp, ent=ent, lse=lse, spx=spx, coef=out["coef_log_prob"], d=d.view(torch.int32))
+    for key, want in results["two_walk"].items():
+        got = results["resident"][key]
+        assert torch.equal(got, want), (key, (got.float() - want.float()).abs().max())
+    # oracle on the scored rows: log-probs / entropy of every live token, gradient rows of a few tokens
+    rows = torch.nonzero(scores).squeeze(1)
+    x = logits[rows.to(dev)].cpu()
+    ls = torch.log_softmax(x.double(), -1)
+    want_lp = ls[torch.arange(n_tok), targets].float()
+    want_ent = -(ls.exp() * ls).sum(-1).float()
+    live = mask != 0
+    torch.testing.assert_close(results["resident"]["lp"].cpu()[live], want_lp[live], atol=2e-5, rtol=0)
+    torch.testing.assert_close(results["resident"]["ent"].cpu()[live], want_ent[live], atol=2e-5, rtol=0)
+    d = results["resident"]["d"].view(torch.float32)
+    coef, coef_ent = out["coef_log_prob"].cpu().double(), out["coef_entropy"].cpu().double()
+    for t in [int(i) for i in torch.nonzero(live).squeeze(1)[:6]]:
+        p = ls[t].exp()
+        onehot = torch.zeros(v, dtype=torch.float64)
+        onehot[targets[t]] = 1.0
+        want = coef[t] * (onehot - p) + coef_ent[t] * p * ((p * x[t].double()).sum() - x[t].double())
+        torch.testing.assert_close(d[rows[t]].cpu().double(), want, atol=2e-6, rtol=1e-4)
 
 
 @pytest.mark.parametrize("v,dtype", [(8 * (18 * 1024 + 1), torch.bfloat16), (8 * (19 * 1024 - 1), torch.bfloat16),
