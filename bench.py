@@ -16,7 +16,10 @@ reports them inside that line as ``other_workloads``; ``--no-secondary`` or ``--
 ``cfg1`` (GRPO plumbing case: 512 responses x 256 tokens, fp32 logits [131072, 32000], rewards -> advantages -> loss),
 ``lmhead`` (fused LM-head + log-prob/entropy forward and dhidden/dweight backward, hidden [32768, 4096], MFMA-bound),
 ``reverse_kl`` (on-policy distillation, student/teacher [16384, 151936], forward + student dlogits),
-``varlen_gspo`` / ``varlen_cispo`` (8 packed sequences of 2k-32k tokens, RLOO advantages, sequence-level losses).
+``varlen_gspo`` / ``varlen_cispo`` (8 packed sequences of 2k-32k tokens, RLOO advantages, sequence-level losses),
+``actor_fwd`` (the forward-only log-prob pass of the ActorFwd / Reference roles over the actor step's logits),
+``actor_fwd_topk`` (the same pass with entropy and the student's top-K ids), ``actor_step_opd_topk`` (the actor step
+with the top-64 on-policy-distillation term).
 """
 
 from __future__ import annotations
@@ -538,6 +541,33 @@ def run_lmhead(a, dev) -> None:
          None)
 
 
+def run_actor_fwd(a, dev) -> None:
+    """The forward-only pass of the ActorFwd / Reference roles (forward_only(get_log_probs_and_entropy), with
+    ``use_rollout_entropy`` off as by default): log-probs of every response row of the actor-step logits, no entropy,
+    no gradient."""
+    import relax_amd
+
+    args = make_args()
+    logits, batch, _ = make_workload(dev, a.seqs, a.seq_len, a.vocab)
+    n_tokens = a.seqs * a.seq_len
+
+    def step():
+        with torch.no_grad():
+            _, out = relax_amd.get_log_probs_and_entropy(
+                logits, args=args, unconcat_tokens=batch["unconcat_tokens"], total_lengths=batch["total_lengths"],
+                response_lengths=batch["response_lengths"], with_entropy=False)
+        return out["log_probs"][-1][-1]
+
+    wall, kernel_ms, _, _ = timed_steps(step, a.warmup, a.steps)
+    row_bytes = float(a.vocab * logits.element_size()) * n_tokens
+    emit(a, n_tokens, wall,
+         f"forward-only log-probs (ActorFwd / Reference roles): {a.seqs} seqs x {a.seq_len} tokens x V={a.vocab} bf16 "
+         f"logits, no entropy, no gradient",
+         {"rows": n_tokens, "vocab": a.vocab},
+         hbm_roofline("logprob_entropy_fwd_kernel<bf16_t, true, 1024, false>", kernel_ms["logprob_entropy_fwd"],
+                      row_bytes, n_tokens, a.vocab, kernel_ms, wall * 1e3 / a.steps), None)
+
+
 def run_actor_fwd_topk(a, dev) -> None:
     """The forward-only pass the actor runs when it also collects the student's top-K ids for on-policy distillation
     (compute_log_prob(collect_topk=True)): log-probs + entropy and ``topk_token_ids`` of every response row of the
@@ -781,7 +811,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="actor_step",
                     choices=["actor_step", "actor_step_opd_topk", "actor_step_fp32", "cfg1", "lmhead", "reverse_kl", "varlen_gspo",
-                             "varlen_cispo", "actor_fwd_topk"])
+                             "varlen_cispo", "actor_fwd", "actor_fwd_topk"])
     ap.add_argument("--seqs", type=int, default=SEQS)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
     ap.add_argument("--vocab", type=int, default=VOCAB)
@@ -873,6 +903,8 @@ def run_workload(a, dev) -> None:
         run_lmhead(a, dev)
     elif a.workload == "reverse_kl":
         run_reverse_kl(a, dev)
+    elif a.workload == "actor_fwd":
+        run_actor_fwd(a, dev)
     elif a.workload == "actor_fwd_topk":
         run_actor_fwd_topk(a, dev)
     else:
@@ -880,8 +912,8 @@ def run_workload(a, dev) -> None:
 
 
 SECONDARY_TRAFFIC = {}  # workload -> collect_live_traffic() result, filled by the plain invocation before it touches the GPU
-SECONDARY = ("lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "cfg1", "actor_fwd_topk", "actor_step_opd_topk",
-             "actor_step_fp32")
+SECONDARY = ("lmhead", "reverse_kl", "varlen_gspo", "varlen_cispo", "cfg1", "actor_fwd", "actor_fwd_topk",
+             "actor_step_opd_topk", "actor_step_fp32")
 
 
 def run_default_with_secondary(a, dev) -> int:

@@ -22,7 +22,10 @@ namespace relax_amd {
 constexpr int kRowThreads = 256;  // backward kernel width
 constexpr int kRowUnroll = 4;
 
-template <typename T, bool VEC, int THREADS>
+// WITH_T = false: neither the entropy nor sum p*x is wanted (the forward-only pass of the ActorFwd / Reference roles,
+// relax/backends/megatron/model.py:844 with use_rollout_entropy off): the scan drops that sum, log_prob and lse are
+// the same bits.
+template <typename T, bool VEC, int THREADS, bool WITH_T = true>
 __global__ __launch_bounds__(THREADS) void logprob_entropy_fwd_kernel(
     const T* __restrict__ logits, int64_t row_stride, int64_t vocab, const int32_t* __restrict__ row_ids,
     const int64_t* __restrict__ targets, float c, float inv_t, float* __restrict__ log_prob,
@@ -37,14 +40,14 @@ __global__ __launch_bounds__(THREADS) void logprob_entropy_fwd_kernel(
     tg = targets[tok];
     if (tg >= 0 && tg < vocab) x_target = Row<T>::load1(x + tg);
   }
-  SoftmaxAcc st = scan_row<T, VEC, true, THREADS>(x, vocab, c);
+  SoftmaxAcc st = scan_row<T, VEC, true, THREADS, ScanNoHook, WITH_T>(x, vocab, c);
   scan_block_merge<THREADS>(st, wave_state);
   if (threadIdx.x == 0) {
     float lse, spx, ent, lp;
     scan_finish(st, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
     log_prob[tok] = lp;
-    if (entropy) entropy[tok] = ent;
-    if (spx_out) spx_out[tok] = spx;
+    if (WITH_T && entropy) entropy[tok] = ent;
+    if (WITH_T && spx_out) spx_out[tok] = spx;
     if (lse_out) lse_out[tok] = lse;
   }
 }
@@ -153,9 +156,14 @@ static int launch_fwd(const void* logits, int64_t n, int64_t vocab, int64_t stri
   const float c = inv_t * kLog2e;
   const T* x = static_cast<const T*>(logits);
   dim3 grid(static_cast<unsigned>(n));
+  const bool with_t = ent || spx;  // neither asked for: the scan leaves sum p*x out
 #define RELAX_AMD_FWD(V, TH)                                                                                        \
-  hipLaunchKernelGGL((logprob_entropy_fwd_kernel<T, V, TH>), grid, dim3(TH), 0, s, x, stride, vocab, row_ids, targets, \
-                     c, inv_t, lp, ent, lse, spx)
+  if (with_t || !V)                                                                                                 \
+    hipLaunchKernelGGL((logprob_entropy_fwd_kernel<T, V, TH, true>), grid, dim3(TH), 0, s, x, stride, vocab, row_ids, \
+                       targets, c, inv_t, lp, ent, lse, spx);                                                       \
+  else                                                                                                              \
+    hipLaunchKernelGGL((logprob_entropy_fwd_kernel<T, V, TH, false>), grid, dim3(TH), 0, s, x, stride, vocab,       \
+                       row_ids, targets, c, inv_t, lp, ent, lse, spx)
   if (!vec) {
     RELAX_AMD_FWD(false, 256);
   } else {

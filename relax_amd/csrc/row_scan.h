@@ -16,7 +16,9 @@ struct SoftmaxAcc {
 };
 
 // Returns the largest of the K values (a float maximum: NaN passes unnoticed here and shows in st.s instead).
-template <int K>
+// WITH_T = false leaves st.t alone (callers that want neither the entropy nor sum p*x: one multiply-add per element
+// less); st.m and st.s, and with them the log-sum-exp, are the same bits either way.
+template <int K, bool WITH_T = true>
 __device__ __forceinline__ float scan_absorb(const float (&v)[K], float c, SoftmaxAcc& st) {
   float vmax = v[0];
 #pragma unroll
@@ -25,14 +27,14 @@ __device__ __forceinline__ float scan_absorb(const float (&v)[K], float c, Softm
   if (mc > st.m) {
     const float sc = fast_exp2(__fsub_rn(st.m, mc));
     st.s = __fmul_rn(st.s, sc);
-    st.t = __fmul_rn(st.t, sc);
+    if (WITH_T) st.t = __fmul_rn(st.t, sc);
     st.m = mc;
   }
 #pragma unroll
   for (int i = 0; i < K; ++i) {
     const float e = fast_exp2(fmaf(v[i], c, -st.m));
     st.s = __fadd_rn(st.s, e);
-    st.t = fmaf(e, v[i], st.t);
+    if (WITH_T) st.t = fmaf(e, v[i], st.t);
   }
   return vmax;
 }
@@ -55,7 +57,7 @@ struct ScanNoHook {
 // Per-lane state over one row.  VEC: 16-byte loads (row base and stride 16-byte aligned) for the whole vectors and
 // scalar loads for the tail; otherwise scalar loads throughout.  STREAM selects non-temporal loads (row not needed
 // again soon) or ordinary cached loads (a second pass over the row follows immediately); it does not change results.
-template <typename T, bool VEC, bool STREAM, int THREADS, typename Hook = ScanNoHook>
+template <typename T, bool VEC, bool STREAM, int THREADS, typename Hook = ScanNoHook, bool WITH_T = true>
 __device__ __forceinline__ SoftmaxAcc scan_row(const T* __restrict__ x, int64_t vocab, float c, Hook&& hook = Hook()) {
   SoftmaxAcc st{kNegHuge, 0.f, 0.f};
   if (VEC) {
@@ -76,21 +78,21 @@ __device__ __forceinline__ SoftmaxAcc scan_row(const T* __restrict__ x, int64_t 
 #pragma unroll
         for (int k = 0; k < VN; ++k) v[u * VN + k] = part[k];
       }
-      hook.absorbed(scan_absorb(v, c, st));
+      hook.absorbed(scan_absorb<sizeof(v) / sizeof(float), WITH_T>(v, c, st));
     }
     for (; i < nvec; i += THREADS) {
       float v[VN];
       Row<T>::unpack(STREAM ? load_stream(xv + i) : xv[i], v);
-      hook.absorbed(scan_absorb(v, c, st));
+      hook.absorbed(scan_absorb<sizeof(v) / sizeof(float), WITH_T>(v, c, st));
     }
     for (int64_t e = nvec * VN + threadIdx.x; e < vocab; e += THREADS) {
       float v[1] = {Row<T>::load1(x + e)};
-      hook.absorbed(scan_absorb(v, c, st));
+      hook.absorbed(scan_absorb<sizeof(v) / sizeof(float), WITH_T>(v, c, st));
     }
   } else {
     for (int64_t e = threadIdx.x; e < vocab; e += THREADS) {
       float v[1] = {Row<T>::load1(x + e)};
-      hook.absorbed(scan_absorb(v, c, st));
+      hook.absorbed(scan_absorb<sizeof(v) / sizeof(float), WITH_T>(v, c, st));
     }
   }
   return st;
