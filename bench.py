@@ -212,7 +212,7 @@ def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
             and KERNEL_CHOICE != "two_walk":
         return f"actor_step_resident_kernel<{dtype}, {shape[0]}, {str(shape[1]).lower()}>"
     if dtype == "float" and vocab % 4 == 0 and threads == 1024 and KERNEL_CHOICE != "two_walk" \
-            and shape in ((37, True), (31, True), (32, False), (40, False)):
+            and shape in ((37, True), (31, True), (32, False), (40, False), (24, True), (25, False)):
         # long fp32 rows, resident as their upper halves
         return f"actor_step_resident_wide_kernel<{shape[0]}, {str(shape[1]).lower()}>"
     return f"actor_step_fused_kernel<{dtype}, true, {threads}>"

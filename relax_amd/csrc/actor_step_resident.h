@@ -20,7 +20,7 @@ int launch_actor_step_resident(const T* logits, int64_t row_stride, int64_t voca
                                float* entropy, float* lse, float* spx, T* dlogits, int64_t d_stride,
                                int compute_units, hipStream_t stream);
 
-// The same for fp32 rows of 128256 .. 163840 entries, kept in the registers as their upper halves when those are all
+// The same for fp32 rows of 100352 .. 163840 entries, kept in the registers as their upper halves when those are all
 // there is to them (actor_step_resident_wide.hip).
 int launch_actor_step_resident_wide(const float* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
                                     const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,

@@ -1,4 +1,4 @@
-// Register-resident fused actor step for fp32 rows too long to sit in the registers as fp32: rows of 128256 ..
+// Register-resident fused actor step for fp32 rows too long to sit in the registers as fp32: rows of 100352 ..
 // 163840 entries, the vocabularies a stock Megatron model hands a custom loss as fp32 [1, T, V] logits
 // (relax/backends/megatron/loss.py:92-97 asserts the dtype).  Same computation, same outputs, bit for bit, as
 // actor_step_fused_kernel<float> (log-prob + entropy forward, per-token policy-loss coefficients, dlogits backward;
@@ -53,7 +53,8 @@ struct WideTokenData {
 
 }  // namespace
 
-// NF full vector positions per thread plus one partially filled position when PARTIAL; NF + PARTIAL is even.
+// NF full vector positions per thread plus one partially filled position when PARTIAL.  Positions are packed in pairs;
+// with an odd count the last register quad is half used.
 template <int NF, bool PARTIAL>
 __global__ __launch_bounds__(kWideThreads, 4) void actor_step_resident_wide_kernel(
     const float* __restrict__ logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
@@ -63,8 +64,8 @@ __global__ __launch_bounds__(kWideThreads, 4) void actor_step_resident_wide_kern
     float* __restrict__ spx_out, float* __restrict__ dlogits, int64_t d_stride) {
   constexpr int THREADS = kWideThreads, kU = kScanUnroll;
   constexpr int NP = NF + (PARTIAL ? 1 : 0);  // vector positions per thread
-  static_assert(NP % 2 == 0 && kU == 4, "positions are packed in pairs and scanned in groups of four");
-  constexpr int NR = NP / 2;                  // packed registers-quads
+  static_assert(kU == 4, "positions are packed in pairs and scanned in groups of four");
+  constexpr int NR = (NP + 1) / 2;            // packed registers-quads
   constexpr int kGroups = (NP + kU - 1) / kU;
   __shared__ float wave_state[THREADS / kWave][3];
   __shared__ uint32_t wave_inexact[THREADS / kWave];
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(kWideThreads, 4) void actor_step_resident_wide_kern
         const int p = kU * g + u;
         int lane_id = tid;
         asm volatile("" : "+v"(lane_id));
-        if (p < NP) land[g & 1][u] = has(p) ? load_stream(xv + lane_id + p * THREADS) : u32x4{0u, 0u, 0u, 0u};
+        land[g & 1][u] = (p < NP && has(p)) ? load_stream(xv + lane_id + p * THREADS) : u32x4{0u, 0u, 0u, 0u};
       }
     };
     request(0);
@@ -319,11 +320,14 @@ int launch_actor_step_resident_wide(const float* logits, int64_t row_stride, int
   const int full = int(nvec / kWideThreads);
   const bool partial = nvec % kWideThreads != 0;
   const dim3 grid(static_cast<unsigned>(n_rows < compute_units ? n_rows : compute_units)), block(kWideThreads);
-  // 151936 / 152064 (37984 / 38016 vectors), 128256 / 129280 (32064 / 32320), 131072 (32768), 163840 (40960)
+  // 151936 / 152064 (37984 / 38016 vectors), 128256 / 129280 (32064 / 32320), 131072 (32768), 163840 (40960),
+  // 100352 / 102400 (25088 / 25600)
   RELAX_AMD_WIDE(37, true)
   RELAX_AMD_WIDE(31, true)
   RELAX_AMD_WIDE(32, false)
   RELAX_AMD_WIDE(40, false)
+  RELAX_AMD_WIDE(24, true)
+  RELAX_AMD_WIDE(25, false)
   return RELAX_AMD_EUNSUPPORTED;
 }
 #undef RELAX_AMD_WIDE

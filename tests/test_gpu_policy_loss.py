@@ -1790,11 +1790,12 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
         assert not results["resident"]["d"].any()
 
 
-@pytest.mark.parametrize("v", [128256, 129280, 131072, 152064, 163840, 4 * (31 * 1024 + 1), 4 * (38 * 1024 - 1)])
+@pytest.mark.parametrize("v", [128256, 129280, 131072, 152064, 163840, 4 * (31 * 1024 + 1), 4 * (38 * 1024 - 1),
+                               100352, 102400, 4 * (24 * 1024 + 1)])
 def test_long_fp32_rows_resident_as_upper_halves_equal_two_walk_kernel_and_oracle(v):
-    """The other row shapes of the kernel that keeps long fp32 rows as their upper halves (31 / 37 full vector
-    positions per thread plus a partial one, 32 and 40 exactly; one lane or all lanes but one at the partial
-    position): widened-bf16 rows and rows with low bits interleaved, every output bit-identical to the two-walk
+    """The other row shapes of the kernel that keeps long fp32 rows as their upper halves (24 / 31 / 37 full vector
+    positions per thread plus a partial one, 25, 32 and 40 exactly; an odd number of positions leaves the last register
+    quad half used; one lane or all lanes but one at the partial position): widened-bf16 rows and rows with low bits interleaved, every output bit-identical to the two-walk
     kernel's; log-probs, entropy and the gradient of the widened rows against the oracle."""
     from relax_amd import ops
 
