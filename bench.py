@@ -100,26 +100,39 @@ def _pmc_pass(counter: str, argv: list, outdir: str, limit_s: int):
     prof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
     if not os.path.exists(prof):
         return None, "rocprofv3 not found"
-    cmd = ["timeout", "-s", "KILL", str(limit_s), prof, "--pmc", counter, "-d", outdir, "-o", "p", "--output-format",
-           "csv", "--", sys.executable, os.path.abspath(__file__), *argv]
+    import signal
+
+    cmd = [prof, "--pmc", counter, "-d", outdir, "-o", "p", "--output-format", "csv", "--", sys.executable,
+           os.path.abspath(__file__), *argv]
     env = dict(os.environ, TMPDIR="/tmp")
     try:
-        r = subprocess.run(cmd, cwd="/tmp", env=env, capture_output=True, text=True, timeout=limit_s + 30)
-    except (OSError, subprocess.TimeoutExpired) as e:
+        # its own process group, so that a pass that overruns is ended together with the program it profiles
+        proc = subprocess.Popen(cmd, cwd="/tmp", env=env, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                                start_new_session=True)
+    except OSError as e:
         return None, f"{type(e).__name__}: {e}"
+    try:
+        out, err = proc.communicate(timeout=limit_s)
+    except subprocess.TimeoutExpired:
+        try:
+            os.killpg(proc.pid, signal.SIGKILL)
+        except ProcessLookupError:
+            pass
+        proc.communicate()
+        return None, f"no result within {limit_s} s"
     files = glob.glob(os.path.join(outdir, "**", "*counter_collection.csv"), recursive=True)
-    if r.returncode != 0 or not files:
-        return None, f"rocprofv3 exit {r.returncode}: {(r.stderr or r.stdout)[-300:]}"
+    if proc.returncode != 0 or not files:
+        return None, f"rocprofv3 exit {proc.returncode}: {(err or out)[-300:]}"
     dispatches = []  # (kernel name, workgroups, counter value)
     with open(files[0], newline="") as f:
         for row in csv.DictReader(f):
             if row.get("Counter_Name") == counter:
                 groups = int(row["Grid_Size"]) // max(1, int(row["Workgroup_Size"]))
                 dispatches.append((row["Kernel_Name"], groups, float(row["Counter_Value"])))
-    return dispatches, " ".join(cmd[3:])
+    return dispatches, " ".join(cmd)
 
 
-def collect_live_traffic(argv: list, limit_s: int = 170):
+def collect_live_traffic(argv: list, limit_s: int = 90):
     """HBM-side bytes per launch of the step's kernels, measured in THIS run: two child runs of this file under
     ``rocprofv3 --pmc`` (FETCH_SIZE, then WRITE_SIZE: one counter per run), each scaled by what the same counter reads
     for the known-size launch the child makes before its timed step (``known_size_streams``).  Must be called before this process touches the GPU.
@@ -865,10 +878,14 @@ def main() -> int:
             return child
 
         LIVE_TRAFFIC = collect_live_traffic(child_args(a.workload))
-        if plain:  # the bandwidth-bound configurations that ride along get their own counter passes
+        if plain and "error" not in LIVE_TRAFFIC:
+            # the bandwidth-bound configurations that ride along get their own counter passes (a few seconds each);
+            # the first pass that fails ends the series, so a box without a working profiler costs one time limit
             for name in SECONDARY:
                 if name != "lmhead":
                     SECONDARY_TRAFFIC[name] = collect_live_traffic(child_args(name))
+                    if "error" in SECONDARY_TRAFFIC[name]:
+                        break
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         return 2
