@@ -232,8 +232,11 @@ def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
 
 
 def bwd_kernel_name(vocab: int) -> str:
-    """Which kernel relax_amd_logprob_entropy_bwd runs for bf16 rows of ``vocab`` entries (the library's rule: the
-    persistent burst form for the row shapes of the register-resident step)."""
+    """Which kernel relax_amd_logprob_entropy_bwd runs for bf16 rows of ``vocab`` entries (the library's rule: one-shot
+    workgroups over 4 KB chunks for rows of whole vectors; with ``--kernel-choice resident`` the persistent burst form
+    for the row shapes of the register-resident step; with ``two_walk`` the row-per-workgroup loop)."""
+    if KERNEL_CHOICE == "auto" and vocab % 8 == 0:
+        return "logprob_entropy_bwd_chunk_kernel<bf16_t>"
     name = fused_step_kernel_name(vocab)
     if name.startswith("actor_step_resident_kernel"):
         return name.replace("actor_step_resident_kernel", "logprob_entropy_bwd_resident_kernel")
@@ -653,7 +656,8 @@ def run_reverse_kl(a, dev) -> None:
         dom, dom_name, necessary = kernel_ms["reverse_kl_step_fused"], kl_step_kernel_name(v), 3.0 * row_bytes * n
         two_pass = 5.0 * row_bytes * n  # forward read of both rows, backward re-read of both, gradient write
     else:
-        dom, dom_name, necessary = kernel_ms["reverse_kl_bwd"], "reverse_kl_bwd_kernel<bf16_t, true>", 3.0 * row_bytes * n
+        dom_name = "reverse_kl_bwd_kernel<bf16_t, true>" if KERNEL_CHOICE == "two_walk" else "reverse_kl_bwd_chunk_kernel<bf16_t>"
+        dom, necessary = kernel_ms["reverse_kl_bwd"], 3.0 * row_bytes * n
         two_pass = None
     emit(a, n, wall,
          f"on-policy distillation: student/teacher bf16 logits [{n}, {v}], full-vocab reverse KL, token-mean, fwd + "

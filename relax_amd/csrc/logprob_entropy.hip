@@ -148,6 +148,56 @@ __global__ __launch_bounds__(kRowThreads) void logprob_entropy_bwd_kernel(
   }
 }
 
+// The same backward in the form the memory system serves fastest when nothing has to stay on chip between a row's
+// read and its write: workgroups of 256 threads that each take 4 KB of a row (one 16-byte vector per thread), in
+// address order over rows and chunks, and exit.  At any moment the chip as a whole sweeps a short window of
+// consecutive addresses instead of one row-sized stream per CU.  The row's coefficients come from uniform (scalar)
+// loads; rows without gradient are written as zeros without a read.  Same arithmetic per element as the kernel above.
+constexpr int kChunkThreads = 256;
+template <typename T>
+__global__ __launch_bounds__(kChunkThreads) void logprob_entropy_bwd_chunk_kernel(
+    const T* __restrict__ logits, int64_t row_stride, int64_t nvec, unsigned chunks_per_row,
+    const int32_t* __restrict__ token_of_row, const int64_t* __restrict__ targets, const float* __restrict__ lse,
+    const float* __restrict__ spx, const float* __restrict__ g_lp, const float* __restrict__ g_ent, float grad_scale,
+    const float* __restrict__ grad_scale_dev, float c, float inv_t, T* __restrict__ dlogits, int64_t d_stride) {
+  constexpr int VN = Row<T>::kPerVec;
+  const unsigned b = blockIdx.x;
+  const unsigned row = b / chunks_per_row, chunk = b - row * chunks_per_row;
+  const int64_t i = int64_t(chunk) * kChunkThreads + threadIdx.x;
+  if (i >= nvec) return;
+  u32x4* dv = reinterpret_cast<u32x4*>(dlogits + int64_t(row) * d_stride);
+  const int64_t tok = token_of_row ? int64_t(token_of_row[row]) : int64_t(row);
+  float glp = 0.f, gh = 0.f;
+  if (tok >= 0) {
+    if (grad_scale_dev) grad_scale *= *grad_scale_dev;
+    glp = g_lp[tok] * grad_scale;
+    gh = g_ent ? g_ent[tok] * grad_scale : 0.f;
+  }
+  if (tok < 0 || (glp == 0.f && gh == 0.f)) {
+    store_stream(dv + i, u32x4{0u, 0u, 0u, 0u});
+    return;
+  }
+  const u32x4 raw = load_stream(reinterpret_cast<const u32x4*>(logits + int64_t(row) * row_stride) + i);
+  const float k0 = -lse[tok] * kLog2e;
+  const float bb = gh * inv_t;
+  const float a0 = -glp * inv_t + (gh != 0.f ? bb * spx[tok] : 0.f);
+  const float a1 = -bb * inv_t;
+  const float hot = glp * inv_t;
+  const int64_t tg = targets[tok];
+  const int64_t tvec = (tg >= 0 && tg < nvec * VN) ? tg / VN : -1;
+  const int tsub = int(tg % VN);
+  float v[VN];
+  Row<T>::unpack(raw, v);
+#pragma unroll
+  for (int k = 0; k < VN; ++k) v[k] = fast_exp2(fmaf(v[k], c, k0)) * fmaf(v[k], a1, a0);
+  if (i == tvec) {
+#pragma unroll
+    for (int k = 0; k < VN; ++k)
+      if (k == tsub) v[k] += hot;
+  }
+  store_stream(dv + i, Row<T>::pack(v));
+}
+
 template <typename T>
 static int launch_fwd(const void* logits, int64_t n, int64_t vocab, int64_t stride, const int32_t* row_ids,
                       const int64_t* targets, float inv_t, float* lp, float* ent, float* lse, float* spx,
@@ -188,10 +238,21 @@ static int launch_bwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t
   dim3 grid(static_cast<unsigned>(n_rows)), block(kRowThreads);
   const T* x = static_cast<const T*>(logits);
   T* d = static_cast<T*>(dlogits);
-  // Long rows of the built shapes take the persistent burst form (same bits, faster).  relax_amd_set_kernel_choice:
-  // TWO_WALK keeps every row length on the row-per-workgroup kernel, RESIDENT fails where the burst form is not
-  // built (for tests that compare the two).
+  // Rows of whole 16-byte vectors take the chunk form (same bits, fastest).  relax_amd_set_kernel_choice: TWO_WALK
+  // keeps every row length on the row-per-workgroup kernel; RESIDENT asks for the persistent burst form and fails
+  // where it is not built (for tests that compare the forms).
   const int choice = kernel_choice();
+  constexpr int VN = Row<T>::kPerVec;
+  if (vec && choice == RELAX_AMD_KERNEL_AUTO && vocab % VN == 0) {
+    const int64_t nvec = vocab / VN;
+    const int64_t chunks = (nvec + kChunkThreads - 1) / kChunkThreads;
+    if (n_rows * chunks <= 2147483647LL) {
+      hipLaunchKernelGGL((logprob_entropy_bwd_chunk_kernel<T>), dim3(static_cast<unsigned>(n_rows * chunks)),
+                         dim3(kChunkThreads), 0, s, x, stride, nvec, static_cast<unsigned>(chunks), token_of_row,
+                         targets, lse, spx, g_lp, g_ent, grad_scale, grad_scale_dev, c, inv_t, d, d_stride);
+      return check_launch("logprob_entropy_bwd");
+    }
+  }
   if (vec && choice != RELAX_AMD_KERNEL_TWO_WALK) {
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess ||

@@ -98,6 +98,40 @@ __global__ __launch_bounds__(kKlThreads) void reverse_kl_fwd_kernel(const T* __r
   }
 }
 
+// The same backward as one-shot workgroups of 256 threads that each take 4 KB of a row (one 16-byte vector of both
+// inputs per thread) in address order and exit: the form the memory system serves fastest when nothing has to stay on
+// chip between a row's reads and its write.  Rows without gradient are written as zeros without a read.
+constexpr int kKlChunkThreads = 256;
+template <typename T>
+__global__ __launch_bounds__(kKlChunkThreads) void reverse_kl_bwd_chunk_kernel(
+    const T* __restrict__ student, const T* __restrict__ teacher, int64_t stride, int64_t nvec, unsigned chunks_per_row,
+    const float* __restrict__ kl, const float* __restrict__ lse_s, const float* __restrict__ lse_t,
+    const float* __restrict__ g, float grad_scale, const float* __restrict__ grad_scale_dev,
+    T* __restrict__ dstudent) {
+  constexpr int VN = Row<T>::kPerVec;
+  const unsigned b = blockIdx.x;
+  const unsigned tok = b / chunks_per_row, chunk = b - tok * chunks_per_row;
+  const int64_t i = int64_t(chunk) * kKlChunkThreads + threadIdx.x;
+  if (i >= nvec) return;
+  u32x4* dv = reinterpret_cast<u32x4*>(dstudent + int64_t(tok) * stride);
+  if (grad_scale_dev) grad_scale *= *grad_scale_dev;
+  const float gt = g[tok] * grad_scale;
+  if (gt == 0.f) {
+    store_stream(dv + i, u32x4{0u, 0u, 0u, 0u});
+    return;
+  }
+  const u32x4 rs = load_stream(reinterpret_cast<const u32x4*>(student + int64_t(tok) * stride) + i);
+  const u32x4 rt = load_stream(reinterpret_cast<const u32x4*>(teacher + int64_t(tok) * stride) + i);
+  const float k0 = -lse_s[tok] * kLog2e;
+  const float k1 = gt * (lse_t[tok] - lse_s[tok] - kl[tok]);
+  float a[VN], bb[VN];
+  Row<T>::unpack(rs, a);
+  Row<T>::unpack(rt, bb);
+#pragma unroll
+  for (int k = 0; k < VN; ++k) a[k] = fast_exp2(fmaf(a[k], kLog2e, k0)) * fmaf(a[k] - bb[k], gt, k1);
+  store_stream(dv + i, Row<T>::pack(a));
+}
+
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kKlThreads) void reverse_kl_bwd_kernel(
     const T* __restrict__ student, const T* __restrict__ teacher, int64_t stride, int64_t vocab,
@@ -363,6 +397,18 @@ static int launch_kl_bwd(const void* s, const void* t, int64_t n, int64_t vocab,
                          void* d, hipStream_t st) {
   const bool vec = aligned16(s) && aligned16(t) && aligned16(d) && (stride * int64_t(sizeof(T))) % 16 == 0;
   dim3 grid(static_cast<unsigned>(n)), block(kKlThreads);
+  // rows of whole 16-byte vectors: the chunk form (same bits); relax_amd_set_kernel_choice(TWO_WALK) keeps the
+  // row-per-workgroup loop for comparisons
+  if (vec && vocab % Row<T>::kPerVec == 0 && kernel_choice() != RELAX_AMD_KERNEL_TWO_WALK) {
+    const int64_t nvec = vocab / Row<T>::kPerVec;
+    const int64_t chunks = (nvec + kKlChunkThreads - 1) / kKlChunkThreads;
+    if (n * chunks <= 2147483647LL) {
+      hipLaunchKernelGGL((reverse_kl_bwd_chunk_kernel<T>), dim3(static_cast<unsigned>(n * chunks)),
+                         dim3(kKlChunkThreads), 0, st, static_cast<const T*>(s), static_cast<const T*>(t), stride, nvec,
+                         static_cast<unsigned>(chunks), kl, ls, lt, g, scale, scale_dev, static_cast<T*>(d));
+      return check_launch("reverse_kl_bwd");
+    }
+  }
   if (vec)
     hipLaunchKernelGGL((reverse_kl_bwd_kernel<T, true>), grid, block, 0, st, static_cast<const T*>(s),
                        static_cast<const T*>(t), stride, vocab, kl, ls, lt, g, scale, scale_dev, static_cast<T*>(d));

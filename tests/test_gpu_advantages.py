@@ -370,6 +370,33 @@ def test_opd_kl_topk_vs_oracle(kl_type, alpha, norm_mode, masked, clamp):
     torch.testing.assert_close(sd.grad.cpu(), sc.grad, atol=2e-5 * gscale, rtol=2e-4)
 
 
+@pytest.mark.parametrize("v,dtype,n", [(151936, torch.bfloat16, 300), (4100 * 8, torch.float16, 200),
+                                       (32000, torch.float32, 300), (8 * 255, torch.bfloat16, 50)])
+def test_reverse_kl_backward_chunk_form_equals_row_per_workgroup_kernel_bitwise(v, dtype, n):
+    """The two kernels behind relax_amd_reverse_kl_bwd (one-shot workgroups that take 4 KB of a row each, the default;
+    the row-per-workgroup loop), with tokens without gradient and a device-side scale: bit-identical gradients."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("reverse KL backward: chunk form vs row loop", v, dtype, n)
+    gen = torch.Generator().manual_seed(v + n)
+    s = (torch.randn(n, v, generator=gen) * 2).to(dtype).to(dev)
+    t = (s.float().cpu() + torch.randn(n, v, generator=gen)).to(dtype).to(dev)
+    kl, ls, lt, s, t = ops.reverse_kl_fwd(s, t)
+    g = torch.rand(n, generator=gen)
+    g[::4] = 0.0
+    g[n // 2:n // 2 + 7] = 0.0
+    scale = torch.tensor([0.61], device=dev)
+    outs = {}
+    for kind in ("two_walk", "auto"):
+        ops.set_kernel_choice(kind)
+        d = ops.reverse_kl_bwd(s, t, kl, ls, lt, g.to(dev), 0.75, scale)
+        torch.cuda.synchronize()
+        outs[kind] = d.view(torch.int16 if dtype != torch.float32 else torch.int32)
+    assert torch.equal(outs["auto"], outs["two_walk"])
+    assert outs["auto"].any() and not outs["auto"][(g == 0).to(dev)].any()
+
+
 def test_opd_kl_two_dimensional_reverse_kl_is_the_elementwise_log_ratio():
     """compute_opd_kl on [R, K] inputs with ``reverse_kl`` returns s - t element by element (opd_utils.py:1126-1138),
     after the lower clamp, with -inf - -inf = NaN at the padding of a union mask like the reference."""

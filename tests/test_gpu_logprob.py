@@ -247,8 +247,9 @@ def test_full_size_properties_headline_shape():
                                        (64000, torch.bfloat16, 900), (65536, torch.float16, 600),
                                        (50304, torch.float32, 700), (65536, torch.float32, 500)])
 def test_backward_burst_form_equals_row_per_workgroup_kernel_bitwise(v, dtype, n):
-    """The two kernels behind relax_amd_logprob_entropy_bwd, switched with relax_amd_set_kernel_choice, on every row
-    shape the persistent burst form is built for (and the ends of two of them), with rows that score no token, tokens
+    """The three kernels behind relax_amd_logprob_entropy_bwd, switched with relax_amd_set_kernel_choice (the default:
+    one-shot workgroups that take 4 KB of a row each; the row-per-workgroup loop; the persistent burst form), on every
+    row shape the burst form is built for (and the ends of two of them), with rows that score no token, tokens
     without gradient (zero rows, in runs and scattered), a device-side gradient scale and targets on a row's first and
     last element: bit-identical gradients."""
     from relax_amd import ops
@@ -274,8 +275,8 @@ def test_backward_burst_form_equals_row_per_workgroup_kernel_bitwise(v, dtype, n
     gen[dead] = 0.0
     scale = torch.tensor([0.37], device=dev)
     outs = {}
-    for kind in ("cached", "resident"):
-        ops.set_kernel_choice("two_walk" if kind == "cached" else "resident")
+    for kind in ("cached", "resident", "auto"):
+        ops.set_kernel_choice({"cached": "two_walk"}.get(kind, kind))
         for with_ent in (True, False):
             d = ops.logprob_entropy_bwd(x, tok, lse, spx, glp.to(dev), gen.to(dev) if with_ent else None,
                                         token_of_row=token_of_row, grad_scale_dev=scale, inv_temperature=0.8)
@@ -283,6 +284,7 @@ def test_backward_burst_form_equals_row_per_workgroup_kernel_bitwise(v, dtype, n
             outs[kind, with_ent] = d.view(torch.int16 if dtype != torch.float32 else torch.int32)
     for with_ent in (True, False):
         assert torch.equal(outs["resident", with_ent], outs["cached", with_ent]), with_ent
+        assert torch.equal(outs["auto", with_ent], outs["cached", with_ent]), with_ent
         assert outs["resident", with_ent].any()
     zero_rows = torch.ones(n, dtype=torch.bool)
     zero_rows[row_ids.cpu().long()[~dead]] = False
