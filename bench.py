@@ -214,13 +214,18 @@ def hbm_roofline(kernel: str, launch_ms: float, necessary_bytes: float, rows: in
 
 def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
     """Which kernel relax_amd_actor_step_fused runs for bf16 / fp32 rows of ``vocab`` entries (the library's own rule:
-    the register-resident kernel in workgroups as wide as the forward-only scan's, where the row shape is built)."""
+    one-shot workgroups sharing each row where that kernel is built; with ``--kernel-choice resident`` the persistent
+    register-resident kernel in workgroups as wide as the forward-only scan's)."""
     per_vec, width, shapes = {"bf16_t": (8, 1024, ((20, False), (19, True), (18, True), (15, True), (16, False), (12, True),
                                                    (8, False), (7, True))),
                               "float": (4, 1024, ((7, True), (8, False), (12, True), (15, True), (16, False)))}[dtype]
     nvec = vocab // per_vec
     threads = 1024 if nvec >= 7168 else 512 if nvec >= 2048 else 256
     shape = (nvec // width, nvec % width != 0)
+    split_shapes = {"bf16_t": ((20, False), (19, True), (18, True), (15, True), (16, False), (12, True)),
+                    "float": ((7, True), (8, False))}[dtype]
+    if vocab % per_vec == 0 and threads == width and shape in split_shapes and KERNEL_CHOICE == "auto":
+        return f"actor_step_split_kernel<{dtype}, {shape[0]}, {str(shape[1]).lower()}>"
     if vocab % per_vec == 0 and threads == width and shape in shapes \
             and KERNEL_CHOICE != "two_walk":
         return f"actor_step_resident_kernel<{dtype}, {shape[0]}, {str(shape[1]).lower()}>"

@@ -226,6 +226,11 @@ static int dispatch_fused(const void* logits, int64_t n_rows, int64_t vocab, int
   // relax_amd_set_kernel_choice: TWO_WALK keeps every row on the two-walk kernel (second walk out of cache); RESIDENT
   // fails for rows the register-resident kernel is not built for
   const int choice = kernel_choice();
+  if (vec && choice == RELAX_AMD_KERNEL_AUTO) {  // one-shot workgroups sharing each row, where built
+    const int rc = launch_actor_step_split<T>(x, stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t, a,
+                                              grad_scale, lp, ent, lse, spx, d, d_stride, s);
+    if (rc != RELAX_AMD_EUNSUPPORTED) return rc;
+  }
   if (vec && choice != RELAX_AMD_KERNEL_TWO_WALK) {
     const int rc = launch_actor_step_resident<T>(x, stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t, a,
                                                  grad_scale, lp, ent, lse, spx, d, d_stride, device_compute_units(), s);

@@ -1,0 +1,411 @@
+// Fused actor step with every row shared between eight one-shot workgroups: the same computation and the same bits
+// as actor_step_resident_kernel (log-prob + entropy forward, per-token policy-loss coefficients, dlogits backward, each
+// logit read once and each gradient written once), in the launch shape this memory system streams fastest: many small
+// workgroups that touch their memory once and retire, dispatched in address order (a mixed read / write stream of
+// this shape moves 6.1 - 6.6 TB/s on the box where 256 persistent row-sized streams move 5.6; this kernel on the
+// 65536 x 151936 bf16 step: 5.81 - 5.85 ms where the persistent kernel takes 6.44 - 6.52, 6.0 ms with 256-thread and
+// 6.3 ms with 64-thread workgroups).
+//
+// A row is scanned by 1024 "virtual threads" exactly as scan_row() lays it out for a 1024-thread workgroup (virtual
+// thread t takes the 16-byte vectors t, t + 1024, ...; four at a time while it has four to go, then single ones).  A
+// workgroup here is 128 of those virtual threads (two waves: virtual waves 2q and 2q + 1 of the row), holds its
+// share of the row in registers (19 vectors per thread at V = 151936 bf16), reduces each wave to its (max, sum exp,
+// sum exp * x) triple by the same butterfly, publishes the two triples, fetches the row's sixteen, merges them in
+// wave order as scan_block_merge() does, and turns its registers into the gradient.  Log-probs, entropy and gradients
+// are therefore bit-identical to the forward-only kernel's and the other fused kernels'.
+//
+// Exchange: a ring of slots in device memory, one per (row mod kRing), of 16 x 3 eight-byte words, each a float and a
+// 32-bit tag, written and read with relaxed device-scope atomics.  The tag names the launch and the lap of the ring: it
+// is read from a device word that a one-workgroup kernel in front of every launch advances (so a captured launch gets
+// fresh tags on every replay), and a reader tells a stale word from the one it waits for without any fence.  The eight
+// workgroups of a row have consecutive indices; a workgroup only waits for those, which are resident or next in
+// dispatch order whatever else the chip runs, so every wait ends.  It is bounded all the same: a workgroup that gives
+// up writes NaN log-probs instead of hanging, and counts itself in a device word.  The ring is one array per process
+// and GPU: launches of this kernel that overlap on one GPU (two streams of one process) can overwrite each other's
+// slots or tags, which ends as such a give-up, never as a wrong number taken for right.
+//
+// Replaces, like the other fused kernels, _VocabParallelLogProbEntropy.forward + .backward
+// (relax/utils/training/ppo_utils.py:481-629) and the per-token part of policy_loss_function
+// (relax/backends/megatron/loss.py:961-1100) for one micro-batch.
+//
+// As in actor_step_resident.hip the row sits at the edge of the register file:
+// hipcc-flags: -mllvm -amdgpu-use-amdgpu-trackers=1
+#include <mutex>
+
+#include "actor_step_resident.h"
+#include "device_utils.h"
+#include "loss_math.h"
+#include "opd_topk_math.h"
+#include "row_scan.h"
+
+namespace relax_amd {
+
+constexpr unsigned kRing = 4096;          // rows whose slots exist at a time
+constexpr int kRowWaves = 16;             // waves of the 1024 virtual threads of a row
+constexpr int kSlotWords = kRowWaves * 3;
+constexpr int kSplitThreads = 128;        // virtual threads per workgroup
+constexpr int kSplit = 1024 / kSplitThreads;
+constexpr unsigned kWaitPolls = 1u << 20;
+constexpr size_t kRingWords = size_t(kRing) * kSlotWords;
+
+// the exchange ring and, behind it, two 32-bit words: the tag counter and the count of waits that gave up
+static __device__ __align__(256) unsigned long long split_ring[kRingWords + 32];
+
+// scan_absorb() over the values of kScanUnroll raw vectors, without holding them all unpacked (as in
+// actor_step_resident.hip: same arithmetic, same order)
+template <typename T>
+__device__ __forceinline__ void split_absorb_raw_group(const u32x4* raw, float c, SoftmaxAcc& st) {
+  constexpr int VN = Row<T>::kPerVec;
+  float vmax = 0.f;
+#pragma unroll
+  for (int u = 0; u < kScanUnroll; ++u) {
+    float v[VN];
+    Row<T>::unpack(raw[u], v);
+#pragma unroll
+    for (int k = 0; k < VN; ++k) vmax = (u == 0 && k == 0) ? v[0] : fmaxf(vmax, v[k]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  const float mc = __fmul_rn(vmax, c);
+  if (mc > st.m) {
+    const float sc = fast_exp2(__fsub_rn(st.m, mc));
+    st.s = __fmul_rn(st.s, sc);
+    st.t = __fmul_rn(st.t, sc);
+    st.m = mc;
+  }
+#pragma unroll
+  for (int u = 0; u < kScanUnroll; ++u) {
+    u32x4 r = raw[u];
+    asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w));
+    float v[VN];
+    Row<T>::unpack(r, v);
+#pragma unroll
+    for (int k = 0; k < VN; ++k) {
+      const float e = fast_exp2(fmaf(v[k], c, -st.m));
+      st.s = __fadd_rn(st.s, e);
+      st.t = fmaf(e, v[k], st.t);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+template <typename T, int NVF, bool PARTIAL, bool TOPK>
+__global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
+    const T* __restrict__ logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
+    const int32_t* __restrict__ token_of_row, const int32_t* __restrict__ sample_ids,
+    const int64_t* __restrict__ targets, float c, float inv_t, relax_amd_policy_loss_args a, float grad_scale,
+    float* __restrict__ log_prob, float* __restrict__ entropy, float* __restrict__ lse_out,
+    float* __restrict__ spx_out, T* __restrict__ dlogits, int64_t d_stride, unsigned long long* __restrict__ ring,
+    unsigned laps) {
+  constexpr int kU = kScanUnroll, ROW_THREADS = 1024;
+  constexpr int VN = Row<T>::kPerVec;
+  constexpr int NV = NVF + (PARTIAL ? 1 : 0);
+  constexpr int kGroups = (NV + kU - 1) / kU;
+  __shared__ float bc[5];
+  __shared__ int64_t bc_target;
+  __shared__ float topk_stage[TOPK ? kTopkStageFloats : 1];
+  __shared__ u32x4 parked[NV][kWave];
+  const int tid = threadIdx.x;
+  const bool wave0 = __builtin_amdgcn_readfirstlane(tid) < kWave;
+  const unsigned part = blockIdx.x % kSplit;
+  const int64_t row = blockIdx.x / kSplit;
+  const int vt = int(part) * kSplitThreads + tid;  // virtual thread of the row
+  const int rem = int(vocab / VN) - NVF * ROW_THREADS;
+  auto has = [&](int j) -> bool { return j < NVF || (PARTIAL && j == NVF && vt < rem); };
+  u32x4* dv = reinterpret_cast<u32x4*>(dlogits + row * d_stride);
+
+  // token of the row, or -1 when the row scores nothing or both of its masks are zero (uniform over the workgroup)
+  int64_t tok = token_of_row ? int64_t(token_of_row[row]) : row;
+  const int64_t t0 = tok;
+  if (tok >= 0) {
+    const float m = a.loss_mask[tok];
+    const float mp = a.pg_loss_mask ? a.pg_loss_mask[tok] : m;
+    if (m == 0.f && mp == 0.f && !a.read_masked_rows) tok = -1;
+  }
+  if (tok < 0) {  // a zero row: no read, no exchange
+    if (t0 >= 0 && part == 0 && tid == 0) {
+      log_prob[t0] = 0.f;
+      entropy[t0] = 0.f;
+      lse_out[t0] = 0.f;
+      spx_out[t0] = 0.f;
+      a.coef_log_prob[t0] = 0.f;
+      if (a.coef_entropy) a.coef_entropy[t0] = 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+      if (has(j)) store_stream(dv + vt + j * ROW_THREADS, u32x4{0u, 0u, 0u, 0u});
+    return;
+  }
+
+  const u32x4* xv = reinterpret_cast<const u32x4*>(logits + row * row_stride);
+  u32x4 reg[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j)
+    if (has(j)) reg[j] = load_stream(xv + vt + j * ROW_THREADS);
+  // this launch's tags: the counter was advanced by `laps` in front of the launch
+  const unsigned tag = reinterpret_cast<const unsigned*>(ring + kRingWords)[0] - laps + 1u + unsigned(row / kRing);
+
+  // the scan, group by group as the vectors arrive, in scan_row()'s order
+  SoftmaxAcc st{kNegHuge, 0.f, 0.f};
+  bool grouped = true;
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g) {
+    if (grouped && kU * g + kU - 1 < NV && has(kU * g + kU - 1)) {
+      split_absorb_raw_group<T>(&reg[kU * g < NV - kU ? kU * g : NV - kU], c, st);
+    } else {
+      grouped = false;
+#pragma unroll
+      for (int u = 0; u < kU; ++u)
+        if (kU * g + u < NV && has(kU * g + u)) {
+          float v[VN];
+          Row<T>::unpack(reg[kU * g + u < NV ? kU * g + u : NV - 1], v);
+          scan_absorb(v, c, st);
+        }
+    }
+    asm volatile("" : "+v"(st.m), "+v"(st.s), "+v"(st.t));
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // each wave to its triple (scan_block_merge()'s first half), published by its lanes 0..2
+  wave_butterfly([&](auto o) {
+    constexpr int O = decltype(o)::value;
+    scan_merge(st, lane_xor<O>(st.m), lane_xor<O>(st.s), lane_xor<O>(st.t));
+  });
+  unsigned long long* slot = ring + size_t(row % kRing) * kSlotWords;
+  {
+    // lane 0's triple, as scan_block_merge() takes it (the butterfly's merge is not symmetric in its last bits)
+    const float m0 = lane_value(st.m), s0 = lane_value(st.s), t0v = lane_value(st.t);
+    const int lane = tid & (kWave - 1), vwave = vt / kWave;
+    if (lane < 3) {
+      const float val = lane == 0 ? m0 : (lane == 1 ? s0 : t0v);
+      __hip_atomic_store(slot + vwave * 3 + lane, (static_cast<unsigned long long>(tag) << 32) | __float_as_uint(val),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+
+  if (wave0) {
+    // thread 0 runs a serial stretch from here to the barrier while the other waves of the workgroup wait
+    __builtin_amdgcn_s_setprio(3);
+    // wave 0's share of the row waits in LDS meanwhile: thread 0's loss arithmetic needs some thirty registers of its
+    // own, which every wave of the kernel would otherwise have to set aside next to the row
+#pragma unroll
+    for (int j = 0; j < NV; ++j) parked[j][tid] = reg[j];
+    // thread 0's view of the token, fetched while the triples travel
+    TokenInputs tin{};
+    float x_target = 0.f, den = 1.f, pg_den = 1.f;
+    int64_t tg = -1;
+    if (tid == 0) {
+      tin = load_token_inputs(a, tok);
+      tg = targets[tok];
+      if (tg >= 0 && tg < vocab) x_target = Row<T>::load1(logits + row * row_stride + tg);
+      const int32_t sid = sample_ids ? sample_ids[tok] : 0;
+      den = a.sample_denom ? a.sample_denom[sid] : 1.0f;
+      pg_den = a.pg_sample_denom ? a.pg_sample_denom[sid] : den;
+    }
+    TopkGather gathered{};
+    TopkRowShape topk_shape{};
+    if constexpr (TOPK) {
+      int lane = tid;
+      asm volatile("" : "+v"(lane));
+      gathered = topk_gather<T>(a, logits + row * row_stride, vocab, tok, lane);
+      topk_shape = topk_row_shape(a, tok);
+    }
+    // lanes 0 .. 47 fetch one word of the row's sixteen triples each
+    float word = 0.f;
+    bool gave_up = false;
+    if (tid < kSlotWords) {
+      unsigned polls = 0;
+      while (true) {
+        const unsigned long long w = __hip_atomic_load(slot + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (unsigned(w >> 32) == tag) {
+          word = __uint_as_float(unsigned(w));
+          break;
+        }
+        if (++polls > kWaitPolls) {
+          gave_up = true;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+    }
+    const bool any_gave_up = __any(gave_up);
+    // the sixteen waves in index order, as thread 0 of a 1024-thread workgroup merges them
+    auto of_lane = [&](int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(word), l)); };
+    SoftmaxAcc whole{of_lane(0), of_lane(1), of_lane(2)};
+#pragma unroll
+    for (int i = 1; i < kRowWaves; ++i) scan_merge(whole, of_lane(3 * i), of_lane(3 * i + 1), of_lane(3 * i + 2));
+    float lse = 0.f, spx = 0.f, ent = 0.f, lp = 0.f;
+    if (tid == 0) {
+      scan_finish(whole, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
+      if (any_gave_up) {
+        lp = lse = __builtin_nanf("");
+        atomicAdd(reinterpret_cast<unsigned*>(ring + kRingWords) + 1, 1u);
+      }
+      if (part == 0) {
+        log_prob[tok] = lp;
+        entropy[tok] = ent;
+        lse_out[tok] = lse;
+        spx_out[tok] = spx;
+      }
+    }
+    float g_topk = 0.f;
+    if constexpr (TOPK) {
+      int lane = tid;
+      asm volatile("" : "+v"(lane));
+      g_topk = topk_distill_row(a, gathered, topk_shape, tok, lane_value(lse), inv_t, lane_value(lp),
+                                lane_value(tin.has_old ? tin.old_lp : lp), lane_value(tin.extra_lp), lane, topk_stage);
+    }
+    if (tid == 0) {
+      relax_amd_policy_loss_args al = a;
+      asm volatile("" : "+s"(al.eps_clip), "+s"(al.eps_clip_high), "+s"(al.eps_clip_c), "+s"(al.entropy_coef),
+                   "+s"(al.kl_coef), "+s"(al.tis_lo), "+s"(al.tis_hi), "+s"(al.tau_pos), "+s"(al.tau_neg));
+      const TokenResult tr = token_terms(al, tin, lp, ent, false, 0.f, den, pg_den);
+      if (part == 0) {
+        a.coef_log_prob[tok] = tr.coef_lp;
+        if (a.coef_entropy) a.coef_entropy[tok] = tr.coef_ent;
+      }
+      const float glp = tr.coef_lp * grad_scale, gh = tr.coef_ent * grad_scale;
+      const float gsm = TOPK ? glp + g_topk * grad_scale : glp;
+      const float b = gh * inv_t;
+      bc[0] = -lse * kLog2e;           // k0: p = exp2(x*c + k0)
+      bc[1] = -gsm * inv_t + b * spx;  // a0
+      bc[2] = -b * inv_t;              // a1: d = p * (a0 + a1*x)
+      bc[3] = glp * inv_t;             // added at the target
+      bc[4] = (gsm == 0.f && glp == 0.f && gh == 0.f) ? 1.f : 0.f;
+      bc_target = tg;
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) reg[j] = parked[j][tid];
+    __builtin_amdgcn_s_setprio(0);
+  }
+  __syncthreads();
+  const float k0 = bc[0], a0 = bc[1], a1 = bc[2], hot = bc[3];
+  const int64_t tgt = bc_target;
+  const bool emit_zero = bc[4] != 0.f;
+  const int tvec = (tgt >= 0 && tgt < vocab) ? int(tgt / VN) : -1;
+  const int tsub = int(tgt % VN);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    int lane_id = vt;
+    asm volatile("" : "+v"(lane_id));
+    const int idx = lane_id + j * ROW_THREADS;
+    float v[VN];
+    Row<T>::unpack(reg[j], v);
+#pragma unroll
+    for (int k = 0; k < VN; ++k) {
+      v[k] = fast_exp2(fmaf(v[k], c, k0)) * fmaf(v[k], a1, a0);
+      if (k == VN / 2 - 1) __builtin_amdgcn_sched_barrier(0);
+    }
+    if (idx == tvec) {
+#pragma unroll
+      for (int k = 0; k < VN; ++k)
+        if (k == tsub) v[k] += hot;
+    }
+    if (has(j)) store_stream(dv + idx, emit_zero ? u32x4{0u, 0u, 0u, 0u} : Row<T>::pack(v));
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// Advances the tag counter by the laps of the launch that follows; clears the ring when the 32-bit counter would wrap
+// (a tag of a past lap could otherwise come round again).
+__global__ __launch_bounds__(256) void split_ring_advance_kernel(unsigned long long* ring, unsigned laps) {
+  unsigned* counter = reinterpret_cast<unsigned*>(ring + kRingWords);
+  const unsigned now = counter[0];
+  const bool wrap = now > 0xffffffffu - laps - 1u;
+  if (wrap)
+    for (size_t i = threadIdx.x; i < kRingWords; i += 256) ring[i] = 0ull;
+  __syncthreads();
+  if (threadIdx.x == 0) counter[0] = (wrap ? 0u : now) + laps;
+}
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex ring_mutex;
+unsigned long long* ring_ptr[kMaxDevices] = {};
+}  // namespace
+
+// the current device's ring (looked up once per device, with that device current)
+static int split_ring_of_device(unsigned long long** ring) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("actor_step_split: no usable current device (%s)",
+              e == hipSuccess ? "index out of range" : hipGetErrorString(e));
+    return RELAX_AMD_EINVAL;
+  }
+  std::lock_guard<std::mutex> lock(ring_mutex);
+  if (!ring_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(split_ring));
+    if (e != hipSuccess || !p) {
+      set_error("actor_step_split: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return RELAX_AMD_ELAUNCH;
+    }
+    ring_ptr[dev] = static_cast<unsigned long long*>(p);
+  }
+  *ring = ring_ptr[dev];
+  return RELAX_AMD_OK;
+}
+
+#define RELAX_AMD_SPLIT(NVF, PARTIAL)                                                                                 \
+  if (full == NVF && partial == PARTIAL) {                                                                            \
+    if (a.topk_ids)                                                                                                   \
+      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, true>), grid, block, 0, stream, logits,           \
+                         row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
+                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps);                    \
+    else                                                                                                              \
+      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, false>), grid, block, 0, stream, logits,          \
+                         row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
+                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps);                    \
+    return check_launch("actor_step_split");                                                                          \
+  }
+
+template <typename T>
+int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
+                            const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,
+                            float inv_t, const relax_amd_policy_loss_args& a, float grad_scale, float* log_prob,
+                            float* entropy, float* lse, float* spx, T* dlogits, int64_t d_stride,
+                            hipStream_t stream) {
+  constexpr int VN = Row<T>::kPerVec;
+  if (vocab % VN != 0 || scan_threads(vocab, VN) != 1024 || n_rows * kSplit > 2147483647LL)
+    return RELAX_AMD_EUNSUPPORTED;
+  const int64_t nvec = vocab / VN;
+  const int full = int(nvec / 1024);
+  const bool partial = nvec % 1024 != 0;
+  if constexpr (sizeof(T) == 2) {
+    if (!((full == 20 && !partial) || (full == 19 && partial) || (full == 18 && partial) || (full == 15 && partial) ||
+          (full == 16 && !partial) || (full == 12 && partial)))
+      return RELAX_AMD_EUNSUPPORTED;
+  } else {
+    if (!((full == 7 && partial) || (full == 8 && !partial))) return RELAX_AMD_EUNSUPPORTED;
+  }
+  unsigned long long* ring = nullptr;
+  if (int rc = split_ring_of_device(&ring)) return rc;
+  const unsigned laps = unsigned((n_rows + kRing - 1) / kRing);
+  hipLaunchKernelGGL(split_ring_advance_kernel, dim3(1), dim3(256), 0, stream, ring, laps);
+  const dim3 grid(static_cast<unsigned>(n_rows * kSplit)), block(kSplitThreads);
+  if constexpr (sizeof(T) == 2) {
+    RELAX_AMD_SPLIT(20, false)
+    RELAX_AMD_SPLIT(19, true)
+    RELAX_AMD_SPLIT(18, true)
+    RELAX_AMD_SPLIT(15, true)
+    RELAX_AMD_SPLIT(16, false)
+    RELAX_AMD_SPLIT(12, true)
+  } else {
+    RELAX_AMD_SPLIT(7, true)
+    RELAX_AMD_SPLIT(8, false)
+  }
+  return RELAX_AMD_EUNSUPPORTED;
+}
+#undef RELAX_AMD_SPLIT
+
+template int launch_actor_step_split<float>(const float*, int64_t, int64_t, int64_t, const int32_t*, const int32_t*,
+                                            const int64_t*, float, const relax_amd_policy_loss_args&, float, float*,
+                                            float*, float*, float*, float*, int64_t, hipStream_t);
+template int launch_actor_step_split<bf16_t>(const bf16_t*, int64_t, int64_t, int64_t, const int32_t*, const int32_t*,
+                                             const int64_t*, float, const relax_amd_policy_loss_args&, float, float*,
+                                             float*, float*, float*, bf16_t*, int64_t, hipStream_t);
+template int launch_actor_step_split<f16_t>(const f16_t*, int64_t, int64_t, int64_t, const int32_t*, const int32_t*,
+                                            const int64_t*, float, const relax_amd_policy_loss_args&, float, float*,
+                                            float*, float*, float*, f16_t*, int64_t, hipStream_t);
+
+}  // namespace relax_amd
+

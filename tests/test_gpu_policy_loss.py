@@ -1246,8 +1246,10 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
 def test_topk_opd_term_in_the_register_resident_step(v, dtype, k, variant):
     """The top-K distillation term inside the single launch on the row shapes of the register-resident kernel (several
     rows per persistent workgroup, K below and above one wave's width, the union mask, clips): loss, metrics and
-    dlogits against the two-launch path and against the oracle."""
+    dlogits against the two-launch path and against the oracle; the default kernel (one-shot workgroups sharing each
+    row) and the persistent one bit for bit."""
     import relax_amd
+    from relax_amd import ops
 
     dev = require_gpu()
     announce("top-K OPD in the resident step", v, dtype, k, variant)
@@ -1280,6 +1282,14 @@ def test_topk_opd_term_in_the_register_resident_step(v, dtype, k, variant):
         loss, met = relax_amd.policy_loss_function(P.make_args(relax_amd_single_pass=mode, **kw), db, lg, None)
         loss.backward()
         outs[mode] = (loss.detach(), met, lg.grad)
+    ops.set_kernel_choice("resident")
+    lg = logits.to(dev).requires_grad_()
+    loss, met = relax_amd.policy_loss_function(P.make_args(relax_amd_single_pass="auto", **kw), db, lg, None)
+    loss.backward()
+    ops.set_kernel_choice("auto")
+    assert torch.equal(loss.detach(), outs["auto"][0]) and torch.equal(lg.grad, outs["auto"][2])
+    for key, w in outs["auto"][1].items():
+        assert torch.equal(met[key], w), key
     ulp = {torch.bfloat16: 2.0 ** -7, torch.float32: 1e-5}[dtype]
     assert abs(outs["auto"][0].item() - outs["off"][0].item()) < 1e-5 * max(1.0, abs(outs["off"][0].item()))
     assert set(outs["auto"][1]) == set(outs["off"][1])
@@ -1716,7 +1726,7 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
 
 
 @pytest.mark.parametrize("v,dtype,n_rows,values", [
-    (100352, torch.bfloat16, 700, "plain"), (32000, torch.float32, 1500, "plain"),
+    (100352, torch.bfloat16, 700, "plain"), (32000, torch.float32, 1500, "plain"), (151936, torch.bfloat16, 300, "plain"),
     # long fp32 rows, kept in the registers as their upper halves: bf16 values widened to fp32 (what a bf16 output
     # layer followed by .float() delivers: one read of the row), fp32 values with low bits (the row is read again), and
     # rows of both kinds next to each other, one of them with a single low bit in its last element
@@ -1724,13 +1734,14 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
 @pytest.mark.parametrize("pattern", ["all_dead", "one_live_last", "few_live", "random", "all_live_no_map",
                                      "zero_advantage"])
 def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dtype, n_rows, values):
-    """The two kernels behind relax_amd_actor_step_fused, switched with relax_amd_set_kernel_choice, on row / token
-    layouts that stress the persistent loop of the register-resident one: no live row at all, a single live row at
+    """The kernels behind relax_amd_actor_step_fused, switched with relax_amd_set_kernel_choice (two-walk, persistent
+    register-resident, and the default: one-shot workgroups that share each row and exchange their partial sums
+    through device memory, where built), on row / token layouts that stress the persistent loop of the
+    register-resident one and the zero-row path of the others: no live row at all, a single live row at
     the very end, fewer live rows than workgroups, random prompt rows and masked tokens over several rows per
     workgroup, no row map (every row scores its own token), and tokens whose gradient coefficients vanish (zero
-    rows without a look at the logits); on 16-bit rows of 12 full vectors per thread plus a partial one (one
-    1024-thread workgroup per CU) and on fp32 rows of 32000 entries.  Every output
-    must be bit-identical."""
+    rows without a look at the logits); on 16-bit rows of 12 and of 18 full vectors per thread plus a partial one and on
+    fp32 rows of 32000 entries.  Every output must be bit-identical."""
     from relax_amd import ops
 
     dev = require_gpu()
@@ -1776,18 +1787,73 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
                   entropy_coef=0.01)
     targets = torch.randint(0, v, (n_tok,), generator=g).to(dev)
     results = {}
-    for kind in ("cached", "resident"):
-        ops.set_kernel_choice("two_walk" if kind == "cached" else "resident")
+    for kind in ("cached", "resident", "auto", "auto_again"):
+        ops.set_kernel_choice({"cached": "two_walk", "resident": "resident"}.get(kind, "auto"))
         out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, token_of_row, sample_ids, n_tok, 1.0, 1.0, **kw)
         torch.cuda.synchronize()
         results[kind] = dict(lp=lp, ent=ent, lse=lse, spx=spx, coef=out["coef_log_prob"],
                              d=d.view(torch.int16 if dtype != torch.float32 else torch.int32),
                              coef_ent=out["coef_entropy"], metrics=out["metrics"])
-    for key, want in results["cached"].items():
-        got = results["resident"][key]
-        assert torch.equal(got, want), (pattern, key, (got.float() - want.float()).abs().max())
+    for kind in ("resident", "auto", "auto_again"):
+        for key, want in results["cached"].items():
+            got = results[kind][key]
+            assert torch.equal(got, want), (kind, pattern, key, (got.float() - want.float()).abs().max())
     if pattern == "all_dead":
-        assert not results["resident"]["d"].any()
+        assert not results["resident"]["d"].any() and not results["auto"]["d"].any()
+
+
+def test_default_fused_step_replayed_from_a_captured_graph():
+    """The default fused step tags the partial sums its workgroups exchange with a counter that a small kernel in front
+    of the launch advances on the device, so a captured launch gets fresh tags on every replay: three replays on fresh
+    logits, with eager launches between them, each bit-identical to the two-walk kernel on the same inputs."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("fused step under graph capture")
+    v, n_rows = 100352, 300
+    g = torch.Generator().manual_seed(5)
+    scores = torch.rand(n_rows, generator=g) > 0.25
+    idx = torch.cumsum(scores.int(), 0) - 1
+    token_of_row = torch.where(scores, idx, torch.full_like(idx, -1)).int().to(dev)
+    n_tok = int(scores.sum())
+    mask = (torch.rand(n_tok, generator=g) > 0.2).float()
+    base = -11.0 + 0.3 * torch.randn(n_tok, generator=g)
+    kw = dict(advantages=torch.randn(n_tok, generator=g).to(dev), loss_mask=mask.to(dev),
+              cu_resp=torch.tensor([0, n_tok], dtype=torch.int64, device=dev), old_log_prob=base.to(dev),
+              ref_log_prob=(base + 0.1 * torch.randn(n_tok, generator=g)).to(dev), kl_kind="k3", kl_coef=1e-3,
+              entropy_coef=0.01, sample_denom=torch.tensor([max(1.0, mask.sum().item())], device=dev),
+              loss_kind="ppo", eps_clip=0.2, eps_clip_high=0.28)
+    sample_ids = torch.zeros(n_tok, dtype=torch.int32, device=dev)
+    targets = torch.randint(0, v, (n_tok,), generator=g).to(dev)
+    logits = (torch.randn(n_rows, v, generator=g) * 2).bfloat16().to(dev)
+
+    def run():
+        out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, token_of_row, sample_ids, n_tok, 1.0, 1.0, **kw)
+        return dict(lp=lp, ent=ent, lse=lse, coef=out["coef_log_prob"], d=d.view(torch.int16))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()  # warm-up outside the capture (the library looks its exchange buffer up on first use)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run()
+    for rep in range(3):
+        logits.copy_((torch.randn(n_rows, v, generator=g) * 2).bfloat16())
+        graph.replay()
+        torch.cuda.synchronize()
+        got = {k: t.clone() for k, t in captured.items()}
+        eager = run()  # an eager launch between the replays
+        ops.set_kernel_choice("two_walk")
+        want = run()
+        ops.set_kernel_choice("auto")
+        torch.cuda.synchronize()
+        for key in want:
+            assert torch.equal(got[key], want[key]), (rep, key)
+            assert torch.equal(eager[key], want[key]), (rep, key, "eager")
+        assert not torch.isnan(got["lp"]).any()
 
 
 @pytest.mark.parametrize("v", [128256, 129280, 131072, 152064, 163840, 4 * (31 * 1024 + 1), 4 * (38 * 1024 - 1),
@@ -1881,15 +1947,16 @@ def test_register_resident_kernel_at_the_edges_of_its_row_shapes(v, dtype):
               loss_kind="ppo", eps_clip=0.2, eps_clip_high=0.28)
     sample_ids = torch.zeros(n_tok, dtype=torch.int32, device=dev)
     results = {}
-    for kind in ("cached", "resident"):
-        ops.set_kernel_choice("two_walk" if kind == "cached" else "resident")
+    for kind in ("cached", "resident", "auto"):
+        ops.set_kernel_choice({"cached": "two_walk", "resident": "resident"}.get(kind, "auto"))
         out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets.to(dev), token_of_row, sample_ids, n_tok, 1.0,
                                                          1.0, **kw)
         torch.cuda.synchronize()
         results[kind] = dict(lp=lp, ent=ent, lse=lse, spx=spx, coef=out["coef_log_prob"],
                              d=d.view(torch.int16 if dtype != torch.float32 else torch.int32))
-    for key, want in results["cached"].items():
-        assert torch.equal(results["resident"][key], want), key
+    for kind in ("resident", "auto"):
+        for key, want in results["cached"].items():
+            assert torch.equal(results[kind][key], want), (kind, key)
     assert results["resident"]["d"].any()
 
 
