@@ -72,16 +72,26 @@ int relax_amd_version(void);
 /* Message of the last failing call on this thread ("" if none). Host pointer, valid until the next call. */
 const char* relax_amd_last_error(void);
 
-/* which of two bit-identical kernels the fused entry points launch (see relax_amd_set_kernel_choice) */
+/* which of their bit-identical kernels the fused entry points launch (see relax_amd_set_kernel_choice) */
 enum { RELAX_AMD_KERNEL_AUTO = 0, RELAX_AMD_KERNEL_TWO_WALK = 1, RELAX_AMD_KERNEL_RESIDENT = 2 };
 /*
  * relax_amd_actor_step_fused, relax_amd_logprob_entropy_bwd and relax_amd_reverse_kl_step_fused each hold a
- * register-resident kernel for the row lengths it is built for and a two-walk (row-per-workgroup) kernel for every
- * row length; both give the same bits.  AUTO (the default) takes the resident one where it exists.  TWO_WALK keeps
- * every row on the two-walk kernel; RESIDENT makes those entry points fail with RELAX_AMD_EUNSUPPORTED where no
- * resident kernel is built, so that a comparison of the two cannot pass on one kernel compared with itself.
+ * persistent register-resident kernel for the row lengths it is built for and a two-walk (row-per-workgroup) kernel
+ * for every row length; the first two also hold a kernel of one-shot workgroups in address order (the actor step:
+ * eight workgroups share a row and exchange their partial softmax sums through a ring in device memory; the
+ * backward: one workgroup per 4 KB of a row).  All give the same bits.  AUTO (the default) takes the one-shot form
+ * where it exists, else the resident one, else the two-walk kernel.  TWO_WALK keeps every row on the two-walk
+ * kernel; RESIDENT takes the persistent kernel and makes those entry points fail with RELAX_AMD_EUNSUPPORTED where
+ * none is built, so that a comparison of kernels cannot pass on one kernel compared with itself.
  * Process-wide, read atomically at each launch; returns the previous choice, or RELAX_AMD_EINVAL.  No counterpart
  * in the reference: it exists for tests and measurements.
+ *
+ * The actor step's one-shot kernel keeps its exchange ring (1.5 MB) in a static array of the library, one copy per
+ * GPU and process.  Launches of relax_amd_actor_step_fused that overlap on one GPU (two streams of one process) must
+ * not both take that kernel: they could overwrite each other's slots, which the kernel notices (bounded waits) and
+ * reports as NaN log-probs rather than wrong numbers.  Launches in stream order, captured graphs and their replays
+ * are fine (the tags that tell one launch's partial sums from another's come from a counter in device memory that a
+ * small kernel in front of each launch advances).
  */
 int relax_amd_set_kernel_choice(int choice);
 
@@ -448,10 +458,13 @@ int relax_amd_logprob_entropy_topk_fwd(const void* logits, int dtype, int64_t n_
  *   dlogits     [n_rows, vocab] out, every row written (zero rows where token_of_row < 0 or the coefficients vanish)
  * With loss->topk_ids set the step also evaluates the top-K distillation signal of every row it reads (see the
  * argument block); the caller adds the K one-hot parts of its gradient with relax_amd_sparse_row_add afterwards.
- * Two kernels sit behind this entry point and are chosen by row length and element type: a register-resident one
- * (one read and one write of HBM per row; 16-bit rows of 57352 .. 65536 and 100352 .. 163840 entries, fp32 rows of
- * 28676 .. 32768, 49156 .. 53248 and 61444 .. 65536 entries, in the built shapes) and a two-walk one for everything else; relax_amd_set_kernel_choice(RELAX_AMD_KERNEL_TWO_WALK)
- * forces the latter.  Same results.
+ * Three kernels sit behind this entry point and are chosen by row length and element type, all with the same
+ * results bit for bit: one-shot workgroups that share each row (one read and one write of HBM per row; 16-bit rows of
+ * 100352 .. 163840 entries and fp32 rows of 28676 .. 32768 entries, in the built shapes: the default where built, see
+ * relax_amd_set_kernel_choice for the ring in device memory it exchanges partial sums through), a persistent
+ * register-resident one (the same traffic; those shapes, 16-bit rows of 57352 .. 65536 and fp32 rows of
+ * 49156 .. 53248, 61444 .. 65536 and, as upper halves, 100352 .. 163840 entries) and a two-walk one for everything
+ * else; relax_amd_set_kernel_choice(RELAX_AMD_KERNEL_RESIDENT / RELAX_AMD_KERNEL_TWO_WALK) forces the second / third.
  */
 int relax_amd_actor_step_fused(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                                const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,

@@ -51,8 +51,8 @@ constexpr size_t kRingWords = size_t(kRing) * kSlotWords;
 // the exchange ring and, behind it, two 32-bit words: the tag counter and the count of waits that gave up
 static __device__ __align__(256) unsigned long long split_ring[kRingWords + 32];
 
-// scan_absorb() over the values of kScanUnroll raw vectors, without holding them all unpacked (as in
-// actor_step_resident.hip: same arithmetic, same order)
+// scan_absorb() over the values of kScanUnroll raw vectors (as in actor_step_resident.hip: same arithmetic, same
+// order)
 template <typename T>
 __device__ __forceinline__ void split_absorb_raw_group(const u32x4* raw, float c, SoftmaxAcc& st) {
   constexpr int VN = Row<T>::kPerVec;
@@ -74,10 +74,9 @@ __device__ __forceinline__ void split_absorb_raw_group(const u32x4* raw, float c
   }
 #pragma unroll
   for (int u = 0; u < kScanUnroll; ++u) {
-    u32x4 r = raw[u];
-    asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w));
     float v[VN];
-    Row<T>::unpack(r, v);
+    Row<T>::unpack(raw[u], v);  // the compiler keeps the first walk's values: with wave 0's share parked in LDS
+                                // during thread 0's arithmetic there is room for them next to the row
 #pragma unroll
     for (int k = 0; k < VN; ++k) {
       const float e = fast_exp2(fmaf(v[k], c, -st.m));
@@ -103,7 +102,10 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
   __shared__ float bc[5];
   __shared__ int64_t bc_target;
   __shared__ float topk_stage[TOPK ? kTopkStageFloats : 1];
-  __shared__ u32x4 parked[NV][kWave];
+  // vectors of wave 0's share that wait in LDS during thread 0's serial stretch (see there): all of them, or as many
+  // as leave room for eight workgroups per CU next to the top-K term's staging area
+  constexpr int kPark = NV < (TOPK ? 15 : 19) ? NV : (TOPK ? 15 : 19);
+  __shared__ u32x4 parked[kPark][kWave];
   const int tid = threadIdx.x;
   const bool wave0 = __builtin_amdgcn_readfirstlane(tid) < kWave;
   const unsigned part = blockIdx.x % kSplit;
@@ -187,7 +189,7 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
     // wave 0's share of the row waits in LDS meanwhile: thread 0's loss arithmetic needs some thirty registers of its
     // own, which every wave of the kernel would otherwise have to set aside next to the row
 #pragma unroll
-    for (int j = 0; j < NV; ++j) parked[j][tid] = reg[j];
+    for (int j = 0; j < kPark; ++j) parked[j][tid] = reg[j];
     // thread 0's view of the token, fetched while the triples travel
     TokenInputs tin{};
     float x_target = 0.f, den = 1.f, pg_den = 1.f;
@@ -273,7 +275,7 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
       bc_target = tg;
     }
 #pragma unroll
-    for (int j = 0; j < NV; ++j) reg[j] = parked[j][tid];
+    for (int j = 0; j < kPark; ++j) reg[j] = parked[j][tid];
     __builtin_amdgcn_s_setprio(0);
   }
   __syncthreads();
@@ -282,6 +284,12 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
   const bool emit_zero = bc[4] != 0.f;
   const int tvec = (tgt >= 0 && tgt < vocab) ? int(tgt / VN) : -1;
   const int tsub = int(tgt % VN);
+  if (emit_zero) {  // uniform over the workgroup: both gradient coefficients vanish, a zero row whatever the logits hold
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+      if (has(j)) store_stream(dv + vt + j * ROW_THREADS, u32x4{0u, 0u, 0u, 0u});
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     int lane_id = vt;
@@ -294,12 +302,17 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
       v[k] = fast_exp2(fmaf(v[k], c, k0)) * fmaf(v[k], a1, a0);
       if (k == VN / 2 - 1) __builtin_amdgcn_sched_barrier(0);
     }
-    if (idx == tvec) {
+    u32x4 out = Row<T>::pack(v);
+    // The element at the target gets `hot` added before it is rounded.  One wave in 300 holds it: that wave takes a
+    // jump (the ballot is wave-uniform) and packs the vector again; as a per-lane select on every vector the same
+    // update costs two vector instructions per element, an eighth of the kernel's arithmetic.
+    if (__builtin_amdgcn_ballot_w64(idx == tvec) != 0ull) {
 #pragma unroll
       for (int k = 0; k < VN; ++k)
-        if (k == tsub) v[k] += hot;
+        if (idx == tvec && k == tsub) v[k] += hot;
+      out = Row<T>::pack(v);
     }
-    if (has(j)) store_stream(dv + idx, emit_zero ? u32x4{0u, 0u, 0u, 0u} : Row<T>::pack(v));
+    if (has(j)) store_stream(dv + idx, out);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
