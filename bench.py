@@ -231,8 +231,8 @@ def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
         return f"actor_step_resident_kernel<{dtype}, {shape[0]}, {str(shape[1]).lower()}>"
     if dtype == "float" and vocab % 4 == 0 and threads == 1024 and KERNEL_CHOICE != "two_walk" \
             and shape in ((37, True), (31, True), (32, False), (40, False), (24, True), (25, False)):
-        # long fp32 rows, resident as their upper halves
-        return f"actor_step_resident_wide_kernel<{shape[0]}, {str(shape[1]).lower()}>"
+        # long fp32 rows, held as their upper halves (one-shot workgroups sharing each row, or one persistent workgroup)
+        return f"actor_step_{'split' if KERNEL_CHOICE == 'auto' else 'resident'}_wide_kernel<{shape[0]}, {str(shape[1]).lower()}>"
     return f"actor_step_fused_kernel<{dtype}, true, {threads}>"
 
 

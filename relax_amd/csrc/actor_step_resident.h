@@ -38,4 +38,11 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
                             float* entropy, float* lse, float* spx, T* dlogits, int64_t d_stride,
                             hipStream_t stream);
 
+// launch_actor_step_resident_wide's rows in the one-shot form (actor_step_split.hip), same bits.
+int launch_actor_step_split_wide(const float* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
+                                 const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,
+                                 float inv_t, const relax_amd_policy_loss_args& a, float grad_scale, float* log_prob,
+                                 float* entropy, float* lse, float* spx, float* dlogits, int64_t d_stride,
+                                 hipStream_t stream);
+
 }  // namespace relax_amd

@@ -1888,15 +1888,16 @@ def test_long_fp32_rows_resident_as_upper_halves_equal_two_walk_kernel_and_oracl
               loss_kind="ppo", eps_clip=0.2, eps_clip_high=0.28)
     sample_ids = torch.zeros(n_tok, dtype=torch.int32, device=dev)
     results = {}
-    for kind in ("two_walk", "resident"):
+    for kind in ("two_walk", "resident", "auto"):  # auto: the one-shot form of the same kernel
         ops.set_kernel_choice(kind)
         out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets.to(dev), token_of_row, sample_ids, n_tok, 1.0,
                                                          1.0, **kw)
         torch.cuda.synchronize()
         results[kind] = dict(lp=lp, ent=ent, lse=lse, spx=spx, coef=out["coef_log_prob"], d=d.view(torch.int32))
-    for key, want in results["two_walk"].items():
-        got = results["resident"][key]
-        assert torch.equal(got, want), (key, (got.float() - want.float()).abs().max())
+    for kind in ("resident", "auto"):
+        for key, want in results["two_walk"].items():
+            got = results[kind][key]
+            assert torch.equal(got, want), (kind, key, (got.float() - want.float()).abs().max())
     # oracle on the scored rows: log-probs / entropy of every live token, gradient rows of a few tokens
     rows = torch.nonzero(scores).squeeze(1)
     x = logits[rows.to(dev)].cpu()
