@@ -222,8 +222,7 @@ def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
     nvec = vocab // per_vec
     threads = 1024 if nvec >= 7168 else 512 if nvec >= 2048 else 256
     shape = (nvec // width, nvec % width != 0)
-    split_shapes = {"bf16_t": ((20, False), (19, True), (18, True), (15, True), (16, False), (12, True)),
-                    "float": ((7, True), (8, False))}[dtype]
+    split_shapes = shapes  # the one-shot kernel is built for the shapes of the persistent one
     if vocab % per_vec == 0 and threads == width and shape in split_shapes and KERNEL_CHOICE == "auto":
         return f"actor_step_split_kernel<{dtype}, {shape[0]}, {str(shape[1]).lower()}>"
     if vocab % per_vec == 0 and threads == width and shape in shapes \

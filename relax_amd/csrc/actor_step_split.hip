@@ -650,12 +650,15 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
   const int64_t nvec = vocab / VN;
   const int full = int(nvec / 1024);
   const bool partial = nvec % 1024 != 0;
+  // the row shapes launch_actor_step_resident is built for
   if constexpr (sizeof(T) == 2) {
     if (!((full == 20 && !partial) || (full == 19 && partial) || (full == 18 && partial) || (full == 15 && partial) ||
-          (full == 16 && !partial) || (full == 12 && partial)))
+          (full == 16 && !partial) || (full == 12 && partial) || (full == 8 && !partial) || (full == 7 && partial)))
       return RELAX_AMD_EUNSUPPORTED;
   } else {
-    if (!((full == 7 && partial) || (full == 8 && !partial))) return RELAX_AMD_EUNSUPPORTED;
+    if (!((full == 7 && partial) || (full == 8 && !partial) || (full == 12 && partial) || (full == 15 && partial) ||
+          (full == 16 && !partial)))
+      return RELAX_AMD_EUNSUPPORTED;
   }
   unsigned long long* ring = nullptr;
   if (int rc = split_ring_of_device(&ring)) return rc;
@@ -669,9 +672,14 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
     RELAX_AMD_SPLIT(15, true)
     RELAX_AMD_SPLIT(16, false)
     RELAX_AMD_SPLIT(12, true)
+    RELAX_AMD_SPLIT(8, false)
+    RELAX_AMD_SPLIT(7, true)
   } else {
     RELAX_AMD_SPLIT(7, true)
     RELAX_AMD_SPLIT(8, false)
+    RELAX_AMD_SPLIT(12, true)
+    RELAX_AMD_SPLIT(15, true)
+    RELAX_AMD_SPLIT(16, false)
   }
   return RELAX_AMD_EUNSUPPORTED;
 }
