@@ -223,6 +223,10 @@ def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
     threads = 1024 if nvec >= 7168 else 512 if nvec >= 2048 else 256
     shape = (nvec // width, nvec % width != 0)
     split_shapes = shapes  # the one-shot kernel is built for the shapes of the persistent one
+    if dtype == "bf16_t" and vocab % per_vec == 0 and threads == 512 and KERNEL_CHOICE == "auto" \
+            and (nvec // 512, nvec % 512 != 0) in ((7, True), (8, False), (12, True)):
+        # and for 16-bit rows of 32000 / 32768 / 50304 entries, scanned by 512 virtual threads
+        return f"actor_step_split_kernel<{dtype}, {nvec // 512}, {str(nvec % 512 != 0).lower()}, false, 512>"
     if vocab % per_vec == 0 and threads == width and shape in split_shapes and KERNEL_CHOICE == "auto":
         return f"actor_step_split_kernel<{dtype}, {shape[0]}, {str(shape[1]).lower()}>"
     if vocab % per_vec == 0 and threads == width and shape in shapes \

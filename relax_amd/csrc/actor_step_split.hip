@@ -99,14 +99,15 @@ __device__ __forceinline__ void split_publish(unsigned long long* slot, unsigned
   }
 }
 
-// Wave 0 of a workgroup: lanes 0 .. 47 fetch one word of the row's sixteen triples each (waiting, boundedly, for the
-// tag of this launch and lap), then every lane merges the sixteen in wave order, as thread 0 of a 1024-thread
-// workgroup does in scan_block_merge().
+// Wave 0 of a workgroup: lanes 0 .. 3 * ROW_WAVES - 1 fetch one word of the row's triples each (waiting, boundedly,
+// for the tag of this launch and lap), then every lane merges the ROW_WAVES triples in wave order, as thread 0 of a
+// workgroup of that many waves does in scan_block_merge().
+template <int ROW_WAVES = kRowWaves>
 __device__ __forceinline__ SoftmaxAcc split_collect(const unsigned long long* slot, unsigned tag, int tid,
                                                     bool& any_gave_up) {
   float word = 0.f;
   bool gave_up = false;
-  if (tid < kSlotWords) {
+  if (tid < ROW_WAVES * 3) {
     unsigned polls = 0;
     while (true) {
       const unsigned long long w = __hip_atomic_load(slot + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -125,11 +126,13 @@ __device__ __forceinline__ SoftmaxAcc split_collect(const unsigned long long* sl
   auto of_lane = [&](int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(word), l)); };
   SoftmaxAcc whole{of_lane(0), of_lane(1), of_lane(2)};
 #pragma unroll
-  for (int i = 1; i < kRowWaves; ++i) scan_merge(whole, of_lane(3 * i), of_lane(3 * i + 1), of_lane(3 * i + 2));
+  for (int i = 1; i < ROW_WAVES; ++i) scan_merge(whole, of_lane(3 * i), of_lane(3 * i + 1), of_lane(3 * i + 2));
   return whole;
 }
 
-template <typename T, int NVF, bool PARTIAL, bool TOPK>
+// ROW_THREADS: the virtual threads that scan a row, i.e. the width scan_threads() gives the forward-only kernel for this
+// row length (1024, or 512 for rows of 2048 .. 7167 vectors); ROW_THREADS / 128 workgroups share a row.
+template <typename T, int NVF, bool PARTIAL, bool TOPK, int ROW_THREADS = 1024>
 __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
     const T* __restrict__ logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
     const int32_t* __restrict__ token_of_row, const int32_t* __restrict__ sample_ids,
@@ -137,7 +140,7 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
     float* __restrict__ log_prob, float* __restrict__ entropy, float* __restrict__ lse_out,
     float* __restrict__ spx_out, T* __restrict__ dlogits, int64_t d_stride, unsigned long long* __restrict__ ring,
     unsigned laps) {
-  constexpr int kU = kScanUnroll, ROW_THREADS = 1024;
+  constexpr int kU = kScanUnroll, kParts = ROW_THREADS / kSplitThreads;
   constexpr int VN = Row<T>::kPerVec;
   constexpr int NV = NVF + (PARTIAL ? 1 : 0);
   constexpr int kGroups = (NV + kU - 1) / kU;
@@ -150,8 +153,8 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
   __shared__ u32x4 parked[kPark][kWave];
   const int tid = threadIdx.x;
   const bool wave0 = __builtin_amdgcn_readfirstlane(tid) < kWave;
-  const unsigned part = blockIdx.x % kSplit;
-  const int64_t row = blockIdx.x / kSplit;
+  const unsigned part = blockIdx.x % kParts;
+  const int64_t row = blockIdx.x / kParts;
   const int vt = int(part) * kSplitThreads + tid;  // virtual thread of the row
   const int rem = int(vocab / VN) - NVF * ROW_THREADS;
   auto has = [&](int j) -> bool { return j < NVF || (PARTIAL && j == NVF && vt < rem); };
@@ -244,7 +247,7 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
       topk_shape = topk_row_shape(a, tok);
     }
     bool any_gave_up = false;
-    const SoftmaxAcc whole = split_collect(slot, tag, tid, any_gave_up);
+    const SoftmaxAcc whole = split_collect<ROW_THREADS / kWave>(slot, tag, tid, any_gave_up);
     float lse = 0.f, spx = 0.f, ent = 0.f, lp = 0.f;
     if (tid == 0) {
       scan_finish(whole, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
@@ -625,18 +628,19 @@ static int split_ring_of_device(unsigned long long** ring) {
   return RELAX_AMD_OK;
 }
 
-#define RELAX_AMD_SPLIT(NVF, PARTIAL)                                                                                 \
-  if (full == NVF && partial == PARTIAL) {                                                                            \
+#define RELAX_AMD_SPLIT_ROW(WIDTH, NVF, PARTIAL)                                                                      \
+  if (width == WIDTH && full == NVF && partial == PARTIAL) {                                                          \
     if (a.topk_ids)                                                                                                   \
-      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, true>), grid, block, 0, stream, logits,           \
+      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, true, WIDTH>), grid, block, 0, stream, logits,    \
                          row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
                          grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps);                    \
     else                                                                                                              \
-      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, false>), grid, block, 0, stream, logits,          \
+      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, false, WIDTH>), grid, block, 0, stream, logits,   \
                          row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
                          grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps);                    \
     return check_launch("actor_step_split");                                                                          \
   }
+#define RELAX_AMD_SPLIT(NVF, PARTIAL) RELAX_AMD_SPLIT_ROW(1024, NVF, PARTIAL)
 
 template <typename T>
 int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
@@ -645,13 +649,17 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
                             float* entropy, float* lse, float* spx, T* dlogits, int64_t d_stride,
                             hipStream_t stream) {
   constexpr int VN = Row<T>::kPerVec;
-  if (vocab % VN != 0 || scan_threads(vocab, VN) != 1024 || n_rows * kSplit > 2147483647LL)
-    return RELAX_AMD_EUNSUPPORTED;
+  const int width = scan_threads(vocab, VN);  // the virtual threads of a row: the forward-only kernel's workgroup
+  if (vocab % VN != 0 || width < 512 || n_rows * kSplit > 2147483647LL) return RELAX_AMD_EUNSUPPORTED;
   const int64_t nvec = vocab / VN;
-  const int full = int(nvec / 1024);
-  const bool partial = nvec % 1024 != 0;
-  // the row shapes launch_actor_step_resident is built for
-  if constexpr (sizeof(T) == 2) {
+  const int full = int(nvec / width);
+  const bool partial = nvec % width != 0;
+  // the row shapes launch_actor_step_resident is built for, and 16-bit rows of 3585 .. 4096 and 6145 .. 6656 vectors
+  // (32000 / 32768 and 50304 entries) scanned by 512 virtual threads
+  if (width == 512) {
+    if (sizeof(T) != 2 || !((full == 7 && partial) || (full == 8 && !partial) || (full == 12 && partial)))
+      return RELAX_AMD_EUNSUPPORTED;
+  } else if constexpr (sizeof(T) == 2) {
     if (!((full == 20 && !partial) || (full == 19 && partial) || (full == 18 && partial) || (full == 15 && partial) ||
           (full == 16 && !partial) || (full == 12 && partial) || (full == 8 && !partial) || (full == 7 && partial)))
       return RELAX_AMD_EUNSUPPORTED;
@@ -664,8 +672,11 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
   if (int rc = split_ring_of_device(&ring)) return rc;
   const unsigned laps = unsigned((n_rows + kRing - 1) / kRing);
   hipLaunchKernelGGL(split_ring_advance_kernel, dim3(1), dim3(256), 0, stream, ring, laps);
-  const dim3 grid(static_cast<unsigned>(n_rows * kSplit)), block(kSplitThreads);
+  const dim3 grid(static_cast<unsigned>(n_rows * (width / kSplitThreads))), block(kSplitThreads);
   if constexpr (sizeof(T) == 2) {
+    RELAX_AMD_SPLIT_ROW(512, 7, true)
+    RELAX_AMD_SPLIT_ROW(512, 8, false)
+    RELAX_AMD_SPLIT_ROW(512, 12, true)
     RELAX_AMD_SPLIT(20, false)
     RELAX_AMD_SPLIT(19, true)
     RELAX_AMD_SPLIT(18, true)
@@ -684,6 +695,7 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
   return RELAX_AMD_EUNSUPPORTED;
 }
 #undef RELAX_AMD_SPLIT
+#undef RELAX_AMD_SPLIT_ROW
 
 #define RELAX_AMD_SPLIT_WIDE(NF, PARTIAL)                                                                             \
   if (full == NF && partial == PARTIAL) {                                                                             \

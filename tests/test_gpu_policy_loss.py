@@ -1727,6 +1727,8 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
 
 @pytest.mark.parametrize("v,dtype,n_rows,values", [
     (100352, torch.bfloat16, 700, "plain"), (32000, torch.float32, 1500, "plain"), (151936, torch.bfloat16, 300, "plain"),
+    # 16-bit rows scanned by 512 threads: no persistent kernel exists for them, the one-shot kernel does
+    (32000, torch.bfloat16, 1500, "short"), (50304, torch.float16, 1000, "short"),
     # long fp32 rows, kept in the registers as their upper halves: bf16 values widened to fp32 (what a bf16 output
     # layer followed by .float() delivers: one read of the row), fp32 values with low bits (the row is read again), and
     # rows of both kinds next to each other, one of them with a single low bit in its last element
@@ -1788,6 +1790,8 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
     targets = torch.randint(0, v, (n_tok,), generator=g).to(dev)
     results = {}
     for kind in ("cached", "resident", "auto", "auto_again"):
+        if values == "short" and kind == "resident":
+            kind = "auto"  # (RESIDENT fails for these rows by design)
         ops.set_kernel_choice({"cached": "two_walk", "resident": "resident"}.get(kind, "auto"))
         out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, token_of_row, sample_ids, n_tok, 1.0, 1.0, **kw)
         torch.cuda.synchronize()
@@ -1795,11 +1799,13 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
                              d=d.view(torch.int16 if dtype != torch.float32 else torch.int32),
                              coef_ent=out["coef_entropy"], metrics=out["metrics"])
     for kind in ("resident", "auto", "auto_again"):
+        if kind not in results:
+            continue
         for key, want in results["cached"].items():
             got = results[kind][key]
             assert torch.equal(got, want), (kind, pattern, key, (got.float() - want.float()).abs().max())
     if pattern == "all_dead":
-        assert not results["resident"]["d"].any() and not results["auto"]["d"].any()
+        assert not results["auto_again"]["d"].any() and not results["auto"]["d"].any()
 
 
 def test_default_fused_step_replayed_from_a_captured_graph():
@@ -1922,7 +1928,10 @@ def test_long_fp32_rows_resident_as_upper_halves_equal_two_walk_kernel_and_oracl
                                      (8 * (12 * 1024 + 1), torch.float16), (8 * (16 * 1024 - 1), torch.bfloat16),
                                      (4 * (7 * 1024 + 1), torch.float32), (4 * (8 * 1024 - 1), torch.float32),
                                      (8 * (7 * 1024 + 1), torch.bfloat16), (8 * 8 * 1024, torch.float16),
-                                     (4 * (12 * 1024 + 1), torch.float32), (4 * (16 * 1024 - 1), torch.float32)])
+                                     (4 * (12 * 1024 + 1), torch.float32), (4 * (16 * 1024 - 1), torch.float32),
+                                     # 512 virtual threads: one-shot kernel only
+                                     (8 * (7 * 512 + 1), torch.bfloat16), (8 * 8 * 512, torch.float16),
+                                     (8 * (13 * 512 - 1), torch.bfloat16)])
 def test_register_resident_kernel_at_the_edges_of_its_row_shapes(v, dtype):
     """Row lengths at both ends of a built shape: one lane, or all lanes but one, hold a vector at the partially filled
     position.  Every output bit-identical to the two-walk kernel's."""
@@ -1949,6 +1958,8 @@ def test_register_resident_kernel_at_the_edges_of_its_row_shapes(v, dtype):
     sample_ids = torch.zeros(n_tok, dtype=torch.int32, device=dev)
     results = {}
     for kind in ("cached", "resident", "auto"):
+        if kind == "resident" and v // (4 if dtype == torch.float32 else 8) < 7168:
+            continue  # rows scanned by 512 threads have no persistent kernel
         ops.set_kernel_choice({"cached": "two_walk", "resident": "resident"}.get(kind, "auto"))
         out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets.to(dev), token_of_row, sample_ids, n_tok, 1.0,
                                                          1.0, **kw)
@@ -1956,9 +1967,11 @@ def test_register_resident_kernel_at_the_edges_of_its_row_shapes(v, dtype):
         results[kind] = dict(lp=lp, ent=ent, lse=lse, spx=spx, coef=out["coef_log_prob"],
                              d=d.view(torch.int16 if dtype != torch.float32 else torch.int32))
     for kind in ("resident", "auto"):
+        if kind not in results:
+            continue
         for key, want in results["cached"].items():
             assert torch.equal(results[kind][key], want), (kind, key)
-    assert results["resident"]["d"].any()
+    assert results["auto"]["d"].any()
 
 
 def test_forward_only_topk_gather_on_logits_that_require_grad():
