@@ -91,7 +91,8 @@ enum { RELAX_AMD_KERNEL_AUTO = 0, RELAX_AMD_KERNEL_TWO_WALK = 1, RELAX_AMD_KERNE
  * not both take that kernel: they could overwrite each other's slots, which the kernel notices (bounded waits) and
  * reports as NaN log-probs rather than wrong numbers.  Launches in stream order, captured graphs and their replays
  * are fine (the tags that tell one launch's partial sums from another's come from a counter in device memory that a
- * small kernel in front of each launch advances).
+ * small kernel in front of each launch advances); the first call on a GPU looks the ring's address up
+ * (hipGetSymbolAddress), so make one call outside a capture first.
  */
 int relax_amd_set_kernel_choice(int choice);
 
