@@ -67,7 +67,7 @@ __device__ __forceinline__ void split_absorb_raw_group(const u32x4* raw, float c
   }
   const float mc = __fmul_rn(vmax, c);
   if (mc > st.m) {
-    const float sc = fast_exp2(__fsub_rn(st.m, mc));
+    const float sc = fast_exp2(fmaf(-vmax, c, st.m));  // one rounding, spelled out (see scan_finish)
     st.s = __fmul_rn(st.s, sc);
     st.t = __fmul_rn(st.t, sc);
     st.m = mc;

@@ -2,7 +2,8 @@
 // take the same path through this file with the same workgroup shape for a given row length, so for one logits row
 // they produce bit-identical (max, sum exp, sum exp*x): the forward-only pass (old / reference log-probs) and the
 // training forward then agree exactly, which Relax's step-0 check (ppo_kl == 0 for identical weights) relies on.
-// All combining arithmetic is written with explicit fma / mul / add so no context-dependent contraction can creep in.
+// Wherever a product feeds a sum the fused multiply-add is written out, so that no context-dependent contraction of a
+// separate multiply and add can creep in.
 #pragma once
 
 #include "device_utils.h"
@@ -25,7 +26,7 @@ __device__ __forceinline__ float scan_absorb(const float (&v)[K], float c, Softm
   for (int i = 1; i < K; ++i) vmax = fmaxf(vmax, v[i]);
   const float mc = __fmul_rn(vmax, c);
   if (mc > st.m) {
-    const float sc = fast_exp2(__fsub_rn(st.m, mc));
+    const float sc = fast_exp2(fmaf(-vmax, c, st.m));  // one rounding, spelled out (see scan_finish)
     st.s = __fmul_rn(st.s, sc);
     if (WITH_T) st.t = __fmul_rn(st.t, sc);
     st.m = mc;
@@ -122,8 +123,12 @@ __device__ __forceinline__ void scan_block_merge(SoftmaxAcc& st, float (*wave_st
 __device__ __forceinline__ void scan_finish(const SoftmaxAcc& st, float x_target, bool target_ok, float inv_t,
                                             float& lse, float& spx, float& ent, float& lp) {
   lse = fmaf(st.m, kLn2, logf(st.s));
-  spx = __fmul_rn(__fdiv_rn(st.t, st.s), inv_t);
-  ent = __fsub_rn(lse, spx);
+  const float q = __fdiv_rn(st.t, st.s);
+  spx = __fmul_rn(q, inv_t);
+  // A product feeding a sum is written as the fused multiply-add it may become: __fmul_rn / __fsub_rn are a plain
+  // `*` / `-` to this compiler, which contracts them or not depending on the code around the call, so lse - q * inv_t
+  // came out with one rounding in some kernels and two in others when the temperature is not 1.
+  ent = fmaf(-q, inv_t, lse);
   lp = target_ok ? fmaf(x_target, inv_t, -lse) : __builtin_nanf("");
 }
 

@@ -1808,6 +1808,115 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
         assert not results["auto_again"]["d"].any() and not results["auto"]["d"].any()
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_one_shot_step_on_random_layouts_equals_two_walk_kernel_bitwise(seed):
+    """Random row counts (from a single row up), row lengths from every family the one-shot kernel is built for (and
+    their neighbours by one vector), element types, row maps with unscored rows, masks, temperatures and loss options:
+    the default kernel choice against the two-walk kernel, every output bit for bit.  Small row counts leave most of
+    the chip idle, large ones wrap the exchange ring's 4096 slots."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(1000 + seed)
+    families = [(torch.bfloat16, 8, [18 * 1024 + 560, 12 * 1024 + 256, 20 * 1024, 16 * 1024, 15 * 1024 + 1023,
+                                     7 * 1024 + 832, 8 * 1024, 7 * 512 + 416, 8 * 512, 12 * 512 + 144]),
+                (torch.float16, 8, [18 * 1024 + 1, 19 * 1024 + 5, 12 * 512 + 1]),
+                (torch.float32, 4, [7 * 1024 + 832, 8 * 1024, 12 * 1024 + 3, 16 * 1024, 37 * 1024 + 96, 24 * 1024 + 512])]
+    dtype, per_vec, nvecs = families[seed % 3]
+    nvec = nvecs[int(torch.randint(0, len(nvecs), (1,), generator=g))]
+    v = nvec * per_vec
+    budget = 160_000_000 // (v * (4 if dtype == torch.float32 else 2))
+    n_rows = [1, 7, 8, 9, 63][seed % 5] if seed < 10 else int(torch.randint(64, max(65, min(budget, 5000)), (1,), generator=g))
+    announce("one-shot step, random layout", seed, v, dtype, n_rows)
+    logits = (torch.randn(n_rows, v, generator=g) * 2).to(dtype)
+    if dtype == torch.float32 and nvec > 20000 and seed % 2 == 0:
+        logits = logits.bfloat16().float()  # widened rows: the upper-halves form reads them once
+    logits = logits.to(dev)
+    if seed % 4 == 3:
+        token_of_row, n_tok = None, n_rows
+    else:
+        scores = torch.rand(n_rows, generator=g) > 0.3
+        scores[int(torch.randint(0, n_rows, (1,), generator=g))] = True
+        idx = torch.cumsum(scores.int(), 0) - 1
+        token_of_row = torch.where(scores, idx, torch.full_like(idx, -1)).int().to(dev)
+        n_tok = int(scores.sum())
+    mask = (torch.rand(n_tok, generator=g) > 0.25).float()
+    base = -11.0 + 0.3 * torch.randn(n_tok, generator=g)
+    n_a = max(1, n_tok // 2)
+    lens = [n_a, n_tok - n_a] if n_tok > 1 else [1]
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int64, device=dev)
+    sample_ids = torch.cat([torch.full((n,), i, dtype=torch.int32) for i, n in enumerate(lens)]).to(dev)
+    denom = torch.tensor([max(1.0, mask[sample_ids.cpu() == i].sum().item()) for i in range(len(lens))], device=dev)
+    kw = dict(advantages=torch.randn(n_tok, generator=g).to(dev), loss_mask=mask.to(dev), cu_resp=cu,
+              old_log_prob=base.to(dev), sample_denom=denom, loss_kind=["ppo", "cispo", "sapo"][seed % 3],
+              eps_clip=0.2, eps_clip_high=0.28)
+    if seed % 2 == 0:
+        kw.update(ref_log_prob=(base + 0.1 * torch.randn(n_tok, generator=g)).to(dev),
+                  kl_kind=["k1", "k2", "k3", "low_var_kl"][(seed // 2) % 4], kl_coef=1e-3)
+    if seed % 3 != 1:
+        kw.update(entropy_coef=0.01)
+    targets = torch.randint(0, v, (n_tok,), generator=g).to(dev)
+    inv_t = [1.0, 1.0 / 0.7][seed % 2]
+    results = {}
+    for kind in ("two_walk", "auto"):
+        ops.set_kernel_choice(kind)
+        out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, token_of_row, sample_ids, n_tok, inv_t, 1.0, **kw)
+        torch.cuda.synchronize()
+        results[kind] = dict(lp=lp, ent=ent, lse=lse, spx=spx, coef=out["coef_log_prob"], coef_ent=out["coef_entropy"],
+                             d=d.view(torch.int16 if dtype != torch.float32 else torch.int32))
+    ops.set_kernel_choice("auto")
+    for key, want in results["two_walk"].items():
+        got = results["auto"][key]
+        if want is None:
+            assert got is None
+            continue
+        assert torch.equal(got, want), (seed, key, (got.float() - want.float()).abs().max())
+    assert not torch.isnan(results["auto"]["lp"]).any()
+
+
+@pytest.mark.parametrize("v,dtype", [(151936, torch.bfloat16), (32000, torch.float32), (32000, torch.float16),
+                                     (4 * (37 * 1024 + 96), torch.float32)])
+def test_log_probs_and_entropy_of_every_kernel_agree_bitwise_at_a_temperature(v, dtype):
+    """The forward-only pass, the log-prob + top-K pass and the fused step in each of its kernels give one set of bits
+    for log-prob, entropy, log-sum-exp and sum p*x at a temperature other than 1 (where a product of the temperature
+    feeds the entropy's subtraction: written as separate operations the compiler fused it in some kernels and not in
+    others).  This is what lets the reference's step-0 check see exactly zero KL between the passes."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("one set of bits at T = 0.7", v, dtype)
+    g = torch.Generator().manual_seed(v)
+    n = 300
+    logits = (torch.randn(n, v, generator=g) * 2).to(dtype)
+    if dtype == torch.float32 and v > 100000:
+        logits = logits.bfloat16().float()
+    logits = logits.to(dev)
+    targets = torch.randint(0, v, (n,), generator=g).to(dev)
+    inv_t = 1.0 / 0.7
+    want = dict(zip(("lp", "ent", "lse", "spx"), ops.logprob_entropy_fwd(logits, targets, None, inv_t)))
+    got = ops.logprob_entropy_topk_fwd(logits, targets, None, inv_t, 16)
+    for key, t in zip(("lp", "ent", "lse", "spx"), got[:4]):
+        assert torch.equal(t, want[key]), ("top-K forward", key)
+    lp_only = ops.logprob_entropy_fwd(logits, targets, None, inv_t, with_entropy=False)
+    assert torch.equal(lp_only[0], want["lp"]) and torch.equal(lp_only[2], want["lse"])
+    base = want["lp"].cpu() + 0.05 * torch.randn(n, generator=g)
+    kw = dict(advantages=torch.randn(n, generator=g).to(dev), loss_mask=torch.ones(n, device=dev),
+              cu_resp=torch.tensor([0, n], dtype=torch.int64, device=dev), old_log_prob=base.to(dev),
+              sample_denom=torch.tensor([float(n)], device=dev), loss_kind="ppo", eps_clip=0.2, eps_clip_high=0.28,
+              entropy_coef=0.01)
+    sample_ids = torch.zeros(n, dtype=torch.int32, device=dev)
+    per_vec = 4 if dtype == torch.float32 else 8
+    for kind in ("two_walk", "resident", "auto"):
+        if kind == "resident" and v // per_vec < 7168:
+            continue
+        ops.set_kernel_choice(kind)
+        out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, None, sample_ids, n, inv_t, 1.0, **kw)
+        torch.cuda.synchronize()
+        for key, t in (("lp", lp), ("ent", ent), ("lse", lse), ("spx", spx)):
+            assert torch.equal(t, want[key]), (kind, key, (t - want[key]).abs().max())
+    ops.set_kernel_choice("auto")
+
+
 def test_default_fused_step_replayed_from_a_captured_graph():
     """The default fused step tags the partial sums its workgroups exchange with a counter that a small kernel in front
     of the launch advances on the device, so a captured launch gets fresh tags on every replay: three replays on fresh
