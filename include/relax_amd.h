@@ -97,6 +97,15 @@ enum { RELAX_AMD_KERNEL_AUTO = 0, RELAX_AMD_KERNEL_TWO_WALK = 1, RELAX_AMD_KERNE
 int relax_amd_set_kernel_choice(int choice);
 
 /*
+ * For tests of the one-shot actor step's failure handling: max_polls bounds how often a workgroup looks for its
+ * neighbours' partial sums before it gives up (0 = the default, 2^20), wait_tag_offset is added to the tag it looks
+ * for (0 = none; with 1 no wait can succeed).  A launch made with (a few, 1) therefore exercises the give-up path on
+ * every row without any workgroup hanging: log-probs and log-sum-exps of the scored tokens come back NaN.
+ * Process-wide, read at each launch.  No counterpart in the reference.
+ */
+int relax_amd_set_exchange_wait(int max_polls, int wait_tag_offset);
+
+/*
  * Target-token log-prob and full-vocab entropy of each row, one streaming
  * read of the row.  Replaces _VocabParallelLogProbEntropy.forward
  * (relax/utils/training/ppo_utils.py:481-589, single vocab shard) together

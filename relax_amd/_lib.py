@@ -75,6 +75,7 @@ SIGNATURES = {
     "relax_amd_version": (C.c_int, []),
     "relax_amd_last_error": (C.c_char_p, []),
     "relax_amd_set_kernel_choice": (C.c_int, [C.c_int]),
+    "relax_amd_set_exchange_wait": (C.c_int, [C.c_int, C.c_int]),
     "relax_amd_logprob_entropy_fwd": (C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp]),
     "relax_amd_logprob_entropy_bwd": (
         C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _f32, _vp, _i64, _vp]),

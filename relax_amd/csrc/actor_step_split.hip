@@ -30,6 +30,7 @@
 //
 // As in actor_step_resident.hip the row sits at the edge of the register file:
 // hipcc-flags: -mllvm -amdgpu-use-amdgpu-trackers=1
+#include <atomic>
 #include <mutex>
 
 #include "actor_step_resident.h"
@@ -104,7 +105,7 @@ __device__ __forceinline__ void split_publish(unsigned long long* slot, unsigned
 // workgroup of that many waves does in scan_block_merge().
 template <int ROW_WAVES = kRowWaves>
 __device__ __forceinline__ SoftmaxAcc split_collect(const unsigned long long* slot, unsigned tag, int tid,
-                                                    bool& any_gave_up) {
+                                                    unsigned max_polls, bool& any_gave_up) {
   float word = 0.f;
   bool gave_up = false;
   if (tid < ROW_WAVES * 3) {
@@ -115,7 +116,7 @@ __device__ __forceinline__ SoftmaxAcc split_collect(const unsigned long long* sl
         word = __uint_as_float(unsigned(w));
         break;
       }
-      if (++polls > kWaitPolls) {
+      if (++polls > max_polls) {
         gave_up = true;
         break;
       }
@@ -139,7 +140,7 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
     const int64_t* __restrict__ targets, float c, float inv_t, relax_amd_policy_loss_args a, float grad_scale,
     float* __restrict__ log_prob, float* __restrict__ entropy, float* __restrict__ lse_out,
     float* __restrict__ spx_out, T* __restrict__ dlogits, int64_t d_stride, unsigned long long* __restrict__ ring,
-    unsigned laps) {
+    unsigned laps, unsigned max_polls, unsigned wait_tag_offset) {
   constexpr int kU = kScanUnroll, kParts = ROW_THREADS / kSplitThreads;
   constexpr int VN = Row<T>::kPerVec;
   constexpr int NV = NVF + (PARTIAL ? 1 : 0);
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
       topk_shape = topk_row_shape(a, tok);
     }
     bool any_gave_up = false;
-    const SoftmaxAcc whole = split_collect<ROW_THREADS / kWave>(slot, tag, tid, any_gave_up);
+    const SoftmaxAcc whole = split_collect<ROW_THREADS / kWave>(slot, tag + wait_tag_offset, tid, max_polls, any_gave_up);
     float lse = 0.f, spx = 0.f, ent = 0.f, lp = 0.f;
     if (tid == 0) {
       scan_finish(whole, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
@@ -361,7 +362,7 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_wide_kernel
     const int64_t* __restrict__ targets, float c, float inv_t, relax_amd_policy_loss_args a, float grad_scale,
     float* __restrict__ log_prob, float* __restrict__ entropy, float* __restrict__ lse_out,
     float* __restrict__ spx_out, float* __restrict__ dlogits, int64_t d_stride, unsigned long long* __restrict__ ring,
-    unsigned laps) {
+    unsigned laps, unsigned max_polls, unsigned wait_tag_offset) {
   constexpr int kU = kScanUnroll, ROW_THREADS = 1024;
   constexpr int NP = NF + (PARTIAL ? 1 : 0);  // vector positions per thread
   static_assert(kU == 4, "positions are packed in pairs and scanned in groups of four");
@@ -486,7 +487,7 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_wide_kernel
       pg_den = a.pg_sample_denom ? a.pg_sample_denom[sid] : den;
     }
     bool any_gave_up = false;
-    const SoftmaxAcc whole = split_collect(slot, tag, tid, any_gave_up);
+    const SoftmaxAcc whole = split_collect(slot, tag + wait_tag_offset, tid, max_polls, any_gave_up);
     if (tid == 0) {
       float lse = 0.f, spx = 0.f, ent = 0.f, lp = 0.f;
       scan_finish(whole, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
@@ -603,6 +604,8 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::mutex ring_mutex;
 unsigned long long* ring_ptr[kMaxDevices] = {};
+// relax_amd_set_exchange_wait: the bound of a workgroup's wait and an offset added to the tag it waits for
+std::atomic<unsigned> g_max_polls{kWaitPolls}, g_wait_tag_offset{0u};
 }  // namespace
 
 // the current device's ring (looked up once per device, with that device current)
@@ -633,11 +636,13 @@ static int split_ring_of_device(unsigned long long** ring) {
     if (a.topk_ids)                                                                                                   \
       hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, true, WIDTH>), grid, block, 0, stream, logits,    \
                          row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
-                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps);                    \
+                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps, max_polls,          \
+                         tag_offset);                                                                                 \
     else                                                                                                              \
       hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, false, WIDTH>), grid, block, 0, stream, logits,   \
                          row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
-                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps);                    \
+                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps, max_polls,          \
+                         tag_offset);                                                                                 \
     return check_launch("actor_step_split");                                                                          \
   }
 #define RELAX_AMD_SPLIT(NVF, PARTIAL) RELAX_AMD_SPLIT_ROW(1024, NVF, PARTIAL)
@@ -671,6 +676,8 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
   unsigned long long* ring = nullptr;
   if (int rc = split_ring_of_device(&ring)) return rc;
   const unsigned laps = unsigned((n_rows + kRing - 1) / kRing);
+  const unsigned max_polls = g_max_polls.load(std::memory_order_relaxed);
+  const unsigned tag_offset = g_wait_tag_offset.load(std::memory_order_relaxed);
   hipLaunchKernelGGL(split_ring_advance_kernel, dim3(1), dim3(256), 0, stream, ring, laps);
   const dim3 grid(static_cast<unsigned>(n_rows * (width / kSplitThreads))), block(kSplitThreads);
   if constexpr (sizeof(T) == 2) {
@@ -701,7 +708,7 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
   if (full == NF && partial == PARTIAL) {                                                                             \
     hipLaunchKernelGGL((actor_step_split_wide_kernel<NF, PARTIAL>), grid, block, 0, stream, logits, row_stride,      \
                        vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a, grad_scale,       \
-                       log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps);                                  \
+                       log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps, max_polls, tag_offset);           \
     return check_launch("actor_step_split_wide");                                                                     \
   }
 
@@ -722,6 +729,8 @@ int launch_actor_step_split_wide(const float* logits, int64_t row_stride, int64_
   unsigned long long* ring = nullptr;
   if (int rc = split_ring_of_device(&ring)) return rc;
   const unsigned laps = unsigned((n_rows + kRing - 1) / kRing);
+  const unsigned max_polls = g_max_polls.load(std::memory_order_relaxed);
+  const unsigned tag_offset = g_wait_tag_offset.load(std::memory_order_relaxed);
   hipLaunchKernelGGL(split_ring_advance_kernel, dim3(1), dim3(256), 0, stream, ring, laps);
   const dim3 grid(static_cast<unsigned>(n_rows * kSplit)), block(kSplitThreads);
   // 151936 / 152064 (37984 / 38016 vectors), 128256 / 129280 (32064 / 32320), 131072 (32768), 163840 (40960),
@@ -748,3 +757,13 @@ template int launch_actor_step_split<f16_t>(const f16_t*, int64_t, int64_t, int6
 
 }  // namespace relax_amd
 
+
+extern "C" int relax_amd_set_exchange_wait(int max_polls, int wait_tag_offset) {
+  if (max_polls < 0 || wait_tag_offset < 0) {
+    relax_amd::set_error("set_exchange_wait: negative argument");
+    return RELAX_AMD_EINVAL;
+  }
+  relax_amd::g_max_polls.store(max_polls == 0 ? relax_amd::kWaitPolls : unsigned(max_polls), std::memory_order_relaxed);
+  relax_amd::g_wait_tag_offset.store(unsigned(wait_tag_offset), std::memory_order_relaxed);
+  return RELAX_AMD_OK;
+}

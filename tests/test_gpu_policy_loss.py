@@ -1917,6 +1917,51 @@ def test_log_probs_and_entropy_of_every_kernel_agree_bitwise_at_a_temperature(v,
     ops.set_kernel_choice("auto")
 
 
+def test_one_shot_step_gives_up_a_wait_that_cannot_succeed_and_recovers():
+    """Failure handling of the exchange between the workgroups of a row, forced from the host
+    (relax_amd_set_exchange_wait): with the tag a workgroup waits for offset by one, no wait can succeed; bounded to a
+    few looks, every workgroup gives up, writes NaN log-probs / log-sum-exps for its row and exits normally.  The next
+    launch with the defaults restored is exact again (tags moved on, nothing of the failed launch is mistaken for
+    this one's)."""
+    from relax_amd import ops
+    from relax_amd._lib import check, lib
+
+    dev = require_gpu()
+    announce("one-shot step: give-up path")
+    v, n = 100352, 200
+    g = torch.Generator().manual_seed(11)
+    logits = (torch.randn(n, v, generator=g) * 2).bfloat16().to(dev)
+    mask = (torch.rand(n, generator=g) > 0.2).float()
+    base = -11.0 + 0.3 * torch.randn(n, generator=g)
+    kw = dict(advantages=torch.randn(n, generator=g).to(dev), loss_mask=mask.to(dev),
+              cu_resp=torch.tensor([0, n], dtype=torch.int64, device=dev), old_log_prob=base.to(dev),
+              sample_denom=torch.tensor([max(1.0, mask.sum().item())], device=dev), loss_kind="ppo", eps_clip=0.2,
+              eps_clip_high=0.28, entropy_coef=0.01)
+    sample_ids = torch.zeros(n, dtype=torch.int32, device=dev)
+    targets = torch.randint(0, v, (n,), generator=g).to(dev)
+
+    def run():
+        out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, None, sample_ids, n, 1.0, 1.0, **kw)
+        torch.cuda.synchronize()
+        return lp, lse, d
+
+    ops.set_kernel_choice("two_walk")
+    want = run()
+    ops.set_kernel_choice("auto")
+    check(lib.relax_amd_set_exchange_wait(4, 1))
+    try:
+        lp, lse, d = run()
+    finally:
+        check(lib.relax_amd_set_exchange_wait(0, 0))
+    live = (mask != 0).to(dev)
+    assert torch.isnan(lp[live]).all() and torch.isnan(lse[live]).all()
+    assert (lp[~live] == 0).all() and not d[~live].any()  # rows of masked tokens wait for nobody
+    lp, lse, d = run()
+    for got, w in zip((lp, lse, d.view(torch.int16)), (want[0], want[1], want[2].view(torch.int16))):
+        assert torch.equal(got, w)
+    assert lib.relax_amd_set_exchange_wait(-1, 0) != 0
+
+
 def test_default_fused_step_replayed_from_a_captured_graph():
     """The default fused step tags the partial sums its workgroups exchange with a counter that a small kernel in front
     of the launch advances on the device, so a captured launch gets fresh tags on every replay: three replays on fresh
