@@ -98,8 +98,9 @@ int relax_amd_set_kernel_choice(int choice);
 
 /*
  * For tests of the one-shot actor step's failure handling: max_polls bounds how often a workgroup looks for its
- * neighbours' partial sums before it gives up (0 = the default, 2^20), wait_tag_offset is added to the tag it looks
- * for (0 = none; with 1 no wait can succeed).  A launch made with (a few, 1) therefore exercises the give-up path on
+ * neighbours' partial sums before it gives up (0 = the default), wait_tag_offset is added to the tag it looks
+ * for (0 = none; with 1 no wait can succeed; the default bound is 2^17 looks, and the first give-up of a launch ends
+ * the launch's other waits at their next check of a flag).  A launch made with (a few, 1) therefore exercises the give-up path on
  * every row without any workgroup hanging: log-probs and log-sum-exps of the scored tokens come back NaN.
  * Process-wide, read at each launch.  No counterpart in the reference.
  */

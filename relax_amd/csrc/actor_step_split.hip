@@ -46,10 +46,12 @@ constexpr int kRowWaves = 16;             // waves of the 1024 virtual threads o
 constexpr int kSlotWords = kRowWaves * 3;
 constexpr int kSplitThreads = 128;        // virtual threads per workgroup
 constexpr int kSplit = 1024 / kSplitThreads;
-constexpr unsigned kWaitPolls = 1u << 20;
+constexpr unsigned kWaitPolls = 1u << 17;  // looks at a neighbour's word before a wait gives up (a few suffice; each takes microseconds)
 constexpr size_t kRingWords = size_t(kRing) * kSlotWords;
 
-// the exchange ring and, behind it, two 32-bit words: the tag counter and the count of waits that gave up
+// the exchange ring and, behind it, three 32-bit words: the tag counter, the count of waits that gave up, and a flag
+// that the first give-up of a launch raises so that the launch's other waits end at their next look at it (a launch
+// whose exchange is broken then ends within the time of one bounded wait instead of one per workgroup)
 static __device__ __align__(256) unsigned long long split_ring[kRingWords + 32];
 
 // scan_absorb() over the values of kScanUnroll raw vectors (as in actor_step_resident.hip: same arithmetic, same
@@ -105,7 +107,7 @@ __device__ __forceinline__ void split_publish(unsigned long long* slot, unsigned
 // workgroup of that many waves does in scan_block_merge().
 template <int ROW_WAVES = kRowWaves>
 __device__ __forceinline__ SoftmaxAcc split_collect(const unsigned long long* slot, unsigned tag, int tid,
-                                                    unsigned max_polls, bool& any_gave_up) {
+                                                    unsigned max_polls, unsigned* status, bool& any_gave_up) {
   float word = 0.f;
   bool gave_up = false;
   if (tid < ROW_WAVES * 3) {
@@ -116,7 +118,9 @@ __device__ __forceinline__ SoftmaxAcc split_collect(const unsigned long long* sl
         word = __uint_as_float(unsigned(w));
         break;
       }
-      if (++polls > max_polls) {
+      ++polls;
+      if (polls > max_polls ||
+          ((polls & 63u) == 0u && __hip_atomic_load(status + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
         gave_up = true;
         break;
       }
@@ -124,6 +128,10 @@ __device__ __forceinline__ SoftmaxAcc split_collect(const unsigned long long* sl
     }
   }
   any_gave_up = __any(gave_up);
+  if (any_gave_up && tid == 0) {
+    atomicAdd(status + 1, 1u);
+    __hip_atomic_store(status + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
   auto of_lane = [&](int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(word), l)); };
   SoftmaxAcc whole{of_lane(0), of_lane(1), of_lane(2)};
 #pragma unroll
@@ -248,14 +256,12 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
       topk_shape = topk_row_shape(a, tok);
     }
     bool any_gave_up = false;
-    const SoftmaxAcc whole = split_collect<ROW_THREADS / kWave>(slot, tag + wait_tag_offset, tid, max_polls, any_gave_up);
+    const SoftmaxAcc whole = split_collect<ROW_THREADS / kWave>(slot, tag + wait_tag_offset, tid, max_polls,
+                                                                reinterpret_cast<unsigned*>(ring + kRingWords), any_gave_up);
     float lse = 0.f, spx = 0.f, ent = 0.f, lp = 0.f;
     if (tid == 0) {
       scan_finish(whole, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
-      if (any_gave_up) {
-        lp = lse = __builtin_nanf("");
-        atomicAdd(reinterpret_cast<unsigned*>(ring + kRingWords) + 1, 1u);
-      }
+      if (any_gave_up) lp = lse = __builtin_nanf("");
       if (part == 0) {
         log_prob[tok] = lp;
         entropy[tok] = ent;
@@ -487,14 +493,12 @@ __global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_wide_kernel
       pg_den = a.pg_sample_denom ? a.pg_sample_denom[sid] : den;
     }
     bool any_gave_up = false;
-    const SoftmaxAcc whole = split_collect(slot, tag + wait_tag_offset, tid, max_polls, any_gave_up);
+    const SoftmaxAcc whole = split_collect(slot, tag + wait_tag_offset, tid, max_polls,
+                                           reinterpret_cast<unsigned*>(ring + kRingWords), any_gave_up);
     if (tid == 0) {
       float lse = 0.f, spx = 0.f, ent = 0.f, lp = 0.f;
       scan_finish(whole, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
-      if (any_gave_up) {
-        lp = lse = __builtin_nanf("");
-        atomicAdd(reinterpret_cast<unsigned*>(ring + kRingWords) + 1, 1u);
-      }
+      if (any_gave_up) lp = lse = __builtin_nanf("");
       if (part == 0) {
         log_prob[tok] = lp;
         entropy[tok] = ent;
@@ -597,7 +601,10 @@ __global__ __launch_bounds__(256) void split_ring_advance_kernel(unsigned long l
   if (wrap)
     for (size_t i = threadIdx.x; i < kRingWords; i += 256) ring[i] = 0ull;
   __syncthreads();
-  if (threadIdx.x == 0) counter[0] = (wrap ? 0u : now) + laps;
+  if (threadIdx.x == 0) {
+    counter[0] = (wrap ? 0u : now) + laps;
+    counter[2] = 0u;  // no wait of the launch that follows has given up yet
+  }
 }
 
 namespace {
