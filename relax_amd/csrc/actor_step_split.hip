@@ -141,8 +141,10 @@ __device__ __forceinline__ SoftmaxAcc split_collect(const unsigned long long* sl
 
 // ROW_THREADS: the virtual threads that scan a row, i.e. the width scan_threads() gives the forward-only kernel for this
 // row length (1024, or 512 for rows of 2048 .. 7167 vectors); ROW_THREADS / 128 workgroups share a row.
-template <typename T, int NVF, bool PARTIAL, bool TOPK, int ROW_THREADS = 1024>
-__global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_kernel(
+// WAVES_MIN / WAVES_MAX: the waves per SIMD the register allocation aims for (see split_waves_min()).
+template <typename T, int NVF, bool PARTIAL, bool TOPK, int ROW_THREADS, int WAVES_MIN, int WAVES_MAX>
+__global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(WAVES_MIN, WAVES_MAX)))
+void actor_step_split_kernel(
     const T* __restrict__ logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
     const int32_t* __restrict__ token_of_row, const int32_t* __restrict__ sample_ids,
     const int64_t* __restrict__ targets, float c, float inv_t, relax_amd_policy_loss_args a, float grad_scale,
@@ -361,8 +363,9 @@ __device__ __forceinline__ void split_wide_unpack(const u32x4& r, int half, floa
 // halves (38 four-float positions per thread in 19 register quads at V = 151936), scans the fp32 values as they land,
 // ORs the low halves it drops; a wave that dropped nothing computes its gradient from the registers, a wave that did
 // (fp32 logits with real low bits) reads its share again.  Exchange, tags and waits as in actor_step_split_kernel.
+// (three waves per SIMD: 5.80 ms on 32768 x 151936 fp32 rows where four give 5.91 and two 5.75)
 template <int NF, bool PARTIAL>
-__global__ __launch_bounds__(kSplitThreads, 4) void actor_step_split_wide_kernel(
+__global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void actor_step_split_wide_kernel(
     const float* __restrict__ logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
     const int32_t* __restrict__ token_of_row, const int32_t* __restrict__ sample_ids,
     const int64_t* __restrict__ targets, float c, float inv_t, relax_amd_policy_loss_args a, float grad_scale,
@@ -638,15 +641,30 @@ static int split_ring_of_device(unsigned long long** ring) {
   return RELAX_AMD_OK;
 }
 
+// Waves per SIMD the kernel is compiled for.  Long 16-bit rows without the top-K term run fastest with three (six
+// workgroups per CU, up to 168 registers a lane: 5.64 - 5.66 ms on the 65536 x 151936 step where four give 5.74 and
+// two 6.03; rows of 15 and more vectors per thread all gain 1 - 2.5 %), the top-K instantiations and rows of up to 13
+// vectors per thread with four or more (their thread 0 works longer per row, or they need few registers anyway).
+template <int NV, bool TOPK, int VN>
+constexpr int split_waves_min() {
+  return (!TOPK && VN == 8 && NV >= 15) ? 3 : 4;
+}
+template <int NV, bool TOPK, int VN>
+constexpr int split_waves_max() {
+  return (!TOPK && VN == 8 && NV >= 15) ? 3 : 8;
+}
+#define RELAX_AMD_SPLIT_KERNEL(WIDTH, NVF, PARTIAL, TOPK)                                                             \
+  actor_step_split_kernel<T, NVF, PARTIAL, TOPK, WIDTH, split_waves_min<NVF + (PARTIAL ? 1 : 0), TOPK, VN>(),         \
+                          split_waves_max<NVF + (PARTIAL ? 1 : 0), TOPK, VN>()>
 #define RELAX_AMD_SPLIT_ROW(WIDTH, NVF, PARTIAL)                                                                      \
   if (width == WIDTH && full == NVF && partial == PARTIAL) {                                                          \
     if (a.topk_ids)                                                                                                   \
-      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, true, WIDTH>), grid, block, 0, stream, logits,    \
+      hipLaunchKernelGGL((RELAX_AMD_SPLIT_KERNEL(WIDTH, NVF, PARTIAL, true)), grid, block, 0, stream, logits,        \
                          row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
                          grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps, max_polls,          \
                          tag_offset);                                                                                 \
     else                                                                                                              \
-      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, false, WIDTH>), grid, block, 0, stream, logits,   \
+      hipLaunchKernelGGL((RELAX_AMD_SPLIT_KERNEL(WIDTH, NVF, PARTIAL, false)), grid, block, 0, stream, logits,       \
                          row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
                          grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps, max_polls,          \
                          tag_offset);                                                                                 \
@@ -710,6 +728,7 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
 }
 #undef RELAX_AMD_SPLIT
 #undef RELAX_AMD_SPLIT_ROW
+#undef RELAX_AMD_SPLIT_KERNEL
 
 #define RELAX_AMD_SPLIT_WIDE(NF, PARTIAL)                                                                             \
   if (full == NF && partial == PARTIAL) {                                                                             \
