@@ -3,8 +3,8 @@
 // logit read once and each gradient written once), in the launch shape this memory system streams fastest: many small
 // workgroups that touch their memory once and retire, dispatched in address order (a mixed read / write stream of
 // this shape moves 6.1 - 6.6 TB/s on the box where 256 persistent row-sized streams move 5.6; this kernel on the
-// 65536 x 151936 bf16 step: 5.81 - 5.85 ms where the persistent kernel takes 6.44 - 6.52, 6.0 ms with 256-thread and
-// 6.3 ms with 64-thread workgroups).
+// 65536 x 151936 bf16 step: 5.64 - 5.74 ms compiled for three waves per SIMD, 5.74 - 5.89 for four, where the
+// persistent kernel takes 6.44 - 6.58; 6.0 ms with 256-thread and 6.3 ms with 64-thread workgroups).
 //
 // A row is scanned by 1024 "virtual threads" exactly as scan_row() lays it out for a 1024-thread workgroup (virtual
 // thread t takes the 16-byte vectors t, t + 1024, ...; four at a time while it has four to go, then single ones).  A
