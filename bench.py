@@ -257,7 +257,8 @@ def kl_step_kernel_name(vocab: int) -> str:
     shape = (nvec // 1024, nvec % 1024 != 0)
     if vocab % 8 == 0 and shape in ((20, False), (19, True), (18, True), (15, True), (16, False), (12, True)) \
             and KERNEL_CHOICE != "two_walk":
-        return f"reverse_kl_resident_kernel<bf16_t, {shape[0]}, {str(shape[1]).lower()}>"
+        family = "resident" if KERNEL_CHOICE == "resident" else "split"
+        return f"reverse_kl_{family}_kernel<bf16_t, {shape[0]}, {str(shape[1]).lower()}>"
     return f"reverse_kl_step_kernel<bf16_t, true, {1024 if nvec >= 2048 else 256}>"
 
 

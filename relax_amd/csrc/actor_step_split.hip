@@ -14,15 +14,8 @@
 // wave order as scan_block_merge() does, and turns its registers into the gradient.  Log-probs, entropy and gradients
 // are therefore bit-identical to the forward-only kernel's and the other fused kernels'.
 //
-// Exchange: a ring of slots in device memory, one per (row mod kRing), of 16 x 3 eight-byte words, each a float and a
-// 32-bit tag, written and read with relaxed device-scope atomics.  The tag names the launch and the lap of the ring: it
-// is read from a device word that a one-workgroup kernel in front of every launch advances (so a captured launch gets
-// fresh tags on every replay), and a reader tells a stale word from the one it waits for without any fence.  The eight
-// workgroups of a row have consecutive indices; a workgroup only waits for those, which are resident or next in
-// dispatch order whatever else the chip runs, so every wait ends.  It is bounded all the same: a workgroup that gives
-// up writes NaN log-probs instead of hanging, and counts itself in a device word.  The ring is one array per process
-// and GPU: launches of this kernel that overlap on one GPU (two streams of one process) can overwrite each other's
-// slots or tags, which ends as such a give-up, never as a wrong number taken for right.
+// Exchange: the tagged ring of row_exchange.h, a slot of 16 x 3 words per row; a workgroup that gives up its wait
+// writes NaN log-probs instead of hanging.
 //
 // Replaces, like the other fused kernels, _VocabParallelLogProbEntropy.forward + .backward
 // (relax/utils/training/ppo_utils.py:481-629) and the per-token part of policy_loss_function
@@ -31,28 +24,24 @@
 // As in actor_step_resident.hip the row sits at the edge of the register file:
 // hipcc-flags: -mllvm -amdgpu-use-amdgpu-trackers=1
 #include <atomic>
-#include <mutex>
 
 #include "actor_step_resident.h"
 #include "device_utils.h"
 #include "loss_math.h"
 #include "opd_topk_math.h"
+#include "row_exchange.h"
 #include "row_scan.h"
 
 namespace relax_amd {
 
-constexpr unsigned kRing = 4096;          // rows whose slots exist at a time
 constexpr int kRowWaves = 16;             // waves of the 1024 virtual threads of a row
 constexpr int kSlotWords = kRowWaves * 3;
 constexpr int kSplitThreads = 128;        // virtual threads per workgroup
 constexpr int kSplit = 1024 / kSplitThreads;
-constexpr unsigned kWaitPolls = 1u << 17;  // looks at a neighbour's word before a wait gives up (a few suffice; each takes microseconds)
 constexpr size_t kRingWords = size_t(kRing) * kSlotWords;
 
-// the exchange ring and, behind it, three 32-bit words: the tag counter, the count of waits that gave up, and a flag
-// that the first give-up of a launch raises so that the launch's other waits end at their next look at it (a launch
-// whose exchange is broken then ends within the time of one bounded wait instead of one per workgroup)
-static __device__ __align__(256) unsigned long long split_ring[kRingWords + 32];
+// the exchange ring and its status words
+static __device__ __align__(256) unsigned long long split_ring[kRingWords + kRingTailWords];
 
 // scan_absorb() over the values of kScanUnroll raw vectors (as in actor_step_resident.hip: same arithmetic, same
 // order)
@@ -97,8 +86,7 @@ __device__ __forceinline__ void split_publish(unsigned long long* slot, unsigned
   const int lane = vt & (kWave - 1), vwave = vt / kWave;
   if (lane < 3) {
     const float val = lane == 0 ? m0 : (lane == 1 ? s0 : t0);
-    __hip_atomic_store(slot + vwave * 3 + lane, (static_cast<unsigned long long>(tag) << 32) | __float_as_uint(val),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    exchange_store(slot + vwave * 3 + lane, tag, val);
   }
 }
 
@@ -110,28 +98,9 @@ __device__ __forceinline__ SoftmaxAcc split_collect(const unsigned long long* sl
                                                     unsigned max_polls, unsigned* status, bool& any_gave_up) {
   float word = 0.f;
   bool gave_up = false;
-  if (tid < ROW_WAVES * 3) {
-    unsigned polls = 0;
-    while (true) {
-      const unsigned long long w = __hip_atomic_load(slot + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (unsigned(w >> 32) == tag) {
-        word = __uint_as_float(unsigned(w));
-        break;
-      }
-      ++polls;
-      if (polls > max_polls ||
-          ((polls & 63u) == 0u && __hip_atomic_load(status + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
-        gave_up = true;
-        break;
-      }
-      __builtin_amdgcn_s_sleep(1);
-    }
-  }
+  if (tid < ROW_WAVES * 3) gave_up = !exchange_wait(slot + tid, tag, max_polls, status, word);
   any_gave_up = __any(gave_up);
-  if (any_gave_up && tid == 0) {
-    atomicAdd(status + 1, 1u);
-    __hip_atomic_store(status + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  if (any_gave_up && tid == 0) exchange_report_give_up(status);
   auto of_lane = [&](int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(word), l)); };
   SoftmaxAcc whole{of_lane(0), of_lane(1), of_lane(2)};
 #pragma unroll
@@ -200,7 +169,7 @@ void actor_step_split_kernel(
   for (int j = 0; j < NV; ++j)
     if (has(j)) reg[j] = load_stream(xv + vt + j * ROW_THREADS);
   // this launch's tags: the counter was advanced by `laps` in front of the launch
-  const unsigned tag = reinterpret_cast<const unsigned*>(ring + kRingWords)[0] - laps + 1u + unsigned(row / kRing);
+  const unsigned tag = exchange_tag(reinterpret_cast<const unsigned*>(ring + kRingWords), laps, row);
 
   // the scan, group by group as the vectors arrive, in scan_row()'s order
   SoftmaxAcc st{kNegHuge, 0.f, 0.f};
@@ -413,7 +382,7 @@ __global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(3
   }
 
   const u32x4* xv = reinterpret_cast<const u32x4*>(logits + row * row_stride);
-  const unsigned tag = reinterpret_cast<const unsigned*>(ring + kRingWords)[0] - laps + 1u + unsigned(row / kRing);
+  const unsigned tag = exchange_tag(reinterpret_cast<const unsigned*>(ring + kRingWords), laps, row);
   // The row share arrives group by group (four positions = one scan group): the vectors land in `land`, are absorbed
   // into the softmax state as the fp32 values they are, and leave their upper halves in `reg`; the loads of the
   // following group are requested before a group is absorbed.
@@ -595,50 +564,17 @@ __global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(3
   }
 }
 
-// Advances the tag counter by the laps of the launch that follows; clears the ring when the 32-bit counter would wrap
-// (a tag of a past lap could otherwise come round again).
-__global__ __launch_bounds__(256) void split_ring_advance_kernel(unsigned long long* ring, unsigned laps) {
-  unsigned* counter = reinterpret_cast<unsigned*>(ring + kRingWords);
-  const unsigned now = counter[0];
-  const bool wrap = now > 0xffffffffu - laps - 1u;
-  if (wrap)
-    for (size_t i = threadIdx.x; i < kRingWords; i += 256) ring[i] = 0ull;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    counter[0] = (wrap ? 0u : now) + laps;
-    counter[2] = 0u;  // no wait of the launch that follows has given up yet
-  }
-}
-
 namespace {
-constexpr int kMaxDevices = 64;
-std::mutex ring_mutex;
-unsigned long long* ring_ptr[kMaxDevices] = {};
+ExchangeRingCache ring_cache;
 // relax_amd_set_exchange_wait: the bound of a workgroup's wait and an offset added to the tag it waits for
 std::atomic<unsigned> g_max_polls{kWaitPolls}, g_wait_tag_offset{0u};
 }  // namespace
 
-// the current device's ring (looked up once per device, with that device current)
+unsigned exchange_max_polls() { return g_max_polls.load(std::memory_order_relaxed); }
+unsigned exchange_wait_tag_offset() { return g_wait_tag_offset.load(std::memory_order_relaxed); }
+
 static int split_ring_of_device(unsigned long long** ring) {
-  int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
-    set_error("actor_step_split: no usable current device (%s)",
-              e == hipSuccess ? "index out of range" : hipGetErrorString(e));
-    return RELAX_AMD_EINVAL;
-  }
-  std::lock_guard<std::mutex> lock(ring_mutex);
-  if (!ring_ptr[dev]) {
-    void* p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(split_ring));
-    if (e != hipSuccess || !p) {
-      set_error("actor_step_split: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
-      return RELAX_AMD_ELAUNCH;
-    }
-    ring_ptr[dev] = static_cast<unsigned long long*>(p);
-  }
-  *ring = ring_ptr[dev];
-  return RELAX_AMD_OK;
+  return exchange_ring_of_device(ring_cache, reinterpret_cast<const void*>(&split_ring), "actor_step_split", ring);
 }
 
 // Waves per SIMD the kernel is compiled for.  Long 16-bit rows without the top-K term run fastest with three (six
@@ -701,9 +637,9 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
   unsigned long long* ring = nullptr;
   if (int rc = split_ring_of_device(&ring)) return rc;
   const unsigned laps = unsigned((n_rows + kRing - 1) / kRing);
-  const unsigned max_polls = g_max_polls.load(std::memory_order_relaxed);
-  const unsigned tag_offset = g_wait_tag_offset.load(std::memory_order_relaxed);
-  hipLaunchKernelGGL(split_ring_advance_kernel, dim3(1), dim3(256), 0, stream, ring, laps);
+  const unsigned max_polls = exchange_max_polls();
+  const unsigned tag_offset = exchange_wait_tag_offset();
+  hipLaunchKernelGGL(exchange_ring_advance_kernel<kRingWords>, dim3(1), dim3(256), 0, stream, ring, laps);
   const dim3 grid(static_cast<unsigned>(n_rows * (width / kSplitThreads))), block(kSplitThreads);
   if constexpr (sizeof(T) == 2) {
     RELAX_AMD_SPLIT_ROW(512, 7, true)
@@ -755,9 +691,9 @@ int launch_actor_step_split_wide(const float* logits, int64_t row_stride, int64_
   unsigned long long* ring = nullptr;
   if (int rc = split_ring_of_device(&ring)) return rc;
   const unsigned laps = unsigned((n_rows + kRing - 1) / kRing);
-  const unsigned max_polls = g_max_polls.load(std::memory_order_relaxed);
-  const unsigned tag_offset = g_wait_tag_offset.load(std::memory_order_relaxed);
-  hipLaunchKernelGGL(split_ring_advance_kernel, dim3(1), dim3(256), 0, stream, ring, laps);
+  const unsigned max_polls = exchange_max_polls();
+  const unsigned tag_offset = exchange_wait_tag_offset();
+  hipLaunchKernelGGL(exchange_ring_advance_kernel<kRingWords>, dim3(1), dim3(256), 0, stream, ring, laps);
   const dim3 grid(static_cast<unsigned>(n_rows * kSplit)), block(kSplitThreads);
   // 151936 / 152064 (37984 / 38016 vectors), 128256 / 129280 (32064 / 32320), 131072 (32768), 163840 (40960),
   // 100352 / 102400 (25088 / 25600)

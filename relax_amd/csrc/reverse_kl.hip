@@ -90,11 +90,10 @@ __global__ __launch_bounds__(kKlThreads) void reverse_kl_fwd_kernel(const T* __r
       KlState other{lds[k][0], lds[k][1], lds[k][2], lds[k][3], lds[k][4]};
       merge_kl(q, other);
     }
-    const float ls = q.ms * kLn2 + logf(q.ss);
-    const float lt = q.mt * kLn2 + logf(q.st);
-    kl[tok] = q.us / q.ss - ls + lt;
-    lse_s[tok] = ls;
-    lse_t[tok] = lt;
+    const KlRow r = kl_finish(q);
+    kl[tok] = r.kl;
+    lse_s[tok] = r.lse_s;
+    lse_t[tok] = r.lse_t;
   }
 }
 
@@ -279,9 +278,8 @@ __global__ __launch_bounds__(THREADS) void reverse_kl_step_kernel(
       KlState other{lds[k][0], lds[k][1], lds[k][2], lds[k][3], lds[k][4]};
       merge_kl(q, other);
     }
-    const float ls = q.ms * kLn2 + logf(q.ss);
-    const float lt = q.mt * kLn2 + logf(q.st);
-    const float v = q.us / q.ss - ls + lt;
+    const KlRow r = kl_finish(q);
+    const float ls = r.lse_s, lt = r.lse_t, v = r.kl;
     kl[tok] = v;
     lse_s[tok] = ls;
     lse_t[tok] = lt;
@@ -349,6 +347,11 @@ static int launch_kl_step(const void* s, const void* t, int64_t n, int64_t vocab
   // relax_amd_set_kernel_choice: TWO_WALK = the two-walk kernel for every row length; RESIDENT = fail where the
   // register-resident one is not built
   const int choice = kernel_choice();
+  if (vec && choice == RELAX_AMD_KERNEL_AUTO) {  // one-shot workgroups that share each row
+    const int rc = launch_reverse_kl_split<T>(static_cast<const T*>(s), static_cast<const T*>(t), stride, vocab, n, g,
+                                              scale, kl, ls, lt, static_cast<T*>(d), st);
+    if (rc != RELAX_AMD_EUNSUPPORTED) return rc;
+  }
   if (vec && choice != RELAX_AMD_KERNEL_TWO_WALK) {
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess ||

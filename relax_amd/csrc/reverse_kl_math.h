@@ -1,4 +1,4 @@
-// Online-softmax state and update rules shared by the reverse-KL kernels (reverse_kl.hip, reverse_kl_resident.hip).
+// Online-softmax state and update rules shared by the reverse-KL kernels (reverse_kl.hip, reverse_kl_resident.hip, reverse_kl_split.hip).
 #pragma once
 
 #include "device_utils.h"
@@ -44,11 +44,25 @@ __device__ __forceinline__ void absorb_pair(const float (&xs)[K], const float (&
 __device__ __forceinline__ void merge_kl(KlState& a, const KlState& b) {
   const float ms = fmaxf(a.ms, b.ms), mt = fmaxf(a.mt, b.mt);
   const float fa = fast_exp2(a.ms - ms), fb = fast_exp2(b.ms - ms);
-  a.ss = a.ss * fa + b.ss * fb;
-  a.us = a.us * fa + b.us * fb;
-  a.st = a.st * fast_exp2(a.mt - mt) + b.st * fast_exp2(b.mt - mt);
+  // the fused multiply-adds spelled out: left as a * fa + b * fb the compiler picks which product to fuse by
+  // context, and the kernels that share this rule would differ in the last bit
+  a.ss = fmaf(a.ss, fa, b.ss * fb);
+  a.us = fmaf(a.us, fa, b.us * fb);
+  a.st = fmaf(a.st, fast_exp2(a.mt - mt), b.st * fast_exp2(b.mt - mt));
   a.ms = ms;
   a.mt = mt;
+}
+
+// the row's results from its merged state: KL(student || teacher) = sum p_s (x_s - x_t) - lse_s + lse_t
+struct KlRow {
+  float kl, lse_s, lse_t;
+};
+__device__ __forceinline__ KlRow kl_finish(const KlState& q) {
+  KlRow r;
+  r.lse_s = fmaf(q.ms, kLn2, logf(q.ss));
+  r.lse_t = fmaf(q.mt, kLn2, logf(q.st));
+  r.kl = q.us / q.ss - r.lse_s + r.lse_t;
+  return r;
 }
 
 }  // namespace relax_amd

@@ -275,9 +275,8 @@ __global__ __launch_bounds__(kKlResThreads, 4) void reverse_kl_resident_kernel(
         KlState other{lds[k][0], lds[k][1], lds[k][2], lds[k][3], lds[k][4]};
         merge_kl(q, other);
       }
-      const float ls = q.ms * kLn2 + logf(q.ss);
-      const float lt = q.mt * kLn2 + logf(q.st);
-      const float v = q.us / q.ss - ls + lt;
+      const KlRow r = kl_finish(q);
+      const float ls = r.lse_s, lt = r.lse_t, v = r.kl;
       kl[row] = v;
       lse_s[row] = ls;
       lse_t[row] = lt;

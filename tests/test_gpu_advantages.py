@@ -233,8 +233,8 @@ def test_fused_opd_loss_matches_oracle_and_two_launch_path(n, v, dtype, tol):
                                        (100352, torch.bfloat16, 1030), (102400, torch.bfloat16, 40),
                                        (163840, torch.bfloat16, 300), (8 * (19 * 1024 + 3), torch.float16, 530)])
 def test_register_resident_reverse_kl_step_equals_two_walk_kernel_bitwise(v, dtype, n):
-    """The two kernels behind relax_amd_reverse_kl_step_fused, switched with relax_amd_set_kernel_choice, for every
-    row shape the register-resident one is built for (partial and full last vector positions), with more rows than
+    """The three kernels behind relax_amd_reverse_kl_step_fused, switched with relax_amd_set_kernel_choice, for every
+    row shape the register-resident ones are built for (partial and full last vector positions), with more rows than
     workgroups (several rows per persistent workgroup, uneven counts), fewer rows than workgroups, and rows without
     gradient (zero rows, KL still reported) scattered and in runs.  KL, both log-sum-exps and the gradient must be
     bit-identical, and a few rows are checked against the oracle."""
@@ -251,14 +251,18 @@ def test_register_resident_reverse_kl_step_equals_two_walk_kernel_bitwise(v, dty
     g[n // 2:n // 2 + 9] = 0.0
     g[-1] = 0.0
     results = {}
-    for kind in ("cached", "resident"):
-        ops.set_kernel_choice("two_walk" if kind == "cached" else "resident")
-        kl, ls, lt, d = ops.reverse_kl_step_fused(s, t, g, 0.75)
-        torch.cuda.synchronize()
-        results[kind] = dict(kl=kl, lse_s=ls, lse_t=lt, d=d.view(torch.int16))
-    for key, want in results["cached"].items():
-        got = results["resident"][key]
-        assert torch.equal(got, want), (key, (got.float() - want.float()).abs().max())
+    try:
+        for kind in ("cached", "resident", "auto", "auto_again"):
+            ops.set_kernel_choice({"cached": "two_walk", "resident": "resident"}.get(kind, "auto"))
+            kl, ls, lt, d = ops.reverse_kl_step_fused(s, t, g, 0.75)
+            torch.cuda.synchronize()
+            results[kind] = dict(kl=kl, lse_s=ls, lse_t=lt, d=d.view(torch.int16))
+    finally:
+        ops.set_kernel_choice("auto")
+    for kind in ("resident", "auto", "auto_again"):  # auto: one-shot workgroups, eight to a row
+        for key, want in results["cached"].items():
+            got = results[kind][key]
+            assert torch.equal(got, want), (kind, key, (got.float() - want.float()).abs().max())
     d = results["resident"]["d"].view(dtype)
     live = g != 0
     live[2] = False  # identical rows: every gradient entry is p_s * 0
