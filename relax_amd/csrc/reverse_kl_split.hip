@@ -6,9 +6,10 @@
 // A row is scanned by 1024 "virtual threads" exactly as reverse_kl_step_kernel lays it out for a 1024-thread workgroup
 // (virtual thread t takes the 16-byte vectors t, t + 1024, ... of both rows; two at a time while it has two to go,
 // then single ones).  A workgroup here is 128 of those virtual threads (virtual waves 2q and 2q + 1 of the row) and
-// holds its share of BOTH rows in registers (2 x 19 vectors per thread at V = 151936: the kernel is compiled for two
-// waves per SIMD, 256 registers a lane), so the student and the teacher row are each read once; the persistent kernel
-// keeps the student row and reads the teacher row 1.5 times.  Each wave reduces its share to the five-word state
+// holds its share of BOTH rows on chip (2 x 19 vectors per thread at V = 151936: the student's and seven of the
+// teacher's in registers, twelve of the teacher's in LDS, where global -> LDS loads put them without a register in
+// between; six workgroups per CU), so the student and the teacher row are each read once; the persistent kernel keeps
+// the student row and reads the teacher row 1.5 times.  Each wave reduces its share to the five-word state
 // of the two online softmaxes by the same butterfly, publishes it, the workgroup's first wave fetches the row's
 // sixteen states, merges them in wave order as thread 0 of the 1024-thread workgroup does, and the registers turn
 // into the gradient d = p_s * g * ((x_s - x_t) + lse_t - lse_s - KL).
@@ -96,8 +97,13 @@ __device__ __forceinline__ void kl_split_absorb_raw_pairs(u32x4* s_raw, u32x4* t
   }
 }
 
-template <typename T, int NVF, bool PARTIAL>
-__global__ __launch_bounds__(kKlSplitThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void reverse_kl_split_kernel(
+// LDS_VECS: the first LDS_VECS teacher vectors of a thread's share go from global memory straight to LDS (16 bytes
+// per lane and vector, no register in between) and are read from there by the scan and again by the gradient pass;
+// the others and the student's stay in registers.  WAVES_MIN / WAVES_MAX: waves per SIMD the register allocation aims
+// for.
+template <typename T, int NVF, bool PARTIAL, int LDS_VECS, int WAVES_MIN, int WAVES_MAX>
+__global__ __launch_bounds__(kKlSplitThreads) __attribute__((amdgpu_waves_per_eu(WAVES_MIN, WAVES_MAX)))
+void reverse_kl_split_kernel(
     const T* __restrict__ student, const T* __restrict__ teacher, int64_t stride, int64_t vocab, int64_t n_rows,
     const float* __restrict__ g, float grad_scale, float* __restrict__ kl, float* __restrict__ lse_s,
     float* __restrict__ lse_t, T* __restrict__ dstudent, unsigned long long* __restrict__ ring, unsigned laps,
@@ -106,7 +112,10 @@ __global__ __launch_bounds__(kKlSplitThreads) __attribute__((amdgpu_waves_per_eu
   constexpr int VN = Row<T>::kPerVec;
   constexpr int NV = NVF + (PARTIAL ? 1 : 0);
   constexpr int kGroups = (NV + kU - 1) / kU;
+  constexpr int NT = NV - LDS_VECS;  // teacher vectors in registers
+  static_assert(LDS_VECS <= NVF && NT >= 1, "only full vector positions go to LDS");
   __shared__ float bc[2];
+  __shared__ u32x4 tlds[LDS_VECS > 0 ? LDS_VECS : 1][kKlSplitThreads];
   const int tid = threadIdx.x;
   const bool wave0 = __builtin_amdgcn_readfirstlane(tid) < kWave;
   const unsigned part = blockIdx.x % kKlSplit;
@@ -117,13 +126,21 @@ __global__ __launch_bounds__(kKlSplitThreads) __attribute__((amdgpu_waves_per_eu
 
   const u32x4* sv = reinterpret_cast<const u32x4*>(student + row * stride);
   const u32x4* tv = reinterpret_cast<const u32x4*>(teacher + row * stride);
-  u32x4 sreg[NV], treg[NV];
+  u32x4 sreg[NV], treg[NT];
+  {
+    const int wave_base = __builtin_amdgcn_readfirstlane(tid / kWave) * kWave;
 #pragma unroll
-  for (int j = 0; j < NV; ++j)
-    if (has(j)) {
-      sreg[j] = load_stream(sv + vt + j * ROW_THREADS);
-      treg[j] = load_stream(tv + vt + j * ROW_THREADS);
+    for (int j = 0; j < NV; ++j) {
+      if (has(j)) sreg[j] = load_stream(sv + vt + j * ROW_THREADS);
+      if (j < LDS_VECS)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(tv + vt + j * ROW_THREADS),
+                                         (__attribute__((address_space(3))) void*)(&tlds[j][wave_base]), 16, 0, 0);
+      else if (has(j))
+        treg[j - LDS_VECS] = load_stream(tv + vt + j * ROW_THREADS);
     }
+  }
+  // teacher vector j of this thread
+  auto teacher_vec = [&](int j) -> u32x4 { return j < LDS_VECS ? tlds[j < LDS_VECS ? j : 0][tid] : treg[j < LDS_VECS ? 0 : j - LDS_VECS]; };
   unsigned* status = reinterpret_cast<unsigned*>(ring + kKlRingWords);
   const unsigned tag = exchange_tag(status, laps, row);
   const float gt = g[row] * grad_scale;
@@ -135,7 +152,8 @@ __global__ __launch_bounds__(kKlSplitThreads) __attribute__((amdgpu_waves_per_eu
   for (int gi = 0; gi < kGroups; ++gi) {
     const int j0 = kU * gi, j1 = kU * gi + 1;
     if (grouped && j1 < NV && has(j1)) {
-      kl_split_absorb_raw_pairs<T>(&sreg[j0 < NV - 1 ? j0 : 0], &treg[j0 < NV - 1 ? j0 : 0], q);
+      u32x4 tpair[kU] = {teacher_vec(j0), teacher_vec(j1 < NV ? j1 : 0)};
+      kl_split_absorb_raw_pairs<T>(&sreg[j0 < NV - 1 ? j0 : 0], tpair, q);
     } else {
       grouped = false;
 #pragma unroll
@@ -143,7 +161,7 @@ __global__ __launch_bounds__(kKlSplitThreads) __attribute__((amdgpu_waves_per_eu
         if (j0 + u < NV && has(j0 + u)) {
           float a[VN], b[VN];
           Row<T>::unpack(sreg[j0 + u < NV ? j0 + u : NV - 1], a);
-          Row<T>::unpack(treg[j0 + u < NV ? j0 + u : NV - 1], b);
+          Row<T>::unpack(teacher_vec(j0 + u < NV ? j0 + u : NV - 1), b);
           absorb_pair(a, b, q);
         }
     }
@@ -215,10 +233,11 @@ __global__ __launch_bounds__(kKlSplitThreads) __attribute__((amdgpu_waves_per_eu
     int lane_id = vt;
     asm volatile("" : "+v"(lane_id));
     kl_split_launder(sreg[j]);
-    kl_split_launder(treg[j]);
+    u32x4 tvec = teacher_vec(j);
+    kl_split_launder(tvec);
     // one 32-bit word of the two vectors at a time
     const uint32_t sw[4] = {sreg[j].x, sreg[j].y, sreg[j].z, sreg[j].w};
-    const uint32_t tw[4] = {treg[j].x, treg[j].y, treg[j].z, treg[j].w};
+    const uint32_t tw[4] = {tvec.x, tvec.y, tvec.z, tvec.w};
     uint32_t ow[4];
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
@@ -237,6 +256,23 @@ __global__ __launch_bounds__(kKlSplitThreads) __attribute__((amdgpu_waves_per_eu
 
 namespace {
 ExchangeRingCache kl_ring_cache;
+}
+
+// Long rows (12 and more vector positions per thread): three waves per SIMD, i.e. six workgroups per CU, each with
+// twelve teacher vectors per thread (24 KB) in LDS; with both rows in registers only two waves per SIMD fit, which is
+// 9 % slower on 16384 x 151936 rows (2.71 - 2.73 against 2.47 ms).  Shorter rows fit the registers of four and more
+// waves per SIMD as they are.
+template <int NVF>
+constexpr int kl_split_lds_vecs() {
+  return NVF >= 12 ? 12 : 0;
+}
+template <int NVF>
+constexpr int kl_split_waves_min() {
+  return NVF >= 12 ? 3 : 4;
+}
+template <int NVF>
+constexpr int kl_split_waves_max() {
+  return NVF >= 12 ? 3 : 8;
 }
 
 template <typename T>
@@ -264,9 +300,13 @@ int launch_reverse_kl_split(const T* student, const T* teacher, int64_t stride, 
     const int64_t nvec = vocab / VN;
     const int full = int(nvec / kKlRowThreads);
     const bool partial = nvec % kKlRowThreads != 0;
-    // the row shapes launch_reverse_kl_resident is built for
+    // the row shapes launch_reverse_kl_resident is built for, and rows of 6145 .. 8192 vectors (50304, 64000 / 65536
+    // entries: 1.91 / 2.33 / 2.08 ms on 32768 rows where the two-walk kernel takes 2.11 / 2.79 / 2.74).  Rows of
+    // 32000 entries, four vectors per thread, are left to the two-walk kernel: here the exchange outweighs the second
+    // read (2.77 against 2.52 ms on 65536 rows).
     if (!((full == 20 && !partial) || (full == 19 && partial) || (full == 18 && partial) || (full == 15 && partial) ||
-          (full == 16 && !partial) || (full == 12 && partial)))
+          (full == 16 && !partial) || (full == 12 && partial) || (full == 8 && !partial) || (full == 7 && partial) ||
+          (full == 6 && partial)))
       return RELAX_AMD_EUNSUPPORTED;
     unsigned long long* ring = nullptr;
     if (int rc = exchange_ring_of_device(kl_ring_cache, reinterpret_cast<const void*>(&kl_split_ring),
@@ -279,8 +319,10 @@ int launch_reverse_kl_split(const T* student, const T* teacher, int64_t stride, 
     const dim3 grid(static_cast<unsigned>(n_rows * kKlSplit)), block(kKlSplitThreads);
 #define RELAX_AMD_KL_SPLIT(NVF, PARTIAL)                                                                              \
   if (full == NVF && partial == PARTIAL) {                                                                            \
-    hipLaunchKernelGGL((reverse_kl_split_kernel<T, NVF, PARTIAL>), grid, block, 0, stream, student, teacher, stride, \
-                       vocab, n_rows, g, grad_scale, kl, lse_s, lse_t, dstudent, ring, laps, max_polls, tag_offset); \
+    hipLaunchKernelGGL((reverse_kl_split_kernel<T, NVF, PARTIAL, kl_split_lds_vecs<NVF>(), kl_split_waves_min<NVF>(), \
+                                                kl_split_waves_max<NVF>()>),                                          \
+                       grid, block, 0, stream, student, teacher, stride, vocab, n_rows, g, grad_scale, kl, lse_s,    \
+                       lse_t, dstudent, ring, laps, max_polls, tag_offset);                                           \
     return check_launch("reverse_kl_split");                                                                          \
   }
     RELAX_AMD_KL_SPLIT(20, false)
@@ -289,6 +331,9 @@ int launch_reverse_kl_split(const T* student, const T* teacher, int64_t stride, 
     RELAX_AMD_KL_SPLIT(15, true)
     RELAX_AMD_KL_SPLIT(16, false)
     RELAX_AMD_KL_SPLIT(12, true)
+    RELAX_AMD_KL_SPLIT(8, false)
+    RELAX_AMD_KL_SPLIT(7, true)
+    RELAX_AMD_KL_SPLIT(6, true)
 #undef RELAX_AMD_KL_SPLIT
     return RELAX_AMD_EUNSUPPORTED;
   }

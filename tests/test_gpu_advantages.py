@@ -277,6 +277,79 @@ def test_register_resident_reverse_kl_step_equals_two_walk_kernel_bitwise(v, dty
     torch.testing.assert_close(d[rows].float().cpu(), sc.grad.float(), atol=2e-3, rtol=ulp)
 
 
+@pytest.mark.parametrize("v,dtype,n", [(50304, torch.bfloat16, 700), (64000, torch.bfloat16, 300),
+                                       (65536, torch.float16, 9), (8 * 7169, torch.float16, 515)])
+def test_one_shot_reverse_kl_step_on_short_rows_equals_two_walk_kernel_bitwise(v, dtype, n):
+    """Rows of 6145 .. 8192 sixteen-byte vectors, which only the two-walk kernel and the one-shot workgroups (the
+    default) are built for: KL, both log-sum-exps and the gradient bit-identical, twice in a row (the second launch finds
+    the first one's words in the exchange ring)."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("one-shot reverse KL vs two-walk, short rows", v, dtype, n)
+    gen = torch.Generator(device=dev).manual_seed(v + n)
+    s = (torch.randn((n, v), device=dev, generator=gen) * 3).to(dtype)
+    t = (s.float() + torch.randn((n, v), device=dev, generator=gen)).to(dtype)
+    s[0, v - 1] = 30.0
+    g = (torch.rand(n, device=dev, generator=gen) > 0.2).float() * torch.rand(n, device=dev, generator=gen)
+    g[-1] = 0.0
+    results = {}
+    try:
+        for kind in ("two_walk", "auto", "auto_again"):
+            ops.set_kernel_choice("two_walk" if kind == "two_walk" else "auto")
+            kl, ls, lt, d = ops.reverse_kl_step_fused(s, t, g, 1.25)
+            torch.cuda.synchronize()
+            results[kind] = dict(kl=kl, lse_s=ls, lse_t=lt, d=d.view(torch.int16))
+    finally:
+        ops.set_kernel_choice("auto")
+    for kind in ("auto", "auto_again"):
+        for key, want in results["two_walk"].items():
+            assert torch.equal(results[kind][key], want), (kind, key)
+    assert (results["auto"]["d"][g == 0] == 0).all() and torch.isfinite(results["auto"]["kl"]).all()
+    rows = [0, n - 2]
+    sc = s[rows].cpu().requires_grad_()
+    want = D.full_vocab_reverse_kl(sc, t[rows].cpu())
+    (want * (1.25 * g[rows].cpu())).sum().backward()
+    torch.testing.assert_close(results["auto"]["kl"][rows].cpu(), want.detach(), atol=2e-3, rtol=0)
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    torch.testing.assert_close(results["auto"]["d"].view(dtype)[rows].float().cpu(), sc.grad.float(), atol=2e-3, rtol=ulp)
+
+
+def test_one_shot_reverse_kl_step_gives_up_a_wait_that_cannot_succeed_and_recovers():
+    """Failure handling of the exchange between the workgroups of a row, forced from the host
+    (relax_amd_set_exchange_wait): with the awaited tag offset by one no wait can succeed; every workgroup gives up
+    after a few looks, the row's KL and log-sum-exps come back NaN, every kernel exits normally, and the next launch
+    with the defaults restored is exact again."""
+    from relax_amd import ops
+    from relax_amd._lib import check, lib
+
+    dev = require_gpu()
+    announce("one-shot reverse KL: give-up path")
+    v, n = 151936, 120
+    gen = torch.Generator(device=dev).manual_seed(3)
+    s = (torch.randn((n, v), device=dev, generator=gen) * 2).bfloat16()
+    t = (s.float() + torch.randn((n, v), device=dev, generator=gen)).bfloat16()
+    g = torch.rand(n, device=dev, generator=gen)
+
+    def run():
+        out = ops.reverse_kl_step_fused(s, t, g, 1.0)
+        torch.cuda.synchronize()
+        return out
+
+    ops.set_kernel_choice("two_walk")
+    want = run()
+    ops.set_kernel_choice("auto")
+    check(lib.relax_amd_set_exchange_wait(4, 1))
+    try:
+        kl, ls, lt, d = run()
+    finally:
+        check(lib.relax_amd_set_exchange_wait(0, 0))
+    assert torch.isnan(kl).all() and torch.isnan(ls).all() and torch.isnan(lt).all()
+    got = run()
+    for a, b in zip(got, want):
+        assert torch.equal(a.view(torch.int16) if a.dtype == torch.bfloat16 else a, b.view(torch.int16) if b.dtype == torch.bfloat16 else b)
+
+
 def test_opd_token_mean_literal(literals):
     from relax_amd.opd_utils import compute_opd_kl, reduce_opd_loss
 
