@@ -77,19 +77,19 @@ enum { RELAX_AMD_KERNEL_AUTO = 0, RELAX_AMD_KERNEL_TWO_WALK = 1, RELAX_AMD_KERNE
 /*
  * relax_amd_actor_step_fused, relax_amd_logprob_entropy_bwd and relax_amd_reverse_kl_step_fused each hold a
  * persistent register-resident kernel for the row lengths it is built for and a two-walk (row-per-workgroup) kernel
- * for every row length; the first two also hold a kernel of one-shot workgroups in address order (the actor step:
- * eight workgroups share a row and exchange their partial softmax sums through a ring in device memory; the
- * backward: one workgroup per 4 KB of a row).  All give the same bits.  AUTO (the default) takes the one-shot form
+ * for every row length; each also holds a kernel of one-shot workgroups in address order (the actor step and the
+ * reverse-KL step: eight workgroups share a row and exchange their partial softmax sums through a ring in device
+ * memory; the backward: one workgroup per 4 KB of a row).  All give the same bits.  AUTO (the default) takes the one-shot form
  * where it exists, else the resident one, else the two-walk kernel.  TWO_WALK keeps every row on the two-walk
  * kernel; RESIDENT takes the persistent kernel and makes those entry points fail with RELAX_AMD_EUNSUPPORTED where
  * none is built, so that a comparison of kernels cannot pass on one kernel compared with itself.
  * Process-wide, read atomically at each launch; returns the previous choice, or RELAX_AMD_EINVAL.  No counterpart
  * in the reference: it exists for tests and measurements.
  *
- * The actor step's one-shot kernel keeps its exchange ring (1.5 MB) in a static array of the library, one copy per
- * GPU and process.  Launches of relax_amd_actor_step_fused that overlap on one GPU (two streams of one process) must
- * not both take that kernel: they could overwrite each other's slots, which the kernel notices (bounded waits) and
- * reports as NaN log-probs rather than wrong numbers.  Launches in stream order, captured graphs and their replays
+ * The one-shot kernels of the actor step and of the reverse-KL step each keep their exchange ring (1.5 MB / 2.5 MB)
+ * in a static array of the library, one copy per GPU and process.  Launches of the same entry point that overlap on
+ * one GPU (two streams of one process) must not both take that kernel: they could overwrite each other's slots, which
+ * the kernel notices (bounded waits) and reports as NaN log-probs (NaN KL) rather than wrong numbers.  Launches in stream order, captured graphs and their replays
  * are fine (the tags that tell one launch's partial sums from another's come from a counter in device memory that a
  * small kernel in front of each launch advances); the first call on a GPU looks the ring's address up
  * (hipGetSymbolAddress), so make one call outside a capture first.
@@ -97,11 +97,12 @@ enum { RELAX_AMD_KERNEL_AUTO = 0, RELAX_AMD_KERNEL_TWO_WALK = 1, RELAX_AMD_KERNE
 int relax_amd_set_kernel_choice(int choice);
 
 /*
- * For tests of the one-shot actor step's failure handling: max_polls bounds how often a workgroup looks for its
+ * For tests of the failure handling of the one-shot actor and reverse-KL steps: max_polls bounds how often a workgroup looks for its
  * neighbours' partial sums before it gives up (0 = the default), wait_tag_offset is added to the tag it looks
  * for (0 = none; with 1 no wait can succeed; the default bound is 2^17 looks, and the first give-up of a launch ends
  * the launch's other waits at their next check of a flag).  A launch made with (a few, 1) therefore exercises the give-up path on
- * every row without any workgroup hanging: log-probs and log-sum-exps of the scored tokens come back NaN.
+ * every row without any workgroup hanging: log-probs and log-sum-exps of the scored tokens (the reverse-KL step: KL
+ * and both log-sum-exps of every token) come back NaN.
  * Process-wide, read at each launch.  No counterpart in the reference.
  */
 int relax_amd_set_exchange_wait(int max_polls, int wait_tag_offset);
@@ -341,10 +342,13 @@ int relax_amd_reverse_kl_bwd(const void* student, const void* teacher, int dtype
  * known before the forward runs: the masked token mean of reduce_opd_loss (relax/utils/opd/opd_utils.py:1355-1365),
  * g[t] = mask[t] / clamp_min(sum mask, 1).  Same outputs as relax_amd_reverse_kl_fwd followed by
  * relax_amd_reverse_kl_bwd (dstudent row stride = row_stride); each workgroup re-reads its two rows out of cache, so
- * HBM moves 3*V*s bytes per token instead of 5*V*s.  Two kernels sit behind it, with bit-identical results: 16-bit
- * rows of the built vocabulary shapes (12 / 15 / 18 / 19 full 16-byte vectors per thread of a 1024-thread workgroup
- * plus a partial one, or 16 / 20 exactly) keep the student row in registers and stream the teacher row past it twice; other
- * rows, and every row after relax_amd_set_kernel_choice(RELAX_AMD_KERNEL_TWO_WALK), walk both rows twice.
+ * HBM moves 3*V*s bytes per token instead of 5*V*s.  Three kernels sit behind it, with bit-identical results: 16-bit
+ * rows of the built vocabulary shapes (12 / 15 / 18 / 19 full 16-byte vectors per thread of 1024 threads plus a
+ * partial one, or 16 / 20 exactly; the default kernel also 6 / 7 plus a partial one and 8 exactly) are shared by eight
+ * one-shot workgroups that keep both rows' shares on chip, so each row is read once (the default), or, after
+ * relax_amd_set_kernel_choice(RELAX_AMD_KERNEL_RESIDENT), kept as the student row in the registers of one persistent
+ * workgroup that streams the teacher row past it twice; other rows, and every row after
+ * relax_amd_set_kernel_choice(RELAX_AMD_KERNEL_TWO_WALK), walk both rows twice.
  */
 int relax_amd_reverse_kl_step_fused(const void* student, const void* teacher, int dtype, int64_t n_tokens,
                                     int64_t vocab, int64_t row_stride, const float* g, float grad_scale, float* kl,
