@@ -45,8 +45,10 @@ static __device__ __align__(256) unsigned long long split_ring[kRingWords + kRin
 
 // scan_absorb() over the values of kScanUnroll raw vectors (as in actor_step_resident.hip: same arithmetic, same
 // order)
-template <typename T>
-__device__ __forceinline__ void split_absorb_raw_group(const u32x4* raw, float c, SoftmaxAcc& st) {
+// KEEP: whether the second walk may use the values the first one unpacked (32 registers for 16-bit rows); without, the
+// raw vectors are marked as changed in between, so that the compiler unpacks them again
+template <typename T, bool KEEP = true>
+__device__ __forceinline__ void split_absorb_raw_group(u32x4* raw, float c, SoftmaxAcc& st) {
   constexpr int VN = Row<T>::kPerVec;
   float vmax = 0.f;
 #pragma unroll
@@ -66,6 +68,7 @@ __device__ __forceinline__ void split_absorb_raw_group(const u32x4* raw, float c
   }
 #pragma unroll
   for (int u = 0; u < kScanUnroll; ++u) {
+    if constexpr (!KEEP) asm volatile("" : "+v"(raw[u].x), "+v"(raw[u].y), "+v"(raw[u].z), "+v"(raw[u].w));
     float v[VN];
     Row<T>::unpack(raw[u], v);  // the compiler keeps the first walk's values: with wave 0's share parked in LDS
                                 // during thread 0's arithmetic there is room for them next to the row
@@ -108,10 +111,28 @@ __device__ __forceinline__ SoftmaxAcc split_collect(const unsigned long long* sl
   return whole;
 }
 
+// this workgroup's LDS_VECS x 128 vectors of the row that live in LDS (only instantiated, and only allocated, for
+// LDS_VECS > 0)
+template <int LDS_VECS>
+__device__ __forceinline__ u32x4* split_lds_rows() {
+  __shared__ u32x4 rows[LDS_VECS * kSplitThreads];
+  return rows;
+}
+
+// where wave 0's share waits during thread 0's serial stretch (only instantiated, and only allocated, for PARK > 0)
+template <int PARK>
+__device__ __forceinline__ u32x4 (*split_parked())[kWave] {
+  __shared__ u32x4 parked[PARK][kWave];
+  return parked;
+}
+
 // ROW_THREADS: the virtual threads that scan a row, i.e. the width scan_threads() gives the forward-only kernel for this
 // row length (1024, or 512 for rows of 2048 .. 7167 vectors); ROW_THREADS / 128 workgroups share a row.
 // WAVES_MIN / WAVES_MAX: the waves per SIMD the register allocation aims for (see split_waves_min()).
-template <typename T, int NVF, bool PARTIAL, bool TOPK, int ROW_THREADS, int WAVES_MIN, int WAVES_MAX>
+// LDS_VECS: rows longer than the register file holds at three waves per SIMD (16-bit vocabularies above 163840 entries)
+// keep the first LDS_VECS vectors of every thread's share in LDS, where global -> LDS loads put them without a
+// register in between; wave 0 then has registers to spare for thread 0's serial stretch and parks nothing.
+template <typename T, int NVF, bool PARTIAL, bool TOPK, int ROW_THREADS, int WAVES_MIN, int WAVES_MAX, int LDS_VECS = 0>
 __global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(WAVES_MIN, WAVES_MAX)))
 void actor_step_split_kernel(
     const T* __restrict__ logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
@@ -129,8 +150,11 @@ void actor_step_split_kernel(
   __shared__ float topk_stage[TOPK ? kTopkStageFloats : 1];
   // vectors of wave 0's share that wait in LDS during thread 0's serial stretch (see there): all of them, or as many
   // as leave room for eight workgroups per CU next to the top-K term's staging area
-  constexpr int kPark = NV < (TOPK ? 15 : 19) ? NV : (TOPK ? 15 : 19);
-  __shared__ u32x4 parked[kPark][kWave];
+  constexpr int kPark = LDS_VECS > 0 ? 0 : (NV < (TOPK ? 15 : 19) ? NV : (TOPK ? 15 : 19));
+  u32x4(*parked)[kWave] = nullptr;
+  if constexpr (kPark > 0) parked = split_parked<kPark>();
+  constexpr int NR = NV - LDS_VECS;  // vectors of the share in registers
+  static_assert(LDS_VECS <= NVF && NR >= kU, "only full vector positions go to LDS");
   const int tid = threadIdx.x;
   const bool wave0 = __builtin_amdgcn_readfirstlane(tid) < kWave;
   const unsigned part = blockIdx.x % kParts;
@@ -164,10 +188,31 @@ void actor_step_split_kernel(
   }
 
   const u32x4* xv = reinterpret_cast<const u32x4*>(logits + row * row_stride);
-  u32x4 reg[NV];
+  u32x4 reg[NR];
+  if constexpr (LDS_VECS > 0) {
+    u32x4* rows = split_lds_rows<LDS_VECS>();
+    const int wave_base = __builtin_amdgcn_readfirstlane(tid / kWave) * kWave;
 #pragma unroll
-  for (int j = 0; j < NV; ++j)
-    if (has(j)) reg[j] = load_stream(xv + vt + j * ROW_THREADS);
+    for (int j = 0; j < NV; ++j) {
+      if (j < LDS_VECS)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xv + vt + j * ROW_THREADS),
+                                         (__attribute__((address_space(3))) void*)(rows + j * kSplitThreads + wave_base),
+                                         16, 0, 0);
+      else if (has(j))
+        reg[j - LDS_VECS] = load_stream(xv + vt + j * ROW_THREADS);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+      if (has(j)) reg[j] = load_stream(xv + vt + j * ROW_THREADS);
+  }
+  // vector j of this thread's share
+  auto vec = [&](int j) -> u32x4 {
+    if constexpr (LDS_VECS > 0) {
+      if (j < LDS_VECS) return split_lds_rows<LDS_VECS>()[(j < LDS_VECS ? j : 0) * kSplitThreads + tid];
+    }
+    return reg[j < LDS_VECS ? 0 : j - LDS_VECS];
+  };
   // this launch's tags: the counter was advanced by `laps` in front of the launch
   const unsigned tag = exchange_tag(reinterpret_cast<const unsigned*>(ring + kRingWords), laps, row);
 
@@ -177,14 +222,21 @@ void actor_step_split_kernel(
 #pragma unroll
   for (int g = 0; g < kGroups; ++g) {
     if (grouped && kU * g + kU - 1 < NV && has(kU * g + kU - 1)) {
-      split_absorb_raw_group<T>(&reg[kU * g < NV - kU ? kU * g : NV - kU], c, st);
+      if constexpr (LDS_VECS > 0) {
+        u32x4 grp[kU];
+#pragma unroll
+        for (int u = 0; u < kU; ++u) grp[u] = vec((kU * g < NV - kU ? kU * g : NV - kU) + u);
+        split_absorb_raw_group<T, false>(grp, c, st);
+      } else {
+        split_absorb_raw_group<T>(&reg[kU * g < NV - kU ? kU * g : NV - kU], c, st);
+      }
     } else {
       grouped = false;
 #pragma unroll
       for (int u = 0; u < kU; ++u)
         if (kU * g + u < NV && has(kU * g + u)) {
           float v[VN];
-          Row<T>::unpack(reg[kU * g + u < NV ? kU * g + u : NV - 1], v);
+          Row<T>::unpack(vec(kU * g + u < NV ? kU * g + u : NV - 1), v);
           scan_absorb(v, c, st);
         }
     }
@@ -288,7 +340,7 @@ void actor_step_split_kernel(
     asm volatile("" : "+v"(lane_id));
     const int idx = lane_id + j * ROW_THREADS;
     float v[VN];
-    Row<T>::unpack(reg[j], v);
+    Row<T>::unpack(vec(j), v);
 #pragma unroll
     for (int k = 0; k < VN; ++k) {
       v[k] = fast_exp2(fmaf(v[k], c, k0)) * fmaf(v[k], a1, a0);
@@ -607,6 +659,17 @@ constexpr int split_waves_max() {
     return check_launch("actor_step_split");                                                                          \
   }
 #define RELAX_AMD_SPLIT(NVF, PARTIAL) RELAX_AMD_SPLIT_ROW(1024, NVF, PARTIAL)
+// rows of more than 20 vectors per thread: twelve of them in LDS (24 KB of the 26 a workgroup can have when six share
+// a CU), three waves per SIMD; the top-K term is left to the two-walk kernel for these rows
+#define RELAX_AMD_SPLIT_LDS(NVF, PARTIAL)                                                                             \
+  if (width == 1024 && full == NVF && partial == PARTIAL) {                                                           \
+    hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, false, 1024, 3, 3, (NVF >= 30 ? 13 : 12)>), grid,  \
+                       block, 0, stream,                                                                              \
+                       logits, row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t,  \
+                       a, grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps, max_polls,         \
+                       tag_offset);                                                                                   \
+    return check_launch("actor_step_split");                                                                          \
+  }
 
 template <typename T>
 int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
@@ -626,8 +689,12 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
     if (sizeof(T) != 2 || !((full == 7 && partial) || (full == 8 && !partial) || (full == 12 && partial)))
       return RELAX_AMD_EUNSUPPORTED;
   } else if constexpr (sizeof(T) == 2) {
-    if (!((full == 20 && !partial) || (full == 19 && partial) || (full == 18 && partial) || (full == 15 && partial) ||
-          (full == 16 && !partial) || (full == 12 && partial) || (full == 8 && !partial) || (full == 7 && partial)))
+    const bool lds_row = (full == 24 && partial) || (full == 30 && partial) || (full == 31 && partial) ||
+                         (full == 32 && !partial);
+    if (lds_row && a.topk_ids) return RELAX_AMD_EUNSUPPORTED;
+    if (!(lds_row || (full == 20 && !partial) || (full == 19 && partial) || (full == 18 && partial) ||
+          (full == 15 && partial) || (full == 16 && !partial) || (full == 12 && partial) || (full == 8 && !partial) ||
+          (full == 7 && partial)))
       return RELAX_AMD_EUNSUPPORTED;
   } else {
     if (!((full == 7 && partial) || (full == 8 && !partial) || (full == 12 && partial) || (full == 15 && partial) ||
@@ -645,6 +712,11 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
     RELAX_AMD_SPLIT_ROW(512, 7, true)
     RELAX_AMD_SPLIT_ROW(512, 8, false)
     RELAX_AMD_SPLIT_ROW(512, 12, true)
+    // 200064 / 201088 / 202048 (25008 / 25136 / 25256 vectors), 250880 (31360), 256000 (32000), 262144 (32768) entries
+    RELAX_AMD_SPLIT_LDS(24, true)
+    RELAX_AMD_SPLIT_LDS(30, true)
+    RELAX_AMD_SPLIT_LDS(31, true)
+    RELAX_AMD_SPLIT_LDS(32, false)
     RELAX_AMD_SPLIT(20, false)
     RELAX_AMD_SPLIT(19, true)
     RELAX_AMD_SPLIT(18, true)
@@ -662,6 +734,7 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
   }
   return RELAX_AMD_EUNSUPPORTED;
 }
+#undef RELAX_AMD_SPLIT_LDS
 #undef RELAX_AMD_SPLIT
 #undef RELAX_AMD_SPLIT_ROW
 #undef RELAX_AMD_SPLIT_KERNEL

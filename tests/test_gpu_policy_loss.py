@@ -1729,6 +1729,8 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
     (100352, torch.bfloat16, 700, "plain"), (32000, torch.float32, 1500, "plain"), (151936, torch.bfloat16, 300, "plain"),
     # 16-bit rows scanned by 512 threads: no persistent kernel exists for them, the one-shot kernel does
     (32000, torch.bfloat16, 1500, "short"), (50304, torch.float16, 1000, "short"),
+    # 16-bit rows of more than 20 vectors per thread: the one-shot kernel keeps twelve of them in LDS
+    (202048, torch.bfloat16, 300, "short"), (262144, torch.float16, 200, "short"),
     # long fp32 rows, kept in the registers as their upper halves: bf16 values widened to fp32 (what a bf16 output
     # layer followed by .float() delivers: one read of the row), fp32 values with low bits (the row is read again), and
     # rows of both kinds next to each other, one of them with a single low bit in its last element
@@ -1819,8 +1821,9 @@ def test_one_shot_step_on_random_layouts_equals_two_walk_kernel_bitwise(seed):
     dev = require_gpu()
     g = torch.Generator().manual_seed(1000 + seed)
     families = [(torch.bfloat16, 8, [18 * 1024 + 560, 12 * 1024 + 256, 20 * 1024, 16 * 1024, 15 * 1024 + 1023,
-                                     7 * 1024 + 832, 8 * 1024, 7 * 512 + 416, 8 * 512, 12 * 512 + 144]),
-                (torch.float16, 8, [18 * 1024 + 1, 19 * 1024 + 5, 12 * 512 + 1]),
+                                     7 * 1024 + 832, 8 * 1024, 7 * 512 + 416, 8 * 512, 12 * 512 + 144,
+                                     24 * 1024 + 680, 31 * 1024 + 256, 32 * 1024]),
+                (torch.float16, 8, [18 * 1024 + 1, 19 * 1024 + 5, 12 * 512 + 1, 30 * 1024 + 640, 24 * 1024 + 1]),
                 (torch.float32, 4, [7 * 1024 + 832, 8 * 1024, 12 * 1024 + 3, 16 * 1024, 37 * 1024 + 96, 24 * 1024 + 512])]
     dtype, per_vec, nvecs = families[seed % 3]
     nvec = nvecs[int(torch.randint(0, len(nvecs), (1,), generator=g))]
@@ -1875,7 +1878,7 @@ def test_one_shot_step_on_random_layouts_equals_two_walk_kernel_bitwise(seed):
 
 
 @pytest.mark.parametrize("v,dtype", [(151936, torch.bfloat16), (32000, torch.float32), (32000, torch.float16),
-                                     (4 * (37 * 1024 + 96), torch.float32)])
+                                     (4 * (37 * 1024 + 96), torch.float32), (256000, torch.bfloat16)])
 def test_log_probs_and_entropy_of_every_kernel_agree_bitwise_at_a_temperature(v, dtype):
     """The forward-only pass, the log-prob + top-K pass and the fused step in each of its kernels give one set of bits
     for log-prob, entropy, log-sum-exp and sum p*x at a temperature other than 1 (where a product of the temperature
@@ -1906,15 +1909,18 @@ def test_log_probs_and_entropy_of_every_kernel_agree_bitwise_at_a_temperature(v,
               entropy_coef=0.01)
     sample_ids = torch.zeros(n, dtype=torch.int32, device=dev)
     per_vec = 4 if dtype == torch.float32 else 8
-    for kind in ("two_walk", "resident", "auto"):
-        if kind == "resident" and v // per_vec < 7168:
-            continue
-        ops.set_kernel_choice(kind)
-        out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, None, sample_ids, n, inv_t, 1.0, **kw)
-        torch.cuda.synchronize()
-        for key, t in (("lp", lp), ("ent", ent), ("lse", lse), ("spx", spx)):
-            assert torch.equal(t, want[key]), (kind, key, (t - want[key]).abs().max())
-    ops.set_kernel_choice("auto")
+    try:
+        for kind in ("two_walk", "resident", "auto"):
+            # no persistent kernel for rows scanned by 512 threads or of more than 20 vectors per thread
+            if kind == "resident" and (v // per_vec < 7168 or (per_vec == 8 and v // per_vec > 20 * 1024)):
+                continue
+            ops.set_kernel_choice(kind)
+            out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, None, sample_ids, n, inv_t, 1.0, **kw)
+            torch.cuda.synchronize()
+            for key, t in (("lp", lp), ("ent", ent), ("lse", lse), ("spx", spx)):
+                assert torch.equal(t, want[key]), (kind, key, (t - want[key]).abs().max())
+    finally:
+        ops.set_kernel_choice("auto")
 
 
 def test_one_shot_step_gives_up_a_wait_that_cannot_succeed_and_recovers():
