@@ -222,7 +222,8 @@ def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
     nvec = vocab // per_vec
     threads = 1024 if nvec >= 7168 else 512 if nvec >= 2048 else 256
     shape = (nvec // width, nvec % width != 0)
-    split_shapes = shapes  # the one-shot kernel is built for the shapes of the persistent one
+    # the one-shot kernel is built for the shapes of the persistent one and, 16-bit, for four shapes of longer rows
+    split_shapes = shapes + (((24, True), (30, True), (31, True), (32, False)) if dtype == "bf16_t" else ())
     if dtype == "bf16_t" and vocab % per_vec == 0 and threads == 512 and KERNEL_CHOICE == "auto" \
             and (nvec // 512, nvec % 512 != 0) in ((7, True), (8, False), (12, True)):
         # and for 16-bit rows of 32000 / 32768 / 50304 entries, scanned by 512 virtual threads
