@@ -42,6 +42,12 @@ constexpr size_t kRingWords = size_t(kRing) * kSlotWords;
 
 // the exchange ring and its status words
 static __device__ __align__(256) unsigned long long split_ring[kRingWords + kRingTailWords];
+// The logits at a token's top-K ids, gathered once per row: each workgroup of a row fetches its share of the K
+// scattered entries and publishes them here (one tagged word per entry, the ring's tags and status words), every
+// workgroup's first wave collects all K.  Gathered by each of the eight workgroups for itself, the K scattered lines
+// crossed the fabric eight times per row (3.4 GB on 65536 x 151936 rows with K = 64, a tenth of the step's traffic).
+constexpr size_t kTopkRingWords = size_t(kRing) * RELAX_AMD_FUSED_TOPK_MAX;
+static __device__ __align__(256) unsigned long long split_topk_ring[kTopkRingWords];
 
 // scan_absorb() over the values of kScanUnroll raw vectors (as in actor_step_resident.hip: same arithmetic, same
 // order)
@@ -140,7 +146,7 @@ void actor_step_split_kernel(
     const int64_t* __restrict__ targets, float c, float inv_t, relax_amd_policy_loss_args a, float grad_scale,
     float* __restrict__ log_prob, float* __restrict__ entropy, float* __restrict__ lse_out,
     float* __restrict__ spx_out, T* __restrict__ dlogits, int64_t d_stride, unsigned long long* __restrict__ ring,
-    unsigned laps, unsigned max_polls, unsigned wait_tag_offset) {
+    unsigned long long* __restrict__ topk_ring, unsigned laps, unsigned max_polls, unsigned wait_tag_offset) {
   constexpr int kU = kScanUnroll, kParts = ROW_THREADS / kSplitThreads;
   constexpr int VN = Row<T>::kPerVec;
   constexpr int NV = NVF + (PARTIAL ? 1 : 0);
@@ -188,6 +194,17 @@ void actor_step_split_kernel(
   }
 
   const u32x4* xv = reinterpret_cast<const u32x4*>(logits + row * row_stride);
+  // this workgroup's share of the row's K gathered logits: entries part * chunk .. + chunk, one per lane of the second
+  // wave; the id is requested ahead of the row, the logit behind it
+  int my_k = -1;
+  int64_t my_id = -1;
+  if constexpr (TOPK) {
+    const int kmax = a.topk_k, chunk = (kmax + kParts - 1) / kParts, t1 = tid - kWave;
+    if (t1 >= 0 && t1 < chunk && int(part) * chunk + t1 < kmax) {
+      my_k = int(part) * chunk + t1;
+      my_id = a.topk_ids[tok * kmax + my_k];
+    }
+  }
   u32x4 reg[NR];
   if constexpr (LDS_VECS > 0) {
     u32x4* rows = split_lds_rows<LDS_VECS>();
@@ -215,6 +232,10 @@ void actor_step_split_kernel(
   };
   // this launch's tags: the counter was advanced by `laps` in front of the launch
   const unsigned tag = exchange_tag(reinterpret_cast<const unsigned*>(ring + kRingWords), laps, row);
+  float my_gathered = 0.f;
+  if constexpr (TOPK) {
+    if (my_k >= 0) my_gathered = topk_gather_one<T>(a, logits + row * row_stride, vocab, my_id);
+  }
 
   // the scan, group by group as the vectors arrive, in scan_row()'s order
   SoftmaxAcc st{kNegHuge, 0.f, 0.f};
@@ -250,6 +271,11 @@ void actor_step_split_kernel(
   });
   unsigned long long* slot = ring + size_t(row % kRing) * kSlotWords;
   split_publish(slot, tag, vt, st);
+  unsigned long long* topk_slot = nullptr;
+  if constexpr (TOPK) {
+    topk_slot = topk_ring + size_t(row % kRing) * RELAX_AMD_FUSED_TOPK_MAX;
+    if (my_k >= 0) exchange_store(topk_slot + my_k, tag, my_gathered);
+  }
 
   if (wave0) {
     // thread 0 runs a serial stretch from here to the barrier while the other waves of the workgroup wait
@@ -275,12 +301,26 @@ void actor_step_split_kernel(
     if constexpr (TOPK) {
       int lane = tid;
       asm volatile("" : "+v"(lane));
-      gathered = topk_gather<T>(a, logits + row * row_stride, vocab, tok, lane);
+      gathered = topk_gather_meta(a, tok, lane);
       topk_shape = topk_row_shape(a, tok);
     }
     bool any_gave_up = false;
     const SoftmaxAcc whole = split_collect<ROW_THREADS / kWave>(slot, tag + wait_tag_offset, tid, max_polls,
                                                                 reinterpret_cast<unsigned*>(ring + kRingWords), any_gave_up);
+    if constexpr (TOPK) {
+      // the row's gathered logits, entry lane + 64 i from the workgroup that fetched it
+      unsigned* status = reinterpret_cast<unsigned*>(ring + kRingWords);
+      bool gave_up = any_gave_up;
+#pragma unroll
+      for (int i = 0; i < kTopkPerLane; ++i) {
+        const int k = tid + i * kWave;
+        if (k < a.topk_k && !gave_up)
+          gave_up = !exchange_wait(topk_slot + k, tag + wait_tag_offset, max_polls, status, gathered.x[i]);
+      }
+      const bool any_topk_gave_up = __any(gave_up);
+      if (any_topk_gave_up && !any_gave_up && tid == 0) exchange_report_give_up(status);
+      any_gave_up = any_topk_gave_up;
+    }
     float lse = 0.f, spx = 0.f, ent = 0.f, lp = 0.f;
     if (tid == 0) {
       scan_finish(whole, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
@@ -297,7 +337,8 @@ void actor_step_split_kernel(
       int lane = tid;
       asm volatile("" : "+v"(lane));
       g_topk = topk_distill_row(a, gathered, topk_shape, tok, lane_value(lse), inv_t, lane_value(lp),
-                                lane_value(tin.has_old ? tin.old_lp : lp), lane_value(tin.extra_lp), lane, topk_stage);
+                                lane_value(tin.has_old ? tin.old_lp : lp), lane_value(tin.extra_lp), lane, topk_stage,
+                                part == 0);
     }
     if (tid == 0) {
       relax_amd_policy_loss_args al = a;
@@ -617,7 +658,7 @@ __global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(3
 }
 
 namespace {
-ExchangeRingCache ring_cache;
+ExchangeRingCache ring_cache, topk_ring_cache;
 // relax_amd_set_exchange_wait: the bound of a workgroup's wait and an offset added to the tag it waits for
 std::atomic<unsigned> g_max_polls{kWaitPolls}, g_wait_tag_offset{0u};
 }  // namespace
@@ -627,6 +668,10 @@ unsigned exchange_wait_tag_offset() { return g_wait_tag_offset.load(std::memory_
 
 static int split_ring_of_device(unsigned long long** ring) {
   return exchange_ring_of_device(ring_cache, reinterpret_cast<const void*>(&split_ring), "actor_step_split", ring);
+}
+static int split_topk_ring_of_device(unsigned long long** ring) {
+  return exchange_ring_of_device(topk_ring_cache, reinterpret_cast<const void*>(&split_topk_ring), "actor_step_split",
+                                 ring);
 }
 
 // Waves per SIMD the kernel is compiled for.  Long 16-bit rows without the top-K term run fastest with three (six
@@ -649,13 +694,13 @@ constexpr int split_waves_max() {
     if (a.topk_ids)                                                                                                   \
       hipLaunchKernelGGL((RELAX_AMD_SPLIT_KERNEL(WIDTH, NVF, PARTIAL, true)), grid, block, 0, stream, logits,        \
                          row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
-                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps, max_polls,          \
-                         tag_offset);                                                                                 \
+                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, topk_ring, laps,          \
+                         max_polls, tag_offset);                                                                      \
     else                                                                                                              \
       hipLaunchKernelGGL((RELAX_AMD_SPLIT_KERNEL(WIDTH, NVF, PARTIAL, false)), grid, block, 0, stream, logits,       \
                          row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
-                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps, max_polls,          \
-                         tag_offset);                                                                                 \
+                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, topk_ring, laps,          \
+                         max_polls, tag_offset);                                                                      \
     return check_launch("actor_step_split");                                                                          \
   }
 #define RELAX_AMD_SPLIT(NVF, PARTIAL) RELAX_AMD_SPLIT_ROW(1024, NVF, PARTIAL)
@@ -666,8 +711,8 @@ constexpr int split_waves_max() {
     hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, false, 1024, 3, 3, (NVF >= 30 ? 13 : 12)>), grid,  \
                        block, 0, stream,                                                                              \
                        logits, row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t,  \
-                       a, grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps, max_polls,         \
-                       tag_offset);                                                                                   \
+                       a, grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, topk_ring, laps,         \
+                       max_polls, tag_offset);                                                                        \
     return check_launch("actor_step_split");                                                                          \
   }
 
@@ -703,10 +748,13 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
   }
   unsigned long long* ring = nullptr;
   if (int rc = split_ring_of_device(&ring)) return rc;
+  unsigned long long* topk_ring = nullptr;
+  if (int rc = split_topk_ring_of_device(&topk_ring)) return rc;
   const unsigned laps = unsigned((n_rows + kRing - 1) / kRing);
   const unsigned max_polls = exchange_max_polls();
   const unsigned tag_offset = exchange_wait_tag_offset();
-  hipLaunchKernelGGL(exchange_ring_advance_kernel<kRingWords>, dim3(1), dim3(256), 0, stream, ring, laps);
+  hipLaunchKernelGGL(exchange_ring_advance_kernel<kRingWords>, dim3(1), dim3(256), 0, stream, ring, laps,
+                     topk_ring, kTopkRingWords);
   const dim3 grid(static_cast<unsigned>(n_rows * (width / kSplitThreads))), block(kSplitThreads);
   if constexpr (sizeof(T) == 2) {
     RELAX_AMD_SPLIT_ROW(512, 7, true)
@@ -766,7 +814,8 @@ int launch_actor_step_split_wide(const float* logits, int64_t row_stride, int64_
   const unsigned laps = unsigned((n_rows + kRing - 1) / kRing);
   const unsigned max_polls = exchange_max_polls();
   const unsigned tag_offset = exchange_wait_tag_offset();
-  hipLaunchKernelGGL(exchange_ring_advance_kernel<kRingWords>, dim3(1), dim3(256), 0, stream, ring, laps);
+  hipLaunchKernelGGL(exchange_ring_advance_kernel<kRingWords>, dim3(1), dim3(256), 0, stream, ring, laps,
+                     static_cast<unsigned long long*>(nullptr), size_t(0));
   const dim3 grid(static_cast<unsigned>(n_rows * kSplit)), block(kSplitThreads);
   // 151936 / 152064 (37984 / 38016 vectors), 128256 / 129280 (32064 / 32320), 131072 (32768), 163840 (40960),
   // 100352 / 102400 (25088 / 25600)

@@ -184,6 +184,33 @@ __device__ __forceinline__ TopkGather topk_gather(const relax_amd_policy_loss_ar
   return g;
 }
 
+// topk_gather() without the logits (x stays 0): the teacher's log-probs and which ids are sentinels, both contiguous
+// reads, for a caller that receives the gathered logits from elsewhere (the one-shot actor step shares the scattered
+// gather between the workgroups of a row).
+__device__ __forceinline__ TopkGather topk_gather_meta(const relax_amd_policy_loss_args& a, int64_t tok, int lane) {
+  TopkGather g;
+  const int kmax = a.topk_k;
+  const int64_t* ids = a.topk_ids + tok * kmax;
+  const float* teacher = a.topk_teacher_log_prob + tok * kmax;
+#pragma unroll
+  for (int i = 0; i < kTopkPerLane; ++i) {
+    const int k = lane + i * kWave;
+    g.x[i] = g.t[i] = 0.f;
+    g.real[i] = false;
+    if (k < kmax) {
+      g.t[i] = teacher[k];
+      g.real[i] = ids[k] >= 0;
+    }
+  }
+  return g;
+}
+// the logit topk_gather() puts in x for entry k of token `tok`
+template <typename T>
+__device__ __forceinline__ float topk_gather_one(const relax_amd_policy_loss_args& a, const T* x, int64_t vocab,
+                                                 int64_t id) {
+  return id < 0 ? -INFINITY : (id >= vocab ? 0.f : Row<T>::load1(x + id));
+}
+
 // Token `tok`'s entry count and union-mask length for the signal (the whole list / no mask without the arrays): two
 // more scalars that can be on their way before the row's log-sum-exp is known.
 struct TopkRowShape {
@@ -198,12 +225,14 @@ __device__ __forceinline__ TopkRowShape topk_row_shape(const relax_amd_policy_lo
 // clips and weight, topk_kl / topk_grad written.  `g` = this lane's topk_gather(), `shape` = topk_row_shape() of the
 // token, `weight` = the signal's weight in the loss, `old` = the token's old log-prob (the current one when there is
 // none).  Returns, in every lane, the sum of d loss / d log p[id_k] over the non-sentinel ids: what the row's softmax
-// is multiplied by, next to the policy terms' own coefficient.  `stage` = kTopkStageFloats floats of LDS.
+// is multiplied by, next to the policy terms' own coefficient.  `stage` = kTopkStageFloats floats of LDS.  `emit`:
+// whether this caller writes topk_kl / topk_grad (one of several workgroups that evaluate the same token does).
 constexpr int kTopkStageFloats = 4 * RELAX_AMD_FUSED_TOPK_MAX;
 
 __device__ __forceinline__ float topk_distill_row(const relax_amd_policy_loss_args& a, const TopkGather& g,
                                                   const TopkRowShape& shape, int64_t tok, float lse, float inv_t,
-                                                  float lp, float old, float weight, int lane, float* stage) {
+                                                  float lp, float old, float weight, int lane, float* stage,
+                                                  bool emit = true) {
   const int kmax = a.topk_k;
   const int width = shape.width < 0 ? 0 : (shape.width > kmax ? kmax : shape.width);
   const int nvalid = shape.nvalid;
@@ -238,10 +267,10 @@ __device__ __forceinline__ float topk_distill_row(const relax_amd_policy_loss_ar
         d = f * sv[k];
         if (g.real[i] && d != 0.f) total += d;
       }
-      a.topk_grad[tok * kmax + k] = d;
+      if (emit) a.topk_grad[tok * kmax + k] = d;
     }
   }
-  if (lane == 0) a.topk_kl[tok] = kl;
+  if (lane == 0 && emit) a.topk_kl[tok] = kl;
   return wave_sum(total);
 }
 

@@ -315,7 +315,8 @@ int launch_reverse_kl_split(const T* student, const T* teacher, int64_t stride, 
     const unsigned laps = unsigned((n_rows + kRing - 1) / kRing);
     const unsigned max_polls = exchange_max_polls();
     const unsigned tag_offset = exchange_wait_tag_offset();
-    hipLaunchKernelGGL(exchange_ring_advance_kernel<kKlRingWords>, dim3(1), dim3(256), 0, stream, ring, laps);
+    hipLaunchKernelGGL(exchange_ring_advance_kernel<kKlRingWords>, dim3(1), dim3(256), 0, stream, ring, laps,
+                       static_cast<unsigned long long*>(nullptr), size_t(0));
     const dim3 grid(static_cast<unsigned>(n_rows * kKlSplit)), block(kKlSplitThreads);
 #define RELAX_AMD_KL_SPLIT(NVF, PARTIAL)                                                                              \
   if (full == NVF && partial == PARTIAL) {                                                                            \

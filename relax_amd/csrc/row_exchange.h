@@ -35,14 +35,19 @@ unsigned exchange_max_polls();
 unsigned exchange_wait_tag_offset();
 
 // Advances the tag counter by the laps of the launch that follows; clears the ring when the 32-bit counter would wrap
-// (a tag of a past lap could otherwise come round again).
+// (a tag of a past lap could otherwise come round again), and with it `extra` (a second array of tagged words that
+// shares the ring's tags, or null).
 template <size_t RING_WORDS>
-__global__ __launch_bounds__(256) void exchange_ring_advance_kernel(unsigned long long* ring, unsigned laps) {
+__global__ __launch_bounds__(256) void exchange_ring_advance_kernel(unsigned long long* ring, unsigned laps,
+                                                                    unsigned long long* extra, size_t extra_words) {
   unsigned* counter = reinterpret_cast<unsigned*>(ring + RING_WORDS);
   const unsigned now = counter[0];
   const bool wrap = now > 0xffffffffu - laps - 1u;
-  if (wrap)
+  if (wrap) {
     for (size_t i = threadIdx.x; i < RING_WORDS; i += 256) ring[i] = 0ull;
+    if (extra)
+      for (size_t i = threadIdx.x; i < extra_words; i += 256) extra[i] = 0ull;
+  }
   __syncthreads();
   if (threadIdx.x == 0) {
     counter[0] = (wrap ? 0u : now) + laps;

@@ -1242,7 +1242,12 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
 @pytest.mark.parametrize("v,dtype,k,variant", [(100352, torch.bfloat16, 64, "reverse_tail"),
                                                (100352, torch.bfloat16, 200, "union_jsd_clips"),
                                                (151936, torch.bfloat16, 64, "forward_norm"),
-                                               (32000, torch.float32, 96, "low_var")])
+                                               (32000, torch.float32, 96, "low_var"),
+                                               # K = 1, just past one wave's width, and the largest the launch takes:
+                                               # how the one-shot kernel's workgroups share the gather of a row's ids
+                                               (100352, torch.bfloat16, 1, "forward_norm"),
+                                               (163840, torch.bfloat16, 65, "union_jsd_clips"),
+                                               (151936, torch.bfloat16, 256, "reverse_tail")])
 def test_topk_opd_term_in_the_register_resident_step(v, dtype, k, variant):
     """The top-K distillation term inside the single launch on the row shapes of the register-resident kernel (several
     rows per persistent workgroup, K below and above one wave's width, the union mask, clips): loss, metrics and
@@ -1290,6 +1295,22 @@ def test_topk_opd_term_in_the_register_resident_step(v, dtype, k, variant):
     assert torch.equal(loss.detach(), outs["auto"][0]) and torch.equal(lg.grad, outs["auto"][2])
     for key, w in outs["auto"][1].items():
         assert torch.equal(met[key], w), key
+    if variant == "reverse_tail":
+        # the exchange of the one-shot kernel forced to give up from the host (triples and gathered logits alike):
+        # NaN instead of a hang, and the launch after it exact again
+        from relax_amd._lib import check, lib
+        check(lib.relax_amd_set_exchange_wait(4, 1))
+        try:
+            lg = logits.to(dev).requires_grad_()
+            loss, _ = relax_amd.policy_loss_function(P.make_args(relax_amd_single_pass="auto", **kw), db, lg, None)
+            torch.cuda.synchronize()
+        finally:
+            check(lib.relax_amd_set_exchange_wait(0, 0))
+        assert torch.isnan(loss).all()
+        lg = logits.to(dev).requires_grad_()
+        loss, _ = relax_amd.policy_loss_function(P.make_args(relax_amd_single_pass="auto", **kw), db, lg, None)
+        loss.backward()
+        assert torch.equal(loss.detach(), outs["auto"][0]) and torch.equal(lg.grad, outs["auto"][2])
     ulp = {torch.bfloat16: 2.0 ** -7, torch.float32: 1e-5}[dtype]
     assert abs(outs["auto"][0].item() - outs["off"][0].item()) < 1e-5 * max(1.0, abs(outs["off"][0].item()))
     assert set(outs["auto"][1]) == set(outs["off"][1])
