@@ -350,6 +350,58 @@ def test_one_shot_reverse_kl_step_gives_up_a_wait_that_cannot_succeed_and_recove
         assert torch.equal(a.view(torch.int16) if a.dtype == torch.bfloat16 else a, b.view(torch.int16) if b.dtype == torch.bfloat16 else b)
 
 
+def test_default_reverse_kl_step_replayed_from_a_captured_graph():
+    """The default reverse-KL step tags the partial sums its workgroups exchange with a counter that a small kernel in
+    front of the launch advances on the device, so a captured launch gets fresh tags on every replay: three replays on
+    fresh rows, with eager launches between them, each bit-identical to the two-walk kernel on the same inputs."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("reverse-KL step under graph capture")
+    v, n = 100352, 260
+    gen = torch.Generator(device=dev).manual_seed(17)
+    s = torch.empty((n, v), device=dev, dtype=torch.bfloat16)
+    t = torch.empty((n, v), device=dev, dtype=torch.bfloat16)
+    g = torch.rand(n, device=dev, generator=gen)
+    g[5] = 0.0
+
+    def fresh():
+        s.copy_(torch.randn((n, v), device=dev, generator=gen) * 3)
+        t.copy_(s.float() + torch.randn((n, v), device=dev, generator=gen))
+
+    def run():
+        kl, ls, lt, d = ops.reverse_kl_step_fused(s, t, g, 1.0)
+        return dict(kl=kl, lse_s=ls, lse_t=lt, d=d.view(torch.int16))
+
+    fresh()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()  # warm-up outside the capture (the library looks its exchange buffer up on first use)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run()
+    try:
+        for rep in range(3):
+            fresh()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = {k: x.clone() for k, x in captured.items()}
+            eager = run()  # an eager launch between the replays
+            ops.set_kernel_choice("two_walk")
+            want = run()
+            ops.set_kernel_choice("auto")
+            torch.cuda.synchronize()
+            for key in want:
+                assert torch.equal(got[key], want[key]), (rep, key)
+                assert torch.equal(eager[key], want[key]), (rep, key, "eager")
+            assert not torch.isnan(got["kl"]).any()
+    finally:
+        ops.set_kernel_choice("auto")
+
+
 def test_opd_token_mean_literal(literals):
     from relax_amd.opd_utils import compute_opd_kl, reduce_opd_loss
 
