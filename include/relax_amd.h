@@ -344,7 +344,7 @@ int relax_amd_reverse_kl_bwd(const void* student, const void* teacher, int dtype
  * relax_amd_reverse_kl_bwd (dstudent row stride = row_stride); each workgroup re-reads its two rows out of cache, so
  * HBM moves 3*V*s bytes per token instead of 5*V*s.  Three kernels sit behind it, with bit-identical results: 16-bit
  * rows of the built vocabulary shapes (12 / 15 / 18 / 19 full 16-byte vectors per thread of 1024 threads plus a
- * partial one, or 16 / 20 exactly; the default kernel also 6 / 7 plus a partial one and 8 exactly) are shared by eight
+ * partial one, or 16 / 20 exactly; the default kernel also 6 / 7 / 24 / 30 / 31 plus a partial one and 8 / 32 exactly) are shared by eight
  * one-shot workgroups that keep both rows' shares on chip, so each row is read once (the default), or, after
  * relax_amd_set_kernel_choice(RELAX_AMD_KERNEL_RESIDENT), kept as the student row in the registers of one persistent
  * workgroup that streams the teacher row past it twice; other rows, and every row after
@@ -477,7 +477,7 @@ int relax_amd_logprob_entropy_topk_fwd(const void* logits, int dtype, int64_t n_
  * results bit for bit: one-shot workgroups that share each row (one read and one write of HBM per row; 16-bit rows of
  * 28680 .. 32768, 49160 .. 53248, 57352 .. 65536, 100352 .. 163840 and, without the top-K block, 196616 .. 204800 and
  * 245768 .. 262144 entries (these keep part of the row in LDS), fp32 rows of 28676 .. 32768, 49156 .. 53248,
- * 61444 .. 65536 and, as upper halves, 100352 .. 163840 entries, in the built shapes: the default where built, see
+ * 61444 .. 65536 and, as upper halves, 100352 .. 163840 and 245764 .. 249856 entries, in the built shapes: the default where built, see
  * relax_amd_set_kernel_choice for the ring in device memory it exchanges partial sums through), a persistent
  * register-resident one (the same traffic, the same shapes) and a two-walk one for everything
  * else; relax_amd_set_kernel_choice(RELAX_AMD_KERNEL_RESIDENT / RELAX_AMD_KERNEL_TWO_WALK) forces the second / third.

@@ -425,9 +425,11 @@ __device__ __forceinline__ void split_wide_unpack(const u32x4& r, int half, floa
 // halves (38 four-float positions per thread in 19 register quads at V = 151936), scans the fp32 values as they land,
 // ORs the low halves it drops; a wave that dropped nothing computes its gradient from the registers, a wave that did
 // (fp32 logits with real low bits) reads its share again.  Exchange, tags and waits as in actor_step_split_kernel.
-// (three waves per SIMD: 5.80 ms on 32768 x 151936 fp32 rows where four give 5.91 and two 5.75)
-template <int NF, bool PARTIAL>
-__global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void actor_step_split_wide_kernel(
+// (three waves per SIMD: 5.80 ms on 32768 x 151936 fp32 rows where four give 5.91 and two 5.75; rows of 248320
+// entries, 31 register quads per thread, are built for two)
+template <int NF, bool PARTIAL, int WAVES = 3>
+__global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES)))
+void actor_step_split_wide_kernel(
     const float* __restrict__ logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
     const int32_t* __restrict__ token_of_row, const int32_t* __restrict__ sample_ids,
     const int64_t* __restrict__ targets, float c, float inv_t, relax_amd_policy_loss_args a, float grad_scale,
@@ -789,7 +791,8 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
 
 #define RELAX_AMD_SPLIT_WIDE(NF, PARTIAL)                                                                             \
   if (full == NF && partial == PARTIAL) {                                                                             \
-    hipLaunchKernelGGL((actor_step_split_wide_kernel<NF, PARTIAL>), grid, block, 0, stream, logits, row_stride,      \
+    hipLaunchKernelGGL((actor_step_split_wide_kernel<NF, PARTIAL, 3>), grid, block, 0, stream,       \
+                       logits, row_stride,                                                                            \
                        vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a, grad_scale,       \
                        log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps, max_polls, tag_offset);           \
     return check_launch("actor_step_split_wide");                                                                     \
@@ -807,7 +810,7 @@ int launch_actor_step_split_wide(const float* logits, int64_t row_stride, int64_
   const int full = int(nvec / 1024);
   const bool partial = nvec % 1024 != 0;
   if (!((full == 37 && partial) || (full == 31 && partial) || (full == 32 && !partial) || (full == 40 && !partial) ||
-        (full == 24 && partial) || (full == 25 && !partial)))
+        (full == 24 && partial) || (full == 25 && !partial) || (full == 60 && partial)))
     return RELAX_AMD_EUNSUPPORTED;
   unsigned long long* ring = nullptr;
   if (int rc = split_ring_of_device(&ring)) return rc;
@@ -818,7 +821,8 @@ int launch_actor_step_split_wide(const float* logits, int64_t row_stride, int64_
                      static_cast<unsigned long long*>(nullptr), size_t(0));
   const dim3 grid(static_cast<unsigned>(n_rows * kSplit)), block(kSplitThreads);
   // 151936 / 152064 (37984 / 38016 vectors), 128256 / 129280 (32064 / 32320), 131072 (32768), 163840 (40960),
-  // 100352 / 102400 (25088 / 25600)
+  // 100352 / 102400 (25088 / 25600), 248320 (62080)
+  RELAX_AMD_SPLIT_WIDE(60, true)
   RELAX_AMD_SPLIT_WIDE(37, true)
   RELAX_AMD_SPLIT_WIDE(31, true)
   RELAX_AMD_SPLIT_WIDE(32, false)

@@ -261,18 +261,19 @@ ExchangeRingCache kl_ring_cache;
 // Long rows (12 and more vector positions per thread): three waves per SIMD, i.e. six workgroups per CU, each with
 // twelve teacher vectors per thread (24 KB) in LDS; with both rows in registers only two waves per SIMD fit, which is
 // 9 % slower on 16384 x 151936 rows (2.71 - 2.73 against 2.47 ms).  Shorter rows fit the registers of four and more
-// waves per SIMD as they are.
+// waves per SIMD as they are.  Rows of more than 20 vectors per thread (vocabularies of 200 k - 262 k entries): two
+// waves per SIMD (256 registers a lane, four workgroups per CU) with eighteen teacher vectors per thread (36 KB) in LDS.
 template <int NVF>
 constexpr int kl_split_lds_vecs() {
-  return NVF >= 12 ? 12 : 0;
+  return NVF >= 24 ? 18 : NVF >= 12 ? 12 : 0;
 }
 template <int NVF>
 constexpr int kl_split_waves_min() {
-  return NVF >= 12 ? 3 : 4;
+  return NVF >= 24 ? 2 : NVF >= 12 ? 3 : 4;
 }
 template <int NVF>
 constexpr int kl_split_waves_max() {
-  return NVF >= 12 ? 3 : 8;
+  return NVF >= 24 ? 2 : NVF >= 12 ? 3 : 8;
 }
 
 template <typename T>
@@ -304,7 +305,8 @@ int launch_reverse_kl_split(const T* student, const T* teacher, int64_t stride, 
     // entries: 1.91 / 2.33 / 2.08 ms on 32768 rows where the two-walk kernel takes 2.11 / 2.79 / 2.74).  Rows of
     // 32000 entries, four vectors per thread, are left to the two-walk kernel: here the exchange outweighs the second
     // read (2.77 against 2.52 ms on 65536 rows).
-    if (!((full == 20 && !partial) || (full == 19 && partial) || (full == 18 && partial) || (full == 15 && partial) ||
+    if (!((full == 24 && partial) || (full == 30 && partial) || (full == 31 && partial) || (full == 32 && !partial) ||
+          (full == 20 && !partial) || (full == 19 && partial) || (full == 18 && partial) || (full == 15 && partial) ||
           (full == 16 && !partial) || (full == 12 && partial) || (full == 8 && !partial) || (full == 7 && partial) ||
           (full == 6 && partial)))
       return RELAX_AMD_EUNSUPPORTED;
@@ -326,6 +328,11 @@ int launch_reverse_kl_split(const T* student, const T* teacher, int64_t stride, 
                        lse_t, dstudent, ring, laps, max_polls, tag_offset);                                           \
     return check_launch("reverse_kl_split");                                                                          \
   }
+    // 200064 / 201088 / 202048, 248320 / 250880, 256000, 262144 entries
+    RELAX_AMD_KL_SPLIT(24, true)
+    RELAX_AMD_KL_SPLIT(30, true)
+    RELAX_AMD_KL_SPLIT(31, true)
+    RELAX_AMD_KL_SPLIT(32, false)
     RELAX_AMD_KL_SPLIT(20, false)
     RELAX_AMD_KL_SPLIT(19, true)
     RELAX_AMD_KL_SPLIT(18, true)

@@ -1751,7 +1751,9 @@ def test_register_resident_step_over_many_rows_per_workgroup(v, dtype, n_samples
     # 16-bit rows scanned by 512 threads: no persistent kernel exists for them, the one-shot kernel does
     (32000, torch.bfloat16, 1500, "short"), (50304, torch.float16, 1000, "short"),
     # 16-bit rows of more than 20 vectors per thread: the one-shot kernel keeps twelve of them in LDS
-    (202048, torch.bfloat16, 300, "short"), (262144, torch.float16, 200, "short"),
+    (202048, torch.bfloat16, 300, "short"), (262144, torch.float16, 200, "short"), (248320, torch.bfloat16, 200, "short"),
+    # fp32 rows of 248320 entries (the Qwen3.5 vocabulary as stock Megatron hands it to the loss), upper halves
+    (248320, torch.float32, 160, "widened_short"), (248320, torch.float32, 160, "mixed_short"),
     # long fp32 rows, kept in the registers as their upper halves: bf16 values widened to fp32 (what a bf16 output
     # layer followed by .float() delivers: one read of the row), fp32 values with low bits (the row is read again), and
     # rows of both kinds next to each other, one of them with a single low bit in its last element
@@ -1773,9 +1775,10 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
     announce("resident vs two-walk", pattern, v, dtype)
     g = torch.Generator().manual_seed(len(pattern))
     logits = (torch.randn(n_rows, v, generator=g) * 2).to(dtype)
-    if values in ("widened", "mixed"):
+    no_resident = values.endswith("short")  # (RESIDENT fails for these rows by design)
+    if values.startswith(("widened", "mixed")):
         logits = logits.bfloat16().to(dtype)
-    if values == "mixed":
+    if values.startswith("mixed"):
         other = torch.randn(n_rows // 3, v, generator=g) * 2
         logits[1::3][: other.size(0)] = other  # every third row keeps its low bits
         logits[2::3, -1] += 2.0 ** -14         # and the next one differs from a widened row in one bit of one element
@@ -1813,8 +1816,8 @@ def test_register_resident_kernel_equals_two_walk_kernel_bitwise(pattern, v, dty
     targets = torch.randint(0, v, (n_tok,), generator=g).to(dev)
     results = {}
     for kind in ("cached", "resident", "auto", "auto_again"):
-        if values == "short" and kind == "resident":
-            kind = "auto"  # (RESIDENT fails for these rows by design)
+        if no_resident and kind == "resident":
+            kind = "auto"
         ops.set_kernel_choice({"cached": "two_walk", "resident": "resident"}.get(kind, "auto"))
         out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, token_of_row, sample_ids, n_tok, 1.0, 1.0, **kw)
         torch.cuda.synchronize()
