@@ -234,7 +234,8 @@ def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
             and KERNEL_CHOICE != "two_walk":
         return f"actor_step_resident_kernel<{dtype}, {shape[0]}, {str(shape[1]).lower()}>"
     if dtype == "float" and vocab % 4 == 0 and threads == 1024 and KERNEL_CHOICE != "two_walk" \
-            and shape in ((37, True), (31, True), (32, False), (40, False), (24, True), (25, False)):
+            and shape in ((37, True), (31, True), (32, False), (40, False), (24, True), (25, False)) \
+            + (((60, True),) if KERNEL_CHOICE == "auto" else ()):
         # long fp32 rows, held as their upper halves (one-shot workgroups sharing each row, or one persistent workgroup)
         return f"actor_step_{'split' if KERNEL_CHOICE == 'auto' else 'resident'}_wide_kernel<{shape[0]}, {str(shape[1]).lower()}>"
     return f"actor_step_fused_kernel<{dtype}, true, {threads}>"
@@ -257,7 +258,7 @@ def kl_step_kernel_name(vocab: int) -> str:
     nvec = vocab // 8
     shape = (nvec // 1024, nvec % 1024 != 0)
     long_rows = ((20, False), (19, True), (18, True), (15, True), (16, False), (12, True))
-    split_rows = long_rows + ((8, False), (7, True), (6, True))
+    split_rows = long_rows + ((8, False), (7, True), (6, True), (24, True), (30, True), (31, True), (32, False))
     if vocab % 8 == 0 and KERNEL_CHOICE == "auto" and shape in split_rows:
         return f"reverse_kl_split_kernel<bf16_t, {shape[0]}, {str(shape[1]).lower()}>"
     if vocab % 8 == 0 and KERNEL_CHOICE != "two_walk" and shape in long_rows:
