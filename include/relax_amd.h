@@ -475,8 +475,8 @@ int relax_amd_logprob_entropy_topk_fwd(const void* logits, int dtype, int64_t n_
  * argument block); the caller adds the K one-hot parts of its gradient with relax_amd_sparse_row_add afterwards.
  * Three kernels sit behind this entry point and are chosen by row length and element type, all with the same
  * results bit for bit: one-shot workgroups that share each row (one read and one write of HBM per row; 16-bit rows of
- * 28680 .. 32768, 49160 .. 53248, 57352 .. 65536, 100352 .. 163840 and, without the top-K block, 196616 .. 204800 and
- * 245768 .. 262144 entries (these keep part of the row in LDS), fp32 rows of 28676 .. 32768, 49156 .. 53248,
+ * 28680 .. 32768, 49160 .. 53248, 57352 .. 65536, 100352 .. 163840, 196616 .. 204800 and 245768 .. 262144 entries
+ * (the last two ranges keep part of the row in LDS), fp32 rows of 28676 .. 32768, 49156 .. 53248,
  * 61444 .. 65536 and, as upper halves, 100352 .. 163840 and 245764 .. 249856 entries, in the built shapes: the default where built, see
  * relax_amd_set_kernel_choice for the ring in device memory it exchanges partial sums through), a persistent
  * register-resident one (the same traffic, the same shapes) and a two-walk one for everything

@@ -706,15 +706,21 @@ constexpr int split_waves_max() {
     return check_launch("actor_step_split");                                                                          \
   }
 #define RELAX_AMD_SPLIT(NVF, PARTIAL) RELAX_AMD_SPLIT_ROW(1024, NVF, PARTIAL)
-// rows of more than 20 vectors per thread: twelve of them in LDS (24 KB of the 26 a workgroup can have when six share
-// a CU), three waves per SIMD; the top-K term is left to the two-walk kernel for these rows
+// rows of more than 20 vectors per thread: twelve or thirteen of them in LDS (24 - 26 KB of the 26.7 a workgroup can
+// have when six share a CU), three waves per SIMD; with the top-K term (4 KB of LDS more, a longer serial stretch)
+// sixteen in LDS and two waves per SIMD
 #define RELAX_AMD_SPLIT_LDS(NVF, PARTIAL)                                                                             \
   if (width == 1024 && full == NVF && partial == PARTIAL) {                                                           \
-    hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, false, 1024, 3, 3, (NVF >= 30 ? 13 : 12)>), grid,  \
-                       block, 0, stream,                                                                              \
-                       logits, row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t,  \
-                       a, grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, topk_ring, laps,         \
-                       max_polls, tag_offset);                                                                        \
+    if (a.topk_ids)                                                                                                   \
+      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, true, 1024, 2, 2, 16>), grid, block, 0, stream,   \
+                         logits, row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e,       \
+                         inv_t, a, grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, topk_ring,      \
+                         laps, max_polls, tag_offset);                                                                \
+    else                                                                                                              \
+      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, false, 1024, 3, 3, (NVF >= 30 ? 13 : 12)>), grid, \
+                         block, 0, stream, logits, row_stride, vocab, n_rows, token_of_row, sample_ids, targets,     \
+                         inv_t * kLog2e, inv_t, a, grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, \
+                         topk_ring, laps, max_polls, tag_offset);                                                     \
     return check_launch("actor_step_split");                                                                          \
   }
 
@@ -738,7 +744,6 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
   } else if constexpr (sizeof(T) == 2) {
     const bool lds_row = (full == 24 && partial) || (full == 30 && partial) || (full == 31 && partial) ||
                          (full == 32 && !partial);
-    if (lds_row && a.topk_ids) return RELAX_AMD_EUNSUPPORTED;
     if (!(lds_row || (full == 20 && !partial) || (full == 19 && partial) || (full == 18 && partial) ||
           (full == 15 && partial) || (full == 16 && !partial) || (full == 12 && partial) || (full == 8 && !partial) ||
           (full == 7 && partial)))
