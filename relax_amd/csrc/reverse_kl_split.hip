@@ -196,9 +196,8 @@ void reverse_kl_split_kernel(
       gave_up = !exchange_wait(slot + kWave + tid, tag + wait_tag_offset, max_polls, status, hi);
     const bool any_gave_up = __any(gave_up);
     if (any_gave_up && tid == 0) exchange_report_give_up(status);
-    auto word = [&](int i) {
-      return __int_as_float(i < kWave ? __builtin_amdgcn_readlane(__float_as_int(lo), i < kWave ? i : 0)
-                                      : __builtin_amdgcn_readlane(__float_as_int(hi), i < kWave ? 0 : i - kWave));
+    auto word = [&](int i) {  // word i of the slot, in every lane
+      return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(i < kWave ? lo : hi), i & (kWave - 1)));
     };
     KlState whole{word(0), word(1), word(2), word(3), word(4)};
 #pragma unroll
