@@ -86,8 +86,8 @@ enum { RELAX_AMD_KERNEL_AUTO = 0, RELAX_AMD_KERNEL_TWO_WALK = 1, RELAX_AMD_KERNE
  * Process-wide, read atomically at each launch; returns the previous choice, or RELAX_AMD_EINVAL.  No counterpart
  * in the reference: it exists for tests and measurements.
  *
- * The one-shot kernels of the actor step and of the reverse-KL step each keep their exchange ring (1.5 MB / 2.5 MB)
- * in a static array of the library, one copy per GPU and process.  Launches of the same entry point that overlap on
+ * The one-shot kernels of the actor step and of the reverse-KL step each keep their exchange ring (1.5 MB, plus 8 MB
+ * for the logits gathered at a row's top-K ids / 2.5 MB) in static arrays of the library, one copy per GPU and process.  Launches of the same entry point that overlap on
  * one GPU (two streams of one process) must not both take that kernel: they could overwrite each other's slots, which
  * the kernel notices (bounded waits) and reports as NaN log-probs (NaN KL) rather than wrong numbers.  Launches in stream order, captured graphs and their replays
  * are fine (the tags that tell one launch's partial sums from another's come from a counter in device memory that a
