@@ -280,7 +280,10 @@ def test_register_resident_reverse_kl_step_equals_two_walk_kernel_bitwise(v, dty
 @pytest.mark.parametrize("v,dtype,n", [(50304, torch.bfloat16, 700), (64000, torch.bfloat16, 300),
                                        (65536, torch.float16, 9), (8 * 7169, torch.float16, 515),
                                        (248320, torch.bfloat16, 150), (202048, torch.float16, 130),
-                                       (256000, torch.bfloat16, 70), (262144, torch.float16, 20)])
+                                       (256000, torch.bfloat16, 70), (262144, torch.float16, 20),
+                                       # one lane, and all lanes but one, at the partial vector position
+                                       (8 * (30 * 1024 + 1), torch.float16, 40), (8 * (31 * 1024 + 1023), torch.bfloat16, 40),
+                                       (8 * (6 * 1024 + 1), torch.bfloat16, 300), (8 * (7 * 1024 + 1023), torch.float16, 300)])
 def test_one_shot_reverse_kl_step_on_short_rows_equals_two_walk_kernel_bitwise(v, dtype, n):
     """Rows of 6145 .. 8192 sixteen-byte vectors and of more than 20 vectors per thread (vocabularies of 200 k - 262 k
     entries: eighteen teacher vectors per thread in LDS, two waves per SIMD), which only the two-walk kernel and the
