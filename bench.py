@@ -233,11 +233,13 @@ def fused_step_kernel_name(vocab: int, dtype: str = "bf16_t") -> str:
     if vocab % per_vec == 0 and threads == width and shape in shapes \
             and KERNEL_CHOICE != "two_walk":
         return f"actor_step_resident_kernel<{dtype}, {shape[0]}, {str(shape[1]).lower()}>"
-    if dtype == "float" and vocab % 4 == 0 and threads == 1024 and KERNEL_CHOICE != "two_walk" \
-            and shape in ((37, True), (31, True), (32, False), (40, False), (24, True), (25, False)) \
-            + (((60, True),) if KERNEL_CHOICE == "auto" else ()):
-        # long fp32 rows, held as their upper halves (one-shot workgroups sharing each row, or one persistent workgroup)
-        return f"actor_step_{'split' if KERNEL_CHOICE == 'auto' else 'resident'}_wide_kernel<{shape[0]}, {str(shape[1]).lower()}>"
+    wide = ((37, True), (31, True), (32, False), (40, False), (24, True), (25, False))
+    if dtype == "float" and vocab % 4 == 0 and threads == 1024 and KERNEL_CHOICE == "auto" and shape in wide + ((60, True),):
+        # long fp32 rows: one-shot workgroups that keep part of their row share in LDS
+        return f"actor_step_split_kernel<{dtype}, {shape[0]}, {str(shape[1]).lower()}>"
+    if dtype == "float" and vocab % 4 == 0 and threads == 1024 and KERNEL_CHOICE == "resident" and shape in wide:
+        # one persistent workgroup per row, the row held as its upper halves
+        return f"actor_step_resident_wide_kernel<{shape[0]}, {str(shape[1]).lower()}>"
     return f"actor_step_fused_kernel<{dtype}, true, {threads}>"
 
 

@@ -477,7 +477,7 @@ int relax_amd_logprob_entropy_topk_fwd(const void* logits, int dtype, int64_t n_
  * results bit for bit: one-shot workgroups that share each row (one read and one write of HBM per row; 16-bit rows of
  * 28680 .. 32768, 49160 .. 53248, 57352 .. 65536, 100352 .. 163840, 196616 .. 204800 and 245768 .. 262144 entries
  * (the last two ranges keep part of the row in LDS), fp32 rows of 28676 .. 32768, 49156 .. 53248,
- * 61444 .. 65536 and, as upper halves, 100352 .. 163840 and 245764 .. 249856 entries, in the built shapes: the default where built, see
+ * 61444 .. 65536 and, part of the row in LDS, 100352 .. 163840 and 245764 .. 249856 entries, in the built shapes: the default where built, see
  * relax_amd_set_kernel_choice for the ring in device memory it exchanges partial sums through), a persistent
  * register-resident one (the same traffic, the same shapes) and a two-walk one for everything
  * else; relax_amd_set_kernel_choice(RELAX_AMD_KERNEL_RESIDENT / RELAX_AMD_KERNEL_TWO_WALK) forces the second / third.

@@ -230,11 +230,6 @@ static int dispatch_fused(const void* logits, int64_t n_rows, int64_t vocab, int
     const int rc = launch_actor_step_split<T>(x, stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t, a,
                                               grad_scale, lp, ent, lse, spx, d, d_stride, s);
     if (rc != RELAX_AMD_EUNSUPPORTED) return rc;
-    if constexpr (sizeof(T) == 4) {
-      const int rcw = launch_actor_step_split_wide(x, stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t,
-                                                   a, grad_scale, lp, ent, lse, spx, d, d_stride, s);
-      if (rcw != RELAX_AMD_EUNSUPPORTED) return rcw;
-    }
   }
   if (vec && choice != RELAX_AMD_KERNEL_TWO_WALK) {
     const int rc = launch_actor_step_resident<T>(x, stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t, a,

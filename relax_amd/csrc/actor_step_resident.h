@@ -30,19 +30,12 @@ int launch_actor_step_resident_wide(const float* logits, int64_t row_stride, int
 
 // The same step, same bits, with every row shared between eight one-shot 128-thread workgroups that exchange their
 // waves' partial softmax sums through device memory (actor_step_split.hip); the row shapes of
-// launch_actor_step_resident with 1024 virtual threads.
+// launch_actor_step_resident and launch_actor_step_resident_wide, and longer and shorter rows besides.
 template <typename T>
 int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
                             const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,
                             float inv_t, const relax_amd_policy_loss_args& a, float grad_scale, float* log_prob,
                             float* entropy, float* lse, float* spx, T* dlogits, int64_t d_stride,
                             hipStream_t stream);
-
-// launch_actor_step_resident_wide's rows in the one-shot form (actor_step_split.hip), same bits.
-int launch_actor_step_split_wide(const float* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
-                                 const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,
-                                 float inv_t, const relax_amd_policy_loss_args& a, float grad_scale, float* log_prob,
-                                 float* entropy, float* lse, float* spx, float* dlogits, int64_t d_stride,
-                                 hipStream_t stream);
 
 }  // namespace relax_amd

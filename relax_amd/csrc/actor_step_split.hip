@@ -402,263 +402,6 @@ void actor_step_split_kernel(
   }
 }
 
-// ---- fp32 rows of 100352 .. 163840 entries, held as their upper halves (see actor_step_resident_wide.hip) -----------
-
-// upper halves of two four-float vectors, in memory order
-__device__ __forceinline__ u32x4 split_wide_pack(const u32x4& a, const u32x4& b) {
-  return u32x4{(a.x >> 16) | (a.y & 0xffff0000u), (a.z >> 16) | (a.w & 0xffff0000u), (b.x >> 16) | (b.y & 0xffff0000u),
-               (b.z >> 16) | (b.w & 0xffff0000u)};
-}
-__device__ __forceinline__ uint32_t split_wide_low_bits(const u32x4& a) { return (a.x | a.y | a.z | a.w) & 0xffffu; }
-// vector `half` (0 / 1) of a packed pair, widened again
-__device__ __forceinline__ void split_wide_unpack(const u32x4& r, int half, float (&o)[4]) {
-  const uint32_t w0 = half ? r.z : r.x, w1 = half ? r.w : r.y;
-  o[0] = __uint_as_float(w0 << 16);
-  o[1] = __uint_as_float(w0 & 0xffff0000u);
-  o[2] = __uint_as_float(w1 << 16);
-  o[3] = __uint_as_float(w1 & 0xffff0000u);
-}
-
-// The one-shot form of actor_step_resident_wide_kernel: same rows (fp32 logits that are a bf16 output layer's values
-// widened by .float(), the dtype stock Megatron hands a custom loss, relax/backends/megatron/loss.py:92-97), same
-// arithmetic in the same order, same bits.  A workgroup of 128 virtual threads keeps its share of the row as upper
-// halves (38 four-float positions per thread in 19 register quads at V = 151936), scans the fp32 values as they land,
-// ORs the low halves it drops; a wave that dropped nothing computes its gradient from the registers, a wave that did
-// (fp32 logits with real low bits) reads its share again.  Exchange, tags and waits as in actor_step_split_kernel.
-// (three waves per SIMD: 5.80 ms on 32768 x 151936 fp32 rows where four give 5.91 and two 5.75; rows of 248320
-// entries, 31 register quads per thread, are built for two)
-template <int NF, bool PARTIAL, int WAVES = 3>
-__global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES)))
-void actor_step_split_wide_kernel(
-    const float* __restrict__ logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
-    const int32_t* __restrict__ token_of_row, const int32_t* __restrict__ sample_ids,
-    const int64_t* __restrict__ targets, float c, float inv_t, relax_amd_policy_loss_args a, float grad_scale,
-    float* __restrict__ log_prob, float* __restrict__ entropy, float* __restrict__ lse_out,
-    float* __restrict__ spx_out, float* __restrict__ dlogits, int64_t d_stride, unsigned long long* __restrict__ ring,
-    unsigned laps, unsigned max_polls, unsigned wait_tag_offset) {
-  constexpr int kU = kScanUnroll, ROW_THREADS = 1024;
-  constexpr int NP = NF + (PARTIAL ? 1 : 0);  // vector positions per thread
-  static_assert(kU == 4, "positions are packed in pairs and scanned in groups of four");
-  constexpr int NR = (NP + 1) / 2;            // packed register quads
-  constexpr int kGroups = (NP + kU - 1) / kU;
-  constexpr int kPark = NR < 19 ? NR : 19;
-  __shared__ float bc[5];
-  __shared__ int64_t bc_target;
-  __shared__ u32x4 parked[kPark][kWave];
-  const int tid = threadIdx.x;
-  const bool wave0 = __builtin_amdgcn_readfirstlane(tid) < kWave;
-  const unsigned part = blockIdx.x % kSplit;
-  const int64_t row = blockIdx.x / kSplit;
-  const int vt = int(part) * kSplitThreads + tid;  // virtual thread of the row
-  const int rem = int(vocab / 4) - NF * ROW_THREADS;
-  auto has = [&](int p) -> bool { return p < NF || (PARTIAL && p == NF && vt < rem); };
-  u32x4* dv = reinterpret_cast<u32x4*>(dlogits + row * d_stride);
-
-  int64_t tok = token_of_row ? int64_t(token_of_row[row]) : row;
-  const int64_t t0 = tok;
-  if (tok >= 0) {
-    const float m = a.loss_mask[tok];
-    const float mp = a.pg_loss_mask ? a.pg_loss_mask[tok] : m;
-    if (m == 0.f && mp == 0.f && !a.read_masked_rows) tok = -1;
-  }
-  if (tok < 0) {  // a zero row: no read, no exchange
-    if (t0 >= 0 && part == 0 && tid == 0) {
-      log_prob[t0] = 0.f;
-      entropy[t0] = 0.f;
-      lse_out[t0] = 0.f;
-      spx_out[t0] = 0.f;
-      a.coef_log_prob[t0] = 0.f;
-      if (a.coef_entropy) a.coef_entropy[t0] = 0.f;
-    }
-#pragma unroll
-    for (int p = 0; p < NP; ++p)
-      if (has(p)) store_stream(dv + vt + p * ROW_THREADS, u32x4{0u, 0u, 0u, 0u});
-    return;
-  }
-
-  const u32x4* xv = reinterpret_cast<const u32x4*>(logits + row * row_stride);
-  const unsigned tag = exchange_tag(reinterpret_cast<const unsigned*>(ring + kRingWords), laps, row);
-  // The row share arrives group by group (four positions = one scan group): the vectors land in `land`, are absorbed
-  // into the softmax state as the fp32 values they are, and leave their upper halves in `reg`; the loads of the
-  // following group are requested before a group is absorbed.
-  u32x4 reg[NR];
-  SoftmaxAcc st{kNegHuge, 0.f, 0.f};
-  uint32_t low = 0u;
-  {
-    u32x4 land[2][kU];
-    bool grouped = true;
-    auto request = [&](int g) {
-#pragma unroll
-      for (int u = 0; u < kU; ++u) {
-        const int p = kU * g + u;
-        int lane_id = vt;
-        asm volatile("" : "+v"(lane_id));
-        land[g & 1][u] = (p < NP && has(p)) ? load_stream(xv + lane_id + p * ROW_THREADS) : u32x4{0u, 0u, 0u, 0u};
-      }
-    };
-    request(0);
-#pragma unroll
-    for (int g = 0; g < kGroups; ++g) {
-      if (g + 1 < kGroups) request(g + 1);
-      u32x4(&l)[kU] = land[g & 1];
-      if (grouped && kU * g + kU - 1 < NP && has(kU * g + kU - 1)) {
-        float v[kU * 4];
-#pragma unroll
-        for (int u = 0; u < kU; ++u) {
-          float four[4];
-          Row<float>::unpack(l[u], four);
-#pragma unroll
-          for (int k = 0; k < 4; ++k) v[u * 4 + k] = four[k];
-        }
-        scan_absorb(v, c, st);
-      } else {
-        grouped = false;
-#pragma unroll
-        for (int u = 0; u < kU; ++u)
-          if (kU * g + u < NP && has(kU * g + u)) {
-            float v[4];
-            Row<float>::unpack(l[u], v);
-            scan_absorb(v, c, st);
-          }
-      }
-#pragma unroll
-      for (int u = 0; u < kU; u += 2)
-        if (kU * g + u < NP) {
-          low |= split_wide_low_bits(l[u]) | split_wide_low_bits(l[u + 1]);
-          u32x4 r = split_wide_pack(l[u], l[u + 1]);
-          // packed here and now: left to itself the compiler parks the landed vectors in scratch memory and packs
-          // them when the gradient pass first asks for the result
-          asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w), "+v"(low));
-          reg[(kU * g + u) / 2] = r;
-        }
-      asm volatile("" : "+v"(st.m), "+v"(st.s), "+v"(st.t));
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  }
-  // did any lane of this wave drop non-zero low halves?  Then the wave takes its values from memory again below.
-  const bool reread = __builtin_amdgcn_ballot_w64(low != 0u) != 0ull;
-  wave_butterfly([&](auto o) {
-    constexpr int O = decltype(o)::value;
-    scan_merge(st, lane_xor<O>(st.m), lane_xor<O>(st.s), lane_xor<O>(st.t));
-  });
-  unsigned long long* slot = ring + size_t(row % kRing) * kSlotWords;
-  split_publish(slot, tag, vt, st);
-
-  if (wave0) {
-    __builtin_amdgcn_s_setprio(3);
-#pragma unroll
-    for (int j = 0; j < kPark; ++j) parked[j][tid] = reg[j];
-    TokenInputs tin{};
-    float x_target = 0.f, den = 1.f, pg_den = 1.f;
-    int64_t tg = -1;
-    if (tid == 0) {
-      tin = load_token_inputs(a, tok);
-      tg = targets[tok];
-      if (tg >= 0 && tg < vocab) x_target = logits[row * row_stride + tg];
-      const int32_t sid = sample_ids ? sample_ids[tok] : 0;
-      den = a.sample_denom ? a.sample_denom[sid] : 1.0f;
-      pg_den = a.pg_sample_denom ? a.pg_sample_denom[sid] : den;
-    }
-    bool any_gave_up = false;
-    const SoftmaxAcc whole = split_collect(slot, tag + wait_tag_offset, tid, max_polls,
-                                           reinterpret_cast<unsigned*>(ring + kRingWords), any_gave_up);
-    if (tid == 0) {
-      float lse = 0.f, spx = 0.f, ent = 0.f, lp = 0.f;
-      scan_finish(whole, x_target, tg >= 0 && tg < vocab, inv_t, lse, spx, ent, lp);
-      if (any_gave_up) lp = lse = __builtin_nanf("");
-      if (part == 0) {
-        log_prob[tok] = lp;
-        entropy[tok] = ent;
-        lse_out[tok] = lse;
-        spx_out[tok] = spx;
-      }
-      relax_amd_policy_loss_args al = a;
-      asm volatile("" : "+s"(al.eps_clip), "+s"(al.eps_clip_high), "+s"(al.eps_clip_c), "+s"(al.entropy_coef),
-                   "+s"(al.kl_coef), "+s"(al.tis_lo), "+s"(al.tis_hi), "+s"(al.tau_pos), "+s"(al.tau_neg));
-      const TokenResult tr = token_terms(al, tin, lp, ent, false, 0.f, den, pg_den);
-      if (part == 0) {
-        a.coef_log_prob[tok] = tr.coef_lp;
-        if (a.coef_entropy) a.coef_entropy[tok] = tr.coef_ent;
-      }
-      const float glp = tr.coef_lp * grad_scale, gh = tr.coef_ent * grad_scale;
-      const float b = gh * inv_t;
-      bc[0] = -lse * kLog2e;           // k0: p = exp2(x*c + k0)
-      bc[1] = -glp * inv_t + b * spx;  // a0
-      bc[2] = -b * inv_t;              // a1: d = p * (a0 + a1*x)
-      bc[3] = glp * inv_t;             // added at the target
-      bc[4] = (glp == 0.f && gh == 0.f) ? 1.f : 0.f;
-      bc_target = tg;
-    }
-#pragma unroll
-    for (int j = 0; j < kPark; ++j) reg[j] = parked[j][tid];
-    __builtin_amdgcn_s_setprio(0);
-  }
-  __syncthreads();
-  const float k0 = bc[0], a0 = bc[1], a1 = bc[2], hot = bc[3];
-  const int64_t tgt = bc_target;
-  const bool emit_zero = bc[4] != 0.f;
-  const int tvec = (tgt >= 0 && tgt < vocab) ? int(tgt / 4) : -1;
-  const int tsub = int(tgt % 4);
-  if (emit_zero) {
-#pragma unroll
-    for (int p = 0; p < NP; ++p)
-      if (has(p)) store_stream(dv + vt + p * ROW_THREADS, u32x4{0u, 0u, 0u, 0u});
-    return;
-  }
-  // gradient of one vector position; the element at the target gets `hot` added before it is stored, by the one wave
-  // of the row that holds it (a wave-uniform jump)
-  auto gradient_of = [&](float (&v)[4], int idx) -> u32x4 {
-#pragma unroll
-    for (int k = 0; k < 4; ++k) v[k] = fast_exp2(fmaf(v[k], c, k0)) * fmaf(v[k], a1, a0);
-    if (__builtin_amdgcn_ballot_w64(idx == tvec) != 0ull) {
-#pragma unroll
-      for (int k = 0; k < 4; ++k)
-        if (idx == tvec && k == tsub) v[k] += hot;
-    }
-    return Row<float>::pack(v);
-  };
-  if (!reread) {
-#pragma unroll
-    for (int p = 0; p < NP; ++p) {
-      int lane_id = vt;
-      asm volatile("" : "+v"(lane_id));
-      const int idx = lane_id + p * ROW_THREADS;
-      float v[4];
-      split_wide_unpack(reg[p / 2], p & 1, v);
-      const u32x4 out = gradient_of(v, idx);
-      if (has(p)) store_stream(dv + idx, out);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  } else {
-    // the registers hold rounded values: this wave's own words come from memory once more, four positions at a time
-#pragma unroll
-    for (int g = 0; g < kGroups; ++g) {
-      u32x4 raw[kU];
-#pragma unroll
-      for (int u = 0; u < kU; ++u) {
-        const int p = kU * g + u;
-        int lane_id = vt;
-        asm volatile("" : "+v"(lane_id));
-        if (p < NP) raw[u] = has(p) ? load_stream(xv + lane_id + p * ROW_THREADS) : u32x4{0u, 0u, 0u, 0u};
-      }
-#pragma unroll
-      for (int u = 0; u < kU; ++u) {
-        const int p = kU * g + u;
-        if (p < NP) {
-          int lane_id = vt;
-          asm volatile("" : "+v"(lane_id));
-          const int idx = lane_id + p * ROW_THREADS;
-          float v[4];
-          Row<float>::unpack(raw[u], v);
-          const u32x4 out = gradient_of(v, idx);
-          if (has(p)) store_stream(dv + idx, out);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  }
-}
-
 namespace {
 ExchangeRingCache ring_cache, topk_ring_cache;
 // relax_amd_set_exchange_wait: the bound of a workgroup's wait and an offset added to the tag it waits for
@@ -706,21 +449,37 @@ constexpr int split_waves_max() {
     return check_launch("actor_step_split");                                                                          \
   }
 #define RELAX_AMD_SPLIT(NVF, PARTIAL) RELAX_AMD_SPLIT_ROW(1024, NVF, PARTIAL)
-// rows of more than 20 vectors per thread: twelve or thirteen of them in LDS (24 - 26 KB of the 26.7 a workgroup can
-// have when six share a CU), three waves per SIMD; with the top-K term (4 KB of LDS more, a longer serial stretch)
-// sixteen in LDS and two waves per SIMD
-#define RELAX_AMD_SPLIT_LDS(NVF, PARTIAL)                                                                             \
+// Rows of more vectors per thread than the register file holds at three waves per SIMD (16-bit rows of more than 20,
+// fp32 rows of more than 16): part of every thread's share sits in LDS.  16-bit: twelve or thirteen vectors (24 - 26 KB
+// of the 26.7 a workgroup can have when six share a CU), three waves per SIMD.  fp32 rows of up to 40 vectors per
+// thread (100352 .. 163840 entries): thirteen in LDS, three waves; of 61 (248320 entries): nineteen in LDS (38 KB), two
+// waves.  With the top-K term (4 KB of LDS more, a longer serial stretch): sixteen in LDS and two waves per SIMD.
+template <int NV, bool TOPK, int VN>
+constexpr int split_lds_vecs() {
+  return TOPK ? 16 : (VN == 4 && NV > 40) ? 19 : (VN == 8 && NV <= 25) ? 12 : 13;
+}
+template <int NV, bool TOPK, int VN>
+constexpr int split_lds_waves() {
+  return (TOPK || (VN == 4 && NV > 40)) ? 2 : 3;
+}
+#define RELAX_AMD_SPLIT_LDS_KERNEL(NVF, PARTIAL, TOPK)                                                                \
+  actor_step_split_kernel<T, NVF, PARTIAL, TOPK, 1024, split_lds_waves<NVF + (PARTIAL ? 1 : 0), TOPK, VN>(),          \
+                          split_lds_waves<NVF + (PARTIAL ? 1 : 0), TOPK, VN>(),                                       \
+                          split_lds_vecs<NVF + (PARTIAL ? 1 : 0), TOPK, VN>()>
+#define RELAX_AMD_SPLIT_LDS(NVF, PARTIAL, WITH_TOPK)                                                                  \
   if (width == 1024 && full == NVF && partial == PARTIAL) {                                                           \
-    if (a.topk_ids)                                                                                                   \
-      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, true, 1024, 2, 2, 16>), grid, block, 0, stream,   \
-                         logits, row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e,       \
-                         inv_t, a, grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, topk_ring,      \
-                         laps, max_polls, tag_offset);                                                                \
-    else                                                                                                              \
-      hipLaunchKernelGGL((actor_step_split_kernel<T, NVF, PARTIAL, false, 1024, 3, 3, (NVF >= 30 ? 13 : 12)>), grid, \
-                         block, 0, stream, logits, row_stride, vocab, n_rows, token_of_row, sample_ids, targets,     \
-                         inv_t * kLog2e, inv_t, a, grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, \
-                         topk_ring, laps, max_polls, tag_offset);                                                     \
+    if (a.topk_ids) {                                                                                                 \
+      if constexpr (WITH_TOPK)                                                                                        \
+        hipLaunchKernelGGL((RELAX_AMD_SPLIT_LDS_KERNEL(NVF, PARTIAL, true)), grid, block, 0, stream, logits,         \
+                           row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,   \
+                           grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, topk_ring, laps,        \
+                           max_polls, tag_offset);                                                                    \
+    } else {                                                                                                          \
+      hipLaunchKernelGGL((RELAX_AMD_SPLIT_LDS_KERNEL(NVF, PARTIAL, false)), grid, block, 0, stream, logits,          \
+                         row_stride, vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a,     \
+                         grad_scale, log_prob, entropy, lse, spx, dlogits, d_stride, ring, topk_ring, laps,          \
+                         max_polls, tag_offset);                                                                      \
+    }                                                                                                                 \
     return check_launch("actor_step_split");                                                                          \
   }
 
@@ -749,8 +508,14 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
           (full == 7 && partial)))
       return RELAX_AMD_EUNSUPPORTED;
   } else {
-    if (!((full == 7 && partial) || (full == 8 && !partial) || (full == 12 && partial) || (full == 15 && partial) ||
-          (full == 16 && !partial)))
+    // fp32: 100352 / 102400 (25088 / 25600 vectors), 128256 / 129280 (32064 / 32320), 131072 (32768), 151936 / 152064 /
+    // 154880 (37984 / 38016 / 38720), 163840 (40960), 248320 (62080; the top-K term is left to the two-walk kernel)
+    const bool lds_row = (full == 24 && partial) || (full == 25 && !partial) || (full == 31 && partial) ||
+                         (full == 32 && !partial) || (full == 37 && partial) || (full == 40 && !partial) ||
+                         (full == 60 && partial);
+    if (full == 60 && a.topk_ids) return RELAX_AMD_EUNSUPPORTED;
+    if (!(lds_row || (full == 7 && partial) || (full == 8 && !partial) || (full == 12 && partial) ||
+          (full == 15 && partial) || (full == 16 && !partial)))
       return RELAX_AMD_EUNSUPPORTED;
   }
   unsigned long long* ring = nullptr;
@@ -768,10 +533,10 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
     RELAX_AMD_SPLIT_ROW(512, 8, false)
     RELAX_AMD_SPLIT_ROW(512, 12, true)
     // 200064 / 201088 / 202048 (25008 / 25136 / 25256 vectors), 250880 (31360), 256000 (32000), 262144 (32768) entries
-    RELAX_AMD_SPLIT_LDS(24, true)
-    RELAX_AMD_SPLIT_LDS(30, true)
-    RELAX_AMD_SPLIT_LDS(31, true)
-    RELAX_AMD_SPLIT_LDS(32, false)
+    RELAX_AMD_SPLIT_LDS(24, true, true)
+    RELAX_AMD_SPLIT_LDS(30, true, true)
+    RELAX_AMD_SPLIT_LDS(31, true, true)
+    RELAX_AMD_SPLIT_LDS(32, false, true)
     RELAX_AMD_SPLIT(20, false)
     RELAX_AMD_SPLIT(19, true)
     RELAX_AMD_SPLIT(18, true)
@@ -781,6 +546,13 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
     RELAX_AMD_SPLIT(8, false)
     RELAX_AMD_SPLIT(7, true)
   } else {
+    RELAX_AMD_SPLIT_LDS(37, true, true)
+    RELAX_AMD_SPLIT_LDS(31, true, true)
+    RELAX_AMD_SPLIT_LDS(32, false, true)
+    RELAX_AMD_SPLIT_LDS(40, false, true)
+    RELAX_AMD_SPLIT_LDS(24, true, true)
+    RELAX_AMD_SPLIT_LDS(25, false, true)
+    RELAX_AMD_SPLIT_LDS(60, true, false)
     RELAX_AMD_SPLIT(7, true)
     RELAX_AMD_SPLIT(8, false)
     RELAX_AMD_SPLIT(12, true)
@@ -790,53 +562,11 @@ int launch_actor_step_split(const T* logits, int64_t row_stride, int64_t vocab, 
   return RELAX_AMD_EUNSUPPORTED;
 }
 #undef RELAX_AMD_SPLIT_LDS
+#undef RELAX_AMD_SPLIT_LDS_KERNEL
 #undef RELAX_AMD_SPLIT
 #undef RELAX_AMD_SPLIT_ROW
 #undef RELAX_AMD_SPLIT_KERNEL
 
-#define RELAX_AMD_SPLIT_WIDE(NF, PARTIAL)                                                                             \
-  if (full == NF && partial == PARTIAL) {                                                                             \
-    hipLaunchKernelGGL((actor_step_split_wide_kernel<NF, PARTIAL, 3>), grid, block, 0, stream,       \
-                       logits, row_stride,                                                                            \
-                       vocab, n_rows, token_of_row, sample_ids, targets, inv_t * kLog2e, inv_t, a, grad_scale,       \
-                       log_prob, entropy, lse, spx, dlogits, d_stride, ring, laps, max_polls, tag_offset);           \
-    return check_launch("actor_step_split_wide");                                                                     \
-  }
-
-int launch_actor_step_split_wide(const float* logits, int64_t row_stride, int64_t vocab, int64_t n_rows,
-                                 const int32_t* token_of_row, const int32_t* sample_ids, const int64_t* targets,
-                                 float inv_t, const relax_amd_policy_loss_args& a, float grad_scale, float* log_prob,
-                                 float* entropy, float* lse, float* spx, float* dlogits, int64_t d_stride,
-                                 hipStream_t stream) {
-  // the top-K distillation block is evaluated by the two-walk kernel for these rows
-  if (a.topk_ids || vocab % 4 != 0 || scan_threads(vocab, 4) != 1024 || n_rows * kSplit > 2147483647LL)
-    return RELAX_AMD_EUNSUPPORTED;
-  const int64_t nvec = vocab / 4;
-  const int full = int(nvec / 1024);
-  const bool partial = nvec % 1024 != 0;
-  if (!((full == 37 && partial) || (full == 31 && partial) || (full == 32 && !partial) || (full == 40 && !partial) ||
-        (full == 24 && partial) || (full == 25 && !partial) || (full == 60 && partial)))
-    return RELAX_AMD_EUNSUPPORTED;
-  unsigned long long* ring = nullptr;
-  if (int rc = split_ring_of_device(&ring)) return rc;
-  const unsigned laps = unsigned((n_rows + kRing - 1) / kRing);
-  const unsigned max_polls = exchange_max_polls();
-  const unsigned tag_offset = exchange_wait_tag_offset();
-  hipLaunchKernelGGL(exchange_ring_advance_kernel<kRingWords>, dim3(1), dim3(256), 0, stream, ring, laps,
-                     static_cast<unsigned long long*>(nullptr), size_t(0));
-  const dim3 grid(static_cast<unsigned>(n_rows * kSplit)), block(kSplitThreads);
-  // 151936 / 152064 (37984 / 38016 vectors), 128256 / 129280 (32064 / 32320), 131072 (32768), 163840 (40960),
-  // 100352 / 102400 (25088 / 25600), 248320 (62080)
-  RELAX_AMD_SPLIT_WIDE(60, true)
-  RELAX_AMD_SPLIT_WIDE(37, true)
-  RELAX_AMD_SPLIT_WIDE(31, true)
-  RELAX_AMD_SPLIT_WIDE(32, false)
-  RELAX_AMD_SPLIT_WIDE(40, false)
-  RELAX_AMD_SPLIT_WIDE(24, true)
-  RELAX_AMD_SPLIT_WIDE(25, false)
-  return RELAX_AMD_EUNSUPPORTED;
-}
-#undef RELAX_AMD_SPLIT_WIDE
 
 template int launch_actor_step_split<float>(const float*, int64_t, int64_t, int64_t, const int32_t*, const int32_t*,
                                             const int64_t*, float, const relax_amd_policy_loss_args&, float, float*,
