@@ -1250,7 +1250,9 @@ def test_policy_loss_with_opd_term_vs_oracle(case, single_pass):
                                                (151936, torch.bfloat16, 256, "reverse_tail"),
                                                # rows of 31 vectors per thread: sixteen of them in LDS, no persistent
                                                # kernel to compare with
-                                               (248320, torch.bfloat16, 64, "reverse_tail")])
+                                               (248320, torch.bfloat16, 64, "reverse_tail"),
+                                               # fp32 rows of 38 vectors per thread, sixteen of them in LDS
+                                               (151936, torch.float32, 64, "union_jsd_clips")])
 def test_topk_opd_term_in_the_register_resident_step(v, dtype, k, variant):
     """The top-K distillation term inside the single launch on the row shapes of the register-resident kernel (several
     rows per persistent workgroup, K below and above one wave's width, the union mask, clips): loss, metrics and
@@ -1291,7 +1293,8 @@ def test_topk_opd_term_in_the_register_resident_step(v, dtype, k, variant):
         loss.backward()
         outs[mode] = (loss.detach(), met, lg.grad)
     # the persistent kernel, or for rows it is not built for the two-walk kernel, bit for bit
-    ops.set_kernel_choice("resident" if v <= 163840 else "two_walk")
+    has_resident = v <= (163840 if dtype != torch.float32 else 65536)
+    ops.set_kernel_choice("resident" if has_resident else "two_walk")
     try:
         lg = logits.to(dev).requires_grad_()
         loss, met = relax_amd.policy_loss_function(P.make_args(relax_amd_single_pass="auto", **kw), db, lg, None)
