@@ -187,6 +187,17 @@ def live_traffic_of(kernel: str):
                           f"{t['fetch_scale']:.3f} + {w:.0f} x {t['write_scale']:.3f} KiB (scales: the same counters over known-size launches of this run)")
 
 
+def assert_kernel_ran(entry: str, kernel: str) -> None:
+    """The kernel names above restate the library's dispatch rule; ``relax_amd_last_kernel`` says which family the
+    entry point really launched.  A disagreement would put the roofline figures under the wrong kernel's name."""
+    from relax_amd import ops
+
+    want = kernel.split("<")[0].removesuffix("_kernel")
+    want = {"reverse_kl_step": "reverse_kl_step_fused"}.get(want, want)
+    ran = ops.last_kernel(entry)
+    assert ran == want, f"{entry} launched {ran!r}, this file expected {want!r} ({kernel})"
+
+
 def hbm_roofline(kernel: str, launch_ms: float, necessary_bytes: float, rows: int, vocab: int, kernel_ms: dict,
                  ms_per_step: float, two_pass_bytes: float | None = None) -> dict:
     """Roofline block of a bandwidth-bound launch.  ``achieved`` = the bytes the launch has to move (every input row
@@ -492,10 +503,12 @@ def run_actor_step(a, dev) -> None:
     necessary = row_bytes * (live + n_tokens)
     if "actor_step_fused" in kernel_ms:
         dom, dom_name = kernel_ms["actor_step_fused"], fused_step_kernel_name(a.vocab, "float" if fp32 else "bf16_t")
+        assert_kernel_ran("actor_step_fused", dom_name)
         if a.opd_topk > 0:
             dom_name = dom_name[:-1] + ", true>"  # the instantiation that evaluates the top-K term
     else:  # two launches: the backward (read live rows, write all rows) dominates; the forward read is its own launch
         dom, dom_name = kernel_ms["logprob_entropy_bwd"], bwd_kernel_name(a.vocab)
+        assert_kernel_ran("logprob_entropy_bwd", dom_name)
     emit(a, n_tokens, wall,
          f"Qwen3-8B-shaped actor step: {a.seqs} seqs x {a.seq_len} tokens = {n_tokens} rows x V={a.vocab} "
          f"{'fp32 (bf16 values widened, as Megatron hands them to a custom loss)' if fp32 else 'bf16'} "
@@ -669,6 +682,7 @@ def run_reverse_kl(a, dev) -> None:
     if "reverse_kl_step_fused" in kernel_ms:
         # every token reports its KL, so both rows of every token are read once; one gradient row written per token
         dom, dom_name, necessary = kernel_ms["reverse_kl_step_fused"], kl_step_kernel_name(v), 3.0 * row_bytes * n
+        assert_kernel_ran("reverse_kl_step_fused", dom_name)
         two_pass = 5.0 * row_bytes * n  # forward read of both rows, backward re-read of both, gradient write
     else:
         dom_name = "reverse_kl_bwd_kernel<bf16_t, true>" if KERNEL_CHOICE == "two_walk" else "reverse_kl_bwd_chunk_kernel<bf16_t>"

@@ -95,6 +95,16 @@ enum { RELAX_AMD_KERNEL_AUTO = 0, RELAX_AMD_KERNEL_TWO_WALK = 1, RELAX_AMD_KERNE
  * (hipGetSymbolAddress), so make one call outside a capture first.
  */
 int relax_amd_set_kernel_choice(int choice);
+/*
+ * Which kernel family the last launching call on this thread ended with ("" before any): "actor_step_split",
+ * "actor_step_resident", "actor_step_resident_wide" or "actor_step_fused" (the two-walk kernel) after
+ * relax_amd_actor_step_fused; "reverse_kl_split", "reverse_kl_resident" or "reverse_kl_step_fused" after
+ * relax_amd_reverse_kl_step_fused; "logprob_entropy_bwd_chunk", "logprob_entropy_bwd_resident" or
+ * "logprob_entropy_bwd" after relax_amd_logprob_entropy_bwd; the entry point's own name elsewhere.  Host pointer to a
+ * constant string.  No counterpart in the reference: it lets a caller (and this library's tests) see that a row shape
+ * took the kernel built for it rather than the two-walk kernel, which serves every shape with the same results.
+ */
+const char* relax_amd_last_kernel(void);
 
 /*
  * For tests of the failure handling of the one-shot actor and reverse-KL steps: max_polls bounds how often a workgroup looks for its

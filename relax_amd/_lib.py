@@ -74,6 +74,7 @@ KERNEL_CHOICES = {"auto": 0, "two_walk": 1, "resident": 2}
 SIGNATURES = {
     "relax_amd_version": (C.c_int, []),
     "relax_amd_last_error": (C.c_char_p, []),
+    "relax_amd_last_kernel": (C.c_char_p, []),
     "relax_amd_set_kernel_choice": (C.c_int, [C.c_int]),
     "relax_amd_set_exchange_wait": (C.c_int, [C.c_int, C.c_int]),
     "relax_amd_logprob_entropy_fwd": (C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp]),

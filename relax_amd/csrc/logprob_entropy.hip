@@ -250,7 +250,7 @@ static int launch_bwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t
       hipLaunchKernelGGL((logprob_entropy_bwd_chunk_kernel<T>), dim3(static_cast<unsigned>(n_rows * chunks)),
                          dim3(kChunkThreads), 0, s, x, stride, nvec, static_cast<unsigned>(chunks), token_of_row,
                          targets, lse, spx, g_lp, g_ent, grad_scale, grad_scale_dev, c, inv_t, d, d_stride);
-      return check_launch("logprob_entropy_bwd");
+      return check_launch("logprob_entropy_bwd_chunk");
     }
   }
   if (vec && choice != RELAX_AMD_KERNEL_TWO_WALK) {

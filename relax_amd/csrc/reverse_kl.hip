@@ -409,7 +409,7 @@ static int launch_kl_bwd(const void* s, const void* t, int64_t n, int64_t vocab,
       hipLaunchKernelGGL((reverse_kl_bwd_chunk_kernel<T>), dim3(static_cast<unsigned>(n * chunks)),
                          dim3(kKlChunkThreads), 0, st, static_cast<const T*>(s), static_cast<const T*>(t), stride, nvec,
                          static_cast<unsigned>(chunks), kl, ls, lt, g, scale, scale_dev, static_cast<T*>(d));
-      return check_launch("reverse_kl_bwd");
+      return check_launch("reverse_kl_bwd_chunk");
     }
   }
   if (vec)

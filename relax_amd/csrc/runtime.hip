@@ -8,6 +8,7 @@
 namespace relax_amd {
 
 static thread_local char g_error[512] = "";
+static thread_local const char* g_last_kernel = "";
 
 void set_error(const char* fmt, ...) {
   va_list ap;
@@ -17,6 +18,7 @@ void set_error(const char* fmt, ...) {
 }
 
 int check_launch(const char* what) {
+  g_last_kernel = what;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("%s: kernel launch failed: %s", what, hipGetErrorString(e));
@@ -48,3 +50,4 @@ extern "C" int relax_amd_set_kernel_choice(int choice) {
 
 extern "C" int relax_amd_version(void) { return RELAX_AMD_ABI_VERSION; }
 extern "C" const char* relax_amd_last_error(void) { return relax_amd::g_error; }
+extern "C" const char* relax_amd_last_kernel(void) { return relax_amd::g_last_kernel; }

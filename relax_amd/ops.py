@@ -27,6 +27,20 @@ def set_kernel_choice(name: str) -> str:
     return {v: k for k, v in KERNEL_CHOICES.items()}[prev]
 
 
+_LAST_KERNEL: dict = {}
+
+
+def _note_kernel(entry: str) -> None:
+    _LAST_KERNEL[entry] = lib.relax_amd_last_kernel().decode()
+
+
+def last_kernel(entry: str) -> str:
+    """Which kernel family the last call of ``entry`` ("actor_step_fused" | "reverse_kl_step_fused" |
+    "logprob_entropy_bwd") on this process launched (``relax_amd_last_kernel`` read right behind the call): e.g.
+    "actor_step_split" for the one-shot workgroups, "actor_step_fused" for the two-walk kernel."""
+    return _LAST_KERNEL.get(entry, "")
+
+
 def _need_gpu(*tensors) -> torch.device:
     dev = None
     for t in tensors:
@@ -141,6 +155,7 @@ def logprob_entropy_bwd(logits, targets, lse, spx, g_lp, g_ent=None, token_of_ro
             _p(logits), _code(logits), logits.size(0), logits.size(1), stride, _p(token_of_row), _p(targets), _p(lse),
             _p(spx), _p(g_lp), _p(g_ent), float(grad_scale), _p(grad_scale_dev), float(inv_temperature),
             _p(out), out.stride(0) if out.size(0) > 1 else out.size(1), _stream()))
+    _note_kernel("logprob_entropy_bwd")
     return out
 
 
@@ -398,6 +413,7 @@ def actor_step_fused(logits, targets, token_of_row, sample_ids, n_tokens: int, i
             _p(logits), _code(logits), logits.size(0), logits.size(1), stride, _p(token_of_row), _p(sample_ids),
             _p(targets), float(inv_temperature), C.byref(a), float(grad_scale), _p(lp), _p(ent), _p(lse), _p(spx),
             _p(dlogits), logits.size(1), _stream()))
+    _note_kernel("actor_step_fused")
     a.log_prob, a.entropy = lp.data_ptr(), ent.data_ptr()
     check(lib.relax_amd_policy_loss(C.byref(a), _stream()))
     return out, lp, ent, lse, spx, dlogits
@@ -564,6 +580,7 @@ def reverse_kl_step_fused(student, teacher, g, grad_scale: float = 1.0):
     with _timed("reverse_kl_step_fused"):
         check(lib.relax_amd_reverse_kl_step_fused(_p(s), _p(t), _code(s), n, s.size(1), s.size(1), _p(g),
                                                   float(grad_scale), _p(kl), _p(ls), _p(lt), _p(d), _stream()))
+    _note_kernel("reverse_kl_step_fused")
     return kl, ls, lt, d
 
 

@@ -1956,6 +1956,46 @@ def test_log_probs_and_entropy_of_every_kernel_agree_bitwise_at_a_temperature(v,
         ops.set_kernel_choice("auto")
 
 
+@pytest.mark.parametrize("v", [151936, 152064, 154880, 129280, 163840, 248320])
+def test_vocabularies_of_the_reference_model_scripts_take_the_one_shot_kernels(v):
+    """The vocabulary sizes the reference's model scripts name (scripts/models/*.sh: qwen3-*, qwen25-7B, glm4.7 / glm5,
+    kimi-k2.6, qwen35-* / qwen36-* / qwen38-*, and 129280) in bf16 and in the fp32 stock Megatron hands a custom loss:
+    the fused actor step, the fused reverse-KL step and the backward-only launch each report the kernel built for the
+    shape (relax_amd_last_kernel), not the two-walk kernel that serves every shape."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    announce("fast-path coverage", v)
+    n = 24
+    g = torch.Generator().manual_seed(v)
+    mask = (torch.rand(n, generator=g) > 0.2).float()
+    kw = dict(advantages=torch.randn(n, generator=g).to(dev), loss_mask=mask.to(dev),
+              cu_resp=torch.tensor([0, n], dtype=torch.int64, device=dev),
+              old_log_prob=(-12.0 + 0.3 * torch.randn(n, generator=g)).to(dev),
+              sample_denom=torch.tensor([max(1.0, mask.sum().item())], device=dev), loss_kind="ppo", eps_clip=0.2,
+              eps_clip_high=0.28)
+    sample_ids = torch.zeros(n, dtype=torch.int32, device=dev)
+    targets = torch.randint(0, v, (n,), generator=g).to(dev)
+    for dtype in (torch.bfloat16, torch.float32):
+        logits = (torch.randn(n, v, generator=g) * 2).to(dtype).to(dev)
+        out, lp, ent, lse, spx, d = ops.actor_step_fused(logits, targets, None, sample_ids, n, 1.0, 1.0, **kw)
+        assert ops.last_kernel("actor_step_fused") == "actor_step_split", (dtype, ops.last_kernel("actor_step_fused"))
+        ops.logprob_entropy_bwd(logits, targets, lse, spx, torch.ones(n, device=dev), torch.zeros(n, device=dev))
+        assert ops.last_kernel("logprob_entropy_bwd") == "logprob_entropy_bwd_chunk"
+        assert torch.isfinite(lp[mask.to(dev) != 0]).all()
+    s = (torch.randn(n, v, generator=g) * 2).bfloat16().to(dev)
+    t = (torch.randn(n, v, generator=g) * 2).bfloat16().to(dev)
+    kl, _, _, _ = ops.reverse_kl_step_fused(s, t, torch.ones(n, device=dev), 1.0)
+    assert ops.last_kernel("reverse_kl_step_fused") == "reverse_kl_split"
+    assert torch.isfinite(kl).all()
+    ops.set_kernel_choice("two_walk")
+    try:
+        ops.actor_step_fused(logits, targets, None, sample_ids, n, 1.0, 1.0, **kw)
+        assert ops.last_kernel("actor_step_fused") == "actor_step_fused"
+    finally:
+        ops.set_kernel_choice("auto")
+
+
 def test_one_shot_step_gives_up_a_wait_that_cannot_succeed_and_recovers():
     """Failure handling of the exchange between the workgroups of a row, forced from the host
     (relax_amd_set_exchange_wait): with the tag a workgroup waits for offset by one, no wait can succeed; bounded to a
