@@ -321,6 +321,46 @@ def test_one_shot_reverse_kl_step_on_short_rows_equals_two_walk_kernel_bitwise(v
     torch.testing.assert_close(results["auto"]["d"].view(dtype)[rows].float().cpu(), sc.grad.float(), atol=2e-3, rtol=ulp)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_one_shot_reverse_kl_step_on_random_layouts_equals_two_walk_kernel_bitwise(seed):
+    """Random row counts (from a single row up to more than the exchange ring's 4096 slots), row lengths from every
+    family the one-shot kernel is built for (and their neighbours by one vector), both 16-bit types, random runs of
+    rows without gradient: the default kernel choice against the two-walk kernel, every output bit for bit."""
+    from relax_amd import ops
+
+    dev = require_gpu()
+    gen = torch.Generator(device=dev).manual_seed(2000 + seed)
+    cpu = torch.Generator().manual_seed(2000 + seed)
+    nvecs = [6 * 1024 + 1, 7 * 1024 + 832, 8 * 1024, 12 * 1024 + 256, 15 * 1024 + 1023, 16 * 1024, 18 * 1024 + 560,
+             19 * 1024 + 5, 20 * 1024, 24 * 1024 + 680, 30 * 1024 + 320, 31 * 1024 + 256, 32 * 1024]
+    nvec = nvecs[seed % len(nvecs)] if seed < len(nvecs) else nvecs[int(torch.randint(0, len(nvecs), (1,), generator=cpu))]
+    dtype = [torch.bfloat16, torch.float16][seed % 2]
+    v = nvec * 8
+    budget = 1_200_000_000 // (v * 2 * 2)
+    n = [1, 7, 9, 63][seed % 4] if seed % 3 == 0 else int(torch.randint(64, max(65, min(budget, 6000)), (1,), generator=cpu))
+    if seed == 1:
+        n = 4400  # more rows than the ring has slots
+    announce("one-shot reverse KL, random layout", seed, v, dtype, n)
+    s = (torch.randn((n, v), device=dev, generator=gen) * 3).to(dtype)
+    t = (s.float() + torch.randn((n, v), device=dev, generator=gen)).to(dtype)
+    g = (torch.rand(n, device=dev, generator=gen) > 0.3).float() * torch.rand(n, device=dev, generator=gen)
+    if n > 20:
+        g[n // 3:n // 3 + 11] = 0.0
+    results = {}
+    try:
+        for kind in ("two_walk", "auto"):
+            ops.set_kernel_choice(kind)
+            kl, ls, lt, d = ops.reverse_kl_step_fused(s, t, g, 0.5)
+            torch.cuda.synchronize()
+            results[kind] = dict(kl=kl, lse_s=ls, lse_t=lt, d=d.view(torch.int16))
+        assert ops.last_kernel("reverse_kl_step_fused") == "reverse_kl_split"
+    finally:
+        ops.set_kernel_choice("auto")
+    for key, want in results["two_walk"].items():
+        assert torch.equal(results["auto"][key], want), (seed, key)
+    assert torch.isfinite(results["auto"]["kl"]).all()
+
+
 def test_one_shot_reverse_kl_step_gives_up_a_wait_that_cannot_succeed_and_recovers():
     """Failure handling of the exchange between the workgroups of a row, forced from the host
     (relax_amd_set_exchange_wait): with the awaited tag offset by one no wait can succeed; every workgroup gives up
