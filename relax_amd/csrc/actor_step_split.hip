@@ -17,6 +17,12 @@
 // Exchange: the tagged ring of row_exchange.h, a slot of 16 x 3 words per row; a workgroup that gives up its wait
 // writes NaN log-probs instead of hanging.
 //
+// Rows whose share does not fit the registers of three waves per SIMD (16-bit rows of more than 20 vectors per thread,
+// fp32 rows of more than 16: vocabularies of 100352 .. 163840 entries as fp32, 200 k .. 262 k entries as 16-bit,
+// 248320 as either) keep twelve to nineteen vectors of every thread's share in LDS, put there by global -> LDS loads
+// without a register in between (LDS_VECS).  An fp32 row of 151936 entries is thereby read once as it is (5.85 -
+// 5.95 ms per 32768 rows whether its values are widened bf16 or genuinely fp32).
+//
 // Replaces, like the other fused kernels, _VocabParallelLogProbEntropy.forward + .backward
 // (relax/utils/training/ppo_utils.py:481-629) and the per-token part of policy_loss_function
 // (relax/backends/megatron/loss.py:961-1100) for one micro-batch.
